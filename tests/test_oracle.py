@@ -1,0 +1,281 @@
+"""Pins the CPU oracle (oracle/) before anything is compared against it.
+
+Checks are chosen so that a plausible mistake (dropped scale, wrong GQA grouping, off-by-one in the
+window, transposed operand, wrong sign in dS) fails at least one of them.
+"""
+
+import json
+import os
+
+import numpy as np
+import pytest
+import scipy.special
+import torch
+
+from oracle import brute
+from oracle import ref_attention as ref
+
+
+def _rand(seed, shape):
+    return np.random.default_rng(seed).standard_normal(shape)
+
+
+# ------------------------------------------------------------------ masks: reference's own tables
+
+
+def test_sliding_window_tables(golden_dir):
+    g = json.load(open(os.path.join(golden_dir, "mask_tables.json")))
+    for case in g["sliding_window_5x5"]:
+        fn = ref.sliding_window_causal_mask(case["left_context"])
+        got = fn(np.arange(5)[:, None], np.arange(5)[None, :]).astype(np.int32)
+        assert got.tolist() == case["expected"]
+    for case in g["sliding_window2_with_time_step_3x5"]:
+        fn = ref.sliding_window_causal_mask(2)
+        got = fn(np.arange(3)[:, None] + case["time_step"], np.arange(5)[None, :]).astype(np.int32)
+        assert got.tolist() == case["expected"]
+
+
+def test_causal_and_segment_tables(golden_dir):
+    g = json.load(open(os.path.join(golden_dir, "mask_tables.json")))
+    got = ref.causal_mask(np.arange(3)[:, None], np.arange(3)[None, :]).astype(np.int32)
+    assert got.tolist() == g["causal_3x3"]
+    bias = ref.bool_to_bias(ref.causal_mask(np.arange(3)[:, None], np.arange(3)[None, :]))
+    assert bias[0, 1] == np.float32(-1e15) and bias[1, 0] == 0.0
+    seg = g["segment_4x4"]
+    got = ref.segment_mask(np.asarray(seg["target_segments"]), np.asarray(seg["source_segments"]))
+    assert got[:, None].astype(np.int32).tolist() == seg["expected"]
+
+
+def test_sliding_window_block_map_invariant(golden_dir):
+    g = json.load(open(os.path.join(golden_dir, "mask_tables.json")))["sliding_window_block_map_invariant"]
+    for w in g["sliding_window_sz"]:
+        for t in g["seq_len"]:
+            for blk in g["block_size"]:
+                kw = dict(q_seq_len=t, kv_seq_len=t, block_q=blk, block_k=blk)
+                a = ref.build_mask(ref.sliding_window_causal_mask(w), **kw)
+                b = ref.build_sliding_window_mask(**kw, sliding_window_size=w)
+                assert (a == b).all(), (w, t, blk)
+
+
+def test_mask_spec_sums_biases():
+    seg = torch.tensor([[1, 1, 2, 2]], dtype=torch.int32)
+    spec = ref.MaskSpec(causal=True, segment_ids=seg)
+    bias = spec.bias_rows(1, 0, 4, 4, 4, torch.float32)[0, 0]
+    assert bias[0, 0] == 0 and bias[3, 2] == 0
+    assert bias[0, 1] == -1e15  # causal only
+    assert bias[2, 0] == -1e15  # segment only
+    assert bias[0, 3] == -2e15  # both: composite bias is a plain sum
+    keep = spec.keep_rows(0, 4, 4, 4)[0]
+    assert keep.int().tolist() == [[1, 0, 0, 0], [1, 1, 0, 0], [0, 0, 1, 0], [0, 0, 1, 1]]
+
+
+# ------------------------------------------------------------------ forward values
+
+
+@pytest.mark.parametrize("hq,hkv", [(4, 4), (4, 2), (4, 1)])
+def test_forward_matches_scipy_softmax(hq, hkv):
+    b, t, s, d = 2, 9, 13, 8
+    q, k, v = _rand(1, (b, t, hq, d)), _rand(2, (b, s, hkv, d)), _rand(3, (b, s, hkv, d))
+    scale = 0.37
+    out, lse = ref.reference_mha(torch.from_numpy(q), torch.from_numpy(k), torch.from_numpy(v),
+                                 softmax_scale=scale, return_lse=True, row_block=4)
+    g = hq // hkv
+    kr, vr = np.repeat(k, g, axis=2), np.repeat(v, g, axis=2)  # common.py:475-484
+    logits = np.einsum("bthd,bshd->bhts", q * scale, kr)
+    p = scipy.special.softmax(logits, axis=-1)
+    want = np.einsum("bhts,bshd->bthd", p, vr)
+    np.testing.assert_allclose(out.numpy(), want, rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(lse.numpy(), scipy.special.logsumexp(logits, axis=-1), rtol=1e-12, atol=1e-12)
+    bo, bl = brute.attention_fwd(q, k, v, scale=scale)
+    np.testing.assert_allclose(bo, want, rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(bl, lse.numpy(), rtol=1e-12, atol=1e-12)
+
+
+def test_forward_matches_torch_sdpa_causal():
+    b, t, h, d = 2, 32, 3, 16
+    q, k, v = (torch.from_numpy(_rand(i, (b, t, h, d))) for i in (4, 5, 6))
+    scale = d ** -0.5
+    got = ref.reference_mha(q, k, v, ref.MaskSpec(causal=True), softmax_scale=scale, row_block=8)
+    want = torch.nn.functional.scaled_dot_product_attention(
+        q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2), is_causal=True, scale=scale
+    ).transpose(1, 2)
+    torch.testing.assert_close(got, want, rtol=1e-12, atol=1e-12)
+    bo, _ = brute.attention_fwd(q.numpy(), k.numpy(), v.numpy(), scale=scale, mask_kind=brute.MASK_CAUSAL)
+    np.testing.assert_allclose(bo, want.numpy(), rtol=1e-12, atol=1e-12)
+
+
+def test_closed_forms():
+    b, t, h, d = 1, 16, 2, 8
+    q, k = (torch.from_numpy(_rand(i, (b, t, h, d))) for i in (7, 8))
+    v = torch.from_numpy(_rand(9, (b, t, h, d)))
+    out = ref.reference_mha(q, k, v, ref.MaskSpec(causal=True))
+    torch.testing.assert_close(out[:, 0], v[:, 0])  # causal row 0 sees only key 0
+    const = torch.ones_like(v) * torch.arange(d, dtype=torch.float64)
+    out = ref.reference_mha(q, k, const, ref.MaskSpec(causal=True))
+    torch.testing.assert_close(out, const)  # uniform V => out == V
+    # window 0 == attend to self only.
+    out = ref.reference_mha(q, k, v, ref.MaskSpec(sliding_window=0))
+    torch.testing.assert_close(out, v)
+    # Fully masked row: the bias is additive and finite, and in fp32 (the reference's logits dtype
+    # for fp32 inputs) x + -1e15 == -1e15, so the row becomes a uniform average over ALL keys.
+    spec = ref.MaskSpec(dense_bias=torch.full((1, 1, t, t), ref.NEG_INF))
+    out = ref.reference_mha(q.float(), k.float(), v.float(), spec, mode="faithful")
+    torch.testing.assert_close(out, v.float().mean(dim=1, keepdim=True).expand_as(v), rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("window", [None, 0, 3, 100])
+@pytest.mark.parametrize("with_seg", [False, True])
+def test_masks_against_brute_force(window, with_seg):
+    b, t, hq, hkv, d = 2, 24, 4, 2, 8
+    q, k, v = _rand(10, (b, t, hq, d)), _rand(11, (b, t, hkv, d)), _rand(12, (b, t, hkv, d))
+    seg = ref.packed_segment_ids(3, b, t, max_docs=4) if with_seg else None
+    spec = ref.MaskSpec(causal=window is None, sliding_window=window, segment_ids=seg)
+    got, lse = ref.reference_mha(torch.from_numpy(q), torch.from_numpy(k), torch.from_numpy(v), spec,
+                                 softmax_scale=0.3, return_lse=True, row_block=5)
+    kind = brute.MASK_CAUSAL if window is None else brute.MASK_SLIDING
+    bo, bl = brute.attention_fwd(q, k, v, scale=0.3, mask_kind=kind, window=window or 0,
+                                 segment_ids=None if seg is None else seg.numpy())
+    np.testing.assert_allclose(got.numpy(), bo, rtol=1e-11, atol=1e-11)
+    np.testing.assert_allclose(lse.numpy(), bl, rtol=1e-11, atol=1e-11)
+    # Element-level check of the window edge via per-element python loop.
+    keep = spec.keep_rows(0, t, t, t)
+    for bi in range(b):
+        for i in range(t):
+            for j in range(t):
+                want = i >= j and (window is None or i - j <= window)
+                if seg is not None:
+                    want = want and int(seg[bi, i]) == int(seg[bi, j])
+                assert bool(keep[bi if keep.shape[0] > 1 else 0, i, j]) == want
+
+
+def test_faithful_mode_close_to_highprec_bf16():
+    b, t, hq, hkv, d = 1, 64, 4, 2, 32
+    q = ref.normal_tensor(0, (b, t, hq, d), torch.bfloat16)
+    k = ref.normal_tensor(1, (b, t, hkv, d), torch.bfloat16)
+    v = ref.normal_tensor(2, (b, t, hkv, d), torch.bfloat16)
+    spec = ref.MaskSpec(causal=True)
+    hp = ref.reference_mha(q, k, v, spec, softmax_scale=d ** -0.5)
+    fa = ref.reference_mha(q, k, v, spec, softmax_scale=d ** -0.5, mode="faithful")
+    assert fa.dtype == torch.bfloat16
+    assert ref.max_abs(fa, hp) < 2e-2
+
+
+# ------------------------------------------------------------------ gradients
+
+
+def _loss(q, k, v, do, scale, mask_kind, window, seg):
+    out, _ = brute.attention_fwd(q, k, v, scale=scale, mask_kind=mask_kind, window=window, segment_ids=seg)
+    return float((out * do).sum())
+
+
+def test_gradients_finite_differences():
+    b, t, hq, hkv, d = 1, 6, 4, 2, 3
+    q, k, v, do = (_rand(i, s) for i, s in ((20, (b, t, hq, d)), (21, (b, t, hkv, d)), (22, (b, t, hkv, d)), (23, (b, t, hq, d))))
+    seg = np.asarray([[1, 1, 1, 2, 2, 2]], dtype=np.int32)
+    scale, kind, window = 0.7, brute.MASK_SLIDING, 2
+    dq, dk, dv = brute.attention_bwd(q, k, v, do, scale=scale, mask_kind=kind, window=window, segment_ids=seg)
+    eps = 1e-6
+    for name, x, gx in (("q", q, dq), ("k", k, dk), ("v", v, dv)):
+        num = np.zeros_like(x)
+        it = np.nditer(x, flags=["multi_index"])
+        for _ in it:
+            idx = it.multi_index
+            old = x[idx]
+            x[idx] = old + eps
+            fp = _loss(q, k, v, do, scale, kind, window, seg)
+            x[idx] = old - eps
+            fm = _loss(q, k, v, do, scale, kind, window, seg)
+            x[idx] = old
+            num[idx] = (fp - fm) / (2 * eps)
+        np.testing.assert_allclose(gx, num, rtol=1e-6, atol=1e-7, err_msg=name)
+    # Autodiff of the torch restatement agrees with the analytic brute force.
+    spec = ref.MaskSpec(sliding_window=window, segment_ids=torch.from_numpy(seg))
+    tq, tk, tv = ref.reference_mha_grads(*(torch.from_numpy(x) for x in (q, k, v, do)), spec,
+                                         softmax_scale=scale, row_block=4)
+    np.testing.assert_allclose(tq.numpy(), dq, rtol=1e-10, atol=1e-10)
+    np.testing.assert_allclose(tk.numpy(), dk, rtol=1e-10, atol=1e-10)
+    np.testing.assert_allclose(tv.numpy(), dv, rtol=1e-10, atol=1e-10)
+
+
+def test_gradient_identities():
+    b, t, h, d = 1, 12, 2, 4
+    q, k, v, do = (_rand(i, (b, t, h, d)) for i in (30, 31, 32, 33))
+    dq, dk, dv = brute.attention_bwd(q, k, v, do, scale=0.5, mask_kind=brute.MASK_CAUSAL)
+    # Softmax is shift invariant: adding c*q-independent constant to all logits of a row changes
+    # nothing, which makes sum_k dS_ik = 0; with K shifted by a common vector u the loss is constant
+    # => sum over keys of dK equals 0 projected on any direction of q-space only if mask-free.
+    dq0, dk0, dv0 = brute.attention_bwd(q, k, v, do, scale=0.5)
+    np.testing.assert_allclose(dk0.sum(axis=1), 0.0, atol=1e-12)
+    # dV column sums equal dO column sums (rows of P sum to 1).
+    np.testing.assert_allclose(dv.sum(axis=1), do.sum(axis=1), atol=1e-12)
+    np.testing.assert_allclose(dv0.sum(axis=1), do.sum(axis=1), atol=1e-12)
+    assert np.abs(dq - dq0).max() > 1e-3
+
+
+# ------------------------------------------------------------------ paged KV / decode
+
+
+def test_reconstruct_kv_loop():
+    hkv, total, page, d, b, pps = 2, 6, 4, 3, 2, 3
+    pages = torch.arange(hkv * total * page * d, dtype=torch.float32).reshape(hkv, total, page, d)
+    tables = torch.tensor([[5, 0, 2], [1, 7, 3]], dtype=torch.int32)  # 7 is out of range -> zeros
+    got = ref.reconstruct_kv(tables, pages)
+    assert got.shape == (b, pps * page, hkv, d)
+    for bi in range(b):
+        for j in range(pps * page):
+            pg = int(tables[bi, j // page])
+            for h in range(hkv):
+                want = pages[h, pg, j % page] if pg < total else torch.zeros(d)
+                assert torch.equal(got[bi, j, h], want)
+
+
+def test_paged_decode_equals_dense_and_brute():
+    b, hq, hkv, d, page, pps = 3, 4, 2, 8, 4, 5
+    q, k, v, tables, lengths = ref.paged_inputs(7, batch=b, num_heads=hq, num_kv_heads=hkv, head_dim=d,
+                                                page_size=page, pages_per_seq=pps, min_len=1,
+                                                max_len=page * pps, dtype=torch.float64)
+    got = ref.reference_decode(q, k, v, lengths, softmax_scale=0.4, page_tables=tables)
+    dense_k, dense_v = ref.reconstruct_kv(tables, k), ref.reconstruct_kv(tables, v)
+    want = ref.reference_decode(q, dense_k, dense_v, lengths, softmax_scale=0.4)
+    torch.testing.assert_close(got, want, rtol=0, atol=0)
+    bo = brute.paged_decode(q[:, 0].numpy(), k.numpy(), v.numpy(), tables.numpy(), lengths.numpy(), scale=0.4)
+    np.testing.assert_allclose(got[:, 0].numpy(), bo, rtol=1e-12, atol=1e-12)
+    # Decode == last valid row of a causal prefill over the same keys.
+    for bi in range(b):
+        n = int(lengths[bi])
+        qq = torch.zeros((1, n, hq, d), dtype=torch.float64)
+        qq[0, n - 1] = q[bi, 0]
+        full = ref.reference_mha(qq, dense_k[bi : bi + 1, :n], dense_v[bi : bi + 1, :n],
+                                 ref.MaskSpec(causal=True), softmax_scale=0.4)
+        torch.testing.assert_close(full[0, n - 1], got[bi, 0], rtol=1e-12, atol=1e-12)
+    # Sliding window in decode.
+    gw = ref.reference_decode(q, k, v, lengths, softmax_scale=0.4, page_tables=tables, sliding_window=3)
+    bw = brute.paged_decode(q[:, 0].numpy(), k.numpy(), v.numpy(), tables.numpy(), lengths.numpy(), scale=0.4, window=3)
+    np.testing.assert_allclose(gw[:, 0].numpy(), bw, rtol=1e-12, atol=1e-12)
+
+
+def test_page_permutation_invariance():
+    b, hq, hkv, d, page, pps = 2, 2, 1, 4, 2, 4
+    q, k, v, tables, lengths = ref.paged_inputs(9, batch=b, num_heads=hq, num_kv_heads=hkv, head_dim=d,
+                                                page_size=page, pages_per_seq=pps, min_len=2,
+                                                max_len=page * pps, dtype=torch.float64)
+    base = ref.reference_decode(q, k, v, lengths, page_tables=tables)
+    perm = torch.from_numpy(np.random.default_rng(0).permutation(b * pps))
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(b * pps)
+    k2, v2 = k[:, perm], v[:, perm]
+    tables2 = inv[tables.long()].to(torch.int32)
+    again = ref.reference_decode(q, k2, v2, lengths, page_tables=tables2)
+    assert torch.equal(base, again)
+
+
+def test_synthetic_generators():
+    seg = ref.packed_segment_ids(4, 8, 8192)
+    assert seg.shape == (8, 8192) and seg.dtype == torch.int32
+    assert int(seg.min()) == 1 and int(seg.max()) <= 6
+    assert bool((seg[:, 1:] >= seg[:, :-1]).all())
+    spec = ref.MaskSpec(causal=True)
+    assert ref.count_unmasked_pairs(spec, 2, 64, 64, row_block=16) == 2 * 64 * 65 // 2
+    a = ref.normal_tensor(0, (4, 4), torch.bfloat16)
+    b = ref.normal_tensor(0, (4, 4), torch.bfloat16)
+    assert torch.equal(a, b)
