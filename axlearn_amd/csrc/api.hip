@@ -1,0 +1,194 @@
+// extern "C" entry points of libaxl_attn_hip.so: argument validation, error reporting, dispatch to
+// the kernel launchers.  Nothing here allocates device memory or synchronises.
+#include <cstdarg>
+#include <cstdio>
+#include <cmath>
+
+#include "common.h"
+
+namespace axl {
+
+static thread_local char g_last_error[512] = "";
+
+int set_error(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_last_error, sizeof(g_last_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int launch_flash_fwd(const AxlFlashFwdParams& p, hipStream_t stream);
+int launch_flash_bwd(const AxlFlashBwdParams& p, hipStream_t stream);
+size_t flash_bwd_workspace_bytes(const AxlFlashBwdParams& p);
+int launch_paged_decode(const AxlPagedDecodeParams& p, hipStream_t stream);
+size_t paged_decode_workspace_bytes(const AxlPagedDecodeParams& p);
+int launch_decode(const AxlDecodeParams& p, hipStream_t stream);
+size_t decode_workspace_bytes(const AxlDecodeParams& p);
+
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+static bool strides_ok(const AxlStrides& s, int elem_bytes) {
+  // 16-byte vector loads along head_dim need every row start 16-byte aligned.
+  const int64_t m = 16 / elem_bytes;
+  return s.batch % m == 0 && s.seq % m == 0 && s.head % m == 0;
+}
+
+// Shape rules shared by forward and backward; mirrors BaseFlashAttention.is_supported
+// (axlearn/common/flash_attention/common.py:232-275) for the "makes no sense" cases and
+// PallasGPUFlashAttention.is_supported (gpu_attention.py:939-961) for the unsupported ones.
+static int check_flash_shapes(const char* who, int batch, int q_len, int kv_len, int hq, int hkv,
+                              int d, int dtype, int mask_kind, int window, float scale,
+                              const int32_t* seg) {
+  if (batch <= 0 || q_len <= 0 || kv_len <= 0 || hq <= 0 || hkv <= 0 || d <= 0)
+    return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: non-positive dimension", who);
+  if (hq % hkv != 0)
+    return set_error(AXL_ERR_INVALID_ARGUMENT,
+                     "%s: num_q_heads %d is not divisible by num_kv_heads %d", who, hq, hkv);
+  if (!(scale > 0.f) || !std::isfinite(scale))
+    return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: softmax_scale must be finite and > 0", who);
+  if (dtype != AXL_BF16 && dtype != AXL_F32)
+    return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: unknown dtype %d", who, dtype);
+  if (mask_kind < AXL_MASK_NONE || mask_kind > AXL_MASK_SLIDING_WINDOW)
+    return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: unknown mask_kind %d", who, mask_kind);
+  if (mask_kind == AXL_MASK_SLIDING_WINDOW && window < 0)
+    return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: sliding_window must be >= 0", who);
+  if (seg && q_len != kv_len)
+    return set_error(AXL_ERR_INVALID_ARGUMENT,
+                     "%s: segment_ids need q_len == kv_len (got %d vs %d)", who, q_len, kv_len);
+  if (d != 64 && d != 128)
+    return set_error(AXL_ERR_UNSUPPORTED, "%s: head_dim %d (supported: 64, 128)", who, d);
+  if (q_len % 128 != 0 || kv_len % 128 != 0)
+    return set_error(AXL_ERR_UNSUPPORTED, "%s: q_len %d / kv_len %d not divisible by 128", who,
+                     q_len, kv_len);
+  return AXL_OK;
+}
+
+}  // namespace axl
+
+using namespace axl;
+
+extern "C" {
+
+const char* axl_last_error(void) { return g_last_error; }
+
+int axl_abi_version(void) { return AXL_ATTN_ABI_VERSION; }
+
+int axl_flash_fwd(const AxlFlashFwdParams* p, void* stream) {
+  if (!p) return set_error(AXL_ERR_INVALID_ARGUMENT, "axl_flash_fwd: params is NULL");
+  int rc = check_flash_shapes("axl_flash_fwd", p->batch, p->q_len, p->kv_len, p->num_q_heads,
+                              p->num_kv_heads, p->head_dim, p->dtype, p->mask_kind,
+                              p->sliding_window, p->softmax_scale, p->segment_ids);
+  if (rc != AXL_OK) return rc;
+  if (!p->q || !p->k || !p->v || !p->out)
+    return set_error(AXL_ERR_INVALID_ARGUMENT, "axl_flash_fwd: NULL tensor pointer");
+  const int eb = p->dtype == AXL_BF16 ? 2 : 4;
+  if (!aligned16(p->q) || !aligned16(p->k) || !aligned16(p->v) || !aligned16(p->out) ||
+      !strides_ok(p->q_strides, eb) || !strides_ok(p->k_strides, eb) ||
+      !strides_ok(p->v_strides, eb) || !strides_ok(p->out_strides, eb))
+    return set_error(AXL_ERR_UNSUPPORTED, "axl_flash_fwd: tensors must be 16-byte aligned rows");
+  if (p->segment_ids && !aligned16(p->segment_ids))
+    return set_error(AXL_ERR_UNSUPPORTED, "axl_flash_fwd: segment_ids must be 16-byte aligned");
+  return launch_flash_fwd(*p, (hipStream_t)stream);
+}
+
+size_t axl_flash_bwd_workspace_bytes(const AxlFlashBwdParams* p) {
+  if (!p) return 0;
+  return flash_bwd_workspace_bytes(*p);
+}
+
+int axl_flash_bwd(const AxlFlashBwdParams* p, void* stream) {
+  if (!p) return set_error(AXL_ERR_INVALID_ARGUMENT, "axl_flash_bwd: params is NULL");
+  int rc = check_flash_shapes("axl_flash_bwd", p->batch, p->q_len, p->kv_len, p->num_q_heads,
+                              p->num_kv_heads, p->head_dim, p->dtype, p->mask_kind,
+                              p->sliding_window, p->softmax_scale, p->segment_ids);
+  if (rc != AXL_OK) return rc;
+  if (!p->q || !p->k || !p->v || !p->out || !p->d_out || !p->lse || !p->dq || !p->dk || !p->dv)
+    return set_error(AXL_ERR_INVALID_ARGUMENT, "axl_flash_bwd: NULL tensor pointer");
+  const int eb = p->dtype == AXL_BF16 ? 2 : 4;
+  const void* ptrs[] = {p->q, p->k, p->v, p->out, p->d_out, p->dq, p->dk, p->dv};
+  for (const void* x : ptrs)
+    if (!aligned16(x))
+      return set_error(AXL_ERR_UNSUPPORTED, "axl_flash_bwd: tensors must be 16-byte aligned");
+  const AxlStrides* ss[] = {&p->q_strides,     &p->k_strides,  &p->v_strides,  &p->out_strides,
+                            &p->d_out_strides, &p->dq_strides, &p->dk_strides, &p->dv_strides};
+  for (const AxlStrides* s : ss)
+    if (!strides_ok(*s, eb))
+      return set_error(AXL_ERR_UNSUPPORTED, "axl_flash_bwd: rows must be 16-byte aligned");
+  if (p->segment_ids && !aligned16(p->segment_ids))
+    return set_error(AXL_ERR_UNSUPPORTED, "axl_flash_bwd: segment_ids must be 16-byte aligned");
+  const size_t need = flash_bwd_workspace_bytes(*p);
+  if (!p->workspace || p->workspace_bytes < need || !aligned16(p->workspace))
+    return set_error(AXL_ERR_WORKSPACE, "axl_flash_bwd: workspace needs %zu bytes, got %zu", need,
+                     p->workspace ? p->workspace_bytes : (size_t)0);
+  return launch_flash_bwd(*p, (hipStream_t)stream);
+}
+
+static int check_decode_common(const char* who, int batch, int hq, int hkv, int d, int dtype,
+                               float scale) {
+  if (batch <= 0 || hq <= 0 || hkv <= 0 || d <= 0)
+    return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: non-positive dimension", who);
+  if (hq % hkv != 0)
+    return set_error(AXL_ERR_INVALID_ARGUMENT,
+                     "%s: num_q_heads %d is not divisible by num_kv_heads %d", who, hq, hkv);
+  if (!(scale > 0.f) || !std::isfinite(scale))
+    return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: softmax_scale must be finite and > 0", who);
+  if (dtype != AXL_BF16)
+    return set_error(AXL_ERR_UNSUPPORTED, "%s: only bf16 is supported", who);
+  if (d != 128 && d != 64)
+    return set_error(AXL_ERR_UNSUPPORTED, "%s: head_dim %d (supported: 64, 128)", who, d);
+  if (hq / hkv > 16)
+    return set_error(AXL_ERR_UNSUPPORTED, "%s: more than 16 query heads per kv head", who);
+  return AXL_OK;
+}
+
+size_t axl_paged_decode_workspace_bytes(const AxlPagedDecodeParams* p) {
+  if (!p) return 0;
+  return paged_decode_workspace_bytes(*p);
+}
+
+int axl_paged_decode(const AxlPagedDecodeParams* p, void* stream) {
+  if (!p) return set_error(AXL_ERR_INVALID_ARGUMENT, "axl_paged_decode: params is NULL");
+  int rc = check_decode_common("axl_paged_decode", p->batch, p->num_q_heads, p->num_kv_heads,
+                               p->head_dim, p->dtype, p->softmax_scale);
+  if (rc != AXL_OK) return rc;
+  if (p->num_pages <= 0 || p->page_size <= 0 || p->pages_per_seq <= 0)
+    return set_error(AXL_ERR_INVALID_ARGUMENT, "axl_paged_decode: non-positive page geometry");
+  if (!p->q || !p->k_pages || !p->v_pages || !p->page_tables || !p->lengths || !p->out)
+    return set_error(AXL_ERR_INVALID_ARGUMENT, "axl_paged_decode: NULL tensor pointer");
+  if (p->page_size != 16)
+    return set_error(AXL_ERR_UNSUPPORTED, "axl_paged_decode: page_size %d (supported: 16)",
+                     p->page_size);
+  if (!aligned16(p->q) || !aligned16(p->k_pages) || !aligned16(p->v_pages) || !aligned16(p->out))
+    return set_error(AXL_ERR_UNSUPPORTED, "axl_paged_decode: tensors must be 16-byte aligned");
+  const size_t need = paged_decode_workspace_bytes(*p);
+  if (!p->workspace || p->workspace_bytes < need || !aligned16(p->workspace))
+    return set_error(AXL_ERR_WORKSPACE, "axl_paged_decode: workspace needs %zu bytes, got %zu",
+                     need, p->workspace ? p->workspace_bytes : (size_t)0);
+  return launch_paged_decode(*p, (hipStream_t)stream);
+}
+
+size_t axl_decode_workspace_bytes(const AxlDecodeParams* p) {
+  if (!p) return 0;
+  return decode_workspace_bytes(*p);
+}
+
+int axl_decode(const AxlDecodeParams* p, void* stream) {
+  if (!p) return set_error(AXL_ERR_INVALID_ARGUMENT, "axl_decode: params is NULL");
+  int rc = check_decode_common("axl_decode", p->batch, p->num_q_heads, p->num_kv_heads,
+                               p->head_dim, p->dtype, p->softmax_scale);
+  if (rc != AXL_OK) return rc;
+  if (p->kv_len <= 0) return set_error(AXL_ERR_INVALID_ARGUMENT, "axl_decode: kv_len <= 0");
+  if (!p->q || !p->k || !p->v || !p->lengths || !p->out)
+    return set_error(AXL_ERR_INVALID_ARGUMENT, "axl_decode: NULL tensor pointer");
+  if (!aligned16(p->q) || !aligned16(p->k) || !aligned16(p->v) || !aligned16(p->out) ||
+      !strides_ok(p->k_strides, 2) || !strides_ok(p->v_strides, 2))
+    return set_error(AXL_ERR_UNSUPPORTED, "axl_decode: tensors must be 16-byte aligned rows");
+  const size_t need = decode_workspace_bytes(*p);
+  if (!p->workspace || p->workspace_bytes < need || !aligned16(p->workspace))
+    return set_error(AXL_ERR_WORKSPACE, "axl_decode: workspace needs %zu bytes, got %zu", need,
+                     p->workspace ? p->workspace_bytes : (size_t)0);
+  return launch_decode(*p, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,79 @@
+// Shared device helpers for the CDNA4 (gfx950) attention kernels: MFMA operand types, LDS address
+// casts, bf16 packing and the softmax constants.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/axl_attn.h"
+
+namespace axl {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float floatx4;
+typedef __attribute__((__vector_size__(2 * sizeof(float)))) float floatx2;
+typedef __attribute__((__vector_size__(4 * sizeof(short)))) short shortx4;
+typedef __attribute__((__vector_size__(8 * sizeof(short)))) short shortx8;
+typedef __attribute__((__vector_size__(4 * sizeof(int)))) int intx4;
+
+#define AXL_LDS(T, p) ((__attribute__((address_space(3))) T*)(p))
+
+// Masked logits use the reference's finite sentinel (axlearn/common/attention_bias.py:43), never
+// -inf, so that exp(masked - max) underflows to exactly 0 without producing NaN on rows whose
+// first tiles are fully masked.
+constexpr float kNegInf = -1e15f;
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+__device__ __forceinline__ bf16x2 pack_bf16(float a, float b) {
+  floatx2 v = {a, b};
+  return __builtin_convertvector(v, bf16x2);
+}
+
+// Eight fp32 -> one MFMA bf16 operand (round to nearest even, v_cvt_pk_bf16_f32).
+__device__ __forceinline__ bf16x8 pack_bf16x8(float a0, float a1, float a2, float a3, float a4,
+                                              float a5, float a6, float a7) {
+  union {
+    bf16x8 v;
+    bf16x2 p[4];
+  } u;
+  u.p[0] = pack_bf16(a0, a1);
+  u.p[1] = pack_bf16(a2, a3);
+  u.p[2] = pack_bf16(a4, a5);
+  u.p[3] = pack_bf16(a6, a7);
+  return u.v;
+}
+
+// Transposing LDS read (ds_read_b64_tr_b16).  Within each group of 16 lanes, lane j supplies the
+// address of 4 contiguous 16-bit elements; lane i receives, as element e, element (i % 4) of the
+// data addressed by lane 4*e + i/4.  With lane j pointing at row (j / 4), columns 4*(j % 4)..+3 of
+// a row-major tile, lane i ends up with column i of rows 0..3: a 4x16 -> 16x4 transpose.
+__device__ __forceinline__ shortx4 lds_read_tr16(const void* lds_addr) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16(AXL_LDS(shortx4, lds_addr));
+}
+
+__device__ __forceinline__ float xor32_max(float x) {
+  return fmaxf(x, __shfl_xor(x, 32, 64));
+}
+__device__ __forceinline__ float xor32_sum(float x) { return x + __shfl_xor(x, 32, 64); }
+
+// Row index permutation that swaps bits 2 and 3.  Feeding MFMA 32x32 A-operand lane m with tile
+// row pi(m) makes accumulator register r of lane group g hold tile row 16*(r/8) + 8*g + (r%8), so
+// registers 8t..8t+7 are exactly the 8 consecutive rows the next MFMA wants as its K-slice.
+__device__ __forceinline__ int swap_bits_2_3(int m) {
+  return (m & ~12) | ((m & 4) << 1) | ((m & 8) >> 1);
+}
+
+struct Strides3 {
+  int64_t b, s, h;
+};
+
+int set_error(int code, const char* fmt, ...);
+
+}  // namespace axl

@@ -1,0 +1,469 @@
+// Flash-attention forward for gfx950.
+//
+// Replaces axlearn/common/flash_attention/gpu_attention.py:114-243 (`_mha_forward_kernel`) and its
+// launcher (:293-425).  Same mathematics (FlashAttention-2 online softmax, fp32 statistics, P
+// rounded to the value dtype before PV, out = acc / l, lse = m + log l) on a different machine
+// mapping:
+//
+//   * one workgroup = 4 wavefronts = 128 query rows of one (batch, query head); each wavefront owns
+//     32 query rows and keeps their Q fragments in registers for the whole kernel;
+//   * K/V tiles of 64 keys are staged through LDS (double buffered) and shared by the 4 wavefronts;
+//   * the logits are produced TRANSPOSED, S^T = K Q^T, with v_mfma_f32_32x32x16_bf16: a lane then
+//     owns one query column and 16 keys per 32-key sub-tile, so the softmax row statistics are
+//     in-register reductions plus a single exchange with lane^32, and exp(S^T) is already in the
+//     B-operand layout of the second MFMA, O^T += V^T P^T: P never touches LDS;
+//   * V^T fragments come from the row-major V tile through the transposing LDS read
+//     (ds_read_b64_tr_b16);
+//   * GQA reads the shared kv head directly (no repeated KV in HBM), and workgroups that share a kv
+//     head are placed on the same XCD so its L2 serves the re-reads.
+#include "common.h"
+
+namespace axl {
+
+struct FwdArgs {
+  const void* q;
+  const void* k;
+  const void* v;
+  void* out;
+  float* lse;
+  const int32_t* seg;
+  Strides3 qs, ks, vs, os;
+  int B, T, S, Hq, Hkv;
+  int mask_kind, window, q_off;
+  float scale;
+};
+
+// Decodes blockIdx.x into (query block, batch, query head).  Heaviest query blocks (most visible
+// keys under a causal mask) are issued first; when the (batch, kv head) pairs divide evenly over
+// the 8 XCDs, all workgroups of a pair run on one XCD (workgroup i is dispatched to XCD i % 8).
+__device__ __forceinline__ void decode_block(int bid, int nqb, int B, int Hq, int Hkv, int& qb,
+                                             int& b, int& h) {
+  const int G = Hq / Hkv;
+  const int npairs = B * Hkv;
+  if (npairs % 8 == 0) {
+    const int xcd = bid & 7, slot = bid >> 3;
+    const int per_qb = (npairs >> 3) * G;
+    const int qb_rev = slot / per_qb, rem = slot % per_qb;
+    const int pair = xcd + 8 * (rem / G);
+    qb = nqb - 1 - qb_rev;
+    b = pair / Hkv;
+    h = (pair % Hkv) * G + rem % G;
+  } else {
+    const int per_qb = B * Hq;
+    const int qb_rev = bid / per_qb, rem = bid % per_qb;
+    qb = nqb - 1 - qb_rev;
+    b = rem / Hq;
+    h = rem % Hq;
+  }
+}
+
+template <int D>
+struct FwdTile {
+  static constexpr int BQ = 128;              // query rows per workgroup
+  static constexpr int BK = 64;               // keys per LDS tile
+  static constexpr int KSTRIDE = D * 2 + 16;  // bytes per K row in LDS (16 B pad: b128 reads)
+  static constexpr int VSTRIDE = D * 2 + 64;  // bytes per V row in LDS (64 B pad: tr reads)
+  static constexpr int KBYTES = BK * KSTRIDE;
+  static constexpr int VBYTES = BK * VSTRIDE;
+  static constexpr int CHUNKS = BK * D * 2 / 16 / 256;  // 16-byte chunks per thread per tile
+  static constexpr int LDS_BYTES = 2 * (KBYTES + VBYTES);
+};
+
+template <int D>
+__global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
+  using Tile = FwdTile<D>;
+  constexpr int KK = D / 16;  // MFMA k-steps over head_dim
+  constexpr int DT = D / 32;  // 32-row output tiles over head_dim
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  char* const k_lds = smem;
+  char* const v_lds = smem + 2 * Tile::KBYTES;
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+  int qb, b, h;
+  decode_block(blockIdx.x, a.T / Tile::BQ, a.B, a.Hq, a.Hkv, qb, b, h);
+  const int hk = h / (a.Hq / a.Hkv);
+  const int q0_wg = qb * Tile::BQ;
+  const int q0 = q0_wg + wave * 32;
+
+  const __bf16* qp = (const __bf16*)a.q + b * a.qs.b + (int64_t)(q0 + l32) * a.qs.s + h * a.qs.h;
+  const __bf16* kp = (const __bf16*)a.k + b * a.ks.b + hk * a.ks.h;
+  const __bf16* vp = (const __bf16*)a.v + b * a.vs.b + hk * a.vs.h;
+
+  // Q fragments: B operand of S^T = K Q^T; lane (query l32, k-group g) holds d = 16kk + 8g .. +7.
+  bf16x8 qf[KK];
+#pragma unroll
+  for (int kk = 0; kk < KK; kk++) qf[kk] = *(const bf16x8*)(qp + 16 * kk + 8 * g);
+
+  // Visible key range of this workgroup.
+  int k_begin = 0, k_end = a.S;
+  if (a.mask_kind != AXL_MASK_NONE) {
+    k_end = min(a.S, q0_wg + Tile::BQ + a.q_off);
+    if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) k_begin = max(0, q0_wg + a.q_off - a.window);
+  }
+  const int t_begin = k_begin / Tile::BK;
+  const int t_end = (k_end + Tile::BK - 1) / Tile::BK;
+
+  const int qpos = q0 + l32 + a.q_off;       // this lane's query position
+  const int qpos_min = q0 + a.q_off, qpos_max = q0 + 31 + a.q_off;  // of the wavefront
+  const int seg_q = a.seg ? a.seg[(int64_t)b * a.T + q0 + l32] : 0;
+  const int32_t* seg_k = a.seg ? a.seg + (int64_t)b * a.T : nullptr;
+
+  floatx16 o[DT];
+#pragma unroll
+  for (int i = 0; i < DT; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) o[i][r] = 0.f;
+  float m_run = kNegInf;  // running row max of the raw (unscaled) logits
+  float l_run = 0.f;      // this lane's share of the running row sum (lanes l and l^32 split it)
+  const float c = a.scale * kLog2e;
+
+  // Global -> LDS staging: thread handles chunks tid + 256*i.
+  uint4 kreg[Tile::CHUNKS], vreg[Tile::CHUNKS];
+  auto load_tile = [&](int t) {
+    const int k0 = t * Tile::BK;
+#pragma unroll
+    for (int i = 0; i < Tile::CHUNKS; i++) {
+      const int cidx = tid + 256 * i;
+      const int row = cidx / (D / 8), cc = cidx % (D / 8);
+      kreg[i] = *(const uint4*)(kp + (int64_t)(k0 + row) * a.ks.s + cc * 8);
+      vreg[i] = *(const uint4*)(vp + (int64_t)(k0 + row) * a.vs.s + cc * 8);
+    }
+  };
+  auto store_tile = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < Tile::CHUNKS; i++) {
+      const int cidx = tid + 256 * i;
+      const int row = cidx / (D / 8), cc = cidx % (D / 8);
+      *(uint4*)(k_lds + buf * Tile::KBYTES + row * Tile::KSTRIDE + cc * 16) = kreg[i];
+      *(uint4*)(v_lds + buf * Tile::VBYTES + row * Tile::VSTRIDE + cc * 16) = vreg[i];
+    }
+  };
+
+  if (t_begin < t_end) {
+    load_tile(t_begin);
+    store_tile(0);
+  }
+  __syncthreads();
+
+  // Per-lane LDS read offsets.
+  const int k_row_off = swap_bits_2_3(l32) * Tile::KSTRIDE + g * 16;
+  const int j16 = lane & 15, half = (lane >> 4) & 1;
+  const int v_lane_off = (8 * g + (j16 >> 2)) * Tile::VSTRIDE + (16 * half + 4 * (j16 & 3)) * 2;
+
+  for (int t = t_begin; t < t_end; t++) {
+    const int buf = (t - t_begin) & 1;
+    const bool has_next = t + 1 < t_end;
+    if (has_next) load_tile(t + 1);
+
+    const int k0 = t * Tile::BK;
+    bool skip = false;
+    bool need_mask = false;
+    if (a.mask_kind != AXL_MASK_NONE) {
+      skip = k0 > qpos_max;
+      need_mask = k0 + Tile::BK - 1 > qpos_min;
+      if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) {
+        skip = skip || (qpos_min - (k0 + Tile::BK - 1) > a.window);
+        need_mask = need_mask || (qpos_max - k0 > a.window);
+      }
+    }
+    if (!skip) {
+      const char* kt = k_lds + buf * Tile::KBYTES;
+      const char* vt = v_lds + buf * Tile::VBYTES;
+      floatx16 s[2];
+#pragma unroll
+      for (int ks = 0; ks < 2; ks++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) s[ks][r] = 0.f;
+        const char* ka = kt + ks * 32 * Tile::KSTRIDE + k_row_off;
+#pragma unroll
+        for (int kk = 0; kk < KK; kk++) {
+          const bf16x8 kf = *(const bf16x8*)(ka + kk * 32);
+          s[ks] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kk], s[ks], 0, 0, 0);
+        }
+      }
+      // Register r of sub-tile ks in lane group g is key k0 + 32ks + 16(r/8) + 8g + (r%8).
+      if (need_mask) {
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++) {
+          const int diff0 = qpos - (k0 + 32 * ks + 8 * g);  // qpos - kpos for r == 0
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            const int diff = diff0 - (16 * (r / 8) + (r % 8));
+            bool keep = diff >= 0;
+            if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) keep = keep && diff <= a.window;
+            s[ks][r] = keep ? s[ks][r] : kNegInf;
+          }
+        }
+      }
+      if (seg_k) {
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++) {
+#pragma unroll
+          for (int t8 = 0; t8 < 2; t8++) {
+            const int4* sp = (const int4*)(seg_k + k0 + 32 * ks + 16 * t8 + 8 * g);
+            const int4 s0 = sp[0], s1 = sp[1];
+            const int ids[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+              s[ks][8 * t8 + j] = (ids[j] == seg_q) ? s[ks][8 * t8 + j] : kNegInf;
+          }
+        }
+      }
+      float mx = m_run;
+#pragma unroll
+      for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[ks][r]);
+      mx = xor32_max(mx);
+      const float mc = mx * c;
+      const float corr = fast_exp2(m_run * c - mc);
+      m_run = mx;
+      float lsum = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const float p = fast_exp2(__builtin_fmaf(s[ks][r], c, -mc));
+          s[ks][r] = p;
+          lsum += p;
+        }
+      l_run = l_run * corr + lsum;
+#pragma unroll
+      for (int i = 0; i < DT; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[i][r] *= corr;
+      // O^T += V^T P^T.
+#pragma unroll
+      for (int ks = 0; ks < 2; ks++) {
+#pragma unroll
+        for (int t8 = 0; t8 < 2; t8++) {
+          const bf16x8 pb = pack_bf16x8(s[ks][8 * t8 + 0], s[ks][8 * t8 + 1], s[ks][8 * t8 + 2],
+                                        s[ks][8 * t8 + 3], s[ks][8 * t8 + 4], s[ks][8 * t8 + 5],
+                                        s[ks][8 * t8 + 6], s[ks][8 * t8 + 7]);
+          const char* va = vt + (32 * ks + 16 * t8) * Tile::VSTRIDE + v_lane_off;
+#pragma unroll
+          for (int dt = 0; dt < DT; dt++) {
+            union {
+              bf16x8 v;
+              shortx4 hlf[2];
+            } vf;
+            vf.hlf[0] = lds_read_tr16(va + dt * 64);
+            vf.hlf[1] = lds_read_tr16(va + dt * 64 + 4 * Tile::VSTRIDE);
+            o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pb, o[dt], 0, 0, 0);
+          }
+        }
+      }
+    }
+    if (has_next) store_tile(buf ^ 1);
+    __syncthreads();
+  }
+
+  // Epilogue: out = acc / l ; lse = m*scale + ln(l).
+  const float l_tot = xor32_sum(l_run);
+  const float inv_l = 1.0f / l_tot;
+  __bf16* op = (__bf16*)a.out + b * a.os.b + (int64_t)(q0 + l32) * a.os.s + h * a.os.h;
+#pragma unroll
+  for (int dt = 0; dt < DT; dt++) {
+#pragma unroll
+    for (int rq = 0; rq < 4; rq++) {
+      union {
+        bf16x2 p[2];
+        uint2 u;
+      } w;
+      w.p[0] = pack_bf16(o[dt][4 * rq + 0] * inv_l, o[dt][4 * rq + 1] * inv_l);
+      w.p[1] = pack_bf16(o[dt][4 * rq + 2] * inv_l, o[dt][4 * rq + 3] * inv_l);
+      *(uint2*)(op + 32 * dt + 8 * rq + 4 * g) = w.u;
+    }
+  }
+  if (a.lse && g == 0) {
+    a.lse[((int64_t)b * a.Hq + h) * a.T + q0 + l32] = (m_run * c + fast_log2(l_tot)) * kLn2;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// fp32 forward: same mapping with v_mfma_f32_32x32x2_f32 (true fp32 multiply-accumulate), K and V
+// staged in LDS as fp32; exp via the accurate libm path.  Each wavefront owns 32 query rows and a
+// 32-key tile per step.
+// ---------------------------------------------------------------------------------------------
+template <int D>
+struct FwdTileF32 {
+  static constexpr int BQ = 128;
+  static constexpr int BK = 32;
+  static constexpr int KSTRIDE = D * 4 + 4;   // bytes; +1 word: lanes read a column of rows
+  static constexpr int VSTRIDE = D * 4;       // lanes read consecutive d of one row: no pad needed
+  static constexpr int KBYTES = BK * KSTRIDE;
+  static constexpr int VBYTES = BK * VSTRIDE;
+  static constexpr int QSTRIDE = D * 4 + 4;
+  static constexpr int QBYTES = BQ * QSTRIDE;
+  static constexpr int LDS_BYTES = QBYTES + KBYTES + VBYTES;
+};
+
+template <int D>
+__global__ __launch_bounds__(256) void flash_fwd_f32_kernel(const FwdArgs a) {
+  using Tile = FwdTileF32<D>;
+  constexpr int DT = D / 32;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  float* const q_lds = (float*)smem;
+  float* const k_lds = (float*)(smem + Tile::QBYTES);
+  float* const v_lds = (float*)(smem + Tile::QBYTES + Tile::KBYTES);
+  constexpr int QS = Tile::QSTRIDE / 4, KS = Tile::KSTRIDE / 4, VS = Tile::VSTRIDE / 4;
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+  int qb, b, h;
+  decode_block(blockIdx.x, a.T / Tile::BQ, a.B, a.Hq, a.Hkv, qb, b, h);
+  const int hk = h / (a.Hq / a.Hkv);
+  const int q0_wg = qb * Tile::BQ;
+  const int q0 = q0_wg + wave * 32;
+
+  const float* qg = (const float*)a.q + b * a.qs.b + (int64_t)q0_wg * a.qs.s + h * a.qs.h;
+  const float* kp = (const float*)a.k + b * a.ks.b + hk * a.ks.h;
+  const float* vp = (const float*)a.v + b * a.vs.b + hk * a.vs.h;
+
+  // Stage the 128 x D query block (fp32) in LDS once.
+  for (int i = tid; i < Tile::BQ * (D / 4); i += 256) {
+    const int row = i / (D / 4), c4 = i % (D / 4);
+    const float4 x = *(const float4*)(qg + (int64_t)row * a.qs.s + c4 * 4);
+    float* dst = q_lds + row * QS + c4 * 4;
+    dst[0] = x.x; dst[1] = x.y; dst[2] = x.z; dst[3] = x.w;
+  }
+
+  int k_begin = 0, k_end = a.S;
+  if (a.mask_kind != AXL_MASK_NONE) {
+    k_end = min(a.S, q0_wg + Tile::BQ + a.q_off);
+    if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) k_begin = max(0, q0_wg + a.q_off - a.window);
+  }
+  const int t_begin = k_begin / Tile::BK;
+  const int t_end = (k_end + Tile::BK - 1) / Tile::BK;
+  const int qpos = q0 + l32 + a.q_off;
+  const int qpos_min = q0 + a.q_off, qpos_max = q0 + 31 + a.q_off;
+  const int seg_q = a.seg ? a.seg[(int64_t)b * a.T + q0 + l32] : 0;
+  const int32_t* seg_k = a.seg ? a.seg + (int64_t)b * a.T : nullptr;
+
+  floatx16 o[DT];
+#pragma unroll
+  for (int i = 0; i < DT; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) o[i][r] = 0.f;
+  float m_run = kNegInf, l_run = 0.f;
+  const float* q_row = q_lds + (wave * 32 + l32) * QS;
+
+  for (int t = t_begin; t < t_end; t++) {
+    const int k0 = t * Tile::BK;
+    __syncthreads();  // previous tile fully consumed (and Q staged on the first pass)
+    for (int i = tid; i < Tile::BK * (D / 4); i += 256) {
+      const int row = i / (D / 4), c4 = i % (D / 4);
+      const float4 x = *(const float4*)(kp + (int64_t)(k0 + row) * a.ks.s + c4 * 4);
+      const float4 y = *(const float4*)(vp + (int64_t)(k0 + row) * a.vs.s + c4 * 4);
+      float* kd = k_lds + row * KS + c4 * 4;
+      kd[0] = x.x; kd[1] = x.y; kd[2] = x.z; kd[3] = x.w;
+      *(float4*)(v_lds + row * VS + c4 * 4) = y;
+    }
+    __syncthreads();
+    bool skip = false;
+    if (a.mask_kind != AXL_MASK_NONE) {
+      skip = k0 > qpos_max;
+      if (a.mask_kind == AXL_MASK_SLIDING_WINDOW)
+        skip = skip || (qpos_min - (k0 + Tile::BK - 1) > a.window);
+    }
+    if (skip) continue;
+    // S^T[key][q]: A = K (lane: key row l32, k index g), B = Q^T (lane: query l32, k index g).
+    floatx16 s;
+#pragma unroll
+    for (int r = 0; r < 16; r++) s[r] = 0.f;
+    const float* k_row = k_lds + l32 * KS;
+#pragma unroll 8
+    for (int d2 = 0; d2 < D / 2; d2++) {
+      s = __builtin_amdgcn_mfma_f32_32x32x2f32(k_row[2 * d2 + g], q_row[2 * d2 + g], s, 0, 0, 0);
+    }
+    // Register r of lane group g is key k0 + 8(r/4) + 4g + (r%4).
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int kpos = k0 + 8 * (r / 4) + 4 * g + (r % 4);
+      bool keep = true;
+      if (a.mask_kind != AXL_MASK_NONE) {
+        const int diff = qpos - kpos;
+        keep = diff >= 0;
+        if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) keep = keep && diff <= a.window;
+      }
+      if (seg_k) keep = keep && (seg_k[kpos] == seg_q);
+      s[r] = keep ? s[r] * a.scale : kNegInf;
+    }
+    float mx = m_run;
+#pragma unroll
+    for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[r]);
+    mx = xor32_max(mx);
+    const float corr = expf(m_run - mx);
+    m_run = mx;
+    float lsum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      s[r] = expf(s[r] - mx);
+      lsum += s[r];
+    }
+    l_run = l_run * corr + lsum;
+#pragma unroll
+    for (int i = 0; i < DT; i++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) o[i][r] *= corr;
+    // O^T[d][q] += V^T[d][key] P^T[key][q]; one key per lane group per MFMA: group g supplies
+    // register r, i.e. key 8(r/4) + 4g + (r%4).
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const float* v_row = v_lds + (8 * (r / 4) + 4 * g + (r % 4)) * VS + l32;
+#pragma unroll
+      for (int dt = 0; dt < DT; dt++)
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(v_row[32 * dt], s[r], o[dt], 0, 0, 0);
+    }
+  }
+
+  const float l_tot = xor32_sum(l_run);
+  const float inv_l = 1.0f / l_tot;
+  float* op = (float*)a.out + b * a.os.b + (int64_t)(q0 + l32) * a.os.s + h * a.os.h;
+#pragma unroll
+  for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+    for (int rq = 0; rq < 4; rq++) {
+      float4 w = {o[dt][4 * rq + 0] * inv_l, o[dt][4 * rq + 1] * inv_l, o[dt][4 * rq + 2] * inv_l,
+                  o[dt][4 * rq + 3] * inv_l};
+      *(float4*)(op + 32 * dt + 8 * rq + 4 * g) = w;
+    }
+  if (a.lse && g == 0) a.lse[((int64_t)b * a.Hq + h) * a.T + q0 + l32] = m_run + logf(l_tot);
+}
+
+static Strides3 to_s3(const AxlStrides& s) { return Strides3{s.batch, s.seq, s.head}; }
+
+int launch_flash_fwd(const AxlFlashFwdParams& p, hipStream_t stream) {
+  FwdArgs a;
+  a.q = p.q; a.k = p.k; a.v = p.v; a.out = p.out; a.lse = p.lse; a.seg = p.segment_ids;
+  a.qs = to_s3(p.q_strides); a.ks = to_s3(p.k_strides); a.vs = to_s3(p.v_strides);
+  a.os = to_s3(p.out_strides);
+  a.B = p.batch; a.T = p.q_len; a.S = p.kv_len; a.Hq = p.num_q_heads; a.Hkv = p.num_kv_heads;
+  a.mask_kind = p.mask_kind; a.window = p.sliding_window; a.q_off = p.q_pos_offset;
+  a.scale = p.softmax_scale;
+  const int grid = (p.q_len / 128) * p.batch * p.num_q_heads;
+  hipError_t err = hipSuccess;
+#define AXL_LAUNCH_FWD(KERNEL, TILE)                                                            \
+  do {                                                                                          \
+    err = hipFuncSetAttribute((const void*)KERNEL, hipFuncAttributeMaxDynamicSharedMemorySize,  \
+                              TILE::LDS_BYTES);                                                 \
+    if (err == hipSuccess) {                                                                    \
+      hipLaunchKernelGGL(KERNEL, dim3(grid), dim3(256), TILE::LDS_BYTES, stream, a);            \
+      err = hipGetLastError();                                                                  \
+    }                                                                                           \
+  } while (0)
+  if (p.dtype == AXL_BF16) {
+    if (p.head_dim == 128) AXL_LAUNCH_FWD(flash_fwd_bf16_kernel<128>, FwdTile<128>);
+    else AXL_LAUNCH_FWD(flash_fwd_bf16_kernel<64>, FwdTile<64>);
+  } else {
+    if (p.head_dim == 128) AXL_LAUNCH_FWD(flash_fwd_f32_kernel<128>, FwdTileF32<128>);
+    else AXL_LAUNCH_FWD(flash_fwd_f32_kernel<64>, FwdTileF32<64>);
+  }
+#undef AXL_LAUNCH_FWD
+  if (err != hipSuccess)
+    return set_error(AXL_ERR_LAUNCH, "axl_flash_fwd: launch failed: %s", hipGetErrorString(err));
+  return AXL_OK;
+}
+
+}  // namespace axl

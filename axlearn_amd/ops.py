@@ -1,0 +1,203 @@
+"""Tensor-level wrappers over the C ABI: allocate outputs/workspace with torch, pass raw pointers.
+
+These are the functions the `BaseFlashAttention`-shaped classes in `axlearn_amd.flash_attention`
+call. Inputs must be CUDA(ROCm) tensors; torch is used for device memory and streams only.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from axlearn_amd import _lib
+from axlearn_amd._lib import (
+    MASK_CAUSAL,
+    MASK_NONE,
+    MASK_SLIDING_WINDOW,
+    AxlDecodeParams,
+    AxlError,
+    AxlFlashBwdParams,
+    AxlFlashFwdParams,
+    AxlPagedDecodeParams,
+)
+
+__all__ = [
+    "MASK_NONE",
+    "MASK_CAUSAL",
+    "MASK_SLIDING_WINDOW",
+    "flash_fwd",
+    "flash_bwd",
+    "paged_decode",
+    "decode",
+]
+
+
+def _require_cuda(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise AxlError(_lib.AXL_ERR_INVALID_ARGUMENT, "all tensors must live on the GPU")
+
+
+def _seg(segment_ids: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    if segment_ids is None:
+        return None
+    if segment_ids.dtype != torch.int32 or not segment_ids.is_contiguous():
+        segment_ids = segment_ids.to(torch.int32).contiguous()
+    return segment_ids
+
+
+def flash_fwd(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    *,
+    softmax_scale: float = 1.0,
+    mask_kind: int = MASK_NONE,
+    sliding_window: int = 0,
+    segment_ids: Optional[torch.Tensor] = None,
+    q_pos_offset: int = 0,
+    return_lse: bool = True,
+):
+    """q [B,T,Hq,D], k/v [B,S,Hkv,D] -> (out [B,T,Hq,D], lse [B,Hq,T] fp32 or None)."""
+    _require_cuda(q, k, v, segment_ids)
+    lib = _lib.load()
+    b, t, hq, d = q.shape
+    s, hkv = k.shape[1], k.shape[2]
+    out = torch.empty((b, t, hq, d), dtype=q.dtype, device=q.device)
+    lse = torch.empty((b, hq, t), dtype=torch.float32, device=q.device) if return_lse else None
+    seg = _seg(segment_ids)
+    p = AxlFlashFwdParams(
+        q=q.data_ptr(), k=k.data_ptr(), v=v.data_ptr(), out=out.data_ptr(), lse=_lib.ptr(lse),
+        segment_ids=_lib.ptr(seg),
+        q_strides=_lib.strides4(q), k_strides=_lib.strides4(k), v_strides=_lib.strides4(v),
+        out_strides=_lib.strides4(out),
+        batch=b, q_len=t, kv_len=s, num_q_heads=hq, num_kv_heads=hkv, head_dim=d,
+        dtype=_lib.dtype_code(q.dtype), mask_kind=mask_kind, sliding_window=int(sliding_window),
+        q_pos_offset=int(q_pos_offset), softmax_scale=float(softmax_scale),
+    )
+    if k.dtype != q.dtype or v.dtype != q.dtype:
+        raise AxlError(_lib.AXL_ERR_UNSUPPORTED, "q, k, v must share one dtype")
+    _lib.check(lib.axl_flash_fwd(ctypes.byref(p), _lib.current_stream_ptr()))
+    return out, lse
+
+
+def flash_bwd(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    out: torch.Tensor,
+    lse: torch.Tensor,
+    d_out: torch.Tensor,
+    *,
+    softmax_scale: float = 1.0,
+    mask_kind: int = MASK_NONE,
+    sliding_window: int = 0,
+    segment_ids: Optional[torch.Tensor] = None,
+    q_pos_offset: int = 0,
+):
+    """Returns (dq [B,T,Hq,D], dk [B,S,Hkv,D], dv [B,S,Hkv,D]) in the dtype of q."""
+    _require_cuda(q, k, v, out, lse, d_out, segment_ids)
+    lib = _lib.load()
+    b, t, hq, d = q.shape
+    s, hkv = k.shape[1], k.shape[2]
+    dq = torch.empty((b, t, hq, d), dtype=q.dtype, device=q.device)
+    dk = torch.empty((b, s, hkv, d), dtype=k.dtype, device=q.device)
+    dv = torch.empty((b, s, hkv, d), dtype=v.dtype, device=q.device)
+    seg = _seg(segment_ids)
+    if lse.dtype != torch.float32 or not lse.is_contiguous():
+        raise AxlError(_lib.AXL_ERR_INVALID_ARGUMENT, "lse must be contiguous float32 [B,Hq,T]")
+    p = AxlFlashBwdParams(
+        q=q.data_ptr(), k=k.data_ptr(), v=v.data_ptr(), out=out.data_ptr(),
+        d_out=d_out.data_ptr(), lse=lse.data_ptr(), dq=dq.data_ptr(), dk=dk.data_ptr(),
+        dv=dv.data_ptr(), segment_ids=_lib.ptr(seg),
+        q_strides=_lib.strides4(q), k_strides=_lib.strides4(k), v_strides=_lib.strides4(v),
+        out_strides=_lib.strides4(out), d_out_strides=_lib.strides4(d_out),
+        dq_strides=_lib.strides4(dq), dk_strides=_lib.strides4(dk), dv_strides=_lib.strides4(dv),
+        batch=b, q_len=t, kv_len=s, num_q_heads=hq, num_kv_heads=hkv, head_dim=d,
+        dtype=_lib.dtype_code(q.dtype), mask_kind=mask_kind, sliding_window=int(sliding_window),
+        q_pos_offset=int(q_pos_offset), softmax_scale=float(softmax_scale),
+        workspace=None, workspace_bytes=0,
+    )
+    need = lib.axl_flash_bwd_workspace_bytes(ctypes.byref(p))
+    ws = torch.empty((max(int(need), 16),), dtype=torch.uint8, device=q.device)
+    p.workspace = ws.data_ptr()
+    p.workspace_bytes = ws.numel()
+    _lib.check(lib.axl_flash_bwd(ctypes.byref(p), _lib.current_stream_ptr()))
+    return dq, dk, dv
+
+
+def paged_decode(
+    q: torch.Tensor,
+    k_pages: torch.Tensor,
+    v_pages: torch.Tensor,
+    page_tables: torch.Tensor,
+    lengths: torch.Tensor,
+    *,
+    softmax_scale: float = 1.0,
+    sliding_window: int = -1,
+    workspace: Optional[torch.Tensor] = None,
+    out: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """q [B,Hq,D]; pools [Hkv,P,page,D]; page_tables [B,pps] int32; lengths [B] int32 -> [B,Hq,D]."""
+    _require_cuda(q, k_pages, v_pages, page_tables, lengths)
+    lib = _lib.load()
+    b, hq, d = q.shape
+    hkv, num_pages, page_size, _ = k_pages.shape
+    for name, x in (("q", q), ("k_pages", k_pages), ("v_pages", v_pages), ("page_tables", page_tables), ("lengths", lengths)):
+        if not x.is_contiguous():
+            raise AxlError(_lib.AXL_ERR_UNSUPPORTED, f"{name} must be contiguous")
+    if page_tables.dtype != torch.int32 or lengths.dtype != torch.int32:
+        raise AxlError(_lib.AXL_ERR_INVALID_ARGUMENT, "page_tables and lengths must be int32")
+    if out is None:
+        out = torch.empty((b, hq, d), dtype=q.dtype, device=q.device)
+    p = AxlPagedDecodeParams(
+        q=q.data_ptr(), k_pages=k_pages.data_ptr(), v_pages=v_pages.data_ptr(),
+        page_tables=page_tables.data_ptr(), lengths=lengths.data_ptr(), out=out.data_ptr(),
+        batch=b, num_q_heads=hq, num_kv_heads=hkv, head_dim=d, num_pages=num_pages,
+        page_size=page_size, pages_per_seq=page_tables.shape[1],
+        dtype=_lib.dtype_code(q.dtype), sliding_window=int(sliding_window),
+        softmax_scale=float(softmax_scale), workspace=None, workspace_bytes=0,
+    )
+    need = int(lib.axl_paged_decode_workspace_bytes(ctypes.byref(p)))
+    if workspace is None or workspace.numel() * workspace.element_size() < need:
+        workspace = torch.empty((max(need, 16),), dtype=torch.uint8, device=q.device)
+    p.workspace = workspace.data_ptr()
+    p.workspace_bytes = workspace.numel() * workspace.element_size()
+    _lib.check(lib.axl_paged_decode(ctypes.byref(p), _lib.current_stream_ptr()))
+    return out
+
+
+def decode(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    lengths: torch.Tensor,
+    *,
+    softmax_scale: float = 1.0,
+    sliding_window: int = -1,
+) -> torch.Tensor:
+    """q [B,Hq,D]; k/v [B,S,Hkv,D]; lengths [B] int32 -> [B,Hq,D]."""
+    _require_cuda(q, k, v, lengths)
+    lib = _lib.load()
+    b, hq, d = q.shape
+    s, hkv = k.shape[1], k.shape[2]
+    if not q.is_contiguous():
+        raise AxlError(_lib.AXL_ERR_UNSUPPORTED, "q must be contiguous")
+    if lengths.dtype != torch.int32 or not lengths.is_contiguous():
+        raise AxlError(_lib.AXL_ERR_INVALID_ARGUMENT, "lengths must be contiguous int32")
+    out = torch.empty((b, hq, d), dtype=q.dtype, device=q.device)
+    p = AxlDecodeParams(
+        q=q.data_ptr(), k=k.data_ptr(), v=v.data_ptr(), lengths=lengths.data_ptr(),
+        out=out.data_ptr(), k_strides=_lib.strides4(k), v_strides=_lib.strides4(v),
+        batch=b, kv_len=s, num_q_heads=hq, num_kv_heads=hkv, head_dim=d,
+        dtype=_lib.dtype_code(q.dtype), sliding_window=int(sliding_window),
+        softmax_scale=float(softmax_scale), workspace=None, workspace_bytes=0,
+    )
+    need = int(lib.axl_decode_workspace_bytes(ctypes.byref(p)))
+    ws = torch.empty((max(need, 16),), dtype=torch.uint8, device=q.device)
+    p.workspace = ws.data_ptr()
+    p.workspace_bytes = ws.numel()
+    _lib.check(lib.axl_decode(ctypes.byref(p), _lib.current_stream_ptr()))
+    return out
