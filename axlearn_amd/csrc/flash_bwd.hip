@@ -1,7 +1,528 @@
+// Flash-attention backward for gfx950: delta pre-pass, dK/dV kernel, dQ kernel.
+//
+// Replaces axlearn/common/flash_attention/gpu_attention.py:621-786 (`_mha_backward`):
+//   delta = rowsum(out * dO) in fp32                                   (:653-658)
+//   `_mha_backward_kernel_dkdv` (:436-528):  p = exp(qk - lse); dv += p^T dO;
+//        dp = dO v^T; ds = p * (dp - delta) * scale; dk += ds^T q
+//   `_mha_backward_kernel_dq`  (:533-616):  dq += ds k
+// p and ds are rounded to bf16 before their MFMAs, accumulation is fp32, as in the reference
+// (:513, :518, :608).
+//
+// Machine mapping (all GEMMs are v_mfma_f32_32x32x16_bf16):
+//   dK/dV: a workgroup owns 128 keys of one (batch, kv head); each wavefront keeps the K and V
+//     fragments of its 32 keys in registers as B operands, streams 32-query Q/dO tiles through LDS,
+//     and loops over ALL query heads of the kv head's group, so dK/dV need no atomics and no
+//     repeated-KV reduction pass.  S = Q K^T and dP = dO V^T land with lane = key and
+//     registers = queries; exp(S) and dS are then already B operands for dV^T += dO^T P and
+//     dK^T += Q^T dS, whose A operands are transposing LDS reads of the same dO / Q tiles.
+//   dQ: a workgroup owns 128 queries (32 per wavefront, Q and dO fragments in registers) and
+//     streams 64-key K/V tiles through LDS exactly like the forward; S^T = K Q^T, dP^T = V dO^T,
+//     dQ^T += K^T dS^T with K^T from transposing LDS reads.
 #include "common.h"
+
 namespace axl {
-size_t flash_bwd_workspace_bytes(const AxlFlashBwdParams& p) { return 16; }
-int launch_flash_bwd(const AxlFlashBwdParams& p, hipStream_t stream) {
-  return set_error(AXL_ERR_UNSUPPORTED, "axl_flash_bwd: not built yet");
+
+struct BwdArgs {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* out;
+  const void* dout;
+  const float* lse;
+  float* delta;  // workspace [B, Hq, T]
+  void* dq;
+  void* dk;
+  void* dv;
+  const int32_t* seg;
+  Strides3 qs, ks, vs, os, dos, dqs, dks, dvs;
+  int B, T, S, Hq, Hkv;
+  int mask_kind, window, q_off;
+  float scale;
+};
+
+// ---------------------------------------------------------------------------------------------
+// delta[b,h,t] = sum_d out[b,t,h,d] * dO[b,t,h,d]; 16 lanes per row, 16 bytes per lane per step.
+// ---------------------------------------------------------------------------------------------
+template <typename T, int D>
+__global__ __launch_bounds__(256) void bwd_delta_kernel(const BwdArgs a) {
+  constexpr int VEC = 16 / sizeof(T);         // elements per 16-byte load
+  constexpr int STEPS = D / (16 * VEC);       // loads per lane to cover a row with 16 lanes
+  const int64_t row = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);  // over B*T*Hq
+  const int sub = threadIdx.x & 15;
+  const int64_t rows = (int64_t)a.B * a.T * a.Hq;
+  float acc = 0.f;
+  int b = 0, t = 0, h = 0;
+  if (row < rows) {
+    h = (int)(row % a.Hq);
+    t = (int)((row / a.Hq) % a.T);
+    b = (int)(row / ((int64_t)a.Hq * a.T));
+    const T* o = (const T*)a.out + b * a.os.b + (int64_t)t * a.os.s + h * a.os.h;
+    const T* d = (const T*)a.dout + b * a.dos.b + (int64_t)t * a.dos.s + h * a.dos.h;
+#pragma unroll
+    for (int s = 0; s < (STEPS > 0 ? STEPS : 1); s++) {
+      const int off = (s * 16 + sub) * VEC;
+      if (off < D) {
+        union { uint4 u; T e[VEC]; } x, y;
+        x.u = *(const uint4*)(o + off);
+        y.u = *(const uint4*)(d + off);
+#pragma unroll
+        for (int i = 0; i < VEC; i++) acc += (float)x.e[i] * (float)y.e[i];
+      }
+    }
+  }
+  acc += __shfl_xor(acc, 1, 64);
+  acc += __shfl_xor(acc, 2, 64);
+  acc += __shfl_xor(acc, 4, 64);
+  acc += __shfl_xor(acc, 8, 64);
+  if (row < rows && sub == 0) a.delta[((int64_t)b * a.Hq + h) * a.T + t] = acc;
 }
+
+// ---------------------------------------------------------------------------------------------
+// dK / dV.
+// ---------------------------------------------------------------------------------------------
+template <int D>
+struct DkvTile {
+  static constexpr int BKV = 128;              // keys per workgroup (32 per wavefront)
+  static constexpr int BQ = 32;                // query rows per LDS tile
+  static constexpr int STRIDE = D * 2 + 16;    // bytes per Q / dO row in LDS
+  static constexpr int TILE_BYTES = BQ * STRIDE;
+  static constexpr int CHUNKS = (BQ * D * 2 / 16 + 255) / 256;  // 16-byte chunks per thread per tensor
+  static constexpr int LDS_BYTES = 4 * TILE_BYTES;              // {Q, dO} x double buffer
+};
+
+template <int D>
+__global__ __launch_bounds__(256) void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
+  using Tile = DkvTile<D>;
+  constexpr int KK = D / 16, DT = D / 32;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  char* const q_lds = smem;                          // 2 buffers
+  char* const do_lds = smem + 2 * Tile::TILE_BYTES;  // 2 buffers
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+  const int G = a.Hq / a.Hkv;
+  const int nkb = a.S / Tile::BKV;
+  // blockIdx -> (key block, batch, kv head); earliest key blocks (most queries under a causal
+  // mask) first.
+  const int kb = blockIdx.x / (a.B * a.Hkv);
+  const int rem = blockIdx.x % (a.B * a.Hkv);
+  const int b = rem / a.Hkv, hk = rem % a.Hkv;
+  (void)nkb;
+  const int k0_wg = kb * Tile::BKV;
+  const int k0 = k0_wg + wave * 32;  // this wavefront's keys
+
+  // K and V fragments (B operands): lane (key l32, k-group g) holds d = 16kk + 8g .. +7.
+  const __bf16* kp = (const __bf16*)a.k + b * a.ks.b + (int64_t)(k0 + l32) * a.ks.s + hk * a.ks.h;
+  const __bf16* vp = (const __bf16*)a.v + b * a.vs.b + (int64_t)(k0 + l32) * a.vs.s + hk * a.vs.h;
+  bf16x8 kf[KK], vf[KK];
+#pragma unroll
+  for (int kk = 0; kk < KK; kk++) {
+    kf[kk] = *(const bf16x8*)(kp + 16 * kk + 8 * g);
+    vf[kk] = *(const bf16x8*)(vp + 16 * kk + 8 * g);
+  }
+  const int kpos = k0 + l32;
+  const int seg_k = a.seg ? a.seg[(int64_t)b * a.T + k0 + l32] : 0;
+
+  // Query rows that can see any key of this workgroup.
+  int q_begin = 0, q_end = a.T;
+  if (a.mask_kind != AXL_MASK_NONE) {
+    q_begin = max(0, k0_wg - a.q_off);
+    if (a.mask_kind == AXL_MASK_SLIDING_WINDOW)
+      q_end = min(a.T, k0_wg + Tile::BKV - 1 + a.window - a.q_off + 1);
+  }
+  const int t_begin = q_begin / Tile::BQ;
+  const int t_end = max(t_begin, (q_end + Tile::BQ - 1) / Tile::BQ);
+  const int nt = t_end - t_begin;
+  const int total = nt * G;  // iterations: query head (outer) x query tile (inner)
+
+  floatx16 dk_acc[DT], dv_acc[DT];
+#pragma unroll
+  for (int i = 0; i < DT; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) dk_acc[i][r] = dv_acc[i][r] = 0.f;
+  const float c = a.scale * kLog2e;
+
+  uint4 qreg[Tile::CHUNKS], dreg[Tile::CHUNKS];
+  auto load_tile = [&](int it) {
+    const int hq = hk * G + it / nt;
+    const int q0 = (t_begin + it % nt) * Tile::BQ;
+    const __bf16* qg = (const __bf16*)a.q + b * a.qs.b + hq * a.qs.h;
+    const __bf16* dg = (const __bf16*)a.dout + b * a.dos.b + hq * a.dos.h;
+#pragma unroll
+    for (int i = 0; i < Tile::CHUNKS; i++) {
+      const int cidx = tid + 256 * i;
+      const int row = cidx / (D / 8), cc = cidx % (D / 8);
+      if (row < Tile::BQ) {
+        qreg[i] = *(const uint4*)(qg + (int64_t)(q0 + row) * a.qs.s + cc * 8);
+        dreg[i] = *(const uint4*)(dg + (int64_t)(q0 + row) * a.dos.s + cc * 8);
+      }
+    }
+  };
+  auto store_tile = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < Tile::CHUNKS; i++) {
+      const int cidx = tid + 256 * i;
+      const int row = cidx / (D / 8), cc = cidx % (D / 8);
+      if (row < Tile::BQ) {
+        *(uint4*)(q_lds + buf * Tile::TILE_BYTES + row * Tile::STRIDE + cc * 16) = qreg[i];
+        *(uint4*)(do_lds + buf * Tile::TILE_BYTES + row * Tile::STRIDE + cc * 16) = dreg[i];
+      }
+    }
+  };
+  if (total > 0) {
+    load_tile(0);
+    store_tile(0);
+  }
+  __syncthreads();
+
+  const int a_row_off = swap_bits_2_3(l32) * Tile::STRIDE + g * 16;  // normal (row = query) reads
+  const int j16 = lane & 15, half = (lane >> 4) & 1;
+  const int tr_off = (8 * g + (j16 >> 2)) * Tile::STRIDE + (16 * half + 4 * (j16 & 3)) * 2;
+
+  for (int it = 0; it < total; it++) {
+    const int buf = it & 1;
+    const bool has_next = it + 1 < total;
+    if (has_next) load_tile(it + 1);
+    const int hq = hk * G + it / nt;
+    const int q0 = (t_begin + it % nt) * Tile::BQ;
+    const int qpos_min = q0 + a.q_off, qpos_max = q0 + Tile::BQ - 1 + a.q_off;
+    bool skip = false, need_mask = false;
+    if (a.mask_kind != AXL_MASK_NONE) {
+      skip = k0 > qpos_max;
+      need_mask = k0 + 31 > qpos_min;
+      if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) {
+        skip = skip || (qpos_min - (k0 + 31) > a.window);
+        need_mask = need_mask || (qpos_max - k0 > a.window);
+      }
+    }
+    if (!skip) {
+      const char* qt = q_lds + buf * Tile::TILE_BYTES;
+      const char* dt_ = do_lds + buf * Tile::TILE_BYTES;
+      floatx16 s, dp;
+#pragma unroll
+      for (int r = 0; r < 16; r++) s[r] = dp[r] = 0.f;
+#pragma unroll
+      for (int kk = 0; kk < KK; kk++) {
+        const bf16x8 qa = *(const bf16x8*)(qt + a_row_off + kk * 32);
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa, kf[kk], s, 0, 0, 0);
+      }
+#pragma unroll
+      for (int kk = 0; kk < KK; kk++) {
+        const bf16x8 da = *(const bf16x8*)(dt_ + a_row_off + kk * 32);
+        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da, vf[kk], dp, 0, 0, 0);
+      }
+      // Register r of lane group g is query q0 + 16(r/8) + 8g + (r%8); the lane is key kpos.
+      const float* lse_p = a.lse + ((int64_t)b * a.Hq + hq) * a.T + q0 + 8 * g;
+      const float* del_p = a.delta + ((int64_t)b * a.Hq + hq) * a.T + q0 + 8 * g;
+      float lse_r[16], del_r[16];
+#pragma unroll
+      for (int t8 = 0; t8 < 2; t8++) {
+        const float4 l0 = *(const float4*)(lse_p + 16 * t8), l1 = *(const float4*)(lse_p + 16 * t8 + 4);
+        const float4 d0 = *(const float4*)(del_p + 16 * t8), d1 = *(const float4*)(del_p + 16 * t8 + 4);
+        lse_r[8 * t8 + 0] = l0.x; lse_r[8 * t8 + 1] = l0.y; lse_r[8 * t8 + 2] = l0.z; lse_r[8 * t8 + 3] = l0.w;
+        lse_r[8 * t8 + 4] = l1.x; lse_r[8 * t8 + 5] = l1.y; lse_r[8 * t8 + 6] = l1.z; lse_r[8 * t8 + 7] = l1.w;
+        del_r[8 * t8 + 0] = d0.x; del_r[8 * t8 + 1] = d0.y; del_r[8 * t8 + 2] = d0.z; del_r[8 * t8 + 3] = d0.w;
+        del_r[8 * t8 + 4] = d1.x; del_r[8 * t8 + 5] = d1.y; del_r[8 * t8 + 6] = d1.z; del_r[8 * t8 + 7] = d1.w;
+      }
+      int seg_r[16];
+      if (a.seg) {
+        const int32_t* sp = a.seg + (int64_t)b * a.T + q0 + 8 * g;
+#pragma unroll
+        for (int t8 = 0; t8 < 2; t8++) {
+          const int4 s0 = *(const int4*)(sp + 16 * t8), s1 = *(const int4*)(sp + 16 * t8 + 4);
+          seg_r[8 * t8 + 0] = s0.x; seg_r[8 * t8 + 1] = s0.y; seg_r[8 * t8 + 2] = s0.z; seg_r[8 * t8 + 3] = s0.w;
+          seg_r[8 * t8 + 4] = s1.x; seg_r[8 * t8 + 5] = s1.y; seg_r[8 * t8 + 6] = s1.z; seg_r[8 * t8 + 7] = s1.w;
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        bool keep = true;
+        if (need_mask) {
+          const int diff = (q0 + a.q_off + 16 * (r / 8) + 8 * g + (r % 8)) - kpos;
+          keep = diff >= 0;
+          if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) keep = keep && diff <= a.window;
+        }
+        if (a.seg) keep = keep && (seg_r[r] == seg_k);
+        const float sv = keep ? s[r] : kNegInf;
+        const float p = fast_exp2(__builtin_fmaf(sv, c, -lse_r[r] * kLog2e));
+        s[r] = p;
+        dp[r] = p * (dp[r] - del_r[r]);
+      }
+      // dV^T += dO^T P ; dK^T += Q^T dS  (scale applied once at the end).
+#pragma unroll
+      for (int t8 = 0; t8 < 2; t8++) {
+        const bf16x8 pb = pack_bf16x8(s[8 * t8 + 0], s[8 * t8 + 1], s[8 * t8 + 2], s[8 * t8 + 3],
+                                      s[8 * t8 + 4], s[8 * t8 + 5], s[8 * t8 + 6], s[8 * t8 + 7]);
+        const bf16x8 dsb = pack_bf16x8(dp[8 * t8 + 0], dp[8 * t8 + 1], dp[8 * t8 + 2], dp[8 * t8 + 3],
+                                       dp[8 * t8 + 4], dp[8 * t8 + 5], dp[8 * t8 + 6], dp[8 * t8 + 7]);
+        const char* da = dt_ + 16 * t8 * Tile::STRIDE + tr_off;
+        const char* qa = qt + 16 * t8 * Tile::STRIDE + tr_off;
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++) {
+          union { bf16x8 v; shortx4 hlf[2]; } fa, fb;
+          fa.hlf[0] = lds_read_tr16(da + dt * 64);
+          fa.hlf[1] = lds_read_tr16(da + dt * 64 + 4 * Tile::STRIDE);
+          dv_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa.v, pb, dv_acc[dt], 0, 0, 0);
+          fb.hlf[0] = lds_read_tr16(qa + dt * 64);
+          fb.hlf[1] = lds_read_tr16(qa + dt * 64 + 4 * Tile::STRIDE);
+          dk_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb.v, dsb, dk_acc[dt], 0, 0, 0);
+        }
+      }
+    }
+    if (has_next) store_tile(buf ^ 1);
+    __syncthreads();
+  }
+
+  __bf16* dkp = (__bf16*)a.dk + b * a.dks.b + (int64_t)(k0 + l32) * a.dks.s + hk * a.dks.h;
+  __bf16* dvp = (__bf16*)a.dv + b * a.dvs.b + (int64_t)(k0 + l32) * a.dvs.s + hk * a.dvs.h;
+#pragma unroll
+  for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+    for (int rq = 0; rq < 4; rq++) {
+      union { bf16x2 p[2]; uint2 u; } w;
+      w.p[0] = pack_bf16(dk_acc[dt][4 * rq + 0] * a.scale, dk_acc[dt][4 * rq + 1] * a.scale);
+      w.p[1] = pack_bf16(dk_acc[dt][4 * rq + 2] * a.scale, dk_acc[dt][4 * rq + 3] * a.scale);
+      *(uint2*)(dkp + 32 * dt + 8 * rq + 4 * g) = w.u;
+      w.p[0] = pack_bf16(dv_acc[dt][4 * rq + 0], dv_acc[dt][4 * rq + 1]);
+      w.p[1] = pack_bf16(dv_acc[dt][4 * rq + 2], dv_acc[dt][4 * rq + 3]);
+      *(uint2*)(dvp + 32 * dt + 8 * rq + 4 * g) = w.u;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// dQ.
+// ---------------------------------------------------------------------------------------------
+template <int D>
+struct DqTile {
+  static constexpr int BQ = 128;
+  static constexpr int BK = 64;
+  static constexpr int STRIDE = D * 2 + 16;
+  static constexpr int TILE_BYTES = BK * STRIDE;
+  static constexpr int CHUNKS = BK * D * 2 / 16 / 256;
+  static constexpr int LDS_BYTES = 4 * TILE_BYTES;  // {K, V} x double buffer
+};
+
+template <int D>
+__global__ __launch_bounds__(256) void flash_bwd_dq_bf16_kernel(const BwdArgs a) {
+  using Tile = DqTile<D>;
+  constexpr int KK = D / 16, DT = D / 32;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  char* const k_lds = smem;
+  char* const v_lds = smem + 2 * Tile::TILE_BYTES;
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+  const int nqb = a.T / Tile::BQ;
+  const int per_qb = a.B * a.Hq;
+  const int qb = nqb - 1 - blockIdx.x / per_qb;
+  const int rem = blockIdx.x % per_qb;
+  const int b = rem / a.Hq, h = rem % a.Hq;
+  const int hk = h / (a.Hq / a.Hkv);
+  const int q0_wg = qb * Tile::BQ;
+  const int q0 = q0_wg + wave * 32;
+
+  const __bf16* qp = (const __bf16*)a.q + b * a.qs.b + (int64_t)(q0 + l32) * a.qs.s + h * a.qs.h;
+  const __bf16* dop = (const __bf16*)a.dout + b * a.dos.b + (int64_t)(q0 + l32) * a.dos.s + h * a.dos.h;
+  const __bf16* kp = (const __bf16*)a.k + b * a.ks.b + hk * a.ks.h;
+  const __bf16* vp = (const __bf16*)a.v + b * a.vs.b + hk * a.vs.h;
+  bf16x8 qf[KK], dof[KK];
+#pragma unroll
+  for (int kk = 0; kk < KK; kk++) {
+    qf[kk] = *(const bf16x8*)(qp + 16 * kk + 8 * g);
+    dof[kk] = *(const bf16x8*)(dop + 16 * kk + 8 * g);
+  }
+  const int64_t stat_idx = ((int64_t)b * a.Hq + h) * a.T + q0 + l32;
+  const float lse2 = a.lse[stat_idx] * kLog2e;
+  const float delta = a.delta[stat_idx];
+
+  int k_begin = 0, k_end = a.S;
+  if (a.mask_kind != AXL_MASK_NONE) {
+    k_end = min(a.S, q0_wg + Tile::BQ + a.q_off);
+    if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) k_begin = max(0, q0_wg + a.q_off - a.window);
+  }
+  const int t_begin = k_begin / Tile::BK;
+  const int t_end = (k_end + Tile::BK - 1) / Tile::BK;
+  const int qpos = q0 + l32 + a.q_off;
+  const int qpos_min = q0 + a.q_off, qpos_max = q0 + 31 + a.q_off;
+  const int seg_q = a.seg ? a.seg[(int64_t)b * a.T + q0 + l32] : 0;
+  const int32_t* seg_k = a.seg ? a.seg + (int64_t)b * a.T : nullptr;
+
+  floatx16 dq_acc[DT];
+#pragma unroll
+  for (int i = 0; i < DT; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) dq_acc[i][r] = 0.f;
+  const float c = a.scale * kLog2e;
+
+  uint4 kreg[Tile::CHUNKS], vreg[Tile::CHUNKS];
+  auto load_tile = [&](int t) {
+    const int k0 = t * Tile::BK;
+#pragma unroll
+    for (int i = 0; i < Tile::CHUNKS; i++) {
+      const int cidx = tid + 256 * i;
+      const int row = cidx / (D / 8), cc = cidx % (D / 8);
+      kreg[i] = *(const uint4*)(kp + (int64_t)(k0 + row) * a.ks.s + cc * 8);
+      vreg[i] = *(const uint4*)(vp + (int64_t)(k0 + row) * a.vs.s + cc * 8);
+    }
+  };
+  auto store_tile = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < Tile::CHUNKS; i++) {
+      const int cidx = tid + 256 * i;
+      const int row = cidx / (D / 8), cc = cidx % (D / 8);
+      *(uint4*)(k_lds + buf * Tile::TILE_BYTES + row * Tile::STRIDE + cc * 16) = kreg[i];
+      *(uint4*)(v_lds + buf * Tile::TILE_BYTES + row * Tile::STRIDE + cc * 16) = vreg[i];
+    }
+  };
+  if (t_begin < t_end) {
+    load_tile(t_begin);
+    store_tile(0);
+  }
+  __syncthreads();
+
+  const int a_row_off = swap_bits_2_3(l32) * Tile::STRIDE + g * 16;
+  const int j16 = lane & 15, half = (lane >> 4) & 1;
+  const int tr_off = (8 * g + (j16 >> 2)) * Tile::STRIDE + (16 * half + 4 * (j16 & 3)) * 2;
+
+  for (int t = t_begin; t < t_end; t++) {
+    const int buf = (t - t_begin) & 1;
+    const bool has_next = t + 1 < t_end;
+    if (has_next) load_tile(t + 1);
+    const int k0 = t * Tile::BK;
+    bool skip = false, need_mask = false;
+    if (a.mask_kind != AXL_MASK_NONE) {
+      skip = k0 > qpos_max;
+      need_mask = k0 + Tile::BK - 1 > qpos_min;
+      if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) {
+        skip = skip || (qpos_min - (k0 + Tile::BK - 1) > a.window);
+        need_mask = need_mask || (qpos_max - k0 > a.window);
+      }
+    }
+    if (!skip) {
+      const char* kt = k_lds + buf * Tile::TILE_BYTES;
+      const char* vt = v_lds + buf * Tile::TILE_BYTES;
+#pragma unroll
+      for (int ks = 0; ks < 2; ks++) {
+        floatx16 s, dp;
+#pragma unroll
+        for (int r = 0; r < 16; r++) s[r] = dp[r] = 0.f;
+        const char* ka = kt + ks * 32 * Tile::STRIDE + a_row_off;
+        const char* va = vt + ks * 32 * Tile::STRIDE + a_row_off;
+#pragma unroll
+        for (int kk = 0; kk < KK; kk++) {
+          const bf16x8 kfr = *(const bf16x8*)(ka + kk * 32);
+          s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr, qf[kk], s, 0, 0, 0);
+        }
+#pragma unroll
+        for (int kk = 0; kk < KK; kk++) {
+          const bf16x8 vfr = *(const bf16x8*)(va + kk * 32);
+          dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr, dof[kk], dp, 0, 0, 0);
+        }
+        // Register r of lane group g is key k0 + 32ks + 16(r/8) + 8g + (r%8); the lane is a query.
+        int seg_r[16];
+        if (seg_k) {
+#pragma unroll
+          for (int t8 = 0; t8 < 2; t8++) {
+            const int4* sp = (const int4*)(seg_k + k0 + 32 * ks + 16 * t8 + 8 * g);
+            const int4 s0 = sp[0], s1 = sp[1];
+            seg_r[8 * t8 + 0] = s0.x; seg_r[8 * t8 + 1] = s0.y; seg_r[8 * t8 + 2] = s0.z; seg_r[8 * t8 + 3] = s0.w;
+            seg_r[8 * t8 + 4] = s1.x; seg_r[8 * t8 + 5] = s1.y; seg_r[8 * t8 + 6] = s1.z; seg_r[8 * t8 + 7] = s1.w;
+          }
+        }
+        const int diff0 = qpos - (k0 + 32 * ks + 8 * g);
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          bool keep = true;
+          if (need_mask) {
+            const int diff = diff0 - (16 * (r / 8) + (r % 8));
+            keep = diff >= 0;
+            if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) keep = keep && diff <= a.window;
+          }
+          if (seg_k) keep = keep && (seg_r[r] == seg_q);
+          const float sv = keep ? s[r] : kNegInf;
+          const float p = fast_exp2(__builtin_fmaf(sv, c, -lse2));
+          dp[r] = p * (dp[r] - delta);
+        }
+        // dQ^T[d][q] += K^T[d][key] dS^T[key][q].
+#pragma unroll
+        for (int t8 = 0; t8 < 2; t8++) {
+          const bf16x8 dsb = pack_bf16x8(dp[8 * t8 + 0], dp[8 * t8 + 1], dp[8 * t8 + 2], dp[8 * t8 + 3],
+                                         dp[8 * t8 + 4], dp[8 * t8 + 5], dp[8 * t8 + 6], dp[8 * t8 + 7]);
+          const char* kta = kt + (32 * ks + 16 * t8) * Tile::STRIDE + tr_off;
+#pragma unroll
+          for (int dt = 0; dt < DT; dt++) {
+            union { bf16x8 v; shortx4 hlf[2]; } fa;
+            fa.hlf[0] = lds_read_tr16(kta + dt * 64);
+            fa.hlf[1] = lds_read_tr16(kta + dt * 64 + 4 * Tile::STRIDE);
+            dq_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa.v, dsb, dq_acc[dt], 0, 0, 0);
+          }
+        }
+      }
+    }
+    if (has_next) store_tile(buf ^ 1);
+    __syncthreads();
+  }
+
+  __bf16* dqp = (__bf16*)a.dq + b * a.dqs.b + (int64_t)(q0 + l32) * a.dqs.s + h * a.dqs.h;
+#pragma unroll
+  for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+    for (int rq = 0; rq < 4; rq++) {
+      union { bf16x2 p[2]; uint2 u; } w;
+      w.p[0] = pack_bf16(dq_acc[dt][4 * rq + 0] * a.scale, dq_acc[dt][4 * rq + 1] * a.scale);
+      w.p[1] = pack_bf16(dq_acc[dt][4 * rq + 2] * a.scale, dq_acc[dt][4 * rq + 3] * a.scale);
+      *(uint2*)(dqp + 32 * dt + 8 * rq + 4 * g) = w.u;
+    }
+}
+
+static Strides3 to_s3(const AxlStrides& s) { return Strides3{s.batch, s.seq, s.head}; }
+
+size_t flash_bwd_workspace_bytes(const AxlFlashBwdParams& p) {
+  // delta [B, Hq, T] fp32.
+  return (size_t)p.batch * p.num_q_heads * p.q_len * sizeof(float);
+}
+
+int launch_flash_bwd(const AxlFlashBwdParams& p, hipStream_t stream) {
+  if (p.dtype != AXL_BF16)
+    return set_error(AXL_ERR_UNSUPPORTED, "axl_flash_bwd: only bf16 is supported");
+  BwdArgs a;
+  a.q = p.q; a.k = p.k; a.v = p.v; a.out = p.out; a.dout = p.d_out; a.lse = p.lse;
+  a.delta = (float*)p.workspace;
+  a.dq = p.dq; a.dk = p.dk; a.dv = p.dv; a.seg = p.segment_ids;
+  a.qs = to_s3(p.q_strides); a.ks = to_s3(p.k_strides); a.vs = to_s3(p.v_strides);
+  a.os = to_s3(p.out_strides); a.dos = to_s3(p.d_out_strides); a.dqs = to_s3(p.dq_strides);
+  a.dks = to_s3(p.dk_strides); a.dvs = to_s3(p.dv_strides);
+  a.B = p.batch; a.T = p.q_len; a.S = p.kv_len; a.Hq = p.num_q_heads; a.Hkv = p.num_kv_heads;
+  a.mask_kind = p.mask_kind; a.window = p.sliding_window; a.q_off = p.q_pos_offset;
+  a.scale = p.softmax_scale;
+  hipError_t err = hipSuccess;
+  const int64_t rows = (int64_t)p.batch * p.q_len * p.num_q_heads;
+  const int delta_grid = (int)((rows + 15) / 16);
+  const int dkv_grid = (p.kv_len / 128) * p.batch * p.num_kv_heads;
+  const int dq_grid = (p.q_len / 128) * p.batch * p.num_q_heads;
+#define AXL_LAUNCH(KERNEL, GRID, LDS)                                                           \
+  do {                                                                                          \
+    if (err == hipSuccess && (LDS) > 0)                                                         \
+      err = hipFuncSetAttribute((const void*)KERNEL, hipFuncAttributeMaxDynamicSharedMemorySize, \
+                                (LDS));                                                         \
+    if (err == hipSuccess) {                                                                    \
+      hipLaunchKernelGGL(KERNEL, dim3(GRID), dim3(256), (LDS), stream, a);                      \
+      err = hipGetLastError();                                                                  \
+    }                                                                                           \
+  } while (0)
+  if (p.head_dim == 128) {
+    AXL_LAUNCH((bwd_delta_kernel<__bf16, 128>), delta_grid, 0);
+    AXL_LAUNCH(flash_bwd_dkdv_bf16_kernel<128>, dkv_grid, DkvTile<128>::LDS_BYTES);
+    AXL_LAUNCH(flash_bwd_dq_bf16_kernel<128>, dq_grid, DqTile<128>::LDS_BYTES);
+  } else {
+    AXL_LAUNCH((bwd_delta_kernel<__bf16, 64>), delta_grid, 0);
+    AXL_LAUNCH(flash_bwd_dkdv_bf16_kernel<64>, dkv_grid, DkvTile<64>::LDS_BYTES);
+    AXL_LAUNCH(flash_bwd_dq_bf16_kernel<64>, dq_grid, DqTile<64>::LDS_BYTES);
+  }
+#undef AXL_LAUNCH
+  if (err != hipSuccess)
+    return set_error(AXL_ERR_LAUNCH, "axl_flash_bwd: launch failed: %s", hipGetErrorString(err));
+  return AXL_OK;
+}
+
 }  // namespace axl
