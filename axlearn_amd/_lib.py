@@ -96,6 +96,7 @@ class AxlDecodeParams(ctypes.Structure):
 EXPORTED_SYMBOLS = (
     "axl_flash_fwd",
     "axl_flash_bwd",
+    "axl_flash_bwd_phases",
     "axl_flash_bwd_workspace_bytes",
     "axl_paged_decode",
     "axl_paged_decode_workspace_bytes",
@@ -130,6 +131,8 @@ def load() -> ctypes.CDLL:
         fn = getattr(lib, name)
         fn.restype = ctypes.c_int
         fn.argtypes = [ctypes.POINTER(ptype), ctypes.c_void_p]
+    lib.axl_flash_bwd_phases.restype = ctypes.c_int
+    lib.axl_flash_bwd_phases.argtypes = [ctypes.POINTER(AxlFlashBwdParams), ctypes.c_int, ctypes.c_void_p]
     for name, ptype in (
         ("axl_flash_bwd_workspace_bytes", AxlFlashBwdParams),
         ("axl_paged_decode_workspace_bytes", AxlPagedDecodeParams),

@@ -19,7 +19,7 @@ int set_error(int code, const char* fmt, ...) {
 }
 
 int launch_flash_fwd(const AxlFlashFwdParams& p, hipStream_t stream);
-int launch_flash_bwd(const AxlFlashBwdParams& p, hipStream_t stream);
+int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream);
 size_t flash_bwd_workspace_bytes(const AxlFlashBwdParams& p);
 int launch_paged_decode(const AxlPagedDecodeParams& p, hipStream_t stream);
 size_t paged_decode_workspace_bytes(const AxlPagedDecodeParams& p);
@@ -98,7 +98,13 @@ size_t axl_flash_bwd_workspace_bytes(const AxlFlashBwdParams* p) {
 }
 
 int axl_flash_bwd(const AxlFlashBwdParams* p, void* stream) {
+  return axl_flash_bwd_phases(p, AXL_BWD_DELTA | AXL_BWD_DKDV | AXL_BWD_DQ, stream);
+}
+
+int axl_flash_bwd_phases(const AxlFlashBwdParams* p, int phases, void* stream) {
   if (!p) return set_error(AXL_ERR_INVALID_ARGUMENT, "axl_flash_bwd: params is NULL");
+  if (phases <= 0 || phases > 7)
+    return set_error(AXL_ERR_INVALID_ARGUMENT, "axl_flash_bwd: phases must be in 1..7");
   int rc = check_flash_shapes("axl_flash_bwd", p->batch, p->q_len, p->kv_len, p->num_q_heads,
                               p->num_kv_heads, p->head_dim, p->dtype, p->mask_kind,
                               p->sliding_window, p->softmax_scale, p->segment_ids);
@@ -121,7 +127,7 @@ int axl_flash_bwd(const AxlFlashBwdParams* p, void* stream) {
   if (!p->workspace || p->workspace_bytes < need || !aligned16(p->workspace))
     return set_error(AXL_ERR_WORKSPACE, "axl_flash_bwd: workspace needs %zu bytes, got %zu", need,
                      p->workspace ? p->workspace_bytes : (size_t)0);
-  return launch_flash_bwd(*p, (hipStream_t)stream);
+  return launch_flash_bwd(*p, phases, (hipStream_t)stream);
 }
 
 static int check_decode_common(const char* who, int batch, int hq, int hkv, int d, int dtype,
@@ -137,8 +143,8 @@ static int check_decode_common(const char* who, int batch, int hq, int hkv, int 
     return set_error(AXL_ERR_UNSUPPORTED, "%s: only bf16 is supported", who);
   if (d != 128 && d != 64)
     return set_error(AXL_ERR_UNSUPPORTED, "%s: head_dim %d (supported: 64, 128)", who, d);
-  if (hq / hkv > 16)
-    return set_error(AXL_ERR_UNSUPPORTED, "%s: more than 16 query heads per kv head", who);
+  if (hq / hkv > 8)
+    return set_error(AXL_ERR_UNSUPPORTED, "%s: more than 8 query heads per kv head", who);
   return AXL_OK;
 }
 

@@ -21,10 +21,12 @@ typedef __attribute__((__vector_size__(4 * sizeof(int)))) int intx4;
 
 #define AXL_LDS(T, p) ((__attribute__((address_space(3))) T*)(p))
 
-// Masked logits use the reference's finite sentinel (axlearn/common/attention_bias.py:43), never
-// -inf, so that exp(masked - max) underflows to exactly 0 without producing NaN on rows whose
-// first tiles are fully masked.
+// Running row maxima start at the reference's finite sentinel (axlearn/common/attention_bias.py:43)
+// and masked logits are set to -inf: exp2(-inf - finite) is exactly 0, and (finite - finite) never
+// produces NaN on rows whose first tiles are fully masked.  (A finite masked value would not do:
+// exp2(fma(masked, c, -round(masked * c))) exponentiates the rounding error of a ~1e14 product.)
 constexpr float kNegInf = -1e15f;
+constexpr float kMasked = -__builtin_inff();
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 

@@ -243,7 +243,7 @@ __global__ __launch_bounds__(256) void flash_bwd_dkdv_bf16_kernel(const BwdArgs 
           if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) keep = keep && diff <= a.window;
         }
         if (a.seg) keep = keep && (seg_r[r] == seg_k);
-        const float sv = keep ? s[r] : kNegInf;
+        const float sv = keep ? s[r] : kMasked;
         const float p = fast_exp2(__builtin_fmaf(sv, c, -lse_r[r] * kLog2e));
         s[r] = p;
         dp[r] = p * (dp[r] - del_r[r]);
@@ -439,7 +439,7 @@ __global__ __launch_bounds__(256) void flash_bwd_dq_bf16_kernel(const BwdArgs a)
             if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) keep = keep && diff <= a.window;
           }
           if (seg_k) keep = keep && (seg_r[r] == seg_q);
-          const float sv = keep ? s[r] : kNegInf;
+          const float sv = keep ? s[r] : kMasked;
           const float p = fast_exp2(__builtin_fmaf(sv, c, -lse2));
           dp[r] = p * (dp[r] - delta);
         }
@@ -482,7 +482,7 @@ size_t flash_bwd_workspace_bytes(const AxlFlashBwdParams& p) {
   return (size_t)p.batch * p.num_q_heads * p.q_len * sizeof(float);
 }
 
-int launch_flash_bwd(const AxlFlashBwdParams& p, hipStream_t stream) {
+int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream) {
   if (p.dtype != AXL_BF16)
     return set_error(AXL_ERR_UNSUPPORTED, "axl_flash_bwd: only bf16 is supported");
   BwdArgs a;
@@ -511,13 +511,13 @@ int launch_flash_bwd(const AxlFlashBwdParams& p, hipStream_t stream) {
     }                                                                                           \
   } while (0)
   if (p.head_dim == 128) {
-    AXL_LAUNCH((bwd_delta_kernel<__bf16, 128>), delta_grid, 0);
-    AXL_LAUNCH(flash_bwd_dkdv_bf16_kernel<128>, dkv_grid, DkvTile<128>::LDS_BYTES);
-    AXL_LAUNCH(flash_bwd_dq_bf16_kernel<128>, dq_grid, DqTile<128>::LDS_BYTES);
+    if (phases & AXL_BWD_DELTA) AXL_LAUNCH((bwd_delta_kernel<__bf16, 128>), delta_grid, 0);
+    if (phases & AXL_BWD_DKDV) AXL_LAUNCH(flash_bwd_dkdv_bf16_kernel<128>, dkv_grid, DkvTile<128>::LDS_BYTES);
+    if (phases & AXL_BWD_DQ) AXL_LAUNCH(flash_bwd_dq_bf16_kernel<128>, dq_grid, DqTile<128>::LDS_BYTES);
   } else {
-    AXL_LAUNCH((bwd_delta_kernel<__bf16, 64>), delta_grid, 0);
-    AXL_LAUNCH(flash_bwd_dkdv_bf16_kernel<64>, dkv_grid, DkvTile<64>::LDS_BYTES);
-    AXL_LAUNCH(flash_bwd_dq_bf16_kernel<64>, dq_grid, DqTile<64>::LDS_BYTES);
+    if (phases & AXL_BWD_DELTA) AXL_LAUNCH((bwd_delta_kernel<__bf16, 64>), delta_grid, 0);
+    if (phases & AXL_BWD_DKDV) AXL_LAUNCH(flash_bwd_dkdv_bf16_kernel<64>, dkv_grid, DkvTile<64>::LDS_BYTES);
+    if (phases & AXL_BWD_DQ) AXL_LAUNCH(flash_bwd_dq_bf16_kernel<64>, dq_grid, DqTile<64>::LDS_BYTES);
   }
 #undef AXL_LAUNCH
   if (err != hipSuccess)

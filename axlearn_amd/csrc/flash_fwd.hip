@@ -192,7 +192,7 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
             const int diff = diff0 - (16 * (r / 8) + (r % 8));
             bool keep = diff >= 0;
             if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) keep = keep && diff <= a.window;
-            s[ks][r] = keep ? s[ks][r] : kNegInf;
+            s[ks][r] = keep ? s[ks][r] : kMasked;
           }
         }
       }
@@ -206,7 +206,7 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
             const int ids[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
 #pragma unroll
             for (int j = 0; j < 8; j++)
-              s[ks][8 * t8 + j] = (ids[j] == seg_q) ? s[ks][8 * t8 + j] : kNegInf;
+              s[ks][8 * t8 + j] = (ids[j] == seg_q) ? s[ks][8 * t8 + j] : kMasked;
           }
         }
       }
@@ -217,7 +217,9 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
         for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[ks][r]);
       mx = xor32_max(mx);
       const float mc = mx * c;
-      const float corr = fast_exp2(m_run * c - mc);
+      // Subtract first: (m_run * c - mc) would be contracted into an fma whose result, when the
+      // max did not move, is the rounding error of the product instead of an exact 0.
+      const float corr = fast_exp2((m_run - mx) * c);
       m_run = mx;
       float lsum = 0.f;
 #pragma unroll
@@ -261,7 +263,7 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
 
   // Epilogue: out = acc / l ; lse = m*scale + ln(l).
   const float l_tot = xor32_sum(l_run);
-  const float inv_l = 1.0f / l_tot;
+  const float inv_l = l_tot > 0.f ? 1.0f / l_tot : 0.f;  // a row with no visible key yields zeros
   __bf16* op = (__bf16*)a.out + b * a.os.b + (int64_t)(q0 + l32) * a.os.s + h * a.os.h;
 #pragma unroll
   for (int dt = 0; dt < DT; dt++) {
@@ -388,7 +390,7 @@ __global__ __launch_bounds__(256) void flash_fwd_f32_kernel(const FwdArgs a) {
         if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) keep = keep && diff <= a.window;
       }
       if (seg_k) keep = keep && (seg_k[kpos] == seg_q);
-      s[r] = keep ? s[r] * a.scale : kNegInf;
+      s[r] = keep ? s[r] * a.scale : kMasked;
     }
     float mx = m_run;
 #pragma unroll
@@ -419,7 +421,7 @@ __global__ __launch_bounds__(256) void flash_fwd_f32_kernel(const FwdArgs a) {
   }
 
   const float l_tot = xor32_sum(l_run);
-  const float inv_l = 1.0f / l_tot;
+  const float inv_l = l_tot > 0.f ? 1.0f / l_tot : 0.f;  // a row with no visible key yields zeros
   float* op = (float*)a.out + b * a.os.b + (int64_t)(q0 + l32) * a.os.s + h * a.os.h;
 #pragma unroll
   for (int dt = 0; dt < DT; dt++)

@@ -19,7 +19,8 @@
 //     query dtype, gpu_paged_attention.py:272) and a second small kernel merges them.
 // Keys at index >= length are masked (gpu_paged_attention.py:100, gpu_decoding.py:109); the query
 // position is length-1, so a sliding window w also masks keys with (length-1) - j > w.  A page
-// index outside the pool reads as zeros (kv_cache/paged_kv_cache.py:32).
+// index outside the pool reads as zeros and a negative one counts from the end of the pool, as the
+// reference's gather does (kv_cache/paged_kv_cache.py:32).
 #include "common.h"
 
 namespace axl {
@@ -112,7 +113,8 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
 
   auto page_base = [&](int j, const __bf16* base, const Strides3& st, bool& valid) -> const __bf16* {
     if (PAGED) {
-      const int pg = __builtin_amdgcn_readfirstlane(a.page_tables[(int64_t)b * a.pps + j]);
+      int pg = __builtin_amdgcn_readfirstlane(a.page_tables[(int64_t)b * a.pps + j]);
+      if (pg < 0) pg += a.num_pages;  // negative indices count from the end, as in the reference's gather
       valid = (unsigned)pg < (unsigned)a.num_pages;
       return base + ((int64_t)hk * a.num_pages + (valid ? pg : 0)) * (kPage * D);
     } else {
@@ -167,7 +169,7 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
     bool changed = false;
 #pragma unroll
     for (int r = 0; r < 4; r++) {
-      s[r] = keep ? s[r] : kNegInf;
+      s[r] = keep ? s[r] : kMasked;
       pm[r] = row16_max(s[r]);
       const float mn = fmaxf(m_run[r], pm[r]);
       changed = changed || (mn != m_run[r]);
@@ -186,6 +188,19 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     // ---- O += P V on the coalesced V layout
+    // A page that straddles the length (or the window start) holds tokens whose probability is
+    // exactly 0; their V rows may be uninitialised pool memory, and 0 * NaN would poison the sum,
+    // so those rows are replaced by zeros.  Only boundary pages pay for this.
+    const bool boundary = (j * kPage + kPage > len) || (a.window >= 0 && len - 1 - j * kPage > a.window);
+    if (boundary) {
+#pragma unroll
+      for (int i = 0; i < NLOAD; i++) {
+        const int vpos = j * kPage + TPL * i + vtok;
+        bool vkeep = vpos < len;
+        if (a.window >= 0) vkeep = vkeep && (len - 1 - vpos <= a.window);
+        if (!vkeep) vreg[i] = uint4{0, 0, 0, 0};
+      }
+    }
     if (any_changed) {
 #pragma unroll
       for (int gq = 0; gq < GP; gq++) {

@@ -1,0 +1,181 @@
+"""Flash-attention prefill / training kernels: the HIP replacement for the Pallas path.
+
+Mirrors the kernel entry point `flash_attention(...)` (axlearn/common/flash_attention/
+gpu_attention.py:250-287, custom VJP :428-430, :789) and the dispatch class
+`PallasGPUFlashAttention` (:929-992).  Differences that follow from the machine mapping, not from
+the mathematics:
+  * KV heads are never repeated in memory: the kernels read the shared kv head (the reference
+    repeats, :975-976, and lets autodiff sum dK/dV back);
+  * the mask must be structured (none / causal / sliding window, optionally with segment ids): the
+    kernels evaluate it in closed form from block indices instead of tracing an arbitrary `mask_fn`
+    into a block map.  Anything else is reported as unsupported so the dispatch moves on.
+"""
+
+from __future__ import annotations
+
+import logging
+from typing import Optional, Tuple
+
+import torch
+
+from axlearn_amd import ops
+from axlearn_amd.attention_bias import (
+    BaseAttentionBias,
+    CausalAttentionBias,
+    MaskFn,
+    MaskFnAttentionBias,
+    SegmentIdAttentionBias,
+    SlidingWindowAttentionBias,
+    _SlidingWindowCausalMask,
+    causal_mask,
+    split,
+)
+from axlearn_amd.flash_attention.common import BaseFlashAttention, Nested, Tensor, get_segment_ids
+from axlearn_amd.kv_cache import BaseKVCache
+
+FLASH_ATTN_RESIDUAL_NAME = "flash_residuals"
+
+
+def classify_mask_fn(mask_fn: Optional[MaskFn]) -> Optional[Tuple[int, int]]:
+    """Maps a mask fn to (mask_kind, window) if the kernels can evaluate it in closed form."""
+    if mask_fn is None:
+        return ops.MASK_NONE, 0
+    if mask_fn is causal_mask:
+        return ops.MASK_CAUSAL, 0
+    if isinstance(mask_fn, _SlidingWindowCausalMask):
+        return ops.MASK_SLIDING_WINDOW, mask_fn.sliding_window_size
+    return None
+
+
+def classify_mask_bias(mask: BaseAttentionBias) -> Optional[Tuple[int, int]]:
+    if not mask.has_value():
+        return ops.MASK_NONE, 0
+    if isinstance(mask, SlidingWindowAttentionBias):
+        return ops.MASK_SLIDING_WINDOW, int(mask.sliding_window_size)
+    if isinstance(mask, CausalAttentionBias):
+        return ops.MASK_CAUSAL, 0
+    if isinstance(mask, MaskFnAttentionBias):
+        return classify_mask_fn(mask.mask)
+    return None
+
+
+class _FlashAttentionFn(torch.autograd.Function):
+    """Forward = axl_flash_fwd (saves out and lse), backward = axl_flash_bwd."""
+
+    @staticmethod
+    def forward(ctx, query, key, value, segment_ids, softmax_scale, mask_kind, window):
+        out, lse = ops.flash_fwd(
+            query, key, value, softmax_scale=softmax_scale, mask_kind=mask_kind,
+            sliding_window=window, segment_ids=segment_ids,
+        )
+        ctx.save_for_backward(query, key, value, out, lse)
+        ctx.segment_ids = segment_ids
+        ctx.args = (softmax_scale, mask_kind, window)
+        return out
+
+    @staticmethod
+    def backward(ctx, d_out):
+        query, key, value, out, lse = ctx.saved_tensors
+        softmax_scale, mask_kind, window = ctx.args
+        if d_out.stride(-1) != 1:
+            d_out = d_out.contiguous()
+        dq, dk, dv = ops.flash_bwd(
+            query, key, value, out, lse, d_out, softmax_scale=softmax_scale, mask_kind=mask_kind,
+            sliding_window=window, segment_ids=ctx.segment_ids,
+        )
+        return dq, dk, dv, None, None, None, None
+
+
+# pylint: disable-next=too-many-positional-arguments
+def flash_attention(
+    query: Tensor,
+    key: Tensor,
+    value: Tensor,
+    bias: Optional[Tensor] = None,
+    segment_ids: Optional[Tensor] = None,
+    prng_key: Optional[Tensor] = None,
+    softmax_scale: float = 1.0,
+    mask_fn: Optional[MaskFn] = None,
+    dropout_rate: float = 0.0,
+    block_q: int = 128,
+    block_k: int = 128,
+    num_warps: Optional[int] = None,
+    num_stages: Optional[int] = None,
+    grid=None,
+    interpret: bool = False,
+    debug: bool = False,
+) -> Tensor:
+    """Differentiable flash attention; same signature as gpu_attention.py:250-267.
+
+    query [B,T,Hq,D]; key/value [B,S,Hkv,D] (Hkv may be smaller than Hq); segment_ids [B,T].
+    The Pallas/Triton tuning arguments (block_q .. debug) are accepted and ignored: tiling is fixed
+    by the HIP kernels.  Dense `bias` and dropout are not implemented by the kernels.
+    """
+    del prng_key, block_q, block_k, num_warps, num_stages, grid, debug
+    if interpret:
+        raise NotImplementedError("The HIP kernels have no interpret mode; they only run on the GPU.")
+    if bias is not None:
+        raise NotImplementedError("Dense attention bias is not supported by the HIP kernels.")
+    if dropout_rate != 0.0:
+        raise NotImplementedError("Attention dropout is not supported by the HIP kernels.")
+    kind = classify_mask_fn(mask_fn)
+    if kind is None:
+        raise NotImplementedError(
+            "mask_fn must be None, causal_mask or sliding_window_causal_mask(w) for the HIP kernels."
+        )
+    return _FlashAttentionFn.apply(query, key, value, segment_ids, float(softmax_scale), kind[0], kind[1])
+
+
+class HipFlashAttention(BaseFlashAttention):
+    """MI355X flash attention (forward + backward) behind the dispatch API.
+
+    Takes the slot of `CuDNNGPUFlashAttention` / `PallasGPUFlashAttention`
+    (axlearn/common/flash_attention/utils.py:41-50)."""
+
+    def is_supported(self, input_batch: Nested, kv_cache_type: Optional[type[BaseKVCache]]) -> bool:
+        if not super().is_supported(input_batch=input_batch, kv_cache_type=kv_cache_type):
+            return False
+        if kv_cache_type is not None:
+            return self._log_unsupported(f"{kv_cache_type=} (prefill/training kernel only)")
+        query, key = input_batch["query"], input_batch["key"]
+        if not self._check_block_size(input_batch=input_batch, block_size=128):
+            return False
+        head_dim = query.shape[-1]
+        if head_dim not in (64, 128):
+            return self._log_unsupported(f"{head_dim=} (supported: 64, 128)")
+        if query.dtype not in (torch.bfloat16, torch.float32):
+            return self._log_unsupported(f"{query.dtype=} (supported: bfloat16, float32)")
+        if key.dtype != query.dtype or input_batch["value"].dtype != query.dtype:
+            return self._log_unsupported("query, key and value dtypes differ")
+        if input_batch.get("logit_sink", None) is not None:
+            return self._log_unsupported("logit sink is not supported.")
+        if self.cfg.dropout_rate != 0.0:
+            return self._log_unsupported("dropout is not supported.")
+        if not (self.cfg.softmax_scale > 0.0):
+            return self._log_unsupported(f"{self.cfg.softmax_scale=} must be positive")
+        bias: BaseAttentionBias = input_batch["bias"]
+        mask, segment_ids, explicit_bias = split(bias, MaskFnAttentionBias, SegmentIdAttentionBias)
+        if explicit_bias.has_value():
+            return self._log_unsupported("explicit (dense) bias is not supported.")
+        if classify_mask_bias(mask) is None:
+            return self._log_unsupported("mask_fn is neither causal nor sliding-window causal.")
+        if segment_ids.has_value() and query.shape[1] != key.shape[1]:
+            return self._log_unsupported("segment ids need identical query and key lengths.")
+        if not query.is_cuda:
+            return self._log_unsupported("tensors are not on the GPU.")
+        return True
+
+    def __call__(self, input_batch: Nested) -> Tensor:
+        query, key, value = input_batch["query"], input_batch["key"], input_batch["value"]
+        bias: BaseAttentionBias = input_batch["bias"]
+        mask, segment_ids, explicit_bias = split(bias, MaskFnAttentionBias, SegmentIdAttentionBias)
+        if explicit_bias.has_value():
+            raise NotImplementedError("explicit bias")
+        kind = classify_mask_bias(mask)
+        if kind is None:
+            raise NotImplementedError("unstructured mask_fn")
+        seg = get_segment_ids(query=query, key=key, segment_ids=segment_ids)
+        logging.info("HipFlashAttention: mask_kind=%d window=%d segment_ids=%s", kind[0], kind[1], seg is not None)
+        return _FlashAttentionFn.apply(
+            query, key, value, seg, float(self.cfg.softmax_scale), kind[0], kind[1]
+        )

@@ -29,6 +29,7 @@ __all__ = [
     "MASK_SLIDING_WINDOW",
     "flash_fwd",
     "flash_bwd",
+    "flash_bwd_buffers",
     "paged_decode",
     "decode",
 ]
@@ -96,15 +97,24 @@ def flash_bwd(
     sliding_window: int = 0,
     segment_ids: Optional[torch.Tensor] = None,
     q_pos_offset: int = 0,
+    phases: int = 7,
+    buffers=None,
 ):
-    """Returns (dq [B,T,Hq,D], dk [B,S,Hkv,D], dv [B,S,Hkv,D]) in the dtype of q."""
+    """Returns (dq [B,T,Hq,D], dk [B,S,Hkv,D], dv [B,S,Hkv,D]) in the dtype of q.
+
+    `phases` selects a subset of {1: delta, 2: dK/dV, 4: dQ} (timing / profiling only); `buffers`
+    = (dq, dk, dv, workspace) reuses caller-provided outputs instead of allocating."""
     _require_cuda(q, k, v, out, lse, d_out, segment_ids)
     lib = _lib.load()
     b, t, hq, d = q.shape
     s, hkv = k.shape[1], k.shape[2]
-    dq = torch.empty((b, t, hq, d), dtype=q.dtype, device=q.device)
-    dk = torch.empty((b, s, hkv, d), dtype=k.dtype, device=q.device)
-    dv = torch.empty((b, s, hkv, d), dtype=v.dtype, device=q.device)
+    ws = None
+    if buffers is not None:
+        dq, dk, dv, ws = buffers
+    else:
+        dq = torch.empty((b, t, hq, d), dtype=q.dtype, device=q.device)
+        dk = torch.empty((b, s, hkv, d), dtype=k.dtype, device=q.device)
+        dv = torch.empty((b, s, hkv, d), dtype=v.dtype, device=q.device)
     seg = _seg(segment_ids)
     if lse.dtype != torch.float32 or not lse.is_contiguous():
         raise AxlError(_lib.AXL_ERR_INVALID_ARGUMENT, "lse must be contiguous float32 [B,Hq,T]")
@@ -121,11 +131,19 @@ def flash_bwd(
         workspace=None, workspace_bytes=0,
     )
     need = lib.axl_flash_bwd_workspace_bytes(ctypes.byref(p))
-    ws = torch.empty((max(int(need), 16),), dtype=torch.uint8, device=q.device)
+    if ws is None or ws.numel() * ws.element_size() < need:
+        ws = torch.empty((max(int(need), 16),), dtype=torch.uint8, device=q.device)
     p.workspace = ws.data_ptr()
-    p.workspace_bytes = ws.numel()
-    _lib.check(lib.axl_flash_bwd(ctypes.byref(p), _lib.current_stream_ptr()))
+    p.workspace_bytes = ws.numel() * ws.element_size()
+    _lib.check(lib.axl_flash_bwd_phases(ctypes.byref(p), int(phases), _lib.current_stream_ptr()))
     return dq, dk, dv
+
+
+def flash_bwd_buffers(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor):
+    """Pre-allocates (dq, dk, dv, workspace) for repeated `flash_bwd(..., buffers=...)` calls."""
+    b, t, hq, _ = q.shape
+    ws = torch.empty((b * hq * t * 4,), dtype=torch.uint8, device=q.device)
+    return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), ws
 
 
 def paged_decode(

@@ -1,0 +1,286 @@
+"""Benchmark of the MI355X attention kernel path (one GPU).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c5] [--no-cpu-baseline]
+
+Default workload (BASELINE.json configs[1], "C2"): causal GQA flash attention forward + backward,
+bf16, batch 4, 32 query heads / 8 kv heads, seq 4096, head_dim 128.  A step is one forward
+(axl_flash_fwd) plus one backward (axl_flash_bwd) over one synthetic batch already resident in HBM.
+The paged-decode half of the metric (configs[3], "C4") is measured in the same run and reported in
+the `paged_decode` object of the same JSON line.
+
+Prints ONE JSON line.  `value` = algorithmic TFLOP/s of fwd+bwd (4*B*Hq*T^2*D/2 forward, 2.5x that
+backward).  `roofline` describes the dominant kernel (the dK/dV backward kernel), timed with device
+events around its own launches on the stream it runs on.  `cpu_baseline` times the CPU oracle
+(oracle/ref_attention.py, a restatement of the reference's XLA attention) on a bounded slice of the
+same workload on this machine's host cores.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+HBM_PEAK_GBS = 8000.0           # MI355X HBM3E
+
+METRIC = "flash-attn fwd+bwd TFLOP/s; paged-decode HBM GB/s (% roofline), 1 MI355X"
+
+
+def _events(n):
+    return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+
+
+def _time_region(fn, steps, warmup):
+    """Runs warmup + steps calls of fn; returns ms per step from device events on torch's current
+    stream (the stream every C-ABI call is enqueued on)."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = _events(2)
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+
+def _flash_workload(name):
+    if name == "c2":
+        return dict(label="C2: causal GQA flash fwd+bwd, bf16, B4 Hq32/Hkv8 T4096 D128",
+                    B=4, T=4096, Hq=32, Hkv=8, D=128, mask="causal", window=0, seg=False)
+    if name == "c3":
+        return dict(label="C3: sliding-window(4096) causal MHA + segment ids fwd+bwd, bf16, B8 H16 T8192 D128",
+                    B=8, T=8192, Hq=16, Hkv=16, D=128, mask="sliding", window=4096, seg=True)
+    if name == "c5":
+        return dict(label="C5: long-context causal GQA fwd+bwd, bf16, B1 Hq64/Hkv8 T32768 D128",
+                    B=1, T=32768, Hq=64, Hkv=8, D=128, mask="causal", window=0, seg=False)
+    raise ValueError(name)
+
+
+def packed_segment_ids(seed, batch, seq_len, max_docs=6):
+    """Per row: n ~ U{1..max_docs} documents split at n-1 distinct uniform cut points; ids are the
+    1-based document index (id 0 is reserved for padding)."""
+    rng = np.random.default_rng(seed)
+    out = np.ones((batch, seq_len), dtype=np.int32)
+    for b in range(batch):
+        n = int(rng.integers(1, max_docs + 1))
+        if n > 1:
+            for c in np.sort(rng.choice(np.arange(1, seq_len), size=n - 1, replace=False)):
+                out[b, c:] += 1
+    return torch.from_numpy(out)
+
+
+def count_pairs(seg, window):
+    """Exact number of (batch, query, key) pairs kept by sliding-window-causal AND equal segment."""
+    B, T = seg.shape
+    pos = torch.arange(T, device=seg.device)
+    total = 0
+    for t0 in range(0, T, 1024):
+        qp = pos[t0:t0 + 1024, None]
+        keep = (qp >= pos[None, :]) & (qp - pos[None, :] <= window)
+        keep = keep[None] & (seg[:, t0:t0 + 1024, None] == seg[:, None, :])
+        total += int(keep.sum())
+    return total
+
+
+def bench_flash(cfg, steps, warmup, cpu_baseline):
+    from axlearn_amd import ops
+
+    dev = torch.device("cuda:0")
+    B, T, Hq, Hkv, D = cfg["B"], cfg["T"], cfg["Hq"], cfg["Hkv"], cfg["D"]
+    gen = torch.Generator(device=dev).manual_seed(0)
+    bf = torch.bfloat16
+    q = torch.randn((B, T, Hq, D), device=dev, dtype=torch.float32, generator=gen).to(bf)
+    k = torch.randn((B, T, Hkv, D), device=dev, dtype=torch.float32, generator=gen).to(bf)
+    v = torch.randn((B, T, Hkv, D), device=dev, dtype=torch.float32, generator=gen).to(bf)
+    do = torch.randn((B, T, Hq, D), device=dev, dtype=torch.float32, generator=gen).to(bf)
+    seg = None
+    pairs = None
+    if cfg["seg"]:
+        seg = packed_segment_ids(4, B, T).to(dev)
+        pairs = count_pairs(seg, cfg["window"])
+    mask_kind = {"none": ops.MASK_NONE, "causal": ops.MASK_CAUSAL, "sliding": ops.MASK_SLIDING_WINDOW}[cfg["mask"]]
+    kw = dict(softmax_scale=D ** -0.5, mask_kind=mask_kind, sliding_window=cfg["window"], segment_ids=seg)
+    bufs = ops.flash_bwd_buffers(q, k, v)
+    out, lse = ops.flash_fwd(q, k, v, **kw)
+
+    def step():
+        o, l = ops.flash_fwd(q, k, v, **kw)
+        ops.flash_bwd(q, k, v, o, l, do, buffers=bufs, **kw)
+
+    ms_step = _time_region(step, steps, warmup)
+    # Per-kernel durations, each kernel timed over its own launches.
+    ms_fwd = _time_region(lambda: ops.flash_fwd(q, k, v, **kw), steps, 1)
+    ms_delta = _time_region(lambda: ops.flash_bwd(q, k, v, out, lse, do, buffers=bufs, phases=1, **kw), steps, 1)
+    ms_dkdv = _time_region(lambda: ops.flash_bwd(q, k, v, out, lse, do, buffers=bufs, phases=2, **kw), steps, 1)
+    ms_dq = _time_region(lambda: ops.flash_bwd(q, k, v, out, lse, do, buffers=bufs, phases=4, **kw), steps, 1)
+
+    if pairs is None:
+        gemm = 2.0 * B * Hq * (T * T / 2.0) * D  # one [T,T,D] causal GEMM (the 1/2 convention)
+    else:
+        gemm = 2.0 * Hq * pairs * D               # exact count of unmasked (q,k) pairs
+    fl_fwd, fl_bwd = 2 * gemm, 5 * gemm
+    fl_dkdv, fl_dq = 4 * gemm, 1 * gemm           # S, dP, dV, dK | dQ
+    tf = lambda fl, ms: fl / (ms * 1e-3) / 1e12
+    result = dict(
+        value=tf(fl_fwd + fl_bwd, ms_step), ms_per_step=ms_step,
+        kernels={
+            "flash_fwd_bf16_kernel": dict(ms=ms_fwd, tflops=tf(fl_fwd, ms_fwd), algorithmic_tflop=fl_fwd / 1e12),
+            "bwd_delta_kernel": dict(ms=ms_delta),
+            "flash_bwd_dkdv_bf16_kernel": dict(ms=ms_dkdv, tflops=tf(fl_dkdv, ms_dkdv), algorithmic_tflop=fl_dkdv / 1e12),
+            "flash_bwd_dq_bf16_kernel": dict(ms=ms_dq, tflops=tf(fl_dq, ms_dq), algorithmic_tflop=fl_dq / 1e12),
+        },
+        roofline=dict(
+            kernel="flash_bwd_dkdv_bf16_kernel", bound="mfma", achieved=tf(fl_dkdv, ms_dkdv),
+            peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s", frac=tf(fl_dkdv, ms_dkdv) / MFMA_BF16_PEAK_TFLOPS,
+            traffic=None,
+        ),
+        step_frac_of_mfma_peak=tf(fl_fwd + fl_bwd, ms_step) / MFMA_BF16_PEAK_TFLOPS,
+    )
+    if cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline_flash(cfg)
+    return result
+
+
+def cpu_baseline_flash(cfg):
+    """Times the oracle's fwd+bwd (reverse-mode autodiff of the ReferenceMHA restatement, fp32 math
+    on bf16-rounded inputs) on a slice of the workload: batch element 0, kv heads [0, nkv)."""
+    from oracle import ref_attention as ref
+
+    T, Hq, Hkv, D = cfg["T"], cfg["Hq"], cfg["Hkv"], cfg["D"]
+    G = Hq // Hkv
+    cores = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    nkv = 1
+    t_cap = min(T, 4096)  # rows [0, t_cap) of the causal problem: a self-contained causal sub-problem
+    q = ref.normal_tensor(0, (1, t_cap, nkv * G, D), torch.bfloat16)
+    k = ref.normal_tensor(1, (1, t_cap, nkv, D), torch.bfloat16)
+    v = ref.normal_tensor(2, (1, t_cap, nkv, D), torch.bfloat16)
+    do = ref.normal_tensor(3, (1, t_cap, nkv * G, D), torch.bfloat16)
+    seg = ref.packed_segment_ids(4, 1, t_cap) if cfg["seg"] else None
+    spec = ref.MaskSpec(causal=cfg["mask"] == "causal",
+                        sliding_window=cfg["window"] if cfg["mask"] == "sliding" else None, segment_ids=seg)
+    t0 = time.perf_counter()
+    reps = 0
+    while True:
+        ref.reference_mha_grads(q, k, v, do, spec, softmax_scale=D ** -0.5, row_block=512, dtype=torch.float32)
+        reps += 1
+        dt = time.perf_counter() - t0
+        if dt > 10.0 or reps >= 8:
+            break
+    pairs = ref.count_unmasked_pairs(spec, 1, t_cap, t_cap) if cfg["seg"] else t_cap * t_cap / 2.0
+    flops = 7.0 * 2.0 * (nkv * G) * pairs * D  # fwd (2 GEMMs) + bwd (5 GEMMs), algorithmic
+    return dict(
+        value=flops * reps / dt / 1e12, unit="TFLOP/s", cores=cores, kind="port",
+        sample=f"oracle fwd+bwd (torch-CPU autodiff, fp32) on batch 0, {nkv} kv head ({nkv * G} query heads), "
+               f"rows 0..{t_cap - 1}; {reps} repetitions in {dt:.1f} s",
+    )
+
+
+def bench_paged_decode(steps, warmup, cpu_baseline):
+    """C4: B64, Hq32/Hkv8, D128, page 16, pool of 64*2048 pages, lengths U[512, 32768]."""
+    from axlearn_amd import ops
+
+    dev = torch.device("cuda:0")
+    B, Hq, Hkv, D, page, pps = 64, 32, 8, 128, 16, 2048
+    P = B * pps
+    gen = torch.Generator(device=dev).manual_seed(1)
+    bf = torch.bfloat16
+    kp = torch.empty((Hkv, P, page, D), device=dev, dtype=bf)
+    vp = torch.empty((Hkv, P, page, D), device=dev, dtype=bf)
+    for h in range(Hkv):  # generate per head to bound the fp32 staging buffer
+        kp[h] = torch.randn((P, page, D), device=dev, dtype=torch.float32, generator=gen).to(bf)
+        vp[h] = torch.randn((P, page, D), device=dev, dtype=torch.float32, generator=gen).to(bf)
+    q = torch.randn((B, Hq, D), device=dev, dtype=torch.float32, generator=gen).to(bf)
+    lengths_cpu = torch.from_numpy(np.random.default_rng(5).integers(512, 32769, size=B).astype(np.int32))
+    tables_cpu = torch.from_numpy(np.random.default_rng(6).permutation(P).astype(np.int32)).reshape(B, pps)
+    lengths, tables = lengths_cpu.to(dev), tables_cpu.to(dev)
+    out = torch.empty((B, Hq, D), device=dev, dtype=bf)
+    ws = torch.empty((64 << 20,), device=dev, dtype=torch.uint8)
+    scale = D ** -0.5
+    fn = lambda: ops.paged_decode(q, kp, vp, tables, lengths, softmax_scale=scale, workspace=ws, out=out)
+    ms = _time_region(fn, steps, warmup)
+    live_pages = int(((lengths_cpu.long() + page - 1) // page).sum())
+    # Algorithmic bytes: every live K and V page once, its page-table entry, q and out.
+    algo_bytes = live_pages * page * Hkv * D * 2 * 2 + live_pages * 4 + 2 * B * Hq * D * 2
+    gbs = algo_bytes / (ms * 1e-3) / 1e9
+    res = dict(
+        workload="C4: paged decode, bf16, B64 Hq32/Hkv8 D128, page 16, ctx U[512,32768]",
+        value=gbs, unit="GB/s", ms_per_step=ms, algorithmic_gb=algo_bytes / 1e9,
+        roofline=dict(kernel="decode_split_kernel", bound="hbm", achieved=gbs, peak=HBM_PEAK_GBS, unit="GB/s",
+                      frac=gbs / HBM_PEAK_GBS, traffic=None),
+    )
+    if cpu_baseline:
+        from oracle import ref_attention as ref
+
+        nb = 2  # sequences timed on the CPU
+        cores = min(os.cpu_count() or 1, 16)
+        torch.set_num_threads(cores)
+        kc, vc = kp.cpu(), vp.cpu()
+        qc = q[:nb].cpu().unsqueeze(1)
+        t0 = time.perf_counter()
+        ref.reference_decode(qc, kc, vc, lengths_cpu[:nb], softmax_scale=scale, page_tables=tables_cpu[:nb], mode="faithful")
+        dt = time.perf_counter() - t0
+        nbytes = int(((lengths_cpu[:nb].long() + page - 1) // page).sum()) * page * Hkv * D * 2 * 2
+        res["cpu_baseline"] = dict(
+            value=nbytes / dt / 1e9, unit="GB/s", cores=cores, kind="port",
+            sample=f"oracle ReferenceMHA restatement (page gather + dense attention) on sequences 0..{nb - 1}, {dt:.2f} s",
+        )
+        del kc, vc
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4", "c5"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-decode", action="store_true", help="skip the paged-decode half of the metric")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU only (no collectives, no sharding); use --gpus 1.")
+    if int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: launched with WORLD_SIZE > 1; this build runs on one GPU only.")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the HIP kernels have no CPU path.")
+    cpu_base = not args.no_cpu_baseline
+
+    line = dict(metric=METRIC, n_gpus=1, steps=args.steps, warmup=args.warmup, higher_is_better=True,
+                scaling="weak", vs_baseline=None, dtype="bf16", data="synthetic")
+    if args.workload == "c4":
+        dec = bench_paged_decode(args.steps, args.warmup, cpu_base)
+        line.update(value=dec["value"], unit="GB/s", ms_per_step=dec["ms_per_step"],
+                    config=dict(workload=dec["workload"]), roofline=dec["roofline"])
+        if "cpu_baseline" in dec:
+            line["cpu_baseline"] = dec["cpu_baseline"]
+        line["paged_decode"] = dec
+    else:
+        cfg = _flash_workload(args.workload)
+        res = bench_flash(cfg, args.steps, args.warmup, cpu_base)
+        line.update(value=res["value"], unit="TFLOP/s", ms_per_step=res["ms_per_step"],
+                    config=dict(workload=cfg["label"], batch=cfg["B"], seq_len=cfg["T"], num_q_heads=cfg["Hq"],
+                                num_kv_heads=cfg["Hkv"], head_dim=cfg["D"], mask=cfg["mask"], window=cfg["window"],
+                                segment_ids=cfg["seg"]),
+                    roofline=res["roofline"], kernels=res["kernels"],
+                    step_frac_of_mfma_peak=res["step_frac_of_mfma_peak"])
+        if "cpu_baseline" in res:
+            line["cpu_baseline"] = res["cpu_baseline"]
+        if not args.no_decode:
+            line["paged_decode"] = bench_paged_decode(args.steps, args.warmup, cpu_base)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -115,6 +115,18 @@ size_t axl_flash_bwd_workspace_bytes(const AxlFlashBwdParams* params);
 int axl_flash_bwd(const AxlFlashBwdParams* params, void* stream);
 
 /*
+ * Runs a subset of the backward's kernels, for per-kernel timing and profiling: `phases` is a
+ * bit mask of AXL_BWD_DELTA (delta pre-pass, gpu_attention.py:653-658), AXL_BWD_DKDV
+ * (`_mha_backward_kernel_dkdv`, :436-528) and AXL_BWD_DQ (`_mha_backward_kernel_dq`, :533-616), the
+ * three launches `_mha_backward` makes.  The dK/dV and dQ phases read the delta a previous DELTA
+ * phase left in the same workspace.  axl_flash_bwd(p, s) == axl_flash_bwd_phases(p, 7, s).
+ */
+#define AXL_BWD_DELTA 1
+#define AXL_BWD_DKDV 2
+#define AXL_BWD_DQ 4
+int axl_flash_bwd_phases(const AxlFlashBwdParams* params, int phases, void* stream);
+
+/*
  * Paged-attention decode (one query token per sequence).
  * Replaces: `GPUPagedAttention.__call__` -> vmap(_paged_attention_unbatched) ->
  *   pallas_call(paged_attention_*) + the XLA combine
@@ -122,8 +134,9 @@ int axl_flash_bwd(const AxlFlashBwdParams* params, void* stream);
  *   q [B,Hq,D]; k_pages, v_pages [Hkv, num_pages, page_size, D]; page_tables [B, pages_per_seq]
  *   int32: token j of sequence b is k_pages[h][page_tables[b][j / page_size]][j % page_size]
  *   (axlearn/common/kv_cache/paged_kv_cache.py:21-34); lengths [B] int32: keys j >= lengths[b] are
- *   masked (:100); the query sits at position lengths[b]-1 (:344).  Page indices outside
- *   [0, num_pages) read as zeros, as `reconstruct_kv` does.  out [B,Hq,D] in the dtype of q.
+ *   masked (:100); the query sits at position lengths[b]-1 (:344).  As in `reconstruct_kv`, a page
+ *   index in [-num_pages, 0) counts from the end of the pool and any other index outside
+ *   [0, num_pages) reads as zeros.  out [B,Hq,D] in the dtype of q.
  *   sliding_window < 0 disables the window; otherwise keys with (len-1) - j > w are masked too.
  *   workspace: axl_paged_decode_workspace_bytes(params) bytes (fp32 split-K partials).
  */

@@ -1,0 +1,190 @@
+"""GPU parity tests of the paged and contiguous single-token decode kernels against the CPU oracle.
+
+Shapes follow the reference's decoding tests (decoding_test.py:95-163, :187-269): (B, S, H, D) in
+{(1,1024,32,64), (4,512,48,64), (2,1024,16,128), (1,4096,8,128)}, padding in {0, 111},
+kv_head_factor in {1, 8}, window in {-1, 127}, page size 16.  Page-table and length masking are
+checked bit-exactly (permutation invariance, poison).
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from axlearn_amd import attention_bias as ab
+from axlearn_amd import ops
+from axlearn_amd.flash_attention.hip_decoding import HipDecoding, HipPagedAttention
+from axlearn_amd.flash_attention.utils import flash_attention_implementation
+from axlearn_amd.kv_cache import KVCache, PagedKVCache
+from oracle import brute
+from oracle import ref_attention as ref
+
+pytestmark = pytest.mark.gpu
+
+
+def _ok(got, want):
+    return ref.max_abs(got, want) <= 2e-2 or ref.rel_l2(got, want) <= 1e-2
+
+
+@pytest.mark.parametrize("b,s,h,d", [(1, 1024, 32, 64), (4, 512, 48, 64), (2, 1024, 16, 128), (1, 4096, 8, 128)])
+@pytest.mark.parametrize("padding", [0, 111])
+@pytest.mark.parametrize("kv_head_factor", [1, 8])
+@pytest.mark.parametrize("window", [-1, 127])
+def test_paged_and_contiguous_decode_against_ref(b, s, h, d, padding, kv_head_factor, window):
+    hkv = h // kv_head_factor
+    pps = s // 16
+    q, kp, vp, tables, _ = ref.paged_inputs(3, batch=b, num_heads=h, num_kv_heads=hkv, head_dim=d, page_size=16,
+                                            pages_per_seq=pps, min_len=1, max_len=s)
+    lengths = torch.full((b,), s - padding, dtype=torch.int32)
+    scale = d ** -0.5
+    want = ref.reference_decode(q, kp, vp, lengths, softmax_scale=scale, page_tables=tables,
+                                sliding_window=None if window < 0 else window)[:, 0]
+    got = ops.paged_decode(q[:, 0].cuda(), kp.cuda(), vp.cuda(), tables.cuda(), lengths.cuda(),
+                           softmax_scale=scale, sliding_window=window)
+    assert _ok(got.cpu(), want), (ref.max_abs(got.cpu(), want), ref.rel_l2(got.cpu(), want))
+    kk, vv = ref.reconstruct_kv(tables, kp), ref.reconstruct_kv(tables, vp)
+    got2 = ops.decode(q[:, 0].cuda(), kk.cuda(), vv.cuda(), lengths.cuda(), softmax_scale=scale, sliding_window=window)
+    assert _ok(got2.cpu(), want)
+    # Same arithmetic on the same tokens in the same order: paged and contiguous agree bit for bit.
+    assert torch.equal(got, got2)
+
+
+def test_ragged_lengths_and_brute_force():
+    b, hq, hkv, d, pps = 5, 8, 2, 128, 24
+    q, kp, vp, tables, lengths = ref.paged_inputs(7, batch=b, num_heads=hq, num_kv_heads=hkv, head_dim=d,
+                                                  page_size=16, pages_per_seq=pps, min_len=1, max_len=16 * pps)
+    lengths[0], lengths[1], lengths[2] = 1, 16, 17  # single token, exactly one page, one page + 1
+    scale = 0.11
+    want = brute.paged_decode(q[:, 0].float().numpy(), kp.float().numpy(), vp.float().numpy(), tables.numpy(),
+                              lengths.numpy(), scale=scale)
+    got = ops.paged_decode(q[:, 0].cuda(), kp.cuda(), vp.cuda(), tables.cuda(), lengths.cuda(), softmax_scale=scale)
+    assert _ok(got.cpu(), torch.from_numpy(want))
+    # A single live token: the output is that token's V row exactly.
+    first = int(tables[0, 0])
+    g = hq // hkv
+    for hh in range(hq):
+        assert torch.equal(got[0, hh].cpu(), vp[hh // g, first, 0])
+
+
+def test_page_table_permutation_invariance_bit_exact():
+    b, hq, hkv, d, pps = 4, 8, 2, 128, 40
+    q, kp, vp, tables, lengths = ref.paged_inputs(9, batch=b, num_heads=hq, num_kv_heads=hkv, head_dim=d,
+                                                  page_size=16, pages_per_seq=pps, min_len=30, max_len=16 * pps)
+    base = ops.paged_decode(q[:, 0].cuda(), kp.cuda(), vp.cuda(), tables.cuda(), lengths.cuda(), softmax_scale=0.09)
+    total = b * pps
+    perm = torch.from_numpy(np.random.default_rng(1).permutation(total))
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(total)
+    tables2 = inv[tables.long()].to(torch.int32)
+    again = ops.paged_decode(q[:, 0].cuda(), kp[:, perm].contiguous().cuda(), vp[:, perm].contiguous().cuda(),
+                             tables2.cuda(), lengths.cuda(), softmax_scale=0.09)
+    assert torch.equal(base, again)
+
+
+def test_length_masking_poison_and_oob_pages():
+    b, hq, hkv, d, pps = 3, 4, 1, 128, 20
+    q, kp, vp, tables, lengths = ref.paged_inputs(13, batch=b, num_heads=hq, num_kv_heads=hkv, head_dim=d,
+                                                  page_size=16, pages_per_seq=pps, min_len=10, max_len=16 * pps - 40)
+    qc, tc, lc = q[:, 0].cuda(), tables.cuda(), lengths.cuda()
+    base = ops.paged_decode(qc, kp.cuda(), vp.cuda(), tc, lc, softmax_scale=0.1)
+    kpo, vpo = kp.clone(), vp.clone()
+    for bi in range(b):
+        n = int(lengths[bi])
+        for j in range(n, 16 * pps):  # every token at or beyond the length, incl. whole unused pages
+            pg = int(tables[bi, j // 16])
+            kpo[:, pg, j % 16] = float("nan")
+            vpo[:, pg, j % 16] = float("nan")
+    poisoned = ops.paged_decode(qc, kpo.cuda(), vpo.cuda(), tc, lc, softmax_scale=0.1)
+    assert torch.equal(base, poisoned) and torch.isfinite(poisoned.float()).all()
+    # Out-of-pool page index inside the live range reads as zeros and a negative one counts from
+    # the end of the pool, like reconstruct_kv.
+    t2 = tables.clone()
+    t2[0, 0] = b * pps + 5
+    t2[1, 0] = -3
+    lengths2 = torch.maximum(lengths, torch.tensor(40, dtype=torch.int32))
+    want = ref.reference_decode(q, kp, vp, lengths2, softmax_scale=0.1, page_tables=t2)[:, 0]
+    got = ops.paged_decode(qc, kp.cuda(), vp.cuda(), t2.cuda(), lengths2.cuda(), softmax_scale=0.1)
+    assert _ok(got.cpu(), want)
+
+
+def test_decode_equals_last_row_of_prefill():
+    b, hq, hkv, d, s = 2, 8, 2, 128, 512
+    k = ref.normal_tensor(1, (b, s, hkv, d), torch.bfloat16).cuda()
+    v = ref.normal_tensor(2, (b, s, hkv, d), torch.bfloat16).cuda()
+    q = ref.normal_tensor(0, (b, s, hq, d), torch.bfloat16).cuda()
+    full, _ = ops.flash_fwd(q, k, v, softmax_scale=d ** -0.5, mask_kind=ops.MASK_CAUSAL)
+    lengths = torch.full((b,), s, dtype=torch.int32).cuda()
+    dec = ops.decode(q[:, -1].contiguous(), k, v, lengths, softmax_scale=d ** -0.5)
+    assert _ok(dec.cpu(), full[:, -1].cpu())
+
+
+def test_dispatch_decode_end_to_end():
+    b, hq, hkv, d, pps = 4, 16, 2, 64, 32
+    q, kp, vp, tables, lengths = ref.paged_inputs(21, batch=b, num_heads=hq, num_kv_heads=hkv, head_dim=d,
+                                                  page_size=16, pages_per_seq=pps, min_len=5, max_len=16 * pps)
+    tp = (lengths.long() - 1)[:, None].cuda()
+    sp = torch.arange(16 * pps)[None].cuda()
+    scale = d ** -0.5
+    bias = ab.CompositeAttentionBias([ab.CausalAttentionBias(target_positions=tp, source_positions=sp)])
+    args = dict(query=q.cuda(), key=kp.cuda(), value=vp.cuda(), bias=bias)
+    impl = flash_attention_implementation("gpu", **args, softmax_scale=scale, kv_cache_type=PagedKVCache,
+                                          page_tables=tables.cuda())
+    assert impl is not None and isinstance(impl.fn, HipPagedAttention)
+    got = impl.fn(dict(**args, page_tables=tables.cuda()))
+    want = ref.reference_decode(q, kp, vp, lengths, softmax_scale=scale, page_tables=tables)
+    assert got.shape == (b, 1, hq, d) and _ok(got.cpu(), want)
+    # Contiguous cache through the non-paged table; sliding-window bias.
+    kk, vv = ref.reconstruct_kv(tables, kp).cuda(), ref.reconstruct_kv(tables, vp).cuda()
+    wbias = ab.CompositeAttentionBias([ab.SlidingWindowAttentionBias(
+        ab.sliding_window_causal_mask(50), sliding_window_size=50, target_positions=tp, source_positions=sp)])
+    impl = flash_attention_implementation("gpu", query=q.cuda(), key=kk, value=vv, bias=wbias, softmax_scale=scale,
+                                          kv_cache_type=KVCache)
+    assert impl is not None and isinstance(impl.fn, HipDecoding)
+    got = impl.fn(dict(query=q.cuda(), key=kk, value=vv, bias=wbias))
+    want = ref.reference_decode(q, kp, vp, lengths, softmax_scale=scale, page_tables=tables, sliding_window=50)
+    assert _ok(got.cpu(), want)
+    # Multi-token query with a KV cache is not a decode step: the decode kernel declines and the
+    # prefill kernel does not take cached calls either -> None.
+    q2 = torch.zeros(b, 2, hq, d, dtype=torch.bfloat16, device="cuda")
+    assert flash_attention_implementation("gpu", query=q2, key=kk, value=vv, bias=wbias, kv_cache_type=KVCache) is None
+
+
+def test_baseline_c4_full_size():
+    """BASELINE config 4 at full size; the oracle checks a sample of sequences (incl. the shortest
+    and the longest), the rest is covered by permutation invariance at full size."""
+    B, Hq, Hkv, D, pps = 64, 32, 8, 128, 2048
+    P = B * pps
+    dev = "cuda"
+    gen = torch.Generator(device=dev).manual_seed(1)
+    kp = torch.empty((Hkv, P, 16, D), device=dev, dtype=torch.bfloat16)
+    vp = torch.empty((Hkv, P, 16, D), device=dev, dtype=torch.bfloat16)
+    for h in range(Hkv):
+        kp[h] = torch.randn((P, 16, D), device=dev, generator=gen).to(torch.bfloat16)
+        vp[h] = torch.randn((P, 16, D), device=dev, generator=gen).to(torch.bfloat16)
+    q = torch.randn((B, Hq, D), device=dev, generator=gen).to(torch.bfloat16)
+    lengths = torch.from_numpy(np.random.default_rng(5).integers(512, 32769, size=B).astype(np.int32))
+    tables = torch.from_numpy(np.random.default_rng(6).permutation(P).astype(np.int32)).reshape(B, pps)
+    scale = D ** -0.5
+    out = ops.paged_decode(q, kp, vp, tables.to(dev), lengths.to(dev), softmax_scale=scale)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+    sample = sorted({0, 17, int(lengths.argmin()), int(lengths.argmax())})
+    for bi in sample:
+        n_pages = (int(lengths[bi]) + 15) // 16
+        idx = tables[bi, :n_pages].long().to(dev)
+        k_seq = kp[:, idx].cpu()  # [Hkv, n_pages, 16, D]
+        v_seq = vp[:, idx].cpu()
+        local = torch.arange(n_pages, dtype=torch.int32)[None]
+        want = ref.reference_decode(q[bi:bi + 1].cpu().unsqueeze(1), k_seq, v_seq, lengths[bi:bi + 1],
+                                    softmax_scale=scale, page_tables=local)[:, 0]
+        assert _ok(out[bi:bi + 1].cpu(), want), bi
+    # Swap the physical location of two sequences' pages (pool-level permutation on a slice).
+    tables2 = tables.clone()
+    a, c = tables2[3].clone(), tables2[40].clone()
+    kp2, vp2 = kp, vp  # in place: swap page contents and table entries
+    ka, kc = kp2[:, a.long().to(dev)].clone(), kp2[:, c.long().to(dev)].clone()
+    va, vc = vp2[:, a.long().to(dev)].clone(), vp2[:, c.long().to(dev)].clone()
+    kp2[:, a.long().to(dev)], kp2[:, c.long().to(dev)] = kc, ka
+    vp2[:, a.long().to(dev)], vp2[:, c.long().to(dev)] = vc, va
+    tables2[3], tables2[40] = c, a
+    out2 = ops.paged_decode(q, kp2, vp2, tables2.to(dev), lengths.to(dev), softmax_scale=scale)
+    assert torch.equal(out, out2)

@@ -1,0 +1,327 @@
+"""GPU parity tests of the flash-attention forward/backward kernels against the CPU oracle.
+
+Tolerances are the ones the task states: fp32 <= 1e-5 max-abs; bf16 (fp32 accumulation) <= 2e-2
+max-abs OR <= 1e-2 relative-L2, measured against the oracle's float64 evaluation of the same
+bf16-rounded inputs.  Masking is checked bit-exactly through poison tests.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from axlearn_amd import attention_bias as ab
+from axlearn_amd import ops
+from axlearn_amd.flash_attention.hip_attention import HipFlashAttention, flash_attention
+from axlearn_amd.flash_attention.utils import flash_attention_implementation
+from oracle import brute
+from oracle import ref_attention as ref
+
+pytestmark = pytest.mark.gpu
+
+BF16_MAX_ABS, BF16_REL_L2, FP32_MAX_ABS = 2e-2, 1e-2, 1e-5
+
+
+def _ok_bf16(got, want):
+    return ref.max_abs(got, want) <= BF16_MAX_ABS or ref.rel_l2(got, want) <= BF16_REL_L2
+
+
+def _assert_close(name, got, want, dtype):
+    got = got.detach().cpu()
+    if dtype == torch.float32:
+        err = ref.max_abs(got, want)
+        assert err <= FP32_MAX_ABS, f"{name}: max-abs {err:.3e}"
+    else:
+        assert _ok_bf16(got, want), f"{name}: max-abs {ref.max_abs(got, want):.3e} rel-L2 {ref.rel_l2(got, want):.3e}"
+    assert torch.isfinite(got.float()).all(), name
+
+
+def _inputs(b, t, hq, hkv, d, dtype, s=None):
+    s = s or t
+    q = ref.normal_tensor(0, (b, t, hq, d), dtype)
+    k = ref.normal_tensor(1, (b, s, hkv, d), dtype)
+    v = ref.normal_tensor(2, (b, s, hkv, d), dtype)
+    do = ref.normal_tensor(3, (b, t, hq, d), dtype)
+    return q, k, v, do
+
+
+def _mask_args(kind, window, seg):
+    spec = ref.MaskSpec(causal=kind == "causal", sliding_window=window if kind == "sliding" else None, segment_ids=seg)
+    mk = {"none": ops.MASK_NONE, "causal": ops.MASK_CAUSAL, "sliding": ops.MASK_SLIDING_WINDOW}[kind]
+    return spec, dict(mask_kind=mk, sliding_window=window or 0, segment_ids=None if seg is None else seg.cuda())
+
+
+FWD_CASES = [
+    # b, t, hq, hkv, d, dtype, mask, window, seg      (shapes follow gpu_attention_test.py:105-130)
+    (1, 128, 1, 1, 128, torch.bfloat16, "none", None, False),
+    (2, 256, 4, 4, 64, torch.bfloat16, "causal", None, False),
+    (1, 384, 8, 2, 128, torch.bfloat16, "causal", None, False),
+    (2, 512, 4, 1, 128, torch.bfloat16, "causal", None, True),
+    (2, 512, 2, 2, 64, torch.bfloat16, "sliding", 127, False),
+    (1, 1024, 4, 2, 128, torch.bfloat16, "sliding", 128, True),
+    (1, 1024, 2, 2, 128, torch.bfloat16, "sliding", 129, False),
+    (1, 512, 2, 1, 128, torch.bfloat16, "sliding", 0, False),
+    (1, 256, 2, 2, 128, torch.bfloat16, "none", None, True),
+    (2, 512, 4, 4, 64, torch.float32, "causal", None, False),  # BASELINE config 1
+    (1, 256, 4, 2, 128, torch.float32, "sliding", 100, True),
+    (1, 256, 2, 2, 64, torch.float32, "none", None, False),
+]
+
+
+@pytest.mark.parametrize("b,t,hq,hkv,d,dtype,mask,window,seg", FWD_CASES)
+def test_forward_matches_oracle(b, t, hq, hkv, d, dtype, mask, window, seg):
+    q, k, v, _ = _inputs(b, t, hq, hkv, d, dtype)
+    segs = ref.packed_segment_ids(4, b, t, max_docs=5) if seg else None
+    spec, kw = _mask_args(mask, window, segs)
+    scale = d ** -0.5
+    want, want_lse = ref.reference_mha(q, k, v, spec, softmax_scale=scale, return_lse=True)
+    out, lse = ops.flash_fwd(q.cuda(), k.cuda(), v.cuda(), softmax_scale=scale, **kw)
+    _assert_close("out", out, want, dtype)
+    assert ref.max_abs(lse.cpu(), want_lse) < (1e-5 if dtype == torch.float32 else 1e-3) * max(1.0, float(want_lse.abs().max()))
+    if dtype == torch.bfloat16:
+        # The dtype-faithful restatement (reference rounding points) is as close as the float64 one.
+        faithful = ref.reference_mha(q, k, v, spec, softmax_scale=scale, mode="faithful")
+        assert _ok_bf16(out.cpu(), faithful)
+
+
+def test_forward_kv_longer_than_q_and_scale_one():
+    q, k, v, _ = _inputs(1, 128, 2, 1, 128, torch.bfloat16, s=384)
+    want = ref.reference_mha(q * 0.1, k, v, None, softmax_scale=1.0)
+    out, _ = ops.flash_fwd((q * 0.1).cuda(), k.cuda(), v.cuda(), softmax_scale=1.0)
+    _assert_close("out", out, ref.reference_mha((q * 0.1), k, v, None, softmax_scale=1.0), torch.bfloat16)
+    del want
+
+
+BWD_CASES = [
+    (1, 128, 1, 1, 128, "none", None, False),
+    (2, 256, 4, 4, 64, "causal", None, False),
+    (1, 384, 8, 2, 128, "causal", None, False),
+    (2, 512, 4, 1, 128, "causal", None, True),
+    (1, 1024, 4, 2, 128, "sliding", 300, True),
+    (2, 512, 2, 2, 64, "sliding", 127, False),
+]
+
+
+@pytest.mark.parametrize("b,t,hq,hkv,d,mask,window,seg", BWD_CASES)
+def test_backward_matches_oracle(b, t, hq, hkv, d, mask, window, seg):
+    dtype = torch.bfloat16
+    q, k, v, do = _inputs(b, t, hq, hkv, d, dtype)
+    segs = ref.packed_segment_ids(4, b, t, max_docs=5) if seg else None
+    spec, kw = _mask_args(mask, window, segs)
+    scale = d ** -0.5
+    wq, wk, wv = ref.reference_mha_grads(q, k, v, do, spec, softmax_scale=scale)
+    qc, kc, vc, doc = q.cuda(), k.cuda(), v.cuda(), do.cuda()
+    out, lse = ops.flash_fwd(qc, kc, vc, softmax_scale=scale, **kw)
+    dq, dk, dv = ops.flash_bwd(qc, kc, vc, out, lse, doc, softmax_scale=scale, **kw)
+    _assert_close("dq", dq, wq, dtype)
+    _assert_close("dk", dk, wk, dtype)
+    _assert_close("dv", dv, wv, dtype)
+
+
+def test_against_c_brute_force_tiny():
+    """Independent loop-level checker (oracle/brute_force.c) incl. GQA, window and segments."""
+    b, t, hq, hkv, d = 1, 128, 2, 1, 64
+    q, k, v, do = _inputs(b, t, hq, hkv, d, torch.bfloat16)
+    segs = ref.packed_segment_ids(9, b, t, max_docs=3)
+    scale = 0.2
+    bo, bl = brute.attention_fwd(q.float().numpy(), k.float().numpy(), v.float().numpy(), scale=scale,
+                                 mask_kind=brute.MASK_SLIDING, window=40, segment_ids=segs.numpy())
+    bq, bk, bv = brute.attention_bwd(q.float().numpy(), k.float().numpy(), v.float().numpy(), do.float().numpy(),
+                                     scale=scale, mask_kind=brute.MASK_SLIDING, window=40, segment_ids=segs.numpy())
+    kw = dict(softmax_scale=scale, mask_kind=ops.MASK_SLIDING_WINDOW, sliding_window=40, segment_ids=segs.cuda())
+    out, lse = ops.flash_fwd(q.cuda(), k.cuda(), v.cuda(), **kw)
+    dq, dk, dv = ops.flash_bwd(q.cuda(), k.cuda(), v.cuda(), out, lse, do.cuda(), **kw)
+    for name, got, want in (("out", out, bo), ("dq", dq, bq), ("dk", dk, bk), ("dv", dv, bv)):
+        _assert_close(name, got, torch.from_numpy(want), torch.bfloat16)
+    assert np.abs(lse.cpu().numpy() - bl).max() < 1e-3
+
+
+def test_masking_is_exact_poison():
+    """Masked keys must not influence anything: huge garbage planted in K/V rows that every query
+    of another segment (or outside the window) ignores leaves those queries' outputs bit-identical.
+    The garbage is finite on purpose: the reference masks additively (logit + -1e15) and multiplies
+    the resulting exact-zero probability with V, so a NaN in a masked row of a partially visible
+    tile would propagate through 0 * NaN in the reference's kernels and XLA path alike."""
+    poison = 1e30
+    b, t, h, d = 1, 512, 2, 128
+    q, k, v, do = _inputs(b, t, h, h, d, torch.bfloat16)
+    seg = torch.ones((b, t), dtype=torch.int32)
+    seg[:, 200:330] = 2
+    seg[:, 330:] = 3
+    kw = dict(softmax_scale=d ** -0.5, mask_kind=ops.MASK_CAUSAL, segment_ids=seg.cuda())
+    qc, kc, vc, doc = q.cuda(), k.cuda(), v.cuda(), do.cuda()
+    out0, lse0 = ops.flash_fwd(qc, kc, vc, **kw)
+    dq0, dk0, dv0 = ops.flash_bwd(qc, kc, vc, out0, lse0, doc, **kw)
+    kp, vp = kc.clone(), vc.clone()
+    kp[:, 200:330] = poison
+    vp[:, 200:330] = poison
+    out1, lse1 = ops.flash_fwd(qc, kp, vp, **kw)
+    keep = (seg[0] != 2).cuda()
+    assert torch.equal(out0[:, keep], out1[:, keep]) and torch.equal(lse0[:, :, keep], lse1[:, :, keep])
+    assert torch.isfinite(out1[:, keep].float()).all()
+    # Backward: poison the OTHER segments' queries' upstream gradient instead (dO rows of segment 2):
+    # dK/dV of segments 1 and 3 must not change, dQ rows of segments 1 and 3 neither.
+    dop = doc.clone()
+    dop[:, 200:330] = 7.0
+    dq1, dk1, dv1 = ops.flash_bwd(qc, kc, vc, out0, lse0, dop, **kw)
+    assert torch.equal(dq0[:, keep], dq1[:, keep])
+    assert torch.equal(dk0[:, keep], dk1[:, keep]) and torch.equal(dv0[:, keep], dv1[:, keep])
+    # Sliding window: keys further than w to the left are never read by late queries.
+    w = 100
+    kw = dict(softmax_scale=d ** -0.5, mask_kind=ops.MASK_SLIDING_WINDOW, sliding_window=w)
+    out0, _ = ops.flash_fwd(qc, kc, vc, **kw)
+    kp, vp = kc.clone(), vc.clone()
+    kp[:, :128] = poison
+    vp[:, :128] = poison
+    out1, _ = ops.flash_fwd(qc, kp, vp, **kw)
+    assert torch.equal(out0[:, 127 + w + 1:], out1[:, 127 + w + 1:])
+    # Causal: the future never leaks.
+    kw = dict(softmax_scale=d ** -0.5, mask_kind=ops.MASK_CAUSAL)
+    out0, _ = ops.flash_fwd(qc, kc, vc, **kw)
+    kp, vp = kc.clone(), vc.clone()
+    kp[:, 300:] = poison
+    vp[:, 300:] = poison
+    out1, _ = ops.flash_fwd(qc, kp, vp, **kw)
+    assert torch.equal(out0[:, :300], out1[:, :300])
+
+
+def test_closed_forms_and_determinism():
+    b, t, h, d = 1, 256, 2, 128
+    q, k, v, do = _inputs(b, t, h, h, d, torch.bfloat16)
+    qc, kc, vc = q.cuda(), k.cuda(), v.cuda()
+    kw = dict(softmax_scale=d ** -0.5, mask_kind=ops.MASK_CAUSAL)
+    out, lse = ops.flash_fwd(qc, kc, vc, **kw)
+    assert torch.equal(out[:, 0], vc[:, 0])  # causal row 0 == V[0]
+    out_w0, _ = ops.flash_fwd(qc, kc, vc, softmax_scale=1.0, mask_kind=ops.MASK_SLIDING_WINDOW, sliding_window=0)
+    assert torch.equal(out_w0, vc)  # window 0 == self only
+    const = torch.ones_like(vc) * 0.5
+    out_c, _ = ops.flash_fwd(qc, kc, const, **kw)
+    assert torch.equal(out_c, const)  # uniform V
+    # Bitwise run-to-run determinism (no atomics anywhere), forward and backward.
+    out2, lse2 = ops.flash_fwd(qc, kc, vc, **kw)
+    assert torch.equal(out, out2) and torch.equal(lse, lse2)
+    g1 = ops.flash_bwd(qc, kc, vc, out, lse, do.cuda(), **kw)
+    g2 = ops.flash_bwd(qc, kc, vc, out, lse, do.cuda(), **kw)
+    for a, c in zip(g1, g2):
+        assert torch.equal(a, c)
+
+
+def test_strided_inputs():
+    """q/k/v sliced out of one fused [B,T,H+2Hkv,D] projection (non-contiguous heads stride)."""
+    b, t, hq, hkv, d = 1, 256, 4, 2, 128
+    fused = ref.normal_tensor(5, (b, t, hq + 2 * hkv, d), torch.bfloat16).cuda()
+    q, k, v = fused[:, :, :hq], fused[:, :, hq:hq + hkv], fused[:, :, hq + hkv:]
+    kw = dict(softmax_scale=d ** -0.5, mask_kind=ops.MASK_CAUSAL)
+    out, lse = ops.flash_fwd(q, k, v, **kw)
+    out_c, lse_c = ops.flash_fwd(q.contiguous(), k.contiguous(), v.contiguous(), **kw)
+    assert torch.equal(out, out_c) and torch.equal(lse, lse_c)
+    do = torch.randn_like(out)
+    g = ops.flash_bwd(q, k, v, out, lse, do, **kw)
+    gc = ops.flash_bwd(q.contiguous(), k.contiguous(), v.contiguous(), out, lse, do, **kw)
+    for a, c in zip(g, gc):
+        assert torch.equal(a, c)
+
+
+def test_dispatch_and_autograd_end_to_end():
+    b, t, hq, hkv, d = 2, 256, 4, 2, 128
+    q, k, v, do = _inputs(b, t, hq, hkv, d, torch.bfloat16)
+    segs = ref.packed_segment_ids(4, b, t, max_docs=3)
+    pos = dict(target_positions=torch.arange(t)[None], source_positions=torch.arange(t)[None])
+    bias = ab.CompositeAttentionBias([
+        ab.SlidingWindowAttentionBias(ab.sliding_window_causal_mask(64), sliding_window_size=64, **pos),
+        ab.SegmentIdAttentionBias(segs.cuda()),
+    ])
+    qd, kd, vd = (x.cuda().requires_grad_(True) for x in (q, k, v))
+    scale = d ** -0.5
+    impl = flash_attention_implementation("gpu", query=qd, key=kd, value=vd, bias=bias, softmax_scale=scale)
+    assert impl is not None and isinstance(impl.fn, HipFlashAttention)
+    out = impl.fn(dict(query=qd, key=kd, value=vd, bias=bias))
+    # Same loss as the reference's tests: mean of the output (gpu_attention_test.py:59-92).
+    out.float().mean().backward()
+    spec = ref.MaskSpec(sliding_window=64, segment_ids=segs)
+    want = ref.reference_mha(q, k, v, spec, softmax_scale=scale)
+    ones = torch.full_like(want, 1.0 / want.numel())
+    wq, wk, wv = ref.reference_mha_grads(q, k, v, ones, spec, softmax_scale=scale)
+    _assert_close("out", out, want, torch.bfloat16)
+    for name, got, exp in (("dq", qd.grad, wq), ("dk", kd.grad, wk), ("dv", vd.grad, wv)):
+        assert ref.rel_l2(got.cpu(), exp) < 2e-2, name  # gradients of a mean are ~1e-6: relative check
+    # Function-level entry point with a mask fn.
+    o2 = flash_attention(qd, kd, vd, segment_ids=segs.cuda(), softmax_scale=scale,
+                         mask_fn=ab.sliding_window_causal_mask(64))
+    assert torch.equal(o2, out)
+    # A dense bias is not something these kernels do: dispatch must decline, not guess.
+    dense = ab.CompositeAttentionBias([ab.TensorAttentionBias(torch.zeros(1, 1, t, t, device="cuda"))])
+    assert flash_attention_implementation("gpu", query=qd, key=kd, value=vd, bias=dense) is None
+
+
+# ----------------------------------------------------------------------------- BASELINE sizes
+
+
+def _sampled_fwd_bwd_check(B, T, Hq, Hkv, D, mask, window, seg, samples, dq_rows):
+    """Full-size run on the GPU; the oracle checks sampled (batch, kv head) groups on query-row
+    windows (a causal row only needs the keys before it), and size-independent identities check
+    the rest: sum_s dV == sum_t dO and sum_s dK == 0 for every (batch, kv head)."""
+    dev = "cuda"
+    gen = torch.Generator(device=dev).manual_seed(0)
+    mk = lambda h: torch.randn((B, T, h, D), device=dev, generator=gen).to(torch.bfloat16)
+    q, k, v, do = mk(Hq), mk(Hkv), mk(Hkv), mk(Hq)
+    segs = ref.packed_segment_ids(4, B, T) if seg else None
+    spec_kw = dict(causal=mask == "causal", sliding_window=window if mask == "sliding" else None)
+    _, kw = _mask_args(mask, window, segs)
+    scale = D ** -0.5
+    out, lse = ops.flash_fwd(q, k, v, softmax_scale=scale, **kw)
+    dq, dk, dv = ops.flash_bwd(q, k, v, out, lse, do, softmax_scale=scale, **kw)
+    torch.cuda.synchronize()
+    G = Hq // Hkv
+    for (b, hk) in samples:
+        hs = slice(hk * G, (hk + 1) * G)
+        for (r0, r1) in dq_rows:
+            # Query rows [r0, r1) against keys [0, r1): exact for causal / sliding masks.
+            qs, ks, vs = q[b:b + 1, r0:r1, hs].cpu(), k[b:b + 1, :r1, hk:hk + 1].cpu(), v[b:b + 1, :r1, hk:hk + 1].cpu()
+            sub = ref.MaskSpec(**spec_kw, segment_ids=None if segs is None else segs[b:b + 1, :r1],
+                               target_positions=torch.arange(r0, r1)[None], source_positions=torch.arange(r1)[None])
+            if segs is not None:
+                # segment mask of the sub-problem: rows r0..r1 vs keys 0..r1
+                sub.segment_ids = None
+                keep = segs[b:b + 1, r0:r1, None] == segs[b:b + 1, None, :r1]
+                sub.dense_bias = ref.bool_to_bias(keep)[:, None]
+            want = ref.reference_mha(qs, ks, vs, sub, softmax_scale=scale, row_block=128)
+            assert _ok_bf16(out[b:b + 1, r0:r1, hs].cpu(), want), ("out", b, hk, r0)
+            # dq of these rows only depends on these rows.
+            wq, _, _ = ref.reference_mha_grads(qs, ks, vs, do[b:b + 1, r0:r1, hs].cpu(), sub, softmax_scale=scale, row_block=128)
+            assert _ok_bf16(dq[b:b + 1, r0:r1, hs].cpu(), wq), ("dq", b, hk, r0)
+    # Identities over the whole tensors (fp32 sums of bf16 values).
+    dv_sum = dv.float().sum(dim=1)                                   # [B, Hkv, D]
+    do_sum = do.float().sum(dim=1).reshape(B, Hkv, G, D).sum(dim=2)
+    assert ref.rel_l2(dv_sum.cpu(), do_sum.cpu()) < 1e-2
+    dk_sum = dk.float().sum(dim=1)
+    assert float(dk_sum.abs().max()) < 2e-2 * float(dk.float().abs().max()) * (T ** 0.5)
+    return out, dq, dk, dv
+
+
+def test_baseline_c2_full_size():
+    _sampled_fwd_bwd_check(4, 4096, 32, 8, 128, "causal", None, False,
+                           samples=[(0, 0), (3, 7)], dq_rows=[(0, 128), (1920, 2048), (3968, 4096)])
+
+
+def test_baseline_c2_dkdv_sampled():
+    """dK/dV of one (batch, kv head) at the C2 shape against the oracle on that whole group."""
+    B, T, Hq, Hkv, D = 1, 4096, 4, 1, 128
+    q, k, v, do = _inputs(B, T, Hq, Hkv, D, torch.bfloat16)
+    scale = D ** -0.5
+    spec = ref.MaskSpec(causal=True)
+    wq, wk, wv = ref.reference_mha_grads(q, k, v, do, spec, softmax_scale=scale, dtype=torch.float32)
+    kw = dict(softmax_scale=scale, mask_kind=ops.MASK_CAUSAL)
+    out, lse = ops.flash_fwd(q.cuda(), k.cuda(), v.cuda(), **kw)
+    dq, dk, dv = ops.flash_bwd(q.cuda(), k.cuda(), v.cuda(), out, lse, do.cuda(), **kw)
+    for name, got, want in (("dq", dq, wq), ("dk", dk, wk), ("dv", dv, wv)):
+        _assert_close(name, got, want, torch.bfloat16)
+
+
+def test_baseline_c3_full_size():
+    _sampled_fwd_bwd_check(8, 8192, 16, 16, 128, "sliding", 4096, True,
+                           samples=[(0, 0), (5, 11)], dq_rows=[(0, 128), (4096, 4224), (8064, 8192)])
+
+
+def test_baseline_c5_full_size():
+    _sampled_fwd_bwd_check(1, 32768, 64, 8, 128, "causal", None, False,
+                           samples=[(0, 3)], dq_rows=[(0, 128), (16384, 16512), (32640, 32768)])

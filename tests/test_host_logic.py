@@ -1,0 +1,332 @@
+"""CPU-only tests: mask algebra, block maps, kernel-class support gates, dispatch, and that the C-ABI
+library loads and exports every symbol include/axl_attn.h declares.  No kernel is launched here."""
+
+import ctypes
+import json
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from axlearn_amd import _lib
+from axlearn_amd import attention_bias as ab
+from axlearn_amd.flash_attention import common
+from axlearn_amd.flash_attention.hip_attention import (
+    HipFlashAttention,
+    classify_mask_bias,
+    classify_mask_fn,
+    flash_attention,
+)
+from axlearn_amd.flash_attention.hip_decoding import HipDecoding, HipPagedAttention
+from axlearn_amd.flash_attention.utils import (
+    BACKENDS,
+    PAGED_ATTN_BACKENDS,
+    flash_attention_implementation,
+)
+from axlearn_amd.kv_cache import KVCache, PagedKVCache
+from axlearn_amd import ops
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+# ----------------------------------------------------------------------------- mask algebra
+
+
+def test_mask_tables_from_reference_tests(golden_dir):
+    g = json.load(open(os.path.join(golden_dir, "mask_tables.json")))
+    for case in g["sliding_window_5x5"]:
+        fn = ab.sliding_window_causal_mask(case["left_context"])
+        got = fn(torch.arange(5)[:, None], torch.arange(5)[None, :]).int().tolist()
+        assert got == case["expected"]
+    for case in g["sliding_window2_with_time_step_3x5"]:
+        fn = ab.sliding_window_causal_mask(2)
+        got = fn(torch.arange(3)[:, None] + case["time_step"], torch.arange(5)[None, :]).int().tolist()
+        assert got == case["expected"]
+    assert ab.causal_mask(torch.arange(3)[:, None], torch.arange(3)[None, :]).int().tolist() == g["causal_3x3"]
+    seg = g["segment_4x4"]
+    bias = ab.make_segment_mask(target_segments=torch.tensor(seg["target_segments"]),
+                                source_segments=torch.tensor(seg["source_segments"]))
+    assert (bias == 0).int().tolist() == seg["expected"]
+    assert float(bias.min()) == pytest.approx(-1e15)
+    with pytest.raises(ValueError):
+        ab.sliding_window_causal_mask(-1)
+
+
+def test_composite_bias_and_split():
+    t = 6
+    pos = dict(target_positions=torch.arange(t)[None], source_positions=torch.arange(t)[None])
+    seg_ids = torch.tensor([[1, 1, 1, 2, 2, 0]])
+    dense = torch.randn(1, 1, t, t)
+    bias = ab.CompositeAttentionBias(
+        [ab.CausalAttentionBias(**pos), ab.SegmentIdAttentionBias(seg_ids), ab.TensorAttentionBias(dense)]
+    )
+    assert bias.eval_shape() == (1, 1, t, t)
+    mask, seg, rest = ab.split(bias, ab.MaskFnAttentionBias, ab.SegmentIdAttentionBias)
+    assert isinstance(mask, ab.CausalAttentionBias) and isinstance(seg, ab.SegmentIdAttentionBias)
+    assert rest.has_value()
+    total = mask.value() + seg.value() + rest.value()
+    torch.testing.assert_close(total, bias.value())
+    # Doubly masked element carries -2e15: biases are summed, not min-ed.
+    assert float(bias.value()[0, 0, 0, 5]) < -1.5e15
+    # Absent types come back as ZeroAttentionBias.
+    m2, s2, r2 = ab.split(ab.CompositeAttentionBias([ab.TensorAttentionBias(dense)]),
+                          ab.MaskFnAttentionBias, ab.SegmentIdAttentionBias)
+    assert not m2.has_value() and not s2.has_value() and r2.has_value()
+    assert isinstance(m2, ab.ZeroAttentionBias) and m2 == ab.ZeroAttentionBias()
+    assert not ab.CompositeAttentionBias([]).has_value()
+    with pytest.raises(ValueError):
+        ab.CompositeAttentionBias([]).eval_shape()
+
+
+def test_structured_masks_combine():
+    t = 8
+    pos = dict(target_positions=torch.arange(t)[None], source_positions=torch.arange(t)[None])
+    mk = lambda w: ab.SlidingWindowAttentionBias(ab.sliding_window_causal_mask(w), sliding_window_size=w, **pos)
+    bias = ab.CompositeAttentionBias([ab.CausalAttentionBias(**pos), mk(5), mk(3)])
+    mask, rest = ab.split(bias, ab.MaskFnAttentionBias)
+    assert not rest.has_value()
+    assert classify_mask_bias(mask) == (ops.MASK_SLIDING_WINDOW, 3)
+    torch.testing.assert_close(mask.value(), mk(3).value())
+    assert classify_mask_fn(None) == (ops.MASK_NONE, 0)
+    assert classify_mask_fn(ab.causal_mask) == (ops.MASK_CAUSAL, 0)
+    assert classify_mask_fn(ab.sliding_window_causal_mask(7)) == (ops.MASK_SLIDING_WINDOW, 7)
+    assert classify_mask_fn(lambda q, k: q == k) is None
+    # A generic mask fn next to a causal one collapses to an opaque AND.
+    generic = ab.MaskFnAttentionBias(lambda q, k: (q - k) % 2 == 0, **pos)
+    mask, _ = ab.split(ab.CompositeAttentionBias([ab.CausalAttentionBias(**pos), generic]), ab.MaskFnAttentionBias)
+    assert classify_mask_bias(mask) is None
+    want = ab.causal_mask(torch.arange(t)[:, None], torch.arange(t)[None]) & ((torch.arange(t)[:, None] - torch.arange(t)[None]) % 2 == 0)
+    assert torch.equal(mask.bool_value()[0, 0], want)
+
+
+def test_as_attention_bias():
+    assert isinstance(ab.as_attention_bias(None), ab.ZeroAttentionBias)
+    assert isinstance(ab.as_attention_bias(torch.zeros(2, 2)), ab.TensorAttentionBias)
+    with pytest.raises(ValueError):
+        ab.as_attention_bias(torch.zeros(2, 2, dtype=torch.int32))
+    with pytest.raises(ValueError):
+        ab.bool_to_bias(torch.zeros(2, 2))
+
+
+# ----------------------------------------------------------------------------- block maps
+
+
+def test_block_maps(golden_dir):
+    g = json.load(open(os.path.join(golden_dir, "mask_tables.json")))["sliding_window_block_map_invariant"]
+    for w in g["sliding_window_sz"]:
+        for t in g["seq_len"]:
+            for blk in g["block_size"]:
+                kw = dict(q_seq_len=t, kv_seq_len=t, block_q=blk, block_k=blk)
+                a = common.build_mask(ab.sliding_window_causal_mask(w), **kw)
+                b = common.build_sliding_window_mask(**kw, sliding_window_size=w)
+                assert (a == b).all(), (w, t, blk)
+    # Brute force "tile keeps any element", unequal blocks.
+    fn = ab.sliding_window_causal_mask(37)
+    t, bq, bk = 256, 32, 64
+    got = common.build_mask(fn, q_seq_len=t, kv_seq_len=t, block_q=bq, block_k=bk)
+    full = fn(torch.arange(t)[:, None], torch.arange(t)[None, :]).numpy()
+    want = full.reshape(t // bq, bq, t // bk, bk).any(axis=(1, 3))
+    assert (got == want).all()
+    assert (common.build_sliding_window_mask(q_seq_len=t, kv_seq_len=t, block_q=bq, block_k=bk, sliding_window_size=37) == want).all()
+    info = common.query_iterator_indices(want)
+    for i in range(want.shape[0]):
+        n = info.kv_block_offset_size[i]
+        assert list(info.kv_block_offset[i, :n]) == list(np.nonzero(want[i])[0])
+    off, size = common.key_value_iterator_indices(want)
+    for j in range(want.shape[1]):
+        assert list(off[j, : size[j]]) == list(np.nonzero(want[:, j])[0])
+
+
+def test_kernel_tile_ranges_match_block_map():
+    """The closed-form key range the forward kernel iterates (128-row query block, 64-key tiles)
+    covers exactly the live tiles of the reference's block map."""
+    t, window = 1024, 300
+    live = common.build_mask(ab.sliding_window_causal_mask(window), q_seq_len=t, kv_seq_len=t, block_q=128, block_k=64)
+    for qb in range(t // 128):
+        k_end = min(t, qb * 128 + 128)
+        k_begin = max(0, qb * 128 - window)
+        rng = set(range(k_begin // 64, (k_end + 63) // 64))
+        assert rng == set(np.nonzero(live[qb])[0])
+
+
+# ----------------------------------------------------------------------------- support gates
+
+
+def _batch(t=128, s=128, hq=4, hkv=2, d=128, dtype=torch.bfloat16, bias=None, b=2):
+    pos = dict(target_positions=torch.arange(t)[None], source_positions=torch.arange(s)[None])
+    return dict(
+        query=torch.zeros(b, t, hq, d, dtype=dtype), key=torch.zeros(b, s, hkv, d, dtype=dtype),
+        value=torch.zeros(b, s, hkv, d, dtype=dtype),
+        bias=bias if bias is not None else ab.CompositeAttentionBias([ab.CausalAttentionBias(**pos)]),
+    )
+
+
+def test_is_supported_raises_on_illogical_shapes():
+    fa = HipFlashAttention.default_config().instantiate()
+    bad = _batch()
+    bad["key"] = torch.zeros(3, 128, 2, 128, dtype=torch.bfloat16)
+    bad["value"] = bad["key"]
+    with pytest.raises(ValueError, match="batch size"):
+        fa.is_supported(bad, kv_cache_type=None)
+    bad = _batch(hq=5, hkv=2)
+    with pytest.raises(ValueError, match="divisible"):
+        fa.is_supported(bad, kv_cache_type=None)
+    bad = _batch()
+    bad["value"] = torch.zeros(2, 64, 2, 128, dtype=torch.bfloat16)
+    with pytest.raises(ValueError):
+        fa.is_supported(bad, kv_cache_type=None)
+    bad = _batch()
+    del bad["bias"]
+    with pytest.raises(ValueError):
+        fa.is_supported(bad, kv_cache_type=None)
+    dec = HipDecoding.default_config().set(dropout_rate=0.1).instantiate()
+    with pytest.raises(ValueError, match="Dropout"):
+        dec.is_supported(_batch(t=1), kv_cache_type=KVCache)
+
+
+def test_is_supported_returns_false_when_merely_unsupported(caplog):
+    fa = HipFlashAttention.default_config().instantiate()
+    assert not fa.is_supported(_batch(t=100, s=100), kv_cache_type=None)  # not a multiple of 128
+    assert not fa.is_supported(_batch(d=72), kv_cache_type=None)
+    assert not fa.is_supported(_batch(dtype=torch.float16), kv_cache_type=None)
+    assert not fa.is_supported(_batch(), kv_cache_type=KVCache)
+    dense = ab.CompositeAttentionBias([ab.TensorAttentionBias(torch.zeros(1, 1, 128, 128))])
+    assert not fa.is_supported(_batch(bias=dense), kv_cache_type=None)
+    sink = _batch()
+    sink["logit_sink"] = torch.zeros(4)
+    assert not fa.is_supported(sink, kv_cache_type=None)
+    assert not HipFlashAttention.default_config().set(dropout_rate=0.1).instantiate().is_supported(_batch(), None)
+    # Everything fine except the tensors live on the CPU.
+    assert not fa.is_supported(_batch(), kv_cache_type=None)
+    assert fa.name() == "HipFlashAttention"
+    assert fa.get_backend_overrides("x", 3) == 3
+    dec = HipDecoding.default_config().instantiate()
+    assert not dec.is_supported(_batch(t=2), kv_cache_type=KVCache)
+    assert not dec.is_supported(_batch(t=1), kv_cache_type=None)
+    paged = HipPagedAttention.default_config().instantiate()
+    pb = _batch(t=1)
+    with pytest.raises(ValueError):
+        paged.is_supported(pb, kv_cache_type=PagedKVCache)  # no page_tables
+    pb["page_tables"] = torch.zeros(2, 4, dtype=torch.int32)
+    assert not paged.is_supported(pb, kv_cache_type=KVCache)
+
+
+def test_dispatch_tables_and_fallback():
+    assert BACKENDS["gpu"] == [HipDecoding, HipFlashAttention]
+    assert PAGED_ATTN_BACKENDS["gpu"] == [HipPagedAttention]
+    b = _batch()
+    # CPU tensors / unknown backends: no kernel matches -> None (caller falls back to plain attention).
+    assert flash_attention_implementation("gpu", query=b["query"], key=b["key"], value=b["value"], bias=b["bias"]) is None
+    assert flash_attention_implementation("cpu", query=b["query"], key=b["key"], value=b["value"], bias=b["bias"]) is None
+    assert flash_attention_implementation("tpu", query=b["query"], key=b["key"], value=b["value"], bias=b["bias"], dropout_rate=None) is None
+
+
+def test_entry_point_rejects_what_kernels_cannot_do():
+    q = torch.zeros(1, 128, 1, 128, dtype=torch.bfloat16)
+    with pytest.raises(NotImplementedError):
+        flash_attention(q, q, q, bias=torch.zeros(1, 1, 128, 128))
+    with pytest.raises(NotImplementedError):
+        flash_attention(q, q, q, dropout_rate=0.5)
+    with pytest.raises(NotImplementedError):
+        flash_attention(q, q, q, mask_fn=lambda a, b: a == b)
+    with pytest.raises(NotImplementedError):
+        flash_attention(q, q, q, interpret=True)
+    with pytest.raises(_lib.AxlError):
+        flash_attention(q, q, q)  # CPU tensors: there is no CPU path
+
+
+def test_config_protocol():
+    cfg = HipFlashAttention.default_config().set(softmax_scale=0.5, gpu_block_size=64)
+    inst = cfg.instantiate()
+    assert inst.cfg.softmax_scale == 0.5 and inst.cfg.gpu_block_size == 64
+    with pytest.raises(AttributeError):
+        cfg.set(no_such_field=1)
+    assert HipPagedAttention.default_config().sparse_ratio == 0.8
+
+
+# ----------------------------------------------------------------------------- C ABI (no launches)
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "axl_attn.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(axl_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    declared = _declared_functions()
+    assert set(declared) == set(_lib.EXPORTED_SYMBOLS)
+    lib = _lib.load()
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert lib.axl_abi_version() == 1
+    assert lib.axl_last_error() is not None
+
+
+def test_struct_layouts_match_header():
+    """Field order of the ctypes mirrors equals the order in the header."""
+    text = open(os.path.join(ROOT, "include", "axl_attn.h")).read()
+    for cls in (_lib.AxlFlashFwdParams, _lib.AxlFlashBwdParams, _lib.AxlPagedDecodeParams, _lib.AxlDecodeParams):
+        body = re.search(r"typedef struct %s \{(.*?)\} %s;" % (cls.__name__, cls.__name__), text, flags=re.S).group(1)
+        body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+        names = []
+        for decl in body.split(";"):
+            decl = decl.strip()
+            if not decl:
+                continue
+            for part in decl.split(","):
+                names.append(re.findall(r"[A-Za-z_][A-Za-z_0-9]*", part)[-1])
+        assert names == [f[0] for f in cls._fields_], cls.__name__
+
+
+def test_abi_validation_without_gpu():
+    """Argument checks run before any launch, so they are testable on a machine without a GPU."""
+    lib = _lib.load()
+    assert lib.axl_flash_fwd(None, None) == _lib.AXL_ERR_INVALID_ARGUMENT
+    s = _lib.AxlStrides(1 << 20, 1024, 128)
+    p = _lib.AxlFlashFwdParams(q=256, k=256, v=256, out=256, lse=None, segment_ids=None, q_strides=s, k_strides=s,
+                               v_strides=s, out_strides=s, batch=1, q_len=128, kv_len=128, num_q_heads=3,
+                               num_kv_heads=2, head_dim=128, dtype=0, mask_kind=1, sliding_window=0,
+                               q_pos_offset=0, softmax_scale=1.0)
+    assert lib.axl_flash_fwd(ctypes.byref(p), None) == _lib.AXL_ERR_INVALID_ARGUMENT
+    assert b"divisible" in lib.axl_last_error()
+    p.num_q_heads = 4
+    p.head_dim = 72
+    assert lib.axl_flash_fwd(ctypes.byref(p), None) == _lib.AXL_ERR_UNSUPPORTED
+    p.head_dim = 128
+    p.q_len = 100
+    assert lib.axl_flash_fwd(ctypes.byref(p), None) == _lib.AXL_ERR_UNSUPPORTED
+    p.q_len = 128
+    p.softmax_scale = 0.0
+    assert lib.axl_flash_fwd(ctypes.byref(p), None) == _lib.AXL_ERR_INVALID_ARGUMENT
+    p.softmax_scale = 1.0
+    p.q = None
+    assert lib.axl_flash_fwd(ctypes.byref(p), None) == _lib.AXL_ERR_INVALID_ARGUMENT
+    p.q = 257
+    assert lib.axl_flash_fwd(ctypes.byref(p), None) == _lib.AXL_ERR_UNSUPPORTED  # misaligned
+    p.q = 256
+    p.segment_ids = 256
+    p.kv_len = 256
+    assert lib.axl_flash_fwd(ctypes.byref(p), None) == _lib.AXL_ERR_INVALID_ARGUMENT  # seg needs T == S
+    # Backward: workspace too small.
+    bp = _lib.AxlFlashBwdParams(q=256, k=256, v=256, out=256, d_out=256, lse=256, dq=256, dk=256, dv=256,
+                                segment_ids=None, q_strides=s, k_strides=s, v_strides=s, out_strides=s,
+                                d_out_strides=s, dq_strides=s, dk_strides=s, dv_strides=s, batch=2, q_len=256,
+                                kv_len=256, num_q_heads=4, num_kv_heads=2, head_dim=128, dtype=0, mask_kind=1,
+                                sliding_window=0, q_pos_offset=0, softmax_scale=1.0, workspace=256, workspace_bytes=16)
+    assert lib.axl_flash_bwd_workspace_bytes(ctypes.byref(bp)) == 2 * 4 * 256 * 4
+    assert lib.axl_flash_bwd(ctypes.byref(bp), None) == _lib.AXL_ERR_WORKSPACE
+    assert lib.axl_flash_bwd_phases(ctypes.byref(bp), 0, None) == _lib.AXL_ERR_INVALID_ARGUMENT
+    # Paged decode geometry.
+    dp = _lib.AxlPagedDecodeParams(q=256, k_pages=256, v_pages=256, page_tables=256, lengths=256, out=256, batch=2,
+                                   num_q_heads=8, num_kv_heads=2, head_dim=128, num_pages=64, page_size=32,
+                                   pages_per_seq=32, dtype=0, sliding_window=-1, softmax_scale=1.0, workspace=None,
+                                   workspace_bytes=0)
+    assert lib.axl_paged_decode(ctypes.byref(dp), None) == _lib.AXL_ERR_UNSUPPORTED  # page size 32
+    dp.page_size = 16
+    assert lib.axl_paged_decode(ctypes.byref(dp), None) == _lib.AXL_ERR_WORKSPACE
+    assert lib.axl_paged_decode_workspace_bytes(ctypes.byref(dp)) > 0
+    dp.num_q_heads = 64
+    assert lib.axl_paged_decode(ctypes.byref(dp), None) == _lib.AXL_ERR_UNSUPPORTED  # 32 heads per kv head
