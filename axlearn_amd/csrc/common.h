@@ -18,6 +18,7 @@ typedef __attribute__((__vector_size__(2 * sizeof(float)))) float floatx2;
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short shortx4;
 typedef __attribute__((__vector_size__(8 * sizeof(short)))) short shortx8;
 typedef __attribute__((__vector_size__(4 * sizeof(int)))) int intx4;
+typedef __attribute__((__vector_size__(4 * sizeof(unsigned)))) unsigned u32x4;
 
 #define AXL_LDS(T, p) ((__attribute__((address_space(3))) T*)(p))
 

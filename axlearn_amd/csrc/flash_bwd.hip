@@ -142,36 +142,33 @@ __global__ __launch_bounds__(256) void flash_bwd_dkdv_bf16_kernel(const BwdArgs 
     for (int r = 0; r < 16; r++) dk_acc[i][r] = dv_acc[i][r] = 0.f;
   const float c = a.scale * kLog2e;
 
-  uint4 qreg[Tile::CHUNKS], dreg[Tile::CHUNKS];
-  auto load_tile = [&](int it) {
-    const int hq = hk * G + it / nt;
-    const int q0 = (t_begin + it % nt) * Tile::BQ;
-    const __bf16* qg = (const __bf16*)a.q + b * a.qs.b + hq * a.qs.h;
-    const __bf16* dg = (const __bf16*)a.dout + b * a.dos.b + hq * a.dos.h;
-#pragma unroll
-    for (int i = 0; i < Tile::CHUNKS; i++) {
-      const int cidx = tid + 256 * i;
-      const int row = cidx / (D / 8), cc = cidx % (D / 8);
-      if (row < Tile::BQ) {
-        qreg[i] = *(const uint4*)(qg + (int64_t)(q0 + row) * a.qs.s + cc * 8);
-        dreg[i] = *(const uint4*)(dg + (int64_t)(q0 + row) * a.dos.s + cc * 8);
-      }
-    }
-  };
-  auto store_tile = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < Tile::CHUNKS; i++) {
-      const int cidx = tid + 256 * i;
-      const int row = cidx / (D / 8), cc = cidx % (D / 8);
-      if (row < Tile::BQ) {
-        *(uint4*)(q_lds + buf * Tile::TILE_BYTES + row * Tile::STRIDE + cc * 16) = qreg[i];
-        *(uint4*)(do_lds + buf * Tile::TILE_BYTES + row * Tile::STRIDE + cc * 16) = dreg[i];
-      }
-    }
-  };
+  // Global -> LDS staging through registers: thread handles 16-byte chunks tid + 256*i of a tile
+  // (plain unrolled code, no lambdas: the staging arrays must stay in registers).
+  static_assert(Tile::BQ * (D / 8) % 256 == 0, "tile must be a whole number of 256-thread passes");
+  u32x4 qreg[Tile::CHUNKS], dreg[Tile::CHUNKS];
+  const int st_row = tid / (D / 8), st_cc = tid % (D / 8);
+  constexpr int ROWS_PER_PASS = 256 / (D / 8);
+  const __bf16* const q_base = (const __bf16*)a.q + b * a.qs.b + (int64_t)st_row * a.qs.s + st_cc * 8;
+  const __bf16* const d_base = (const __bf16*)a.dout + b * a.dos.b + (int64_t)st_row * a.dos.s + st_cc * 8;
+  char* const q_st = q_lds + st_row * Tile::STRIDE + st_cc * 16;
+  char* const d_st = do_lds + st_row * Tile::STRIDE + st_cc * 16;
+#define AXL_LOAD_TILE(IT_)                                                                        \
+  {                                                                                               \
+    const int hq_ = hk * G + (IT_) / nt;                                                          \
+    const int64_t q0_ = (int64_t)(t_begin + (IT_) % nt) * Tile::BQ;                               \
+    _Pragma("unroll") for (int i = 0; i < Tile::CHUNKS; i++) {                                    \
+      qreg[i] = *(const u32x4*)(q_base + hq_ * a.qs.h + (q0_ + i * ROWS_PER_PASS) * a.qs.s);      \
+      dreg[i] = *(const u32x4*)(d_base + hq_ * a.dos.h + (q0_ + i * ROWS_PER_PASS) * a.dos.s);    \
+    }                                                                                             \
+  }
+#define AXL_STORE_TILE(BUF_)                                                                      \
+  _Pragma("unroll") for (int i = 0; i < Tile::CHUNKS; i++) {                                      \
+    *(u32x4*)(q_st + (BUF_) * Tile::TILE_BYTES + i * ROWS_PER_PASS * Tile::STRIDE) = qreg[i];     \
+    *(u32x4*)(d_st + (BUF_) * Tile::TILE_BYTES + i * ROWS_PER_PASS * Tile::STRIDE) = dreg[i];     \
+  }
   if (total > 0) {
-    load_tile(0);
-    store_tile(0);
+    AXL_LOAD_TILE(0)
+    AXL_STORE_TILE(0)
   }
   __syncthreads();
 
@@ -182,7 +179,7 @@ __global__ __launch_bounds__(256) void flash_bwd_dkdv_bf16_kernel(const BwdArgs 
   for (int it = 0; it < total; it++) {
     const int buf = it & 1;
     const bool has_next = it + 1 < total;
-    if (has_next) load_tile(it + 1);
+    if (has_next) AXL_LOAD_TILE(it + 1)
     const int hq = hk * G + it / nt;
     const int q0 = (t_begin + it % nt) * Tile::BQ;
     const int qpos_min = q0 + a.q_off, qpos_max = q0 + Tile::BQ - 1 + a.q_off;
@@ -269,11 +266,15 @@ __global__ __launch_bounds__(256) void flash_bwd_dkdv_bf16_kernel(const BwdArgs 
         }
       }
     }
-    if (has_next) store_tile(buf ^ 1);
+    if (has_next) {
+      AXL_STORE_TILE(buf ^ 1)
+    }
     __syncthreads();
   }
+#undef AXL_LOAD_TILE
+#undef AXL_STORE_TILE
 
-  __bf16* dkp = (__bf16*)a.dk + b * a.dks.b + (int64_t)(k0 + l32) * a.dks.s + hk * a.dks.h;
+  __bf16* dkp =(__bf16*)a.dk + b * a.dks.b + (int64_t)(k0 + l32) * a.dks.s + hk * a.dks.h;
   __bf16* dvp = (__bf16*)a.dv + b * a.dvs.b + (int64_t)(k0 + l32) * a.dvs.s + hk * a.dvs.h;
 #pragma unroll
   for (int dt = 0; dt < DT; dt++)
@@ -354,29 +355,28 @@ __global__ __launch_bounds__(256) void flash_bwd_dq_bf16_kernel(const BwdArgs a)
     for (int r = 0; r < 16; r++) dq_acc[i][r] = 0.f;
   const float c = a.scale * kLog2e;
 
-  uint4 kreg[Tile::CHUNKS], vreg[Tile::CHUNKS];
-  auto load_tile = [&](int t) {
-    const int k0 = t * Tile::BK;
-#pragma unroll
-    for (int i = 0; i < Tile::CHUNKS; i++) {
-      const int cidx = tid + 256 * i;
-      const int row = cidx / (D / 8), cc = cidx % (D / 8);
-      kreg[i] = *(const uint4*)(kp + (int64_t)(k0 + row) * a.ks.s + cc * 8);
-      vreg[i] = *(const uint4*)(vp + (int64_t)(k0 + row) * a.vs.s + cc * 8);
-    }
-  };
-  auto store_tile = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < Tile::CHUNKS; i++) {
-      const int cidx = tid + 256 * i;
-      const int row = cidx / (D / 8), cc = cidx % (D / 8);
-      *(uint4*)(k_lds + buf * Tile::TILE_BYTES + row * Tile::STRIDE + cc * 16) = kreg[i];
-      *(uint4*)(v_lds + buf * Tile::TILE_BYTES + row * Tile::STRIDE + cc * 16) = vreg[i];
-    }
-  };
+  // Global -> LDS staging through registers (plain unrolled code so the arrays stay in registers).
+  u32x4 kreg[Tile::CHUNKS], vreg[Tile::CHUNKS];
+  const int st_row = tid / (D / 8), st_cc = tid % (D / 8);
+  constexpr int ROWS_PER_PASS = 256 / (D / 8);
+  const __bf16* const kg = kp + (int64_t)st_row * a.ks.s + st_cc * 8;
+  const __bf16* const vg = vp + (int64_t)st_row * a.vs.s + st_cc * 8;
+  char* const k_st = k_lds + st_row * Tile::STRIDE + st_cc * 16;
+  char* const v_st = v_lds + st_row * Tile::STRIDE + st_cc * 16;
+#define AXL_LOAD_TILE(T_)                                                                       \
+  _Pragma("unroll") for (int i = 0; i < Tile::CHUNKS; i++) {                                    \
+    const int64_t row_ = (int64_t)(T_) * Tile::BK + i * ROWS_PER_PASS;                          \
+    kreg[i] = *(const u32x4*)(kg + row_ * a.ks.s);                                              \
+    vreg[i] = *(const u32x4*)(vg + row_ * a.vs.s);                                              \
+  }
+#define AXL_STORE_TILE(BUF_)                                                                    \
+  _Pragma("unroll") for (int i = 0; i < Tile::CHUNKS; i++) {                                    \
+    *(u32x4*)(k_st + (BUF_) * Tile::TILE_BYTES + i * ROWS_PER_PASS * Tile::STRIDE) = kreg[i];   \
+    *(u32x4*)(v_st + (BUF_) * Tile::TILE_BYTES + i * ROWS_PER_PASS * Tile::STRIDE) = vreg[i];   \
+  }
   if (t_begin < t_end) {
-    load_tile(t_begin);
-    store_tile(0);
+    AXL_LOAD_TILE(t_begin)
+    AXL_STORE_TILE(0)
   }
   __syncthreads();
 
@@ -387,7 +387,9 @@ __global__ __launch_bounds__(256) void flash_bwd_dq_bf16_kernel(const BwdArgs a)
   for (int t = t_begin; t < t_end; t++) {
     const int buf = (t - t_begin) & 1;
     const bool has_next = t + 1 < t_end;
-    if (has_next) load_tile(t + 1);
+    if (has_next) {
+      AXL_LOAD_TILE(t + 1)
+    }
     const int k0 = t * Tile::BK;
     bool skip = false, need_mask = false;
     if (a.mask_kind != AXL_MASK_NONE) {
@@ -459,11 +461,15 @@ __global__ __launch_bounds__(256) void flash_bwd_dq_bf16_kernel(const BwdArgs a)
         }
       }
     }
-    if (has_next) store_tile(buf ^ 1);
+    if (has_next) {
+      AXL_STORE_TILE(buf ^ 1)
+    }
     __syncthreads();
   }
+#undef AXL_LOAD_TILE
+#undef AXL_STORE_TILE
 
-  __bf16* dqp = (__bf16*)a.dq + b * a.dqs.b + (int64_t)(q0 + l32) * a.dqs.s + h * a.dqs.h;
+  __bf16* dqp =(__bf16*)a.dq + b * a.dqs.b + (int64_t)(q0 + l32) * a.dqs.s + h * a.dqs.h;
 #pragma unroll
   for (int dt = 0; dt < DT; dt++)
 #pragma unroll

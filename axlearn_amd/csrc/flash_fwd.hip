@@ -118,31 +118,29 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
   float l_run = 0.f;      // this lane's share of the running row sum (lanes l and l^32 split it)
   const float c = a.scale * kLog2e;
 
-  // Global -> LDS staging: thread handles chunks tid + 256*i.
-  uint4 kreg[Tile::CHUNKS], vreg[Tile::CHUNKS];
-  auto load_tile = [&](int t) {
-    const int k0 = t * Tile::BK;
-#pragma unroll
-    for (int i = 0; i < Tile::CHUNKS; i++) {
-      const int cidx = tid + 256 * i;
-      const int row = cidx / (D / 8), cc = cidx % (D / 8);
-      kreg[i] = *(const uint4*)(kp + (int64_t)(k0 + row) * a.ks.s + cc * 8);
-      vreg[i] = *(const uint4*)(vp + (int64_t)(k0 + row) * a.vs.s + cc * 8);
-    }
-  };
-  auto store_tile = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < Tile::CHUNKS; i++) {
-      const int cidx = tid + 256 * i;
-      const int row = cidx / (D / 8), cc = cidx % (D / 8);
-      *(uint4*)(k_lds + buf * Tile::KBYTES + row * Tile::KSTRIDE + cc * 16) = kreg[i];
-      *(uint4*)(v_lds + buf * Tile::VBYTES + row * Tile::VSTRIDE + cc * 16) = vreg[i];
-    }
-  };
+  // Global -> LDS staging through registers: thread handles 16-byte chunks tid + 256*i of a tile.
+  u32x4 kreg[Tile::CHUNKS], vreg[Tile::CHUNKS];
+  const int st_row = tid / (D / 8), st_cc = tid % (D / 8);   // chunk 0 of this thread
+  constexpr int ROWS_PER_PASS = 256 / (D / 8);               // rows covered by 256 threads
+  const __bf16* kg = kp + (int64_t)st_row * a.ks.s + st_cc * 8;
+  const __bf16* vg = vp + (int64_t)st_row * a.vs.s + st_cc * 8;
+  char* const k_st = k_lds + st_row * Tile::KSTRIDE + st_cc * 16;
+  char* const v_st = v_lds + st_row * Tile::VSTRIDE + st_cc * 16;
+#define AXL_LOAD_TILE(T_)                                                                     \
+  _Pragma("unroll") for (int i = 0; i < Tile::CHUNKS; i++) {                                  \
+    const int64_t row_ = (int64_t)(T_) * Tile::BK + i * ROWS_PER_PASS;                        \
+    kreg[i] = *(const u32x4*)(kg + row_ * a.ks.s);                                            \
+    vreg[i] = *(const u32x4*)(vg + row_ * a.vs.s);                                            \
+  }
+#define AXL_STORE_TILE(BUF_)                                                                  \
+  _Pragma("unroll") for (int i = 0; i < Tile::CHUNKS; i++) {                                  \
+    *(u32x4*)(k_st + (BUF_) * Tile::KBYTES + i * ROWS_PER_PASS * Tile::KSTRIDE) = kreg[i];    \
+    *(u32x4*)(v_st + (BUF_) * Tile::VBYTES + i * ROWS_PER_PASS * Tile::VSTRIDE) = vreg[i];    \
+  }
 
   if (t_begin < t_end) {
-    load_tile(t_begin);
-    store_tile(0);
+    AXL_LOAD_TILE(t_begin)
+    AXL_STORE_TILE(0)
   }
   __syncthreads();
 
@@ -154,7 +152,9 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
   for (int t = t_begin; t < t_end; t++) {
     const int buf = (t - t_begin) & 1;
     const bool has_next = t + 1 < t_end;
-    if (has_next) load_tile(t + 1);
+    if (has_next) {
+      AXL_LOAD_TILE(t + 1)
+    }
 
     const int k0 = t * Tile::BK;
     bool skip = false;
@@ -257,9 +257,13 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
         }
       }
     }
-    if (has_next) store_tile(buf ^ 1);
+    if (has_next) {
+      AXL_STORE_TILE(buf ^ 1)
+    }
     __syncthreads();
   }
+#undef AXL_LOAD_TILE
+#undef AXL_STORE_TILE
 
   // Epilogue: out = acc / l ; lse = m*scale + ln(l).
   const float l_tot = xor32_sum(l_run);
