@@ -73,6 +73,11 @@ __device__ __forceinline__ int swap_bits_2_3(int m) {
   return (m & ~12) | ((m & 4) << 1) | ((m & 8) >> 1);
 }
 
+// s_waitcnt vmcnt(0) only (expcnt and lgkmcnt fields left at "no wait").  Placed before a main loop
+// it retires the loads of loop-invariant fragments, so the compiler's wait-count bookkeeping does
+// not make every iteration wait on the loads it has just issued for the NEXT tile.
+__device__ __forceinline__ void wait_all_vmem() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
 struct Strides3 {
   int64_t b, s, h;
 };

@@ -87,11 +87,13 @@ struct DkvTile {
   static constexpr int STRIDE = D * 2 + 16;    // bytes per Q / dO row in LDS
   static constexpr int TILE_BYTES = BQ * STRIDE;
   static constexpr int CHUNKS = (BQ * D * 2 / 16 + 255) / 256;  // 16-byte chunks per thread per tensor
-  static constexpr int LDS_BYTES = 4 * TILE_BYTES;              // {Q, dO} x double buffer
+  static constexpr int STAT_BYTES = 3 * BQ * 4;                 // lse, delta, segment id per query row
+  static constexpr int LDS_BYTES = 4 * TILE_BYTES + 2 * STAT_BYTES;  // {Q, dO} x 2 buffers + row stats x 2
 };
 
 template <int D>
-__global__ __launch_bounds__(256) void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
   using Tile = DkvTile<D>;
   constexpr int KK = D / 16, DT = D / 32;
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -152,6 +154,13 @@ __global__ __launch_bounds__(256) void flash_bwd_dkdv_bf16_kernel(const BwdArgs 
   const __bf16* const d_base = (const __bf16*)a.dout + b * a.dos.b + (int64_t)st_row * a.dos.s + st_cc * 8;
   char* const q_st = q_lds + st_row * Tile::STRIDE + st_cc * 16;
   char* const d_st = do_lds + st_row * Tile::STRIDE + st_cc * 16;
+  // Row statistics of the tile travel with it: threads 0..7 fetch lse, 8..15 delta, 16..23 the
+  // segment ids (16 bytes each); stat_lds holds [lse | delta | seg] x BQ per buffer.
+  char* const stat_lds = smem + 4 * Tile::TILE_BYTES;
+  u32x4 sreg = {0, 0, 0, 0};
+  const int st_kind = tid >> 3, st_part = tid & 7;  // kind 0: lse, 1: delta, 2: segment ids
+  const bool st_active = st_kind < 2 || (st_kind == 2 && a.seg != nullptr);
+  static_assert(Tile::BQ == 32, "row-stat staging assumes 8 x 16 bytes per kind");
 #define AXL_LOAD_TILE(IT_)                                                                        \
   {                                                                                               \
     const int hq_ = hk * G + (IT_) / nt;                                                          \
@@ -160,16 +169,28 @@ __global__ __launch_bounds__(256) void flash_bwd_dkdv_bf16_kernel(const BwdArgs 
       qreg[i] = *(const u32x4*)(q_base + hq_ * a.qs.h + (q0_ + i * ROWS_PER_PASS) * a.qs.s);      \
       dreg[i] = *(const u32x4*)(d_base + hq_ * a.dos.h + (q0_ + i * ROWS_PER_PASS) * a.dos.s);    \
     }                                                                                             \
+    if (st_active) {                                                                              \
+      const int64_t row_ = ((int64_t)b * a.Hq + hq_) * a.T + q0_ + 4 * st_part;                   \
+      const void* src_ = st_kind == 0 ? (const void*)(a.lse + row_)                               \
+                       : st_kind == 1 ? (const void*)(a.delta + row_)                             \
+                                      : (const void*)(a.seg + (int64_t)b * a.T + q0_ + 4 * st_part); \
+      sreg = *(const u32x4*)src_;                                                                 \
+    }                                                                                             \
   }
 #define AXL_STORE_TILE(BUF_)                                                                      \
-  _Pragma("unroll") for (int i = 0; i < Tile::CHUNKS; i++) {                                      \
-    *(u32x4*)(q_st + (BUF_) * Tile::TILE_BYTES + i * ROWS_PER_PASS * Tile::STRIDE) = qreg[i];     \
-    *(u32x4*)(d_st + (BUF_) * Tile::TILE_BYTES + i * ROWS_PER_PASS * Tile::STRIDE) = dreg[i];     \
+  {                                                                                               \
+    _Pragma("unroll") for (int i = 0; i < Tile::CHUNKS; i++) {                                    \
+      *(u32x4*)(q_st + (BUF_) * Tile::TILE_BYTES + i * ROWS_PER_PASS * Tile::STRIDE) = qreg[i];   \
+      *(u32x4*)(d_st + (BUF_) * Tile::TILE_BYTES + i * ROWS_PER_PASS * Tile::STRIDE) = dreg[i];   \
+    }                                                                                             \
+    if (tid < 24)                                                                                 \
+      *(u32x4*)(stat_lds + (BUF_) * Tile::STAT_BYTES + st_kind * (Tile::BQ * 4) + st_part * 16) = sreg; \
   }
   if (total > 0) {
     AXL_LOAD_TILE(0)
     AXL_STORE_TILE(0)
   }
+  wait_all_vmem();  // stationary fragments have landed: nothing issued before the loop is pending
   __syncthreads();
 
   const int a_row_off = swap_bits_2_3(l32) * Tile::STRIDE + g * 16;  // normal (row = query) reads
@@ -198,52 +219,73 @@ __global__ __launch_bounds__(256) void flash_bwd_dkdv_bf16_kernel(const BwdArgs 
       floatx16 s, dp;
 #pragma unroll
       for (int r = 0; r < 16; r++) s[r] = dp[r] = 0.f;
+      // All A fragments of both chains are requested from LDS before the first MFMA so that the
+      // matrix pipe never waits on an LDS round trip between two MFMAs (one wavefront per SIMD:
+      // there is nobody else to cover that latency).
+      bf16x8 qfr[KK], dfr[KK];
 #pragma unroll
-      for (int kk = 0; kk < KK; kk++) {
-        const bf16x8 qa = *(const bf16x8*)(qt + a_row_off + kk * 32);
-        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa, kf[kk], s, 0, 0, 0);
-      }
+      for (int kk = 0; kk < KK; kk++) qfr[kk] = *(const bf16x8*)(qt + a_row_off + kk * 32);
 #pragma unroll
-      for (int kk = 0; kk < KK; kk++) {
-        const bf16x8 da = *(const bf16x8*)(dt_ + a_row_off + kk * 32);
-        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da, vf[kk], dp, 0, 0, 0);
-      }
+      for (int kk = 0; kk < KK; kk++) dfr[kk] = *(const bf16x8*)(dt_ + a_row_off + kk * 32);
+      __builtin_amdgcn_sched_barrier(0);  // keep the reads ahead of the MFMAs
+#pragma unroll
+      for (int kk = 0; kk < KK; kk++)
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qfr[kk], kf[kk], s, 0, 0, 0);
+#pragma unroll
+      for (int kk = 0; kk < KK; kk++)
+        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dfr[kk], vf[kk], dp, 0, 0, 0);
+      // Transposed fragments for the second pair of GEMMs do not depend on P: request them now, so
+      // they arrive while the softmax arithmetic runs.
+      union TrFrag { bf16x8 v; shortx4 hlf[2]; };
+      TrFrag dtr[2][DT], qtr[2][DT];
+#pragma unroll
+      for (int t8 = 0; t8 < 2; t8++)
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++) {
+          const char* da = dt_ + 16 * t8 * Tile::STRIDE + tr_off + dt * 64;
+          const char* qa = qt + 16 * t8 * Tile::STRIDE + tr_off + dt * 64;
+          dtr[t8][dt].hlf[0] = lds_read_tr16(da);
+          dtr[t8][dt].hlf[1] = lds_read_tr16(da + 4 * Tile::STRIDE);
+          qtr[t8][dt].hlf[0] = lds_read_tr16(qa);
+          qtr[t8][dt].hlf[1] = lds_read_tr16(qa + 4 * Tile::STRIDE);
+        }
+      __builtin_amdgcn_sched_barrier(0);
       // Register r of lane group g is query q0 + 16(r/8) + 8g + (r%8); the lane is key kpos.
-      const float* lse_p = a.lse + ((int64_t)b * a.Hq + hq) * a.T + q0 + 8 * g;
-      const float* del_p = a.delta + ((int64_t)b * a.Hq + hq) * a.T + q0 + 8 * g;
-      float lse_r[16], del_r[16];
+      const char* st = stat_lds + buf * Tile::STAT_BYTES + 8 * g * 4;  // rows 8g.. of [lse|delta|seg]
+      floatx4 lse_v[4], del_v[4];
 #pragma unroll
       for (int t8 = 0; t8 < 2; t8++) {
-        const float4 l0 = *(const float4*)(lse_p + 16 * t8), l1 = *(const float4*)(lse_p + 16 * t8 + 4);
-        const float4 d0 = *(const float4*)(del_p + 16 * t8), d1 = *(const float4*)(del_p + 16 * t8 + 4);
-        lse_r[8 * t8 + 0] = l0.x; lse_r[8 * t8 + 1] = l0.y; lse_r[8 * t8 + 2] = l0.z; lse_r[8 * t8 + 3] = l0.w;
-        lse_r[8 * t8 + 4] = l1.x; lse_r[8 * t8 + 5] = l1.y; lse_r[8 * t8 + 6] = l1.z; lse_r[8 * t8 + 7] = l1.w;
-        del_r[8 * t8 + 0] = d0.x; del_r[8 * t8 + 1] = d0.y; del_r[8 * t8 + 2] = d0.z; del_r[8 * t8 + 3] = d0.w;
-        del_r[8 * t8 + 4] = d1.x; del_r[8 * t8 + 5] = d1.y; del_r[8 * t8 + 6] = d1.z; del_r[8 * t8 + 7] = d1.w;
+        lse_v[2 * t8] = *(const floatx4*)(st + 64 * t8);
+        lse_v[2 * t8 + 1] = *(const floatx4*)(st + 64 * t8 + 16);
+        del_v[2 * t8] = *(const floatx4*)(st + Tile::BQ * 4 + 64 * t8);
+        del_v[2 * t8 + 1] = *(const floatx4*)(st + Tile::BQ * 4 + 64 * t8 + 16);
       }
-      int seg_r[16];
+      // Masks are applied in (at most) two wave-uniform blocks so the common unmasked tile runs
+      // straight-line code.
+      if (need_mask) {
+        const int diff0 = (q0 + a.q_off + 8 * g) - kpos;  // query of r == 0 minus this lane's key
+        const unsigned limit = a.mask_kind == AXL_MASK_SLIDING_WINDOW ? (unsigned)a.window : 0x7fffffffu;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const unsigned diff = (unsigned)(diff0 + 16 * (r / 8) + (r % 8));
+          s[r] = diff <= limit ? s[r] : kMasked;  // 0 <= q - k <= limit
+        }
+      }
       if (a.seg) {
-        const int32_t* sp = a.seg + (int64_t)b * a.T + q0 + 8 * g;
+        intx4 seg_v[4];
 #pragma unroll
         for (int t8 = 0; t8 < 2; t8++) {
-          const int4 s0 = *(const int4*)(sp + 16 * t8), s1 = *(const int4*)(sp + 16 * t8 + 4);
-          seg_r[8 * t8 + 0] = s0.x; seg_r[8 * t8 + 1] = s0.y; seg_r[8 * t8 + 2] = s0.z; seg_r[8 * t8 + 3] = s0.w;
-          seg_r[8 * t8 + 4] = s1.x; seg_r[8 * t8 + 5] = s1.y; seg_r[8 * t8 + 6] = s1.z; seg_r[8 * t8 + 7] = s1.w;
+          seg_v[2 * t8] = *(const intx4*)(st + 2 * Tile::BQ * 4 + 64 * t8);
+          seg_v[2 * t8 + 1] = *(const intx4*)(st + 2 * Tile::BQ * 4 + 64 * t8 + 16);
         }
+#pragma unroll
+        for (int r = 0; r < 16; r++) s[r] = seg_v[r / 4][r % 4] == seg_k ? s[r] : kMasked;
       }
 #pragma unroll
       for (int r = 0; r < 16; r++) {
-        bool keep = true;
-        if (need_mask) {
-          const int diff = (q0 + a.q_off + 16 * (r / 8) + 8 * g + (r % 8)) - kpos;
-          keep = diff >= 0;
-          if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) keep = keep && diff <= a.window;
-        }
-        if (a.seg) keep = keep && (seg_r[r] == seg_k);
-        const float sv = keep ? s[r] : kMasked;
-        const float p = fast_exp2(__builtin_fmaf(sv, c, -lse_r[r] * kLog2e));
+        const float p = fast_exp2(__builtin_fmaf(s[r], c, -lse_v[r / 4][r % 4] * kLog2e));
         s[r] = p;
-        dp[r] = p * (dp[r] - del_r[r]);
+        dp[r] = p * (dp[r] - del_v[r / 4][r % 4]);
       }
       // dV^T += dO^T P ; dK^T += Q^T dS  (scale applied once at the end).
 #pragma unroll
@@ -252,17 +294,10 @@ __global__ __launch_bounds__(256) void flash_bwd_dkdv_bf16_kernel(const BwdArgs 
                                       s[8 * t8 + 4], s[8 * t8 + 5], s[8 * t8 + 6], s[8 * t8 + 7]);
         const bf16x8 dsb = pack_bf16x8(dp[8 * t8 + 0], dp[8 * t8 + 1], dp[8 * t8 + 2], dp[8 * t8 + 3],
                                        dp[8 * t8 + 4], dp[8 * t8 + 5], dp[8 * t8 + 6], dp[8 * t8 + 7]);
-        const char* da = dt_ + 16 * t8 * Tile::STRIDE + tr_off;
-        const char* qa = qt + 16 * t8 * Tile::STRIDE + tr_off;
 #pragma unroll
         for (int dt = 0; dt < DT; dt++) {
-          union { bf16x8 v; shortx4 hlf[2]; } fa, fb;
-          fa.hlf[0] = lds_read_tr16(da + dt * 64);
-          fa.hlf[1] = lds_read_tr16(da + dt * 64 + 4 * Tile::STRIDE);
-          dv_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa.v, pb, dv_acc[dt], 0, 0, 0);
-          fb.hlf[0] = lds_read_tr16(qa + dt * 64);
-          fb.hlf[1] = lds_read_tr16(qa + dt * 64 + 4 * Tile::STRIDE);
-          dk_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb.v, dsb, dk_acc[dt], 0, 0, 0);
+          dv_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dtr[t8][dt].v, pb, dv_acc[dt], 0, 0, 0);
+          dk_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qtr[t8][dt].v, dsb, dk_acc[dt], 0, 0, 0);
         }
       }
     }
@@ -378,6 +413,7 @@ __global__ __launch_bounds__(256) void flash_bwd_dq_bf16_kernel(const BwdArgs a)
     AXL_LOAD_TILE(t_begin)
     AXL_STORE_TILE(0)
   }
+  wait_all_vmem();  // stationary fragments have landed: nothing issued before the loop is pending
   __syncthreads();
 
   const int a_row_off = swap_bits_2_3(l32) * Tile::STRIDE + g * 16;
@@ -421,28 +457,30 @@ __global__ __launch_bounds__(256) void flash_bwd_dq_bf16_kernel(const BwdArgs a)
           dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr, dof[kk], dp, 0, 0, 0);
         }
         // Register r of lane group g is key k0 + 32ks + 16(r/8) + 8g + (r%8); the lane is a query.
-        int seg_r[16];
-        if (seg_k) {
+        // Masks in (at most) two wave-uniform blocks; unmasked tiles run straight-line code.
+        if (need_mask) {
+          const int diff0 = qpos - (k0 + 32 * ks + 8 * g);
+          const unsigned limit = a.mask_kind == AXL_MASK_SLIDING_WINDOW ? (unsigned)a.window : 0x7fffffffu;
 #pragma unroll
-          for (int t8 = 0; t8 < 2; t8++) {
-            const int4* sp = (const int4*)(seg_k + k0 + 32 * ks + 16 * t8 + 8 * g);
-            const int4 s0 = sp[0], s1 = sp[1];
-            seg_r[8 * t8 + 0] = s0.x; seg_r[8 * t8 + 1] = s0.y; seg_r[8 * t8 + 2] = s0.z; seg_r[8 * t8 + 3] = s0.w;
-            seg_r[8 * t8 + 4] = s1.x; seg_r[8 * t8 + 5] = s1.y; seg_r[8 * t8 + 6] = s1.z; seg_r[8 * t8 + 7] = s1.w;
+          for (int r = 0; r < 16; r++) {
+            const unsigned diff = (unsigned)(diff0 - (16 * (r / 8) + (r % 8)));
+            s[r] = diff <= limit ? s[r] : kMasked;  // 0 <= q - k <= limit
           }
         }
-        const int diff0 = qpos - (k0 + 32 * ks + 8 * g);
+        if (seg_k) {
+          intx4 seg_v[4];
+#pragma unroll
+          for (int t8 = 0; t8 < 2; t8++) {
+            const intx4* sp = (const intx4*)(seg_k + k0 + 32 * ks + 16 * t8 + 8 * g);
+            seg_v[2 * t8] = sp[0];
+            seg_v[2 * t8 + 1] = sp[1];
+          }
+#pragma unroll
+          for (int r = 0; r < 16; r++) s[r] = seg_v[r / 4][r % 4] == seg_q ? s[r] : kMasked;
+        }
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-          bool keep = true;
-          if (need_mask) {
-            const int diff = diff0 - (16 * (r / 8) + (r % 8));
-            keep = diff >= 0;
-            if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) keep = keep && diff <= a.window;
-          }
-          if (seg_k) keep = keep && (seg_r[r] == seg_q);
-          const float sv = keep ? s[r] : kMasked;
-          const float p = fast_exp2(__builtin_fmaf(sv, c, -lse2));
+          const float p = fast_exp2(__builtin_fmaf(s[r], c, -lse2));
           dp[r] = p * (dp[r] - delta);
         }
         // dQ^T[d][q] += K^T[d][key] dS^T[key][q].

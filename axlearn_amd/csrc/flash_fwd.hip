@@ -142,6 +142,7 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
     AXL_LOAD_TILE(t_begin)
     AXL_STORE_TILE(0)
   }
+  wait_all_vmem();  // Q fragments have landed: no load issued before the loop is pending inside it
   __syncthreads();
 
   // Per-lane LDS read offsets.
