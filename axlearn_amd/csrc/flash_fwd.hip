@@ -173,15 +173,32 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
       const char* vt = v_lds + buf * Tile::VBYTES;
       floatx16 s[2];
 #pragma unroll
-      for (int ks = 0; ks < 2; ks++) {
+      for (int ks = 0; ks < 2; ks++)
 #pragma unroll
         for (int r = 0; r < 16; r++) s[ks][r] = 0.f;
-        const char* ka = kt + ks * 32 * Tile::KSTRIDE + k_row_off;
+      // 2*KK independent-by-pairs MFMAs (the two sub-tile chains alternate) fed by 2*KK LDS reads.
+      // The schedule below keeps kAhead reads in flight ahead of the MFMA that consumes them, so
+      // the matrix pipe does not sit out an LDS round trip between two MFMAs.
+      {
+        bf16x8 kfr[KK][2];
 #pragma unroll
-        for (int kk = 0; kk < KK; kk++) {
-          const bf16x8 kf = *(const bf16x8*)(ka + kk * 32);
-          s[ks] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[kk], s[ks], 0, 0, 0);
+        for (int kk = 0; kk < KK; kk++)
+#pragma unroll
+          for (int ks = 0; ks < 2; ks++)
+            kfr[kk][ks] = *(const bf16x8*)(kt + ks * 32 * Tile::KSTRIDE + k_row_off + kk * 32);
+#pragma unroll
+        for (int kk = 0; kk < KK; kk++)
+#pragma unroll
+          for (int ks = 0; ks < 2; ks++)
+            s[ks] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr[kk][ks], qf[kk], s[ks], 0, 0, 0);
+        constexpr int kAhead = 6;
+        __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
+#pragma unroll
+        for (int i = 0; i < 2 * KK - kAhead; i++) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
+        __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
       }
       // Register r of sub-tile ks in lane group g is key k0 + 32ks + 16(r/8) + 8g + (r%8).
       if (need_mask) {
@@ -211,17 +228,49 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
           }
         }
       }
+      // V^T fragments do not depend on the softmax: the first kPvAhead of the 4*DT PV steps have
+      // their transposing reads issued now, so they land while the arithmetic below runs.
+      // PV step n = (ks*2 + t8)*DT + dt multiplies V^T[32dt.., keys 32ks+16t8..] with P^T.
+      constexpr int kPvSteps = 4 * DT, kPvAhead = 4;
+      union VFrag {
+        bf16x8 v;
+        shortx4 hlf[2];
+      };
+      VFrag vfr[kPvSteps];
+      const char* const vbase = vt + v_lane_off;
+#define AXL_PV_READ(N_)                                                                        \
+  {                                                                                            \
+    const char* va_ = vbase + (16 * ((N_) / DT)) * Tile::VSTRIDE + ((N_) % DT) * 64;           \
+    vfr[N_].hlf[0] = lds_read_tr16(va_);                                                       \
+    vfr[N_].hlf[1] = lds_read_tr16(va_ + 4 * Tile::VSTRIDE);                                   \
+  }
+#pragma unroll
+      for (int n = 0; n < kPvAhead; n++) AXL_PV_READ(n)
+      __builtin_amdgcn_sched_barrier(0);
+
       float mx = m_run;
 #pragma unroll
       for (int ks = 0; ks < 2; ks++)
 #pragma unroll
         for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[ks][r]);
       mx = xor32_max(mx);
-      const float mc = mx * c;
-      // Subtract first: (m_run * c - mc) would be contracted into an fma whose result, when the
-      // max did not move, is the rounding error of the product instead of an exact 0.
-      const float corr = fast_exp2((m_run - mx) * c);
-      m_run = mx;
+      // Lazy rescaling: the running max (and with it the accumulators) only moves when the new max
+      // exceeds it by more than 2^kLazyLog2 in the exponent; until then exp2 is taken against the
+      // stale max, which scales numerator and denominator alike (values stay below 2^kLazyLog2).
+      constexpr float kLazyLog2 = 8.0f;
+      const bool move = (mx - m_run) * c > kLazyLog2;
+      if (__builtin_amdgcn_ballot_w64(move) != 0) {
+        // Subtract first: (m_run * c - mx * c) would be contracted into an fma whose result, for
+        // equal maxima, is the rounding error of the product instead of an exact 0.
+        const float corr = move ? fast_exp2((m_run - mx) * c) : 1.0f;
+        m_run = move ? mx : m_run;
+        l_run *= corr;
+#pragma unroll
+        for (int i = 0; i < DT; i++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) o[i][r] *= corr;
+      }
+      const float mc = m_run * c;
       float lsum = 0.f;
 #pragma unroll
       for (int ks = 0; ks < 2; ks++)
@@ -231,32 +280,25 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
           s[ks][r] = p;
           lsum += p;
         }
-      l_run = l_run * corr + lsum;
+      l_run += lsum;
+      bf16x8 pb[4];
 #pragma unroll
-      for (int i = 0; i < DT; i++)
+      for (int ks = 0; ks < 2; ks++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) o[i][r] *= corr;
-      // O^T += V^T P^T.
-#pragma unroll
-      for (int ks = 0; ks < 2; ks++) {
-#pragma unroll
-        for (int t8 = 0; t8 < 2; t8++) {
-          const bf16x8 pb = pack_bf16x8(s[ks][8 * t8 + 0], s[ks][8 * t8 + 1], s[ks][8 * t8 + 2],
+        for (int t8 = 0; t8 < 2; t8++)
+          pb[2 * ks + t8] = pack_bf16x8(s[ks][8 * t8 + 0], s[ks][8 * t8 + 1], s[ks][8 * t8 + 2],
                                         s[ks][8 * t8 + 3], s[ks][8 * t8 + 4], s[ks][8 * t8 + 5],
                                         s[ks][8 * t8 + 6], s[ks][8 * t8 + 7]);
-          const char* va = vt + (32 * ks + 16 * t8) * Tile::VSTRIDE + v_lane_off;
+      __builtin_amdgcn_sched_barrier(0);
+      // O^T += V^T P^T, software pipelined: each MFMA issues together with the reads of the step
+      // kPvAhead ahead of it.
 #pragma unroll
-          for (int dt = 0; dt < DT; dt++) {
-            union {
-              bf16x8 v;
-              shortx4 hlf[2];
-            } vf;
-            vf.hlf[0] = lds_read_tr16(va + dt * 64);
-            vf.hlf[1] = lds_read_tr16(va + dt * 64 + 4 * Tile::VSTRIDE);
-            o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pb, o[dt], 0, 0, 0);
-          }
-        }
+      for (int n = 0; n < kPvSteps; n++) {
+        if (n + kPvAhead < kPvSteps) AXL_PV_READ(n + kPvAhead)
+        o[n % DT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr[n].v, pb[n / DT], o[n % DT], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
       }
+#undef AXL_PV_READ
     }
     if (has_next) {
       AXL_STORE_TILE(buf ^ 1)
