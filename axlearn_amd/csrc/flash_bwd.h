@@ -1,0 +1,29 @@
+// Argument block shared by the backward kernels (delta pre-pass, dK/dV, dQ).
+#pragma once
+
+#include "common.h"
+
+namespace axl {
+
+struct BwdArgs {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* out;
+  const void* dout;
+  const float* lse;
+  float* delta;  // workspace [B, Hq, T]
+  void* dq;
+  void* dk;
+  void* dv;
+  const int32_t* seg;
+  Strides3 qs, ks, vs, os, dos, dqs, dks, dvs;
+  int B, T, S, Hq, Hkv;
+  int mask_kind, window, q_off;
+  float scale;
+};
+
+// Enqueues the dK/dV kernel (bf16) for head_dim 64 or 128.
+hipError_t launch_bwd_dkdv_bf16(const BwdArgs& a, int head_dim, hipStream_t stream);
+
+}  // namespace axl

@@ -18,27 +18,9 @@
 //   dQ: a workgroup owns 128 queries (32 per wavefront, Q and dO fragments in registers) and
 //     streams 64-key K/V tiles through LDS exactly like the forward; S^T = K Q^T, dP^T = V dO^T,
 //     dQ^T += K^T dS^T with K^T from transposing LDS reads.
-#include "common.h"
+#include "flash_bwd.h"
 
 namespace axl {
-
-struct BwdArgs {
-  const void* q;
-  const void* k;
-  const void* v;
-  const void* out;
-  const void* dout;
-  const float* lse;
-  float* delta;  // workspace [B, Hq, T]
-  void* dq;
-  void* dk;
-  void* dv;
-  const int32_t* seg;
-  Strides3 qs, ks, vs, os, dos, dqs, dks, dvs;
-  int B, T, S, Hq, Hkv;
-  int mask_kind, window, q_off;
-  float scale;
-};
 
 // ---------------------------------------------------------------------------------------------
 // delta[b,h,t] = sum_d out[b,t,h,d] * dO[b,t,h,d]; 16 lanes per row, 16 bytes per lane per step.
@@ -75,254 +57,6 @@ __global__ __launch_bounds__(256) void bwd_delta_kernel(const BwdArgs a) {
   acc += __shfl_xor(acc, 4, 64);
   acc += __shfl_xor(acc, 8, 64);
   if (row < rows && sub == 0) a.delta[((int64_t)b * a.Hq + h) * a.T + t] = acc;
-}
-
-// ---------------------------------------------------------------------------------------------
-// dK / dV.
-// ---------------------------------------------------------------------------------------------
-template <int D>
-struct DkvTile {
-  static constexpr int BKV = 128;              // keys per workgroup (32 per wavefront)
-  static constexpr int BQ = 32;                // query rows per LDS tile
-  static constexpr int STRIDE = D * 2 + 16;    // bytes per Q / dO row in LDS
-  static constexpr int TILE_BYTES = BQ * STRIDE;
-  static constexpr int CHUNKS = (BQ * D * 2 / 16 + 255) / 256;  // 16-byte chunks per thread per tensor
-  static constexpr int STAT_BYTES = 3 * BQ * 4;                 // lse, delta, segment id per query row
-  static constexpr int LDS_BYTES = 4 * TILE_BYTES + 2 * STAT_BYTES;  // {Q, dO} x 2 buffers + row stats x 2
-};
-
-template <int D>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
-void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
-  using Tile = DkvTile<D>;
-  constexpr int KK = D / 16, DT = D / 32;
-  extern __shared__ __attribute__((aligned(16))) char smem[];
-  char* const q_lds = smem;                          // 2 buffers
-  char* const do_lds = smem + 2 * Tile::TILE_BYTES;  // 2 buffers
-
-  const int tid = threadIdx.x;
-  const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
-  const int G = a.Hq / a.Hkv;
-  const int nkb = a.S / Tile::BKV;
-  // blockIdx -> (key block, batch, kv head); earliest key blocks (most queries under a causal
-  // mask) first.
-  const int kb = blockIdx.x / (a.B * a.Hkv);
-  const int rem = blockIdx.x % (a.B * a.Hkv);
-  const int b = rem / a.Hkv, hk = rem % a.Hkv;
-  (void)nkb;
-  const int k0_wg = kb * Tile::BKV;
-  const int k0 = k0_wg + wave * 32;  // this wavefront's keys
-
-  // K and V fragments (B operands): lane (key l32, k-group g) holds d = 16kk + 8g .. +7.
-  const __bf16* kp = (const __bf16*)a.k + b * a.ks.b + (int64_t)(k0 + l32) * a.ks.s + hk * a.ks.h;
-  const __bf16* vp = (const __bf16*)a.v + b * a.vs.b + (int64_t)(k0 + l32) * a.vs.s + hk * a.vs.h;
-  bf16x8 kf[KK], vf[KK];
-#pragma unroll
-  for (int kk = 0; kk < KK; kk++) {
-    kf[kk] = *(const bf16x8*)(kp + 16 * kk + 8 * g);
-    vf[kk] = *(const bf16x8*)(vp + 16 * kk + 8 * g);
-  }
-  const int kpos = k0 + l32;
-  const int seg_k = a.seg ? a.seg[(int64_t)b * a.T + k0 + l32] : 0;
-
-  // Query rows that can see any key of this workgroup.
-  int q_begin = 0, q_end = a.T;
-  if (a.mask_kind != AXL_MASK_NONE) {
-    q_begin = max(0, k0_wg - a.q_off);
-    if (a.mask_kind == AXL_MASK_SLIDING_WINDOW)
-      q_end = min(a.T, k0_wg + Tile::BKV - 1 + a.window - a.q_off + 1);
-  }
-  const int t_begin = q_begin / Tile::BQ;
-  const int t_end = max(t_begin, (q_end + Tile::BQ - 1) / Tile::BQ);
-  const int nt = t_end - t_begin;
-  const int total = nt * G;  // iterations: query head (outer) x query tile (inner)
-
-  floatx16 dk_acc[DT], dv_acc[DT];
-#pragma unroll
-  for (int i = 0; i < DT; i++)
-#pragma unroll
-    for (int r = 0; r < 16; r++) dk_acc[i][r] = dv_acc[i][r] = 0.f;
-  const float c = a.scale * kLog2e;
-
-  // Global -> LDS staging through registers: thread handles 16-byte chunks tid + 256*i of a tile
-  // (plain unrolled code, no lambdas: the staging arrays must stay in registers).
-  static_assert(Tile::BQ * (D / 8) % 256 == 0, "tile must be a whole number of 256-thread passes");
-  u32x4 qreg[Tile::CHUNKS], dreg[Tile::CHUNKS];
-  const int st_row = tid / (D / 8), st_cc = tid % (D / 8);
-  constexpr int ROWS_PER_PASS = 256 / (D / 8);
-  const __bf16* const q_base = (const __bf16*)a.q + b * a.qs.b + (int64_t)st_row * a.qs.s + st_cc * 8;
-  const __bf16* const d_base = (const __bf16*)a.dout + b * a.dos.b + (int64_t)st_row * a.dos.s + st_cc * 8;
-  char* const q_st = q_lds + st_row * Tile::STRIDE + st_cc * 16;
-  char* const d_st = do_lds + st_row * Tile::STRIDE + st_cc * 16;
-  // Row statistics of the tile travel with it: threads 0..7 fetch lse, 8..15 delta, 16..23 the
-  // segment ids (16 bytes each); stat_lds holds [lse | delta | seg] x BQ per buffer.
-  char* const stat_lds = smem + 4 * Tile::TILE_BYTES;
-  u32x4 sreg = {0, 0, 0, 0};
-  const int st_kind = tid >> 3, st_part = tid & 7;  // kind 0: lse, 1: delta, 2: segment ids
-  const bool st_active = st_kind < 2 || (st_kind == 2 && a.seg != nullptr);
-  static_assert(Tile::BQ == 32, "row-stat staging assumes 8 x 16 bytes per kind");
-#define AXL_LOAD_TILE(IT_)                                                                        \
-  {                                                                                               \
-    const int hq_ = hk * G + (IT_) / nt;                                                          \
-    const int64_t q0_ = (int64_t)(t_begin + (IT_) % nt) * Tile::BQ;                               \
-    _Pragma("unroll") for (int i = 0; i < Tile::CHUNKS; i++) {                                    \
-      qreg[i] = *(const u32x4*)(q_base + hq_ * a.qs.h + (q0_ + i * ROWS_PER_PASS) * a.qs.s);      \
-      dreg[i] = *(const u32x4*)(d_base + hq_ * a.dos.h + (q0_ + i * ROWS_PER_PASS) * a.dos.s);    \
-    }                                                                                             \
-    if (st_active) {                                                                              \
-      const int64_t row_ = ((int64_t)b * a.Hq + hq_) * a.T + q0_ + 4 * st_part;                   \
-      const void* src_ = st_kind == 0 ? (const void*)(a.lse + row_)                               \
-                       : st_kind == 1 ? (const void*)(a.delta + row_)                             \
-                                      : (const void*)(a.seg + (int64_t)b * a.T + q0_ + 4 * st_part); \
-      sreg = *(const u32x4*)src_;                                                                 \
-    }                                                                                             \
-  }
-#define AXL_STORE_TILE(BUF_)                                                                      \
-  {                                                                                               \
-    _Pragma("unroll") for (int i = 0; i < Tile::CHUNKS; i++) {                                    \
-      *(u32x4*)(q_st + (BUF_) * Tile::TILE_BYTES + i * ROWS_PER_PASS * Tile::STRIDE) = qreg[i];   \
-      *(u32x4*)(d_st + (BUF_) * Tile::TILE_BYTES + i * ROWS_PER_PASS * Tile::STRIDE) = dreg[i];   \
-    }                                                                                             \
-    if (tid < 24)                                                                                 \
-      *(u32x4*)(stat_lds + (BUF_) * Tile::STAT_BYTES + st_kind * (Tile::BQ * 4) + st_part * 16) = sreg; \
-  }
-  if (total > 0) {
-    AXL_LOAD_TILE(0)
-    AXL_STORE_TILE(0)
-  }
-  wait_all_vmem();  // stationary fragments have landed: nothing issued before the loop is pending
-  __syncthreads();
-
-  const int a_row_off = swap_bits_2_3(l32) * Tile::STRIDE + g * 16;  // normal (row = query) reads
-  const int j16 = lane & 15, half = (lane >> 4) & 1;
-  const int tr_off = (8 * g + (j16 >> 2)) * Tile::STRIDE + (16 * half + 4 * (j16 & 3)) * 2;
-
-  for (int it = 0; it < total; it++) {
-    const int buf = it & 1;
-    const bool has_next = it + 1 < total;
-    if (has_next) AXL_LOAD_TILE(it + 1)
-    const int hq = hk * G + it / nt;
-    const int q0 = (t_begin + it % nt) * Tile::BQ;
-    const int qpos_min = q0 + a.q_off, qpos_max = q0 + Tile::BQ - 1 + a.q_off;
-    bool skip = false, need_mask = false;
-    if (a.mask_kind != AXL_MASK_NONE) {
-      skip = k0 > qpos_max;
-      need_mask = k0 + 31 > qpos_min;
-      if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) {
-        skip = skip || (qpos_min - (k0 + 31) > a.window);
-        need_mask = need_mask || (qpos_max - k0 > a.window);
-      }
-    }
-    if (!skip) {
-      const char* qt = q_lds + buf * Tile::TILE_BYTES;
-      const char* dt_ = do_lds + buf * Tile::TILE_BYTES;
-      floatx16 s, dp;
-#pragma unroll
-      for (int r = 0; r < 16; r++) s[r] = dp[r] = 0.f;
-      // All A fragments of both chains are requested from LDS before the first MFMA so that the
-      // matrix pipe never waits on an LDS round trip between two MFMAs (one wavefront per SIMD:
-      // there is nobody else to cover that latency).
-      bf16x8 qfr[KK], dfr[KK];
-#pragma unroll
-      for (int kk = 0; kk < KK; kk++) qfr[kk] = *(const bf16x8*)(qt + a_row_off + kk * 32);
-#pragma unroll
-      for (int kk = 0; kk < KK; kk++) dfr[kk] = *(const bf16x8*)(dt_ + a_row_off + kk * 32);
-      __builtin_amdgcn_sched_barrier(0);  // keep the reads ahead of the MFMAs
-#pragma unroll
-      for (int kk = 0; kk < KK; kk++)
-        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qfr[kk], kf[kk], s, 0, 0, 0);
-#pragma unroll
-      for (int kk = 0; kk < KK; kk++)
-        dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dfr[kk], vf[kk], dp, 0, 0, 0);
-      // Transposed fragments for the second pair of GEMMs do not depend on P: request them now, so
-      // they arrive while the softmax arithmetic runs.
-      union TrFrag { bf16x8 v; shortx4 hlf[2]; };
-      TrFrag dtr[2][DT], qtr[2][DT];
-#pragma unroll
-      for (int t8 = 0; t8 < 2; t8++)
-#pragma unroll
-        for (int dt = 0; dt < DT; dt++) {
-          const char* da = dt_ + 16 * t8 * Tile::STRIDE + tr_off + dt * 64;
-          const char* qa = qt + 16 * t8 * Tile::STRIDE + tr_off + dt * 64;
-          dtr[t8][dt].hlf[0] = lds_read_tr16(da);
-          dtr[t8][dt].hlf[1] = lds_read_tr16(da + 4 * Tile::STRIDE);
-          qtr[t8][dt].hlf[0] = lds_read_tr16(qa);
-          qtr[t8][dt].hlf[1] = lds_read_tr16(qa + 4 * Tile::STRIDE);
-        }
-      __builtin_amdgcn_sched_barrier(0);
-      // Register r of lane group g is query q0 + 16(r/8) + 8g + (r%8); the lane is key kpos.
-      const char* st = stat_lds + buf * Tile::STAT_BYTES + 8 * g * 4;  // rows 8g.. of [lse|delta|seg]
-      floatx4 lse_v[4], del_v[4];
-#pragma unroll
-      for (int t8 = 0; t8 < 2; t8++) {
-        lse_v[2 * t8] = *(const floatx4*)(st + 64 * t8);
-        lse_v[2 * t8 + 1] = *(const floatx4*)(st + 64 * t8 + 16);
-        del_v[2 * t8] = *(const floatx4*)(st + Tile::BQ * 4 + 64 * t8);
-        del_v[2 * t8 + 1] = *(const floatx4*)(st + Tile::BQ * 4 + 64 * t8 + 16);
-      }
-      // Masks are applied in (at most) two wave-uniform blocks so the common unmasked tile runs
-      // straight-line code.
-      if (need_mask) {
-        const int diff0 = (q0 + a.q_off + 8 * g) - kpos;  // query of r == 0 minus this lane's key
-        const unsigned limit = a.mask_kind == AXL_MASK_SLIDING_WINDOW ? (unsigned)a.window : 0x7fffffffu;
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-          const unsigned diff = (unsigned)(diff0 + 16 * (r / 8) + (r % 8));
-          s[r] = diff <= limit ? s[r] : kMasked;  // 0 <= q - k <= limit
-        }
-      }
-      if (a.seg) {
-        intx4 seg_v[4];
-#pragma unroll
-        for (int t8 = 0; t8 < 2; t8++) {
-          seg_v[2 * t8] = *(const intx4*)(st + 2 * Tile::BQ * 4 + 64 * t8);
-          seg_v[2 * t8 + 1] = *(const intx4*)(st + 2 * Tile::BQ * 4 + 64 * t8 + 16);
-        }
-#pragma unroll
-        for (int r = 0; r < 16; r++) s[r] = seg_v[r / 4][r % 4] == seg_k ? s[r] : kMasked;
-      }
-#pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const float p = fast_exp2(__builtin_fmaf(s[r], c, -lse_v[r / 4][r % 4] * kLog2e));
-        s[r] = p;
-        dp[r] = p * (dp[r] - del_v[r / 4][r % 4]);
-      }
-      // dV^T += dO^T P ; dK^T += Q^T dS  (scale applied once at the end).
-#pragma unroll
-      for (int t8 = 0; t8 < 2; t8++) {
-        const bf16x8 pb = pack_bf16x8(s[8 * t8 + 0], s[8 * t8 + 1], s[8 * t8 + 2], s[8 * t8 + 3],
-                                      s[8 * t8 + 4], s[8 * t8 + 5], s[8 * t8 + 6], s[8 * t8 + 7]);
-        const bf16x8 dsb = pack_bf16x8(dp[8 * t8 + 0], dp[8 * t8 + 1], dp[8 * t8 + 2], dp[8 * t8 + 3],
-                                       dp[8 * t8 + 4], dp[8 * t8 + 5], dp[8 * t8 + 6], dp[8 * t8 + 7]);
-#pragma unroll
-        for (int dt = 0; dt < DT; dt++) {
-          dv_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(dtr[t8][dt].v, pb, dv_acc[dt], 0, 0, 0);
-          dk_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qtr[t8][dt].v, dsb, dk_acc[dt], 0, 0, 0);
-        }
-      }
-    }
-    if (has_next) {
-      AXL_STORE_TILE(buf ^ 1)
-    }
-    __syncthreads();
-  }
-#undef AXL_LOAD_TILE
-#undef AXL_STORE_TILE
-
-  __bf16* dkp =(__bf16*)a.dk + b * a.dks.b + (int64_t)(k0 + l32) * a.dks.s + hk * a.dks.h;
-  __bf16* dvp = (__bf16*)a.dv + b * a.dvs.b + (int64_t)(k0 + l32) * a.dvs.s + hk * a.dvs.h;
-#pragma unroll
-  for (int dt = 0; dt < DT; dt++)
-#pragma unroll
-    for (int rq = 0; rq < 4; rq++) {
-      union { bf16x2 p[2]; uint2 u; } w;
-      w.p[0] = pack_bf16(dk_acc[dt][4 * rq + 0] * a.scale, dk_acc[dt][4 * rq + 1] * a.scale);
-      w.p[1] = pack_bf16(dk_acc[dt][4 * rq + 2] * a.scale, dk_acc[dt][4 * rq + 3] * a.scale);
-      *(uint2*)(dkp + 32 * dt + 8 * rq + 4 * g) = w.u;
-      w.p[0] = pack_bf16(dv_acc[dt][4 * rq + 0], dv_acc[dt][4 * rq + 1]);
-      w.p[1] = pack_bf16(dv_acc[dt][4 * rq + 2], dv_acc[dt][4 * rq + 3]);
-      *(uint2*)(dvp + 32 * dt + 8 * rq + 4 * g) = w.u;
-    }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -556,11 +290,11 @@ int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream)
   } while (0)
   if (p.head_dim == 128) {
     if (phases & AXL_BWD_DELTA) AXL_LAUNCH((bwd_delta_kernel<__bf16, 128>), delta_grid, 0);
-    if (phases & AXL_BWD_DKDV) AXL_LAUNCH(flash_bwd_dkdv_bf16_kernel<128>, dkv_grid, DkvTile<128>::LDS_BYTES);
+    if ((phases & AXL_BWD_DKDV) && err == hipSuccess) err = launch_bwd_dkdv_bf16(a, 128, stream);
     if (phases & AXL_BWD_DQ) AXL_LAUNCH(flash_bwd_dq_bf16_kernel<128>, dq_grid, DqTile<128>::LDS_BYTES);
   } else {
     if (phases & AXL_BWD_DELTA) AXL_LAUNCH((bwd_delta_kernel<__bf16, 64>), delta_grid, 0);
-    if (phases & AXL_BWD_DKDV) AXL_LAUNCH(flash_bwd_dkdv_bf16_kernel<64>, dkv_grid, DkvTile<64>::LDS_BYTES);
+    if ((phases & AXL_BWD_DKDV) && err == hipSuccess) err = launch_bwd_dkdv_bf16(a, 64, stream);
     if (phases & AXL_BWD_DQ) AXL_LAUNCH(flash_bwd_dq_bf16_kernel<64>, dq_grid, DqTile<64>::LDS_BYTES);
   }
 #undef AXL_LAUNCH

@@ -1,0 +1,346 @@
+// dK / dV kernel of the flash-attention backward for gfx950 (bf16).
+//
+// Replaces axlearn/common/flash_attention/gpu_attention.py:436-528 (`_mha_backward_kernel_dkdv`):
+//   p = exp(qk - lse); dv += p^T dO; dp = dO v^T; ds = p * (dp - delta) * scale; dk += ds^T q,
+// with p and ds rounded to bf16 before their GEMMs and fp32 accumulation (:513, :518).
+//
+// Mapping.  A workgroup owns 128 keys of one (batch, kv head); each of its 4 wavefronts keeps the
+// K and V fragments of 32 keys in registers (B operands) and the fp32 dK^T / dV^T accumulators of
+// those keys (128 registers), and loops over ALL query heads of the kv head's group and all query
+// tiles that can see the keys, so dK/dV need neither atomics nor a pass that sums repeated KV
+// heads.  Query tiles (32 rows of Q and dO plus their lse / delta / segment ids) stream through a
+// three-deep LDS ring.
+//
+// Register pressure allows one wavefront per SIMD, so nobody else can cover this wavefront's
+// latencies; the loop is software pipelined by hand instead.  Iteration j runs
+//   stage A of tile j+1:  S = Q K^T and dP = dO V^T   (2*D/16 MFMAs, lane = key, registers = queries)
+//   stage B of tile j:    P = exp2(S*c - lse), dS = P * (dP - delta) elementwise, then
+//                         dV^T += dO^T P and dK^T += Q^T dS   (D/4 MFMAs, A operands from
+//                         transposing LDS reads of the same dO / Q tiles)
+// and the elementwise work of stage B is issued BETWEEN the MFMAs of stage A, one slice per MFMA, so
+// the VALU and the matrix pipe run at the same time.  Masks are evaluated arithmetically on every
+// tile (no branches inside the loop body: a branch would end the scheduling region).
+#include "flash_bwd.h"
+
+namespace axl {
+
+template <int D>
+struct DkvTile {
+  static constexpr int BKV = 128;            // keys per workgroup (32 per wavefront)
+  static constexpr int BQ = 32;              // query rows per LDS tile
+  // Each tile is kept twice, with the row pitch that makes its access pattern bank-conflict free:
+  // +16 bytes for the row-per-lane 128-bit fragment reads of stage A, +64 bytes for the transposing
+  // reads of stage B (4 rows x 64 bytes per 32 lanes).
+  static constexpr int STRIDE = D * 2 + 16;     // copy read by stage A
+  static constexpr int TSTRIDE = D * 2 + 64;    // copy read by stage B
+  static constexpr int TILE_BYTES = BQ * STRIDE;
+  static constexpr int TTILE_BYTES = BQ * TSTRIDE;
+  static constexpr int TR_BASE = 2 * TILE_BYTES;                 // Q | dO (A copies), then Q | dO (B copies)
+  static constexpr int STAT_BASE = 2 * TILE_BYTES + 2 * TTILE_BYTES;
+  static constexpr int STAT_BYTES = 3 * BQ * 4;  // lse | delta | segment id per query row
+  static constexpr int BUF_BYTES = STAT_BASE + STAT_BYTES;
+  static constexpr int NBUF = 3;
+  static constexpr int CHUNKS = BQ * D * 2 / 16 / 256;  // 16-byte chunks per thread per tensor
+  static constexpr int LDS_BYTES = NBUF * BUF_BYTES;
+};
+
+template <int D, bool HAS_SEG>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
+  using Tile = DkvTile<D>;
+  constexpr int KK = D / 16, DT = D / 32;
+  constexpr int NA = 2 * KK;          // stage-A MFMAs per tile
+  constexpr int NB = 4 * DT;          // stage-B MFMAs per tile
+  constexpr int EPM = 16 / NA;        // stage-B elements handled per stage-A MFMA
+  static_assert(16 % NA == 0 && Tile::BQ == 32, "tiling");
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+  const int G = a.Hq / a.Hkv;
+  // blockIdx -> (key block, batch, kv head); earliest key blocks (most queries under a causal
+  // mask) first.
+  const int kb = blockIdx.x / (a.B * a.Hkv);
+  const int rem = blockIdx.x % (a.B * a.Hkv);
+  const int b = rem / a.Hkv, hk = rem % a.Hkv;
+  const int k0_wg = kb * Tile::BKV;
+  const int k0 = k0_wg + wave * 32;  // this wavefront's keys
+
+  // K and V fragments (B operands): lane (key l32, k-group g) holds d = 16kk + 8g .. +7.
+  const __bf16* kp = (const __bf16*)a.k + b * a.ks.b + (int64_t)(k0 + l32) * a.ks.s + hk * a.ks.h;
+  const __bf16* vp = (const __bf16*)a.v + b * a.vs.b + (int64_t)(k0 + l32) * a.vs.s + hk * a.vs.h;
+  bf16x8 kf[KK], vf[KK];
+#pragma unroll
+  for (int kk = 0; kk < KK; kk++) {
+    kf[kk] = *(const bf16x8*)(kp + 16 * kk + 8 * g);
+    vf[kk] = *(const bf16x8*)(vp + 16 * kk + 8 * g);
+  }
+  const int kpos = k0 + l32;
+  int seg_k = 0;
+  if (HAS_SEG) seg_k = a.seg[(int64_t)b * a.T + k0 + l32];
+
+  // Query rows that can see any key of this workgroup.
+  int q_begin = 0, q_end = a.T;
+  if (a.mask_kind != AXL_MASK_NONE) {
+    q_begin = max(0, k0_wg - a.q_off);
+    if (a.mask_kind == AXL_MASK_SLIDING_WINDOW)
+      q_end = min(a.T, k0_wg + Tile::BKV - 1 + a.window - a.q_off + 1);
+  }
+  const int t_begin = q_begin / Tile::BQ;
+  const int nt = max(0, (q_end + Tile::BQ - 1) / Tile::BQ - t_begin);
+  const int total = nt * G;  // tiles in processing order: query head (outer) x query tile (inner)
+  // keep(q, k)  <=>  (unsigned)(qpos - kpos) <= limit
+  const unsigned limit = a.mask_kind == AXL_MASK_NONE             ? 0xffffffffu
+                         : a.mask_kind == AXL_MASK_SLIDING_WINDOW ? (unsigned)a.window
+                                                                  : 0x7fffffffu;
+
+  floatx16 dk_acc[DT], dv_acc[DT];
+#pragma unroll
+  for (int i = 0; i < DT; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) dk_acc[i][r] = dv_acc[i][r] = 0.f;
+  const float c = a.scale * kLog2e;
+
+  // ---- global -> LDS staging through registers (plain unrolled code: arrays stay in registers).
+  u32x4 qreg[Tile::CHUNKS], dreg[Tile::CHUNKS], sreg = {0, 0, 0, 0};
+  const int st_row = tid / (D / 8), st_cc = tid % (D / 8);
+  constexpr int ROWS_PER_PASS = 256 / (D / 8);
+  const __bf16* const q_base = (const __bf16*)a.q + b * a.qs.b + (int64_t)st_row * a.qs.s + st_cc * 8;
+  const __bf16* const d_base = (const __bf16*)a.dout + b * a.dos.b + (int64_t)st_row * a.dos.s + st_cc * 8;
+  const int st_lds = st_row * Tile::STRIDE + st_cc * 16;
+  const int st_lds_t = Tile::TR_BASE + st_row * Tile::TSTRIDE + st_cc * 16;
+  // Row statistics travel with the tile: threads 0..7 fetch lse (stored pre-multiplied by -log2 e),
+  // 8..15 delta, 16..23 segment ids; the other threads re-read lse and store nothing.
+  const int st_kind = tid >> 3, st_part = tid & 7;
+  // Running per-thread source pointers of the prefetch cursor, advanced by wave-uniform steps: no
+  // 64-bit multiplies inside the loop.  Tile sequence: query head (outer) x query tile (inner).
+  const __bf16* q_src = q_base + (int64_t)(hk * G) * a.qs.h + (int64_t)t_begin * Tile::BQ * a.qs.s;
+  const __bf16* d_src = d_base + (int64_t)(hk * G) * a.dos.h + (int64_t)t_begin * Tile::BQ * a.dos.s;
+  const int64_t stat_row0 = ((int64_t)b * a.Hq + hk * G) * a.T + (int64_t)t_begin * Tile::BQ + 4 * st_part;
+  const char* s_src = st_kind == 1 ? (const char*)(a.delta + stat_row0) : (const char*)(a.lse + stat_row0);
+  if (HAS_SEG && st_kind == 2)
+    s_src = (const char*)(a.seg + (int64_t)b * a.T + (int64_t)t_begin * Tile::BQ + 4 * st_part);
+  const bool s_is_seg = HAS_SEG && st_kind == 2;
+  const int64_t q_step = (int64_t)Tile::BQ * a.qs.s, d_step = (int64_t)Tile::BQ * a.dos.s;
+  const int64_t q_wrap = a.qs.h - (int64_t)(nt - 1) * q_step;    // last tile of a head -> first of next
+  const int64_t d_wrap = a.dos.h - (int64_t)(nt - 1) * d_step;
+  const int64_t s_step = Tile::BQ * 4, s_wrap = ((int64_t)a.T - (int64_t)(nt - 1) * Tile::BQ) * 4;
+  const int64_t seg_wrap = -(int64_t)(nt - 1) * Tile::BQ * 4;   // segment ids do not depend on the head
+#define AXL_LOAD_TILE()                                                                           \
+  {                                                                                               \
+    _Pragma("unroll") for (int i = 0; i < Tile::CHUNKS; i++) {                                    \
+      qreg[i] = *(const u32x4*)(q_src + (int64_t)(i * ROWS_PER_PASS) * a.qs.s);                   \
+      dreg[i] = *(const u32x4*)(d_src + (int64_t)(i * ROWS_PER_PASS) * a.dos.s);                  \
+    }                                                                                             \
+    sreg = *(const u32x4*)s_src;                                                                  \
+  }
+#define AXL_STORE_TILE(BUF_)                                                                      \
+  {                                                                                               \
+    _Pragma("unroll") for (int i = 0; i < Tile::CHUNKS; i++) {                                    \
+      *(u32x4*)((BUF_) + st_lds + i * ROWS_PER_PASS * Tile::STRIDE) = qreg[i];                    \
+      *(u32x4*)((BUF_) + Tile::TILE_BYTES + st_lds + i * ROWS_PER_PASS * Tile::STRIDE) = dreg[i]; \
+      *(u32x4*)((BUF_) + st_lds_t + i * ROWS_PER_PASS * Tile::TSTRIDE) = qreg[i];                 \
+      *(u32x4*)((BUF_) + Tile::TTILE_BYTES + st_lds_t + i * ROWS_PER_PASS * Tile::TSTRIDE) = dreg[i]; \
+    }                                                                                             \
+    if (tid < 24) {                                                                               \
+      union { u32x4 u; floatx4 f; } w_;                                                           \
+      w_.u = sreg;                                                                                \
+      if (st_kind == 0) w_.f = w_.f * (-kLog2e);                                                  \
+      *(u32x4*)((BUF_) + Tile::STAT_BASE + st_kind * (Tile::BQ * 4) + st_part * 16) = w_.u;       \
+    }                                                                                             \
+  }
+  // Prefetch cursor; it stops at the last tile (re-fetching that tile is harmless).
+  int pf_idx = 0, pf_t = 0;
+#define AXL_ADVANCE()                                                       \
+  {                                                                         \
+    const bool adv_ = pf_idx + 1 < total;                                   \
+    const bool wrap_ = adv_ && (pf_t + 1 == nt);                            \
+    pf_idx += adv_ ? 1 : 0;                                                 \
+    pf_t = wrap_ ? 0 : pf_t + (adv_ ? 1 : 0);                               \
+    q_src += adv_ ? (wrap_ ? q_wrap : q_step) : 0;                          \
+    d_src += adv_ ? (wrap_ ? d_wrap : d_step) : 0;                          \
+    s_src += adv_ ? (wrap_ ? (s_is_seg ? seg_wrap : s_wrap) : s_step) : 0;  \
+  }
+
+  char* buf_b = smem;                         // tile j     (stage B)
+  char* buf_a = smem + Tile::BUF_BYTES;       // tile j + 1 (stage A)
+  char* buf_s = smem + 2 * Tile::BUF_BYTES;   // tile j + 2 (being filled)
+
+  const int a_row_off = swap_bits_2_3(l32) * Tile::STRIDE + g * 16;  // normal (row = query) reads
+  const int j16 = lane & 15, half = (lane >> 4) & 1;
+  const int tr_off =
+      Tile::TR_BASE + (8 * g + (j16 >> 2)) * Tile::TSTRIDE + (16 * half + 4 * (j16 & 3)) * 2;
+
+  floatx16 s_cur, dp_cur;
+#pragma unroll
+  for (int r = 0; r < 16; r++) s_cur[r] = dp_cur[r] = 0.f;
+  int q0_b = t_begin * Tile::BQ, q0_a = q0_b;
+
+  if (total > 0) {
+    AXL_LOAD_TILE()
+    AXL_STORE_TILE(buf_b)
+    AXL_ADVANCE()
+    q0_a = (t_begin + pf_t) * Tile::BQ;
+    AXL_LOAD_TILE()
+    AXL_STORE_TILE(buf_a)
+  }
+  wait_all_vmem();  // stationary fragments have landed: nothing issued before the loop is pending
+  __syncthreads();
+  if (total > 0) {
+    // Stage A of tile 0.
+#pragma unroll
+    for (int kk = 0; kk < KK; kk++) {
+      const bf16x8 qa = *(const bf16x8*)(buf_b + a_row_off + kk * 32);
+      const bf16x8 da = *(const bf16x8*)(buf_b + Tile::TILE_BYTES + a_row_off + kk * 32);
+      s_cur = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa, kf[kk], s_cur, 0, 0, 0);
+      dp_cur = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da, vf[kk], dp_cur, 0, 0, 0);
+    }
+  }
+
+  union TrFrag {
+    bf16x8 v;
+    shortx4 hlf[2];
+  };
+
+  for (int j = 0; j < total; j++) {
+    AXL_ADVANCE()
+    const int q0_p = (t_begin + pf_t) * Tile::BQ;
+    AXL_LOAD_TILE()
+
+    // Row statistics of tile j: register r of lane group g is query q0_b + 16(r/8) + 8g + (r%8).
+    const char* st = buf_b + Tile::STAT_BASE + 8 * g * 4;
+    floatx4 lse_v[4], del_v[4];
+    intx4 seg_v[4];
+#pragma unroll
+    for (int t8 = 0; t8 < 2; t8++) {
+      lse_v[2 * t8] = *(const floatx4*)(st + 64 * t8);
+      lse_v[2 * t8 + 1] = *(const floatx4*)(st + 64 * t8 + 16);
+      del_v[2 * t8] = *(const floatx4*)(st + Tile::BQ * 4 + 64 * t8);
+      del_v[2 * t8 + 1] = *(const floatx4*)(st + Tile::BQ * 4 + 64 * t8 + 16);
+      if (HAS_SEG) {
+        seg_v[2 * t8] = *(const intx4*)(st + 2 * Tile::BQ * 4 + 64 * t8);
+        seg_v[2 * t8 + 1] = *(const intx4*)(st + 2 * Tile::BQ * 4 + 64 * t8 + 16);
+      }
+    }
+    const int diff0 = (q0_b + a.q_off + 8 * g) - kpos;  // query of r == 0 minus this lane's key
+
+    // ---- stage A of tile j+1 interleaved with the elementwise part of stage B of tile j.
+    // Stage-A step n: even n -> S chain (Q fragment n/2), odd n -> dP chain (dO fragment n/2).
+    constexpr int kAheadA = 6;
+    bf16x8 afr[NA];
+#define AXL_A_READ(N_) \
+  afr[N_] = *(const bf16x8*)(buf_a + ((N_) % 2) * Tile::TILE_BYTES + a_row_off + ((N_) / 2) * 32);
+#pragma unroll
+    for (int n = 0; n < (kAheadA < NA ? kAheadA : NA); n++) AXL_A_READ(n)
+    floatx16 s_nxt, dp_nxt;
+#pragma unroll
+    for (int r = 0; r < 16; r++) s_nxt[r] = dp_nxt[r] = 0.f;
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int n = 0; n < NA; n++) {
+      if (n + kAheadA < NA) AXL_A_READ(n + kAheadA)
+      if (n % 2 == 0)
+        s_nxt = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afr[n], kf[n / 2], s_nxt, 0, 0, 0);
+      else
+        dp_nxt = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afr[n], vf[n / 2], dp_nxt, 0, 0, 0);
+#pragma unroll
+      for (int e = 0; e < EPM; e++) {
+        const int r = n * EPM + e;
+        const unsigned diff = (unsigned)(diff0 + 16 * (r / 8) + (r % 8));
+        float sv = diff <= limit ? s_cur[r] : kMasked;
+        if (HAS_SEG) sv = seg_v[r / 4][r % 4] == seg_k ? sv : kMasked;
+        const float p = fast_exp2(__builtin_fmaf(sv, c, lse_v[r / 4][r % 4]));  // lse_v = -lse*log2e
+        s_cur[r] = p;
+        dp_cur[r] = p * (dp_cur[r] - del_v[r / 4][r % 4]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#undef AXL_A_READ
+
+    // ---- stage B MFMAs of tile j: dV^T += dO^T P ; dK^T += Q^T dS  (scale applied at the end).
+    bf16x8 pb[2], dsb[2];
+#pragma unroll
+    for (int t8 = 0; t8 < 2; t8++) {
+      pb[t8] = pack_bf16x8(s_cur[8 * t8 + 0], s_cur[8 * t8 + 1], s_cur[8 * t8 + 2], s_cur[8 * t8 + 3],
+                           s_cur[8 * t8 + 4], s_cur[8 * t8 + 5], s_cur[8 * t8 + 6], s_cur[8 * t8 + 7]);
+      dsb[t8] = pack_bf16x8(dp_cur[8 * t8 + 0], dp_cur[8 * t8 + 1], dp_cur[8 * t8 + 2], dp_cur[8 * t8 + 3],
+                            dp_cur[8 * t8 + 4], dp_cur[8 * t8 + 5], dp_cur[8 * t8 + 6], dp_cur[8 * t8 + 7]);
+    }
+    // Step n = t8 * 2DT + dt * 2 + which; which 0: dV (dO^T fragment, P), 1: dK (Q^T fragment, dS).
+    constexpr int kAheadB = 4;
+    TrFrag bfr[NB];
+#define AXL_B_READ(N_)                                                                           \
+  {                                                                                              \
+    const char* p_ = buf_b + (((N_) % 2) == 0 ? Tile::TTILE_BYTES : 0) +                         \
+                     16 * ((N_) / (2 * DT)) * Tile::TSTRIDE + tr_off + (((N_) % (2 * DT)) / 2) * 64; \
+    bfr[N_].hlf[0] = lds_read_tr16(p_);                                                          \
+    bfr[N_].hlf[1] = lds_read_tr16(p_ + 4 * Tile::TSTRIDE);                                      \
+  }
+#pragma unroll
+    for (int n = 0; n < kAheadB; n++) AXL_B_READ(n)
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int n = 0; n < NB; n++) {
+      if (n + kAheadB < NB) AXL_B_READ(n + kAheadB)
+      const int t8 = n / (2 * DT), dt = (n % (2 * DT)) / 2;
+      if (n % 2 == 0)
+        dv_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[n].v, pb[t8], dv_acc[dt], 0, 0, 0);
+      else
+        dk_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[n].v, dsb[t8], dk_acc[dt], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#undef AXL_B_READ
+
+    AXL_STORE_TILE(buf_s)
+    __syncthreads();
+    char* const tmp = buf_b;
+    buf_b = buf_a;
+    buf_a = buf_s;
+    buf_s = tmp;
+    s_cur = s_nxt;
+    dp_cur = dp_nxt;
+    q0_b = q0_a;
+    q0_a = q0_p;
+  }
+#undef AXL_LOAD_TILE
+#undef AXL_STORE_TILE
+#undef AXL_ADVANCE
+
+  __bf16* dkp = (__bf16*)a.dk + b * a.dks.b + (int64_t)(k0 + l32) * a.dks.s + hk * a.dks.h;
+  __bf16* dvp = (__bf16*)a.dv + b * a.dvs.b + (int64_t)(k0 + l32) * a.dvs.s + hk * a.dvs.h;
+#pragma unroll
+  for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+    for (int rq = 0; rq < 4; rq++) {
+      union {
+        bf16x2 p[2];
+        uint2 u;
+      } w;
+      w.p[0] = pack_bf16(dk_acc[dt][4 * rq + 0] * a.scale, dk_acc[dt][4 * rq + 1] * a.scale);
+      w.p[1] = pack_bf16(dk_acc[dt][4 * rq + 2] * a.scale, dk_acc[dt][4 * rq + 3] * a.scale);
+      *(uint2*)(dkp + 32 * dt + 8 * rq + 4 * g) = w.u;
+      w.p[0] = pack_bf16(dv_acc[dt][4 * rq + 0], dv_acc[dt][4 * rq + 1]);
+      w.p[1] = pack_bf16(dv_acc[dt][4 * rq + 2], dv_acc[dt][4 * rq + 3]);
+      *(uint2*)(dvp + 32 * dt + 8 * rq + 4 * g) = w.u;
+    }
+}
+
+template <int D, bool HAS_SEG>
+static hipError_t launch_one(const BwdArgs& a, hipStream_t stream) {
+  using Tile = DkvTile<D>;
+  auto kernel = flash_bwd_dkdv_bf16_kernel<D, HAS_SEG>;
+  hipError_t err = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       Tile::LDS_BYTES);
+  if (err != hipSuccess) return err;
+  const int grid = (a.S / Tile::BKV) * a.B * a.Hkv;
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), Tile::LDS_BYTES, stream, a);
+  return hipGetLastError();
+}
+
+hipError_t launch_bwd_dkdv_bf16(const BwdArgs& a, int head_dim, hipStream_t stream) {
+  const bool seg = a.seg != nullptr;
+  if (head_dim == 128) return seg ? launch_one<128, true>(a, stream) : launch_one<128, false>(a, stream);
+  return seg ? launch_one<64, true>(a, stream) : launch_one<64, false>(a, stream);
+}
+
+}  // namespace axl
