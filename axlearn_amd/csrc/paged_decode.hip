@@ -61,21 +61,80 @@ __device__ __forceinline__ float row16_sum(float x) {
   return x;
 }
 
-template <int D, int GP, bool PAGED>
+// One 16-byte-per-lane direct global->LDS load: lane l's 16 bytes land at lds_base + 16*l.  Issued
+// through inline assembly so that the compiler neither tracks it nor waits for it; completion is
+// in issue order and is awaited with wait_vmem_le<N>().
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ void dma16(const void* gsrc, unsigned lds_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+               :
+               : "v"(gsrc), "s"(lds_base)
+               : "memory", "m0");
+}
+#pragma clang diagnostic pop
+template <int N>
+__device__ __forceinline__ void wait_vmem_le() {
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+__device__ __forceinline__ void wait_lds_reads() { asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory"); }
+
+// XOR swizzle of the 16-byte chunks of a K row inside an LDS tile, so that 16 lanes reading the
+// same logical chunk of 16 different rows hit 16 different bank groups.
+template <int D>
+__device__ __forceinline__ int k_swizzle(int row) {
+  if (D == 128) return ((row & 3) << 2) | ((row >> 2) & 3);
+  return (((row >> 1) & 1) << 2) | ((row >> 2) & 3);
+}
+
+// The same for V rows: the transposing read of a 16-column block touches 32 bytes of 16 rows;
+// rows 0..7 (and 8..15) are spread over all banks.
+template <int D>
+__device__ __forceinline__ int v_swizzle(int row) {
+  if (D == 128) return 2 * (row & 7);
+  return 2 * ((row >> 1) & 3);
+}
+
+template <int D, int GP, int NST>
+struct DecTile {
+  static constexpr int ROW_BYTES = D * 2;
+  static constexpr int TILE_BYTES = kPage * ROW_BYTES;   // K (or V) of one page
+  static constexpr int STAGE_BYTES = 2 * TILE_BYTES;     // K then V
+  static constexpr int RING_BYTES = 4 * NST * STAGE_BYTES;
+  static constexpr int RED_BYTES = 2 * 4 * 16 * 4;
+  static constexpr int RED_BASE = RING_BYTES;
+  static constexpr int LDS_BYTES = RED_BASE + RED_BYTES;
+  static constexpr int RED_O_PITCH = D + 4;              // floats per (wave, head) row of the epilogue
+  static_assert(4 * GP * RED_O_PITCH * 4 <= RING_BYTES, "epilogue staging must fit in the ring");
+};
+
+// Work decomposition: grid (chunk, kv head, sequence); the 4 wavefronts of a workgroup take the
+// pages of the chunk round-robin.  Per page a wavefront computes
+//   S^T = K Q^T     (v_mfma_f32_16x16x32_bf16, A = K rows from LDS, B = Q^T held in registers),
+//   O^T += V^T P^T  (v_mfma_f32_16x16x16_bf16, A = V^T through transposing LDS reads, B = P^T),
+// in the "transposed" form where lane l owns query head l%16 and the tokens 4*(l/16)..+3 of the
+// page: the accumulator layout of S^T is exactly the B-operand layout of the second product, so
+// probabilities never leave registers, and every softmax statistic is per lane.
+template <int D, int GP, bool PAGED, int NST>
 __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
-  constexpr int KSTEPS = D / 32;        // MFMA k-steps over head_dim
+  using Tile = DecTile<D, GP, NST>;
+  constexpr int KSTEPS = D / 32;        // MFMA k-steps over head_dim for S^T
+  constexpr int NB = D / 16;            // 16-row blocks of O^T
   constexpr int SL = D / 8;             // 16-byte slices per token row
-  constexpr int TPL = 64 / SL;          // token rows covered by one wave-wide V load
-  constexpr int NLOAD = kPage / TPL;    // V loads per page
-  constexpr int HG = GP / 4;            // 4-head groups in use (MFMA row groups)
-  __shared__ __attribute__((aligned(16))) float p_lds[4][kPage + 1][16];   // [wave][token | corr][head]
-  __shared__ __attribute__((aligned(16))) float red_o[4 * TPL][GP * D / 4 + 4]; // epilogue partials, see below
-  __shared__ float red_m[4][16], red_l[4][16];
+  constexpr int TPL = 64 / SL;          // token rows covered by one wave-wide load
+  constexpr int NLOAD = kPage / TPL;    // wave-wide loads per K (or V) page
+  constexpr int LPP = 2 * NLOAD;        // loads in flight per page
+  static_assert(LPP * (NST - 1) <= 63, "vmcnt is 6 bits");
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  float(*red_o)[Tile::RED_O_PITCH] = (float(*)[Tile::RED_O_PITCH])smem;  // [wave*GP + head][d], aliases the ring
+  float(*red_m)[16] = (float(*)[16])(smem + Tile::RED_BASE);
+  float(*red_l)[16] = red_m + 4;
 
   const int tid = threadIdx.x;
-  const int wave = tid >> 6, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int chunk = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
-  const int len = a.lengths[b];
+  int len = a.lengths[b];
+  if (!PAGED) len = min(len, a.kv_len);
   int npages = (len + kPage - 1) / kPage;
   npages = min(npages, a.pps);
   int first_page = 0;
@@ -83,195 +142,195 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
   const int c_begin = max(chunk * a.chunk_pages, first_page);
   const int c_end = min((chunk + 1) * a.chunk_pages, npages);
   if (c_begin >= c_end) return;  // nothing live in this chunk (uniform for the whole workgroup)
+  // This wavefront owns pages c_begin + wave + 4*it, it = 0 .. n_my-1.
+  const int n_my = (c_end - c_begin - wave + 3) >> 2;
 
-  // Q as MFMA A operand: lane (head row = lane%16, k-group = lane/16) holds d = 32s + 8kg .. +7.
-  const int qrow = lane & 15, kg = lane >> 4;
+  // Q^T as MFMA B operand: lane (head column = lane%16, k-group = lane/16) holds d = 32s + 8kg .. +7.
+  const int head = lane & 15, kg = lane >> 4;
   bf16x8 qf[KSTEPS];
 #pragma unroll
   for (int s = 0; s < KSTEPS; s++) {
-    if (qrow < a.G) {
-      qf[s] = *(const bf16x8*)(a.q + ((int64_t)b * a.Hq + hk * a.G + qrow) * D + 32 * s + 8 * kg);
+    if (head < a.G) {
+      qf[s] = *(const bf16x8*)(a.q + ((int64_t)b * a.Hq + hk * a.G + head) * D + 32 * s + 8 * kg);
     } else {
 #pragma unroll
       for (int e = 0; e < 8; e++) qf[s][e] = (__bf16)0.f;
     }
   }
-  const int tok = lane & 15;          // K layout / MFMA C layout: token column
-  const int hg = lane >> 4;           // MFMA C layout: heads 4hg..4hg+3
-  const int vslice = lane % SL;       // V layout: 16-byte slice of the row
-  const int vtok = lane / SL;         // V layout: token row within a load
+  // Page ids of this wavefront's pages, one per lane (chunk_pages <= 256).
+  int my_pages = 0;
+  if (PAGED && lane < n_my) my_pages = a.page_tables[(int64_t)b * a.pps + c_begin + wave + 4 * lane];
+
+  const int vslice = lane % SL;       // load layout: 16-byte slice of the row
+  const int vtok = lane / SL;         // load layout: token row within a load
   const float c = a.scale * kLog2e;
 
-  float m_run[4], l_run[4];
+  float m_run = kNegInf, l_run = 0.f;
+  floatx4 o[NB];                      // O^T rows d = 16nb + 4kg + r, column = head
 #pragma unroll
-  for (int r = 0; r < 4; r++) { m_run[r] = kNegInf; l_run[r] = 0.f; }
-  float o[GP][8];
-#pragma unroll
-  for (int gq = 0; gq < GP; gq++)
-#pragma unroll
-    for (int e = 0; e < 8; e++) o[gq][e] = 0.f;
+  for (int nb = 0; nb < NB; nb++) o[nb] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  auto page_base = [&](int j, const __bf16* base, const Strides3& st, bool& valid) -> const __bf16* {
-    if (PAGED) {
-      int pg = __builtin_amdgcn_readfirstlane(a.page_tables[(int64_t)b * a.pps + j]);
-      if (pg < 0) pg += a.num_pages;  // negative indices count from the end, as in the reference's gather
-      valid = (unsigned)pg < (unsigned)a.num_pages;
-      return base + ((int64_t)hk * a.num_pages + (valid ? pg : 0)) * (kPage * D);
-    } else {
-      valid = true;
-      return base + b * st.b + (int64_t)j * kPage * st.s + hk * st.h;
-    }
-  };
+  // Per-lane source offsets (elements) of the wave-wide loads of a page, and LDS read offsets.
+  // Both tiles are stored with their 16-byte chunks XOR-swizzled by a function of the row, which
+  // makes the K reads (16 lanes = 16 rows, same chunk) and the transposing V reads (rows 0..7 of
+  // the same 32-byte column window) hit distinct banks.
   const int64_t k_row_stride = PAGED ? D : a.ks.s;
   const int64_t v_row_stride = PAGED ? D : a.vs.s;
-
-  uint4 kreg[KSTEPS], vreg[NLOAD];
-  auto load_k = [&](int j) {
-    bool valid;
-    const __bf16* base = page_base(j, a.k, a.ks, valid);
+  int k_src[NLOAD], v_src[NLOAD];
 #pragma unroll
-    for (int s = 0; s < KSTEPS; s++) {
-      const bool ok = valid && (PAGED || j * kPage + tok < a.kv_len);
-      kreg[s] = ok ? *(const uint4*)(base + tok * k_row_stride + 32 * s + 8 * kg) : uint4{0, 0, 0, 0};
+  for (int i = 0; i < NLOAD; i++) {
+    const int row = TPL * i + vtok;
+    k_src[i] = (vslice ^ k_swizzle<D>(row)) * 8;     // + row * stride, added per page
+    v_src[i] = (vslice ^ v_swizzle<D>(row)) * 8;
+  }
+  int k_rd[KSTEPS];
+#pragma unroll
+  for (int s = 0; s < KSTEPS; s++) k_rd[s] = (lane & 15) * Tile::ROW_BYTES + (((4 * s + kg) ^ k_swizzle<D>(lane & 15)) << 4);
+  // Transposing V read for block nb: this lane points at row 4kg + (lane%16)/4, columns
+  // 16nb + 4*(lane%4) .. +3, i.e. chunk 2nb + (lane%4)/2, half (lane%4)%2.
+  const int vrow = 4 * kg + ((lane & 15) >> 2);
+  const int v_rd0 = vrow * Tile::ROW_BYTES + ((lane & 2) << 3) + ((lane & 1) << 3);
+  const int v_xor = v_swizzle<D>(vrow) << 4;
+  const unsigned ring_lds = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)smem +
+                            wave * (NST * Tile::STAGE_BYTES);
+  char* ring = smem + wave * (NST * Tile::STAGE_BYTES);
+
+  // Everything the compiler tracks has landed before the first untracked load is issued.
+  wait_all_vmem();
+
+  // Issues the 2*NLOAD loads of this wavefront's page `it` into ring stage `st`.
+  auto issue = [&](int it, int st) {
+    const int j = c_begin + wave + 4 * it;
+    const __bf16 *kb, *vb;
+    if (PAGED) {
+      int pg = __builtin_amdgcn_readlane(my_pages, it);
+      if (pg < 0) pg += a.num_pages;  // negative indices count from the end, as in the reference's gather
+      if ((unsigned)pg >= (unsigned)a.num_pages) pg = 0;  // reads as zeros: see `valid` below
+      const int64_t off = ((int64_t)hk * a.num_pages + pg) * (kPage * D);
+      kb = a.k + off;
+      vb = a.v + off;
+    } else {
+      kb = a.k + b * a.ks.b + hk * a.ks.h;
+      vb = a.v + b * a.vs.b + hk * a.vs.h;
     }
-  };
-  auto load_v = [&](int j) {
-    bool valid;
-    const __bf16* base = page_base(j, a.v, a.vs, valid);
+    const unsigned dst = __builtin_amdgcn_readfirstlane(ring_lds + st * Tile::STAGE_BYTES);
 #pragma unroll
     for (int i = 0; i < NLOAD; i++) {
-      const int t = TPL * i + vtok;
-      const bool ok = valid && (PAGED || j * kPage + t < a.kv_len);
-      vreg[i] = ok ? *(const uint4*)(base + t * v_row_stride + 8 * vslice) : uint4{0, 0, 0, 0};
+      // Rows past the end of a contiguous cache are clamped to its last row; they are masked.
+      const int row = PAGED ? TPL * i + vtok : min(j * kPage + TPL * i + vtok, a.kv_len - 1);
+      dma16(kb + row * k_row_stride + k_src[i], dst + i * 1024);
+    }
+#pragma unroll
+    for (int i = 0; i < NLOAD; i++) {
+      const int row = PAGED ? TPL * i + vtok : min(j * kPage + TPL * i + vtok, a.kv_len - 1);
+      dma16(vb + row * v_row_stride + v_src[i], dst + Tile::TILE_BYTES + i * 1024);
     }
   };
 
-  int j = c_begin + wave;
-  if (j < c_end) {
-    load_k(j);
-    load_v(j);
-  }
-  for (; j < c_end; j += 4) {
-    // ---- scores for this page: S[head][token] = Q K^T
+#pragma unroll
+  for (int st = 0; st < NST; st++)
+    if (st < n_my) issue(st, st);
+
+  int st = 0;
+  for (int it = 0; it < n_my; it++) {
+    const int j = c_begin + wave + 4 * it;
+    // Wait for this page; up to NST-1 younger pages stay in flight.
+    const int younger = min(NST - 1, n_my - 1 - it);
+    if (NST > 3 && younger == 3) wait_vmem_le<(NST > 3 ? 3 : 0) * LPP>();
+    else if (NST > 2 && younger == 2) wait_vmem_le<(NST > 2 ? 2 : 0) * LPP>();
+    else if (NST > 1 && younger == 1) wait_vmem_le<(NST > 1 ? 1 : 0) * LPP>();
+    else wait_vmem_le<0>();
+    bool valid = true;
+    if (PAGED) {
+      int pg = __builtin_amdgcn_readlane(my_pages, it);
+      if (pg < 0) pg += a.num_pages;
+      valid = (unsigned)pg < (unsigned)a.num_pages;
+    }
+    const char* kt = ring + st * Tile::STAGE_BYTES;
+    const char* vt = kt + Tile::TILE_BYTES;
+    bf16x8 kf[KSTEPS];
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks++) kf[ks] = *(const bf16x8*)(kt + k_rd[ks]);
+    shortx4 vf[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++) vf[nb] = lds_read_tr16(vt + v_rd0 + ((nb * 32) ^ v_xor));
+    // ---- scores: S^T[token][head]; this lane: head = lane%16, tokens 4kg + r
     floatx4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int st = 0; st < KSTEPS; st++) {
-      union { uint4 u; bf16x8 v; } kf;
-      kf.u = kreg[st];
-      s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[st], kf.v, s, 0, 0, 0);
-    }
-    const int jn = j + 4;
-    if (jn < c_end) load_k(jn);  // K registers are free again: next page's K goes in flight now
-    const int tpos = j * kPage + tok;
-    bool keep = tpos < len;
-    if (a.window >= 0) keep = keep && (len - 1 - tpos <= a.window);
-    float pm[4], corr[4];
-    bool changed = false;
-#pragma unroll
-    for (int r = 0; r < 4; r++) {
-      s[r] = keep ? s[r] : kMasked;
-      pm[r] = row16_max(s[r]);
-      const float mn = fmaxf(m_run[r], pm[r]);
-      changed = changed || (mn != m_run[r]);
-      corr[r] = fast_exp2((m_run[r] - mn) * c);
-      m_run[r] = mn;
-      s[r] = fast_exp2((s[r] - mn) * c);
-      l_run[r] = l_run[r] * corr[r] + s[r];
-    }
-    const bool any_changed = __builtin_amdgcn_ballot_w64(changed && hg < HG) != 0;
-    if (hg < HG) {
-      *(float4*)&p_lds[wave][tok][4 * hg] = float4{s[0], s[1], s[2], s[3]};
-      if (any_changed && tok == 0)
-        *(float4*)&p_lds[wave][kPage][4 * hg] = float4{corr[0], corr[1], corr[2], corr[3]};
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    // ---- O += P V on the coalesced V layout
+    for (int ks = 0; ks < KSTEPS; ks++) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[ks], qf[ks], s, 0, 0, 0);
     // A page that straddles the length (or the window start) holds tokens whose probability is
     // exactly 0; their V rows may be uninitialised pool memory, and 0 * NaN would poison the sum,
-    // so those rows are replaced by zeros.  Only boundary pages pay for this.
+    // so those rows are replaced by zeros, as are all rows of a page outside the pool.
     const bool boundary = (j * kPage + kPage > len) || (a.window >= 0 && len - 1 - j * kPage > a.window);
-    if (boundary) {
+    if (boundary || !valid) {
+      if (!valid) s = floatx4{0.f, 0.f, 0.f, 0.f};  // a page outside the pool reads as zeros
 #pragma unroll
-      for (int i = 0; i < NLOAD; i++) {
-        const int vpos = j * kPage + TPL * i + vtok;
-        bool vkeep = vpos < len;
-        if (a.window >= 0) vkeep = vkeep && (len - 1 - vpos <= a.window);
-        if (!vkeep) vreg[i] = uint4{0, 0, 0, 0};
+      for (int r = 0; r < 4; r++) {
+        const int tpos = j * kPage + 4 * kg + r;
+        bool keep = tpos < len;
+        if (a.window >= 0) keep = keep && (len - 1 - tpos <= a.window);
+        s[r] = keep ? s[r] : kMasked;
+        if (!keep || !valid) {
+#pragma unroll
+          for (int nb = 0; nb < NB; nb++) vf[nb][r] = 0;
+        }
       }
     }
-    if (any_changed) {
-#pragma unroll
-      for (int gq = 0; gq < GP; gq++) {
-        const float cg = p_lds[wave][kPage][gq];
-#pragma unroll
-        for (int e = 0; e < 8; e++) o[gq][e] *= cg;
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < NLOAD; i++) {
-      float pv[GP];
-#pragma unroll
-      for (int g4 = 0; g4 < GP / 4; g4++) {
-        const float4 x = *(const float4*)&p_lds[wave][TPL * i + vtok][4 * g4];
-        pv[4 * g4 + 0] = x.x; pv[4 * g4 + 1] = x.y; pv[4 * g4 + 2] = x.z; pv[4 * g4 + 3] = x.w;
-      }
-      const uint32_t w[4] = {vreg[i].x, vreg[i].y, vreg[i].z, vreg[i].w};
-      float ve[8];
-#pragma unroll
-      for (int e = 0; e < 4; e++) {
-        ve[2 * e] = __uint_as_float(w[e] << 16);
-        ve[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
-      }
-#pragma unroll
-      for (int gq = 0; gq < GP; gq++)
-#pragma unroll
-        for (int e = 0; e < 8; e++) o[gq][e] = __builtin_fmaf(pv[gq], ve[e], o[gq][e]);
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    if (jn < c_end) load_v(jn);
-  }
-
-  // ---- merge the 4 wavefronts x (64/SL) lane groups of this workgroup.
-#pragma unroll
-  for (int r = 0; r < 4; r++) l_run[r] = row16_sum(l_run[r]);
-  if (tok == 0 && hg < HG) {
+    float mx = fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]));
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float mn = fmaxf(m_run, mx);
+    const bool changed = mn != m_run;
+    const float corr = fast_exp2((m_run - mn) * c);
+    m_run = mn;
+    float psum = 0.f;
 #pragma unroll
     for (int r = 0; r < 4; r++) {
-      red_m[wave][4 * hg + r] = m_run[r];
-      red_l[wave][4 * hg + r] = l_run[r];
+      s[r] = fast_exp2((s[r] - mn) * c);
+      psum += s[r];
+    }
+    l_run = l_run * corr + psum;
+    union { shortx4 v; bf16x2 p[2]; } pf;
+    pf.p[0] = pack_bf16(s[0], s[1]);
+    pf.p[1] = pack_bf16(s[2], s[3]);
+    if (__builtin_amdgcn_ballot_w64(changed) != 0) {
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++) o[nb] *= corr;
+    }
+    // ---- O^T += V^T P^T
+#pragma unroll
+    for (int nb = 0; nb < NB; nb++)
+      o[nb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf[nb], pf.v, o[nb], 0, 0, 0);
+    // Every LDS read of this stage has returned (the MFMAs consumed them) before new data is
+    // directed at it.
+    wait_lds_reads();
+    if (it + NST < n_my) issue(it + NST, st);
+    st = (st + 1 == NST) ? 0 : st + 1;
+  }
+
+  // ---- merge the 4 wavefronts of this workgroup.
+  l_run += __shfl_xor(l_run, 16, 64);
+  l_run += __shfl_xor(l_run, 32, 64);
+  if (kg == 0) {
+    red_m[wave][head] = m_run;
+    red_l[wave][head] = l_run;
+  }
+  __syncthreads();  // also: every wavefront is done with its ring, which red_o aliases
+  {
+    const float mw = fmaxf(fmaxf(red_m[0][head], red_m[1][head]), fmaxf(red_m[2][head], red_m[3][head]));
+    const float f_wave = fast_exp2((m_run - mw) * c);
+    if (head < GP) {
+#pragma unroll
+      for (int nb = 0; nb < NB; nb++)
+        *(float4*)&red_o[wave * GP + head][16 * nb + 4 * kg] =
+            float4{o[nb][0] * f_wave, o[nb][1] * f_wave, o[nb][2] * f_wave, o[nb][3] * f_wave};
     }
   }
   __syncthreads();
-  float f_wave[GP];
-#pragma unroll
-  for (int gq = 0; gq < GP; gq++) {
-    const float mw = fmaxf(fmaxf(red_m[0][gq], red_m[1][gq]), fmaxf(red_m[2][gq], red_m[3][gq]));
-    f_wave[gq] = fast_exp2((red_m[wave][gq] - mw) * c);
-  }
-  // red_o rows: one per partial (wave * TPL + vtok); columns: head-in-quarter * D + d.  The heads
-  // are reduced a quarter at a time to keep the staging buffer small.
-  constexpr int NPART = 4 * TPL;  // partial outputs per element
   float* out_ws = a.ws_o + (((int64_t)b * a.Hkv + hk) * a.nch + chunk) * (GP * D);
-#pragma unroll
-  for (int q4 = 0; q4 < 4; q4++) {  // heads q4*GP/4 .. (q4+1)*GP/4 - 1
-    __syncthreads();
-#pragma unroll
-    for (int gi = 0; gi < GP / 4; gi++) {
-      const int gq = q4 * (GP / 4) + gi;
-      float* dst = &red_o[wave * TPL + vtok][gi * D + 8 * vslice];
-      *(float4*)dst = float4{o[gq][0] * f_wave[gq], o[gq][1] * f_wave[gq], o[gq][2] * f_wave[gq], o[gq][3] * f_wave[gq]};
-      *(float4*)(dst + 4) = float4{o[gq][4] * f_wave[gq], o[gq][5] * f_wave[gq], o[gq][6] * f_wave[gq], o[gq][7] * f_wave[gq]};
-    }
-    __syncthreads();
-    for (int idx = tid; idx < GP / 4 * D; idx += 256) {
-      float acc = 0.f;
-#pragma unroll
-      for (int pidx = 0; pidx < NPART; pidx++) acc += red_o[pidx][idx];
-      out_ws[q4 * (GP / 4) * D + idx] = acc;
-    }
+  for (int idx = tid; idx < GP * D; idx += 256) {
+    const int gq = idx / D, d = idx % D;
+    out_ws[idx] = red_o[gq][d] + red_o[GP + gq][d] + red_o[2 * GP + gq][d] + red_o[3 * GP + gq][d];
   }
   if (tid < GP) {
     const float mw = fmaxf(fmaxf(red_m[0][tid], red_m[1][tid]), fmaxf(red_m[2][tid], red_m[3][tid]));
@@ -311,6 +370,11 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecArgs a) {
     a.out[((int64_t)b * a.Hq + hk * a.G + gq) * D + d] = (__bf16)(acc / l);
   }
 }
+
+// Ring depth (pages in flight per wavefront).  head_dim 128: 2 x 8 KB per wavefront, 69 KB per
+// workgroup, two workgroups per CU.
+constexpr int kStages128 = 2;
+constexpr int kStages64 = 4;
 
 static int pick_chunk_pages(int pps) {
   // 32 pages = 512 tokens = 256 KB of K+V per workgroup at head_dim 128.
@@ -352,17 +416,24 @@ static int launch_common(DecArgs a, int D, hipStream_t stream, const char* who) 
   a.ws_m = ws + n_o;
   a.ws_l = ws + n_o + n_s;
   const dim3 grid(a.nch, a.Hkv, a.B), cgrid(a.Hkv, a.B);
-#define AXL_DEC(DD, GG)                                                                   \
-  do {                                                                                    \
-    hipLaunchKernelGGL((decode_split_kernel<DD, GG, PAGED>), grid, dim3(256), 0, stream, a); \
-    hipLaunchKernelGGL((decode_combine_kernel<DD, GG>), cgrid, dim3(256), 0, stream, a);  \
+#define AXL_DEC(DD, GG, NS)                                                                    \
+  do {                                                                                          \
+    using Tile = DecTile<DD, GG, NS>;                                                           \
+    auto kern = decode_split_kernel<DD, GG, PAGED, NS>;                                         \
+    err = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,    \
+                              Tile::LDS_BYTES);                                                 \
+    if (err == hipSuccess) {                                                                    \
+      hipLaunchKernelGGL(kern, grid, dim3(256), Tile::LDS_BYTES, stream, a);                    \
+      hipLaunchKernelGGL((decode_combine_kernel<DD, GG>), cgrid, dim3(256), 0, stream, a);      \
+    }                                                                                           \
   } while (0)
-  if (D == 128 && gp == 4) AXL_DEC(128, 4);
-  else if (D == 128) AXL_DEC(128, 8);
-  else if (gp == 4) AXL_DEC(64, 4);
-  else AXL_DEC(64, 8);
+  hipError_t err = hipSuccess;
+  if (D == 128 && gp == 4) AXL_DEC(128, 4, kStages128);
+  else if (D == 128) AXL_DEC(128, 8, kStages128);
+  else if (gp == 4) AXL_DEC(64, 4, kStages64);
+  else AXL_DEC(64, 8, kStages64);
 #undef AXL_DEC
-  hipError_t err = hipGetLastError();
+  if (err == hipSuccess) err = hipGetLastError();
   if (err != hipSuccess)
     return set_error(AXL_ERR_LAUNCH, "%s: launch failed: %s", who, hipGetErrorString(err));
   return AXL_OK;
