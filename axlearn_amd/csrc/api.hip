@@ -143,8 +143,8 @@ static int check_decode_common(const char* who, int batch, int hq, int hkv, int 
     return set_error(AXL_ERR_UNSUPPORTED, "%s: only bf16 is supported", who);
   if (d != 128 && d != 64)
     return set_error(AXL_ERR_UNSUPPORTED, "%s: head_dim %d (supported: 64, 128)", who, d);
-  if (hq / hkv > 8)
-    return set_error(AXL_ERR_UNSUPPORTED, "%s: more than 8 query heads per kv head", who);
+  if (hq / hkv > 16)
+    return set_error(AXL_ERR_UNSUPPORTED, "%s: more than 16 query heads per kv head", who);
   return AXL_OK;
 }
 

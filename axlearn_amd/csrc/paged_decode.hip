@@ -95,6 +95,17 @@ __device__ __forceinline__ int v_swizzle(int row) {
   return 2 * ((row >> 1) & 3);
 }
 
+// Sequences per launch: bounds the work-item tables each workgroup keeps in LDS.
+constexpr int kMaxBatch = 512;
+
+// Live chunk range [ch0, ch1) of a sequence of length `len`.
+__device__ __forceinline__ void live_chunks(const DecArgs& a, int len, int& ch0, int& ch1) {
+  const int npages = min((len + kPage - 1) / kPage, a.pps);
+  const int first_page = a.window >= 0 ? max(0, len - 1 - a.window) / kPage : 0;
+  ch0 = first_page / a.chunk_pages;
+  ch1 = max(ch0, (npages + a.chunk_pages - 1) / a.chunk_pages);
+}
+
 template <int D, int GP, int NST>
 struct DecTile {
   static constexpr int ROW_BYTES = D * 2;
@@ -103,7 +114,9 @@ struct DecTile {
   static constexpr int RING_BYTES = 4 * NST * STAGE_BYTES;
   static constexpr int RED_BYTES = 2 * 4 * 16 * 4;
   static constexpr int RED_BASE = RING_BYTES;
-  static constexpr int LDS_BYTES = RED_BASE + RED_BYTES;
+  static constexpr int PFX_BASE = RED_BASE + RED_BYTES;   // int[kMaxBatch + 4]: work-item prefix
+  static constexpr int LEN_BASE = PFX_BASE + (kMaxBatch + 4) * 4;  // int[kMaxBatch]: sequence lengths
+  static constexpr int LDS_BYTES = LEN_BASE + kMaxBatch * 4;
   static constexpr int RED_O_PITCH = D + 4;              // floats per (wave, head) row of the epilogue
   static_assert(4 * GP * RED_O_PITCH * 4 <= RING_BYTES, "epilogue staging must fit in the ring");
 };
@@ -132,16 +145,65 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
-  const int chunk = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
-  int len = a.lengths[b];
-  if (!PAGED) len = min(len, a.kv_len);
-  int npages = (len + kPage - 1) / kPage;
-  npages = min(npages, a.pps);
+  // ---- work items: one per live (sequence, chunk, kv head), kv head fastest.  Every workgroup
+  // builds the same exclusive prefix of live-chunk counts over the batch and then walks the item
+  // list with stride gridDim.x, so chunks past a sequence's length cost nothing.
+  int* pfx = (int*)(smem + Tile::PFX_BASE);
+  int* lens = (int*)(smem + Tile::LEN_BASE);
+  {
+    constexpr int PER = kMaxBatch / 256;  // consecutive sequences per thread
+    int cnt[PER], tsum = 0;
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+      const int bi = tid * PER + i;
+      int n = 0;
+      if (bi < a.B) {
+        int l = a.lengths[bi];
+        if (!PAGED) l = min(l, a.kv_len);
+        lens[bi] = l;
+        int c0, c1;
+        live_chunks(a, l, c0, c1);
+        n = c1 - c0;
+      }
+      cnt[i] = n;
+      tsum += n;
+    }
+    int incl = tsum;  // inclusive scan over the wavefront
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int up = __shfl_up(incl, d, 64);
+      if (lane >= d) incl += up;
+    }
+    int* wsum = (int*)(smem + Tile::RED_BASE);
+    if (lane == 63) wsum[wave] = incl;
+    __syncthreads();
+    int run = incl - tsum;
+    for (int w = 0; w < wave; w++) run += wsum[w];
+#pragma unroll
+    for (int i = 0; i < PER; i++) {
+      const int bi = tid * PER + i;
+      if (bi <= a.B) pfx[bi] = run;
+      run += cnt[i];
+    }
+    if (tid == 255) pfx[kMaxBatch] = run;
+    __syncthreads();
+  }
+  const int n_items = pfx[a.B] * a.Hkv;
+  for (int item = blockIdx.x; item < n_items; item += gridDim.x) {
+  const int hk = item % a.Hkv, u = item / a.Hkv;
+  int b = 0;
+  for (int hi = a.B; hi - b > 1;) {  // last b with pfx[b] <= u
+    const int mid = (b + hi) >> 1;
+    if (pfx[mid] <= u) b = mid; else hi = mid;
+  }
+  const int len = lens[b];
+  int ch0, ch1;
+  live_chunks(a, len, ch0, ch1);
+  const int chunk = ch0 + (u - pfx[b]);
   int first_page = 0;
   if (a.window >= 0) first_page = max(0, (len - 1 - a.window)) / kPage;
   const int c_begin = max(chunk * a.chunk_pages, first_page);
-  const int c_end = min((chunk + 1) * a.chunk_pages, npages);
-  if (c_begin >= c_end) return;  // nothing live in this chunk (uniform for the whole workgroup)
+  const int c_end = min((chunk + 1) * a.chunk_pages, min((len + kPage - 1) / kPage, a.pps));
   // This wavefront owns pages c_begin + wave + 4*it, it = 0 .. n_my-1.
   const int n_my = (c_end - c_begin - wave + 3) >> 2;
 
@@ -254,6 +316,10 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
     shortx4 vf[NB];
 #pragma unroll
     for (int nb = 0; nb < NB; nb++) vf[nb] = lds_read_tr16(vt + v_rd0 + ((nb * 32) ^ v_xor));
+    // The stage is free as soon as its fragments sit in registers: refill it right away so that
+    // the loads of page it+NST overlap the arithmetic of this one.
+    wait_lds_reads();
+    if (it + NST < n_my) issue(it + NST, st);
     // ---- scores: S^T[token][head]; this lane: head = lane%16, tokens 4kg + r
     floatx4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -301,10 +367,6 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
 #pragma unroll
     for (int nb = 0; nb < NB; nb++)
       o[nb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf[nb], pf.v, o[nb], 0, 0, 0);
-    // Every LDS read of this stage has returned (the MFMAs consumed them) before new data is
-    // directed at it.
-    wait_lds_reads();
-    if (it + NST < n_my) issue(it + NST, st);
     st = (st + 1 == NST) ? 0 : st + 1;
   }
 
@@ -341,33 +403,57 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
     a.ws_m[sidx] = mw;
     a.ws_l[sidx] = lw;
   }
+  __syncthreads();  // the ring (and red_m/red_l) are reused by the next item
+  }  // item loop
 }
 
 // Merges the per-chunk partials of one (sequence, kv head): the "final round of flash"
 // (gpu_paged_attention.py:287-296, gpu_decoding.py:277-283).
+constexpr int kMaxChunks = 256;  // per sequence; bounds the combine kernel's LDS tables
+
 template <int D, int GP>
 __global__ __launch_bounds__(256) void decode_combine_kernel(const DecArgs a) {
+  __shared__ float sm[kMaxChunks * GP];   // chunk maxima, then rescale factors
+  __shared__ float sl[kMaxChunks * GP];   // chunk sums
+  __shared__ float s_max[GP], s_inv[GP];
   const int hk = blockIdx.x, b = blockIdx.y;
   const int tid = threadIdx.x;
-  const int len = a.lengths[b];
+  int len = a.lengths[b];
+  if (a.page_tables == nullptr) len = min(len, a.kv_len);
   int npages = min((len + kPage - 1) / kPage, a.pps);
   int first_page = 0;
   if (a.window >= 0) first_page = max(0, (len - 1 - a.window)) / kPage;
   const int ch0 = first_page / a.chunk_pages;
   const int ch1 = (npages + a.chunk_pages - 1) / a.chunk_pages;  // exclusive
+  const int n = max(ch1 - ch0, 0) * GP;
   const float c = a.scale * kLog2e;
-  const int64_t base = ((int64_t)b * a.Hkv + hk) * a.nch;
-  for (int idx = tid; idx < a.G * D; idx += 256) {
-    const int gq = idx / D, d = idx % D;
+  const int64_t base = ((int64_t)b * a.Hkv + hk) * a.nch + ch0;
+  for (int i = tid; i < n; i += 256) {
+    sm[i] = a.ws_m[base * GP + i];
+    sl[i] = a.ws_l[base * GP + i];
+  }
+  __syncthreads();
+  if (tid < GP) {
     float mw = kNegInf;
-    for (int ch = ch0; ch < ch1; ch++) mw = fmaxf(mw, a.ws_m[(base + ch) * GP + gq]);
-    float l = 0.f, acc = 0.f;
-    for (int ch = ch0; ch < ch1; ch++) {
-      const float f = fast_exp2((a.ws_m[(base + ch) * GP + gq] - mw) * c);
-      l += a.ws_l[(base + ch) * GP + gq] * f;
-      acc += a.ws_o[(base + ch) * (GP * D) + gq * D + d] * f;
-    }
-    a.out[((int64_t)b * a.Hq + hk * a.G + gq) * D + d] = (__bf16)(acc / l);
+    for (int i = tid; i < n; i += GP) mw = fmaxf(mw, sm[i]);
+    s_max[tid] = mw;
+  }
+  __syncthreads();
+  for (int i = tid; i < n; i += 256) sm[i] = fast_exp2((sm[i] - s_max[i % GP]) * c);
+  __syncthreads();
+  if (tid < GP) {
+    float l = 0.f;
+    for (int i = tid; i < n; i += GP) l += sl[i] * sm[i];
+    s_inv[tid] = 1.f / l;
+  }
+  __syncthreads();
+  const float* po = a.ws_o + base * (GP * D);
+  for (int idx = tid; idx < a.G * D; idx += 256) {
+    const int gq = idx / D;
+    float acc = 0.f;
+#pragma unroll 8
+    for (int i = 0; i < n; i += GP) acc += po[(int64_t)i * D + idx] * sm[i + gq];
+    a.out[((int64_t)b * a.Hq + hk * a.G) * D + idx] = (__bf16)(acc * s_inv[gq]);
   }
 }
 
@@ -380,6 +466,7 @@ static int pick_chunk_pages(int pps) {
   // 32 pages = 512 tokens = 256 KB of K+V per workgroup at head_dim 128.
   int cp = 32;
   if (pps < cp) cp = ((pps + 3) / 4) * 4;
+  if (pps > cp * kMaxChunks) cp = ((pps + kMaxChunks - 1) / kMaxChunks + 3) / 4 * 4;
   return cp < 4 ? 4 : cp;
 }
 
@@ -387,7 +474,7 @@ static size_t ws_bytes(int B, int Hkv, int nch, int gp, int D) {
   return (size_t)B * Hkv * nch * ((size_t)gp * D + 2 * gp) * sizeof(float);
 }
 
-static int gp_of(int G) { return G <= 4 ? 4 : 8; }
+static int gp_of(int G) { return G <= 4 ? 4 : (G <= 8 ? 8 : 16); }
 
 size_t paged_decode_workspace_bytes(const AxlPagedDecodeParams& p) {
   if (p.pages_per_seq <= 0 || p.num_kv_heads <= 0) return 0;
@@ -404,18 +491,35 @@ size_t decode_workspace_bytes(const AxlDecodeParams& p) {
   return ws_bytes(p.batch, p.num_kv_heads, nch, gp_of(p.num_q_heads / p.num_kv_heads), p.head_dim);
 }
 
+static int cu_count() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+      n = v;
+    else
+      n = 256;
+  }
+  return n;
+}
+
 template <bool PAGED>
 static int launch_common(DecArgs a, int D, hipStream_t stream, const char* who) {
   const int gp = gp_of(a.G);
-  if (a.G > 8) return set_error(AXL_ERR_UNSUPPORTED, "%s: more than 8 query heads per kv head", who);
+  if (a.G > 16) return set_error(AXL_ERR_UNSUPPORTED, "%s: more than 16 query heads per kv head", who);
   a.chunk_pages = pick_chunk_pages(a.pps);
+  if (a.chunk_pages > 256)
+    return set_error(AXL_ERR_UNSUPPORTED, "%s: context longer than %d tokens", who, 256 * kMaxChunks * kPage);
   a.nch = (a.pps + a.chunk_pages - 1) / a.chunk_pages;
   float* ws = a.ws_o;
   const size_t n_o = (size_t)a.B * a.Hkv * a.nch * gp * D;
   const size_t n_s = (size_t)a.B * a.Hkv * a.nch * gp;
   a.ws_m = ws + n_o;
   a.ws_l = ws + n_o + n_s;
-  const dim3 grid(a.nch, a.Hkv, a.B), cgrid(a.Hkv, a.B);
+  // Two workgroups fit a CU (LDS); the split kernel is persistent and strides over its work items.
+  const dim3 grid(2 * cu_count());
+  hipError_t err = hipSuccess;
 #define AXL_DEC(DD, GG, NS)                                                                    \
   do {                                                                                          \
     using Tile = DecTile<DD, GG, NS>;                                                           \
@@ -423,15 +527,30 @@ static int launch_common(DecArgs a, int D, hipStream_t stream, const char* who) 
     err = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,    \
                               Tile::LDS_BYTES);                                                 \
     if (err == hipSuccess) {                                                                    \
-      hipLaunchKernelGGL(kern, grid, dim3(256), Tile::LDS_BYTES, stream, a);                    \
-      hipLaunchKernelGGL((decode_combine_kernel<DD, GG>), cgrid, dim3(256), 0, stream, a);      \
+      hipLaunchKernelGGL(kern, grid, dim3(256), Tile::LDS_BYTES, stream, s);                    \
+      hipLaunchKernelGGL((decode_combine_kernel<DD, GG>), cgrid, dim3(256), 0, stream, s);      \
     }                                                                                           \
   } while (0)
-  hipError_t err = hipSuccess;
-  if (D == 128 && gp == 4) AXL_DEC(128, 4, kStages128);
-  else if (D == 128) AXL_DEC(128, 8, kStages128);
-  else if (gp == 4) AXL_DEC(64, 4, kStages64);
-  else AXL_DEC(64, 8, kStages64);
+  // The kernels keep per-sequence tables in LDS: larger batches go in slices of kMaxBatch.
+  for (int b0 = 0; b0 < a.B && err == hipSuccess; b0 += kMaxBatch) {
+    DecArgs s = a;
+    s.B = a.B - b0 < kMaxBatch ? a.B - b0 : kMaxBatch;
+    s.q = a.q + (size_t)b0 * a.Hq * D;
+    s.out = a.out + (size_t)b0 * a.Hq * D;
+    s.lengths = a.lengths + b0;
+    if (PAGED) s.page_tables = a.page_tables + (size_t)b0 * a.pps;
+    else { s.k = a.k + b0 * a.ks.b; s.v = a.v + b0 * a.vs.b; }
+    s.ws_o = a.ws_o + (size_t)b0 * a.Hkv * a.nch * gp * D;
+    s.ws_m = a.ws_m + (size_t)b0 * a.Hkv * a.nch * gp;
+    s.ws_l = a.ws_l + (size_t)b0 * a.Hkv * a.nch * gp;
+    const dim3 cgrid(a.Hkv, s.B);
+    if (D == 128 && gp == 4) AXL_DEC(128, 4, kStages128);
+    else if (D == 128 && gp == 8) AXL_DEC(128, 8, kStages128);
+    else if (D == 128) AXL_DEC(128, 16, kStages128);
+    else if (gp == 4) AXL_DEC(64, 4, kStages64);
+    else if (gp == 8) AXL_DEC(64, 8, kStages64);
+    else AXL_DEC(64, 16, kStages64);
+  }
 #undef AXL_DEC
   if (err == hipSuccess) err = hipGetLastError();
   if (err != hipSuccess)

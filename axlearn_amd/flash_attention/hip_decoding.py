@@ -51,8 +51,8 @@ def _common_checks(self, input_batch: Nested, heads_per_kv: int) -> bool:
         return self._log_unsupported(f"{query.dtype=} / {input_batch['key'].dtype=} (supported: bfloat16)")
     if query.shape[-1] not in (64, 128):
         return self._log_unsupported(f"head_dim {query.shape[-1]} (supported: 64, 128)")
-    if heads_per_kv > 8:
-        return self._log_unsupported(f"{heads_per_kv} query heads per kv head (supported: <= 8)")
+    if heads_per_kv > 16:
+        return self._log_unsupported(f"{heads_per_kv} query heads per kv head (supported: <= 16)")
     if not (self.cfg.softmax_scale > 0.0):
         return self._log_unsupported(f"{self.cfg.softmax_scale=} must be positive")
     mask, explicit_bias = split(input_batch["bias"], MaskFnAttentionBias)
