@@ -32,9 +32,10 @@ struct DecArgs {
   const int32_t* page_tables;  // [B, pps] (paged only)
   const int32_t* lengths;      // [B]
   __bf16* out;                 // [B, Hq, D]
-  float* ws_o;                 // [B, Hkv, NCH, GP, D]
-  float* ws_m;                 // [B, Hkv, NCH, GP]
-  float* ws_l;                 // [B, Hkv, NCH, GP]
+  float* ws_o;                 // [records, GP, D]; at most B * Hkv * NCH records
+  float* ws_m;                 // [records, GP]
+  float* ws_l;                 // [records, GP]
+  int32_t* ws_tab;             // [B, Hkv, NCH]: record that starts at this chunk, or -1
   Strides3 ks, vs;             // contiguous only
   int B, Hq, Hkv, G;
   int num_pages, pps;          // pool pages; logical pages per sequence (ceil(S/16) if contiguous)
@@ -42,6 +43,8 @@ struct DecArgs {
   int chunk_pages, nch;
   int window;
   float scale;
+  int* ticket;                 // [0] blocks handed out, [1] records written (zeroed by decode_plan_kernel)
+  int deterministic;           // fixed work decomposition: results reproducible bit for bit
 };
 
 constexpr int kPage = 16;
@@ -116,7 +119,8 @@ struct DecTile {
   static constexpr int RED_BASE = RING_BYTES;
   static constexpr int PFX_BASE = RED_BASE + RED_BYTES;   // int[kMaxBatch + 4]: work-item prefix
   static constexpr int LEN_BASE = PFX_BASE + (kMaxBatch + 4) * 4;  // int[kMaxBatch]: sequence lengths
-  static constexpr int LDS_BYTES = LEN_BASE + kMaxBatch * 4;
+  static constexpr int NEXT_BASE = LEN_BASE + kMaxBatch * 4;       // int[4]: next run, record index
+  static constexpr int LDS_BYTES = NEXT_BASE + 16;
   static constexpr int RED_O_PITCH = D + 4;              // floats per (wave, head) row of the epilogue
   static_assert(4 * GP * RED_O_PITCH * 4 <= RING_BYTES, "epilogue staging must fit in the ring");
 };
@@ -188,24 +192,48 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
     if (tid == 255) pfx[kMaxBatch] = run;
     __syncthreads();
   }
-  const int n_items = pfx[a.B] * a.Hkv;
-  for (int item = blockIdx.x; item < n_items; item += gridDim.x) {
-  const int hk = item % a.Hkv, u = item / a.Hkv;
+  // ---- work distribution.  The unit of work is a block of `chunk_pages` pages of one (sequence,
+  // kv head); blocks are numbered sequence-major, then kv head, then position.  A workgroup draws
+  // runs of consecutive blocks from a global counter - long runs while plenty of work is left,
+  // single blocks at the end (guided self-scheduling) - so that workgroups on CUs that get more
+  // of the memory system take more of the work.  The part of a run inside one (sequence, kv head)
+  // is a segment: one contiguous page range, streamed without a break, one partial record.
+  const int n_blocks = pfx[a.B] * a.Hkv;
+  const int n_wg = gridDim.x;
+  // The ids of at most 256 pages are kept in registers.  A fixed decomposition (one block per
+  // record, pages dealt round-robin) makes the result independent of timing.
+  const int max_run = a.deterministic ? 1 : max(1, 256 / a.chunk_pages);
+  const int run0 = min(max_run, max(1, n_blocks / (2 * n_wg)));
+  int* s_next = (int*)(smem + Tile::NEXT_BASE);
+  int* s_page = s_next + 3;  // next page of the segment to hand to a wavefront
+  if (tid == 0) *s_page = 4 * NST;
+  __syncthreads();
+  int run_e = blockIdx.x * run0;
+  int run_end = min(run_e + run0, n_blocks);
+  int handed = n_wg * run0;  // estimate of how many blocks have been handed out
+  while (run_e < n_blocks) {
+  bool first_segment = true;
+  int next_e = 0, next_n = 0;
+  while (run_e < run_end) {
   int b = 0;
-  for (int hi = a.B; hi - b > 1;) {  // last b with pfx[b] <= u
+  for (int hi = a.B; hi - b > 1;) {  // last b with Hkv * pfx[b] <= run_e
     const int mid = (b + hi) >> 1;
-    if (pfx[mid] <= u) b = mid; else hi = mid;
+    if (pfx[mid] * a.Hkv <= run_e) b = mid; else hi = mid;
   }
   const int len = lens[b];
   int ch0, ch1;
   live_chunks(a, len, ch0, ch1);
-  const int chunk = ch0 + (u - pfx[b]);
+  const int rem = run_e - pfx[b] * a.Hkv;
+  const int hk = rem / (ch1 - ch0), cl = rem % (ch1 - ch0);
+  const int seg = min(run_end - run_e, ch1 - ch0 - cl);
   int first_page = 0;
   if (a.window >= 0) first_page = max(0, (len - 1 - a.window)) / kPage;
-  const int c_begin = max(chunk * a.chunk_pages, first_page);
-  const int c_end = min((chunk + 1) * a.chunk_pages, min((len + kPage - 1) / kPage, a.pps));
-  // This wavefront owns pages c_begin + wave + 4*it, it = 0 .. n_my-1.
-  const int n_my = (c_end - c_begin - wave + 3) >> 2;
+  const int c_begin = max((ch0 + cl) * a.chunk_pages, first_page);
+  const int c_end = min((ch0 + cl + seg) * a.chunk_pages, min((len + kPage - 1) / kPage, a.pps));
+  // Pages of the segment are numbered 0 .. n_pg-1.  A wavefront starts with pages wave + 4*i,
+  // i < NST, and draws further ones from a counter in LDS whenever a ring stage frees up, so that
+  // the 4 wavefronts finish together however unevenly the memory system serves them.
+  const int n_pg = c_end - c_begin;
 
   // Q^T as MFMA B operand: lane (head column = lane%16, k-group = lane/16) holds d = 32s + 8kg .. +7.
   const int head = lane & 15, kg = lane >> 4;
@@ -219,9 +247,21 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
       for (int e = 0; e < 8; e++) qf[s][e] = (__bf16)0.f;
     }
   }
-  // Page ids of this wavefront's pages, one per lane (chunk_pages <= 256).
-  int my_pages = 0;
-  if (PAGED && lane < n_my) my_pages = a.page_tables[(int64_t)b * a.pps + c_begin + wave + 4 * lane];
+  // Page ids of the segment (at most 256): register r, lane l holds page 64r + l.
+  int seg_pages[4] = {0, 0, 0, 0};
+  if (PAGED) {
+#pragma unroll
+    for (int r = 0; r < 4; r++)
+      if (64 * r + lane < n_pg) seg_pages[r] = a.page_tables[(int64_t)b * a.pps + c_begin + 64 * r + lane];
+  }
+  auto page_id = [&](int idx) -> int {
+    int pg = __builtin_amdgcn_readlane(seg_pages[0], idx & 63);
+#pragma unroll
+    for (int r = 1; r < 4; r++)
+      if ((idx >> 6) == r) pg = __builtin_amdgcn_readlane(seg_pages[r], idx & 63);
+    if (pg < 0) pg += a.num_pages;  // negative indices count from the end, as in the reference's gather
+    return pg;
+  };
 
   const int vslice = lane % SL;       // load layout: 16-byte slice of the row
   const int vtok = lane / SL;         // load layout: token row within a load
@@ -259,14 +299,24 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
 
   // Everything the compiler tracks has landed before the first untracked load is issued.
   wait_all_vmem();
+  // Draw the next run and this segment's record slot now; the answers are only needed after the
+  // pages of this segment.
+  int rec = 0;
+  if (tid == 0) {
+    if (first_segment) {
+      next_n = min(max_run, max(1, (n_blocks - handed) / (4 * n_wg)));
+      next_e = n_wg * run0 + atomicAdd(&a.ticket[0], next_n);
+    }
+    rec = atomicAdd(&a.ticket[1], 1);
+  }
+  first_segment = false;
 
-  // Issues the 2*NLOAD loads of this wavefront's page `it` into ring stage `st`.
-  auto issue = [&](int it, int st) {
-    const int j = c_begin + wave + 4 * it;
+  // Issues the 2*NLOAD loads of page `idx` of the segment into ring stage `st`.
+  auto issue = [&](int idx, int st) {
+    const int j = c_begin + idx;
     const __bf16 *kb, *vb;
     if (PAGED) {
-      int pg = __builtin_amdgcn_readlane(my_pages, it);
-      if (pg < 0) pg += a.num_pages;  // negative indices count from the end, as in the reference's gather
+      int pg = page_id(idx);
       if ((unsigned)pg >= (unsigned)a.num_pages) pg = 0;  // reads as zeros: see `valid` below
       const int64_t off = ((int64_t)hk * a.num_pages + pg) * (kPage * D);
       kb = a.k + off;
@@ -289,25 +339,32 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
     }
   };
 
+  int ring_idx[NST];     // page held (or awaited) by each ring stage
+  int issued = 0;
 #pragma unroll
-  for (int st = 0; st < NST; st++)
-    if (st < n_my) issue(st, st);
-
+  for (int i = 0; i < NST; i++) {
+    ring_idx[i] = wave + 4 * i;
+    if (ring_idx[i] < n_pg) {
+      issue(ring_idx[i], i);
+      issued++;
+    }
+  }
+  bool exhausted = issued < NST;
   int st = 0;
-  for (int it = 0; it < n_my; it++) {
-    const int j = c_begin + wave + 4 * it;
-    // Wait for this page; up to NST-1 younger pages stay in flight.
-    const int younger = min(NST - 1, n_my - 1 - it);
+  for (int consumed = 0; consumed < issued; consumed++) {
+    int idx = ring_idx[0];
+#pragma unroll
+    for (int i = 1; i < NST; i++)
+      if (st == i) idx = ring_idx[i];
+    const int j = c_begin + idx;
+    // Wait for this page; the younger pages stay in flight.
+    const int younger = issued - consumed - 1;
     if (NST > 3 && younger == 3) wait_vmem_le<(NST > 3 ? 3 : 0) * LPP>();
     else if (NST > 2 && younger == 2) wait_vmem_le<(NST > 2 ? 2 : 0) * LPP>();
     else if (NST > 1 && younger == 1) wait_vmem_le<(NST > 1 ? 1 : 0) * LPP>();
     else wait_vmem_le<0>();
     bool valid = true;
-    if (PAGED) {
-      int pg = __builtin_amdgcn_readlane(my_pages, it);
-      if (pg < 0) pg += a.num_pages;
-      valid = (unsigned)pg < (unsigned)a.num_pages;
-    }
+    if (PAGED) valid = (unsigned)page_id(idx) < (unsigned)a.num_pages;
     const char* kt = ring + st * Tile::STAGE_BYTES;
     const char* vt = kt + Tile::TILE_BYTES;
     bf16x8 kf[KSTEPS];
@@ -319,7 +376,22 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
     // The stage is free as soon as its fragments sit in registers: refill it right away so that
     // the loads of page it+NST overlap the arithmetic of this one.
     wait_lds_reads();
-    if (it + NST < n_my) issue(it + NST, st);
+    if (!exhausted) {
+      int nxt = idx + 4 * NST;
+      if (!a.deterministic) {
+        if (lane == 0) nxt = atomicAdd(s_page, 1);
+        nxt = __builtin_amdgcn_readfirstlane(nxt);
+      }
+      if (nxt < n_pg) {
+        issue(nxt, st);
+#pragma unroll
+        for (int i = 0; i < NST; i++)
+          if (st == i) ring_idx[i] = nxt;
+        issued++;
+      } else {
+        exhausted = true;
+      }
+    }
     // ---- scores: S^T[token][head]; this lane: head = lane%16, tokens 4kg + r
     floatx4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -377,6 +449,7 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
     red_m[wave][head] = m_run;
     red_l[wave][head] = l_run;
   }
+  if (tid == 0) s_next[2] = rec;
   __syncthreads();  // also: every wavefront is done with its ring, which red_o aliases
   {
     const float mw = fmaxf(fmaxf(red_m[0][head], red_m[1][head]), fmaxf(red_m[2][head], red_m[3][head]));
@@ -389,7 +462,8 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
     }
   }
   __syncthreads();
-  float* out_ws = a.ws_o + (((int64_t)b * a.Hkv + hk) * a.nch + chunk) * (GP * D);
+  const int64_t slot = s_next[2];
+  float* out_ws = a.ws_o + slot * (GP * D);
   for (int idx = tid; idx < GP * D; idx += 256) {
     const int gq = idx / D, d = idx % D;
     out_ws[idx] = red_o[gq][d] + red_o[GP + gq][d] + red_o[2 * GP + gq][d] + red_o[3 * GP + gq][d];
@@ -399,12 +473,29 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
     float lw = 0.f;
 #pragma unroll
     for (int w = 0; w < 4; w++) lw += red_l[w][tid] * fast_exp2((red_m[w][tid] - mw) * c);
-    const int64_t sidx = (((int64_t)b * a.Hkv + hk) * a.nch + chunk) * GP + tid;
-    a.ws_m[sidx] = mw;
-    a.ws_l[sidx] = lw;
+    a.ws_m[slot * GP + tid] = mw;
+    a.ws_l[slot * GP + tid] = lw;
+    if (tid == 0) a.ws_tab[((int64_t)b * a.Hkv + hk) * a.nch + cl] = (int)slot;
   }
-  __syncthreads();  // the ring (and red_m/red_l) are reused by the next item
-  }  // item loop
+  if (tid == 0) *s_page = 4 * NST;
+  __syncthreads();  // the ring (and red_m/red_l) are reused by the next segment
+  run_e += seg;
+  }  // segments of the run
+  if (tid == 0) { s_next[0] = next_e; s_next[1] = next_n; }
+  __syncthreads();
+  run_e = s_next[0];
+  run_end = min(run_e + s_next[1], n_blocks);
+  handed = run_e + s_next[1];
+  __syncthreads();  // s_next is rewritten at the end of the next run
+  }  // runs
+}
+
+// Resets the work counters and the record table ahead of the split kernel (a kernel rather than
+// memsets so that the sequence can be captured into a graph).
+__global__ __launch_bounds__(256) void decode_plan_kernel(int* ticket, int32_t* tab, int n_tab) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < 2) ticket[i] = 0;
+  if (i < n_tab) tab[i] = -1;
 }
 
 // Merges the per-chunk partials of one (sequence, kv head): the "final round of flash"
@@ -413,24 +504,38 @@ constexpr int kMaxChunks = 256;  // per sequence; bounds the combine kernel's LD
 
 template <int D, int GP>
 __global__ __launch_bounds__(256) void decode_combine_kernel(const DecArgs a) {
-  __shared__ float sm[kMaxChunks * GP];   // chunk maxima, then rescale factors
-  __shared__ float sl[kMaxChunks * GP];   // chunk sums
+  __shared__ float sm[kMaxChunks * GP];   // record maxima, then rescale factors
+  __shared__ float sl[kMaxChunks * GP];   // record sums
+  __shared__ int s_list[kMaxChunks];      // records of this (sequence, kv head), in chunk order
+  __shared__ int s_count;
   __shared__ float s_max[GP], s_inv[GP];
   const int hk = blockIdx.x, b = blockIdx.y;
   const int tid = threadIdx.x;
   int len = a.lengths[b];
   if (a.page_tables == nullptr) len = min(len, a.kv_len);
-  int npages = min((len + kPage - 1) / kPage, a.pps);
-  int first_page = 0;
-  if (a.window >= 0) first_page = max(0, (len - 1 - a.window)) / kPage;
-  const int ch0 = first_page / a.chunk_pages;
-  const int ch1 = (npages + a.chunk_pages - 1) / a.chunk_pages;  // exclusive
-  const int n = max(ch1 - ch0, 0) * GP;
+  int ch0, ch1;
+  live_chunks(a, len, ch0, ch1);
+  const int nc = ch1 - ch0;               // live chunks = upper bound on records of this (b, hk)
   const float c = a.scale * kLog2e;
-  const int64_t base = ((int64_t)b * a.Hkv + hk) * a.nch + ch0;
+  if (tid < 64) {  // compact the record table row
+    const int32_t* row = a.ws_tab + ((int64_t)b * a.Hkv + hk) * a.nch;
+    int count = 0;
+    for (int base = 0; base < nc; base += 64) {
+      const int i = base + tid;
+      const int r = i < nc ? row[i] : -1;
+      const unsigned long long mask = __builtin_amdgcn_ballot_w64(r >= 0);
+      if (r >= 0) s_list[count + __builtin_popcountll(mask & ((1ull << tid) - 1))] = r;
+      count += __builtin_popcountll(mask);
+    }
+    if (tid == 0) s_count = count;
+  }
+  __syncthreads();
+  const int nl = s_count;
+  const int n = nl * GP;
   for (int i = tid; i < n; i += 256) {
-    sm[i] = a.ws_m[base * GP + i];
-    sl[i] = a.ws_l[base * GP + i];
+    const int64_t r = s_list[i / GP];
+    sm[i] = a.ws_m[r * GP + i % GP];
+    sl[i] = a.ws_l[r * GP + i % GP];
   }
   __syncthreads();
   if (tid < GP) {
@@ -447,12 +552,11 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecArgs a) {
     s_inv[tid] = 1.f / l;
   }
   __syncthreads();
-  const float* po = a.ws_o + base * (GP * D);
   for (int idx = tid; idx < a.G * D; idx += 256) {
     const int gq = idx / D;
     float acc = 0.f;
 #pragma unroll 8
-    for (int i = 0; i < n; i += GP) acc += po[(int64_t)i * D + idx] * sm[i + gq];
+    for (int ci = 0; ci < nl; ci++) acc += a.ws_o[(int64_t)s_list[ci] * (GP * D) + idx] * sm[ci * GP + gq];
     a.out[((int64_t)b * a.Hq + hk * a.G) * D + idx] = (__bf16)(acc * s_inv[gq]);
   }
 }
@@ -471,7 +575,7 @@ static int pick_chunk_pages(int pps) {
 }
 
 static size_t ws_bytes(int B, int Hkv, int nch, int gp, int D) {
-  return (size_t)B * Hkv * nch * ((size_t)gp * D + 2 * gp) * sizeof(float);
+  return (size_t)B * Hkv * nch * ((size_t)gp * D + 2 * gp + 1) * sizeof(float) + 256;  // + headers, counters
 }
 
 static int gp_of(int G) { return G <= 4 ? 4 : (G <= 8 ? 8 : 16); }
@@ -517,6 +621,13 @@ static int launch_common(DecArgs a, int D, hipStream_t stream, const char* who) 
   const size_t n_s = (size_t)a.B * a.Hkv * a.nch * gp;
   a.ws_m = ws + n_o;
   a.ws_l = ws + n_o + n_s;
+  const size_t n_r = (size_t)a.B * a.Hkv * a.nch;
+  a.ws_tab = (int32_t*)(ws + n_o + 2 * n_s);
+  {
+    const char* det = getenv("AXL_DECODE_DETERMINISTIC");
+    a.deterministic = det && det[0] != '\0' && det[0] != '0';
+  }
+  a.ticket = (int*)(ws + n_o + 2 * n_s + n_r);
   // Two workgroups fit a CU (LDS); the split kernel is persistent and strides over its work items.
   const dim3 grid(2 * cu_count());
   hipError_t err = hipSuccess;
@@ -527,6 +638,8 @@ static int launch_common(DecArgs a, int D, hipStream_t stream, const char* who) 
     err = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,    \
                               Tile::LDS_BYTES);                                                 \
     if (err == hipSuccess) {                                                                    \
+      hipLaunchKernelGGL(decode_plan_kernel, dim3((n_tab + 255) / 256), dim3(256), 0, stream,   \
+                         s.ticket, s.ws_tab, n_tab);                                            \
       hipLaunchKernelGGL(kern, grid, dim3(256), Tile::LDS_BYTES, stream, s);                    \
       hipLaunchKernelGGL((decode_combine_kernel<DD, GG>), cgrid, dim3(256), 0, stream, s);      \
     }                                                                                           \
@@ -543,6 +656,8 @@ static int launch_common(DecArgs a, int D, hipStream_t stream, const char* who) 
     s.ws_o = a.ws_o + (size_t)b0 * a.Hkv * a.nch * gp * D;
     s.ws_m = a.ws_m + (size_t)b0 * a.Hkv * a.nch * gp;
     s.ws_l = a.ws_l + (size_t)b0 * a.Hkv * a.nch * gp;
+    s.ws_tab = a.ws_tab + (size_t)b0 * a.Hkv * a.nch;
+    const int n_tab = s.B * a.Hkv * a.nch;
     const dim3 cgrid(a.Hkv, s.B);
     if (D == 128 && gp == 4) AXL_DEC(128, 4, kStages128);
     else if (D == 128 && gp == 8) AXL_DEC(128, 8, kStages128);
