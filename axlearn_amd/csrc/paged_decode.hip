@@ -5,18 +5,27 @@
 // gpu_decoding.py:71-283 (`_attn_forward_kernel`, `_decode_attn_unbatched`).
 //
 // The operation is bound by HBM: every K and V byte of the live context is read exactly once.
-//   * split-K over the context: a workgroup (4 wavefronts) owns `chunk_pages` consecutive logical
-//     pages (16 tokens each) of one (sequence, kv head); chunks past the sequence length exit at
-//     once, so long and short sequences load the chip evenly;
-//   * a wavefront streams one page at a time.  K is read straight into the B-operand layout of
-//     v_mfma_f32_16x16x32_bf16 (lane = token, 64-byte segments per row) and all query heads of the
-//     kv head (padded to 16 rows) are scored with D/32 MFMAs; V is read fully coalesced (16 lanes
-//     cover one 256-byte token row) and accumulated with fp32 FMAs, each 16-lane group keeping its
-//     own partial output for the tokens it owns; register sets are re-issued as soon as they are
-//     consumed so loads for the next page are in flight during the arithmetic of this one;
-//   * probabilities travel from the MFMA layout to the V layout through 1 KB of LDS per wavefront;
-//   * partial (o, m, l) per chunk go to an fp32 workspace (the reference stores partial o in the
-//     query dtype, gpu_paged_attention.py:272) and a second small kernel merges them.
+//   * split-K over the context in blocks of `chunk_pages` logical pages (16 tokens each) of one
+//     (sequence, kv head).  The split kernel is persistent (two workgroups of 4 wavefronts per CU):
+//     every workgroup derives the list of live blocks from the lengths and draws runs of
+//     consecutive blocks from a global counter, long runs first and single blocks at the end, so
+//     that blocks past a sequence's length cost nothing and CUs that are served faster by the
+//     memory system take more of the work;
+//   * K and V pages stream from HBM straight into a private LDS ring per wavefront
+//     (global_load_lds), so the bytes in flight cost no registers; a stage is refilled as soon as
+//     its fragments sit in registers.  The pages of a run are handed to the 4 wavefronts through a
+//     counter in LDS, so they finish together;
+//   * per page a wavefront computes S^T = K Q^T (v_mfma_f32_16x16x32_bf16) for all query heads of
+//     the kv head (padded to 16 columns) and O^T += V^T P^T (v_mfma_f32_16x16x16_bf16, V^T through
+//     transposing LDS reads); the accumulator layout of the first product is the operand layout
+//     of the second, so probabilities never leave registers;
+//   * each run inside one (sequence, kv head) yields one partial record (o, m, l) in an fp32
+//     workspace (the reference stores partial o in the query dtype, gpu_paged_attention.py:272)
+//     and a second small kernel merges the records of a (sequence, kv head) in context order.
+// Work is handed out by timing, so the grouping of the fp32 partial sums - not the set of keys -
+// can differ between two calls; AXL_DECODE_DETERMINISTIC=1 in the environment selects a fixed
+// decomposition (one block per record, pages dealt round-robin) whose result is reproducible bit
+// for bit.
 // Keys at index >= length are masked (gpu_paged_attention.py:100, gpu_decoding.py:109); the query
 // position is length-1, so a sliding window w also masks keys with (length-1) - j > w.  A page
 // index outside the pool reads as zeros and a negative one counts from the end of the pool, as the
@@ -48,21 +57,6 @@ struct DecArgs {
 };
 
 constexpr int kPage = 16;
-
-__device__ __forceinline__ float row16_max(float x) {
-  x = fmaxf(x, __shfl_xor(x, 1, 64));
-  x = fmaxf(x, __shfl_xor(x, 2, 64));
-  x = fmaxf(x, __shfl_xor(x, 4, 64));
-  x = fmaxf(x, __shfl_xor(x, 8, 64));
-  return x;
-}
-__device__ __forceinline__ float row16_sum(float x) {
-  x += __shfl_xor(x, 1, 64);
-  x += __shfl_xor(x, 2, 64);
-  x += __shfl_xor(x, 4, 64);
-  x += __shfl_xor(x, 8, 64);
-  return x;
-}
 
 // One 16-byte-per-lane direct global->LDS load: lane l's 16 bytes land at lds_base + 16*l.  Issued
 // through inline assembly so that the compiler neither tracks it nor waits for it; completion is
@@ -125,8 +119,7 @@ struct DecTile {
   static_assert(4 * GP * RED_O_PITCH * 4 <= RING_BYTES, "epilogue staging must fit in the ring");
 };
 
-// Work decomposition: grid (chunk, kv head, sequence); the 4 wavefronts of a workgroup take the
-// pages of the chunk round-robin.  Per page a wavefront computes
+// Split-K kernel.  Per page a wavefront computes
 //   S^T = K Q^T     (v_mfma_f32_16x16x32_bf16, A = K rows from LDS, B = Q^T held in registers),
 //   O^T += V^T P^T  (v_mfma_f32_16x16x16_bf16, A = V^T through transposing LDS reads, B = P^T),
 // in the "transposed" form where lane l owns query head l%16 and the tokens 4*(l/16)..+3 of the
@@ -149,9 +142,7 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
 
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
-  // ---- work items: one per live (sequence, chunk, kv head), kv head fastest.  Every workgroup
-  // builds the same exclusive prefix of live-chunk counts over the batch and then walks the item
-  // list with stride gridDim.x, so chunks past a sequence's length cost nothing.
+  // ---- every workgroup builds the same exclusive prefix of live-block counts over the batch.
   int* pfx = (int*)(smem + Tile::PFX_BASE);
   int* lens = (int*)(smem + Tile::LEN_BASE);
   {
@@ -235,6 +226,18 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
   // the 4 wavefronts finish together however unevenly the memory system serves them.
   const int n_pg = c_end - c_begin;
 
+  // Draw the next run and this segment's record slot; the round trips overlap the loads of Q and
+  // of the page ids below.
+  int rec = 0;
+  if (tid == 0) {
+    if (first_segment) {
+      next_n = min(max_run, max(1, (n_blocks - handed) / (4 * n_wg)));
+      next_e = atomicAdd(&a.ticket[0], next_n);
+    }
+    rec = atomicAdd(&a.ticket[1], 1);
+  }
+  first_segment = false;
+
   // Q^T as MFMA B operand: lane (head column = lane%16, k-group = lane/16) holds d = 32s + 8kg .. +7.
   const int head = lane & 15, kg = lane >> 4;
   bf16x8 qf[KSTEPS];
@@ -299,17 +302,6 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
 
   // Everything the compiler tracks has landed before the first untracked load is issued.
   wait_all_vmem();
-  // Draw the next run and this segment's record slot now; the answers are only needed after the
-  // pages of this segment.
-  int rec = 0;
-  if (tid == 0) {
-    if (first_segment) {
-      next_n = min(max_run, max(1, (n_blocks - handed) / (4 * n_wg)));
-      next_e = n_wg * run0 + atomicAdd(&a.ticket[0], next_n);
-    }
-    rec = atomicAdd(&a.ticket[1], 1);
-  }
-  first_segment = false;
 
   // Issues the 2*NLOAD loads of page `idx` of the segment into ring stage `st`.
   auto issue = [&](int idx, int st) {
@@ -481,7 +473,7 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
   __syncthreads();  // the ring (and red_m/red_l) are reused by the next segment
   run_e += seg;
   }  // segments of the run
-  if (tid == 0) { s_next[0] = next_e; s_next[1] = next_n; }
+  if (tid == 0) { s_next[0] = n_wg * run0 + next_e; s_next[1] = next_n; }
   __syncthreads();
   run_e = s_next[0];
   run_end = min(run_e + s_next[1], n_blocks);

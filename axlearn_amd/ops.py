@@ -187,6 +187,18 @@ def paged_decode(
     return out
 
 
+def paged_decode_workspace_bytes(batch: int, num_q_heads: int, num_kv_heads: int, head_dim: int,
+                                 pages_per_seq: int, page_size: int = 16) -> int:
+    """Bytes of device workspace `paged_decode` needs for these shapes (bf16)."""
+    lib = _lib.load()
+    p = AxlPagedDecodeParams(
+        batch=batch, num_q_heads=num_q_heads, num_kv_heads=num_kv_heads, head_dim=head_dim,
+        num_pages=batch * pages_per_seq, page_size=page_size, pages_per_seq=pages_per_seq,
+        dtype=_lib.dtype_code(torch.bfloat16), sliding_window=-1, softmax_scale=1.0,
+    )
+    return int(lib.axl_paged_decode_workspace_bytes(ctypes.byref(p)))
+
+
 def decode(
     q: torch.Tensor,
     k: torch.Tensor,

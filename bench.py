@@ -206,7 +206,7 @@ def bench_paged_decode(steps, warmup, cpu_baseline):
     tables_cpu = torch.from_numpy(np.random.default_rng(6).permutation(P).astype(np.int32)).reshape(B, pps)
     lengths, tables = lengths_cpu.to(dev), tables_cpu.to(dev)
     out = torch.empty((B, Hq, D), device=dev, dtype=bf)
-    ws = torch.empty((96 << 20,), device=dev, dtype=torch.uint8)
+    ws = torch.empty((ops.paged_decode_workspace_bytes(B, Hq, Hkv, D, pps),), device=dev, dtype=torch.uint8)
     scale = D ** -0.5
     fn = lambda: ops.paged_decode(q, kp, vp, tables, lengths, softmax_scale=scale, workspace=ws, out=out)
     ms = _time_region(fn, steps, warmup)

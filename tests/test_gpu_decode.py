@@ -230,3 +230,16 @@ def test_baseline_c4_full_size():
     with _deterministic():
         det2 = ops.paged_decode(q, kp2, vp2, tables2.to(dev), lengths.to(dev), softmax_scale=scale)
     assert torch.equal(det, det2)
+
+
+def test_wide_groups_and_batch_slices():
+    """16 query heads per kv head, and a batch larger than one launch's share (512 sequences)."""
+    for (b, hq, hkv, d, pps) in [(3, 32, 2, 128, 12), (2, 16, 1, 64, 9), (700, 4, 2, 64, 3)]:
+        q, kp, vp, tables, lengths = ref.paged_inputs(31, batch=b, num_heads=hq, num_kv_heads=hkv, head_dim=d,
+                                                      page_size=16, pages_per_seq=pps, min_len=1, max_len=16 * pps)
+        want = ref.reference_decode(q, kp, vp, lengths, softmax_scale=0.11, page_tables=tables)[:, 0]
+        got = ops.paged_decode(q[:, 0].cuda(), kp.cuda(), vp.cuda(), tables.cuda(), lengths.cuda(), softmax_scale=0.11)
+        assert _ok(got.cpu(), want), (b, hq, hkv, d, ref.max_abs(got.cpu(), want))
+        kk, vv = ref.reconstruct_kv(tables, kp), ref.reconstruct_kv(tables, vp)
+        got2 = ops.decode(q[:, 0].cuda(), kk.cuda(), vv.cuda(), lengths.cuda(), softmax_scale=0.11)
+        assert _ok(got2.cpu(), want), (b, hq, hkv, d)
