@@ -32,6 +32,11 @@ sys.path.insert(0, ROOT)
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0           # MI355X HBM3E
 
+# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, in KiB; the
+# factors are what the same counters read for a plain 1 GiB copy kernel, `--calibrate-copy`).
+DKDV_TRAFFIC_BYTES = {"c2": 3.21e9}      # flash_bwd_dkdv_bf16_kernel<128>, workload c2
+DECODE_SPLIT_TRAFFIC_BYTES = 4.25e9      # decode_split_kernel<128,4>, workload c4
+
 METRIC = "flash-attn fwd+bwd TFLOP/s; paged-decode HBM GB/s (% roofline), 1 MI355X"
 
 
@@ -56,13 +61,13 @@ def _time_region(fn, steps, warmup):
 
 def _flash_workload(name):
     if name == "c2":
-        return dict(label="C2: causal GQA flash fwd+bwd, bf16, B4 Hq32/Hkv8 T4096 D128",
+        return dict(name="c2", label="C2: causal GQA flash fwd+bwd, bf16, B4 Hq32/Hkv8 T4096 D128",
                     B=4, T=4096, Hq=32, Hkv=8, D=128, mask="causal", window=0, seg=False)
     if name == "c3":
-        return dict(label="C3: sliding-window(4096) causal MHA + segment ids fwd+bwd, bf16, B8 H16 T8192 D128",
+        return dict(name="c3", label="C3: sliding-window(4096) causal MHA + segment ids fwd+bwd, bf16, B8 H16 T8192 D128",
                     B=8, T=8192, Hq=16, Hkv=16, D=128, mask="sliding", window=4096, seg=True)
     if name == "c5":
-        return dict(label="C5: long-context causal GQA fwd+bwd, bf16, B1 Hq64/Hkv8 T32768 D128",
+        return dict(name="c5", label="C5: long-context causal GQA fwd+bwd, bf16, B1 Hq64/Hkv8 T32768 D128",
                     B=1, T=32768, Hq=64, Hkv=8, D=128, mask="causal", window=0, seg=False)
     raise ValueError(name)
 
@@ -143,7 +148,7 @@ def bench_flash(cfg, steps, warmup, cpu_baseline):
         roofline=dict(
             kernel="flash_bwd_dkdv_bf16_kernel", bound="mfma", achieved=tf(fl_dkdv, ms_dkdv),
             peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s", frac=tf(fl_dkdv, ms_dkdv) / MFMA_BF16_PEAK_TFLOPS,
-            traffic=None,
+            traffic=DKDV_TRAFFIC_BYTES.get(cfg["name"]),
         ),
         step_frac_of_mfma_peak=tf(fl_fwd + fl_bwd, ms_step) / MFMA_BF16_PEAK_TFLOPS,
     )
@@ -176,7 +181,7 @@ def cpu_baseline_flash(cfg):
         ref.reference_mha_grads(q, k, v, do, spec, softmax_scale=D ** -0.5, row_block=512, dtype=torch.float32)
         reps += 1
         dt = time.perf_counter() - t0
-        if dt > 10.0 or reps >= 8:
+        if dt > 12.0 or reps >= 64:
             break
     pairs = ref.count_unmasked_pairs(spec, 1, t_cap, t_cap) if cfg["seg"] else t_cap * t_cap / 2.0
     flops = 7.0 * 2.0 * (nkv * G) * pairs * D  # fwd (2 GEMMs) + bwd (5 GEMMs), algorithmic
@@ -218,12 +223,12 @@ def bench_paged_decode(steps, warmup, cpu_baseline):
         workload="C4: paged decode, bf16, B64 Hq32/Hkv8 D128, page 16, ctx U[512,32768]",
         value=gbs, unit="GB/s", ms_per_step=ms, algorithmic_gb=algo_bytes / 1e9,
         roofline=dict(kernel="decode_split_kernel", bound="hbm", achieved=gbs, peak=HBM_PEAK_GBS, unit="GB/s",
-                      frac=gbs / HBM_PEAK_GBS, traffic=None),
+                      frac=gbs / HBM_PEAK_GBS, traffic=DECODE_SPLIT_TRAFFIC_BYTES),
     )
     if cpu_baseline:
         from oracle import ref_attention as ref
 
-        nb = 2  # sequences timed on the CPU
+        nb = 32  # sequences timed on the CPU
         cores = min(os.cpu_count() or 1, 16)
         torch.set_num_threads(cores)
         kc, vc = kp.cpu(), vp.cpu()
@@ -248,6 +253,8 @@ def main():
     ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4", "c5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true", help="skip the paged-decode half of the metric")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy (known traffic) for scaling rocprofv3 byte counters")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU only (no collectives, no sharding); use --gpus 1.")
@@ -256,6 +263,14 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible; the HIP kernels have no CPU path.")
     cpu_base = not args.no_cpu_baseline
+    if args.calibrate_copy:
+        # A plain elementwise copy kernel that reads exactly 1 GiB and writes exactly 1 GiB.
+        src = torch.ones((1 << 28,), device="cuda:0", dtype=torch.float32)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.add(src, 0.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
 
     line = dict(metric=METRIC, n_gpus=1, steps=args.steps, warmup=args.warmup, higher_is_better=True,
                 scaling="weak", vs_baseline=None, dtype="bf16", data="synthetic")

@@ -138,7 +138,13 @@ int axl_flash_bwd_phases(const AxlFlashBwdParams* params, int phases, void* stre
  *   index in [-num_pages, 0) counts from the end of the pool and any other index outside
  *   [0, num_pages) reads as zeros.  out [B,Hq,D] in the dtype of q.
  *   sliding_window < 0 disables the window; otherwise keys with (len-1) - j > w are masked too.
- *   workspace: axl_paged_decode_workspace_bytes(params) bytes (fp32 split-K partials).
+ *   workspace: axl_paged_decode_workspace_bytes(params) bytes (fp32 split-K partial records, a
+ *   record table and two work counters; its contents need not be initialised or preserved).
+ *   Up to 16 query heads per kv head; head_dim 64 or 128; page_size 16; bf16.
+ *   Work is handed to workgroups by timing, so two calls on the same inputs may group the fp32
+ *   partial sums differently (differences far below bf16 resolution before the final rounding).
+ *   With AXL_DECODE_DETERMINISTIC=1 in the environment the decomposition is fixed and the result
+ *   is reproducible bit for bit, at a few percent of bandwidth.  The same holds for axl_decode.
  */
 typedef struct AxlPagedDecodeParams {
   const void* q;
