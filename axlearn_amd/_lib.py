@@ -93,6 +93,19 @@ class AxlDecodeParams(ctypes.Structure):
     ]
 
 
+class AxlPageInsertParams(ctypes.Structure):
+    _fields_ = [
+        ("k_pages", ctypes.c_void_p), ("v_pages", ctypes.c_void_p),
+        ("k_proj", ctypes.c_void_p), ("v_proj", ctypes.c_void_p),
+        ("page_indices", ctypes.c_void_p), ("key_positions", ctypes.c_void_p),
+        ("k_proj_batch_stride", ctypes.c_int64), ("k_proj_head_stride", ctypes.c_int64),
+        ("v_proj_batch_stride", ctypes.c_int64), ("v_proj_head_stride", ctypes.c_int64),
+        ("batch", ctypes.c_int32), ("num_kv_heads", ctypes.c_int32), ("head_dim", ctypes.c_int32),
+        ("num_pages", ctypes.c_int32), ("page_size", ctypes.c_int32), ("pages_per_seq", ctypes.c_int32),
+        ("dtype", ctypes.c_int32), ("broadcast_positions", ctypes.c_int32),
+    ]
+
+
 EXPORTED_SYMBOLS = (
     "axl_flash_fwd",
     "axl_flash_bwd",
@@ -102,6 +115,7 @@ EXPORTED_SYMBOLS = (
     "axl_paged_decode_workspace_bytes",
     "axl_decode",
     "axl_decode_workspace_bytes",
+    "axl_paged_kv_insert",
     "axl_last_error",
     "axl_abi_version",
 )
@@ -127,6 +141,7 @@ def load() -> ctypes.CDLL:
         ("axl_flash_bwd", AxlFlashBwdParams),
         ("axl_paged_decode", AxlPagedDecodeParams),
         ("axl_decode", AxlDecodeParams),
+        ("axl_paged_kv_insert", AxlPageInsertParams),
     ):
         fn = getattr(lib, name)
         fn.restype = ctypes.c_int

@@ -25,6 +25,7 @@ int launch_paged_decode(const AxlPagedDecodeParams& p, hipStream_t stream);
 size_t paged_decode_workspace_bytes(const AxlPagedDecodeParams& p);
 int launch_decode(const AxlDecodeParams& p, hipStream_t stream);
 size_t decode_workspace_bytes(const AxlDecodeParams& p);
+int launch_page_insert(const AxlPageInsertParams& p, hipStream_t stream);
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
@@ -69,6 +70,31 @@ static int check_flash_shapes(const char* who, int batch, int q_len, int kv_len,
 using namespace axl;
 
 extern "C" {
+
+int axl_paged_kv_insert(const AxlPageInsertParams* p, void* stream) {
+  using namespace axl;
+  const char* who = "axl_paged_kv_insert";
+  if (!p) return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: null params", who);
+  if (p->batch <= 0 || p->num_kv_heads <= 0 || p->head_dim <= 0 || p->num_pages <= 0 ||
+      p->page_size <= 0 || p->pages_per_seq <= 0)
+    return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: non-positive dimension", who);
+  if (p->dtype != AXL_BF16 && p->dtype != AXL_F32)
+    return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: unknown dtype %d", who, p->dtype);
+  if (!p->page_indices || !p->key_positions)
+    return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: null page_indices / key_positions", who);
+  if ((p->k_pages == nullptr) != (p->k_proj == nullptr) || (p->v_pages == nullptr) != (p->v_proj == nullptr))
+    return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: a pool and its projection go together", who);
+  if (!p->k_pages && !p->v_pages) return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: nothing to insert", who);
+  const int es = p->dtype == AXL_F32 ? 4 : 2;
+  const int64_t m = 16 / es;
+  if (p->head_dim % m != 0)
+    return set_error(AXL_ERR_UNSUPPORTED, "%s: head_dim %d is not a multiple of %d", who, p->head_dim, (int)m);
+  if (p->k_proj_batch_stride % m || p->k_proj_head_stride % m || p->v_proj_batch_stride % m ||
+      p->v_proj_head_stride % m || !aligned16(p->k_pages) || !aligned16(p->v_pages) ||
+      !aligned16(p->k_proj) || !aligned16(p->v_proj))
+    return set_error(AXL_ERR_UNSUPPORTED, "%s: rows must be 16-byte aligned", who);
+  return launch_page_insert(*p, (hipStream_t)stream);
+}
 
 const char* axl_last_error(void) { return g_last_error; }
 

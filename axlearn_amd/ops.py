@@ -21,6 +21,7 @@ from axlearn_amd._lib import (
     AxlFlashBwdParams,
     AxlFlashFwdParams,
     AxlPagedDecodeParams,
+    AxlPageInsertParams,
 )
 
 __all__ = [
@@ -231,3 +232,51 @@ def decode(
     p.workspace_bytes = ws.numel()
     _lib.check(lib.axl_decode(ctypes.byref(p), _lib.current_stream_ptr()))
     return out
+
+
+def paged_kv_insert(
+    k_pages: Optional[torch.Tensor],
+    v_pages: Optional[torch.Tensor],
+    k_proj: Optional[torch.Tensor],
+    v_proj: Optional[torch.Tensor],
+    page_indices: torch.Tensor,
+    key_positions: torch.Tensor,
+) -> None:
+    """Writes one new token per sequence into the pools, IN PLACE.
+
+    pools [Hkv,P,page,D]; k_proj/v_proj [B,Hkv,D] (any batch/head strides, dense in D);
+    page_indices [B,pps] int32; key_positions [B] int32, or [1] to use one position for all."""
+    pool = k_pages if k_pages is not None else v_pages
+    proj = k_proj if k_proj is not None else v_proj
+    if pool is None or proj is None:
+        raise AxlError(_lib.AXL_ERR_INVALID_ARGUMENT, "nothing to insert")
+    _require_cuda(pool, proj, page_indices, key_positions)
+    lib = _lib.load()
+    hkv, num_pages, page_size, d = pool.shape
+    b = page_indices.shape[0]
+    for name, x in (("k_pages", k_pages), ("v_pages", v_pages), ("page_indices", page_indices),
+                    ("key_positions", key_positions)):
+        if x is not None and not x.is_contiguous():
+            raise AxlError(_lib.AXL_ERR_UNSUPPORTED, f"{name} must be contiguous")
+    for name, x in (("k_proj", k_proj), ("v_proj", v_proj)):
+        if x is not None and (tuple(x.shape) != (b, hkv, d) or x.stride(-1) != 1 or x.dtype != pool.dtype):
+            raise AxlError(_lib.AXL_ERR_INVALID_ARGUMENT, f"{name} must be [B,Hkv,D] of the pool dtype, dense in D")
+    if page_indices.dtype != torch.int32 or key_positions.dtype != torch.int32:
+        raise AxlError(_lib.AXL_ERR_INVALID_ARGUMENT, "page_indices and key_positions must be int32")
+    if key_positions.numel() not in (1, b):
+        raise AxlError(_lib.AXL_ERR_INVALID_ARGUMENT, "key_positions must hold 1 or batch values")
+    p = AxlPageInsertParams(
+        k_pages=None if k_pages is None else k_pages.data_ptr(),
+        v_pages=None if v_pages is None else v_pages.data_ptr(),
+        k_proj=None if k_proj is None else k_proj.data_ptr(),
+        v_proj=None if v_proj is None else v_proj.data_ptr(),
+        page_indices=page_indices.data_ptr(), key_positions=key_positions.data_ptr(),
+        k_proj_batch_stride=0 if k_proj is None else k_proj.stride(0),
+        k_proj_head_stride=0 if k_proj is None else k_proj.stride(1),
+        v_proj_batch_stride=0 if v_proj is None else v_proj.stride(0),
+        v_proj_head_stride=0 if v_proj is None else v_proj.stride(1),
+        batch=b, num_kv_heads=hkv, head_dim=d, num_pages=num_pages, page_size=page_size,
+        pages_per_seq=page_indices.shape[1], dtype=_lib.dtype_code(pool.dtype),
+        broadcast_positions=int(key_positions.numel() == 1 and b > 1),
+    )
+    _lib.check(lib.axl_paged_kv_insert(ctypes.byref(p), _lib.current_stream_ptr()))

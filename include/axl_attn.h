@@ -191,6 +191,39 @@ typedef struct AxlDecodeParams {
 size_t axl_decode_workspace_bytes(const AxlDecodeParams* params);
 int axl_decode(const AxlDecodeParams* params, void* stream);
 
+/*
+ * Insertion of one new token per sequence into the paged KV pools, in place.
+ * Replaces: `gpu_scatter_update_pages_shmap_fn` / `_scatter_pages_kernel`
+ *   (axlearn/common/kv_cache/paged_kv_cache_gpu_kernel.py:16-60) as called for K and for V from
+ *   `PagedKVCache.extend_step` (axlearn/common/kv_cache/paged_kv_cache.py:213-240); both pools are
+ *   updated by one call (either pool/proj pair may be NULL).
+ *   k_pages, v_pages [Hkv, num_pages, page_size, D]; k_proj, v_proj: the new token's projections,
+ *   element (b, h, :) at  b * batch_stride + h * head_stride  (elements), which covers both the
+ *   layer's [B,1,Hkv,D] and the kernel's [Hkv,B,1,D] layouts; page_indices [B, pages_per_seq] int32;
+ *   key_positions [B] int32 (or one value for all sequences when broadcast_positions != 0).
+ *   For sequence b with pos = key_positions[b]: nothing is written unless
+ *   0 <= pos < page_size * pages_per_seq (:26); page = page_indices[b][pos / page_size]; the row
+ *   pages[h][page][pos % page_size][:] is overwritten for every h unless page == 0, the padding page
+ *   (:31, paged_kv_cache.py:120), or page lies outside the pool (dropped, paged_kv_cache.py:56-58).
+ *   Sequences must not share a live page (as in the reference: unique_indices).
+ */
+typedef struct AxlPageInsertParams {
+  void* k_pages;
+  void* v_pages;
+  const void* k_proj;
+  const void* v_proj;
+  const int32_t* page_indices;
+  const int32_t* key_positions;
+  int64_t k_proj_batch_stride, k_proj_head_stride;
+  int64_t v_proj_batch_stride, v_proj_head_stride;
+  int32_t batch, num_kv_heads, head_dim;
+  int32_t num_pages, page_size, pages_per_seq;
+  int32_t dtype;               /* AxlDtype of the pools and projections */
+  int32_t broadcast_positions; /* key_positions holds a single value */
+} AxlPageInsertParams;
+
+int axl_paged_kv_insert(const AxlPageInsertParams* params, void* stream);
+
 /* Message describing the calling thread's most recent failure ("" if none). Never NULL. */
 const char* axl_last_error(void);
 

@@ -18,6 +18,8 @@ Reference files restated here (paths relative to the apple/axlearn checkout):
   `:862-873` (`bool_to_bias`), `:876-882` (`_make_bool_segment_mask`).
 * `axlearn/common/kv_cache/paged_kv_cache.py:21-34` (`reconstruct_kv`): page gather, out-of-range
   page index reads as zeros.
+* `axlearn/common/kv_cache/paged_kv_cache_gpu_kernel.py:16-33` (`_scatter_pages_kernel`): insertion
+  of the new token into the pool.
 * `axlearn/common/flash_attention/gpu_decoding.py:314`, `gpu_paged_attention.py:344`:
   decode length = `target_positions[:, -1] + 1`.
 
@@ -32,6 +34,9 @@ Parity status of each function (what pins it, see tests/test_oracle.py):
 * gradients: pinned by float64 central finite differences and by the independent analytic
   brute force in oracle/brute_force.c.
 * `reconstruct_kv`: pinned by a pure-Python loop on tiny shapes.
+* `scatter_update_pages`: pinned by the element-wise loop the reference documents
+  (paged_kv_cache.py:156-165) written out in pure Python, plus the round trip through
+  `reconstruct_kv`; the padding-page and out-of-range rules are read from the kernel source.
 * XLA:CPU's exact bf16 rounding order inside einsum/softmax cannot be reproduced bit-for-bit without
   running jaxlib (absent here): "faithful" mode reproduces the rounding POINTS only.  parity unpinned
   at ULP level for the bf16 faithful mode; covered by the bf16 tolerance.
@@ -176,6 +181,31 @@ def reconstruct_kv(page_tables: torch.Tensor, pages: torch.Tensor) -> torch.Tens
     g = pages[:, safe]  # [n, b, pps, page_size, d]
     g = torch.where(oob[None, :, :, None, None], torch.zeros((), dtype=pages.dtype), g)
     return g.permute(1, 2, 3, 0, 4).reshape(b, pps * page_size, n, d)
+
+
+def scatter_update_pages(kv_pages: torch.Tensor, kv_proj: torch.Tensor, page_indices: torch.Tensor,
+                         key_positions: torch.Tensor) -> torch.Tensor:
+    """Insertion of one new token per sequence into a paged pool, as the reference's GPU kernel does it
+    (kv_cache/paged_kv_cache_gpu_kernel.py:16-33; the loop it stands for is spelled out in
+    kv_cache/paged_kv_cache.py:156-165).
+
+    kv_pages [H, P, page_size, D]; kv_proj [H, B, 1, D]; page_indices [B, pps]; key_positions [B, 1].
+    Returns an updated copy.  A position outside [0, page_size * pps) writes nothing (:26), page 0 (the
+    padding page) is never written (:31), a page index outside the pool is dropped
+    (paged_kv_cache.py:56-58, mode="drop").  A negative page index is undefined in the reference kernel;
+    it is dropped here (parity unpinned for that case)."""
+    out = kv_pages.clone()
+    h, total, page_size, _ = kv_pages.shape
+    b, pps = page_indices.shape
+    for bi in range(b):
+        pos = int(key_positions[bi if key_positions.shape[0] > 1 else 0, 0])
+        if not 0 <= pos < page_size * pps:
+            continue
+        page = int(page_indices[bi, pos // page_size])
+        if page <= 0 or page >= total:
+            continue
+        out[:, page, pos % page_size] = kv_proj[:, bi, 0].to(out.dtype)
+    return out
 
 
 # ----------------------------------------------------------------------------------------------

@@ -243,3 +243,48 @@ def test_wide_groups_and_batch_slices():
         kk, vv = ref.reconstruct_kv(tables, kp), ref.reconstruct_kv(tables, vp)
         got2 = ops.decode(q[:, 0].cuda(), kk.cuda(), vv.cuda(), lengths.cuda(), softmax_scale=0.11)
         assert _ok(got2.cpu(), want), (b, hq, hkv, d)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("page_size,d", [(16, 128), (8, 64), (32, 128)])
+def test_paged_kv_insert_bit_exact(dtype, page_size, d):
+    """Page insert against the oracle, bit for bit: live rows, padding page, positions and pages out of
+    range, one position broadcast over the batch; then paged decode sees the new token."""
+    from axlearn_amd import kv_cache as kvc
+
+    hkv, b, pps = 4, 9, 6
+    total = b * pps + 1
+    g = torch.Generator().manual_seed(5)
+    kp = torch.randn((hkv, total, page_size, d), generator=g).to(dtype)
+    vp = torch.randn((hkv, total, page_size, d), generator=g).to(dtype)
+    perm = torch.from_numpy(np.random.default_rng(3).permutation(total - 1).astype(np.int32) + 1)
+    tables = perm[: b * pps].reshape(b, pps).clone()
+    pos = torch.from_numpy(np.random.default_rng(4).integers(0, page_size * pps, size=(b, 1)).astype(np.int32))
+    tables[1, int(pos[1, 0]) // page_size] = 0            # padding page: never written
+    pos[2, 0] = page_size * pps                           # position past the table
+    pos[3, 0] = -3                                        # negative position
+    tables[4, int(pos[4, 0]) // page_size] = total + 5    # page outside the pool
+    k_new = torch.randn((b, 1, hkv, d), generator=g)
+    v_new = torch.randn((b, 1, hkv, d), generator=g)
+    want_k = ref.scatter_update_pages(kp, k_new.to(dtype).permute(2, 0, 1, 3), tables, pos)
+    want_v = ref.scatter_update_pages(vp, v_new.to(dtype).permute(2, 0, 1, 3), tables, pos)
+    kd, vd = kp.cuda(), vp.cuda()
+    kvc.paged_extend_step(kd, vd, tables.cuda(), k_proj=k_new.cuda(), v_proj=v_new.cuda(), key_positions=pos.cuda())
+    assert torch.equal(kd.cpu(), want_k) and torch.equal(vd.cpu(), want_v)
+    assert int((want_k != kp).any(dim=-1).sum()) == hkv * (b - 4)
+    # The reference's kernel-level entry point: one pool, projections laid out [heads, batch, 1, D].
+    kd2 = kp.cuda()
+    out = kvc.scatter_update_pages_kernel(kv_pages=kd2, kv_proj=k_new.to(dtype).permute(2, 0, 1, 3).contiguous().cuda(),
+                                          page_indices=tables.cuda(), key_positions=pos.cuda())
+    assert out is kd2 and torch.equal(kd2.cpu(), want_k)
+    # One position for the whole batch.
+    kd3 = kp.cuda()
+    one = torch.tensor([[page_size + 1]], dtype=torch.int32)
+    ops.paged_kv_insert(kd3, None, k_new[:, 0].to(dtype).cuda(), None, tables.cuda(), one.reshape(-1).cuda())
+    assert torch.equal(kd3.cpu(), ref.scatter_update_pages(kp, k_new.to(dtype).permute(2, 0, 1, 3), tables, one))
+    if dtype == torch.bfloat16 and page_size == 16:
+        lengths = (pos[:, 0] + 1).clamp(min=1, max=page_size * pps).to(torch.int32)
+        q = torch.randn((b, 1, hkv * 2, d), generator=g).to(dtype)
+        want = ref.reference_decode(q, want_k, want_v, lengths, softmax_scale=0.1, page_tables=tables)[:, 0]
+        got = ops.paged_decode(q[:, 0].cuda(), kd, vd, tables.cuda(), lengths.cuda(), softmax_scale=0.1)
+        assert _ok(got.cpu(), want)

@@ -229,6 +229,40 @@ def test_reconstruct_kv_loop():
                 assert torch.equal(got[bi, j, h], want)
 
 
+def test_scatter_update_pages_loop():
+    """The oracle's page insert against the element-wise loop documented in
+    kv_cache/paged_kv_cache.py:156-165, with the GPU kernel's guards (paged_kv_cache_gpu_kernel.py:26,31):
+    position out of range -> nothing; page 0 -> nothing; page outside the pool -> dropped."""
+    h, total, page, d, b, pps = 2, 7, 4, 3, 5, 3
+    pages = torch.arange(h * total * page * d, dtype=torch.float32).reshape(h, total, page, d)
+    proj = -1.0 - torch.arange(h * b * d, dtype=torch.float32).reshape(h, b, 1, d)
+    tables = torch.tensor([[5, 1, 2], [3, 0, 4], [6, 6, 6], [2, 9, 1], [4, 3, 5]], dtype=torch.int32)
+    pos = torch.tensor([[6], [5], [12], [4], [-1]], dtype=torch.int32)
+    # seq 0 -> page 1 row 2; seq 1 -> page 0 (padding, skipped); seq 2 -> pos 12 out of range;
+    # seq 3 -> page 9 outside the pool (dropped); seq 4 -> negative position.
+    got = ref.scatter_update_pages(pages, proj, tables, pos)
+    want = pages.clone()
+    for i in range(b):
+        p = int(pos[i, 0])
+        if p < 0 or p >= page * pps:
+            continue
+        actual = int(tables[i, p // page])
+        if actual == 0 or actual >= total:
+            continue
+        for kh in range(h):
+            for e in range(d):
+                want[kh, actual, p % page, e] = proj[kh, i, 0, e]
+    assert torch.equal(got, want)
+    assert int((got != pages).any(dim=-1).sum()) == h  # exactly one row per head changed
+    # Round trip: the inserted token shows up at its position in the gathered cache.
+    dense = ref.reconstruct_kv(tables, got)
+    assert torch.equal(dense[0, 6], proj[:, 0, 0])
+    # One position broadcast over the batch (paged_kv_cache.py:216-217).
+    tables2 = torch.tensor([[1, 2], [3, 4]], dtype=torch.int32)
+    got2 = ref.scatter_update_pages(pages, proj[:, :2], tables2, torch.tensor([[5]], dtype=torch.int32))
+    assert torch.equal(got2[:, 2, 1], proj[:, 0, 0]) and torch.equal(got2[:, 4, 1], proj[:, 1, 0])
+
+
 def test_paged_decode_equals_dense_and_brute():
     b, hq, hkv, d, page, pps = 3, 4, 2, 8, 4, 5
     q, k, v, tables, lengths = ref.paged_inputs(7, batch=b, num_heads=hq, num_kv_heads=hkv, head_dim=d,
