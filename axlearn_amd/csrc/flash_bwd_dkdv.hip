@@ -39,7 +39,7 @@ struct DkvTile {
   static constexpr int STAT_BASE = 2 * TILE_BYTES + 2 * TTILE_BYTES;
   static constexpr int STAT_BYTES = 3 * BQ * 4;  // lse | delta | segment id per query row
   static constexpr int BUF_BYTES = STAT_BASE + STAT_BYTES;
-  static constexpr int NBUF = 3;
+  static constexpr int NBUF = 4;
   static constexpr int CHUNKS = BQ * D * 2 / 16 / 256;  // 16-byte chunks per thread per tensor
   static constexpr int LDS_BYTES = NBUF * BUF_BYTES;
 };
@@ -51,8 +51,7 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
   constexpr int KK = D / 16, DT = D / 32;
   constexpr int NA = 2 * KK;          // stage-A MFMAs per tile
   constexpr int NB = 4 * DT;          // stage-B MFMAs per tile
-  constexpr int EPM = 16 / NA;        // stage-B elements handled per stage-A MFMA
-  static_assert(16 % NA == 0 && Tile::BQ == 32, "tiling");
+  static_assert(Tile::BQ == 32, "tiling");
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   const int tid = threadIdx.x;
@@ -162,146 +161,226 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
     s_src += adv_ ? (wrap_ ? (s_is_seg ? seg_wrap : s_wrap) : s_step) : 0;  \
   }
 
-  char* buf_b = smem;                         // tile j     (stage B)
-  char* buf_a = smem + Tile::BUF_BYTES;       // tile j + 1 (stage A)
-  char* buf_s = smem + 2 * Tile::BUF_BYTES;   // tile j + 2 (being filled)
+  char* buf_b = smem;                         // tile j     (stage B reads)
+  char* buf_e = smem + Tile::BUF_BYTES;       // tile j + 1 (next stage B; its statistics are in registers)
+  char* buf_a = smem + 2 * Tile::BUF_BYTES;   // tile j + 2 (stage A reads)
+  char* buf_s = smem + 3 * Tile::BUF_BYTES;   // tile j + 3 (being filled from the staging registers)
 
   const int a_row_off = swap_bits_2_3(l32) * Tile::STRIDE + g * 16;  // normal (row = query) reads
   const int j16 = lane & 15, half = (lane >> 4) & 1;
   const int tr_off =
       Tile::TR_BASE + (8 * g + (j16 >> 2)) * Tile::TSTRIDE + (16 * half + 4 * (j16 & 3)) * 2;
 
-  floatx16 s_cur, dp_cur;
+  // Three tiles are in flight: stage A (S = Q K^T, dP = dO V^T) of tile j+2, the elementwise stage
+  // (P = exp2(S c - lse), dS = P (dP - delta)) of tile j+1 and stage B (dV^T += dO^T P,
+  // dK^T += Q^T dS) of tile j; tile j+3 is written to LDS from the staging registers and tile j+4
+  // is requested from memory.  Everything that is not an MFMA - elementwise arithmetic, operand
+  // packing, LDS fragment reads, LDS tile writes, global loads, pointer updates - is dealt out over
+  // the MFMA slots of the iteration, so the matrix pipe never waits for it.
+  floatx16 s_e, dp_e;          // tile j + 1: logits / dP, then P / dS
+  union PackedOperand {
+    bf16x8 v[2];
+    bf16x2 p[8];
+  };
+  PackedOperand pb, dsb;       // tile j: P and dS as MFMA operands
 #pragma unroll
-  for (int r = 0; r < 16; r++) s_cur[r] = dp_cur[r] = 0.f;
-  int q0_b = t_begin * Tile::BQ, q0_a = q0_b;
+  for (int r = 0; r < 16; r++) s_e[r] = dp_e[r] = 0.f;
+
+  floatx4 lse_v[4], del_v[4];
+  intx4 seg_v[4];
+  int diff0 = 0;
+  // Row statistics of the tile in BUF_: register r of lane group g is query q0 + 16(r/8) + 8g + (r%8).
+#define AXL_READ_STATS_PART(BUF_, T8_, LSE_, DEL_, SEG_)                                \
+  {                                                                                     \
+    const char* st_ = (BUF_) + Tile::STAT_BASE + 8 * g * 4;                             \
+    LSE_[2 * (T8_)] = *(const floatx4*)(st_ + 64 * (T8_));                              \
+    LSE_[2 * (T8_) + 1] = *(const floatx4*)(st_ + 64 * (T8_) + 16);                     \
+    DEL_[2 * (T8_)] = *(const floatx4*)(st_ + Tile::BQ * 4 + 64 * (T8_));               \
+    DEL_[2 * (T8_) + 1] = *(const floatx4*)(st_ + Tile::BQ * 4 + 64 * (T8_) + 16);      \
+    if (HAS_SEG) {                                                                      \
+      SEG_[2 * (T8_)] = *(const intx4*)(st_ + 2 * Tile::BQ * 4 + 64 * (T8_));           \
+      SEG_[2 * (T8_) + 1] = *(const intx4*)(st_ + 2 * Tile::BQ * 4 + 64 * (T8_) + 16);  \
+    }                                                                                   \
+  }
+  // Elementwise stage of element R_ of (s_e, dp_e).
+#define AXL_ELEM(R_)                                                                           \
+  {                                                                                            \
+    const int r_ = (R_);                                                                       \
+    const unsigned diff_ = (unsigned)(diff0 + 16 * (r_ / 8) + (r_ % 8));                       \
+    float sv_ = diff_ <= limit ? s_e[r_] : kMasked;                                            \
+    if (HAS_SEG) sv_ = seg_v[r_ / 4][r_ % 4] == seg_k ? sv_ : kMasked;                         \
+    const float p_ = fast_exp2(__builtin_fmaf(sv_, c, lse_v[r_ / 4][r_ % 4])); /* lse_v = -lse*log2e */ \
+    s_e[r_] = p_;                                                                              \
+    dp_e[r_] = p_ * (dp_e[r_] - del_v[r_ / 4][r_ % 4]);                                        \
+  }
+#define AXL_PACK_PAIR(PB_, DSB_, I_)                                    \
+  {                                                                     \
+    PB_.p[I_] = pack_bf16(s_e[2 * (I_)], s_e[2 * (I_) + 1]);            \
+    DSB_.p[I_] = pack_bf16(dp_e[2 * (I_)], dp_e[2 * (I_) + 1]);         \
+  }
+  // Stage A of the tile in BUF_ into (S_, DP_), not interleaved with anything (pipeline fill).
+#define AXL_STAGE_A_PLAIN(BUF_, S_, DP_)                                                        \
+  _Pragma("unroll") for (int kk = 0; kk < KK; kk++) {                                           \
+    const bf16x8 qa_ = *(const bf16x8*)((BUF_) + a_row_off + kk * 32);                          \
+    const bf16x8 da_ = *(const bf16x8*)((BUF_) + Tile::TILE_BYTES + a_row_off + kk * 32);       \
+    S_ = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa_, kf[kk], S_, 0, 0, 0);                     \
+    DP_ = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da_, vf[kk], DP_, 0, 0, 0);                   \
+  }
+  union TrFrag {
+    bf16x8 v;
+    shortx4 hlf[2];
+  };
+#define AXL_B_READ_FROM(BUF_, DST_, N_)                                                          \
+  {                                                                                              \
+    const char* p_ = (BUF_) + (((N_) % 2) == 0 ? Tile::TTILE_BYTES : 0) +                        \
+                     16 * ((N_) / (2 * DT)) * Tile::TSTRIDE + tr_off + (((N_) % (2 * DT)) / 2) * 64; \
+    DST_.hlf[0] = lds_read_tr16(p_);                                                             \
+    DST_.hlf[1] = lds_read_tr16(p_ + 4 * Tile::TSTRIDE);                                         \
+  }
+
+  constexpr int NS = NA + NB;          // MFMAs per iteration: stage B of tile j, then stage A of tile j+2
+  constexpr int ESTEP = NS / 16;       // one of the 16 elements per lane every ESTEP slots
+  static_assert(NS % 16 == 0, "the 16 elements per lane are spread evenly over the MFMA slots");
+  constexpr int kAheadA = 6, kAheadB = 4;
+  constexpr int NWR = 4 * Tile::CHUNKS + 1;   // LDS writes of a tile per thread (two copies of Q and dO, statistics)
+  constexpr int NLD = 2 * Tile::CHUNKS + 1;   // global loads of a tile per thread
+  constexpr int LD_SLOT0 = NS - 2 - NLD;      // loads go in the last slots, writes in the first ones
+  static_assert(1 + NWR <= LD_SLOT0 - 1, "staging registers are written out before they are reloaded");
+  TrFrag bfr_next[kAheadB];            // first stage-B fragments of the next iteration
+  int q0_a = t_begin * Tile::BQ, q0_s = q0_a;  // first query of tiles j+2 and j+3
 
   if (total > 0) {
     AXL_LOAD_TILE()
     AXL_STORE_TILE(buf_b)
     AXL_ADVANCE()
+    const int q0_1 = (t_begin + pf_t) * Tile::BQ;
+    AXL_LOAD_TILE()
+    AXL_STORE_TILE(buf_e)
+    AXL_ADVANCE()
     q0_a = (t_begin + pf_t) * Tile::BQ;
     AXL_LOAD_TILE()
     AXL_STORE_TILE(buf_a)
-  }
-  wait_all_vmem();  // stationary fragments have landed: nothing issued before the loop is pending
-  __syncthreads();
-  if (total > 0) {
-    // Stage A of tile 0.
-#pragma unroll
-    for (int kk = 0; kk < KK; kk++) {
-      const bf16x8 qa = *(const bf16x8*)(buf_b + a_row_off + kk * 32);
-      const bf16x8 da = *(const bf16x8*)(buf_b + Tile::TILE_BYTES + a_row_off + kk * 32);
-      s_cur = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa, kf[kk], s_cur, 0, 0, 0);
-      dp_cur = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da, vf[kk], dp_cur, 0, 0, 0);
-    }
-  }
-
-  union TrFrag {
-    bf16x8 v;
-    shortx4 hlf[2];
-  };
-
-  for (int j = 0; j < total; j++) {
     AXL_ADVANCE()
-    const int q0_p = (t_begin + pf_t) * Tile::BQ;
-    AXL_LOAD_TILE()
-
-    // Row statistics of tile j: register r of lane group g is query q0_b + 16(r/8) + 8g + (r%8).
-    const char* st = buf_b + Tile::STAT_BASE + 8 * g * 4;
-    floatx4 lse_v[4], del_v[4];
-    intx4 seg_v[4];
+    q0_s = (t_begin + pf_t) * Tile::BQ;
+    AXL_LOAD_TILE()                      // tile 3 stays in the staging registers
+    wait_all_vmem();  // nothing issued before the loop is pending, stationary fragments included
+    __syncthreads();
+    // Pipeline fill: stage A and the elementwise stage of tile 0, stage A of tile 1.
+    AXL_STAGE_A_PLAIN(buf_b, s_e, dp_e)
+    AXL_READ_STATS_PART(buf_b, 0, lse_v, del_v, seg_v)
+    AXL_READ_STATS_PART(buf_b, 1, lse_v, del_v, seg_v)
+    diff0 = (t_begin * Tile::BQ + a.q_off + 8 * g) - kpos;
 #pragma unroll
-    for (int t8 = 0; t8 < 2; t8++) {
-      lse_v[2 * t8] = *(const floatx4*)(st + 64 * t8);
-      lse_v[2 * t8 + 1] = *(const floatx4*)(st + 64 * t8 + 16);
-      del_v[2 * t8] = *(const floatx4*)(st + Tile::BQ * 4 + 64 * t8);
-      del_v[2 * t8 + 1] = *(const floatx4*)(st + Tile::BQ * 4 + 64 * t8 + 16);
-      if (HAS_SEG) {
-        seg_v[2 * t8] = *(const intx4*)(st + 2 * Tile::BQ * 4 + 64 * t8);
-        seg_v[2 * t8 + 1] = *(const intx4*)(st + 2 * Tile::BQ * 4 + 64 * t8 + 16);
-      }
-    }
-    const int diff0 = (q0_b + a.q_off + 8 * g) - kpos;  // query of r == 0 minus this lane's key
-
-    // ---- stage A of tile j+1 interleaved with the elementwise part of stage B of tile j.
-    // Stage-A step n: even n -> S chain (Q fragment n/2), odd n -> dP chain (dO fragment n/2).
-    constexpr int kAheadA = 6;
-    bf16x8 afr[NA];
-#define AXL_A_READ(N_) \
-  afr[N_] = *(const bf16x8*)(buf_a + ((N_) % 2) * Tile::TILE_BYTES + a_row_off + ((N_) / 2) * 32);
+    for (int r = 0; r < 16; r++) AXL_ELEM(r)
 #pragma unroll
-    for (int n = 0; n < (kAheadA < NA ? kAheadA : NA); n++) AXL_A_READ(n)
-    floatx16 s_nxt, dp_nxt;
+    for (int i = 0; i < 8; i++) AXL_PACK_PAIR(pb, dsb, i)
 #pragma unroll
-    for (int r = 0; r < 16; r++) s_nxt[r] = dp_nxt[r] = 0.f;
-    __builtin_amdgcn_sched_barrier(0);
+    for (int r = 0; r < 16; r++) s_e[r] = dp_e[r] = 0.f;
+    AXL_STAGE_A_PLAIN(buf_e, s_e, dp_e)
+    AXL_READ_STATS_PART(buf_e, 0, lse_v, del_v, seg_v)
+    AXL_READ_STATS_PART(buf_e, 1, lse_v, del_v, seg_v)
+    diff0 = (q0_1 + a.q_off + 8 * g) - kpos;  // query of r == 0 minus this lane's key
 #pragma unroll
-    for (int n = 0; n < NA; n++) {
-      if (n + kAheadA < NA) AXL_A_READ(n + kAheadA)
-      if (n % 2 == 0)
-        s_nxt = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afr[n], kf[n / 2], s_nxt, 0, 0, 0);
-      else
-        dp_nxt = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afr[n], vf[n / 2], dp_nxt, 0, 0, 0);
-#pragma unroll
-      for (int e = 0; e < EPM; e++) {
-        const int r = n * EPM + e;
-        const unsigned diff = (unsigned)(diff0 + 16 * (r / 8) + (r % 8));
-        float sv = diff <= limit ? s_cur[r] : kMasked;
-        if (HAS_SEG) sv = seg_v[r / 4][r % 4] == seg_k ? sv : kMasked;
-        const float p = fast_exp2(__builtin_fmaf(sv, c, lse_v[r / 4][r % 4]));  // lse_v = -lse*log2e
-        s_cur[r] = p;
-        dp_cur[r] = p * (dp_cur[r] - del_v[r / 4][r % 4]);
-      }
-      __builtin_amdgcn_sched_barrier(0);
-    }
-#undef AXL_A_READ
-
-    // ---- stage B MFMAs of tile j: dV^T += dO^T P ; dK^T += Q^T dS  (scale applied at the end).
-    bf16x8 pb[2], dsb[2];
-#pragma unroll
-    for (int t8 = 0; t8 < 2; t8++) {
-      pb[t8] = pack_bf16x8(s_cur[8 * t8 + 0], s_cur[8 * t8 + 1], s_cur[8 * t8 + 2], s_cur[8 * t8 + 3],
-                           s_cur[8 * t8 + 4], s_cur[8 * t8 + 5], s_cur[8 * t8 + 6], s_cur[8 * t8 + 7]);
-      dsb[t8] = pack_bf16x8(dp_cur[8 * t8 + 0], dp_cur[8 * t8 + 1], dp_cur[8 * t8 + 2], dp_cur[8 * t8 + 3],
-                            dp_cur[8 * t8 + 4], dp_cur[8 * t8 + 5], dp_cur[8 * t8 + 6], dp_cur[8 * t8 + 7]);
-    }
-    // Step n = t8 * 2DT + dt * 2 + which; which 0: dV (dO^T fragment, P), 1: dK (Q^T fragment, dS).
-    constexpr int kAheadB = 4;
-    TrFrag bfr[NB];
-#define AXL_B_READ(N_)                                                                           \
-  {                                                                                              \
-    const char* p_ = buf_b + (((N_) % 2) == 0 ? Tile::TTILE_BYTES : 0) +                         \
-                     16 * ((N_) / (2 * DT)) * Tile::TSTRIDE + tr_off + (((N_) % (2 * DT)) / 2) * 64; \
-    bfr[N_].hlf[0] = lds_read_tr16(p_);                                                          \
-    bfr[N_].hlf[1] = lds_read_tr16(p_ + 4 * Tile::TSTRIDE);                                      \
+    for (int i = 0; i < kAheadB; i++) AXL_B_READ_FROM(buf_b, bfr_next[i], i)
   }
+
+  const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  for (int j = 0; j < total; j++) {
+    bf16x8 afr[NA];
+    TrFrag bfr[NB];
 #pragma unroll
-    for (int n = 0; n < kAheadB; n++) AXL_B_READ(n)
+    for (int i = 0; i < kAheadB; i++) bfr[i] = bfr_next[i];
+    floatx16 s_a, dp_a;
+    PackedOperand pb_n, dsb_n;           // tile j + 1, packed as its elements complete
+    floatx4 lse_n[4], del_n[4];          // statistics of tile j + 2
+    intx4 seg_n[4];
+    int q0_p = q0_s;
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int n = 0; n < NB; n++) {
-      if (n + kAheadB < NB) AXL_B_READ(n + kAheadB)
-      const int t8 = n / (2 * DT), dt = (n % (2 * DT)) / 2;
-      if (n % 2 == 0)
-        dv_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[n].v, pb[t8], dv_acc[dt], 0, 0, 0);
-      else
-        dk_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[n].v, dsb[t8], dk_acc[dt], 0, 0, 0);
+    for (int n = 0; n < NS; n++) {
+      // ---- LDS fragments requested ahead of their MFMA
+      if (n + kAheadB < NB) AXL_B_READ_FROM(buf_b, bfr[n + kAheadB], n + kAheadB)
+      if (n + kAheadA >= NB && n + kAheadA - NB < NA) {
+        const int x = n + kAheadA - NB;
+        afr[x] = *(const bf16x8*)(buf_a + (x % 2) * Tile::TILE_BYTES + a_row_off + (x / 2) * 32);
+      }
+      if (n >= NS - kAheadB) AXL_B_READ_FROM(buf_e, bfr_next[n - (NS - kAheadB)], n - (NS - kAheadB))
+      // ---- the MFMA of this slot.  Stage-B step m = t8 * 2DT + dt * 2 + which (which 0: dV with the
+      // dO^T fragment and P, 1: dK with the Q^T fragment and dS); stage-A step x: even -> S chain
+      // with Q fragment x/2, odd -> dP chain with dO fragment x/2.
+      if (n < NB) {
+        const int t8 = n / (2 * DT), dt = (n % (2 * DT)) / 2;
+        if (n % 2 == 0)
+          dv_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[n].v, pb.v[t8], dv_acc[dt], 0, 0, 0);
+        else
+          dk_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[n].v, dsb.v[t8], dk_acc[dt], 0, 0, 0);
+      } else {
+        const int x = n - NB;
+        if (x % 2 == 0)
+          s_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afr[x], kf[x / 2], x == 0 ? zero16 : s_a, 0, 0, 0);
+        else
+          dp_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afr[x], vf[x / 2], x == 1 ? zero16 : dp_a, 0, 0, 0);
+      }
+      // ---- elementwise stage of tile j+1, one element every ESTEP slots, packed pairwise
+      if (n % ESTEP == 0) AXL_ELEM(n / ESTEP)
+      if (n % (2 * ESTEP) == 2 * ESTEP - 1) AXL_PACK_PAIR(pb_n, dsb_n, n / (2 * ESTEP))
+      // ---- tile j+3: staging registers -> LDS (both copies of Q and dO, then the statistics)
+      if (n >= 1 && n < 1 + 4 * Tile::CHUNKS) {
+        const int w = n - 1, i = w / 4;
+        if (w % 4 == 0) *(u32x4*)(buf_s + st_lds + i * ROWS_PER_PASS * Tile::STRIDE) = qreg[i];
+        if (w % 4 == 1) *(u32x4*)(buf_s + Tile::TILE_BYTES + st_lds + i * ROWS_PER_PASS * Tile::STRIDE) = dreg[i];
+        if (w % 4 == 2) *(u32x4*)(buf_s + st_lds_t + i * ROWS_PER_PASS * Tile::TSTRIDE) = qreg[i];
+        if (w % 4 == 3) *(u32x4*)(buf_s + Tile::TTILE_BYTES + st_lds_t + i * ROWS_PER_PASS * Tile::TSTRIDE) = dreg[i];
+      }
+      if (n == 1 + 4 * Tile::CHUNKS) {
+        if (tid < 24) {
+          union { u32x4 u; floatx4 f; } w_;
+          w_.u = sreg;
+          if (st_kind == 0) w_.f = w_.f * (-kLog2e);
+          *(u32x4*)(buf_s + Tile::STAT_BASE + st_kind * (Tile::BQ * 4) + st_part * 16) = w_.u;
+        }
+      }
+      // ---- tile j+4: advance the cursor, then one global load per slot
+      if (n == LD_SLOT0 - 1) {
+        AXL_ADVANCE()
+        q0_p = (t_begin + pf_t) * Tile::BQ;
+      }
+      if (n >= LD_SLOT0 && n < LD_SLOT0 + 2 * Tile::CHUNKS) {
+        const int w = n - LD_SLOT0, i = w / 2;
+        if (w % 2 == 0) qreg[i] = *(const u32x4*)(q_src + (int64_t)(i * ROWS_PER_PASS) * a.qs.s);
+        else dreg[i] = *(const u32x4*)(d_src + (int64_t)(i * ROWS_PER_PASS) * a.dos.s);
+      }
+      if (n == LD_SLOT0 + 2 * Tile::CHUNKS) sreg = *(const u32x4*)s_src;
+      // ---- statistics of tile j+2 for the next iteration's elementwise stage
+      if (n == NS / 2) AXL_READ_STATS_PART(buf_a, 0, lse_n, del_n, seg_n)
+      if (n == NS / 2 + 1) AXL_READ_STATS_PART(buf_a, 1, lse_n, del_n, seg_n)
       __builtin_amdgcn_sched_barrier(0);
     }
-#undef AXL_B_READ
-
-    AXL_STORE_TILE(buf_s)
     __syncthreads();
     char* const tmp = buf_b;
-    buf_b = buf_a;
+    buf_b = buf_e;
+    buf_e = buf_a;
     buf_a = buf_s;
     buf_s = tmp;
-    s_cur = s_nxt;
-    dp_cur = dp_nxt;
-    q0_b = q0_a;
-    q0_a = q0_p;
+    s_e = s_a;
+    dp_e = dp_a;
+    pb = pb_n;
+    dsb = dsb_n;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      lse_v[i] = lse_n[i];
+      del_v[i] = del_n[i];
+      if (HAS_SEG) seg_v[i] = seg_n[i];
+    }
+    diff0 = (q0_a + a.q_off + 8 * g) - kpos;
+    q0_a = q0_s;
+    q0_s = q0_p;
   }
+#undef AXL_READ_STATS_PART
+#undef AXL_ELEM
+#undef AXL_PACK_PAIR
+#undef AXL_STAGE_A_PLAIN
+#undef AXL_B_READ_FROM
 #undef AXL_LOAD_TILE
 #undef AXL_STORE_TILE
 #undef AXL_ADVANCE
