@@ -78,6 +78,42 @@ __device__ __forceinline__ int swap_bits_2_3(int m) {
 // not make every iteration wait on the loads it has just issued for the NEXT tile.
 __device__ __forceinline__ void wait_all_vmem() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
+// Segment-id pruning of a workgroup's loop range.  `my_id` is the segment id of one of the rows the
+// workgroup owns (every owned row is passed by at least one thread); ids[lo, hi) are the segment ids
+// of the rows it loops over.  A looped row can only match an owned row if its id lies between the
+// smallest and the largest owned id, so [lo, hi) is shrunk to the hull of such rows (empty if there
+// is none).  Called by all 256 threads of the workgroup; contains barriers.
+__device__ __forceinline__ void shrink_to_segment_hull(int my_id, const int32_t* ids, int tid, int& lo, int& hi) {
+  __shared__ int s_rng[4];
+  if (tid == 0) {
+    s_rng[0] = 0x7fffffff;  // smallest owned id
+    s_rng[1] = -0x7fffffff - 1;  // largest owned id
+    s_rng[2] = 0x7fffffff;  // first candidate row
+    s_rng[3] = -1;          // last candidate row
+  }
+  __syncthreads();
+  atomicMin(&s_rng[0], my_id);
+  atomicMax(&s_rng[1], my_id);
+  __syncthreads();
+  const int id_min = s_rng[0], id_max = s_rng[1];
+  int first = 0x7fffffff, last = -1;
+  for (int r = lo + tid; r < hi; r += 256) {
+    const int id = ids[r];
+    if (id >= id_min && id <= id_max) {
+      first = min(first, r);
+      last = max(last, r);
+    }
+  }
+  if (last >= 0) {
+    atomicMin(&s_rng[2], first);
+    atomicMax(&s_rng[3], last);
+  }
+  __syncthreads();
+  lo = max(lo, s_rng[2] == 0x7fffffff ? hi : s_rng[2]);
+  hi = min(hi, s_rng[3] + 1);
+  if (hi < lo) hi = lo;
+}
+
 struct Strides3 {
   int64_t b, s, h;
 };

@@ -85,6 +85,7 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
     if (a.mask_kind == AXL_MASK_SLIDING_WINDOW)
       q_end = min(a.T, k0_wg + Tile::BKV - 1 + a.window - a.q_off + 1);
   }
+  if (HAS_SEG) shrink_to_segment_hull(seg_k, a.seg + (int64_t)b * a.T, tid, q_begin, q_end);
   const int t_begin = q_begin / Tile::BQ;
   const int nt = max(0, (q_end + Tile::BQ - 1) / Tile::BQ - t_begin);
   const int total = nt * G;  // tiles in processing order: query head (outer) x query tile (inner)

@@ -101,13 +101,14 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
     k_end = min(a.S, q0_wg + Tile::BQ + a.q_off);
     if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) k_begin = max(0, q0_wg + a.q_off - a.window);
   }
+  const int seg_q = a.seg ? a.seg[(int64_t)b * a.T + q0 + l32] : 0;
+  const int32_t* seg_k = a.seg ? a.seg + (int64_t)b * a.T : nullptr;
+  if (seg_k) shrink_to_segment_hull(seg_q, seg_k, tid, k_begin, k_end);
   const int t_begin = k_begin / Tile::BK;
   const int t_end = (k_end + Tile::BK - 1) / Tile::BK;
 
   const int qpos = q0 + l32 + a.q_off;       // this lane's query position
   const int qpos_min = q0 + a.q_off, qpos_max = q0 + 31 + a.q_off;  // of the wavefront
-  const int seg_q = a.seg ? a.seg[(int64_t)b * a.T + q0 + l32] : 0;
-  const int32_t* seg_k = a.seg ? a.seg + (int64_t)b * a.T : nullptr;
 
   floatx16 o[DT];
 #pragma unroll
