@@ -61,10 +61,16 @@ __device__ __forceinline__ shortx4 lds_read_tr16(const void* lds_addr) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4i16(AXL_LDS(shortx4, lds_addr));
 }
 
+// Exchange with lane ^ 32 through v_permlane32_swap (no LDS round trip): after the swap the two
+// results hold, between them, this lane's value and its partner's.
 __device__ __forceinline__ float xor32_max(float x) {
-  return fmaxf(x, __shfl_xor(x, 32, 64));
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
 }
-__device__ __forceinline__ float xor32_sum(float x) { return x + __shfl_xor(x, 32, 64); }
+__device__ __forceinline__ float xor32_sum(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
 
 // Row index permutation that swaps bits 2 and 3.  Feeding MFMA 32x32 A-operand lane m with tile
 // row pi(m) makes accumulator register r of lane group g hold tile row 16*(r/8) + 8*g + (r%8), so

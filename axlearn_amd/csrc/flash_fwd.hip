@@ -7,7 +7,10 @@
 //
 //   * one workgroup = 4 wavefronts = 128 query rows of one (batch, query head); each wavefront owns
 //     32 query rows and keeps their Q fragments in registers for the whole kernel;
-//   * K/V tiles of 64 keys are staged through LDS (double buffered) and shared by the 4 wavefronts;
+//   * K/V tiles of 64 keys are shared by the 4 wavefronts through LDS (double buffered); they arrive
+//     by direct global->LDS loads, unpadded and XOR-swizzled, so no registers stage them;
+//   * the S^T MFMAs of tile t+1 are interleaved with the exponentials of tile t, so the matrix pipe
+//     works through the softmax of the wavefront that feeds it;
 //   * the logits are produced TRANSPOSED, S^T = K Q^T, with v_mfma_f32_32x32x16_bf16: a lane then
 //     owns one query column and 16 keys per 32-key sub-tile, so the softmax row statistics are
 //     in-register reductions plus a single exchange with lane^32, and exp(S^T) is already in the
@@ -61,25 +64,51 @@ template <int D>
 struct FwdTile {
   static constexpr int BQ = 128;              // query rows per workgroup
   static constexpr int BK = 64;               // keys per LDS tile
-  static constexpr int KSTRIDE = D * 2 + 16;  // bytes per K row in LDS (16 B pad: b128 reads)
-  static constexpr int VSTRIDE = D * 2 + 64;  // bytes per V row in LDS (64 B pad: tr reads)
-  static constexpr int KBYTES = BK * KSTRIDE;
-  static constexpr int VBYTES = BK * VSTRIDE;
-  static constexpr int CHUNKS = BK * D * 2 / 16 / 256;  // 16-byte chunks per thread per tile
-  static constexpr int LDS_BYTES = 2 * (KBYTES + VBYTES);
+  static constexpr int ROWB = D * 2;          // bytes per K / V row in LDS: unpadded
+  static constexpr int TILE_BYTES = BK * ROWB;
+  static constexpr int NSEG = 4;              // ring of segment-id rows (a tile's ids outlive its K buffer)
+  static constexpr int SEG_BASE = 4 * TILE_BYTES;            // {K, V} x double buffer, then the ids
+  static constexpr int LDS_BYTES = SEG_BASE + NSEG * BK * 4;
+  static constexpr int DMA_PER_WAVE = TILE_BYTES / 1024 / 4;  // direct-to-LDS loads per wavefront per tile
+  // Tiles arrive by direct global->LDS loads, which write 1 KB of consecutive LDS per instruction, so
+  // rows cannot be padded; bank conflicts are avoided by storing the 16-byte chunk c of row R at
+  // chunk index c ^ swz(R) instead (each lane simply fetches the chunk that belongs at its slot).
+  // swz is a GF(2)-linear map of the row's low 4 bits found by exhaustive search with a bank
+  // simulator: conflict-free for the row-per-lane 128-bit reads of K (row order swap_bits_2_3(lane))
+  // and for the transposing 64-bit reads of V, under a 32-bank and a 64-bank model alike.
+  __device__ static __forceinline__ int swz(int row) {
+    return D == 128 ? (((row & 1) ? 4 : 0) ^ ((row & 2) ? 10 : 0) ^ ((row & 4) ? 1 : 0) ^ ((row & 8) ? 3 : 0))
+                    : (((row & 1) ? 2 : 0) ^ ((row & 2) ? 4 : 0) ^ ((row & 4) ? 1 : 0) ^ ((row & 8) ? 3 : 0));
+  }
 };
+
+// One 16-byte-per-lane direct global->LDS load: lane l's 16 bytes land at lds_base + 16*l.  Issued
+// through inline assembly so that the compiler neither tracks it nor waits for it; completion is
+// in issue order and is awaited with wait_dma().
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ void dma16(const void* gsrc, unsigned lds_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+               :
+               : "v"(gsrc), "s"(lds_base)
+               : "memory", "m0");
+}
+#pragma clang diagnostic pop
+__device__ __forceinline__ void wait_dma() { asm volatile("s_waitcnt vmcnt(0)" : : : "memory"); }
 
 template <int D>
 __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
   using Tile = FwdTile<D>;
   constexpr int KK = D / 16;  // MFMA k-steps over head_dim
   constexpr int DT = D / 32;  // 32-row output tiles over head_dim
+  constexpr int CPR = D / 8;  // 16-byte chunks per row
   extern __shared__ __attribute__((aligned(16))) char smem[];
   char* const k_lds = smem;
-  char* const v_lds = smem + 2 * Tile::KBYTES;
+  char* const v_lds = smem + 2 * Tile::TILE_BYTES;
+  char* const seg_lds = smem + Tile::SEG_BASE;
 
   const int tid = threadIdx.x;
-  const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l32 = lane & 31, g = lane >> 5;
   int qb, b, h;
   decode_block(blockIdx.x, a.T / Tile::BQ, a.B, a.Hq, a.Hkv, qb, b, h);
   const int hk = h / (a.Hq / a.Hkv);
@@ -109,6 +138,13 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
 
   const int qpos = q0 + l32 + a.q_off;       // this lane's query position
   const int qpos_min = q0 + a.q_off, qpos_max = q0 + 31 + a.q_off;  // of the wavefront
+  // Tiles this wavefront has to process (the others it only helps to load): [tw_begin, tw_end).
+  int tw_begin = t_begin, tw_end = t_end;
+  if (a.mask_kind != AXL_MASK_NONE) {
+    tw_end = min(t_end, qpos_max / Tile::BK + 1);
+    if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) tw_begin = max(t_begin, (qpos_min - a.window) / Tile::BK);
+    tw_begin = max(tw_begin, t_begin);
+  }
 
   floatx16 o[DT];
 #pragma unroll
@@ -119,195 +155,233 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
   float l_run = 0.f;      // this lane's share of the running row sum (lanes l and l^32 split it)
   const float c = a.scale * kLog2e;
 
-  // Global -> LDS staging through registers: thread handles 16-byte chunks tid + 256*i of a tile.
-  u32x4 kreg[Tile::CHUNKS], vreg[Tile::CHUNKS];
-  const int st_row = tid / (D / 8), st_cc = tid % (D / 8);   // chunk 0 of this thread
-  constexpr int ROWS_PER_PASS = 256 / (D / 8);               // rows covered by 256 threads
-  const __bf16* kg = kp + (int64_t)st_row * a.ks.s + st_cc * 8;
-  const __bf16* vg = vp + (int64_t)st_row * a.vs.s + st_cc * 8;
-  char* const k_st = k_lds + st_row * Tile::KSTRIDE + st_cc * 16;
-  char* const v_st = v_lds + st_row * Tile::VSTRIDE + st_cc * 16;
-#define AXL_LOAD_TILE(T_)                                                                     \
-  _Pragma("unroll") for (int i = 0; i < Tile::CHUNKS; i++) {                                  \
-    const int64_t row_ = (int64_t)(T_) * Tile::BK + i * ROWS_PER_PASS;                        \
-    kreg[i] = *(const u32x4*)(kg + row_ * a.ks.s);                                            \
-    vreg[i] = *(const u32x4*)(vg + row_ * a.vs.s);                                            \
+  // ---- tile loads: wavefront w fetches rows 16w .. 16w+15 of a K (or V) tile, 1 KB per
+  // instruction (1024 / ROWB rows); lane l's chunk slot is l % CPR of row l / CPR.
+  constexpr int RPI = 1024 / Tile::ROWB;  // rows per instruction
+  int k_src[Tile::DMA_PER_WAVE], v_src[Tile::DMA_PER_WAVE];  // element offsets from the tile's first row
+#pragma unroll
+  for (int i = 0; i < Tile::DMA_PER_WAVE; i++) {
+    const int row = 16 * wave + RPI * i + lane / CPR;
+    const int chunk = (lane % CPR) ^ Tile::swz(row);
+    k_src[i] = row * (int)a.ks.s + chunk * 8;
+    v_src[i] = row * (int)a.vs.s + chunk * 8;
   }
-#define AXL_STORE_TILE(BUF_)                                                                  \
-  _Pragma("unroll") for (int i = 0; i < Tile::CHUNKS; i++) {                                  \
-    *(u32x4*)(k_st + (BUF_) * Tile::KBYTES + i * ROWS_PER_PASS * Tile::KSTRIDE) = kreg[i];    \
-    *(u32x4*)(v_st + (BUF_) * Tile::VBYTES + i * ROWS_PER_PASS * Tile::VSTRIDE) = vreg[i];    \
-  }
+  const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
+  auto issue_k = [&](int t, int buf) {
+    const __bf16* src = kp + (int64_t)t * Tile::BK * a.ks.s;
+    const unsigned dst = lds0 + buf * Tile::TILE_BYTES + wave * (16 * Tile::ROWB);
+#pragma unroll
+    for (int i = 0; i < Tile::DMA_PER_WAVE; i++) dma16(src + k_src[i], dst + i * 1024);
+    if (seg_k && wave == 0 && lane < Tile::BK / 4)  // 64 ids = 16 lanes x 16 bytes
+      dma16(seg_k + t * Tile::BK + 4 * lane, lds0 + Tile::SEG_BASE + (t % Tile::NSEG) * (Tile::BK * 4));
+  };
+  auto issue_v = [&](int t, int buf) {
+    const __bf16* src = vp + (int64_t)t * Tile::BK * a.vs.s;
+    const unsigned dst = lds0 + (2 + buf) * Tile::TILE_BYTES + wave * (16 * Tile::ROWB);
+#pragma unroll
+    for (int i = 0; i < Tile::DMA_PER_WAVE; i++) dma16(src + v_src[i], dst + i * 1024);
+  };
 
-  if (t_begin < t_end) {
-    AXL_LOAD_TILE(t_begin)
-    AXL_STORE_TILE(0)
-  }
-  wait_all_vmem();  // Q fragments have landed: no load issued before the loop is pending inside it
-  __syncthreads();
-
-  // Per-lane LDS read offsets.
-  const int k_row_off = swap_bits_2_3(l32) * Tile::KSTRIDE + g * 16;
+  // ---- per-lane LDS read offsets (bytes).  K row reads: row swap_bits_2_3(l32) (+32 per sub-tile),
+  // logical chunk 2kk + g.  V transposing reads: row 8g + j16/4 (+4 for the second half, +16 per
+  // 16-key group), logical byte column (16 half + 4 (j16 % 4)) * 2 + 64 dt.
+  const int k_row = swap_bits_2_3(l32);
+  const int k_row_off = k_row * Tile::ROWB;
+  const int k_xor = Tile::swz(k_row) << 4;
   const int j16 = lane & 15, half = (lane >> 4) & 1;
-  const int v_lane_off = (8 * g + (j16 >> 2)) * Tile::VSTRIDE + (16 * half + 4 * (j16 & 3)) * 2;
+  const int v_row = 8 * g + (j16 >> 2);
+  const int v_col = (16 * half + 4 * (j16 & 3)) * 2;
+  const int v_off0 = v_row * Tile::ROWB + (v_col & 15), v_off1 = v_off0 + 4 * Tile::ROWB;
+  const int v_xor0 = Tile::swz(v_row) << 4, v_xor1 = Tile::swz(v_row + 4) << 4;
+
+  // Everything the compiler tracks (Q, segment ids) has landed before the first untracked load.
+  wait_all_vmem();
+  if (t_begin < t_end) {
+    issue_k(t_begin, 0);
+    issue_v(t_begin, 0);
+    if (t_begin + 1 < t_end) issue_k(t_begin + 1, 1);
+  }
+
+  union VFrag {
+    bf16x8 v;
+    shortx4 hlf[2];
+  };
+  floatx16 s[2];  // logits of the tile whose softmax is next; sub-tile ks holds keys 32ks .. 32ks+31
+#define AXL_K_FRAG(KT_, KK_, KS_) \
+  (*(const bf16x8*)((KT_) + (KS_) * 32 * Tile::ROWB + k_row_off + ((((KK_) * 32) + g * 16) ^ k_xor)))
+  // S^T of one tile, nothing interleaved (pipeline fill).
+#define AXL_S_PLAIN(KT_, S_)                                                                         \
+  {                                                                                                  \
+    _Pragma("unroll") for (int ks = 0; ks < 2; ks++)                                                 \
+      _Pragma("unroll") for (int r = 0; r < 16; r++) S_[ks][r] = 0.f;                                \
+    _Pragma("unroll") for (int kk = 0; kk < KK; kk++)                                                \
+      _Pragma("unroll") for (int ks = 0; ks < 2; ks++)                                               \
+        S_[ks] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(AXL_K_FRAG(KT_, kk, ks), qf[kk], S_[ks], 0, 0, 0); \
+  }
+
+  // Pipeline fill: S^T of the first tile.
+  wait_dma();
+  __syncthreads();
+  if (t_begin < t_end && t_begin >= tw_begin && t_begin < tw_end) AXL_S_PLAIN(k_lds, s)
 
   for (int t = t_begin; t < t_end; t++) {
     const int buf = (t - t_begin) & 1;
-    const bool has_next = t + 1 < t_end;
-    if (has_next) {
-      AXL_LOAD_TILE(t + 1)
+    // K(t+1) and V(t) (requested one iteration ago) become visible to the whole workgroup and every
+    // wavefront is done with S(t) and PV(t-1); the buffers those were read from are then refilled
+    // with K(t+2) and V(t+1).
+    wait_dma();
+    __syncthreads();
+    if (t + 2 < t_end) issue_k(t + 2, buf);
+    if (t + 1 < t_end) issue_v(t + 1, buf ^ 1);
+
+    const bool do_sm = t >= tw_begin && t < tw_end;          // softmax and PV of tile t
+    const bool do_s = t + 1 >= tw_begin && t + 1 < tw_end;   // S of tile t + 1
+    const char* kt = k_lds + (buf ^ 1) * Tile::TILE_BYTES;   // K(t+1)
+    const char* vt = v_lds + buf * Tile::TILE_BYTES;         // V(t)
+    const int k0 = t * Tile::BK;
+    floatx16 s_nxt[2];
+    if (!do_sm) {
+      if (do_s) {
+        AXL_S_PLAIN(kt, s_nxt)
+        s[0] = s_nxt[0];
+        s[1] = s_nxt[1];
+      }
+      continue;
     }
 
-    const int k0 = t * Tile::BK;
-    bool skip = false;
+    // ---- masks of tile t.  Register r of sub-tile ks in lane group g is key k0 + 32ks + 16(r/8) + 8g + (r%8).
     bool need_mask = false;
     if (a.mask_kind != AXL_MASK_NONE) {
-      skip = k0 > qpos_max;
       need_mask = k0 + Tile::BK - 1 > qpos_min;
-      if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) {
-        skip = skip || (qpos_min - (k0 + Tile::BK - 1) > a.window);
-        need_mask = need_mask || (qpos_max - k0 > a.window);
-      }
+      if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) need_mask = need_mask || (qpos_max - k0 > a.window);
     }
-    if (!skip) {
-      const char* kt = k_lds + buf * Tile::KBYTES;
-      const char* vt = v_lds + buf * Tile::VBYTES;
-      floatx16 s[2];
+    if (need_mask) {
 #pragma unroll
-      for (int ks = 0; ks < 2; ks++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) s[ks][r] = 0.f;
-      // 2*KK independent-by-pairs MFMAs (the two sub-tile chains alternate) fed by 2*KK LDS reads.
-      // The schedule below keeps kAhead reads in flight ahead of the MFMA that consumes them, so
-      // the matrix pipe does not sit out an LDS round trip between two MFMAs.
-      {
-        bf16x8 kfr[KK][2];
-#pragma unroll
-        for (int kk = 0; kk < KK; kk++)
-#pragma unroll
-          for (int ks = 0; ks < 2; ks++)
-            kfr[kk][ks] = *(const bf16x8*)(kt + ks * 32 * Tile::KSTRIDE + k_row_off + kk * 32);
-#pragma unroll
-        for (int kk = 0; kk < KK; kk++)
-#pragma unroll
-          for (int ks = 0; ks < 2; ks++)
-            s[ks] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr[kk][ks], qf[kk], s[ks], 0, 0, 0);
-        constexpr int kAhead = 6;
-        __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
-#pragma unroll
-        for (int i = 0; i < 2 * KK - kAhead; i++) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x008, kAhead, 0);
-      }
-      // Register r of sub-tile ks in lane group g is key k0 + 32ks + 16(r/8) + 8g + (r%8).
-      if (need_mask) {
-#pragma unroll
-        for (int ks = 0; ks < 2; ks++) {
-          const int diff0 = qpos - (k0 + 32 * ks + 8 * g);  // qpos - kpos for r == 0
-#pragma unroll
-          for (int r = 0; r < 16; r++) {
-            const int diff = diff0 - (16 * (r / 8) + (r % 8));
-            bool keep = diff >= 0;
-            if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) keep = keep && diff <= a.window;
-            s[ks][r] = keep ? s[ks][r] : kMasked;
-          }
-        }
-      }
-      if (seg_k) {
-#pragma unroll
-        for (int ks = 0; ks < 2; ks++) {
-#pragma unroll
-          for (int t8 = 0; t8 < 2; t8++) {
-            const int4* sp = (const int4*)(seg_k + k0 + 32 * ks + 16 * t8 + 8 * g);
-            const int4 s0 = sp[0], s1 = sp[1];
-            const int ids[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
-#pragma unroll
-            for (int j = 0; j < 8; j++)
-              s[ks][8 * t8 + j] = (ids[j] == seg_q) ? s[ks][8 * t8 + j] : kMasked;
-          }
-        }
-      }
-      // V^T fragments do not depend on the softmax: the first kPvAhead of the 4*DT PV steps have
-      // their transposing reads issued now, so they land while the arithmetic below runs.
-      // PV step n = (ks*2 + t8)*DT + dt multiplies V^T[32dt.., keys 32ks+16t8..] with P^T.
-      constexpr int kPvSteps = 4 * DT, kPvAhead = 4;
-      union VFrag {
-        bf16x8 v;
-        shortx4 hlf[2];
-      };
-      VFrag vfr[kPvSteps];
-      const char* const vbase = vt + v_lane_off;
-#define AXL_PV_READ(N_)                                                                        \
-  {                                                                                            \
-    const char* va_ = vbase + (16 * ((N_) / DT)) * Tile::VSTRIDE + ((N_) % DT) * 64;           \
-    vfr[N_].hlf[0] = lds_read_tr16(va_);                                                       \
-    vfr[N_].hlf[1] = lds_read_tr16(va_ + 4 * Tile::VSTRIDE);                                   \
-  }
-#pragma unroll
-      for (int n = 0; n < kPvAhead; n++) AXL_PV_READ(n)
-      __builtin_amdgcn_sched_barrier(0);
-
-      float mx = m_run;
-#pragma unroll
-      for (int ks = 0; ks < 2; ks++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[ks][r]);
-      mx = xor32_max(mx);
-      // Lazy rescaling: the running max (and with it the accumulators) only moves when the new max
-      // exceeds it by more than 2^kLazyLog2 in the exponent; until then exp2 is taken against the
-      // stale max, which scales numerator and denominator alike (values stay below 2^kLazyLog2).
-      constexpr float kLazyLog2 = 8.0f;
-      const bool move = (mx - m_run) * c > kLazyLog2;
-      if (__builtin_amdgcn_ballot_w64(move) != 0) {
-        // Subtract first: (m_run * c - mx * c) would be contracted into an fma whose result, for
-        // equal maxima, is the rounding error of the product instead of an exact 0.
-        const float corr = move ? fast_exp2((m_run - mx) * c) : 1.0f;
-        m_run = move ? mx : m_run;
-        l_run *= corr;
-#pragma unroll
-        for (int i = 0; i < DT; i++)
-#pragma unroll
-          for (int r = 0; r < 16; r++) o[i][r] *= corr;
-      }
-      const float mc = m_run * c;
-      float lsum = 0.f;
-#pragma unroll
-      for (int ks = 0; ks < 2; ks++)
+      for (int ks = 0; ks < 2; ks++) {
+        const int diff0 = qpos - (k0 + 32 * ks + 8 * g);  // qpos - kpos for r == 0
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-          const float p = fast_exp2(__builtin_fmaf(s[ks][r], c, -mc));
-          s[ks][r] = p;
-          lsum += p;
+          const int diff = diff0 - (16 * (r / 8) + (r % 8));
+          bool keep = diff >= 0;
+          if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) keep = keep && diff <= a.window;
+          s[ks][r] = keep ? s[ks][r] : kMasked;
         }
-      l_run += lsum;
-      bf16x8 pb[4];
+      }
+    }
+    if (seg_k) {
+      const char* sg = seg_lds + (t % Tile::NSEG) * (Tile::BK * 4);
 #pragma unroll
-      for (int ks = 0; ks < 2; ks++)
+      for (int ks = 0; ks < 2; ks++) {
 #pragma unroll
-        for (int t8 = 0; t8 < 2; t8++)
-          pb[2 * ks + t8] = pack_bf16x8(s[ks][8 * t8 + 0], s[ks][8 * t8 + 1], s[ks][8 * t8 + 2],
-                                        s[ks][8 * t8 + 3], s[ks][8 * t8 + 4], s[ks][8 * t8 + 5],
-                                        s[ks][8 * t8 + 6], s[ks][8 * t8 + 7]);
+        for (int t8 = 0; t8 < 2; t8++) {
+          const intx4 s0 = *(const intx4*)(sg + (32 * ks + 16 * t8 + 8 * g) * 4);
+          const intx4 s1 = *(const intx4*)(sg + (32 * ks + 16 * t8 + 8 * g) * 4 + 16);
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
+            s[ks][8 * t8 + j] = (s0[j] == seg_q) ? s[ks][8 * t8 + j] : kMasked;
+            s[ks][8 * t8 + 4 + j] = (s1[j] == seg_q) ? s[ks][8 * t8 + 4 + j] : kMasked;
+          }
+        }
+      }
+    }
+
+    // ---- row maximum and (lazy) rescaling.  The running max, and with it the accumulators, only
+    // moves when the new max exceeds it by more than 2^kLazyLog2 in the exponent; until then exp2 is
+    // taken against the stale max, which scales numerator and denominator alike.
+    float mx = m_run;
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[ks][r]);
+    mx = xor32_max(mx);
+    constexpr float kLazyLog2 = 8.0f;
+    const bool move = (mx - m_run) * c > kLazyLog2;
+    if (__builtin_amdgcn_ballot_w64(move) != 0) {
+      // Subtract first: (m_run * c - mx * c) would be contracted into an fma whose result, for
+      // equal maxima, is the rounding error of the product instead of an exact 0.
+      const float corr = move ? fast_exp2((m_run - mx) * c) : 1.0f;
+      m_run = move ? mx : m_run;
+      l_run *= corr;
+#pragma unroll
+      for (int i = 0; i < DT; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[i][r] *= corr;
+    }
+    const float mc = m_run * c;
+
+    // ---- exp2 of tile t, interleaved with the S^T MFMAs of tile t+1: slot n runs MFMA (kk, ks) =
+    // (n / 2, n % 2) and the exponentials of 32 / (2 KK) elements; LDS fragments are requested
+    // kAhead slots ahead.
+    constexpr int NSL = 2 * KK, EPS = 32 / NSL, kAhead = 6;
+    static_assert(NSL * EPS == 32, "elements must tile the MFMA slots");
+    float lsum = 0.f;
+    union {
+      bf16x8 v[4];
+      bf16x2 p[16];
+    } pb;
+    if (do_s) {
+      bf16x8 kfr[NSL];
+#pragma unroll
+      for (int n = 0; n < (kAhead < NSL ? kAhead : NSL); n++) kfr[n] = AXL_K_FRAG(kt, n / 2, n % 2);
       __builtin_amdgcn_sched_barrier(0);
-      // O^T += V^T P^T, software pipelined: each MFMA issues together with the reads of the step
-      // kPvAhead ahead of it.
 #pragma unroll
-      for (int n = 0; n < kPvSteps; n++) {
-        if (n + kPvAhead < kPvSteps) AXL_PV_READ(n + kPvAhead)
-        o[n % DT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr[n].v, pb[n / DT], o[n % DT], 0, 0, 0);
+      for (int n = 0; n < NSL; n++) {
+        if (n + kAhead < NSL) kfr[n + kAhead] = AXL_K_FRAG(kt, (n + kAhead) / 2, (n + kAhead) % 2);
+        if (n < 2) {
+          const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+          s_nxt[n % 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr[n], qf[n / 2], zero16, 0, 0, 0);
+        } else {
+          s_nxt[n % 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr[n], qf[n / 2], s_nxt[n % 2], 0, 0, 0);
+        }
+#pragma unroll
+        for (int e = 0; e < EPS; e++) {
+          const int idx = n * EPS + e;
+          const float p = fast_exp2(__builtin_fmaf(s[idx / 16][idx % 16], c, -mc));
+          s[idx / 16][idx % 16] = p;
+          lsum += p;
+          if (idx % 2 == 1) pb.p[idx / 2] = pack_bf16(s[idx / 16][idx % 16 - 1], p);
+        }
         __builtin_amdgcn_sched_barrier(0);
       }
-#undef AXL_PV_READ
+    } else {
+#pragma unroll
+      for (int idx = 0; idx < 32; idx++) {
+        const float p = fast_exp2(__builtin_fmaf(s[idx / 16][idx % 16], c, -mc));
+        s[idx / 16][idx % 16] = p;
+        lsum += p;
+        if (idx % 2 == 1) pb.p[idx / 2] = pack_bf16(s[idx / 16][idx % 16 - 1], p);
+      }
     }
-    if (has_next) {
-      AXL_STORE_TILE(buf ^ 1)
-    }
-    __syncthreads();
+    l_run += lsum;
+
+    // ---- O^T += V^T P^T, software pipelined: each MFMA issues together with the transposing reads
+    // of the step kPvAhead ahead of it.  PV step n = (ks*2 + t8)*DT + dt multiplies
+    // V^T[32dt.., keys 32ks+16t8..] with P^T.
+    constexpr int kPvSteps = 4 * DT, kPvAhead = 4;
+    VFrag vfr[kPvSteps];
+#define AXL_PV_READ(N_)                                                                                  \
+  {                                                                                                      \
+    const char* va_ = vt + (16 * ((N_) / DT)) * Tile::ROWB;                                              \
+    vfr[N_].hlf[0] = lds_read_tr16(va_ + v_off0 + (((v_col & ~15) + ((N_) % DT) * 64) ^ v_xor0));        \
+    vfr[N_].hlf[1] = lds_read_tr16(va_ + v_off1 + (((v_col & ~15) + ((N_) % DT) * 64) ^ v_xor1));        \
   }
-#undef AXL_LOAD_TILE
-#undef AXL_STORE_TILE
+#pragma unroll
+    for (int n = 0; n < kPvAhead; n++) AXL_PV_READ(n)
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int n = 0; n < kPvSteps; n++) {
+      if (n + kPvAhead < kPvSteps) AXL_PV_READ(n + kPvAhead)
+      o[n % DT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr[n].v, pb.v[n / DT], o[n % DT], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#undef AXL_PV_READ
+    if (do_s) {
+      s[0] = s_nxt[0];
+      s[1] = s_nxt[1];
+    }
+  }
+#undef AXL_K_FRAG
+#undef AXL_S_PLAIN
 
   // Epilogue: out = acc / l ; lse = m*scale + ln(l).
   const float l_tot = xor32_sum(l_run);
