@@ -84,6 +84,29 @@ __device__ __forceinline__ int swap_bits_2_3(int m) {
 // not make every iteration wait on the loads it has just issued for the NEXT tile.
 __device__ __forceinline__ void wait_all_vmem() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
+// One 16-byte-per-lane direct global->LDS load (global_load_lds_dwordx4): lane l's 16 bytes land at
+// lds_base + 16*l, where lds_base is a wave-uniform LDS byte address.  Issued through inline assembly
+// so that the compiler neither tracks it nor waits for it; such loads complete in issue order and
+// are awaited with wait_vmem_le<N>() (at most N vector-memory operations still outstanding).
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+__device__ __forceinline__ void dma16(const void* gsrc, unsigned lds_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+               :
+               : "v"(gsrc), "s"(lds_base)
+               : "memory", "m0");
+}
+#pragma clang diagnostic pop
+template <int N>
+__device__ __forceinline__ void wait_vmem_le() {
+  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+__device__ __forceinline__ void wait_lds_reads() { asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory"); }
+// LDS byte address of a pointer into shared memory.
+__device__ __forceinline__ unsigned lds_address(const void* p) {
+  return (unsigned)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
+}
+
 // Segment-id pruning of a workgroup's loop range.  `my_id` is the segment id of one of the rows the
 // workgroup owns (every owned row is passed by at least one thread); ids[lo, hi) are the segment ids
 // of the rows it loops over.  A looped row can only match an owned row if its id lies between the

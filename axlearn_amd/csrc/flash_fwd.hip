@@ -82,20 +82,6 @@ struct FwdTile {
   }
 };
 
-// One 16-byte-per-lane direct global->LDS load: lane l's 16 bytes land at lds_base + 16*l.  Issued
-// through inline assembly so that the compiler neither tracks it nor waits for it; completion is
-// in issue order and is awaited with wait_dma().
-#pragma clang diagnostic push
-#pragma clang diagnostic ignored "-Winline-asm"
-__device__ __forceinline__ void dma16(const void* gsrc, unsigned lds_base) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-               :
-               : "v"(gsrc), "s"(lds_base)
-               : "memory", "m0");
-}
-#pragma clang diagnostic pop
-__device__ __forceinline__ void wait_dma() { asm volatile("s_waitcnt vmcnt(0)" : : : "memory"); }
-
 template <int D>
 __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
   using Tile = FwdTile<D>;
@@ -166,7 +152,7 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
     k_src[i] = row * (int)a.ks.s + chunk * 8;
     v_src[i] = row * (int)a.vs.s + chunk * 8;
   }
-  const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
+  const unsigned lds0 = lds_address(smem);
   auto issue_k = [&](int t, int buf) {
     const __bf16* src = kp + (int64_t)t * Tile::BK * a.ks.s;
     const unsigned dst = lds0 + buf * Tile::TILE_BYTES + wave * (16 * Tile::ROWB);
@@ -220,7 +206,7 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
   }
 
   // Pipeline fill: S^T of the first tile.
-  wait_dma();
+  wait_vmem_le<0>();
   __syncthreads();
   if (t_begin < t_end && t_begin >= tw_begin && t_begin < tw_end) AXL_S_PLAIN(k_lds, s)
 
@@ -229,7 +215,7 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
     // K(t+1) and V(t) (requested one iteration ago) become visible to the whole workgroup and every
     // wavefront is done with S(t) and PV(t-1); the buffers those were read from are then refilled
     // with K(t+2) and V(t+1).
-    wait_dma();
+    wait_vmem_le<0>();
     __syncthreads();
     if (t + 2 < t_end) issue_k(t + 2, buf);
     if (t + 1 < t_end) issue_v(t + 1, buf ^ 1);

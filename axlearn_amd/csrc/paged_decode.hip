@@ -58,24 +58,6 @@ struct DecArgs {
 
 constexpr int kPage = 16;
 
-// One 16-byte-per-lane direct global->LDS load: lane l's 16 bytes land at lds_base + 16*l.  Issued
-// through inline assembly so that the compiler neither tracks it nor waits for it; completion is
-// in issue order and is awaited with wait_vmem_le<N>().
-#pragma clang diagnostic push
-#pragma clang diagnostic ignored "-Winline-asm"
-__device__ __forceinline__ void dma16(const void* gsrc, unsigned lds_base) {
-  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-               :
-               : "v"(gsrc), "s"(lds_base)
-               : "memory", "m0");
-}
-#pragma clang diagnostic pop
-template <int N>
-__device__ __forceinline__ void wait_vmem_le() {
-  asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
-}
-__device__ __forceinline__ void wait_lds_reads() { asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory"); }
-
 // XOR swizzle of the 16-byte chunks of a K row inside an LDS tile, so that 16 lanes reading the
 // same logical chunk of 16 different rows hit 16 different bank groups.
 template <int D>
@@ -296,7 +278,7 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
   const int vrow = 4 * kg + ((lane & 15) >> 2);
   const int v_rd0 = vrow * Tile::ROW_BYTES + ((lane & 2) << 3) + ((lane & 1) << 3);
   const int v_xor = v_swizzle<D>(vrow) << 4;
-  const unsigned ring_lds = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)smem +
+  const unsigned ring_lds = lds_address(smem) +
                             wave * (NST * Tile::STAGE_BYTES);
   char* ring = smem + wave * (NST * Tile::STAGE_BYTES);
 
