@@ -288,3 +288,42 @@ def test_paged_kv_insert_bit_exact(dtype, page_size, d):
         want = ref.reference_decode(q, want_k, want_v, lengths, softmax_scale=0.1, page_tables=tables)[:, 0]
         got = ops.paged_decode(q[:, 0].cuda(), kd, vd, tables.cuda(), lengths.cuda(), softmax_scale=0.1)
         assert _ok(got.cpu(), want)
+
+
+def test_decode_edge_lengths_and_random_shapes():
+    """Lengths of 1, of exactly one page, of a whole number of pages and of the full table; window 0
+    (the query sees only itself); then a seeded sweep of random shapes against the oracle."""
+    hq, hkv, d, pps = 8, 2, 128, 7
+    lengths = torch.tensor([1, 16, 17, 32, 111, 112], dtype=torch.int32)
+    b = lengths.numel()
+    q, kp, vp, tables, _ = ref.paged_inputs(41, batch=b, num_heads=hq, num_kv_heads=hkv, head_dim=d, page_size=16,
+                                            pages_per_seq=pps, min_len=1, max_len=16 * pps)
+    for window in (-1, 0, 5):
+        want = ref.reference_decode(q, kp, vp, lengths, softmax_scale=0.2, page_tables=tables,
+                                    sliding_window=None if window < 0 else window)[:, 0]
+        got = ops.paged_decode(q[:, 0].cuda(), kp.cuda(), vp.cuda(), tables.cuda(), lengths.cuda(),
+                               softmax_scale=0.2, sliding_window=window)
+        assert _ok(got.cpu(), want), (window, ref.max_abs(got.cpu(), want))
+    # window 0: the output is exactly the V row of the last token.
+    got = ops.paged_decode(q[:, 0].cuda(), kp.cuda(), vp.cuda(), tables.cuda(), lengths.cuda(),
+                           softmax_scale=0.2, sliding_window=0)
+    for bi in range(b):
+        n = int(lengths[bi]) - 1
+        row = vp[:, int(tables[bi, n // 16]), n % 16]  # [hkv, d]
+        assert torch.equal(got[bi].cpu(), row.repeat_interleave(hq // hkv, dim=0))
+    rng = np.random.default_rng(17)
+    for _ in range(8):
+        d = int(rng.choice([64, 128]))
+        hkv = int(rng.choice([1, 2, 4]))
+        g = int(rng.choice([1, 2, 3, 4, 8, 16]))
+        b = int(rng.integers(1, 6))
+        pps = int(rng.integers(1, 70))
+        window = int(rng.choice([-1, -1, 3, 100]))
+        q, kp, vp, tables, lengths = ref.paged_inputs(int(rng.integers(1 << 20)), batch=b, num_heads=hkv * g,
+                                                      num_kv_heads=hkv, head_dim=d, page_size=16, pages_per_seq=pps,
+                                                      min_len=1, max_len=16 * pps)
+        want = ref.reference_decode(q, kp, vp, lengths, softmax_scale=d ** -0.5, page_tables=tables,
+                                    sliding_window=None if window < 0 else window)[:, 0]
+        got = ops.paged_decode(q[:, 0].cuda(), kp.cuda(), vp.cuda(), tables.cuda(), lengths.cuda(),
+                               softmax_scale=d ** -0.5, sliding_window=window)
+        assert _ok(got.cpu(), want), (b, hkv, g, d, pps, window, ref.max_abs(got.cpu(), want))

@@ -117,6 +117,50 @@ def test_backward_matches_oracle(b, t, hq, hkv, d, mask, window, seg):
     _assert_close("dv", dv, wv, dtype)
 
 
+@pytest.mark.parametrize("mask,window", [("none", None), ("causal", None), ("sliding", 200)])
+def test_arbitrary_segment_ids_forward_and_backward(mask, window):
+    """Segment ids are compared for equality only (attention_bias.py:876-882): ids need not be sorted,
+    contiguous or non-zero.  Random ids in {0..3} changing every 1..40 positions mask most tiles
+    partially and some wholly, which is what the kernels' segment pruning has to survive."""
+    b, t, hq, hkv, d = 2, 768, 4, 2, 128
+    rng = np.random.default_rng(11)
+    seg = np.zeros((b, t), dtype=np.int32)
+    for bi in range(b):
+        pos = 0
+        while pos < t:
+            n = int(rng.integers(1, 41))
+            seg[bi, pos:pos + n] = int(rng.integers(0, 4))
+            pos += n
+    seg[1, 256:512] = 7                      # one id that fills whole tiles
+    segs = torch.from_numpy(seg)
+    q, k, v, do = _inputs(b, t, hq, hkv, d, torch.bfloat16)
+    spec, kw = _mask_args(mask, window, segs)
+    scale = d ** -0.5
+    want = ref.reference_mha(q, k, v, spec, softmax_scale=scale)
+    wq, wk, wv = ref.reference_mha_grads(q, k, v, do, spec, softmax_scale=scale)
+    qc, kc, vc, doc = q.cuda(), k.cuda(), v.cuda(), do.cuda()
+    out, lse = ops.flash_fwd(qc, kc, vc, softmax_scale=scale, **kw)
+    _assert_close("out", out, want, torch.bfloat16)
+    dq, dk, dv = ops.flash_bwd(qc, kc, vc, out, lse, doc, softmax_scale=scale, **kw)
+    _assert_close("dq", dq, wq, torch.bfloat16)
+    _assert_close("dk", dk, wk, torch.bfloat16)
+    _assert_close("dv", dv, wv, torch.bfloat16)
+
+
+def test_query_offset_chunk_against_full_prefill():
+    """Incremental prefill: a chunk of queries at positions q_off .. q_off+T-1 over S > T keys equals
+    the same rows of a full causal / sliding-window prefill, bit for bit (same tiles, same order)."""
+    b, s_len, hq, hkv, d, t, q_off = 1, 512, 4, 2, 128, 128, 384
+    q, k, v, _ = _inputs(b, s_len, hq, hkv, d, torch.bfloat16)
+    qc, kc, vc = q.cuda(), k.cuda(), v.cuda()
+    for kw in (dict(mask_kind=ops.MASK_CAUSAL), dict(mask_kind=ops.MASK_SLIDING_WINDOW, sliding_window=150)):
+        full, full_lse = ops.flash_fwd(qc, kc, vc, softmax_scale=d ** -0.5, **kw)
+        part, part_lse = ops.flash_fwd(qc[:, q_off:q_off + t].contiguous(), kc, vc, softmax_scale=d ** -0.5,
+                                       q_pos_offset=q_off, **kw)
+        assert torch.equal(part, full[:, q_off:q_off + t])
+        assert torch.equal(part_lse, full_lse[:, :, q_off:q_off + t])
+
+
 def test_against_c_brute_force_tiny():
     """Independent loop-level checker (oracle/brute_force.c) incl. GQA, window and segments."""
     b, t, hq, hkv, d = 1, 128, 2, 1, 64
