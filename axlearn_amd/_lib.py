@@ -20,6 +20,9 @@ MASK_NONE, MASK_CAUSAL, MASK_SLIDING_WINDOW = 0, 1, 2
 AXL_OK, AXL_ERR_INVALID_ARGUMENT, AXL_ERR_UNSUPPORTED, AXL_ERR_WORKSPACE, AXL_ERR_LAUNCH = 0, -1, -2, -3, -4
 
 
+ABI_VERSION = 2  # AXL_ATTN_ABI_VERSION of include/axl_attn.h these structures mirror
+
+
 class AxlError(RuntimeError):
     """A C-ABI call returned a negative status."""
 
@@ -44,6 +47,7 @@ class AxlFlashFwdParams(ctypes.Structure):
         ("dtype", ctypes.c_int32), ("mask_kind", ctypes.c_int32),
         ("sliding_window", ctypes.c_int32), ("q_pos_offset", ctypes.c_int32),
         ("softmax_scale", ctypes.c_float),
+        ("logit_sink", ctypes.c_void_p),
     ]
 
 
@@ -63,6 +67,7 @@ class AxlFlashBwdParams(ctypes.Structure):
         ("sliding_window", ctypes.c_int32), ("q_pos_offset", ctypes.c_int32),
         ("softmax_scale", ctypes.c_float),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
+        ("logit_sink", ctypes.c_void_p), ("d_logit_sink", ctypes.c_void_p),
     ]
 
 
@@ -136,6 +141,11 @@ def load() -> ctypes.CDLL:
     lib = ctypes.CDLL(LIB_PATH)
     lib.axl_last_error.restype = ctypes.c_char_p
     lib.axl_abi_version.restype = ctypes.c_int
+    if lib.axl_abi_version() != ABI_VERSION:
+        raise RuntimeError(
+            f"{LIB_PATH} has ABI version {lib.axl_abi_version()}, this binding expects {ABI_VERSION}: "
+            "rebuild it with `make -C axlearn_amd/csrc`."
+        )
     for name, ptype in (
         ("axl_flash_fwd", AxlFlashFwdParams),
         ("axl_flash_bwd", AxlFlashBwdParams),

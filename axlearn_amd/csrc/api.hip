@@ -149,6 +149,8 @@ int axl_flash_bwd_phases(const AxlFlashBwdParams* p, int phases, void* stream) {
       return set_error(AXL_ERR_UNSUPPORTED, "axl_flash_bwd: rows must be 16-byte aligned");
   if (p->segment_ids && !aligned16(p->segment_ids))
     return set_error(AXL_ERR_UNSUPPORTED, "axl_flash_bwd: segment_ids must be 16-byte aligned");
+  if (p->d_logit_sink && !p->logit_sink)
+    return set_error(AXL_ERR_INVALID_ARGUMENT, "axl_flash_bwd: d_logit_sink without logit_sink");
   const size_t need = flash_bwd_workspace_bytes(*p);
   if (!p->workspace || p->workspace_bytes < need || !aligned16(p->workspace))
     return set_error(AXL_ERR_WORKSPACE, "axl_flash_bwd: workspace needs %zu bytes, got %zu", need,

@@ -60,6 +60,33 @@ __global__ __launch_bounds__(256) void bwd_delta_kernel(const BwdArgs a) {
 }
 
 // ---------------------------------------------------------------------------------------------
+// Gradient of the per-head sink logit.  The sink's probability in row (b, h, t) is
+// exp(sink[h] - lse[b,h,t]) and it has no value row (dP = 0), so dL/dsink is
+// -sum_{b,t} exp(sink[h] - lse) * delta.  One workgroup per head; fixed summation order.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void bwd_dsink_kernel(const float* __restrict__ sink,
+                                                        const float* __restrict__ lse,
+                                                        const float* __restrict__ delta,
+                                                        float* __restrict__ d_sink, int B, int Hq,
+                                                        int T) {
+  __shared__ float red[256];
+  const int h = blockIdx.x, tid = threadIdx.x;
+  const float sk = sink[h];
+  float acc = 0.f;
+  for (int b = 0; b < B; b++) {
+    const int64_t base = ((int64_t)b * Hq + h) * T;
+    for (int t = tid; t < T; t += 256) acc -= expf(sk - lse[base + t]) * delta[base + t];
+  }
+  red[tid] = acc;
+  __syncthreads();
+  for (int w = 128; w > 0; w >>= 1) {
+    if (tid < w) red[tid] += red[tid + w];
+    __syncthreads();
+  }
+  if (tid == 0) d_sink[h] = red[0];
+}
+
+// ---------------------------------------------------------------------------------------------
 // dQ.
 // ---------------------------------------------------------------------------------------------
 template <int D>
@@ -299,6 +326,11 @@ int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream)
     if (phases & AXL_BWD_DQ) AXL_LAUNCH(flash_bwd_dq_bf16_kernel<64>, dq_grid, DqTile<64>::LDS_BYTES);
   }
 #undef AXL_LAUNCH
+  if ((phases & AXL_BWD_DELTA) && p.d_logit_sink && err == hipSuccess) {
+    hipLaunchKernelGGL(bwd_dsink_kernel, dim3(p.num_q_heads), dim3(256), 0, stream, p.logit_sink,
+                       p.lse, a.delta, p.d_logit_sink, p.batch, p.num_q_heads, p.q_len);
+    err = hipGetLastError();
+  }
   if (err != hipSuccess)
     return set_error(AXL_ERR_LAUNCH, "axl_flash_bwd: launch failed: %s", hipGetErrorString(err));
   return AXL_OK;

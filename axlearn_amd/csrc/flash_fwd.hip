@@ -30,6 +30,7 @@ struct FwdArgs {
   void* out;
   float* lse;
   const int32_t* seg;
+  const float* sink;  // [Hq] logit of the per-head attention sink, or nullptr
   Strides3 qs, ks, vs, os;
   int B, T, S, Hq, Hkv;
   int mask_kind, window, q_off;
@@ -140,6 +141,12 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
   float m_run = kNegInf;  // running row max of the raw (unscaled) logits
   float l_run = 0.f;      // this lane's share of the running row sum (lanes l and l^32 split it)
   const float c = a.scale * kLog2e;
+  if (a.sink) {
+    // The sink is one more logit per row, with no value row (attention.py:608-626): it enters the
+    // running softmax state as an already-processed key of weight exp(sink - m) = 1.
+    m_run = a.sink[h] / a.scale;
+    l_run = g == 0 ? 1.f : 0.f;
+  }
 
   // ---- tile loads: wavefront w fetches rows 16w .. 16w+15 of a K (or V) tile, 1 KB per
   // instruction (1024 / ROWB rows); lane l's chunk slot is l % CPR of row l / CPR.
@@ -457,6 +464,10 @@ __global__ __launch_bounds__(256) void flash_fwd_f32_kernel(const FwdArgs a) {
 #pragma unroll
     for (int r = 0; r < 16; r++) o[i][r] = 0.f;
   float m_run = kNegInf, l_run = 0.f;
+  if (a.sink) {  // the sink logit counts as an already-processed key without a value row
+    m_run = a.sink[h];
+    l_run = g == 0 ? 1.f : 0.f;
+  }
   const float* q_row = q_lds + (wave * 32 + l32) * QS;
 
   for (int t = t_begin; t < t_end; t++) {
@@ -547,6 +558,7 @@ static Strides3 to_s3(const AxlStrides& s) { return Strides3{s.batch, s.seq, s.h
 int launch_flash_fwd(const AxlFlashFwdParams& p, hipStream_t stream) {
   FwdArgs a;
   a.q = p.q; a.k = p.k; a.v = p.v; a.out = p.out; a.lse = p.lse; a.seg = p.segment_ids;
+  a.sink = p.logit_sink;
   a.qs = to_s3(p.q_strides); a.ks = to_s3(p.k_strides); a.vs = to_s3(p.v_strides);
   a.os = to_s3(p.out_strides);
   a.B = p.batch; a.T = p.q_len; a.S = p.kv_len; a.Hq = p.num_q_heads; a.Hkv = p.num_kv_heads;

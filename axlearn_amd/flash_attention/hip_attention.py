@@ -59,31 +59,62 @@ def classify_mask_bias(mask: BaseAttentionBias) -> Optional[Tuple[int, int]]:
     return None
 
 
+def padded_head_dim(head_dim: int) -> Optional[int]:
+    """Head dim the kernels run at for a given model head dim (None if it does not fit).
+
+    The Pallas kernel pads the head dim to the next power of two inside its blocks and masks the
+    extra columns (gpu_attention.py:172-176, :328); here the tensors are zero-padded to the next
+    compiled width instead: zero columns of q/k add nothing to the logits and zero columns of v
+    give zero output columns, which are sliced off again."""
+    for width in (64, 128):
+        if head_dim <= width:
+            return width
+    return None
+
+
+def _pad_last(x: Tensor, width: int) -> Tensor:
+    return x if x.shape[-1] == width else torch.nn.functional.pad(x, (0, width - x.shape[-1]))
+
+
+def _attend(query, key, value, segment_ids, softmax_scale, mask_kind, window, logit_sink=None):
+    """Pads the head dim if needed and runs the differentiable kernel pair."""
+    head_dim = query.shape[-1]
+    width = padded_head_dim(head_dim)
+    if width is None:
+        raise NotImplementedError(f"{head_dim=} > 128 is not supported by the HIP kernels.")
+    out = _FlashAttentionFn.apply(
+        _pad_last(query, width), _pad_last(key, width), _pad_last(value, width), segment_ids,
+        softmax_scale, mask_kind, window, logit_sink,
+    )
+    return out if width == head_dim else out[..., :head_dim]
+
+
 class _FlashAttentionFn(torch.autograd.Function):
     """Forward = axl_flash_fwd (saves out and lse), backward = axl_flash_bwd."""
 
     @staticmethod
-    def forward(ctx, query, key, value, segment_ids, softmax_scale, mask_kind, window):
+    def forward(ctx, query, key, value, segment_ids, softmax_scale, mask_kind, window, logit_sink):
         out, lse = ops.flash_fwd(
             query, key, value, softmax_scale=softmax_scale, mask_kind=mask_kind,
-            sliding_window=window, segment_ids=segment_ids,
+            sliding_window=window, segment_ids=segment_ids, logit_sink=logit_sink,
         )
-        ctx.save_for_backward(query, key, value, out, lse)
+        ctx.save_for_backward(query, key, value, out, lse, logit_sink)
         ctx.segment_ids = segment_ids
         ctx.args = (softmax_scale, mask_kind, window)
         return out
 
     @staticmethod
     def backward(ctx, d_out):
-        query, key, value, out, lse = ctx.saved_tensors
+        query, key, value, out, lse, logit_sink = ctx.saved_tensors
         softmax_scale, mask_kind, window = ctx.args
         if d_out.stride(-1) != 1:
             d_out = d_out.contiguous()
-        dq, dk, dv = ops.flash_bwd(
+        grads = ops.flash_bwd(
             query, key, value, out, lse, d_out, softmax_scale=softmax_scale, mask_kind=mask_kind,
-            sliding_window=window, segment_ids=ctx.segment_ids,
+            sliding_window=window, segment_ids=ctx.segment_ids, logit_sink=logit_sink,
         )
-        return dq, dk, dv, None, None, None, None
+        d_sink = grads[3].to(logit_sink.dtype) if logit_sink is not None else None
+        return grads[0], grads[1], grads[2], None, None, None, None, d_sink
 
 
 # pylint: disable-next=too-many-positional-arguments
@@ -123,7 +154,7 @@ def flash_attention(
         raise NotImplementedError(
             "mask_fn must be None, causal_mask or sliding_window_causal_mask(w) for the HIP kernels."
         )
-    return _FlashAttentionFn.apply(query, key, value, segment_ids, float(softmax_scale), kind[0], kind[1])
+    return _attend(query, key, value, segment_ids, float(softmax_scale), kind[0], kind[1])
 
 
 class HipFlashAttention(BaseFlashAttention):
@@ -141,14 +172,15 @@ class HipFlashAttention(BaseFlashAttention):
         if not self._check_block_size(input_batch=input_batch, block_size=128):
             return False
         head_dim = query.shape[-1]
-        if head_dim not in (64, 128):
-            return self._log_unsupported(f"{head_dim=} (supported: 64, 128)")
+        if padded_head_dim(head_dim) is None:  # same limit as gpu_attention.py:954
+            return self._log_unsupported(f"{head_dim=} > 128")
         if query.dtype not in (torch.bfloat16, torch.float32):
             return self._log_unsupported(f"{query.dtype=} (supported: bfloat16, float32)")
         if key.dtype != query.dtype or input_batch["value"].dtype != query.dtype:
             return self._log_unsupported("query, key and value dtypes differ")
-        if input_batch.get("logit_sink", None) is not None:
-            return self._log_unsupported("logit sink is not supported.")
+        logit_sink = input_batch.get("logit_sink", None)
+        if logit_sink is not None and not logit_sink.is_cuda:
+            return self._log_unsupported("logit sink is not on the GPU.")
         if self.cfg.dropout_rate != 0.0:
             return self._log_unsupported("dropout is not supported.")
         if not (self.cfg.softmax_scale > 0.0):
@@ -176,6 +208,7 @@ class HipFlashAttention(BaseFlashAttention):
             raise NotImplementedError("unstructured mask_fn")
         seg = get_segment_ids(query=query, key=key, segment_ids=segment_ids)
         logging.info("HipFlashAttention: mask_kind=%d window=%d segment_ids=%s", kind[0], kind[1], seg is not None)
-        return _FlashAttentionFn.apply(
-            query, key, value, seg, float(self.cfg.softmax_scale), kind[0], kind[1]
+        return _attend(
+            query, key, value, seg, float(self.cfg.softmax_scale), kind[0], kind[1],
+            input_batch.get("logit_sink", None),
         )

@@ -42,6 +42,14 @@ def _require_cuda(*tensors):
             raise AxlError(_lib.AXL_ERR_INVALID_ARGUMENT, "all tensors must live on the GPU")
 
 
+def _sink(logit_sink: Optional[torch.Tensor], num_heads: int) -> Optional[torch.Tensor]:
+    if logit_sink is None:
+        return None
+    if tuple(logit_sink.shape) != (num_heads,):
+        raise AxlError(_lib.AXL_ERR_INVALID_ARGUMENT, f"logit_sink must have shape [{num_heads}]")
+    return logit_sink.detach().to(torch.float32).contiguous()
+
+
 def _seg(segment_ids: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
     if segment_ids is None:
         return None
@@ -61,15 +69,19 @@ def flash_fwd(
     segment_ids: Optional[torch.Tensor] = None,
     q_pos_offset: int = 0,
     return_lse: bool = True,
+    logit_sink: Optional[torch.Tensor] = None,
 ):
-    """q [B,T,Hq,D], k/v [B,S,Hkv,D] -> (out [B,T,Hq,D], lse [B,Hq,T] fp32 or None)."""
-    _require_cuda(q, k, v, segment_ids)
+    """q [B,T,Hq,D], k/v [B,S,Hkv,D] -> (out [B,T,Hq,D], lse [B,Hq,T] fp32 or None).
+
+    logit_sink [Hq]: optional per-head sink logit (joins the softmax and lse, carries no value)."""
+    _require_cuda(q, k, v, segment_ids, logit_sink)
     lib = _lib.load()
     b, t, hq, d = q.shape
     s, hkv = k.shape[1], k.shape[2]
     out = torch.empty((b, t, hq, d), dtype=q.dtype, device=q.device)
     lse = torch.empty((b, hq, t), dtype=torch.float32, device=q.device) if return_lse else None
     seg = _seg(segment_ids)
+    sink = _sink(logit_sink, hq)
     p = AxlFlashFwdParams(
         q=q.data_ptr(), k=k.data_ptr(), v=v.data_ptr(), out=out.data_ptr(), lse=_lib.ptr(lse),
         segment_ids=_lib.ptr(seg),
@@ -78,6 +90,7 @@ def flash_fwd(
         batch=b, q_len=t, kv_len=s, num_q_heads=hq, num_kv_heads=hkv, head_dim=d,
         dtype=_lib.dtype_code(q.dtype), mask_kind=mask_kind, sliding_window=int(sliding_window),
         q_pos_offset=int(q_pos_offset), softmax_scale=float(softmax_scale),
+        logit_sink=_lib.ptr(sink),
     )
     if k.dtype != q.dtype or v.dtype != q.dtype:
         raise AxlError(_lib.AXL_ERR_UNSUPPORTED, "q, k, v must share one dtype")
@@ -100,12 +113,14 @@ def flash_bwd(
     q_pos_offset: int = 0,
     phases: int = 7,
     buffers=None,
+    logit_sink: Optional[torch.Tensor] = None,
 ):
-    """Returns (dq [B,T,Hq,D], dk [B,S,Hkv,D], dv [B,S,Hkv,D]) in the dtype of q.
+    """Returns (dq [B,T,Hq,D], dk [B,S,Hkv,D], dv [B,S,Hkv,D]) in the dtype of q, followed by
+    d_logit_sink [Hq] fp32 when `logit_sink` (the one the forward was given) is passed.
 
     `phases` selects a subset of {1: delta, 2: dK/dV, 4: dQ} (timing / profiling only); `buffers`
     = (dq, dk, dv, workspace) reuses caller-provided outputs instead of allocating."""
-    _require_cuda(q, k, v, out, lse, d_out, segment_ids)
+    _require_cuda(q, k, v, out, lse, d_out, segment_ids, logit_sink)
     lib = _lib.load()
     b, t, hq, d = q.shape
     s, hkv = k.shape[1], k.shape[2]
@@ -119,6 +134,8 @@ def flash_bwd(
     seg = _seg(segment_ids)
     if lse.dtype != torch.float32 or not lse.is_contiguous():
         raise AxlError(_lib.AXL_ERR_INVALID_ARGUMENT, "lse must be contiguous float32 [B,Hq,T]")
+    sink = _sink(logit_sink, hq)
+    d_sink = torch.empty((hq,), dtype=torch.float32, device=q.device) if sink is not None else None
     p = AxlFlashBwdParams(
         q=q.data_ptr(), k=k.data_ptr(), v=v.data_ptr(), out=out.data_ptr(),
         d_out=d_out.data_ptr(), lse=lse.data_ptr(), dq=dq.data_ptr(), dk=dk.data_ptr(),
@@ -129,7 +146,7 @@ def flash_bwd(
         batch=b, q_len=t, kv_len=s, num_q_heads=hq, num_kv_heads=hkv, head_dim=d,
         dtype=_lib.dtype_code(q.dtype), mask_kind=mask_kind, sliding_window=int(sliding_window),
         q_pos_offset=int(q_pos_offset), softmax_scale=float(softmax_scale),
-        workspace=None, workspace_bytes=0,
+        workspace=None, workspace_bytes=0, logit_sink=_lib.ptr(sink), d_logit_sink=_lib.ptr(d_sink),
     )
     need = lib.axl_flash_bwd_workspace_bytes(ctypes.byref(p))
     if ws is None or ws.numel() * ws.element_size() < need:
@@ -137,6 +154,8 @@ def flash_bwd(
     p.workspace = ws.data_ptr()
     p.workspace_bytes = ws.numel() * ws.element_size()
     _lib.check(lib.axl_flash_bwd_phases(ctypes.byref(p), int(phases), _lib.current_stream_ptr()))
+    if sink is not None:
+        return dq, dk, dv, d_sink
     return dq, dk, dv
 
 

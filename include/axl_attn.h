@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define AXL_ATTN_ABI_VERSION 1
+#define AXL_ATTN_ABI_VERSION 2
 
 typedef enum AxlStatus {
   AXL_OK = 0,
@@ -75,6 +75,10 @@ typedef struct AxlFlashFwdParams {
   int32_t sliding_window; /* left context w (keeps w+1 keys); used when mask_kind == SLIDING */
   int32_t q_pos_offset;   /* position of query row 0 */
   float softmax_scale;    /* > 0; multiplies q.k before masking and softmax */
+  const float* logit_sink; /* [Hq] fp32 or NULL: one extra logit per row of head h that takes part in
+                              the softmax (and in lse) but has no value row, so the attention
+                              weights of the real keys sum to less than 1
+                              (axlearn/common/attention.py:608-626; not scaled, never masked) */
 } AxlFlashFwdParams;
 
 int axl_flash_fwd(const AxlFlashFwdParams* params, void* stream);
@@ -87,6 +91,9 @@ int axl_flash_fwd(const AxlFlashFwdParams* params, void* stream);
  *   dk, dv [B,S,Hkv,D] in the dtype of q/k/v.  dk/dv are already summed over the Hq/Hkv query
  *   heads of each kv head (what autodiff of `repeat_kv_heads` does in the reference).
  *   workspace: axl_flash_bwd_workspace_bytes(params) bytes of device scratch (holds delta).
+ *   With a logit sink, dq/dk/dv need nothing beyond an lse that includes the sink; its own gradient
+ *   is a per-head reduction of delta (the Pallas kernels have no sink: gpu_attention.py:957-959
+ *   declines it, so this follows the XLA path, flash_attention/common.py:502-511).
  */
 typedef struct AxlFlashBwdParams {
   const void* q;
@@ -109,6 +116,9 @@ typedef struct AxlFlashBwdParams {
   float softmax_scale;
   void* workspace;
   size_t workspace_bytes;
+  const float* logit_sink; /* [Hq] fp32 or NULL; must be what the forward that produced lse was given */
+  float* d_logit_sink;     /* [Hq] fp32 out or NULL: -sum over (b, t) of exp(sink - lse) * delta,
+                              written (not accumulated) by the DELTA phase */
 } AxlFlashBwdParams;
 
 size_t axl_flash_bwd_workspace_bytes(const AxlFlashBwdParams* params);

@@ -228,8 +228,13 @@ def reference_mha(
     page_tables: Optional[torch.Tensor] = None,
     row_block: int = 512,
     return_lse: bool = False,
+    logit_sink: Optional[torch.Tensor] = None,
 ):
     """`ReferenceMHA.__call__` (flash_attention/common.py:492-519), query-row-blocked.
+
+    logit_sink [Hq]: `softmax_with_biases` (attention.py:608-626) prepends it to every row of head
+    h's biased logits, takes the softmax over S+1 entries and drops the sink's column again, so the
+    returned probabilities sum to less than 1.  The returned lse includes the sink.
 
     query [B,T,Hq,D]; key/value [B,S,Hkv,D] (or page pools [Hkv,P,page,D] with `page_tables`).
 
@@ -279,10 +284,18 @@ def reference_mha(
             bias = mask.bias_rows(b, t0, t1, t, s, torch.float32)
             if bias is not None:
                 logits = logits + bias.to(cdt)
-        m = logits.max(dim=-1, keepdim=True).values
-        e = torch.exp(logits - m)
-        z = e.sum(dim=-1, keepdim=True)
-        probs = e / z
+        if logit_sink is not None:
+            sink = logit_sink.to(logits.dtype).reshape(1, hq, 1, 1).expand(b, hq, t1 - t0, 1)
+            with_sink = torch.cat([sink, logits], dim=-1)
+            m = with_sink.max(dim=-1, keepdim=True).values
+            e_all = torch.exp(with_sink - m)
+            z = e_all.sum(dim=-1, keepdim=True)
+            probs = (e_all / z)[..., 1:]
+        else:
+            m = logits.max(dim=-1, keepdim=True).values
+            e = torch.exp(logits - m)
+            z = e.sum(dim=-1, keepdim=True)
+            probs = e / z
         lse[:, :, t0:t1] = (m + torch.log(z)).squeeze(-1)
         if mode == "faithful":
             probs = _round_to(probs, in_dtype).to(cdt)
@@ -306,9 +319,11 @@ def reference_mha_grads(
     softmax_scale: float = 1.0,
     row_block: int = 512,
     dtype=torch.float64,
+    logit_sink: Optional[torch.Tensor] = None,
 ):
-    """Gradients of `sum(reference_mha(q,k,v) * d_out)` w.r.t. q, k, v by reverse-mode autodiff of
-    the restatement above, in `dtype` on the given inputs, query-row-blocked.
+    """Gradients of `sum(reference_mha(q,k,v) * d_out)` w.r.t. q, k, v (and the logit sink, returned
+    as a fourth tensor when one is given) by reverse-mode autodiff of the restatement above, in
+    `dtype` on the given inputs, query-row-blocked.
 
     The reference obtains these from `jax.grad` of `ReferenceMHA` (gpu_attention_test.py:59-92).
     """
@@ -320,6 +335,7 @@ def reference_mha_grads(
     v = value.to(dtype).clone().requires_grad_(True)
     dq = torch.empty((b, t, hq, d), dtype=dtype)
     do = d_out.to(dtype)
+    sink = None if logit_sink is None else logit_sink.to(dtype).clone().requires_grad_(True)
     for t0 in range(0, t, row_block):
         t1 = min(t, t0 + row_block)
         qb_leaf = query[:, t0:t1].to(dtype).clone().requires_grad_(True)
@@ -328,10 +344,17 @@ def reference_mha_grads(
         bias = mask.bias_rows(b, t0, t1, t, s, torch.float32)
         if bias is not None:
             logits = logits + bias.to(dtype)
-        probs = torch.softmax(logits, dim=-1).reshape(b, hkv, g, t1 - t0, s)
+        if sink is not None:
+            col = sink.reshape(1, hq, 1, 1).expand(b, hq, t1 - t0, 1)
+            probs = torch.softmax(torch.cat([col, logits], dim=-1), dim=-1)[..., 1:]
+        else:
+            probs = torch.softmax(logits, dim=-1)
+        probs = probs.reshape(b, hkv, g, t1 - t0, s)
         ctx = torch.einsum("bkgts,bksd->btkgd", probs, v.permute(0, 2, 1, 3)).reshape(b, t1 - t0, hq, d)
         (ctx * do[:, t0:t1]).sum().backward()
         dq[:, t0:t1] = qb_leaf.grad
+    if sink is not None:
+        return dq, k.grad, v.grad, sink.grad
     return dq, k.grad, v.grad
 
 

@@ -297,6 +297,99 @@ def test_dispatch_and_autograd_end_to_end():
     assert flash_attention_implementation("gpu", query=qd, key=kd, value=vd, bias=dense) is None
 
 
+# ----------------------------------------------------------------------------- logit sink, head dims
+
+
+@pytest.mark.parametrize("b,t,hq,hkv,d,dtype,mask,window,seg", [
+    (2, 256, 4, 2, 128, torch.bfloat16, "causal", None, False),
+    (1, 512, 4, 4, 64, torch.bfloat16, "sliding", 100, True),
+    (1, 384, 2, 1, 128, torch.bfloat16, "none", None, False),
+    (1, 256, 4, 2, 64, torch.float32, "causal", None, True),
+    (1, 128, 2, 2, 128, torch.float32, "none", None, False),
+])
+def test_logit_sink_forward_and_backward(b, t, hq, hkv, d, dtype, mask, window, seg):
+    q, k, v, do = _inputs(b, t, hq, hkv, d, dtype)
+    segs = ref.packed_segment_ids(4, b, t, max_docs=4) if seg else None
+    spec, kw = _mask_args(mask, window, segs)
+    scale = d ** -0.5
+    # Sinks from well below to well above the typical row maximum (logits are ~N(0, 1)).
+    sink = torch.linspace(-3.0, 6.0, hq, dtype=torch.float32)
+    want, want_lse = ref.reference_mha(q, k, v, spec, softmax_scale=scale, logit_sink=sink, return_lse=True)
+    out, lse = ops.flash_fwd(q.cuda(), k.cuda(), v.cuda(), softmax_scale=scale, logit_sink=sink.cuda(), **kw)
+    _assert_close("out", out, want, dtype)
+    assert ref.max_abs(lse.cpu(), want_lse) < (1e-5 if dtype == torch.float32 else 1e-3) * max(1.0, float(want_lse.abs().max()))
+    # The sink must matter in this test: without it the output differs visibly.
+    plain, _ = ops.flash_fwd(q.cuda(), k.cuda(), v.cuda(), softmax_scale=scale, **kw)
+    assert ref.max_abs(plain.cpu(), want) > 0.05
+    if dtype != torch.bfloat16:
+        return  # the backward kernels are bf16 only
+    wq, wk, wv, ws = ref.reference_mha_grads(q, k, v, do, spec, softmax_scale=scale, logit_sink=sink)
+    dq, dk, dv, dsink = ops.flash_bwd(q.cuda(), k.cuda(), v.cuda(), out, lse, do.cuda(), softmax_scale=scale,
+                                     logit_sink=sink.cuda(), **kw)
+    _assert_close("dq", dq, wq, dtype)
+    _assert_close("dk", dk, wk, dtype)
+    _assert_close("dv", dv, wv, dtype)
+    assert dsink.dtype == torch.float32 and ref.rel_l2(dsink.cpu(), ws) < 1e-2, (dsink.cpu(), ws)
+    # Extreme sinks: far below every logit it is invisible (bit-identical output), far above it
+    # takes all the mass; neither produces non-finite values.
+    low, _ = ops.flash_fwd(q.cuda(), k.cuda(), v.cuda(), softmax_scale=scale,
+                           logit_sink=torch.full((hq,), -1e4, device="cuda"), **kw)
+    assert torch.equal(low, plain)
+    high, high_lse = ops.flash_fwd(q.cuda(), k.cuda(), v.cuda(), softmax_scale=scale,
+                                   logit_sink=torch.full((hq,), 1e4, device="cuda"), **kw)
+    assert high.abs().max() == 0 and torch.allclose(high_lse, torch.full_like(high_lse, 1e4))
+
+
+def test_logit_sink_through_dispatch_with_autograd():
+    b, t, hq, hkv, d = 1, 256, 4, 2, 64
+    q, k, v, _ = _inputs(b, t, hq, hkv, d, torch.bfloat16)
+    sink = torch.tensor([0.5, -1.0, 2.0, 0.0])
+    qd, kd, vd = (x.cuda().requires_grad_(True) for x in (q, k, v))
+    sd = sink.cuda().requires_grad_(True)
+    pos = dict(target_positions=torch.arange(t)[None], source_positions=torch.arange(t)[None])
+    bias = ab.CompositeAttentionBias([ab.CausalAttentionBias(**pos)])
+    scale = d ** -0.5
+    impl = flash_attention_implementation("gpu", query=qd, key=kd, value=vd, bias=bias, softmax_scale=scale,
+                                          logit_sink=sd)
+    assert impl is not None and isinstance(impl.fn, HipFlashAttention)
+    out = impl.fn(dict(query=qd, key=kd, value=vd, bias=bias, logit_sink=sd))
+    do = ref.normal_tensor(9, (b, t, hq, d), torch.bfloat16)
+    (out.float() * do.cuda().float()).sum().backward()
+    spec = ref.MaskSpec(causal=True)
+    want = ref.reference_mha(q, k, v, spec, softmax_scale=scale, logit_sink=sink)
+    wq, wk, wv, ws = ref.reference_mha_grads(q, k, v, do, spec, softmax_scale=scale, logit_sink=sink)
+    _assert_close("out", out, want, torch.bfloat16)
+    for name, got, exp in (("dq", qd.grad, wq), ("dk", kd.grad, wk), ("dv", vd.grad, wv)):
+        _assert_close(name, got, exp, torch.bfloat16)
+    assert sd.grad.shape == (hq,) and ref.rel_l2(sd.grad.cpu(), ws) < 1e-2
+
+
+@pytest.mark.parametrize("d", [32, 80, 96, 120])
+def test_head_dims_between_the_compiled_widths(d):
+    # Any head dim up to 128 is accepted, as by the Pallas kernel (gpu_attention.py:172-176, :954):
+    # the host zero-pads to 64 or 128 and slices the result; gradients flow through the padding.
+    b, t, hq, hkv = 1, 256, 4, 2
+    q, k, v, do = _inputs(b, t, hq, hkv, d, torch.bfloat16)
+    qd, kd, vd = (x.cuda().requires_grad_(True) for x in (q, k, v))
+    scale = d ** -0.5
+    out = flash_attention(qd, kd, vd, softmax_scale=scale, mask_fn=ab.causal_mask)
+    assert out.shape == (b, t, hq, d)
+    (out.float() * do.cuda().float()).sum().backward()
+    spec = ref.MaskSpec(causal=True)
+    want = ref.reference_mha(q, k, v, spec, softmax_scale=scale)
+    wq, wk, wv = ref.reference_mha_grads(q, k, v, do, spec, softmax_scale=scale)
+    _assert_close("out", out, want, torch.bfloat16)
+    for name, got, exp in (("dq", qd.grad, wq), ("dk", kd.grad, wk), ("dv", vd.grad, wv)):
+        assert got.shape == exp.shape
+        _assert_close(name, got, exp, torch.bfloat16)
+    pos = dict(target_positions=torch.arange(t)[None], source_positions=torch.arange(t)[None])
+    bias = ab.CompositeAttentionBias([ab.CausalAttentionBias(**pos)])
+    fa = HipFlashAttention.default_config().set(softmax_scale=scale).instantiate()
+    batch = dict(query=qd.detach(), key=kd.detach(), value=vd.detach(), bias=bias)
+    assert fa.is_supported(batch, kv_cache_type=None)
+    assert torch.equal(fa(batch), out.detach())
+
+
 # ----------------------------------------------------------------------------- BASELINE sizes
 
 

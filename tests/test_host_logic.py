@@ -261,7 +261,9 @@ def test_library_exports_every_declared_symbol():
     lib = _lib.load()
     for name in declared:
         assert hasattr(lib, name), name
-    assert lib.axl_abi_version() == 1
+    header = open(os.path.join(ROOT, "include", "axl_attn.h")).read()
+    declared_version = int(re.search(r"#define AXL_ATTN_ABI_VERSION (\d+)", header).group(1))
+    assert lib.axl_abi_version() == declared_version == _lib.ABI_VERSION
     assert lib.axl_last_error() is not None
 
 

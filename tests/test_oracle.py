@@ -212,6 +212,69 @@ def test_gradient_identities():
     assert np.abs(dq - dq0).max() > 1e-3
 
 
+# ------------------------------------------------------------------ logit sink
+
+
+def _sink_as_extra_key(q, k, v, sink, scale):
+    """The sink written as an ordinary key, so that the sink-free oracle (pinned above) applies:
+    one more coordinate holds sink_h / scale in the queries of head h, 1 in the extra key and 0 in
+    the real keys, and the extra key's value row is zero."""
+    b, t, hq, d = q.shape
+    s, hkv = k.shape[1], k.shape[2]
+    qa = np.concatenate([q, np.broadcast_to((sink / scale)[None, None, :, None], (b, t, hq, 1))], axis=-1)
+    ka = np.zeros((b, s + 1, hkv, d + 1))
+    ka[:, 1:, :, :d] = k
+    ka[:, 0, :, d] = 1.0
+    va = np.zeros((b, s + 1, hkv, d + 1))
+    va[:, 1:, :, :d] = v
+    return qa, ka, va
+
+
+def test_logit_sink_equals_an_extra_key_with_zero_value():
+    b, t, s, hq, hkv, d = 2, 7, 11, 4, 2, 5
+    q, k, v, do = (_rand(i, sh) for i, sh in ((60, (b, t, hq, d)), (61, (b, s, hkv, d)), (62, (b, s, hkv, d)), (63, (b, t, hq, d))))
+    sink = np.asarray([0.9, -1.3, 0.0, 2.5])
+    scale = 0.41
+    tq, tk, tv, tdo, tsink = (torch.from_numpy(x) for x in (q, k, v, do, sink))
+    out, lse = ref.reference_mha(tq, tk, tv, softmax_scale=scale, logit_sink=tsink, return_lse=True, row_block=3)
+    qa, ka, va = _sink_as_extra_key(q, k, v, sink, scale)
+    want, want_lse = ref.reference_mha(*(torch.from_numpy(x) for x in (qa, ka, va)), softmax_scale=scale, return_lse=True)
+    np.testing.assert_allclose(out.numpy(), want.numpy()[..., :d], rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(lse.numpy(), want_lse.numpy(), rtol=1e-12, atol=1e-12)
+    # The C brute force agrees on the augmented problem too.
+    bo, _ = brute.attention_fwd(qa, ka, va, scale=scale)
+    np.testing.assert_allclose(out.numpy(), bo[..., :d], rtol=1e-12, atol=1e-12)
+    # Gradients: those of the real coordinates carry over; d sink_h = sum_{b,t} dq'[b,t,h,D] / scale.
+    dq, dk, dv, dsink = ref.reference_mha_grads(tq, tk, tv, tdo, softmax_scale=scale, logit_sink=tsink, row_block=3)
+    doa = np.concatenate([do, np.zeros((b, t, hq, 1))], axis=-1)
+    aq, ak, av = brute.attention_bwd(qa, ka, va, doa, scale=scale)
+    np.testing.assert_allclose(dq.numpy(), aq[..., :d], rtol=1e-10, atol=1e-12)
+    np.testing.assert_allclose(dk.numpy(), ak[:, 1:, :, :d], rtol=1e-10, atol=1e-12)
+    np.testing.assert_allclose(dv.numpy(), av[:, 1:, :, :d], rtol=1e-10, atol=1e-12)
+    np.testing.assert_allclose(dsink.numpy(), aq[..., d].sum(axis=(0, 1)) / scale, rtol=1e-10, atol=1e-12)
+
+
+def test_logit_sink_closed_forms():
+    b, t, h, d = 1, 8, 2, 4
+    q, k, v = (torch.from_numpy(_rand(i, (b, t, h, d))) for i in (64, 65, 66))
+    # Equal logits everywhere (q == 0) and sink 0: S + 1 equal weights, one of them on nothing.
+    out = ref.reference_mha(torch.zeros_like(q), k, v, logit_sink=torch.zeros(h, dtype=torch.float64))
+    torch.testing.assert_close(out, (v.sum(dim=1, keepdim=True) / (t + 1)).expand_as(v))
+    # A sink far below every logit changes nothing; one far above takes all the mass.
+    base = ref.reference_mha(q, k, v, ref.MaskSpec(causal=True))
+    low = ref.reference_mha(q, k, v, ref.MaskSpec(causal=True), logit_sink=torch.full((h,), -1e4, dtype=torch.float64))
+    torch.testing.assert_close(low, base)
+    high = ref.reference_mha(q, k, v, ref.MaskSpec(causal=True), logit_sink=torch.full((h,), 1e4, dtype=torch.float64))
+    assert high.abs().max() == 0
+    # Causal row 0 sees key 0 and the sink: weight sigmoid(s00 - sink) on v0.  The mask bias does
+    # not touch the sink (attention.py:596-598).
+    sink = torch.tensor([0.3, -0.7], dtype=torch.float64)
+    out, lse = ref.reference_mha(q, k, v, ref.MaskSpec(causal=True), logit_sink=sink, return_lse=True)
+    s00 = (q[:, 0] * k[:, 0]).sum(-1)  # [b, h]
+    torch.testing.assert_close(out[:, 0], torch.sigmoid(s00 - sink)[..., None] * v[:, 0])
+    torch.testing.assert_close(lse[:, :, 0], torch.logaddexp(s00, sink.expand_as(s00)))
+
+
 # ------------------------------------------------------------------ paged KV / decode
 
 
