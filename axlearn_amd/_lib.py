@@ -20,7 +20,7 @@ MASK_NONE, MASK_CAUSAL, MASK_SLIDING_WINDOW = 0, 1, 2
 AXL_OK, AXL_ERR_INVALID_ARGUMENT, AXL_ERR_UNSUPPORTED, AXL_ERR_WORKSPACE, AXL_ERR_LAUNCH = 0, -1, -2, -3, -4
 
 
-ABI_VERSION = 2  # AXL_ATTN_ABI_VERSION of include/axl_attn.h these structures mirror
+ABI_VERSION = 3  # AXL_ATTN_ABI_VERSION of include/axl_attn.h these structures mirror
 
 
 class AxlError(RuntimeError):
@@ -33,6 +33,18 @@ class AxlError(RuntimeError):
 
 class AxlStrides(ctypes.Structure):
     _fields_ = [("batch", ctypes.c_int64), ("seq", ctypes.c_int64), ("head", ctypes.c_int64)]
+
+
+class AxlAttnAux(ctypes.Structure):
+    _fields_ = [
+        ("bias", ctypes.c_void_p),
+        ("bias_batch_stride", ctypes.c_int64), ("bias_head_stride", ctypes.c_int64),
+        ("bias_row_stride", ctypes.c_int64),
+        ("bias_dtype", ctypes.c_int32), ("dropout_rate", ctypes.c_float),
+        ("dropout_mask", ctypes.c_void_p),
+        ("drop_batch_stride", ctypes.c_int64), ("drop_head_stride", ctypes.c_int64),
+        ("drop_row_stride", ctypes.c_int64),
+    ]
 
 
 class AxlFlashFwdParams(ctypes.Structure):
@@ -48,6 +60,7 @@ class AxlFlashFwdParams(ctypes.Structure):
         ("sliding_window", ctypes.c_int32), ("q_pos_offset", ctypes.c_int32),
         ("softmax_scale", ctypes.c_float),
         ("logit_sink", ctypes.c_void_p),
+        ("aux", AxlAttnAux),
     ]
 
 
@@ -68,6 +81,7 @@ class AxlFlashBwdParams(ctypes.Structure):
         ("softmax_scale", ctypes.c_float),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
         ("logit_sink", ctypes.c_void_p), ("d_logit_sink", ctypes.c_void_p),
+        ("aux", AxlAttnAux),
     ]
 
 

@@ -65,6 +65,47 @@ static int check_flash_shapes(const char* who, int batch, int q_len, int kv_len,
   return AXL_OK;
 }
 
+AuxArgs make_aux_args(const AxlAttnAux& x, float softmax_scale) {
+  AuxArgs a;
+  const int es = x.bias_dtype == AXL_F32 ? 4 : 2;
+  a.bias = (const char*)x.bias;
+  a.drop = x.dropout_mask;
+  a.bias_sb = x.bias_batch_stride * es; a.bias_sh = x.bias_head_stride * es; a.bias_sr = x.bias_row_stride * es;
+  a.drop_sb = x.drop_batch_stride; a.drop_sh = x.drop_head_stride; a.drop_sr = x.drop_row_stride;
+  a.bias_f32 = x.bias_dtype == AXL_F32;
+  a.inv_scale = 1.0f / softmax_scale;
+  a.keep_scale = x.dropout_mask ? 1.0f / (1.0f - x.dropout_rate) : 1.0f;
+  return a;
+}
+
+// The kernels read 8 consecutive bias elements / mask bytes per access (4 in the fp32 forward).
+int check_aux(const char* who, const AxlAttnAux& x, int batch, int hq, int q_len, int kv_len) {
+  (void)batch; (void)hq; (void)q_len;
+  if (x.bias) {
+    if (x.bias_dtype != AXL_BF16 && x.bias_dtype != AXL_F32)
+      return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: unknown bias dtype %d", who, x.bias_dtype);
+    const int64_t m = x.bias_dtype == AXL_F32 ? 4 : 8;
+    if (x.bias_batch_stride < 0 || x.bias_head_stride < 0 || x.bias_row_stride < kv_len)
+      return set_error(AXL_ERR_INVALID_ARGUMENT,
+                       "%s: bias strides must be >= 0 and its row stride >= kv_len", who);
+    if (!aligned16(x.bias) || x.bias_batch_stride % m || x.bias_head_stride % m || x.bias_row_stride % m)
+      return set_error(AXL_ERR_UNSUPPORTED, "%s: bias rows must be 16-byte aligned", who);
+  }
+  if (x.dropout_mask) {
+    if (!(x.dropout_rate >= 0.f) || !(x.dropout_rate < 1.f))
+      return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: dropout_rate must be in [0, 1)", who);
+    if (x.drop_batch_stride < 0 || x.drop_head_stride < 0 || x.drop_row_stride < kv_len)
+      return set_error(AXL_ERR_INVALID_ARGUMENT,
+                       "%s: dropout mask strides must be >= 0 and its row stride >= kv_len", who);
+    if ((reinterpret_cast<uintptr_t>(x.dropout_mask) & 7) || x.drop_batch_stride % 8 ||
+        x.drop_head_stride % 8 || x.drop_row_stride % 8)
+      return set_error(AXL_ERR_UNSUPPORTED, "%s: dropout mask rows must be 8-byte aligned", who);
+  } else if (x.dropout_rate != 0.f) {
+    return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: dropout_rate without a dropout_mask", who);
+  }
+  return AXL_OK;
+}
+
 }  // namespace axl
 
 using namespace axl;
@@ -115,6 +156,8 @@ int axl_flash_fwd(const AxlFlashFwdParams* p, void* stream) {
     return set_error(AXL_ERR_UNSUPPORTED, "axl_flash_fwd: tensors must be 16-byte aligned rows");
   if (p->segment_ids && !aligned16(p->segment_ids))
     return set_error(AXL_ERR_UNSUPPORTED, "axl_flash_fwd: segment_ids must be 16-byte aligned");
+  rc = check_aux("axl_flash_fwd", p->aux, p->batch, p->num_q_heads, p->q_len, p->kv_len);
+  if (rc != AXL_OK) return rc;
   return launch_flash_fwd(*p, (hipStream_t)stream);
 }
 
@@ -149,6 +192,8 @@ int axl_flash_bwd_phases(const AxlFlashBwdParams* p, int phases, void* stream) {
       return set_error(AXL_ERR_UNSUPPORTED, "axl_flash_bwd: rows must be 16-byte aligned");
   if (p->segment_ids && !aligned16(p->segment_ids))
     return set_error(AXL_ERR_UNSUPPORTED, "axl_flash_bwd: segment_ids must be 16-byte aligned");
+  rc = check_aux("axl_flash_bwd", p->aux, p->batch, p->num_q_heads, p->q_len, p->kv_len);
+  if (rc != AXL_OK) return rc;
   if (p->d_logit_sink && !p->logit_sink)
     return set_error(AXL_ERR_INVALID_ARGUMENT, "axl_flash_bwd: d_logit_sink without logit_sink");
   const size_t need = flash_bwd_workspace_bytes(*p);

@@ -147,6 +147,48 @@ struct Strides3 {
   int64_t b, s, h;
 };
 
+// Dense bias / dropout mask of the prefill kernels (AxlAttnAux), in kernel-argument form.
+struct AuxArgs {
+  const char* bias;     // nullptr = none
+  const uint8_t* drop;  // nullptr = none; nonzero byte = dropped
+  int64_t bias_sb, bias_sh, bias_sr;  // BYTES per batch / head / query row
+  int64_t drop_sb, drop_sh, drop_sr;  // bytes
+  int bias_f32;         // element type of bias: 1 fp32, 0 bf16
+  float inv_scale;      // 1 / softmax_scale: bias in units of the raw (unscaled) logits
+  float keep_scale;     // 1 / (1 - dropout_rate)
+};
+
+AuxArgs make_aux_args(const AxlAttnAux& x, float softmax_scale);
+int check_aux(const char* who, const AxlAttnAux& x, int batch, int hq, int q_len, int kv_len);
+
+// N consecutive bias elements (N = 4 or 8) starting at byte offset `off` of the ELEMENT index, i.e.
+// p points at the row, `col` is the first key; returns them as fp32.
+template <int N>
+__device__ __forceinline__ void load_bias(const char* row, int col, int is_f32, float (&out)[N]) {
+  if (is_f32) {
+#pragma unroll
+    for (int i = 0; i < N / 4; i++) {
+      const floatx4 v = *(const floatx4*)(row + (int64_t)col * 4 + 16 * i);
+#pragma unroll
+      for (int j = 0; j < 4; j++) out[4 * i + j] = v[j];
+    }
+  } else {
+    union {
+      uint32_t u[N / 2];
+      __bf16 e[N];
+    } w;
+    if constexpr (N == 8) {
+      const u32x4 v = *(const u32x4*)(row + (int64_t)col * 2);
+      w.u[0] = v[0]; w.u[1] = v[1]; w.u[2] = v[2]; w.u[3] = v[3];
+    } else {
+      const uint2 v = *(const uint2*)(row + (int64_t)col * 2);
+      w.u[0] = v.x; w.u[1] = v.y;
+    }
+#pragma unroll
+    for (int i = 0; i < N; i++) out[i] = (float)w.e[i];
+  }
+}
+
 int set_error(int code, const char* fmt, ...);
 
 }  // namespace axl

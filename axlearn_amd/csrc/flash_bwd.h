@@ -21,9 +21,11 @@ struct BwdArgs {
   int B, T, S, Hq, Hkv;
   int mask_kind, window, q_off;
   float scale;
+  AuxArgs aux;  // dense bias / dropout mask (read only by the AUX instantiations)
 };
 
-// Enqueues the dK/dV kernel (bf16) for head_dim 64 or 128.
-hipError_t launch_bwd_dkdv_bf16(const BwdArgs& a, int head_dim, hipStream_t stream);
+// Enqueues the dK/dV kernel (bf16) for head_dim 64 or 128; `aux` selects the instantiation that
+// reads the dense bias / dropout mask.
+hipError_t launch_bwd_dkdv_bf16(const BwdArgs& a, int head_dim, bool aux, hipStream_t stream);
 
 }  // namespace axl

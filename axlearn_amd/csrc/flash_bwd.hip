@@ -99,7 +99,7 @@ struct DqTile {
   static constexpr int LDS_BYTES = 4 * TILE_BYTES;  // {K, V} x double buffer
 };
 
-template <int D>
+template <int D, bool AUX>
 __global__ __launch_bounds__(256) void flash_bwd_dq_bf16_kernel(const BwdArgs a) {
   using Tile = DqTile<D>;
   constexpr int KK = D / 16, DT = D / 32;
@@ -144,6 +144,12 @@ __global__ __launch_bounds__(256) void flash_bwd_dq_bf16_kernel(const BwdArgs a)
   const int t_end = (k_end + Tile::BK - 1) / Tile::BK;
   const int qpos = q0 + l32 + a.q_off;
   const int qpos_min = q0 + a.q_off, qpos_max = q0 + 31 + a.q_off;
+  const char* bias_row = nullptr;   // dense bias / dropout mask rows of this lane's query
+  const uint8_t* drop_row = nullptr;
+  if constexpr (AUX) {
+    if (a.aux.bias) bias_row = a.aux.bias + b * a.aux.bias_sb + h * a.aux.bias_sh + (int64_t)(q0 + l32) * a.aux.bias_sr;
+    if (a.aux.drop) drop_row = a.aux.drop + b * a.aux.drop_sb + h * a.aux.drop_sh + (int64_t)(q0 + l32) * a.aux.drop_sr;
+  }
 
   floatx16 dq_acc[DT];
 #pragma unroll
@@ -219,6 +225,30 @@ __global__ __launch_bounds__(256) void flash_bwd_dq_bf16_kernel(const BwdArgs a)
           dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr, dof[kk], dp, 0, 0, 0);
         }
         // Register r of lane group g is key k0 + 32ks + 16(r/8) + 8g + (r%8); the lane is a query.
+        if constexpr (AUX) {
+          // logits = scale * qk + bias, kept in raw units as qk + bias / scale; a dropped element
+          // has dP = 0, a kept one dP / (1 - rate) (gpu_attention.py:601-603).
+          if (bias_row) {
+#pragma unroll
+            for (int t8 = 0; t8 < 2; t8++) {
+              float bv[8];
+              load_bias<8>(bias_row, k0 + 32 * ks + 16 * t8 + 8 * g, a.aux.bias_f32, bv);
+#pragma unroll
+              for (int j = 0; j < 8; j++) s[8 * t8 + j] = __builtin_fmaf(bv[j], a.aux.inv_scale, s[8 * t8 + j]);
+            }
+          }
+          if (drop_row) {
+#pragma unroll
+            for (int t8 = 0; t8 < 2; t8++) {
+              const uint2 w = *(const uint2*)(drop_row + k0 + 32 * ks + 16 * t8 + 8 * g);
+#pragma unroll
+              for (int j = 0; j < 8; j++) {
+                const unsigned byte = ((j < 4 ? w.x : w.y) >> (8 * (j % 4))) & 0xffu;
+                dp[8 * t8 + j] = byte ? 0.f : dp[8 * t8 + j] * a.aux.keep_scale;
+              }
+            }
+          }
+        }
         // Masks in (at most) two wave-uniform blocks; unmasked tiles run straight-line code.
         if (need_mask) {
           const int diff0 = qpos - (k0 + 32 * ks + 8 * g);
@@ -301,6 +331,8 @@ int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream)
   a.B = p.batch; a.T = p.q_len; a.S = p.kv_len; a.Hq = p.num_q_heads; a.Hkv = p.num_kv_heads;
   a.mask_kind = p.mask_kind; a.window = p.sliding_window; a.q_off = p.q_pos_offset;
   a.scale = p.softmax_scale;
+  a.aux = make_aux_args(p.aux, p.softmax_scale);
+  const bool aux = p.aux.bias || p.aux.dropout_mask;
   hipError_t err = hipSuccess;
   const int64_t rows = (int64_t)p.batch * p.q_len * p.num_q_heads;
   const int delta_grid = (int)((rows + 15) / 16);
@@ -318,12 +350,14 @@ int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream)
   } while (0)
   if (p.head_dim == 128) {
     if (phases & AXL_BWD_DELTA) AXL_LAUNCH((bwd_delta_kernel<__bf16, 128>), delta_grid, 0);
-    if ((phases & AXL_BWD_DKDV) && err == hipSuccess) err = launch_bwd_dkdv_bf16(a, 128, stream);
-    if (phases & AXL_BWD_DQ) AXL_LAUNCH(flash_bwd_dq_bf16_kernel<128>, dq_grid, DqTile<128>::LDS_BYTES);
+    if ((phases & AXL_BWD_DKDV) && err == hipSuccess) err = launch_bwd_dkdv_bf16(a, 128, aux, stream);
+    if ((phases & AXL_BWD_DQ) && aux) AXL_LAUNCH((flash_bwd_dq_bf16_kernel<128, true>), dq_grid, DqTile<128>::LDS_BYTES);
+    if ((phases & AXL_BWD_DQ) && !aux) AXL_LAUNCH((flash_bwd_dq_bf16_kernel<128, false>), dq_grid, DqTile<128>::LDS_BYTES);
   } else {
     if (phases & AXL_BWD_DELTA) AXL_LAUNCH((bwd_delta_kernel<__bf16, 64>), delta_grid, 0);
-    if ((phases & AXL_BWD_DKDV) && err == hipSuccess) err = launch_bwd_dkdv_bf16(a, 64, stream);
-    if (phases & AXL_BWD_DQ) AXL_LAUNCH(flash_bwd_dq_bf16_kernel<64>, dq_grid, DqTile<64>::LDS_BYTES);
+    if ((phases & AXL_BWD_DKDV) && err == hipSuccess) err = launch_bwd_dkdv_bf16(a, 64, aux, stream);
+    if ((phases & AXL_BWD_DQ) && aux) AXL_LAUNCH((flash_bwd_dq_bf16_kernel<64, true>), dq_grid, DqTile<64>::LDS_BYTES);
+    if ((phases & AXL_BWD_DQ) && !aux) AXL_LAUNCH((flash_bwd_dq_bf16_kernel<64, false>), dq_grid, DqTile<64>::LDS_BYTES);
   }
 #undef AXL_LAUNCH
   if ((phases & AXL_BWD_DELTA) && p.d_logit_sink && err == hipSuccess) {

@@ -44,7 +44,7 @@ struct DkvTile {
   static constexpr int LDS_BYTES = NBUF * BUF_BYTES;
 };
 
-template <int D, bool HAS_SEG>
+template <int D, bool HAS_SEG, bool AUX>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
   using Tile = DkvTile<D>;
@@ -150,13 +150,14 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
     }                                                                                             \
   }
   // Prefetch cursor; it stops at the last tile (re-fetching that tile is harmless).
-  int pf_idx = 0, pf_t = 0;
+  int pf_idx = 0, pf_t = 0, pf_h = 0;  // tile number, query tile within the head, head within the group
 #define AXL_ADVANCE()                                                       \
   {                                                                         \
     const bool adv_ = pf_idx + 1 < total;                                   \
     const bool wrap_ = adv_ && (pf_t + 1 == nt);                            \
     pf_idx += adv_ ? 1 : 0;                                                 \
     pf_t = wrap_ ? 0 : pf_t + (adv_ ? 1 : 0);                               \
+    pf_h += wrap_ ? 1 : 0;                                                  \
     q_src += adv_ ? (wrap_ ? q_wrap : q_step) : 0;                          \
     d_src += adv_ ? (wrap_ ? d_wrap : d_step) : 0;                          \
     s_src += adv_ ? (wrap_ ? (s_is_seg ? seg_wrap : s_wrap) : s_step) : 0;  \
@@ -210,9 +211,43 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
     const unsigned diff_ = (unsigned)(diff0 + 16 * (r_ / 8) + (r_ % 8));                       \
     float sv_ = diff_ <= limit ? s_e[r_] : kMasked;                                            \
     if (HAS_SEG) sv_ = seg_v[r_ / 4][r_ % 4] == seg_k ? sv_ : kMasked;                         \
-    const float p_ = fast_exp2(__builtin_fmaf(sv_, c, lse_v[r_ / 4][r_ % 4])); /* lse_v = -lse*log2e */ \
-    s_e[r_] = p_;                                                                              \
-    dp_e[r_] = p_ * (dp_e[r_] - del_v[r_ / 4][r_ % 4]);                                        \
+    float off_ = lse_v[r_ / 4][r_ % 4]; /* -lse * log2 e */                                    \
+    float dpv_ = dp_e[r_];                                                                     \
+    bool kept_ = true;                                                                         \
+    if constexpr (AUX) {                                                                       \
+      /* bias raw bits: fp32 as loaded, bf16 in the low half; zero when there is no bias */    \
+      off_ = __builtin_fmaf(__builtin_bit_cast(float, braw_v[r_] << bias_shift), kLog2e, off_); \
+      kept_ = draw_v[r_] == 0;                                                                 \
+      dpv_ = kept_ ? dpv_ * a.aux.keep_scale : 0.f; /* gpu_attention.py:509-512 */            \
+    }                                                                                          \
+    const float p_ = fast_exp2(__builtin_fmaf(sv_, c, off_));                                  \
+    s_e[r_] = kept_ ? p_ : 0.f; /* P that multiplies dO: dropped entries removed */            \
+    dp_e[r_] = p_ * (dpv_ - del_v[r_ / 4][r_ % 4]);                                            \
+  }
+  // Dense bias / dropout mask (AUX): this lane's key column of the 16 query rows of a tile, one
+  // element per register, requested a whole iteration before the elementwise stage consumes it.
+  uint32_t braw_v[16], draw_v[16];
+#pragma unroll
+  for (int r = 0; r < 16; r++) braw_v[r] = draw_v[r] = 0;
+  const int bias_shift = a.aux.bias_f32 ? 0 : 16;
+  const int bias_es = a.aux.bias_f32 ? 4 : 2;
+#define AXL_AUX_ROW0(H_, Q0_, BP_, DP_)                                                              \
+  {                                                                                                  \
+    const int64_t head_ = hk * G + (H_), row_ = (Q0_) + 8 * g;                                       \
+    BP_ = a.aux.bias ? a.aux.bias + b * a.aux.bias_sb + head_ * a.aux.bias_sh + row_ * a.aux.bias_sr + \
+                           (int64_t)kpos * bias_es                                                   \
+                     : nullptr;                                                                      \
+    DP_ = a.aux.drop ? a.aux.drop + b * a.aux.drop_sb + head_ * a.aux.drop_sh + row_ * a.aux.drop_sr + kpos \
+                     : nullptr;                                                                      \
+  }
+#define AXL_AUX_LOAD(BP_, DP_, R_, BDST_, DDST_)                                                     \
+  {                                                                                                  \
+    const int64_t rr_ = 16 * ((R_) / 8) + ((R_) % 8);                                                \
+    if (BP_) {                                                                                       \
+      const char* e_ = (BP_) + rr_ * a.aux.bias_sr;                                                  \
+      BDST_[R_] = a.aux.bias_f32 ? *(const uint32_t*)e_ : (uint32_t)*(const uint16_t*)e_;            \
+    }                                                                                                \
+    if (DP_) DDST_[R_] = *((DP_) + rr_ * a.aux.drop_sr);                                             \
   }
 #define AXL_PACK_PAIR(PB_, DSB_, I_)                                    \
   {                                                                     \
@@ -249,21 +284,31 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
   static_assert(1 + NWR <= LD_SLOT0 - 1, "staging registers are written out before they are reloaded");
   TrFrag bfr_next[kAheadB];            // first stage-B fragments of the next iteration
   int q0_a = t_begin * Tile::BQ, q0_s = q0_a;  // first query of tiles j+2 and j+3
+  int h_a = 0, h_s = 0;                        // and their heads within the group
 
   if (total > 0) {
     AXL_LOAD_TILE()
     AXL_STORE_TILE(buf_b)
     AXL_ADVANCE()
-    const int q0_1 = (t_begin + pf_t) * Tile::BQ;
+    const int q0_1 = (t_begin + pf_t) * Tile::BQ, h_1 = pf_h;
     AXL_LOAD_TILE()
     AXL_STORE_TILE(buf_e)
     AXL_ADVANCE()
     q0_a = (t_begin + pf_t) * Tile::BQ;
+    h_a = pf_h;
     AXL_LOAD_TILE()
     AXL_STORE_TILE(buf_a)
     AXL_ADVANCE()
     q0_s = (t_begin + pf_t) * Tile::BQ;
+    h_s = pf_h;
     AXL_LOAD_TILE()                      // tile 3 stays in the staging registers
+    if constexpr (AUX) {                 // bias / dropout columns of tile 0
+      const char* bp_;
+      const uint8_t* dp_;
+      AXL_AUX_ROW0(0, t_begin * Tile::BQ, bp_, dp_)
+#pragma unroll
+      for (int r = 0; r < 16; r++) AXL_AUX_LOAD(bp_, dp_, r, braw_v, draw_v)
+    }
     wait_all_vmem();  // nothing issued before the loop is pending, stationary fragments included
     __syncthreads();
     // Pipeline fill: stage A and the elementwise stage of tile 0, stage A of tile 1.
@@ -280,6 +325,13 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
     AXL_STAGE_A_PLAIN(buf_e, s_e, dp_e)
     AXL_READ_STATS_PART(buf_e, 0, lse_v, del_v, seg_v)
     AXL_READ_STATS_PART(buf_e, 1, lse_v, del_v, seg_v)
+    if constexpr (AUX) {                 // ... and of tile 1, for the first iteration
+      const char* bp_;
+      const uint8_t* dp_;
+      AXL_AUX_ROW0(h_1, q0_1, bp_, dp_)
+#pragma unroll
+      for (int r = 0; r < 16; r++) AXL_AUX_LOAD(bp_, dp_, r, braw_v, draw_v)
+    }
     diff0 = (q0_1 + a.q_off + 8 * g) - kpos;  // query of r == 0 minus this lane's key
 #pragma unroll
     for (int i = 0; i < kAheadB; i++) AXL_B_READ_FROM(buf_b, bfr_next[i], i)
@@ -295,7 +347,15 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
     PackedOperand pb_n, dsb_n;           // tile j + 1, packed as its elements complete
     floatx4 lse_n[4], del_n[4];          // statistics of tile j + 2
     intx4 seg_n[4];
-    int q0_p = q0_s;
+    int q0_p = q0_s, h_p = h_s;
+    uint32_t braw_n[16], draw_n[16];     // bias / dropout columns of tile j + 2
+    const char* bias_t = nullptr;
+    const uint8_t* drop_t = nullptr;
+    if constexpr (AUX) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) braw_n[r] = draw_n[r] = 0;
+      AXL_AUX_ROW0(h_a, q0_a, bias_t, drop_t)
+    }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int n = 0; n < NS; n++) {
@@ -345,6 +405,10 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
       if (n == LD_SLOT0 - 1) {
         AXL_ADVANCE()
         q0_p = (t_begin + pf_t) * Tile::BQ;
+        h_p = pf_h;
+      }
+      if constexpr (AUX) {
+        if (n % ESTEP == 0) AXL_AUX_LOAD(bias_t, drop_t, n / ESTEP, braw_n, draw_n)
       }
       if (n >= LD_SLOT0 && n < LD_SLOT0 + 2 * Tile::CHUNKS) {
         const int w = n - LD_SLOT0, i = w / 2;
@@ -373,10 +437,21 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
       del_v[i] = del_n[i];
       if (HAS_SEG) seg_v[i] = seg_n[i];
     }
+    if constexpr (AUX) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        braw_v[r] = braw_n[r];
+        draw_v[r] = draw_n[r];
+      }
+    }
     diff0 = (q0_a + a.q_off + 8 * g) - kpos;
     q0_a = q0_s;
     q0_s = q0_p;
+    h_a = h_s;
+    h_s = h_p;
   }
+#undef AXL_AUX_ROW0
+#undef AXL_AUX_LOAD
 #undef AXL_READ_STATS_PART
 #undef AXL_ELEM
 #undef AXL_PACK_PAIR
@@ -399,16 +474,17 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
       w.p[0] = pack_bf16(dk_acc[dt][4 * rq + 0] * a.scale, dk_acc[dt][4 * rq + 1] * a.scale);
       w.p[1] = pack_bf16(dk_acc[dt][4 * rq + 2] * a.scale, dk_acc[dt][4 * rq + 3] * a.scale);
       *(uint2*)(dkp + 32 * dt + 8 * rq + 4 * g) = w.u;
-      w.p[0] = pack_bf16(dv_acc[dt][4 * rq + 0], dv_acc[dt][4 * rq + 1]);
-      w.p[1] = pack_bf16(dv_acc[dt][4 * rq + 2], dv_acc[dt][4 * rq + 3]);
+      const float vs = AUX ? a.aux.keep_scale : 1.0f;  // kept probabilities are P / (1 - rate)
+      w.p[0] = pack_bf16(dv_acc[dt][4 * rq + 0] * vs, dv_acc[dt][4 * rq + 1] * vs);
+      w.p[1] = pack_bf16(dv_acc[dt][4 * rq + 2] * vs, dv_acc[dt][4 * rq + 3] * vs);
       *(uint2*)(dvp + 32 * dt + 8 * rq + 4 * g) = w.u;
     }
 }
 
-template <int D, bool HAS_SEG>
+template <int D, bool HAS_SEG, bool AUX>
 static hipError_t launch_one(const BwdArgs& a, hipStream_t stream) {
   using Tile = DkvTile<D>;
-  auto kernel = flash_bwd_dkdv_bf16_kernel<D, HAS_SEG>;
+  auto kernel = flash_bwd_dkdv_bf16_kernel<D, HAS_SEG, AUX>;
   hipError_t err = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                                        Tile::LDS_BYTES);
   if (err != hipSuccess) return err;
@@ -417,10 +493,14 @@ static hipError_t launch_one(const BwdArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
-hipError_t launch_bwd_dkdv_bf16(const BwdArgs& a, int head_dim, hipStream_t stream) {
+hipError_t launch_bwd_dkdv_bf16(const BwdArgs& a, int head_dim, bool aux, hipStream_t stream) {
   const bool seg = a.seg != nullptr;
-  if (head_dim == 128) return seg ? launch_one<128, true>(a, stream) : launch_one<128, false>(a, stream);
-  return seg ? launch_one<64, true>(a, stream) : launch_one<64, false>(a, stream);
+  if (aux) {
+    if (head_dim == 128) return seg ? launch_one<128, true, true>(a, stream) : launch_one<128, false, true>(a, stream);
+    return seg ? launch_one<64, true, true>(a, stream) : launch_one<64, false, true>(a, stream);
+  }
+  if (head_dim == 128) return seg ? launch_one<128, true, false>(a, stream) : launch_one<128, false, false>(a, stream);
+  return seg ? launch_one<64, true, false>(a, stream) : launch_one<64, false, false>(a, stream);
 }
 
 }  // namespace axl

@@ -31,6 +31,7 @@ struct FwdArgs {
   float* lse;
   const int32_t* seg;
   const float* sink;  // [Hq] logit of the per-head attention sink, or nullptr
+  AuxArgs aux;        // dense bias / dropout mask (read only by the AUX instantiations)
   Strides3 qs, ks, vs, os;
   int B, T, S, Hq, Hkv;
   int mask_kind, window, q_off;
@@ -83,7 +84,7 @@ struct FwdTile {
   }
 };
 
-template <int D>
+template <int D, bool AUX>
 __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
   using Tile = FwdTile<D>;
   constexpr int KK = D / 16;  // MFMA k-steps over head_dim
@@ -123,6 +124,14 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
   const int t_begin = k_begin / Tile::BK;
   const int t_end = (k_end + Tile::BK - 1) / Tile::BK;
 
+  // Dense bias / dropout mask rows of this lane's query (AUX instantiation only).  The bias joins
+  // the raw logits as bias / scale, so the scale folded into the exponent applies to both.
+  const char* bias_row = nullptr;
+  const uint8_t* drop_row = nullptr;
+  if constexpr (AUX) {
+    if (a.aux.bias) bias_row = a.aux.bias + b * a.aux.bias_sb + h * a.aux.bias_sh + (int64_t)(q0 + l32) * a.aux.bias_sr;
+    if (a.aux.drop) drop_row = a.aux.drop + b * a.aux.drop_sb + h * a.aux.drop_sh + (int64_t)(q0 + l32) * a.aux.drop_sr;
+  }
   const int qpos = q0 + l32 + a.q_off;       // this lane's query position
   const int qpos_min = q0 + a.q_off, qpos_max = q0 + 31 + a.q_off;  // of the wavefront
   // Tiles this wavefront has to process (the others it only helps to load): [tw_begin, tw_end).
@@ -243,6 +252,38 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
     }
 
     // ---- masks of tile t.  Register r of sub-tile ks in lane group g is key k0 + 32ks + 16(r/8) + 8g + (r%8).
+    uint2 dm[2][2] = {};  // dropout bytes of the lane's 4 runs of 8 keys
+    if constexpr (AUX) {
+      if (bias_row) {
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+          for (int t8 = 0; t8 < 2; t8++) {
+            float bv[8];
+            load_bias<8>(bias_row, k0 + 32 * ks + 16 * t8 + 8 * g, a.aux.bias_f32, bv);
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+              s[ks][8 * t8 + j] = __builtin_fmaf(bv[j], a.aux.inv_scale, s[ks][8 * t8 + j]);
+          }
+      }
+      if (drop_row) {
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+          for (int t8 = 0; t8 < 2; t8++)
+            dm[ks][t8] = *(const uint2*)(drop_row + k0 + 32 * ks + 16 * t8 + 8 * g);
+      }
+    }
+    // Probability that enters P V: zero where the dropout mask says so (the row sum keeps it).
+    auto after_dropout = [&](int idx, float p) {
+      if constexpr (AUX) {
+        const int ks = idx / 16, r = idx % 16;
+        const unsigned w = (r % 8) < 4 ? dm[ks][r / 8].x : dm[ks][r / 8].y;
+        return ((w >> (8 * (r % 4))) & 0xffu) ? 0.f : p;
+      } else {
+        return p;
+      }
+    };
     bool need_mask = false;
     if (a.mask_kind != AXL_MASK_NONE) {
       need_mask = k0 + Tile::BK - 1 > qpos_min;
@@ -330,9 +371,10 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
         for (int e = 0; e < EPS; e++) {
           const int idx = n * EPS + e;
           const float p = fast_exp2(__builtin_fmaf(s[idx / 16][idx % 16], c, -mc));
-          s[idx / 16][idx % 16] = p;
           lsum += p;
-          if (idx % 2 == 1) pb.p[idx / 2] = pack_bf16(s[idx / 16][idx % 16 - 1], p);
+          const float pu = after_dropout(idx, p);
+          s[idx / 16][idx % 16] = pu;
+          if (idx % 2 == 1) pb.p[idx / 2] = pack_bf16(s[idx / 16][idx % 16 - 1], pu);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -340,9 +382,10 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
 #pragma unroll
       for (int idx = 0; idx < 32; idx++) {
         const float p = fast_exp2(__builtin_fmaf(s[idx / 16][idx % 16], c, -mc));
-        s[idx / 16][idx % 16] = p;
         lsum += p;
-        if (idx % 2 == 1) pb.p[idx / 2] = pack_bf16(s[idx / 16][idx % 16 - 1], p);
+        const float pu = after_dropout(idx, p);
+        s[idx / 16][idx % 16] = pu;
+        if (idx % 2 == 1) pb.p[idx / 2] = pack_bf16(s[idx / 16][idx % 16 - 1], pu);
       }
     }
     l_run += lsum;
@@ -378,7 +421,8 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
 
   // Epilogue: out = acc / l ; lse = m*scale + ln(l).
   const float l_tot = xor32_sum(l_run);
-  const float inv_l = l_tot > 0.f ? 1.0f / l_tot : 0.f;  // a row with no visible key yields zeros
+  float inv_l = l_tot > 0.f ? 1.0f / l_tot : 0.f;  // a row with no visible key yields zeros
+  if constexpr (AUX) inv_l *= a.aux.keep_scale;
   __bf16* op = (__bf16*)a.out + b * a.os.b + (int64_t)(q0 + l32) * a.os.s + h * a.os.h;
 #pragma unroll
   for (int dt = 0; dt < DT; dt++) {
@@ -457,6 +501,10 @@ __global__ __launch_bounds__(256) void flash_fwd_f32_kernel(const FwdArgs a) {
   const int qpos_min = q0 + a.q_off, qpos_max = q0 + 31 + a.q_off;
   const int seg_q = a.seg ? a.seg[(int64_t)b * a.T + q0 + l32] : 0;
   const int32_t* seg_k = a.seg ? a.seg + (int64_t)b * a.T : nullptr;
+  const char* bias_row = nullptr;
+  const uint8_t* drop_row = nullptr;
+  if (a.aux.bias) bias_row = a.aux.bias + b * a.aux.bias_sb + h * a.aux.bias_sh + (int64_t)(q0 + l32) * a.aux.bias_sr;
+  if (a.aux.drop) drop_row = a.aux.drop + b * a.aux.drop_sb + h * a.aux.drop_sh + (int64_t)(q0 + l32) * a.aux.drop_sr;
 
   floatx16 o[DT];
 #pragma unroll
@@ -499,6 +547,15 @@ __global__ __launch_bounds__(256) void flash_fwd_f32_kernel(const FwdArgs a) {
       s = __builtin_amdgcn_mfma_f32_32x32x2f32(k_row[2 * d2 + g], q_row[2 * d2 + g], s, 0, 0, 0);
     }
     // Register r of lane group g is key k0 + 8(r/4) + 4g + (r%4).
+    if (bias_row) {  // logits = scale * qk + bias: pre-divide so the common scale below applies
+#pragma unroll
+      for (int r4 = 0; r4 < 4; r4++) {
+        float bv[4];
+        load_bias<4>(bias_row, k0 + 8 * r4 + 4 * g, a.aux.bias_f32, bv);
+#pragma unroll
+        for (int j = 0; j < 4; j++) s[4 * r4 + j] += bv[j] * a.aux.inv_scale;
+      }
+    }
 #pragma unroll
     for (int r = 0; r < 16; r++) {
       const int kpos = k0 + 8 * (r / 4) + 4 * g + (r % 4);
@@ -524,6 +581,14 @@ __global__ __launch_bounds__(256) void flash_fwd_f32_kernel(const FwdArgs a) {
       lsum += s[r];
     }
     l_run = l_run * corr + lsum;
+    if (drop_row) {  // dropped probabilities leave P V but stay in the row sum
+#pragma unroll
+      for (int r4 = 0; r4 < 4; r4++) {
+        const unsigned w = *(const unsigned*)(drop_row + k0 + 8 * r4 + 4 * g);
+#pragma unroll
+        for (int j = 0; j < 4; j++) s[4 * r4 + j] = ((w >> (8 * j)) & 0xffu) ? 0.f : s[4 * r4 + j];
+      }
+    }
 #pragma unroll
     for (int i = 0; i < DT; i++)
 #pragma unroll
@@ -540,7 +605,7 @@ __global__ __launch_bounds__(256) void flash_fwd_f32_kernel(const FwdArgs a) {
   }
 
   const float l_tot = xor32_sum(l_run);
-  const float inv_l = l_tot > 0.f ? 1.0f / l_tot : 0.f;  // a row with no visible key yields zeros
+  const float inv_l = (l_tot > 0.f ? 1.0f / l_tot : 0.f) * a.aux.keep_scale;  // no visible key: zeros
   float* op = (float*)a.out + b * a.os.b + (int64_t)(q0 + l32) * a.os.s + h * a.os.h;
 #pragma unroll
   for (int dt = 0; dt < DT; dt++)
@@ -559,6 +624,8 @@ int launch_flash_fwd(const AxlFlashFwdParams& p, hipStream_t stream) {
   FwdArgs a;
   a.q = p.q; a.k = p.k; a.v = p.v; a.out = p.out; a.lse = p.lse; a.seg = p.segment_ids;
   a.sink = p.logit_sink;
+  a.aux = make_aux_args(p.aux, p.softmax_scale);
+  const bool aux = p.aux.bias || p.aux.dropout_mask;
   a.qs = to_s3(p.q_strides); a.ks = to_s3(p.k_strides); a.vs = to_s3(p.v_strides);
   a.os = to_s3(p.out_strides);
   a.B = p.batch; a.T = p.q_len; a.S = p.kv_len; a.Hq = p.num_q_heads; a.Hkv = p.num_kv_heads;
@@ -576,8 +643,13 @@ int launch_flash_fwd(const AxlFlashFwdParams& p, hipStream_t stream) {
     }                                                                                           \
   } while (0)
   if (p.dtype == AXL_BF16) {
-    if (p.head_dim == 128) AXL_LAUNCH_FWD(flash_fwd_bf16_kernel<128>, FwdTile<128>);
-    else AXL_LAUNCH_FWD(flash_fwd_bf16_kernel<64>, FwdTile<64>);
+    if (p.head_dim == 128) {
+      if (aux) AXL_LAUNCH_FWD((flash_fwd_bf16_kernel<128, true>), FwdTile<128>);
+      else AXL_LAUNCH_FWD((flash_fwd_bf16_kernel<128, false>), FwdTile<128>);
+    } else {
+      if (aux) AXL_LAUNCH_FWD((flash_fwd_bf16_kernel<64, true>), FwdTile<64>);
+      else AXL_LAUNCH_FWD((flash_fwd_bf16_kernel<64, false>), FwdTile<64>);
+    }
   } else {
     if (p.head_dim == 128) AXL_LAUNCH_FWD(flash_fwd_f32_kernel<128>, FwdTileF32<128>);
     else AXL_LAUNCH_FWD(flash_fwd_f32_kernel<64>, FwdTileF32<64>);

@@ -6,9 +6,13 @@ gpu_attention.py:250-287, custom VJP :428-430, :789) and the dispatch class
 the mathematics:
   * KV heads are never repeated in memory: the kernels read the shared kv head (the reference
     repeats, :975-976, and lets autodiff sum dK/dV back);
-  * the mask must be structured (none / causal / sliding window, optionally with segment ids): the
-    kernels evaluate it in closed form from block indices instead of tracing an arbitrary `mask_fn`
-    into a block map.  Anything else is reported as unsupported so the dispatch moves on.
+  * structured masks (none / causal / sliding window, optionally with segment ids) are evaluated
+    in closed form from block indices; any other `mask_fn` is materialised once as a dense 0 / -1e15
+    bias `[1,1,T,S]` (what `MaskFnAttentionBias.value()` is) and takes the dense-bias kernels,
+    instead of being traced into a block map;
+  * dropout masks are drawn with torch's generator, not JAX's PRNG: the kernels take the mask as an
+    input (as the Pallas kernel does, gpu_attention.py:374-385), so results agree with the reference
+    for a given mask, not for a given key.
 """
 
 from __future__ import annotations
@@ -27,6 +31,7 @@ from axlearn_amd.attention_bias import (
     SegmentIdAttentionBias,
     SlidingWindowAttentionBias,
     _SlidingWindowCausalMask,
+    bool_to_bias,
     causal_mask,
     split,
 )
@@ -76,7 +81,31 @@ def _pad_last(x: Tensor, width: int) -> Tensor:
     return x if x.shape[-1] == width else torch.nn.functional.pad(x, (0, width - x.shape[-1]))
 
 
-def _attend(query, key, value, segment_ids, softmax_scale, mask_kind, window, logit_sink=None):
+def get_dropout_mask(shape, *, prng_key, rate: float, device) -> Tensor:
+    """Bool mask of `shape`, True = dropped with probability `rate` (layers.py:140-142).
+
+    prng_key: a torch.Generator on `device`, or an int / integer tensor used as its seed."""
+    if isinstance(prng_key, torch.Generator):
+        gen = prng_key
+    else:
+        if prng_key is None:
+            raise ValueError("prng_key must be provided when dropout_rate > 0.")
+        seed = int(torch.as_tensor(prng_key).reshape(-1)[-1].item()) if not isinstance(prng_key, int) else prng_key
+        gen = torch.Generator(device=device)
+        gen.manual_seed(seed & 0x7FFFFFFFFFFFFFFF)
+    return torch.rand(shape, generator=gen, device=device, dtype=torch.float32) < rate
+
+
+def mask_fn_as_bias(mask_fn: MaskFn, q_len: int, kv_len: int, device, q_pos_offset: int = 0) -> Tensor:
+    """An arbitrary mask fn as the dense bias `[1,1,T,S]` it stands for (attention_bias.py:862-873)."""
+    qp = torch.arange(q_len, device=device)[:, None] + q_pos_offset
+    kp = torch.arange(kv_len, device=device)[None, :]
+    keep = torch.as_tensor(mask_fn(qp, kp), device=device).expand(q_len, kv_len)
+    return bool_to_bias(keep)[None, None].to(torch.float32)
+
+
+def _attend(query, key, value, segment_ids, softmax_scale, mask_kind, window, logit_sink=None,
+            bias=None, dropout_mask=None, dropout_rate=0.0):
     """Pads the head dim if needed and runs the differentiable kernel pair."""
     head_dim = query.shape[-1]
     width = padded_head_dim(head_dim)
@@ -84,7 +113,7 @@ def _attend(query, key, value, segment_ids, softmax_scale, mask_kind, window, lo
         raise NotImplementedError(f"{head_dim=} > 128 is not supported by the HIP kernels.")
     out = _FlashAttentionFn.apply(
         _pad_last(query, width), _pad_last(key, width), _pad_last(value, width), segment_ids,
-        softmax_scale, mask_kind, window, logit_sink,
+        softmax_scale, mask_kind, window, logit_sink, bias, dropout_mask, dropout_rate,
     )
     return out if width == head_dim else out[..., :head_dim]
 
@@ -93,13 +122,16 @@ class _FlashAttentionFn(torch.autograd.Function):
     """Forward = axl_flash_fwd (saves out and lse), backward = axl_flash_bwd."""
 
     @staticmethod
-    def forward(ctx, query, key, value, segment_ids, softmax_scale, mask_kind, window, logit_sink):
+    def forward(ctx, query, key, value, segment_ids, softmax_scale, mask_kind, window, logit_sink,
+                bias, dropout_mask, dropout_rate):
+        aux = dict(bias=bias, dropout_mask=dropout_mask, dropout_rate=dropout_rate)
         out, lse = ops.flash_fwd(
             query, key, value, softmax_scale=softmax_scale, mask_kind=mask_kind,
-            sliding_window=window, segment_ids=segment_ids, logit_sink=logit_sink,
+            sliding_window=window, segment_ids=segment_ids, logit_sink=logit_sink, **aux,
         )
         ctx.save_for_backward(query, key, value, out, lse, logit_sink)
         ctx.segment_ids = segment_ids
+        ctx.aux = aux  # not differentiated: the bias gets no gradient (gpu_attention.py:786)
         ctx.args = (softmax_scale, mask_kind, window)
         return out
 
@@ -111,10 +143,10 @@ class _FlashAttentionFn(torch.autograd.Function):
             d_out = d_out.contiguous()
         grads = ops.flash_bwd(
             query, key, value, out, lse, d_out, softmax_scale=softmax_scale, mask_kind=mask_kind,
-            sliding_window=window, segment_ids=ctx.segment_ids, logit_sink=logit_sink,
+            sliding_window=window, segment_ids=ctx.segment_ids, logit_sink=logit_sink, **ctx.aux,
         )
         d_sink = grads[3].to(logit_sink.dtype) if logit_sink is not None else None
-        return grads[0], grads[1], grads[2], None, None, None, None, d_sink
+        return grads[0], grads[1], grads[2], None, None, None, None, d_sink, None, None, None
 
 
 # pylint: disable-next=too-many-positional-arguments
@@ -139,22 +171,26 @@ def flash_attention(
     """Differentiable flash attention; same signature as gpu_attention.py:250-267.
 
     query [B,T,Hq,D]; key/value [B,S,Hkv,D] (Hkv may be smaller than Hq); segment_ids [B,T].
-    The Pallas/Triton tuning arguments (block_q .. debug) are accepted and ignored: tiling is fixed
-    by the HIP kernels.  Dense `bias` and dropout are not implemented by the kernels.
+    bias [B|1,Hq|1,T,S]: dense additive logit bias (no gradient).  dropout_rate > 0 draws a mask from
+    `prng_key` (see `get_dropout_mask`).  The Pallas/Triton tuning arguments (block_q .. debug) are
+    accepted and ignored: tiling is fixed by the HIP kernels.
     """
-    del prng_key, block_q, block_k, num_warps, num_stages, grid, debug
+    del block_q, block_k, num_warps, num_stages, grid, debug
     if interpret:
         raise NotImplementedError("The HIP kernels have no interpret mode; they only run on the GPU.")
-    if bias is not None:
-        raise NotImplementedError("Dense attention bias is not supported by the HIP kernels.")
-    if dropout_rate != 0.0:
-        raise NotImplementedError("Attention dropout is not supported by the HIP kernels.")
+    if not 0.0 <= dropout_rate < 1.0:
+        raise ValueError(f"Dropout rate must be in [0, 1). Got {dropout_rate=}")
     kind = classify_mask_fn(mask_fn)
-    if kind is None:
-        raise NotImplementedError(
-            "mask_fn must be None, causal_mask or sliding_window_causal_mask(w) for the HIP kernels."
-        )
-    return _attend(query, key, value, segment_ids, float(softmax_scale), kind[0], kind[1])
+    if kind is None:  # arbitrary mask fn: as a dense bias
+        dense = mask_fn_as_bias(mask_fn, query.shape[1], key.shape[1], query.device)
+        bias = dense if bias is None else bias.to(torch.float32) + dense
+        kind = (ops.MASK_NONE, 0)
+    dropout_mask = None
+    if dropout_rate > 0.0:
+        shape = (query.shape[0], query.shape[2], query.shape[1], key.shape[1])
+        dropout_mask = get_dropout_mask(shape, prng_key=prng_key, rate=dropout_rate, device=query.device)
+    return _attend(query, key, value, segment_ids, float(softmax_scale), kind[0], kind[1],
+                   bias=bias, dropout_mask=dropout_mask, dropout_rate=float(dropout_rate))
 
 
 class HipFlashAttention(BaseFlashAttention):
@@ -181,16 +217,14 @@ class HipFlashAttention(BaseFlashAttention):
         logit_sink = input_batch.get("logit_sink", None)
         if logit_sink is not None and not logit_sink.is_cuda:
             return self._log_unsupported("logit sink is not on the GPU.")
-        if self.cfg.dropout_rate != 0.0:
-            return self._log_unsupported("dropout is not supported.")
+        if not 0.0 <= self.cfg.dropout_rate < 1.0:
+            raise ValueError(f"Dropout rate must be in [0, 1). Got {self.cfg.dropout_rate=}")
+        if self.cfg.dropout_rate > 0.0 and input_batch.get("prng_key", None) is None:
+            return self._log_unsupported("dropout needs input_batch['prng_key'].")
         if not (self.cfg.softmax_scale > 0.0):
             return self._log_unsupported(f"{self.cfg.softmax_scale=} must be positive")
         bias: BaseAttentionBias = input_batch["bias"]
-        mask, segment_ids, explicit_bias = split(bias, MaskFnAttentionBias, SegmentIdAttentionBias)
-        if explicit_bias.has_value():
-            return self._log_unsupported("explicit (dense) bias is not supported.")
-        if classify_mask_bias(mask) is None:
-            return self._log_unsupported("mask_fn is neither causal nor sliding-window causal.")
+        _, segment_ids, _ = split(bias, MaskFnAttentionBias, SegmentIdAttentionBias)
         if segment_ids.has_value() and query.shape[1] != key.shape[1]:
             return self._log_unsupported("segment ids need identical query and key lengths.")
         if not query.is_cuda:
@@ -201,14 +235,24 @@ class HipFlashAttention(BaseFlashAttention):
         query, key, value = input_batch["query"], input_batch["key"], input_batch["value"]
         bias: BaseAttentionBias = input_batch["bias"]
         mask, segment_ids, explicit_bias = split(bias, MaskFnAttentionBias, SegmentIdAttentionBias)
-        if explicit_bias.has_value():
-            raise NotImplementedError("explicit bias")
+        dense = explicit_bias.value() if explicit_bias.has_value() else None  # [B|1,H|1,T,S]
         kind = classify_mask_bias(mask)
-        if kind is None:
-            raise NotImplementedError("unstructured mask_fn")
+        if kind is None:  # a mask fn the kernels have no closed form for: its dense value
+            mask_bias = mask.value().to(torch.float32)
+            dense = mask_bias if dense is None else dense.to(torch.float32) + mask_bias
+            kind = (ops.MASK_NONE, 0)
+        if dense is not None:
+            dense = dense.to(query.device)
         seg = get_segment_ids(query=query, key=key, segment_ids=segment_ids)
-        logging.info("HipFlashAttention: mask_kind=%d window=%d segment_ids=%s", kind[0], kind[1], seg is not None)
+        rate = float(self.cfg.dropout_rate)
+        dropout_mask = None
+        if rate > 0.0:
+            shape = (query.shape[0], query.shape[2], query.shape[1], key.shape[1])
+            dropout_mask = get_dropout_mask(shape, prng_key=input_batch.get("prng_key", None), rate=rate,
+                                            device=query.device)
+        logging.info("HipFlashAttention: mask_kind=%d window=%d segment_ids=%s dense_bias=%s dropout=%g",
+                     kind[0], kind[1], seg is not None, dense is not None, rate)
         return _attend(
             query, key, value, seg, float(self.cfg.softmax_scale), kind[0], kind[1],
-            input_batch.get("logit_sink", None),
+            input_batch.get("logit_sink", None), bias=dense, dropout_mask=dropout_mask, dropout_rate=rate,
         )

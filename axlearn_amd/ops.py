@@ -7,7 +7,7 @@ call. Inputs must be CUDA(ROCm) tensors; torch is used for device memory and str
 from __future__ import annotations
 
 import ctypes
-from typing import Optional
+from typing import Optional, Tuple
 
 import torch
 
@@ -50,6 +50,41 @@ def _sink(logit_sink: Optional[torch.Tensor], num_heads: int) -> Optional[torch.
     return logit_sink.detach().to(torch.float32).contiguous()
 
 
+def _aux(bias, dropout_mask, dropout_rate, b, hq, t, s) -> Tuple[_lib.AxlAttnAux, tuple]:
+    """Builds the AxlAttnAux block; returns it with the tensors it points at (keep them alive)."""
+    aux = _lib.AxlAttnAux()
+    keep = []
+    if bias is not None:
+        if bias.dim() != 4 or bias.shape[0] not in (1, b) or bias.shape[1] not in (1, hq) or tuple(bias.shape[2:]) != (t, s):
+            raise AxlError(_lib.AXL_ERR_INVALID_ARGUMENT, f"bias must be [{b}|1, {hq}|1, {t}, {s}], got {tuple(bias.shape)}")
+        if bias.dtype not in (torch.bfloat16, torch.float32):
+            bias = bias.to(torch.float32)
+        if bias.stride(-1) != 1:
+            bias = bias.contiguous()
+        keep.append(bias)
+        aux.bias = bias.data_ptr()
+        aux.bias_batch_stride = bias.stride(0) if bias.shape[0] > 1 else 0
+        aux.bias_head_stride = bias.stride(1) if bias.shape[1] > 1 else 0
+        aux.bias_row_stride = bias.stride(2)
+        aux.bias_dtype = _lib.dtype_code(bias.dtype)
+    if dropout_mask is not None:
+        if tuple(dropout_mask.shape) != (b, hq, t, s):
+            raise AxlError(_lib.AXL_ERR_INVALID_ARGUMENT, f"dropout_mask must be [{b}, {hq}, {t}, {s}]")
+        if dropout_mask.dtype == torch.bool:
+            dropout_mask = dropout_mask.view(torch.uint8) if dropout_mask.is_contiguous() else dropout_mask.to(torch.uint8)
+        if dropout_mask.dtype != torch.uint8:
+            raise AxlError(_lib.AXL_ERR_INVALID_ARGUMENT, "dropout_mask must be bool or uint8 (nonzero = dropped)")
+        if dropout_mask.stride(-1) != 1:
+            dropout_mask = dropout_mask.contiguous()
+        keep.append(dropout_mask)
+        aux.dropout_mask = dropout_mask.data_ptr()
+        aux.drop_batch_stride, aux.drop_head_stride, aux.drop_row_stride = dropout_mask.stride()[:3]
+        aux.dropout_rate = float(dropout_rate)
+    elif dropout_rate:
+        raise AxlError(_lib.AXL_ERR_INVALID_ARGUMENT, "dropout_rate needs a dropout_mask (the kernels draw no random numbers)")
+    return aux, tuple(keep)
+
+
 def _seg(segment_ids: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
     if segment_ids is None:
         return None
@@ -70,11 +105,16 @@ def flash_fwd(
     q_pos_offset: int = 0,
     return_lse: bool = True,
     logit_sink: Optional[torch.Tensor] = None,
+    bias: Optional[torch.Tensor] = None,
+    dropout_mask: Optional[torch.Tensor] = None,
+    dropout_rate: float = 0.0,
 ):
     """q [B,T,Hq,D], k/v [B,S,Hkv,D] -> (out [B,T,Hq,D], lse [B,Hq,T] fp32 or None).
 
-    logit_sink [Hq]: optional per-head sink logit (joins the softmax and lse, carries no value)."""
-    _require_cuda(q, k, v, segment_ids, logit_sink)
+    logit_sink [Hq]: optional per-head sink logit (joins the softmax and lse, carries no value).
+    bias [B|1,Hq|1,T,S] bf16/fp32: dense additive logit bias.  dropout_mask [B,Hq,T,S] bool/uint8
+    (True = dropped) with dropout_rate: kept probabilities are scaled by 1 / (1 - rate)."""
+    _require_cuda(q, k, v, segment_ids, logit_sink, bias, dropout_mask)
     lib = _lib.load()
     b, t, hq, d = q.shape
     s, hkv = k.shape[1], k.shape[2]
@@ -82,6 +122,7 @@ def flash_fwd(
     lse = torch.empty((b, hq, t), dtype=torch.float32, device=q.device) if return_lse else None
     seg = _seg(segment_ids)
     sink = _sink(logit_sink, hq)
+    aux, _keep = _aux(bias, dropout_mask, dropout_rate, b, hq, t, s)
     p = AxlFlashFwdParams(
         q=q.data_ptr(), k=k.data_ptr(), v=v.data_ptr(), out=out.data_ptr(), lse=_lib.ptr(lse),
         segment_ids=_lib.ptr(seg),
@@ -90,7 +131,7 @@ def flash_fwd(
         batch=b, q_len=t, kv_len=s, num_q_heads=hq, num_kv_heads=hkv, head_dim=d,
         dtype=_lib.dtype_code(q.dtype), mask_kind=mask_kind, sliding_window=int(sliding_window),
         q_pos_offset=int(q_pos_offset), softmax_scale=float(softmax_scale),
-        logit_sink=_lib.ptr(sink),
+        logit_sink=_lib.ptr(sink), aux=aux,
     )
     if k.dtype != q.dtype or v.dtype != q.dtype:
         raise AxlError(_lib.AXL_ERR_UNSUPPORTED, "q, k, v must share one dtype")
@@ -114,13 +155,18 @@ def flash_bwd(
     phases: int = 7,
     buffers=None,
     logit_sink: Optional[torch.Tensor] = None,
+    bias: Optional[torch.Tensor] = None,
+    dropout_mask: Optional[torch.Tensor] = None,
+    dropout_rate: float = 0.0,
 ):
     """Returns (dq [B,T,Hq,D], dk [B,S,Hkv,D], dv [B,S,Hkv,D]) in the dtype of q, followed by
     d_logit_sink [Hq] fp32 when `logit_sink` (the one the forward was given) is passed.
 
     `phases` selects a subset of {1: delta, 2: dK/dV, 4: dQ} (timing / profiling only); `buffers`
-    = (dq, dk, dv, workspace) reuses caller-provided outputs instead of allocating."""
-    _require_cuda(q, k, v, out, lse, d_out, segment_ids, logit_sink)
+    = (dq, dk, dv, workspace) reuses caller-provided outputs instead of allocating.  bias,
+    dropout_mask and dropout_rate must be the ones the forward was given (the bias gets no gradient,
+    as in gpu_attention.py:786)."""
+    _require_cuda(q, k, v, out, lse, d_out, segment_ids, logit_sink, bias, dropout_mask)
     lib = _lib.load()
     b, t, hq, d = q.shape
     s, hkv = k.shape[1], k.shape[2]
@@ -136,6 +182,7 @@ def flash_bwd(
         raise AxlError(_lib.AXL_ERR_INVALID_ARGUMENT, "lse must be contiguous float32 [B,Hq,T]")
     sink = _sink(logit_sink, hq)
     d_sink = torch.empty((hq,), dtype=torch.float32, device=q.device) if sink is not None else None
+    aux, _keep = _aux(bias, dropout_mask, dropout_rate, b, hq, t, s)
     p = AxlFlashBwdParams(
         q=q.data_ptr(), k=k.data_ptr(), v=v.data_ptr(), out=out.data_ptr(),
         d_out=d_out.data_ptr(), lse=lse.data_ptr(), dq=dq.data_ptr(), dk=dk.data_ptr(),
@@ -147,6 +194,7 @@ def flash_bwd(
         dtype=_lib.dtype_code(q.dtype), mask_kind=mask_kind, sliding_window=int(sliding_window),
         q_pos_offset=int(q_pos_offset), softmax_scale=float(softmax_scale),
         workspace=None, workspace_bytes=0, logit_sink=_lib.ptr(sink), d_logit_sink=_lib.ptr(d_sink),
+        aux=aux,
     )
     need = lib.axl_flash_bwd_workspace_bytes(ctypes.byref(p))
     if ws is None or ws.numel() * ws.element_size() < need:

@@ -33,6 +33,15 @@ Parity status of each function (what pins it, see tests/test_oracle.py):
   closed-form special cases (uniform V, causal row 0, GQA == MHA on repeated KV).
 * gradients: pinned by float64 central finite differences and by the independent analytic
   brute force in oracle/brute_force.c.
+* logit sink: pinned by rewriting the sink as one more key with a zero value row (an extra head-dim
+  coordinate carries sink / scale), which the sink-free functions and the C brute force evaluate,
+  gradients included; plus closed forms (equal logits, sigmoid for a single visible key).
+* dropout with a given mask: pinned by linearity in V (the output for mask M is the sum over keys j
+  of (1 - M[., j]) / (1 - rate) times the output for V with only row j kept) and by float64 finite
+  differences for the gradients.  The reference draws its masks with JAX's PRNG, which is not
+  reproduced here: parity is defined for a given mask.
+* dense bias: a bias that repeats the causal / segment mask as -1e15 entries must equal the
+  structured mask; a rank-one bias u_t + w_s is absorbed into augmented q / k coordinates.
 * `reconstruct_kv`: pinned by a pure-Python loop on tiny shapes.
 * `scatter_update_pages`: pinned by the element-wise loop the reference documents
   (paged_kv_cache.py:156-165) written out in pure Python, plus the round trip through
@@ -229,8 +238,14 @@ def reference_mha(
     row_block: int = 512,
     return_lse: bool = False,
     logit_sink: Optional[torch.Tensor] = None,
+    dropout_mask: Optional[torch.Tensor] = None,
+    dropout_rate: float = 0.0,
 ):
     """`ReferenceMHA.__call__` (flash_attention/common.py:492-519), query-row-blocked.
+
+    dropout_mask [B,Hq,T,S] bool (True = dropped) with dropout_rate: `dropout(probs, rate, mask)`
+    (flash_attention/common.py:512-518, layers.py:145-166) = where(mask, 0, probs) / (1 - rate),
+    applied to the finished probabilities; lse is unaffected.
 
     logit_sink [Hq]: `softmax_with_biases` (attention.py:608-626) prepends it to every row of head
     h's biased logits, takes the softmax over S+1 entries and drops the sink's column again, so the
@@ -299,6 +314,10 @@ def reference_mha(
         lse[:, :, t0:t1] = (m + torch.log(z)).squeeze(-1)
         if mode == "faithful":
             probs = _round_to(probs, in_dtype).to(cdt)
+        if dropout_mask is not None:
+            probs = torch.where(dropout_mask[:, :, t0:t1], torch.zeros_like(probs), probs) / (1.0 - dropout_rate)
+            if mode == "faithful":
+                probs = _round_to(probs, in_dtype).to(cdt)
         pb = probs.reshape(b, hkv, g, t1 - t0, s)
         ctx = torch.einsum("bkgts,bksd->btkgd", pb, vt).reshape(b, t1 - t0, hq, d)
         out[:, t0:t1] = ctx
@@ -320,6 +339,8 @@ def reference_mha_grads(
     row_block: int = 512,
     dtype=torch.float64,
     logit_sink: Optional[torch.Tensor] = None,
+    dropout_mask: Optional[torch.Tensor] = None,
+    dropout_rate: float = 0.0,
 ):
     """Gradients of `sum(reference_mha(q,k,v) * d_out)` w.r.t. q, k, v (and the logit sink, returned
     as a fourth tensor when one is given) by reverse-mode autodiff of the restatement above, in
@@ -349,6 +370,8 @@ def reference_mha_grads(
             probs = torch.softmax(torch.cat([col, logits], dim=-1), dim=-1)[..., 1:]
         else:
             probs = torch.softmax(logits, dim=-1)
+        if dropout_mask is not None:
+            probs = torch.where(dropout_mask[:, :, t0:t1], torch.zeros_like(probs), probs) / (1.0 - dropout_rate)
         probs = probs.reshape(b, hkv, g, t1 - t0, s)
         ctx = torch.einsum("bkgts,bksd->btkgd", probs, v.permute(0, 2, 1, 3)).reshape(b, t1 - t0, hq, d)
         (ctx * do[:, t0:t1]).sum().backward()

@@ -292,9 +292,16 @@ def test_dispatch_and_autograd_end_to_end():
     o2 = flash_attention(qd, kd, vd, segment_ids=segs.cuda(), softmax_scale=scale,
                          mask_fn=ab.sliding_window_causal_mask(64))
     assert torch.equal(o2, out)
-    # A dense bias is not something these kernels do: dispatch must decline, not guess.
-    dense = ab.CompositeAttentionBias([ab.TensorAttentionBias(torch.zeros(1, 1, t, t, device="cuda"))])
-    assert flash_attention_implementation("gpu", query=qd, key=kd, value=vd, bias=dense) is None
+    # A dense bias of zeros goes through the dense-bias kernels and changes nothing.
+    dense = ab.CompositeAttentionBias([
+        ab.SlidingWindowAttentionBias(ab.sliding_window_causal_mask(64), sliding_window_size=64, **pos),
+        ab.SegmentIdAttentionBias(segs.cuda()),
+        ab.TensorAttentionBias(torch.zeros(1, 1, t, t, device="cuda")),
+    ])
+    impl = flash_attention_implementation("gpu", query=qd, key=kd, value=vd, bias=dense, softmax_scale=scale)
+    assert impl is not None and isinstance(impl.fn, HipFlashAttention)
+    o3 = impl.fn(dict(query=qd, key=kd, value=vd, bias=dense))
+    assert ref.max_abs(o3.detach().cpu().float(), out.detach().cpu().float()) < 1e-2
 
 
 # ----------------------------------------------------------------------------- logit sink, head dims
@@ -388,6 +395,138 @@ def test_head_dims_between_the_compiled_widths(d):
     batch = dict(query=qd.detach(), key=kd.detach(), value=vd.detach(), bias=bias)
     assert fa.is_supported(batch, kv_cache_type=None)
     assert torch.equal(fa(batch), out.detach())
+
+
+# ----------------------------------------------------------------------------- dense bias, dropout
+
+
+def _dense_bias(seed, shape, dtype):
+    # Values of a few units, as relative-position biases have; a band of -1e15 entries as masks have.
+    g = torch.Generator().manual_seed(seed)
+    bias = torch.randn(shape, generator=g) * 2.0
+    t, s = shape[-2:]
+    band = (torch.arange(t)[:, None] - torch.arange(s)[None, :]).abs() % 37 == 5
+    return torch.where(band, torch.tensor(ref.NEG_INF), bias).to(dtype)
+
+
+AUX_CASES = [
+    # b, t, s, hq, hkv, d, dtype, mask, window, seg, bias shape (None = none), bias dtype, dropout rate
+    (2, 256, 256, 4, 2, 128, torch.bfloat16, "none", None, False, "bh", torch.bfloat16, 0.0),
+    (2, 256, 256, 4, 2, 128, torch.bfloat16, "causal", None, True, "1h", torch.float32, 0.0),
+    (1, 384, 384, 4, 4, 64, torch.bfloat16, "sliding", 100, False, "11", torch.float32, 0.0),
+    (2, 256, 256, 4, 2, 128, torch.bfloat16, "causal", None, False, None, None, 0.3),
+    (1, 384, 384, 6, 2, 64, torch.bfloat16, "none", None, True, None, None, 0.1),
+    (2, 256, 384, 4, 1, 128, torch.bfloat16, "none", None, False, "b1", torch.bfloat16, 0.2),
+    (1, 256, 256, 8, 2, 64, torch.bfloat16, "causal", None, True, "bh", torch.float32, 0.5),
+    (1, 256, 256, 2, 2, 64, torch.float32, "causal", None, False, "bh", torch.float32, 0.25),
+    (1, 128, 256, 2, 1, 128, torch.float32, "none", None, False, "1h", torch.bfloat16, 0.0),
+]
+
+
+@pytest.mark.parametrize("b,t,s,hq,hkv,d,dtype,mask,window,seg,bias_kind,bias_dtype,rate", AUX_CASES)
+def test_dense_bias_and_dropout_forward_and_backward(b, t, s, hq, hkv, d, dtype, mask, window, seg, bias_kind,
+                                                     bias_dtype, rate):
+    q, k, v, do = _inputs(b, t, hq, hkv, d, dtype, s=s)
+    segs = ref.packed_segment_ids(4, b, t, max_docs=4) if seg else None
+    spec, kw = _mask_args(mask, window, segs)
+    bias = None
+    if bias_kind is not None:
+        shape = (b if bias_kind[0] == "b" else 1, hq if bias_kind[1] == "h" else 1, t, s)
+        bias = _dense_bias(11, shape, bias_dtype)
+        spec.dense_bias = bias.float()
+    drop = None
+    if rate > 0:
+        drop = torch.rand((b, hq, t, s), generator=torch.Generator().manual_seed(12)) < rate
+    scale = d ** -0.5
+    okw = dict(softmax_scale=scale, dropout_mask=drop, dropout_rate=rate)
+    want, want_lse = ref.reference_mha(q, k, v, spec, return_lse=True, **okw)
+    gkw = dict(softmax_scale=scale, bias=None if bias is None else bias.cuda(),
+               dropout_mask=None if drop is None else drop.cuda(), dropout_rate=rate, **kw)
+    out, lse = ops.flash_fwd(q.cuda(), k.cuda(), v.cuda(), **gkw)
+    _assert_close("out", out, want, dtype)
+    assert ref.max_abs(lse.cpu(), want_lse) < (1e-5 if dtype == torch.float32 else 1e-3) * max(1.0, float(want_lse.abs().max()))
+    # The optional inputs must matter in this test.
+    plain, _ = ops.flash_fwd(q.cuda(), k.cuda(), v.cuda(), softmax_scale=scale, **kw)
+    assert ref.max_abs(plain.cpu(), want) > 0.05
+    if dtype != torch.bfloat16:
+        return  # the backward kernels are bf16 only
+    wq, wk, wv = ref.reference_mha_grads(q, k, v, do, spec, **okw)
+    dq, dk, dv = ops.flash_bwd(q.cuda(), k.cuda(), v.cuda(), out, lse, do.cuda(), **gkw)
+    _assert_close("dq", dq, wq, dtype)
+    _assert_close("dk", dk, wk, dtype)
+    _assert_close("dv", dv, wv, dtype)
+
+
+def test_dropout_mask_is_applied_exactly():
+    # Poison: a value row of 1e30 behind a dropped probability must leave no trace; dropping
+    # everything gives exact zeros with an untouched lse; dropping nothing at rate r is a rescale.
+    b, t, hq, hkv, d = 1, 256, 2, 1, 128
+    q, k, v, _ = _inputs(b, t, hq, hkv, d, torch.bfloat16)
+    drop = torch.zeros((b, hq, t, t), dtype=torch.bool)
+    drop[:, :, :, 77] = True
+    vp = v.clone()
+    vp[:, 77] = 1e30
+    kw = dict(softmax_scale=d ** -0.5, mask_kind=ops.MASK_CAUSAL, dropout_rate=0.5)
+    got, lse = ops.flash_fwd(q.cuda(), k.cuda(), vp.cuda(), dropout_mask=drop.cuda(), **kw)
+    want, _ = ops.flash_fwd(q.cuda(), k.cuda(), v.cuda(), dropout_mask=drop.cuda(), **kw)
+    assert torch.isfinite(got.float()).all() and torch.equal(got, want)
+    base, base_lse = ops.flash_fwd(q.cuda(), k.cuda(), v.cuda(), softmax_scale=d ** -0.5, mask_kind=ops.MASK_CAUSAL)
+    assert torch.equal(lse, base_lse)
+    zero, zlse = ops.flash_fwd(q.cuda(), k.cuda(), v.cuda(), dropout_mask=torch.ones_like(drop).cuda(), **kw)
+    assert zero.abs().max() == 0 and torch.equal(zlse, base_lse)
+    none, _ = ops.flash_fwd(q.cuda(), k.cuda(), v.cuda(), dropout_mask=torch.zeros_like(drop).cuda(), **kw)
+    assert ref.max_abs(none.cpu().float(), base.cpu().float() * 2) < 2e-2
+    # A bias of -1e15 on a column acts as a mask for that column (poison again), in fwd and bwd.
+    bias = torch.zeros((1, 1, t, t))
+    bias[..., 77] = ref.NEG_INF
+    got, lse = ops.flash_fwd(q.cuda(), k.cuda(), vp.cuda(), bias=bias.cuda(), softmax_scale=d ** -0.5)
+    assert torch.isfinite(got.float()).all()
+    do = ref.normal_tensor(5, (b, t, hq, d), torch.bfloat16).cuda()
+    dq, dk, dv = ops.flash_bwd(q.cuda(), k.cuda(), vp.cuda(), got, lse, do, bias=bias.cuda(), softmax_scale=d ** -0.5)
+    assert dk[:, 77].abs().max() == 0 and dv[:, 77].abs().max() == 0
+    assert all(torch.isfinite(x.float()).all() for x in (dq, dk, dv))
+
+
+def test_arbitrary_mask_fn_explicit_bias_and_dropout_through_dispatch():
+    b, t, hq, hkv, d = 2, 256, 4, 2, 64
+    q, k, v, do = _inputs(b, t, hq, hkv, d, torch.bfloat16)
+    qd, kd, vd = (x.cuda().requires_grad_(True) for x in (q, k, v))
+    scale = d ** -0.5
+
+    def strided_causal(qp, kp):  # not a mask the kernels have a closed form for
+        return (qp >= kp) & ((qp - kp) % 3 != 1)
+
+    rel = _dense_bias(21, (1, hq, t, t), torch.float32)
+    rel = torch.where(rel < -1e14, torch.zeros(()), rel)
+    pos = dict(target_positions=torch.arange(t)[None].cuda(), source_positions=torch.arange(t)[None].cuda())
+    bias = ab.CompositeAttentionBias([
+        ab.MaskFnAttentionBias(strided_causal, **pos),
+        ab.TensorAttentionBias(rel.cuda()),
+    ])
+    rate = 0.2
+    impl = flash_attention_implementation("gpu", query=qd, key=kd, value=vd, bias=bias, softmax_scale=scale,
+                                          dropout_rate=rate)
+    assert impl is None  # dropout without a prng_key cannot be served
+    fa = HipFlashAttention.default_config().set(softmax_scale=scale, dropout_rate=rate).instantiate()
+    batch = dict(query=qd, key=kd, value=vd, bias=bias, prng_key=1234)
+    assert fa.is_supported(batch, kv_cache_type=None)
+    out = fa(batch)
+    (out.float() * do.cuda().float()).sum().backward()
+    from axlearn_amd.flash_attention.hip_attention import get_dropout_mask
+    drop = get_dropout_mask((b, hq, t, t), prng_key=1234, rate=rate, device="cuda").cpu()
+    assert 0.15 < drop.float().mean() < 0.25
+    keep = strided_causal(torch.arange(t)[:, None], torch.arange(t)[None, :])
+    spec = ref.MaskSpec(dense_bias=rel + torch.where(keep, 0.0, ref.NEG_INF)[None, None])
+    okw = dict(softmax_scale=scale, dropout_mask=drop, dropout_rate=rate)
+    want = ref.reference_mha(q, k, v, spec, **okw)
+    wq, wk, wv = ref.reference_mha_grads(q, k, v, do, spec, **okw)
+    _assert_close("out", out, want, torch.bfloat16)
+    for name, got, exp in (("dq", qd.grad, wq), ("dk", kd.grad, wk), ("dv", vd.grad, wv)):
+        _assert_close(name, got, exp, torch.bfloat16)
+    # Function-level entry point: same mask fn, same key, same result.
+    o2 = flash_attention(qd, kd, vd, bias=rel.cuda(), softmax_scale=scale, mask_fn=strided_causal,
+                         dropout_rate=rate, prng_key=1234)
+    assert torch.equal(o2, out)
 
 
 # ----------------------------------------------------------------------------- BASELINE sizes

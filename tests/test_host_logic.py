@@ -226,15 +226,36 @@ def test_dispatch_tables_and_fallback():
 def test_entry_point_rejects_what_kernels_cannot_do():
     q = torch.zeros(1, 128, 1, 128, dtype=torch.bfloat16)
     with pytest.raises(NotImplementedError):
-        flash_attention(q, q, q, bias=torch.zeros(1, 1, 128, 128))
-    with pytest.raises(NotImplementedError):
-        flash_attention(q, q, q, dropout_rate=0.5)
-    with pytest.raises(NotImplementedError):
-        flash_attention(q, q, q, mask_fn=lambda a, b: a == b)
-    with pytest.raises(NotImplementedError):
         flash_attention(q, q, q, interpret=True)
+    with pytest.raises(ValueError, match="Dropout rate"):
+        flash_attention(q, q, q, dropout_rate=1.0)
+    with pytest.raises(ValueError, match="prng_key"):
+        flash_attention(q, q, q, dropout_rate=0.5)  # a mask cannot be drawn without a key
+    with pytest.raises(NotImplementedError, match="128"):
+        big = torch.zeros(1, 128, 1, 256, dtype=torch.bfloat16)
+        flash_attention(big, big, big)
+    # CPU tensors: there is no CPU path, whatever the optional inputs are.
     with pytest.raises(_lib.AxlError):
-        flash_attention(q, q, q)  # CPU tensors: there is no CPU path
+        flash_attention(q, q, q)
+    with pytest.raises(_lib.AxlError):
+        flash_attention(q, q, q, bias=torch.zeros(1, 1, 128, 128))
+    with pytest.raises(_lib.AxlError):
+        flash_attention(q, q, q, mask_fn=lambda a, b: a == b)
+
+
+def test_arbitrary_mask_fn_and_dropout_mask_helpers():
+    from axlearn_amd.flash_attention.hip_attention import get_dropout_mask, mask_fn_as_bias, padded_head_dim
+
+    bias = mask_fn_as_bias(lambda a, b: (a - b) % 3 == 0, 4, 5, "cpu", q_pos_offset=1)
+    assert bias.shape == (1, 1, 4, 5) and bias.dtype == torch.float32
+    want = torch.tensor([[(t + 1 - s) % 3 == 0 for s in range(5)] for t in range(4)])
+    assert torch.equal(bias[0, 0] == 0, want) and torch.equal(bias[0, 0] == ab.NEG_INF, ~want)
+    m1 = get_dropout_mask((2, 3, 8, 16), prng_key=7, rate=0.4, device="cpu")
+    m2 = get_dropout_mask((2, 3, 8, 16), prng_key=torch.tensor([0, 7]), rate=0.4, device="cpu")
+    m3 = get_dropout_mask((2, 3, 8, 16), prng_key=8, rate=0.4, device="cpu")
+    assert m1.dtype == torch.bool and torch.equal(m1, m2) and not torch.equal(m1, m3)
+    assert 0.25 < m1.float().mean() < 0.55
+    assert [padded_head_dim(d) for d in (8, 64, 65, 128, 129)] == [64, 64, 128, 128, None]
 
 
 def test_config_protocol():
@@ -270,7 +291,8 @@ def test_library_exports_every_declared_symbol():
 def test_struct_layouts_match_header():
     """Field order of the ctypes mirrors equals the order in the header."""
     text = open(os.path.join(ROOT, "include", "axl_attn.h")).read()
-    for cls in (_lib.AxlFlashFwdParams, _lib.AxlFlashBwdParams, _lib.AxlPagedDecodeParams, _lib.AxlDecodeParams):
+    for cls in (_lib.AxlAttnAux, _lib.AxlFlashFwdParams, _lib.AxlFlashBwdParams, _lib.AxlPagedDecodeParams,
+                _lib.AxlDecodeParams, _lib.AxlPageInsertParams):
         body = re.search(r"typedef struct %s \{(.*?)\} %s;" % (cls.__name__, cls.__name__), text, flags=re.S).group(1)
         body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
         names = []

@@ -275,6 +275,93 @@ def test_logit_sink_closed_forms():
     torch.testing.assert_close(lse[:, :, 0], torch.logaddexp(s00, sink.expand_as(s00)))
 
 
+# ------------------------------------------------------------------ dense bias, dropout
+
+
+def test_dense_bias_against_structured_masks_and_rank_one_form():
+    b, t, hq, hkv, d = 2, 10, 4, 2, 6
+    q, k, v = (torch.from_numpy(_rand(i, sh)) for i, sh in ((70, (b, t, hq, d)), (71, (b, t, hkv, d)), (72, (b, t, hkv, d))))
+    seg = torch.tensor([[1, 1, 1, 2, 2, 2, 2, 3, 3, 3], [5, 5, 5, 5, 5, 0, 0, 0, 0, 0]], dtype=torch.int32)
+    # The causal + segment mask written out as a dense bias of 0 / -1e15 entries.
+    keep = (torch.arange(t)[:, None] >= torch.arange(t)[None, :])[None] & (seg[:, :, None] == seg[:, None, :])
+    dense = torch.where(keep, 0.0, ref.NEG_INF)[:, None]
+    want = ref.reference_mha(q, k, v, ref.MaskSpec(causal=True, segment_ids=seg), softmax_scale=0.3)
+    got = ref.reference_mha(q, k, v, ref.MaskSpec(dense_bias=dense), softmax_scale=0.3)
+    torch.testing.assert_close(got, want, rtol=1e-12, atol=1e-12)
+    # A rank-one bias u[b,h,t] + w[b,h,s] is the product of two augmented coordinates:
+    # q' = [q, u/scale, 1/scale], k' = [k, 1, w]; needs one kv head per query head.
+    hq = hkv
+    q = q[:, :, :hkv]
+    # Dyadic values: the oracle carries biases in fp32 (attention.py:579), where these sums are exact.
+    u, w = np.round(_rand(73, (b, hq, t)) * 8) / 8, np.round(_rand(74, (b, hq, t)) * 8) / 8
+    bias = torch.from_numpy(u[:, :, :, None] + w[:, :, None, :])
+    scale = 0.3
+    got, lse = ref.reference_mha(q, k, v, ref.MaskSpec(dense_bias=bias), softmax_scale=scale, return_lse=True)
+    qa = np.concatenate([q.numpy(), u.transpose(0, 2, 1)[..., None] / scale, np.full((b, t, hq, 1), 1 / scale)], axis=-1)
+    ka = np.concatenate([k.numpy(), np.ones((b, t, hkv, 1)), w.transpose(0, 2, 1)[..., None]], axis=-1)
+    va = np.concatenate([v.numpy(), np.zeros((b, t, hkv, 2))], axis=-1)
+    bo, bl = brute.attention_fwd(qa, ka, va, scale=scale)
+    np.testing.assert_allclose(got.numpy(), bo[..., :d], rtol=1e-11, atol=1e-12)
+    np.testing.assert_allclose(lse.numpy(), bl, rtol=1e-11, atol=1e-12)
+
+
+def test_dropout_is_linear_in_the_value_rows():
+    b, t, s, hq, hkv, d = 1, 5, 7, 4, 2, 3
+    q, k, v = (torch.from_numpy(_rand(i, sh)) for i, sh in ((75, (b, t, hq, d)), (76, (b, s, hkv, d)), (77, (b, s, hkv, d))))
+    rate = 0.3
+    mask = torch.from_numpy(np.random.default_rng(78).random((b, hq, t, s)) < rate)
+    assert mask.any() and not mask.all()
+    got, lse = ref.reference_mha(q, k, v, softmax_scale=0.8, dropout_mask=mask, dropout_rate=rate, return_lse=True, row_block=2)
+    base, base_lse = ref.reference_mha(q, k, v, softmax_scale=0.8, return_lse=True)
+    torch.testing.assert_close(lse, base_lse)  # dropout acts after the softmax
+    want = torch.zeros_like(got)
+    for j in range(s):
+        vj = torch.zeros_like(v)
+        vj[:, j] = v[:, j]
+        oj = ref.reference_mha(q, k, vj, softmax_scale=0.8)  # P[., j] * v_j, undropped (pinned above)
+        keep = (~mask[:, :, :, j]).permute(0, 2, 1)[..., None].to(oj.dtype)  # [b, t, hq, 1]
+        want += keep * oj / (1 - rate)
+    torch.testing.assert_close(got, want, rtol=1e-12, atol=1e-12)
+    # Nothing dropped: a pure rescale.
+    none = ref.reference_mha(q, k, v, softmax_scale=0.8, dropout_mask=torch.zeros_like(mask), dropout_rate=rate)
+    torch.testing.assert_close(none, base / (1 - rate))
+
+
+def test_dropout_bias_sink_gradients_finite_differences():
+    b, t, hq, hkv, d = 1, 5, 2, 1, 3
+    rng = np.random.default_rng(79)
+    q, k, v, do = (rng.standard_normal(sh) for sh in ((b, t, hq, d), (b, t, hkv, d), (b, t, hkv, d), (b, t, hq, d)))
+    sink = rng.standard_normal(hq)
+    bias = torch.from_numpy(rng.standard_normal((1, hq, t, t)))
+    rate = 0.25
+    mask = torch.from_numpy(rng.random((b, hq, t, t)) < rate)
+    spec = ref.MaskSpec(causal=True, dense_bias=bias)
+    kw = dict(softmax_scale=0.6, dropout_mask=mask, dropout_rate=rate)
+
+    def loss(q_, k_, v_, s_):
+        out = ref.reference_mha(*(torch.from_numpy(x) for x in (q_, k_, v_)), spec, logit_sink=torch.from_numpy(s_), **kw)
+        return float((out * torch.from_numpy(do)).sum())
+
+    grads = ref.reference_mha_grads(*(torch.from_numpy(x) for x in (q, k, v, do)), spec,
+                                    logit_sink=torch.from_numpy(sink), row_block=2, **kw)
+    eps = 1e-6
+    args = [q, k, v, sink]
+    for i, name in enumerate(("q", "k", "v", "sink")):
+        x = args[i]
+        num = np.zeros_like(x)
+        it = np.nditer(x, flags=["multi_index"])
+        for _ in it:
+            idx = it.multi_index
+            old = x[idx]
+            x[idx] = old + eps
+            fp = loss(*args)
+            x[idx] = old - eps
+            fm = loss(*args)
+            x[idx] = old
+            num[idx] = (fp - fm) / (2 * eps)
+        np.testing.assert_allclose(grads[i].numpy(), num, rtol=1e-6, atol=1e-7, err_msg=name)
+
+
 # ------------------------------------------------------------------ paged KV / decode
 
 
