@@ -189,15 +189,13 @@ def test_is_supported_raises_on_illogical_shapes():
 def test_is_supported_returns_false_when_merely_unsupported(caplog):
     fa = HipFlashAttention.default_config().instantiate()
     assert not fa.is_supported(_batch(t=100, s=100), kv_cache_type=None)  # not a multiple of 128
-    assert not fa.is_supported(_batch(d=72), kv_cache_type=None)
     assert not fa.is_supported(_batch(dtype=torch.float16), kv_cache_type=None)
     assert not fa.is_supported(_batch(), kv_cache_type=KVCache)
-    dense = ab.CompositeAttentionBias([ab.TensorAttentionBias(torch.zeros(1, 1, 128, 128))])
-    assert not fa.is_supported(_batch(bias=dense), kv_cache_type=None)
-    sink = _batch()
-    sink["logit_sink"] = torch.zeros(4)
-    assert not fa.is_supported(sink, kv_cache_type=None)
+    assert not fa.is_supported(_batch(d=136), kv_cache_type=None)  # head_dim > 128, gpu_attention.py:954
+    # Dropout needs a key to draw the mask from; an impossible rate is an error, not "unsupported".
     assert not HipFlashAttention.default_config().set(dropout_rate=0.1).instantiate().is_supported(_batch(), None)
+    with pytest.raises(ValueError, match="Dropout rate"):
+        HipFlashAttention.default_config().set(dropout_rate=1.5).instantiate().is_supported(_batch(), None)
     # Everything fine except the tensors live on the CPU.
     assert not fa.is_supported(_batch(), kv_cache_type=None)
     assert fa.name() == "HipFlashAttention"
