@@ -20,7 +20,7 @@ MASK_NONE, MASK_CAUSAL, MASK_SLIDING_WINDOW = 0, 1, 2
 AXL_OK, AXL_ERR_INVALID_ARGUMENT, AXL_ERR_UNSUPPORTED, AXL_ERR_WORKSPACE, AXL_ERR_LAUNCH = 0, -1, -2, -3, -4
 
 
-ABI_VERSION = 3  # AXL_ATTN_ABI_VERSION of include/axl_attn.h these structures mirror
+ABI_VERSION = 4  # AXL_ATTN_ABI_VERSION of include/axl_attn.h these structures mirror
 
 
 class AxlError(RuntimeError):
@@ -61,6 +61,7 @@ class AxlFlashFwdParams(ctypes.Structure):
         ("softmax_scale", ctypes.c_float),
         ("logit_sink", ctypes.c_void_p),
         ("aux", AxlAttnAux),
+        ("q_pos_offsets", ctypes.c_void_p),
     ]
 
 

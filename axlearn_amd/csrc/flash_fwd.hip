@@ -31,6 +31,7 @@ struct FwdArgs {
   float* lse;
   const int32_t* seg;
   const float* sink;  // [Hq] logit of the per-head attention sink, or nullptr
+  const int32_t* q_offs;  // [B] per-sequence addition to q_off, or nullptr
   AuxArgs aux;        // dense bias / dropout mask (read only by the AUX instantiations)
   Strides3 qs, ks, vs, os;
   int B, T, S, Hq, Hkv;
@@ -100,6 +101,7 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
   int qb, b, h;
   decode_block(blockIdx.x, a.T / Tile::BQ, a.B, a.Hq, a.Hkv, qb, b, h);
   const int hk = h / (a.Hq / a.Hkv);
+  const int q_off = a.q_off + (a.q_offs ? a.q_offs[b] : 0);  // position of this sequence's query row 0
   const int q0_wg = qb * Tile::BQ;
   const int q0 = q0_wg + wave * 32;
 
@@ -115,8 +117,8 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
   // Visible key range of this workgroup.
   int k_begin = 0, k_end = a.S;
   if (a.mask_kind != AXL_MASK_NONE) {
-    k_end = min(a.S, q0_wg + Tile::BQ + a.q_off);
-    if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) k_begin = max(0, q0_wg + a.q_off - a.window);
+    k_end = min(a.S, q0_wg + Tile::BQ + q_off);
+    if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) k_begin = max(0, q0_wg + q_off - a.window);
   }
   const int seg_q = a.seg ? a.seg[(int64_t)b * a.T + q0 + l32] : 0;
   const int32_t* seg_k = a.seg ? a.seg + (int64_t)b * a.T : nullptr;
@@ -132,8 +134,8 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
     if (a.aux.bias) bias_row = a.aux.bias + b * a.aux.bias_sb + h * a.aux.bias_sh + (int64_t)(q0 + l32) * a.aux.bias_sr;
     if (a.aux.drop) drop_row = a.aux.drop + b * a.aux.drop_sb + h * a.aux.drop_sh + (int64_t)(q0 + l32) * a.aux.drop_sr;
   }
-  const int qpos = q0 + l32 + a.q_off;       // this lane's query position
-  const int qpos_min = q0 + a.q_off, qpos_max = q0 + 31 + a.q_off;  // of the wavefront
+  const int qpos = q0 + l32 + q_off;       // this lane's query position
+  const int qpos_min = q0 + q_off, qpos_max = q0 + 31 + q_off;  // of the wavefront
   // Tiles this wavefront has to process (the others it only helps to load): [tw_begin, tw_end).
   int tw_begin = t_begin, tw_end = t_end;
   if (a.mask_kind != AXL_MASK_NONE) {
@@ -475,6 +477,7 @@ __global__ __launch_bounds__(256) void flash_fwd_f32_kernel(const FwdArgs a) {
   int qb, b, h;
   decode_block(blockIdx.x, a.T / Tile::BQ, a.B, a.Hq, a.Hkv, qb, b, h);
   const int hk = h / (a.Hq / a.Hkv);
+  const int q_off = a.q_off + (a.q_offs ? a.q_offs[b] : 0);  // position of this sequence's query row 0
   const int q0_wg = qb * Tile::BQ;
   const int q0 = q0_wg + wave * 32;
 
@@ -492,13 +495,13 @@ __global__ __launch_bounds__(256) void flash_fwd_f32_kernel(const FwdArgs a) {
 
   int k_begin = 0, k_end = a.S;
   if (a.mask_kind != AXL_MASK_NONE) {
-    k_end = min(a.S, q0_wg + Tile::BQ + a.q_off);
-    if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) k_begin = max(0, q0_wg + a.q_off - a.window);
+    k_end = min(a.S, q0_wg + Tile::BQ + q_off);
+    if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) k_begin = max(0, q0_wg + q_off - a.window);
   }
   const int t_begin = k_begin / Tile::BK;
   const int t_end = (k_end + Tile::BK - 1) / Tile::BK;
-  const int qpos = q0 + l32 + a.q_off;
-  const int qpos_min = q0 + a.q_off, qpos_max = q0 + 31 + a.q_off;
+  const int qpos = q0 + l32 + q_off;
+  const int qpos_min = q0 + q_off, qpos_max = q0 + 31 + q_off;
   const int seg_q = a.seg ? a.seg[(int64_t)b * a.T + q0 + l32] : 0;
   const int32_t* seg_k = a.seg ? a.seg + (int64_t)b * a.T : nullptr;
   const char* bias_row = nullptr;
@@ -630,6 +633,7 @@ int launch_flash_fwd(const AxlFlashFwdParams& p, hipStream_t stream) {
   a.os = to_s3(p.out_strides);
   a.B = p.batch; a.T = p.q_len; a.S = p.kv_len; a.Hq = p.num_q_heads; a.Hkv = p.num_kv_heads;
   a.mask_kind = p.mask_kind; a.window = p.sliding_window; a.q_off = p.q_pos_offset;
+  a.q_offs = p.q_pos_offsets;
   a.scale = p.softmax_scale;
   const int grid = (p.q_len / 128) * p.batch * p.num_q_heads;
   hipError_t err = hipSuccess;

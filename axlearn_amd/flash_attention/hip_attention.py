@@ -35,8 +35,9 @@ from axlearn_amd.attention_bias import (
     causal_mask,
     split,
 )
+from axlearn_amd.config import config_class
 from axlearn_amd.flash_attention.common import BaseFlashAttention, Nested, Tensor, get_segment_ids
-from axlearn_amd.kv_cache import BaseKVCache
+from axlearn_amd.kv_cache import BaseKVCache, KVCache
 
 FLASH_ATTN_RESIDUAL_NAME = "flash_residuals"
 
@@ -105,7 +106,7 @@ def mask_fn_as_bias(mask_fn: MaskFn, q_len: int, kv_len: int, device, q_pos_offs
 
 
 def _attend(query, key, value, segment_ids, softmax_scale, mask_kind, window, logit_sink=None,
-            bias=None, dropout_mask=None, dropout_rate=0.0):
+            bias=None, dropout_mask=None, dropout_rate=0.0, save_residuals=True):
     """Pads the head dim if needed and runs the differentiable kernel pair."""
     head_dim = query.shape[-1]
     width = padded_head_dim(head_dim)
@@ -113,23 +114,31 @@ def _attend(query, key, value, segment_ids, softmax_scale, mask_kind, window, lo
         raise NotImplementedError(f"{head_dim=} > 128 is not supported by the HIP kernels.")
     out = _FlashAttentionFn.apply(
         _pad_last(query, width), _pad_last(key, width), _pad_last(value, width), segment_ids,
-        softmax_scale, mask_kind, window, logit_sink, bias, dropout_mask, dropout_rate,
+        softmax_scale, mask_kind, window, logit_sink, bias, dropout_mask, dropout_rate, save_residuals,
     )
     return out if width == head_dim else out[..., :head_dim]
 
 
 class _FlashAttentionFn(torch.autograd.Function):
-    """Forward = axl_flash_fwd (saves out and lse), backward = axl_flash_bwd."""
+    """Forward = axl_flash_fwd, backward = axl_flash_bwd.
+
+    The residuals (out, lse) are what the reference tags `flash_residuals` for its remat policies
+    (gpu_attention.py:423, remat.py:13-58).  With save_residuals=False they are not kept: the
+    backward re-runs the forward kernel on the saved q, k, v first, trading one forward pass for
+    [B,T,Hq,D] + [B,Hq,T] of memory, and produces bit-identical gradients."""
 
     @staticmethod
     def forward(ctx, query, key, value, segment_ids, softmax_scale, mask_kind, window, logit_sink,
-                bias, dropout_mask, dropout_rate):
+                bias, dropout_mask, dropout_rate, save_residuals):
         aux = dict(bias=bias, dropout_mask=dropout_mask, dropout_rate=dropout_rate)
         out, lse = ops.flash_fwd(
             query, key, value, softmax_scale=softmax_scale, mask_kind=mask_kind,
             sliding_window=window, segment_ids=segment_ids, logit_sink=logit_sink, **aux,
         )
-        ctx.save_for_backward(query, key, value, out, lse, logit_sink)
+        if save_residuals:
+            ctx.save_for_backward(query, key, value, out, lse, logit_sink)
+        else:
+            ctx.save_for_backward(query, key, value, None, None, logit_sink)
         ctx.segment_ids = segment_ids
         ctx.aux = aux  # not differentiated: the bias gets no gradient (gpu_attention.py:786)
         ctx.args = (softmax_scale, mask_kind, window)
@@ -139,6 +148,11 @@ class _FlashAttentionFn(torch.autograd.Function):
     def backward(ctx, d_out):
         query, key, value, out, lse, logit_sink = ctx.saved_tensors
         softmax_scale, mask_kind, window = ctx.args
+        if out is None:  # residuals were not saved: recompute them
+            out, lse = ops.flash_fwd(
+                query, key, value, softmax_scale=softmax_scale, mask_kind=mask_kind,
+                sliding_window=window, segment_ids=ctx.segment_ids, logit_sink=logit_sink, **ctx.aux,
+            )
         if d_out.stride(-1) != 1:
             d_out = d_out.contiguous()
         grads = ops.flash_bwd(
@@ -146,7 +160,7 @@ class _FlashAttentionFn(torch.autograd.Function):
             sliding_window=window, segment_ids=ctx.segment_ids, logit_sink=logit_sink, **ctx.aux,
         )
         d_sink = grads[3].to(logit_sink.dtype) if logit_sink is not None else None
-        return grads[0], grads[1], grads[2], None, None, None, None, d_sink, None, None, None
+        return grads[0], grads[1], grads[2], None, None, None, None, d_sink, None, None, None, None
 
 
 # pylint: disable-next=too-many-positional-arguments
@@ -197,16 +211,49 @@ class HipFlashAttention(BaseFlashAttention):
     """MI355X flash attention (forward + backward) behind the dispatch API.
 
     Takes the slot of `CuDNNGPUFlashAttention` / `PallasGPUFlashAttention`
-    (axlearn/common/flash_attention/utils.py:41-50)."""
+    (axlearn/common/flash_attention/utils.py:41-50).
+
+    With `kv_cache_type=KVCache` and more than one query row it serves incremental prefill: a chunk
+    of queries per sequence, each chunk sitting at its own offset into the (contiguous) cache, as
+    given by a causal / sliding-window bias with per-batch `target_positions`
+    (utils_test.py:361-478).  That mode is forward only."""
+
+    @config_class
+    class Config(BaseFlashAttention.Config):
+        # False: do not keep (out, lse) for the backward, recompute them there instead; the
+        # counterpart of leaving `flash_residuals` out of the remat policy's saved names.
+        save_residuals: bool = True
+
+    _kv_cache_type = None
+
+    def _incremental_supported(self, input_batch: Nested) -> bool:
+        query, key = input_batch["query"], input_batch["key"]
+        if key.shape[1] % 128 != 0:
+            return self._log_unsupported(f"{key.shape[1]=} is not divisible by 128")
+        if self.cfg.dropout_rate != 0.0:
+            raise ValueError("Dropout rate cannot be set for decoding!")
+        mask, segment_ids, explicit_bias = split(input_batch["bias"], MaskFnAttentionBias, SegmentIdAttentionBias)
+        if segment_ids.has_value() or explicit_bias.has_value():
+            return self._log_unsupported("incremental prefill takes a causal or sliding-window mask only.")
+        kind = classify_mask_bias(mask)
+        if kind is None or kind[0] == ops.MASK_NONE or getattr(mask, "target_positions", None) is None:
+            return self._log_unsupported("incremental prefill needs a causal / sliding-window mask with target_positions.")
+        if mask.target_positions.shape[1] != query.shape[1]:
+            return self._log_unsupported("target_positions do not match the query length.")
+        return True
 
     def is_supported(self, input_batch: Nested, kv_cache_type: Optional[type[BaseKVCache]]) -> bool:
         if not super().is_supported(input_batch=input_batch, kv_cache_type=kv_cache_type):
             return False
-        if kv_cache_type is not None:
-            return self._log_unsupported(f"{kv_cache_type=} (prefill/training kernel only)")
+        if kv_cache_type is not None and kv_cache_type != KVCache:
+            return self._log_unsupported(f"{kv_cache_type=}")
         query, key = input_batch["query"], input_batch["key"]
-        if not self._check_block_size(input_batch=input_batch, block_size=128):
+        if kv_cache_type == KVCache:
+            if not self._incremental_supported(input_batch):
+                return False
+        elif not self._check_block_size(input_batch=input_batch, block_size=128):
             return False
+        self._kv_cache_type = kv_cache_type
         head_dim = query.shape[-1]
         if padded_head_dim(head_dim) is None:  # same limit as gpu_attention.py:954
             return self._log_unsupported(f"{head_dim=} > 128")
@@ -231,7 +278,30 @@ class HipFlashAttention(BaseFlashAttention):
             return self._log_unsupported("tensors are not on the GPU.")
         return True
 
+    def _incremental_prefill(self, input_batch: Nested) -> Tensor:
+        """Queries at per-sequence offsets into the cache; rows padded up to the 128-row block."""
+        query, key, value = input_batch["query"], input_batch["key"], input_batch["value"]
+        mask, _, _ = split(input_batch["bias"], MaskFnAttentionBias, SegmentIdAttentionBias)
+        kind = classify_mask_bias(mask)
+        b, t, _, head_dim = query.shape
+        positions = mask.target_positions.to(query.device)
+        offsets = positions[:, 0].to(torch.int32).expand(b).contiguous()
+        consecutive = positions[:, :1] + torch.arange(t, device=query.device)[None]
+        if not torch.equal(positions, consecutive.to(positions.dtype)):
+            raise NotImplementedError("target_positions of a chunk must be consecutive.")
+        width = padded_head_dim(head_dim)
+        rows = -(-t // 128) * 128
+        q = torch.nn.functional.pad(query.detach(), (0, width - head_dim, 0, 0, 0, rows - t))
+        out, _ = ops.flash_fwd(
+            q, _pad_last(key.detach(), width), _pad_last(value.detach(), width),
+            softmax_scale=float(self.cfg.softmax_scale), mask_kind=kind[0], sliding_window=kind[1],
+            q_pos_offsets=offsets, logit_sink=input_batch.get("logit_sink", None), return_lse=False,
+        )
+        return out[:, :t, :, :head_dim]
+
     def __call__(self, input_batch: Nested) -> Tensor:
+        if self._kv_cache_type == KVCache:
+            return self._incremental_prefill(input_batch)
         query, key, value = input_batch["query"], input_batch["key"], input_batch["value"]
         bias: BaseAttentionBias = input_batch["bias"]
         mask, segment_ids, explicit_bias = split(bias, MaskFnAttentionBias, SegmentIdAttentionBias)
@@ -255,4 +325,5 @@ class HipFlashAttention(BaseFlashAttention):
         return _attend(
             query, key, value, seg, float(self.cfg.softmax_scale), kind[0], kind[1],
             input_batch.get("logit_sink", None), bias=dense, dropout_mask=dropout_mask, dropout_rate=rate,
+            save_residuals=bool(self.get_backend_overrides("save_residuals", self.cfg.save_residuals)),
         )

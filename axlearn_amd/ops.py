@@ -108,15 +108,21 @@ def flash_fwd(
     bias: Optional[torch.Tensor] = None,
     dropout_mask: Optional[torch.Tensor] = None,
     dropout_rate: float = 0.0,
+    q_pos_offsets: Optional[torch.Tensor] = None,
 ):
     """q [B,T,Hq,D], k/v [B,S,Hkv,D] -> (out [B,T,Hq,D], lse [B,Hq,T] fp32 or None).
 
+    q_pos_offsets [B] int32: per-sequence position of query row 0, added to q_pos_offset.
     logit_sink [Hq]: optional per-head sink logit (joins the softmax and lse, carries no value).
     bias [B|1,Hq|1,T,S] bf16/fp32: dense additive logit bias.  dropout_mask [B,Hq,T,S] bool/uint8
     (True = dropped) with dropout_rate: kept probabilities are scaled by 1 / (1 - rate)."""
-    _require_cuda(q, k, v, segment_ids, logit_sink, bias, dropout_mask)
+    _require_cuda(q, k, v, segment_ids, logit_sink, bias, dropout_mask, q_pos_offsets)
     lib = _lib.load()
     b, t, hq, d = q.shape
+    if q_pos_offsets is not None:
+        if tuple(q_pos_offsets.shape) != (b,):
+            raise AxlError(_lib.AXL_ERR_INVALID_ARGUMENT, f"q_pos_offsets must have shape [{b}]")
+        q_pos_offsets = q_pos_offsets.to(torch.int32).contiguous()
     s, hkv = k.shape[1], k.shape[2]
     out = torch.empty((b, t, hq, d), dtype=q.dtype, device=q.device)
     lse = torch.empty((b, hq, t), dtype=torch.float32, device=q.device) if return_lse else None
@@ -131,7 +137,7 @@ def flash_fwd(
         batch=b, q_len=t, kv_len=s, num_q_heads=hq, num_kv_heads=hkv, head_dim=d,
         dtype=_lib.dtype_code(q.dtype), mask_kind=mask_kind, sliding_window=int(sliding_window),
         q_pos_offset=int(q_pos_offset), softmax_scale=float(softmax_scale),
-        logit_sink=_lib.ptr(sink), aux=aux,
+        logit_sink=_lib.ptr(sink), aux=aux, q_pos_offsets=_lib.ptr(q_pos_offsets),
     )
     if k.dtype != q.dtype or v.dtype != q.dtype:
         raise AxlError(_lib.AXL_ERR_UNSUPPORTED, "q, k, v must share one dtype")

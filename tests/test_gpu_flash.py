@@ -529,6 +529,72 @@ def test_arbitrary_mask_fn_explicit_bias_and_dropout_through_dispatch():
     assert torch.equal(o2, out)
 
 
+# ----------------------------------------------------------------------------- incremental prefill, remat
+
+
+@pytest.mark.parametrize("bias_type", ["causal", "sliding"])
+@pytest.mark.parametrize("prefix_len", [[64] * 4, [32, 40, 48, 56]])
+@pytest.mark.parametrize("suffix_len", [16, 64, 160])
+def test_incremental_prefill_matches_full_forward(bias_type, prefix_len, suffix_len):
+    # The reference's test of the same name (utils_test.py:361-478): each sequence appends a chunk of
+    # queries after a prefix of its own length; the result must equal those rows of a full forward.
+    from axlearn_amd.kv_cache import KVCache
+
+    b, hq, hkv, d, kv_len = 4, 4, 2, 64, 256
+    q, k, v, _ = _inputs(b, kv_len, hq, hkv, d, torch.bfloat16)
+    prefix = torch.tensor(prefix_len)
+    window = 4
+
+    def make_bias(target_positions):
+        pos = dict(target_positions=target_positions.cuda(), source_positions=torch.arange(kv_len)[None].cuda())
+        if bias_type == "causal":
+            return ab.CompositeAttentionBias([ab.CausalAttentionBias(**pos)])
+        return ab.CompositeAttentionBias([
+            ab.SlidingWindowAttentionBias(ab.sliding_window_causal_mask(window), sliding_window_size=window, **pos)])
+
+    qc, kc, vc = q.cuda(), k.cuda(), v.cuda()
+    fwd_bias = make_bias(torch.arange(kv_len)[None].expand(b, kv_len))
+    fwd = flash_attention_implementation("gpu", query=qc, key=kc, value=vc, bias=fwd_bias)
+    fwd_out = fwd.fn(dict(query=qc, key=kc, value=vc, bias=fwd_bias))
+    incr_positions = torch.arange(suffix_len)[None] + prefix[:, None]
+    incr_bias = make_bias(incr_positions)
+    rows = incr_positions.cuda()[:, :, None, None].expand(b, suffix_len, hq, d)
+    suffix_q = torch.gather(qc, 1, rows)
+    incr = flash_attention_implementation("gpu", query=suffix_q, key=kc, value=vc, bias=incr_bias, kv_cache_type=KVCache)
+    assert incr is not None and isinstance(incr.fn, HipFlashAttention)
+    incr_out = incr.fn(dict(query=suffix_q, key=kc, value=vc, bias=incr_bias))
+    assert incr_out.shape == (b, suffix_len, hq, d)
+    assert torch.equal(incr_out, torch.gather(fwd_out, 1, rows))
+    # And against the oracle evaluated with the per-batch positions.
+    spec = ref.MaskSpec(causal=bias_type == "causal", sliding_window=window if bias_type == "sliding" else None,
+                        target_positions=incr_positions, source_positions=torch.arange(kv_len)[None])
+    want = ref.reference_mha(suffix_q.cpu(), k, v, spec)
+    _assert_close("incremental", incr_out, want, torch.bfloat16)
+
+
+def test_backward_without_saved_residuals_is_bit_identical():
+    b, t, hq, hkv, d = 2, 256, 4, 2, 128
+    q, k, v, do = _inputs(b, t, hq, hkv, d, torch.bfloat16)
+    pos = dict(target_positions=torch.arange(t)[None], source_positions=torch.arange(t)[None])
+    bias = ab.CompositeAttentionBias([ab.CausalAttentionBias(**pos)])
+    sink = torch.tensor([0.1, -0.4, 1.0, 0.0], device="cuda")
+    grads = []
+    for cfg in (dict(), dict(save_residuals=False), dict(backend_overrides=dict(save_residuals=False))):
+        qd, kd, vd = (x.cuda().requires_grad_(True) for x in (q, k, v))
+        sd = sink.clone().requires_grad_(True)
+        fa = HipFlashAttention.default_config().set(softmax_scale=d ** -0.5, **cfg).instantiate()
+        batch = dict(query=qd, key=kd, value=vd, bias=bias, logit_sink=sd)
+        assert fa.is_supported(batch, kv_cache_type=None)
+        out = fa(batch)
+        saved = [x for x in out.grad_fn.saved_tensors if x is not None]
+        assert len(saved) == (6 if not cfg else 4)  # q, k, v, sink (+ out, lse)
+        (out.float() * do.cuda().float()).sum().backward()
+        grads.append((out.detach(), qd.grad, kd.grad, vd.grad, sd.grad))
+    for other in grads[1:]:
+        for x, y in zip(grads[0], other):
+            assert torch.equal(x, y)
+
+
 # ----------------------------------------------------------------------------- BASELINE sizes
 
 

@@ -190,7 +190,8 @@ def test_is_supported_returns_false_when_merely_unsupported(caplog):
     fa = HipFlashAttention.default_config().instantiate()
     assert not fa.is_supported(_batch(t=100, s=100), kv_cache_type=None)  # not a multiple of 128
     assert not fa.is_supported(_batch(dtype=torch.float16), kv_cache_type=None)
-    assert not fa.is_supported(_batch(), kv_cache_type=KVCache)
+    assert not fa.is_supported(_batch(), kv_cache_type=PagedKVCache)
+    assert not fa.is_supported(_batch(s=100), kv_cache_type=KVCache)  # cache length not a multiple of 128
     assert not fa.is_supported(_batch(d=136), kv_cache_type=None)  # head_dim > 128, gpu_attention.py:954
     # Dropout needs a key to draw the mask from; an impossible rate is an error, not "unsupported".
     assert not HipFlashAttention.default_config().set(dropout_rate=0.1).instantiate().is_supported(_batch(), None)
