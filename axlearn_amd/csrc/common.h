@@ -107,6 +107,19 @@ __device__ __forceinline__ unsigned lds_address(const void* p) {
   return (unsigned)(uintptr_t)(__attribute__((address_space(3))) const char*)p;
 }
 
+// XOR swizzle of unpadded LDS tiles whose rows hold D bf16 (2D bytes).  Tiles that arrive by direct
+// global->LDS loads cannot be padded (an instruction writes 1 KB of consecutive LDS), so bank
+// conflicts are avoided by storing the 16-byte chunk c of row R at chunk index c ^ tile_swizzle(R):
+// each lane simply fetches the chunk that belongs at its slot.  The map is GF(2)-linear in the
+// row's low 4 bits and was found by exhaustive search with a bank simulator: conflict-free for
+// row-per-lane 128-bit reads in the row order swap_bits_2_3(lane) and for the transposing 64-bit
+// reads (ds_read_b64_tr_b16) alike, under a 32-bank and a 64-bank model.
+template <int D>
+__device__ __forceinline__ int tile_swizzle(int row) {
+  return D == 128 ? (((row & 1) ? 4 : 0) ^ ((row & 2) ? 10 : 0) ^ ((row & 4) ? 1 : 0) ^ ((row & 8) ? 3 : 0))
+                  : (((row & 1) ? 2 : 0) ^ ((row & 2) ? 4 : 0) ^ ((row & 4) ? 1 : 0) ^ ((row & 8) ? 3 : 0));
+}
+
 // Segment-id pruning of a workgroup's loop range.  `my_id` is the segment id of one of the rows the
 // workgroup owns (every owned row is passed by at least one thread); ids[lo, hi) are the segment ids
 // of the rows it loops over.  A looped row can only match an owned row if its id lies between the

@@ -12,7 +12,8 @@ struct BwdArgs {
   const void* out;
   const void* dout;
   const float* lse;
-  float* delta;  // workspace [B, Hq, T]
+  float* delta;  // workspace [B, Hq, T]: rowsum(out * dO)
+  float* lse2;   // workspace [B, Hq, T]: -lse * log2(e), the exponent offset of the dK/dV kernel
   void* dq;
   void* dk;
   void* dv;

@@ -24,6 +24,8 @@ namespace axl {
 
 // ---------------------------------------------------------------------------------------------
 // delta[b,h,t] = sum_d out[b,t,h,d] * dO[b,t,h,d]; 16 lanes per row, 16 bytes per lane per step.
+// Also leaves lse2 = -lse * log2(e) next to it: the dK/dV kernel streams both rows of statistics
+// into LDS with direct loads, which cannot scale on the way.
 // ---------------------------------------------------------------------------------------------
 template <typename T, int D>
 __global__ __launch_bounds__(256) void bwd_delta_kernel(const BwdArgs a) {
@@ -56,7 +58,11 @@ __global__ __launch_bounds__(256) void bwd_delta_kernel(const BwdArgs a) {
   acc += __shfl_xor(acc, 2, 64);
   acc += __shfl_xor(acc, 4, 64);
   acc += __shfl_xor(acc, 8, 64);
-  if (row < rows && sub == 0) a.delta[((int64_t)b * a.Hq + h) * a.T + t] = acc;
+  if (row < rows && sub == 0) {
+    const int64_t idx = ((int64_t)b * a.Hq + h) * a.T + t;
+    a.delta[idx] = acc;
+    a.lse2[idx] = a.lse[idx] * (-kLog2e);
+  }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -314,8 +320,8 @@ __global__ __launch_bounds__(256) void flash_bwd_dq_bf16_kernel(const BwdArgs a)
 static Strides3 to_s3(const AxlStrides& s) { return Strides3{s.batch, s.seq, s.head}; }
 
 size_t flash_bwd_workspace_bytes(const AxlFlashBwdParams& p) {
-  // delta [B, Hq, T] fp32.
-  return (size_t)p.batch * p.num_q_heads * p.q_len * sizeof(float);
+  // delta and lse2, [B, Hq, T] fp32 each.
+  return 2 * (size_t)p.batch * p.num_q_heads * p.q_len * sizeof(float);
 }
 
 int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream) {
@@ -324,6 +330,7 @@ int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream)
   BwdArgs a;
   a.q = p.q; a.k = p.k; a.v = p.v; a.out = p.out; a.dout = p.d_out; a.lse = p.lse;
   a.delta = (float*)p.workspace;
+  a.lse2 = a.delta + (size_t)p.batch * p.num_q_heads * p.q_len;
   a.dq = p.dq; a.dk = p.dk; a.dv = p.dv; a.seg = p.segment_ids;
   a.qs = to_s3(p.q_strides); a.ks = to_s3(p.k_strides); a.vs = to_s3(p.v_strides);
   a.os = to_s3(p.out_strides); a.dos = to_s3(p.d_out_strides); a.dqs = to_s3(p.dq_strides);

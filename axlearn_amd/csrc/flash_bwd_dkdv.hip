@@ -8,8 +8,10 @@
 // K and V fragments of 32 keys in registers (B operands) and the fp32 dK^T / dV^T accumulators of
 // those keys (128 registers), and loops over ALL query heads of the kv head's group and all query
 // tiles that can see the keys, so dK/dV need neither atomics nor a pass that sums repeated KV
-// heads.  Query tiles (32 rows of Q and dO plus their lse / delta / segment ids) stream through a
-// three-deep LDS ring.
+// heads.  Query tiles (32 rows of Q and dO plus their scaled lse / delta / segment ids) stream
+// through a five-deep LDS ring, filled by direct global->LDS loads: no staging registers and no LDS
+// store instructions, one unpadded XOR-swizzled copy per tile that serves both the row-per-lane
+// fragment reads of stage A and the transposing reads of stage B without bank conflicts.
 //
 // Register pressure allows one wavefront per SIMD, so nobody else can cover this wavefront's
 // latencies; the loop is software pipelined by hand instead.  Iteration j runs
@@ -28,19 +30,15 @@ template <int D>
 struct DkvTile {
   static constexpr int BKV = 128;            // keys per workgroup (32 per wavefront)
   static constexpr int BQ = 32;              // query rows per LDS tile
-  // Each tile is kept twice, with the row pitch that makes its access pattern bank-conflict free:
-  // +16 bytes for the row-per-lane 128-bit fragment reads of stage A, +64 bytes for the transposing
-  // reads of stage B (4 rows x 64 bytes per 32 lanes).
-  static constexpr int STRIDE = D * 2 + 16;     // copy read by stage A
-  static constexpr int TSTRIDE = D * 2 + 64;    // copy read by stage B
-  static constexpr int TILE_BYTES = BQ * STRIDE;
-  static constexpr int TTILE_BYTES = BQ * TSTRIDE;
-  static constexpr int TR_BASE = 2 * TILE_BYTES;                 // Q | dO (A copies), then Q | dO (B copies)
-  static constexpr int STAT_BASE = 2 * TILE_BYTES + 2 * TTILE_BYTES;
-  static constexpr int STAT_BYTES = 3 * BQ * 4;  // lse | delta | segment id per query row
+  static constexpr int ROWB = D * 2;         // bytes per row: unpadded, chunks swizzled (tile_swizzle)
+  static constexpr int TILE_BYTES = BQ * ROWB;                   // Q tile, then the dO tile
+  static constexpr int STAT_BASE = 2 * TILE_BYTES;
+  static constexpr int STAT_BYTES = 4 * BQ * 4;  // -lse*log2e | delta | segment id | (unused) per query row
   static constexpr int BUF_BYTES = STAT_BASE + STAT_BYTES;
-  static constexpr int NBUF = 4;
-  static constexpr int CHUNKS = BQ * D * 2 / 16 / 256;  // 16-byte chunks per thread per tensor
+  static constexpr int NBUF = 5;
+  static constexpr int RPI = 1024 / ROWB;                        // rows per direct-to-LDS instruction
+  static constexpr int DMA_PER_WAVE = BQ / 4 / RPI;              // per tensor per tile (8 rows per wavefront)
+  static constexpr int DMA_PER_TILE = 2 * DMA_PER_WAVE + 1;      // Q, dO and one row of statistics
   static constexpr int LDS_BYTES = NBUF * BUF_BYTES;
 };
 
@@ -55,7 +53,7 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
   const int tid = threadIdx.x;
-  const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l32 = lane & 31, g = lane >> 5;
   const int G = a.Hq / a.Hkv;
   // blockIdx -> (key block, batch, kv head); earliest key blocks (most queries under a causal
   // mask) first.
@@ -101,53 +99,48 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
     for (int r = 0; r < 16; r++) dk_acc[i][r] = dv_acc[i][r] = 0.f;
   const float c = a.scale * kLog2e;
 
-  // ---- global -> LDS staging through registers (plain unrolled code: arrays stay in registers).
-  u32x4 qreg[Tile::CHUNKS], dreg[Tile::CHUNKS], sreg = {0, 0, 0, 0};
-  const int st_row = tid / (D / 8), st_cc = tid % (D / 8);
-  constexpr int ROWS_PER_PASS = 256 / (D / 8);
-  const __bf16* const q_base = (const __bf16*)a.q + b * a.qs.b + (int64_t)st_row * a.qs.s + st_cc * 8;
-  const __bf16* const d_base = (const __bf16*)a.dout + b * a.dos.b + (int64_t)st_row * a.dos.s + st_cc * 8;
-  const int st_lds = st_row * Tile::STRIDE + st_cc * 16;
-  const int st_lds_t = Tile::TR_BASE + st_row * Tile::TSTRIDE + st_cc * 16;
-  // Row statistics travel with the tile: threads 0..7 fetch lse (stored pre-multiplied by -log2 e),
-  // 8..15 delta, 16..23 segment ids; the other threads re-read lse and store nothing.
-  const int st_kind = tid >> 3, st_part = tid & 7;
-  // Running per-thread source pointers of the prefetch cursor, advanced by wave-uniform steps: no
-  // 64-bit multiplies inside the loop.  Tile sequence: query head (outer) x query tile (inner).
-  const __bf16* q_src = q_base + (int64_t)(hk * G) * a.qs.h + (int64_t)t_begin * Tile::BQ * a.qs.s;
-  const __bf16* d_src = d_base + (int64_t)(hk * G) * a.dos.h + (int64_t)t_begin * Tile::BQ * a.dos.s;
-  const int64_t stat_row0 = ((int64_t)b * a.Hq + hk * G) * a.T + (int64_t)t_begin * Tile::BQ + 4 * st_part;
-  const char* s_src = st_kind == 1 ? (const char*)(a.delta + stat_row0) : (const char*)(a.lse + stat_row0);
-  if (HAS_SEG && st_kind == 2)
-    s_src = (const char*)(a.seg + (int64_t)b * a.T + (int64_t)t_begin * Tile::BQ + 4 * st_part);
+  // ---- tile loads: direct global->LDS, 1 KB (RPI rows) per instruction.  Wavefront w fetches rows
+  // 8w .. 8w+7 of the Q and of the dO tile; lane l fills chunk slot l % CPR of row l / CPR with the
+  // global chunk that the swizzle puts there.  Lanes 0..7 of wavefront w also fetch one row of
+  // statistics (4 query rows each): w = 0 the scaled lse, 1 delta, 2 the segment ids.
+  constexpr int CPR = D / 8;  // 16-byte chunks per row
+  int q_lane[Tile::DMA_PER_WAVE], d_lane[Tile::DMA_PER_WAVE];  // element offsets from the tile's first row
+#pragma unroll
+  for (int i = 0; i < Tile::DMA_PER_WAVE; i++) {
+    const int row = 8 * wave + Tile::RPI * i + lane / CPR;
+    const int chunk = (lane % CPR) ^ tile_swizzle<D>(row);
+    q_lane[i] = row * (int)a.qs.s + chunk * 8;
+    d_lane[i] = row * (int)a.dos.s + chunk * 8;
+  }
+  const int st_kind = wave;
+  // Running source pointers of the prefetch cursor, advanced by wave-uniform steps: no 64-bit
+  // multiplies inside the loop.  Tile sequence: query head (outer) x query tile (inner).
+  const __bf16* q_src = (const __bf16*)a.q + b * a.qs.b + (int64_t)(hk * G) * a.qs.h + (int64_t)t_begin * Tile::BQ * a.qs.s;
+  const __bf16* d_src = (const __bf16*)a.dout + b * a.dos.b + (int64_t)(hk * G) * a.dos.h + (int64_t)t_begin * Tile::BQ * a.dos.s;
+  const int64_t stat_row0 = ((int64_t)b * a.Hq + hk * G) * a.T + (int64_t)t_begin * Tile::BQ + 4 * (lane & 7);
   const bool s_is_seg = HAS_SEG && st_kind == 2;
+  const char* s_src = st_kind == 1 ? (const char*)(a.delta + stat_row0) : (const char*)(a.lse2 + stat_row0);
+  if (s_is_seg) s_src = (const char*)(a.seg + (int64_t)b * a.T + (int64_t)t_begin * Tile::BQ + 4 * (lane & 7));
   const int64_t q_step = (int64_t)Tile::BQ * a.qs.s, d_step = (int64_t)Tile::BQ * a.dos.s;
   const int64_t q_wrap = a.qs.h - (int64_t)(nt - 1) * q_step;    // last tile of a head -> first of next
   const int64_t d_wrap = a.dos.h - (int64_t)(nt - 1) * d_step;
   const int64_t s_step = Tile::BQ * 4, s_wrap = ((int64_t)a.T - (int64_t)(nt - 1) * Tile::BQ) * 4;
   const int64_t seg_wrap = -(int64_t)(nt - 1) * Tile::BQ * 4;   // segment ids do not depend on the head
-#define AXL_LOAD_TILE()                                                                           \
+  const unsigned lds0 = lds_address(smem);
+  // The k-th of the DMA_PER_TILE loads of the cursor's tile into the buffer at LDS address BUF_.
+#define AXL_DMA(BUF_, K_)                                                                          \
   {                                                                                               \
-    _Pragma("unroll") for (int i = 0; i < Tile::CHUNKS; i++) {                                    \
-      qreg[i] = *(const u32x4*)(q_src + (int64_t)(i * ROWS_PER_PASS) * a.qs.s);                   \
-      dreg[i] = *(const u32x4*)(d_src + (int64_t)(i * ROWS_PER_PASS) * a.dos.s);                  \
-    }                                                                                             \
-    sreg = *(const u32x4*)s_src;                                                                  \
+    if ((K_) < Tile::DMA_PER_WAVE)                                                                \
+      dma16(q_src + q_lane[(K_) % Tile::DMA_PER_WAVE], (BUF_) + wave * (8 * Tile::ROWB) + (K_) * 1024); \
+    else if ((K_) < 2 * Tile::DMA_PER_WAVE)                                                       \
+      dma16(d_src + d_lane[(K_) % Tile::DMA_PER_WAVE],                                            \
+            (BUF_) + Tile::TILE_BYTES + wave * (8 * Tile::ROWB) + ((K_) - Tile::DMA_PER_WAVE) * 1024); \
+    else if (lane < 8)                                                                            \
+      dma16(s_src, (BUF_) + Tile::STAT_BASE + st_kind * (Tile::BQ * 4));                          \
   }
-#define AXL_STORE_TILE(BUF_)                                                                      \
+#define AXL_DMA_TILE(BUF_)                                                                         \
   {                                                                                               \
-    _Pragma("unroll") for (int i = 0; i < Tile::CHUNKS; i++) {                                    \
-      *(u32x4*)((BUF_) + st_lds + i * ROWS_PER_PASS * Tile::STRIDE) = qreg[i];                    \
-      *(u32x4*)((BUF_) + Tile::TILE_BYTES + st_lds + i * ROWS_PER_PASS * Tile::STRIDE) = dreg[i]; \
-      *(u32x4*)((BUF_) + st_lds_t + i * ROWS_PER_PASS * Tile::TSTRIDE) = qreg[i];                 \
-      *(u32x4*)((BUF_) + Tile::TTILE_BYTES + st_lds_t + i * ROWS_PER_PASS * Tile::TSTRIDE) = dreg[i]; \
-    }                                                                                             \
-    if (tid < 24) {                                                                               \
-      union { u32x4 u; floatx4 f; } w_;                                                           \
-      w_.u = sreg;                                                                                \
-      if (st_kind == 0) w_.f = w_.f * (-kLog2e);                                                  \
-      *(u32x4*)((BUF_) + Tile::STAT_BASE + st_kind * (Tile::BQ * 4) + st_part * 16) = w_.u;       \
-    }                                                                                             \
+    _Pragma("unroll") for (int k_ = 0; k_ < Tile::DMA_PER_TILE; k_++) AXL_DMA(BUF_, k_)           \
   }
   // Prefetch cursor; it stops at the last tile (re-fetching that tile is harmless).
   int pf_idx = 0, pf_t = 0, pf_h = 0;  // tile number, query tile within the head, head within the group
@@ -166,19 +159,29 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
   char* buf_b = smem;                         // tile j     (stage B reads)
   char* buf_e = smem + Tile::BUF_BYTES;       // tile j + 1 (next stage B; its statistics are in registers)
   char* buf_a = smem + 2 * Tile::BUF_BYTES;   // tile j + 2 (stage A reads)
-  char* buf_s = smem + 3 * Tile::BUF_BYTES;   // tile j + 3 (being filled from the staging registers)
+  char* buf_n = smem + 3 * Tile::BUF_BYTES;   // tile j + 3 (requested one iteration ago, awaited at the end of this one)
+  char* buf_s = smem + 4 * Tile::BUF_BYTES;   // tile j + 4 (requested during this iteration)
 
-  const int a_row_off = swap_bits_2_3(l32) * Tile::STRIDE + g * 16;  // normal (row = query) reads
+  // Per-lane read offsets (bytes) into a swizzled tile.  Stage A: row swap_bits_2_3(l32), logical
+  // chunk 2kk + g.  Stage B (transposing reads): row 8g + j16/4 (+4 for the second half, +16 for the
+  // second group of 16 queries), logical byte column (16 half + 4 (j16 % 4)) * 2 + 64 dt.
+  const int a_row = swap_bits_2_3(l32);
+  const int a_row_off = a_row * Tile::ROWB;
+  const int a_xor = tile_swizzle<D>(a_row) << 4;
   const int j16 = lane & 15, half = (lane >> 4) & 1;
-  const int tr_off =
-      Tile::TR_BASE + (8 * g + (j16 >> 2)) * Tile::TSTRIDE + (16 * half + 4 * (j16 & 3)) * 2;
+  const int t_row = 8 * g + (j16 >> 2);
+  const int t_col = (16 * half + 4 * (j16 & 3)) * 2;
+  const int t_off0 = t_row * Tile::ROWB + (t_col & 15), t_off1 = t_off0 + 4 * Tile::ROWB;
+  const int t_xor0 = tile_swizzle<D>(t_row) << 4, t_xor1 = tile_swizzle<D>(t_row + 4) << 4;
+#define AXL_A_FRAG(BUF_, WHICH_, KK_) \
+  (*(const bf16x8*)((BUF_) + (WHICH_) * Tile::TILE_BYTES + a_row_off + ((((KK_) * 32) + g * 16) ^ a_xor)))
 
   // Three tiles are in flight: stage A (S = Q K^T, dP = dO V^T) of tile j+2, the elementwise stage
   // (P = exp2(S c - lse), dS = P (dP - delta)) of tile j+1 and stage B (dV^T += dO^T P,
-  // dK^T += Q^T dS) of tile j; tile j+3 is written to LDS from the staging registers and tile j+4
-  // is requested from memory.  Everything that is not an MFMA - elementwise arithmetic, operand
-  // packing, LDS fragment reads, LDS tile writes, global loads, pointer updates - is dealt out over
-  // the MFMA slots of the iteration, so the matrix pipe never waits for it.
+  // dK^T += Q^T dS) of tile j; tile j+3 is landing in LDS and tile j+4 is requested.  Everything
+  // that is not an MFMA - elementwise arithmetic, operand packing, LDS fragment reads, tile load
+  // requests, pointer updates - is dealt out over the MFMA slots of the iteration, so the matrix
+  // pipe never waits for it.
   floatx16 s_e, dp_e;          // tile j + 1: logits / dP, then P / dS
   union PackedOperand {
     bf16x8 v[2];
@@ -257,8 +260,8 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
   // Stage A of the tile in BUF_ into (S_, DP_), not interleaved with anything (pipeline fill).
 #define AXL_STAGE_A_PLAIN(BUF_, S_, DP_)                                                        \
   _Pragma("unroll") for (int kk = 0; kk < KK; kk++) {                                           \
-    const bf16x8 qa_ = *(const bf16x8*)((BUF_) + a_row_off + kk * 32);                          \
-    const bf16x8 da_ = *(const bf16x8*)((BUF_) + Tile::TILE_BYTES + a_row_off + kk * 32);       \
+    const bf16x8 qa_ = AXL_A_FRAG(BUF_, 0, kk);                                                 \
+    const bf16x8 da_ = AXL_A_FRAG(BUF_, 1, kk);                                                 \
     S_ = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa_, kf[kk], S_, 0, 0, 0);                     \
     DP_ = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da_, vf[kk], DP_, 0, 0, 0);                   \
   }
@@ -268,40 +271,39 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
   };
 #define AXL_B_READ_FROM(BUF_, DST_, N_)                                                          \
   {                                                                                              \
-    const char* p_ = (BUF_) + (((N_) % 2) == 0 ? Tile::TTILE_BYTES : 0) +                        \
-                     16 * ((N_) / (2 * DT)) * Tile::TSTRIDE + tr_off + (((N_) % (2 * DT)) / 2) * 64; \
-    DST_.hlf[0] = lds_read_tr16(p_);                                                             \
-    DST_.hlf[1] = lds_read_tr16(p_ + 4 * Tile::TSTRIDE);                                         \
+    const char* p_ = (BUF_) + (((N_) % 2) == 0 ? Tile::TILE_BYTES : 0) + 16 * ((N_) / (2 * DT)) * Tile::ROWB; \
+    const int col_ = (t_col & ~15) + (((N_) % (2 * DT)) / 2) * 64;                               \
+    DST_.hlf[0] = lds_read_tr16(p_ + t_off0 + (col_ ^ t_xor0));                                  \
+    DST_.hlf[1] = lds_read_tr16(p_ + t_off1 + (col_ ^ t_xor1));                                  \
   }
 
   constexpr int NS = NA + NB;          // MFMAs per iteration: stage B of tile j, then stage A of tile j+2
   constexpr int ESTEP = NS / 16;       // one of the 16 elements per lane every ESTEP slots
   static_assert(NS % 16 == 0, "the 16 elements per lane are spread evenly over the MFMA slots");
   constexpr int kAheadA = 6, kAheadB = 4;
-  constexpr int NWR = 4 * Tile::CHUNKS + 1;   // LDS writes of a tile per thread (two copies of Q and dO, statistics)
-  constexpr int NLD = 2 * Tile::CHUNKS + 1;   // global loads of a tile per thread
-  constexpr int LD_SLOT0 = NS - 2 - NLD;      // loads go in the last slots, writes in the first ones
-  static_assert(1 + NWR <= LD_SLOT0 - 1, "staging registers are written out before they are reloaded");
+  constexpr int NLD = Tile::DMA_PER_TILE;     // direct-to-LDS loads of a tile per wavefront
+  constexpr int LD_SLOT0 = 2;                 // one per slot from here on, after the cursor moved in slot 1
+  static_assert(LD_SLOT0 + NLD <= NS, "the loads of a tile fit into one iteration");
   TrFrag bfr_next[kAheadB];            // first stage-B fragments of the next iteration
   int q0_a = t_begin * Tile::BQ, q0_s = q0_a;  // first query of tiles j+2 and j+3
   int h_a = 0, h_s = 0;                        // and their heads within the group
 
   if (total > 0) {
-    AXL_LOAD_TILE()
-    AXL_STORE_TILE(buf_b)
+    // Everything the compiler tracks (stationary fragments, segment ids) has landed before the first
+    // untracked load, so its own wait counts never cover a tile load.
+    wait_all_vmem();
+    AXL_DMA_TILE(lds_address(buf_b))
     AXL_ADVANCE()
     const int q0_1 = (t_begin + pf_t) * Tile::BQ, h_1 = pf_h;
-    AXL_LOAD_TILE()
-    AXL_STORE_TILE(buf_e)
+    AXL_DMA_TILE(lds_address(buf_e))
     AXL_ADVANCE()
     q0_a = (t_begin + pf_t) * Tile::BQ;
     h_a = pf_h;
-    AXL_LOAD_TILE()
-    AXL_STORE_TILE(buf_a)
+    AXL_DMA_TILE(lds_address(buf_a))
     AXL_ADVANCE()
     q0_s = (t_begin + pf_t) * Tile::BQ;
     h_s = pf_h;
-    AXL_LOAD_TILE()                      // tile 3 stays in the staging registers
+    AXL_DMA_TILE(lds_address(buf_n))
     if constexpr (AUX) {                 // bias / dropout columns of tile 0
       const char* bp_;
       const uint8_t* dp_;
@@ -309,7 +311,7 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
 #pragma unroll
       for (int r = 0; r < 16; r++) AXL_AUX_LOAD(bp_, dp_, r, braw_v, draw_v)
     }
-    wait_all_vmem();  // nothing issued before the loop is pending, stationary fragments included
+    wait_all_vmem();  // tiles 0..3 have landed; nothing issued before the loop is pending
     __syncthreads();
     // Pipeline fill: stage A and the elementwise stage of tile 0, stage A of tile 1.
     AXL_STAGE_A_PLAIN(buf_b, s_e, dp_e)
@@ -348,6 +350,7 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
     floatx4 lse_n[4], del_n[4];          // statistics of tile j + 2
     intx4 seg_n[4];
     int q0_p = q0_s, h_p = h_s;
+    const unsigned lds_s = lds_address(buf_s);
     uint32_t braw_n[16], draw_n[16];     // bias / dropout columns of tile j + 2
     const char* bias_t = nullptr;
     const uint8_t* drop_t = nullptr;
@@ -363,7 +366,7 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
       if (n + kAheadB < NB) AXL_B_READ_FROM(buf_b, bfr[n + kAheadB], n + kAheadB)
       if (n + kAheadA >= NB && n + kAheadA - NB < NA) {
         const int x = n + kAheadA - NB;
-        afr[x] = *(const bf16x8*)(buf_a + (x % 2) * Tile::TILE_BYTES + a_row_off + (x / 2) * 32);
+        afr[x] = AXL_A_FRAG(buf_a, x % 2, x / 2);
       }
       if (n >= NS - kAheadB) AXL_B_READ_FROM(buf_e, bfr_next[n - (NS - kAheadB)], n - (NS - kAheadB))
       // ---- the MFMA of this slot.  Stage-B step m = t8 * 2DT + dt * 2 + which (which 0: dV with the
@@ -385,23 +388,7 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
       // ---- elementwise stage of tile j+1, one element every ESTEP slots, packed pairwise
       if (n % ESTEP == 0) AXL_ELEM(n / ESTEP)
       if (n % (2 * ESTEP) == 2 * ESTEP - 1) AXL_PACK_PAIR(pb_n, dsb_n, n / (2 * ESTEP))
-      // ---- tile j+3: staging registers -> LDS (both copies of Q and dO, then the statistics)
-      if (n >= 1 && n < 1 + 4 * Tile::CHUNKS) {
-        const int w = n - 1, i = w / 4;
-        if (w % 4 == 0) *(u32x4*)(buf_s + st_lds + i * ROWS_PER_PASS * Tile::STRIDE) = qreg[i];
-        if (w % 4 == 1) *(u32x4*)(buf_s + Tile::TILE_BYTES + st_lds + i * ROWS_PER_PASS * Tile::STRIDE) = dreg[i];
-        if (w % 4 == 2) *(u32x4*)(buf_s + st_lds_t + i * ROWS_PER_PASS * Tile::TSTRIDE) = qreg[i];
-        if (w % 4 == 3) *(u32x4*)(buf_s + Tile::TTILE_BYTES + st_lds_t + i * ROWS_PER_PASS * Tile::TSTRIDE) = dreg[i];
-      }
-      if (n == 1 + 4 * Tile::CHUNKS) {
-        if (tid < 24) {
-          union { u32x4 u; floatx4 f; } w_;
-          w_.u = sreg;
-          if (st_kind == 0) w_.f = w_.f * (-kLog2e);
-          *(u32x4*)(buf_s + Tile::STAT_BASE + st_kind * (Tile::BQ * 4) + st_part * 16) = w_.u;
-        }
-      }
-      // ---- tile j+4: advance the cursor, then one global load per slot
+      // ---- tile j+4: advance the cursor, then one direct-to-LDS load per slot
       if (n == LD_SLOT0 - 1) {
         AXL_ADVANCE()
         q0_p = (t_begin + pf_t) * Tile::BQ;
@@ -410,22 +397,24 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
       if constexpr (AUX) {
         if (n % ESTEP == 0) AXL_AUX_LOAD(bias_t, drop_t, n / ESTEP, braw_n, draw_n)
       }
-      if (n >= LD_SLOT0 && n < LD_SLOT0 + 2 * Tile::CHUNKS) {
-        const int w = n - LD_SLOT0, i = w / 2;
-        if (w % 2 == 0) qreg[i] = *(const u32x4*)(q_src + (int64_t)(i * ROWS_PER_PASS) * a.qs.s);
-        else dreg[i] = *(const u32x4*)(d_src + (int64_t)(i * ROWS_PER_PASS) * a.dos.s);
-      }
-      if (n == LD_SLOT0 + 2 * Tile::CHUNKS) sreg = *(const u32x4*)s_src;
+      if (n >= LD_SLOT0 && n < LD_SLOT0 + NLD) AXL_DMA(lds_s, n - LD_SLOT0)
       // ---- statistics of tile j+2 for the next iteration's elementwise stage
       if (n == NS / 2) AXL_READ_STATS_PART(buf_a, 0, lse_n, del_n, seg_n)
       if (n == NS / 2 + 1) AXL_READ_STATS_PART(buf_a, 1, lse_n, del_n, seg_n)
       __builtin_amdgcn_sched_barrier(0);
     }
+    // Tile j+3 (requested during the previous iteration) has landed once at most this iteration's
+    // loads are outstanding; after the barrier every wavefront's part of it is visible, and nobody
+    // reads tile j's buffer any more, which the next iteration refills.  (With a bias or a dropout
+    // mask, at least 27 of their element loads - 11 of the previous iteration, 16 of this one - are
+    // younger than tile j+3's loads as well; 24 leaves a margin.)
+    wait_vmem_le<NLD + (AUX ? 24 : 0)>();
     __syncthreads();
     char* const tmp = buf_b;
     buf_b = buf_e;
     buf_e = buf_a;
-    buf_a = buf_s;
+    buf_a = buf_n;
+    buf_n = buf_s;
     buf_s = tmp;
     s_e = s_a;
     dp_e = dp_a;
@@ -452,13 +441,18 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
   }
 #undef AXL_AUX_ROW0
 #undef AXL_AUX_LOAD
+  // The cursor re-requests the last tile during the final iterations (which keeps the count of
+  // outstanding loads the same in every iteration); none of those may still be in flight when this
+  // workgroup's LDS is handed to the next one.
+  wait_all_vmem();
 #undef AXL_READ_STATS_PART
 #undef AXL_ELEM
 #undef AXL_PACK_PAIR
 #undef AXL_STAGE_A_PLAIN
 #undef AXL_B_READ_FROM
-#undef AXL_LOAD_TILE
-#undef AXL_STORE_TILE
+#undef AXL_DMA
+#undef AXL_DMA_TILE
+#undef AXL_A_FRAG
 #undef AXL_ADVANCE
 
   __bf16* dkp = (__bf16*)a.dk + b * a.dks.b + (int64_t)(k0 + l32) * a.dks.s + hk * a.dks.h;

@@ -73,16 +73,8 @@ struct FwdTile {
   static constexpr int SEG_BASE = 4 * TILE_BYTES;            // {K, V} x double buffer, then the ids
   static constexpr int LDS_BYTES = SEG_BASE + NSEG * BK * 4;
   static constexpr int DMA_PER_WAVE = TILE_BYTES / 1024 / 4;  // direct-to-LDS loads per wavefront per tile
-  // Tiles arrive by direct global->LDS loads, which write 1 KB of consecutive LDS per instruction, so
-  // rows cannot be padded; bank conflicts are avoided by storing the 16-byte chunk c of row R at
-  // chunk index c ^ swz(R) instead (each lane simply fetches the chunk that belongs at its slot).
-  // swz is a GF(2)-linear map of the row's low 4 bits found by exhaustive search with a bank
-  // simulator: conflict-free for the row-per-lane 128-bit reads of K (row order swap_bits_2_3(lane))
-  // and for the transposing 64-bit reads of V, under a 32-bank and a 64-bank model alike.
-  __device__ static __forceinline__ int swz(int row) {
-    return D == 128 ? (((row & 1) ? 4 : 0) ^ ((row & 2) ? 10 : 0) ^ ((row & 4) ? 1 : 0) ^ ((row & 8) ? 3 : 0))
-                    : (((row & 1) ? 2 : 0) ^ ((row & 2) ? 4 : 0) ^ ((row & 4) ? 1 : 0) ^ ((row & 8) ? 3 : 0));
-  }
+  // Tiles arrive by direct global->LDS loads: unpadded rows, chunks XOR-swizzled (tile_swizzle).
+  __device__ static __forceinline__ int swz(int row) { return tile_swizzle<D>(row); }
 };
 
 template <int D, bool AUX>

@@ -216,7 +216,7 @@ def flash_bwd(
 def flash_bwd_buffers(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor):
     """Pre-allocates (dq, dk, dv, workspace) for repeated `flash_bwd(..., buffers=...)` calls."""
     b, t, hq, _ = q.shape
-    ws = torch.empty((b * hq * t * 4,), dtype=torch.uint8, device=q.device)
+    ws = torch.empty((2 * b * hq * t * 4,), dtype=torch.uint8, device=q.device)  # delta and scaled lse, fp32
     return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), ws
 
 

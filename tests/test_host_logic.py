@@ -339,7 +339,7 @@ def test_abi_validation_without_gpu():
                                 d_out_strides=s, dq_strides=s, dk_strides=s, dv_strides=s, batch=2, q_len=256,
                                 kv_len=256, num_q_heads=4, num_kv_heads=2, head_dim=128, dtype=0, mask_kind=1,
                                 sliding_window=0, q_pos_offset=0, softmax_scale=1.0, workspace=256, workspace_bytes=16)
-    assert lib.axl_flash_bwd_workspace_bytes(ctypes.byref(bp)) == 2 * 4 * 256 * 4
+    assert lib.axl_flash_bwd_workspace_bytes(ctypes.byref(bp)) == 2 * (2 * 4 * 256 * 4)  # delta and scaled lse
     assert lib.axl_flash_bwd(ctypes.byref(bp), None) == _lib.AXL_ERR_WORKSPACE
     assert lib.axl_flash_bwd_phases(ctypes.byref(bp), 0, None) == _lib.AXL_ERR_INVALID_ARGUMENT
     # Paged decode geometry.
