@@ -277,6 +277,23 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
     DST_.hlf[1] = lds_read_tr16(p_ + t_off1 + (col_ ^ t_xor1));                                  \
   }
 
+  // The same reads inside the loop, from per-lane offsets that are computed once: per iteration only
+  // the ring buffer's base is added (the Q / dO tile and the 16-row group are immediate offsets).
+  int a_off[KK], tb_off[2][DT];
+#pragma unroll
+  for (int kk = 0; kk < KK; kk++) a_off[kk] = a_row_off + ((kk * 32 + g * 16) ^ a_xor);
+#pragma unroll
+  for (int dt = 0; dt < DT; dt++) {
+    tb_off[0][dt] = t_off0 + (((t_col & ~15) + dt * 64) ^ t_xor0);
+    tb_off[1][dt] = t_off1 + (((t_col & ~15) + dt * 64) ^ t_xor1);
+  }
+#define AXL_B_READ_AT(AD_, DST_, N_)                                                             \
+  {                                                                                              \
+    const int imm_ = (((N_) % 2) == 0 ? Tile::TILE_BYTES : 0) + 16 * ((N_) / (2 * DT)) * Tile::ROWB;     \
+    DST_.hlf[0] = lds_read_tr16(AD_[0][((N_) % (2 * DT)) / 2] + imm_);                           \
+    DST_.hlf[1] = lds_read_tr16(AD_[1][((N_) % (2 * DT)) / 2] + imm_);                           \
+  }
+
   constexpr int NS = NA + NB;          // MFMAs per iteration: stage B of tile j, then stage A of tile j+2
   constexpr int ESTEP = NS / 16;       // one of the 16 elements per lane every ESTEP slots
   static_assert(NS % 16 == 0, "the 16 elements per lane are spread evenly over the MFMA slots");
@@ -351,6 +368,18 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
     intx4 seg_n[4];
     int q0_p = q0_s, h_p = h_s;
     const unsigned lds_s = lds_address(buf_s);
+    const char* a_ad[KK];                // this iteration's fragment addresses: stage A in tile j+2,
+    const char* b_ad[2][DT];             // stage B in tile j,
+    const char* e_ad[2][DT];             // and the first stage-B fragments of tile j+1
+#pragma unroll
+    for (int kk = 0; kk < KK; kk++) a_ad[kk] = buf_a + a_off[kk];
+#pragma unroll
+    for (int dt = 0; dt < DT; dt++) {
+      b_ad[0][dt] = buf_b + tb_off[0][dt];
+      b_ad[1][dt] = buf_b + tb_off[1][dt];
+      e_ad[0][dt] = buf_e + tb_off[0][dt];
+      e_ad[1][dt] = buf_e + tb_off[1][dt];
+    }
     uint32_t braw_n[16], draw_n[16];     // bias / dropout columns of tile j + 2
     const char* bias_t = nullptr;
     const uint8_t* drop_t = nullptr;
@@ -363,12 +392,12 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
 #pragma unroll
     for (int n = 0; n < NS; n++) {
       // ---- LDS fragments requested ahead of their MFMA
-      if (n + kAheadB < NB) AXL_B_READ_FROM(buf_b, bfr[n + kAheadB], n + kAheadB)
+      if (n + kAheadB < NB) AXL_B_READ_AT(b_ad, bfr[n + kAheadB], n + kAheadB)
       if (n + kAheadA >= NB && n + kAheadA - NB < NA) {
         const int x = n + kAheadA - NB;
-        afr[x] = AXL_A_FRAG(buf_a, x % 2, x / 2);
+        afr[x] = *(const bf16x8*)(a_ad[x / 2] + (x % 2) * Tile::TILE_BYTES);
       }
-      if (n >= NS - kAheadB) AXL_B_READ_FROM(buf_e, bfr_next[n - (NS - kAheadB)], n - (NS - kAheadB))
+      if (n >= NS - kAheadB) AXL_B_READ_AT(e_ad, bfr_next[n - (NS - kAheadB)], n - (NS - kAheadB))
       // ---- the MFMA of this slot.  Stage-B step m = t8 * 2DT + dt * 2 + which (which 0: dV with the
       // dO^T fragment and P, 1: dK with the Q^T fragment and dS); stage-A step x: even -> S chain
       // with Q fragment x/2, odd -> dP chain with dO fragment x/2.
@@ -450,6 +479,7 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
 #undef AXL_PACK_PAIR
 #undef AXL_STAGE_A_PLAIN
 #undef AXL_B_READ_FROM
+#undef AXL_B_READ_AT
 #undef AXL_DMA
 #undef AXL_DMA_TILE
 #undef AXL_A_FRAG
