@@ -29,4 +29,7 @@ struct BwdArgs {
 // reads the dense bias / dropout mask.
 hipError_t launch_bwd_dkdv_bf16(const BwdArgs& a, int head_dim, bool aux, hipStream_t stream);
 
+// Enqueues the dQ kernel (bf16, no dense bias / dropout mask) for head_dim 64 or 128.
+hipError_t launch_bwd_dq_bf16(const BwdArgs& a, int head_dim, hipStream_t stream);
+
 }  // namespace axl

@@ -359,12 +359,12 @@ int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream)
     if (phases & AXL_BWD_DELTA) AXL_LAUNCH((bwd_delta_kernel<__bf16, 128>), delta_grid, 0);
     if ((phases & AXL_BWD_DKDV) && err == hipSuccess) err = launch_bwd_dkdv_bf16(a, 128, aux, stream);
     if ((phases & AXL_BWD_DQ) && aux) AXL_LAUNCH((flash_bwd_dq_bf16_kernel<128, true>), dq_grid, DqTile<128>::LDS_BYTES);
-    if ((phases & AXL_BWD_DQ) && !aux) AXL_LAUNCH((flash_bwd_dq_bf16_kernel<128, false>), dq_grid, DqTile<128>::LDS_BYTES);
+    if ((phases & AXL_BWD_DQ) && !aux && err == hipSuccess) err = launch_bwd_dq_bf16(a, 128, stream);
   } else {
     if (phases & AXL_BWD_DELTA) AXL_LAUNCH((bwd_delta_kernel<__bf16, 64>), delta_grid, 0);
     if ((phases & AXL_BWD_DKDV) && err == hipSuccess) err = launch_bwd_dkdv_bf16(a, 64, aux, stream);
     if ((phases & AXL_BWD_DQ) && aux) AXL_LAUNCH((flash_bwd_dq_bf16_kernel<64, true>), dq_grid, DqTile<64>::LDS_BYTES);
-    if ((phases & AXL_BWD_DQ) && !aux) AXL_LAUNCH((flash_bwd_dq_bf16_kernel<64, false>), dq_grid, DqTile<64>::LDS_BYTES);
+    if ((phases & AXL_BWD_DQ) && !aux && err == hipSuccess) err = launch_bwd_dq_bf16(a, 64, stream);
   }
 #undef AXL_LAUNCH
   if ((phases & AXL_BWD_DELTA) && p.d_logit_sink && err == hipSuccess) {

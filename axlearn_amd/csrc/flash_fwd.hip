@@ -39,30 +39,6 @@ struct FwdArgs {
   float scale;
 };
 
-// Decodes blockIdx.x into (query block, batch, query head).  Heaviest query blocks (most visible
-// keys under a causal mask) are issued first; when the (batch, kv head) pairs divide evenly over
-// the 8 XCDs, all workgroups of a pair run on one XCD (workgroup i is dispatched to XCD i % 8).
-__device__ __forceinline__ void decode_block(int bid, int nqb, int B, int Hq, int Hkv, int& qb,
-                                             int& b, int& h) {
-  const int G = Hq / Hkv;
-  const int npairs = B * Hkv;
-  if (npairs % 8 == 0) {
-    const int xcd = bid & 7, slot = bid >> 3;
-    const int per_qb = (npairs >> 3) * G;
-    const int qb_rev = slot / per_qb, rem = slot % per_qb;
-    const int pair = xcd + 8 * (rem / G);
-    qb = nqb - 1 - qb_rev;
-    b = pair / Hkv;
-    h = (pair % Hkv) * G + rem % G;
-  } else {
-    const int per_qb = B * Hq;
-    const int qb_rev = bid / per_qb, rem = bid % per_qb;
-    qb = nqb - 1 - qb_rev;
-    b = rem / Hq;
-    h = rem % Hq;
-  }
-}
-
 template <int D>
 struct FwdTile {
   static constexpr int BQ = 128;              // query rows per workgroup
