@@ -96,6 +96,24 @@ __device__ __forceinline__ void dma16(const void* gsrc, unsigned lds_base) {
                : "v"(gsrc), "s"(lds_base)
                : "memory", "m0");
 }
+// Two such loads from one scalar base: lane l's two 16-byte pieces come from sbase + voff0 and
+// sbase + voff1_biased + 1024 (the instruction offset of the second load moves its global address
+// as well as its LDS address, so the caller passes the second offset minus 1024) and land at
+// lds_base + 16*l and lds_base + 1024 + 16*l.  No vector instruction forms an address.
+__device__ __forceinline__ void dma16x2(unsigned voff0, unsigned voff1_biased, const void* sbase, unsigned lds_base) {
+  asm volatile(
+      "s_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %2\n\tglobal_load_lds_dwordx4 %1, %2 offset:1024"
+      :
+      : "v"(voff0), "v"(voff1_biased), "s"(sbase), "s"(lds_base)
+      : "memory", "m0");
+}
+// One such load from a scalar base plus a per-lane byte offset.
+__device__ __forceinline__ void dma16s(unsigned voff, const void* sbase, unsigned lds_base) {
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :
+               : "v"(voff), "s"(sbase), "s"(lds_base)
+               : "memory", "m0");
+}
 #pragma clang diagnostic pop
 template <int N>
 __device__ __forceinline__ void wait_vmem_le() {

@@ -22,6 +22,8 @@
 // and the elementwise work of stage B is issued BETWEEN the MFMAs of stage A, one slice per MFMA, so
 // the VALU and the matrix pipe run at the same time.  Masks are evaluated arithmetically on every
 // tile (no branches inside the loop body: a branch would end the scheduling region).
+#include <type_traits>
+
 #include "flash_bwd.h"
 
 namespace axl {
@@ -207,25 +209,44 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
       SEG_[2 * (T8_) + 1] = *(const intx4*)(st_ + 2 * Tile::BQ * 4 + 64 * (T8_) + 16);  \
     }                                                                                   \
   }
-  // Elementwise stage of element R_ of (s_e, dp_e).
-#define AXL_ELEM(R_)                                                                           \
+  // Elementwise stage of element R_ of (s_e, dp_e) in three phases which the pipelined loop issues in
+  // three consecutive MFMA slots, so that no instruction waits for the result of the one before it
+  // (v_exp_f32 in particular has a long latency): exponent, exponential, products.  MASKED_ selects
+  // the mask arithmetic (tiles that no mask touches run without it).
+#define AXL_ELEM_1(R_, MASKED_)                                                                \
   {                                                                                            \
     const int r_ = (R_);                                                                       \
-    const unsigned diff_ = (unsigned)(diff0 + 16 * (r_ / 8) + (r_ % 8));                       \
-    float sv_ = diff_ <= limit ? s_e[r_] : kMasked;                                            \
-    if (HAS_SEG) sv_ = seg_v[r_ / 4][r_ % 4] == seg_k ? sv_ : kMasked;                         \
+    float sv_ = s_e[r_];                                                                       \
+    if (MASKED_) {                                                                             \
+      const unsigned diff_ = (unsigned)(diff0 + 16 * (r_ / 8) + (r_ % 8));                     \
+      sv_ = diff_ <= limit ? sv_ : kMasked;                                                    \
+      if (HAS_SEG) sv_ = seg_v[r_ / 4][r_ % 4] == seg_k ? sv_ : kMasked;                       \
+    }                                                                                          \
     float off_ = lse_v[r_ / 4][r_ % 4]; /* -lse * log2 e */                                    \
-    float dpv_ = dp_e[r_];                                                                     \
-    bool kept_ = true;                                                                         \
     if constexpr (AUX) {                                                                       \
       /* bias raw bits: fp32 as loaded, bf16 in the low half; zero when there is no bias */    \
       off_ = __builtin_fmaf(__builtin_bit_cast(float, braw_v[r_] << bias_shift), kLog2e, off_); \
-      kept_ = draw_v[r_] == 0;                                                                 \
-      dpv_ = kept_ ? dpv_ * a.aux.keep_scale : 0.f; /* gpu_attention.py:509-512 */            \
     }                                                                                          \
-    const float p_ = fast_exp2(__builtin_fmaf(sv_, c, off_));                                  \
-    s_e[r_] = kept_ ? p_ : 0.f; /* P that multiplies dO: dropped entries removed */            \
+    s_e[r_] = __builtin_fmaf(sv_, c, off_);                                                    \
+  }
+#define AXL_ELEM_2(R_) s_e[R_] = fast_exp2(s_e[R_]);
+#define AXL_ELEM_3(R_)                                                                         \
+  {                                                                                            \
+    const int r_ = (R_);                                                                       \
+    const float p_ = s_e[r_];                                                                  \
+    float dpv_ = dp_e[r_];                                                                     \
+    if constexpr (AUX) {                                                                       \
+      const bool kept_ = draw_v[r_] == 0;                                                      \
+      dpv_ = kept_ ? dpv_ * a.aux.keep_scale : 0.f; /* gpu_attention.py:509-512 */            \
+      s_e[r_] = kept_ ? p_ : 0.f; /* P that multiplies dO: dropped entries removed */          \
+    }                                                                                          \
     dp_e[r_] = p_ * (dpv_ - del_v[r_ / 4][r_ % 4]);                                            \
+  }
+#define AXL_ELEM(R_)                                                                           \
+  {                                                                                            \
+    AXL_ELEM_1(R_, true)                                                                       \
+    AXL_ELEM_2(R_)                                                                             \
+    AXL_ELEM_3(R_)                                                                             \
   }
   // Dense bias / dropout mask (AUX): this lane's key column of the 16 query rows of a tile, one
   // element per register, requested a whole iteration before the elementwise stage consumes it.
@@ -295,7 +316,7 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
   }
 
   constexpr int NS = NA + NB;          // MFMAs per iteration: stage B of tile j, then stage A of tile j+2
-  constexpr int ESTEP = NS / 16;       // one of the 16 elements per lane every ESTEP slots
+  constexpr int ESTEP = NS / 16;       // bias / dropout loads: one of the 16 elements per lane every ESTEP slots
   static_assert(NS % 16 == 0, "the 16 elements per lane are spread evenly over the MFMA slots");
   constexpr int kAheadA = 6, kAheadB = 4;
   constexpr int NLD = Tile::DMA_PER_TILE;     // direct-to-LDS loads of a tile per wavefront
@@ -357,7 +378,12 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
   }
 
   const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  for (int j = 0; j < total; j++) {
+  // Iterations [j_from, j_to); MASKED_C says whether their elementwise tiles (j + 1) need mask
+  // arithmetic.  The loop is instantiated once per run of iterations of one kind instead of branching
+  // inside one loop.
+  auto run = [&](int j_from, int j_to, auto masked_c) __attribute__((always_inline)) {
+    constexpr bool MASKED = decltype(masked_c)::value;
+  for (int j = j_from; j < j_to; j++) {
     bf16x8 afr[NA];
     TrFrag bfr[NB];
 #pragma unroll
@@ -414,9 +440,17 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
         else
           dp_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afr[x], vf[x / 2], x == 1 ? zero16 : dp_a, 0, 0, 0);
       }
-      // ---- elementwise stage of tile j+1, one element every ESTEP slots, packed pairwise
-      if (n % ESTEP == 0) AXL_ELEM(n / ESTEP)
-      if (n % (2 * ESTEP) == 2 * ESTEP - 1) AXL_PACK_PAIR(pb_n, dsb_n, n / (2 * ESTEP))
+      // ---- elementwise stage of tile j+1: element e starts in slot e (NS-3)/16 and takes three
+      // slots; pairs are packed one slot after their second element is complete
+#pragma unroll
+      for (int e = 0; e < 16; e++) {
+        if (e * (NS - 3) / 16 + 2 == n) AXL_ELEM_3(e)
+        if (e * (NS - 3) / 16 + 1 == n) AXL_ELEM_2(e)
+        if (e * (NS - 3) / 16 == n) AXL_ELEM_1(e, MASKED)
+      }
+#pragma unroll
+      for (int i = 0; i < 8; i++)
+        if ((2 * i + 1) * (NS - 3) / 16 + 3 == n) AXL_PACK_PAIR(pb_n, dsb_n, i)
       // ---- tile j+4: advance the cursor, then one direct-to-LDS load per slot
       if (n == LD_SLOT0 - 1) {
         AXL_ADVANCE()
@@ -468,6 +502,34 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
     h_a = h_s;
     h_s = h_p;
   }
+  };
+  // Tile t (within a head's run of nt tiles) needs no mask for this wavefront's 32 keys when its
+  // queries all see them: t in [u_lo, u_hi].  In processing order (head outer, tile inner) the
+  // elementwise tile of iteration j is e = j + 1.
+  auto floor_div = [](int x, int y) { return x >= 0 ? x / y : -((-x + y - 1) / y); };
+  int u_lo = 0, u_hi = nt - 1;
+  if (a.mask_kind != AXL_MASK_NONE) {
+    u_lo = max(0, floor_div(k0 + 31 - a.q_off + Tile::BQ - 1, Tile::BQ) - t_begin);
+    if (a.mask_kind == AXL_MASK_SLIDING_WINDOW)
+      u_hi = min(nt - 1, floor_div(a.window + k0 - 31 - a.q_off, Tile::BQ) - t_begin);
+  }
+  if (HAS_SEG || AUX) u_lo = nt;  // every tile takes the masked path
+  u_lo = min(u_lo, nt);
+  u_hi = max(u_hi, u_lo - 1);
+  {
+    int j = 0;
+    auto run_to = [&](int e_end, auto masked_c) __attribute__((always_inline)) {
+      const int j_end = min(total, e_end - 1);
+      run(j, j_end, masked_c);
+      j = max(j, j_end);
+    };
+    for (int hh = 0; hh < G; hh++) {
+      run_to(hh * nt + u_lo, std::true_type{});
+      run_to(hh * nt + u_hi + 1, std::false_type{});
+      run_to((hh + 1) * nt, std::true_type{});
+    }
+    run(j, total, std::true_type{});  // the last iteration (its elementwise tile is past the end)
+  }
 #undef AXL_AUX_ROW0
 #undef AXL_AUX_LOAD
   // The cursor re-requests the last tile during the final iterations (which keeps the count of
@@ -476,6 +538,9 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
   wait_all_vmem();
 #undef AXL_READ_STATS_PART
 #undef AXL_ELEM
+#undef AXL_ELEM_1
+#undef AXL_ELEM_2
+#undef AXL_ELEM_3
 #undef AXL_PACK_PAIR
 #undef AXL_STAGE_A_PLAIN
 #undef AXL_B_READ_FROM

@@ -25,9 +25,9 @@
 
 namespace axl {
 
-template <int D, bool HAS_SEG>
+template <int D, bool HAS_SEG, int NW>
 struct DqRing {
-  static constexpr int BQ = 128;             // query rows per workgroup (32 per wavefront)
+  static constexpr int BQ = 32 * NW;         // query rows per workgroup (32 per wavefront)
   static constexpr int BK = 64;              // keys per LDS tile (two sub-tiles of 32)
   static constexpr int ROWB = D * 2;         // bytes per row: unpadded, chunks swizzled (tile_swizzle)
   static constexpr int SUB_BYTES = 32 * ROWB;                    // one sub-tile of K or V
@@ -37,15 +37,15 @@ struct DqRing {
   static constexpr int BUF_BYTES = SEG_BASE + SEG_BYTES;
   static constexpr int NBUF = 4;
   static constexpr int RPI = 1024 / ROWB;                        // rows per direct-to-LDS instruction
-  static constexpr int DMA_PER_WAVE = BK / 4 / RPI;              // per tensor per tile (16 rows per wavefront)
+  static constexpr int DMA_PER_WAVE = BK / NW / RPI;             // per tensor per tile (BK / NW rows per wavefront)
   static constexpr int DMA_PER_TILE = 2 * DMA_PER_WAVE + (HAS_SEG ? 1 : 0);
   static constexpr int LDS_BYTES = NBUF * BUF_BYTES;
 };
 
-template <int D, bool HAS_SEG>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+template <int D, bool HAS_SEG, int NW>
+__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4, NW / 4)))
 void flash_bwd_dq_ring_kernel(const BwdArgs a) {
-  using Tile = DqRing<D, HAS_SEG>;
+  using Tile = DqRing<D, HAS_SEG, NW>;
   constexpr int KK = D / 16, DT = D / 32;
   constexpr int NA = 2 * KK;          // stage-A MFMAs per sub-tile
   constexpr int NB = 2 * DT;          // stage-B MFMAs per sub-tile
@@ -54,10 +54,13 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l32 = lane & 31, g = lane >> 5;
   int qb, b, h;
-  decode_block(blockIdx.x, a.T / Tile::BQ, a.B, a.Hq, a.Hkv, qb, b, h);
+  decode_block(blockIdx.x, (a.T + Tile::BQ - 1) / Tile::BQ, a.B, a.Hq, a.Hkv, qb, b, h);
   const int hk = h / (a.Hq / a.Hkv);
   const int q0_wg = qb * Tile::BQ;
-  const int q0 = q0_wg + wave * 32;  // this wavefront's queries
+  // This wavefront's queries.  T is a multiple of 128 but not necessarily of BQ: a wavefront past the
+  // end works on the last 32 rows instead (it still takes part in the tile loads) and stores nothing.
+  const bool live = q0_wg + wave * 32 < a.T;
+  const int q0 = live ? q0_wg + wave * 32 : a.T - 32;
 
   // Q and dO fragments (B operands): lane (query l32, k-group g) holds d = 16kk + 8g .. +7.
   const __bf16* qp = (const __bf16*)a.q + b * a.qs.b + (int64_t)(q0 + l32) * a.qs.s + h * a.qs.h;
@@ -104,34 +107,48 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
   // global chunk that the swizzle puts there.  Lanes 0..15 also fetch the 64 segment ids of the keys
   // (every wavefront issues that same load, so all wavefronts count the same loads in flight).
   constexpr int CPR = D / 8;  // 16-byte chunks per row
-  constexpr int ROWS_PER_WAVE = Tile::BK / 4;
-  int k_lane[Tile::DMA_PER_WAVE], v_lane[Tile::DMA_PER_WAVE];  // element offsets from the tile's first row
+  constexpr int ROWS_PER_WAVE = Tile::BK / NW;
+  constexpr bool PAIRS = Tile::DMA_PER_WAVE % 2 == 0;  // tile loads are issued in pairs when there are several
+  unsigned k_lane[Tile::DMA_PER_WAVE], v_lane[Tile::DMA_PER_WAVE];  // byte offsets from the tile's first row
 #pragma unroll
   for (int i = 0; i < Tile::DMA_PER_WAVE; i++) {
     const int row = ROWS_PER_WAVE * wave + Tile::RPI * i + lane / CPR;
     const int chunk = (lane % CPR) ^ tile_swizzle<D>(row);
-    k_lane[i] = row * (int)a.ks.s + chunk * 8;
-    v_lane[i] = row * (int)a.vs.s + chunk * 8;
+    // the second load of a pair carries an instruction offset of 1024, which also moves its source
+    k_lane[i] = (unsigned)(row * (int)a.ks.s + chunk * 8) * 2 - (PAIRS ? (i % 2) * 1024 : 0);
+    v_lane[i] = (unsigned)(row * (int)a.vs.s + chunk * 8) * 2 - (PAIRS ? (i % 2) * 1024 : 0);
   }
   const __bf16* k_src = (const __bf16*)a.k + b * a.ks.b + hk * a.ks.h + (int64_t)key0 * a.ks.s;
   const __bf16* v_src = (const __bf16*)a.v + b * a.vs.b + hk * a.vs.h + (int64_t)key0 * a.vs.s;
   const int32_t* s_src = HAS_SEG ? a.seg + (int64_t)b * a.T + key0 + 4 * (lane & 15) : nullptr;
   const int64_t k_step = (int64_t)Tile::BK * a.ks.s, v_step = (int64_t)Tile::BK * a.vs.s;
-  // The k-th of the DMA_PER_TILE loads of the cursor's tile into the buffer at LDS address BUF_.
+  // The k-th group of loads (pairs of K loads, pairs of V loads, then the segment ids) of the cursor's
+  // tile into the buffer at LDS address BUF_.
+  constexpr int GRP_PER_TENSOR = PAIRS ? Tile::DMA_PER_WAVE / 2 : Tile::DMA_PER_WAVE;
+  constexpr int NGRP = 2 * GRP_PER_TENSOR + (HAS_SEG ? 1 : 0);
 #define AXL_DMA(BUF_, K_)                                                                          \
   {                                                                                               \
-    if ((K_) < Tile::DMA_PER_WAVE)                                                                \
-      dma16(k_src + k_lane[(K_) % Tile::DMA_PER_WAVE],                                            \
-            (BUF_) + wave * (ROWS_PER_WAVE * Tile::ROWB) + (K_) * 1024);                          \
-    else if ((K_) < 2 * Tile::DMA_PER_WAVE)                                                       \
-      dma16(v_src + v_lane[(K_) % Tile::DMA_PER_WAVE],                                            \
-            (BUF_) + Tile::TILE_BYTES + wave * (ROWS_PER_WAVE * Tile::ROWB) + ((K_) - Tile::DMA_PER_WAVE) * 1024); \
-    else if (lane < 16)                                                                           \
+    constexpr int per_ = PAIRS ? 2 : 1;                                                           \
+    if ((K_) < GRP_PER_TENSOR) {                                                                  \
+      const unsigned dst_ = (BUF_) + wave * (ROWS_PER_WAVE * Tile::ROWB) + per_ * (K_) * 1024;    \
+      if constexpr (PAIRS) dma16x2(k_lane[(2 * (K_)) % Tile::DMA_PER_WAVE], k_lane[(2 * (K_) + 1) % Tile::DMA_PER_WAVE], k_src, dst_); \
+      else dma16s(k_lane[(K_) % Tile::DMA_PER_WAVE], k_src, dst_);                                \
+    } else if ((K_) < 2 * GRP_PER_TENSOR) {                                                       \
+      constexpr int kv_ = ((K_) - GRP_PER_TENSOR) % GRP_PER_TENSOR;                               \
+      const unsigned dst_ = (BUF_) + Tile::TILE_BYTES + wave * (ROWS_PER_WAVE * Tile::ROWB) + per_ * kv_ * 1024; \
+      if constexpr (PAIRS) dma16x2(v_lane[(2 * kv_) % Tile::DMA_PER_WAVE], v_lane[(2 * kv_ + 1) % Tile::DMA_PER_WAVE], v_src, dst_); \
+      else dma16s(v_lane[kv_ % Tile::DMA_PER_WAVE], v_src, dst_);                                 \
+    } else if (lane < 16) {                                                                       \
       dma16(s_src, (BUF_) + Tile::SEG_BASE);                                                      \
+    }                                                                                             \
   }
 #define AXL_DMA_TILE(BUF_)                                                                         \
   {                                                                                               \
-    _Pragma("unroll") for (int k_ = 0; k_ < Tile::DMA_PER_TILE; k_++) AXL_DMA(BUF_, k_)           \
+    AXL_DMA(BUF_, 0) AXL_DMA(BUF_, 1)                                                             \
+    if constexpr (NGRP > 2) AXL_DMA(BUF_, 2)                                                      \
+    if constexpr (NGRP > 3) AXL_DMA(BUF_, 3)                                                      \
+    if constexpr (NGRP > 4) AXL_DMA(BUF_, 4)                                                      \
+    static_assert(NGRP <= 5, "groups of tile loads");                                             \
   }
   // Prefetch cursor; it stops at the last tile (re-fetching that tile is harmless).
   int pf_idx = 0;
@@ -243,7 +260,8 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
   constexpr int kAheadA = (NB < 6 ? NB : 6), kAheadB = (NB < 4 ? NB : 4);
   constexpr int NLD = Tile::DMA_PER_TILE;     // direct-to-LDS loads of a tile per wavefront
   constexpr int LD_SLOT0 = 2;                 // one per slot from here on, after the cursor moved in slot 1
-  static_assert(LD_SLOT0 + NLD <= 2 * NS, "the loads of a tile fit into one trip");
+  constexpr int LD_STRIDE = 2;                // a group of loads every other slot
+  static_assert(LD_SLOT0 + LD_STRIDE * NGRP <= 2 * NS, "the loads of a tile fit into one trip");
   TrFrag bfr_next[kAheadB];            // first stage-B fragments of the next step
   const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
@@ -329,7 +347,11 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
         if ((2 * i + 1) * (NS - 3) / 16 + 3 == n) DSB_N.p[i] = pack_bf16(DP_E[2 * i], DP_E[2 * i + 1]); \
       /* ---- tile t+3: advance the cursor, then one direct-to-LDS load per slot */                    \
       if ((H_) * NS + n == LD_SLOT0 - 1) AXL_ADVANCE()                                                 \
-      if ((H_) * NS + n >= LD_SLOT0 && (H_) * NS + n < LD_SLOT0 + NLD) AXL_DMA(lds_s, (H_) * NS + n - LD_SLOT0) \
+      if ((H_) * NS + n == LD_SLOT0) AXL_DMA(lds_s, 0)                                                 \
+      if ((H_) * NS + n == LD_SLOT0 + LD_STRIDE) AXL_DMA(lds_s, 1)                                     \
+      if (NGRP > 2 && (H_) * NS + n == LD_SLOT0 + 2 * LD_STRIDE) AXL_DMA(lds_s, 2 % NGRP)              \
+      if (NGRP > 3 && (H_) * NS + n == LD_SLOT0 + 3 * LD_STRIDE) AXL_DMA(lds_s, 3 % NGRP)              \
+      if (NGRP > 4 && (H_) * NS + n == LD_SLOT0 + 4 * LD_STRIDE) AXL_DMA(lds_s, 4 % NGRP)              \
       /* ---- segment ids of sub-tile j+2 for the next step's elementwise stage */                     \
       if (HAS_SEG && n == NS / 2) AXL_READ_SEG_PART(buf_a, H_, 0, SEG_N)                               \
       if (HAS_SEG && n == NS / 2 + 1) AXL_READ_SEG_PART(buf_a, H_, 1, SEG_N)                           \
@@ -406,6 +428,7 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
 #undef AXL_DMA_TILE
 #undef AXL_ADVANCE
 
+  if (!live) return;
   __bf16* dqp = (__bf16*)a.dq + b * a.dqs.b + (int64_t)(q0 + l32) * a.dqs.s + h * a.dqs.h;
 #pragma unroll
   for (int dt = 0; dt < DT; dt++)
@@ -421,15 +444,19 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
     }
 }
 
+#ifndef AXL_DQ_WAVES
+#define AXL_DQ_WAVES 4
+#endif
 template <int D, bool HAS_SEG>
 static hipError_t launch_one(const BwdArgs& a, hipStream_t stream) {
-  using Tile = DqRing<D, HAS_SEG>;
-  auto kernel = flash_bwd_dq_ring_kernel<D, HAS_SEG>;
+  constexpr int NW = AXL_DQ_WAVES;
+  using Tile = DqRing<D, HAS_SEG, NW>;
+  auto kernel = flash_bwd_dq_ring_kernel<D, HAS_SEG, NW>;
   hipError_t err = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                                        Tile::LDS_BYTES);
   if (err != hipSuccess) return err;
-  const int grid = (a.T / Tile::BQ) * a.B * a.Hq;
-  hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), Tile::LDS_BYTES, stream, a);
+  const int grid = ((a.T + Tile::BQ - 1) / Tile::BQ) * a.B * a.Hq;
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(64 * NW), Tile::LDS_BYTES, stream, a);
   return hipGetLastError();
 }
 
