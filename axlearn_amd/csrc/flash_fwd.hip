@@ -19,6 +19,8 @@
 //     (ds_read_b64_tr_b16);
 //   * GQA reads the shared kv head directly (no repeated KV in HBM), and workgroups that share a kv
 //     head are placed on the same XCD so its L2 serves the re-reads.
+#include <type_traits>
+
 #include "common.h"
 
 namespace axl {
@@ -54,7 +56,8 @@ struct FwdTile {
 };
 
 template <int D, bool AUX>
-__global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void flash_fwd_bf16_kernel(const FwdArgs a) {
   using Tile = FwdTile<D>;
   constexpr int KK = D / 16;  // MFMA k-steps over head_dim
   constexpr int DT = D / 32;  // 32-row output tiles over head_dim
@@ -130,20 +133,22 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
   // ---- tile loads: wavefront w fetches rows 16w .. 16w+15 of a K (or V) tile, 1 KB per
   // instruction (1024 / ROWB rows); lane l's chunk slot is l % CPR of row l / CPR.
   constexpr int RPI = 1024 / Tile::ROWB;  // rows per instruction
-  int k_src[Tile::DMA_PER_WAVE], v_src[Tile::DMA_PER_WAVE];  // element offsets from the tile's first row
+  static_assert(Tile::DMA_PER_WAVE % 2 == 0, "tile loads are issued in pairs");
+  unsigned k_src[Tile::DMA_PER_WAVE], v_src[Tile::DMA_PER_WAVE];  // byte offsets from the tile's first row
 #pragma unroll
   for (int i = 0; i < Tile::DMA_PER_WAVE; i++) {
     const int row = 16 * wave + RPI * i + lane / CPR;
     const int chunk = (lane % CPR) ^ Tile::swz(row);
-    k_src[i] = row * (int)a.ks.s + chunk * 8;
-    v_src[i] = row * (int)a.vs.s + chunk * 8;
+    // the second load of a pair carries an instruction offset of 1024, which also moves its source
+    k_src[i] = (unsigned)(row * (int)a.ks.s + chunk * 8) * 2 - (i % 2) * 1024;
+    v_src[i] = (unsigned)(row * (int)a.vs.s + chunk * 8) * 2 - (i % 2) * 1024;
   }
   const unsigned lds0 = lds_address(smem);
   auto issue_k = [&](int t, int buf) {
     const __bf16* src = kp + (int64_t)t * Tile::BK * a.ks.s;
     const unsigned dst = lds0 + buf * Tile::TILE_BYTES + wave * (16 * Tile::ROWB);
 #pragma unroll
-    for (int i = 0; i < Tile::DMA_PER_WAVE; i++) dma16(src + k_src[i], dst + i * 1024);
+    for (int i = 0; i < Tile::DMA_PER_WAVE; i += 2) dma16x2(k_src[i], k_src[i + 1], src, dst + i * 1024);
     if (seg_k && wave == 0 && lane < Tile::BK / 4)  // 64 ids = 16 lanes x 16 bytes
       dma16(seg_k + t * Tile::BK + 4 * lane, lds0 + Tile::SEG_BASE + (t % Tile::NSEG) * (Tile::BK * 4));
   };
@@ -151,7 +156,7 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
     const __bf16* src = vp + (int64_t)t * Tile::BK * a.vs.s;
     const unsigned dst = lds0 + (2 + buf) * Tile::TILE_BYTES + wave * (16 * Tile::ROWB);
 #pragma unroll
-    for (int i = 0; i < Tile::DMA_PER_WAVE; i++) dma16(src + v_src[i], dst + i * 1024);
+    for (int i = 0; i < Tile::DMA_PER_WAVE; i += 2) dma16x2(v_src[i], v_src[i + 1], src, dst + i * 1024);
   };
 
   // ---- per-lane LDS read offsets (bytes).  K row reads: row swap_bits_2_3(l32) (+32 per sub-tile),
@@ -178,7 +183,9 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
     bf16x8 v;
     shortx4 hlf[2];
   };
-  floatx16 s[2];  // logits of the tile whose softmax is next; sub-tile ks holds keys 32ks .. 32ks+31
+  // Logits of the tile whose softmax is next (sub-tile ks holds keys 32ks .. 32ks+31) and of the tile
+  // after it: two register sets that swap roles from tile to tile, so nothing is copied.
+  floatx16 s_even[2], s_odd[2];
 #define AXL_K_FRAG(KT_, KK_, KS_) \
   (*(const bf16x8*)((KT_) + (KS_) * 32 * Tile::ROWB + k_row_off + ((((KK_) * 32) + g * 16) ^ k_xor)))
   // S^T of one tile, nothing interleaved (pipeline fill).
@@ -194,10 +201,12 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
   // Pipeline fill: S^T of the first tile.
   wait_vmem_le<0>();
   __syncthreads();
-  if (t_begin < t_end && t_begin >= tw_begin && t_begin < tw_end) AXL_S_PLAIN(k_lds, s)
+  if (t_begin < t_end && t_begin >= tw_begin && t_begin < tw_end) AXL_S_PLAIN(k_lds, s_even)
 
-  for (int t = t_begin; t < t_end; t++) {
-    const int buf = (t - t_begin) & 1;
+  // One tile: softmax and P V of tile t (logits in s), S^T of tile t+1 (into s_nxt).  buf_c is the
+  // parity of the tile, i.e. which half of the double buffers holds it.
+  auto tile_step = [&](int t, auto buf_c, floatx16 (&s)[2], floatx16 (&s_nxt)[2]) __attribute__((always_inline)) {
+    constexpr int buf = decltype(buf_c)::value;
     // K(t+1) and V(t) (requested one iteration ago) become visible to the whole workgroup and every
     // wavefront is done with S(t) and PV(t-1); the buffers those were read from are then refilled
     // with K(t+2) and V(t+1).
@@ -211,14 +220,9 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
     const char* kt = k_lds + (buf ^ 1) * Tile::TILE_BYTES;   // K(t+1)
     const char* vt = v_lds + buf * Tile::TILE_BYTES;         // V(t)
     const int k0 = t * Tile::BK;
-    floatx16 s_nxt[2];
     if (!do_sm) {
-      if (do_s) {
-        AXL_S_PLAIN(kt, s_nxt)
-        s[0] = s_nxt[0];
-        s[1] = s_nxt[1];
-      }
-      continue;
+      if (do_s) AXL_S_PLAIN(kt, s_nxt)
+      return;
     }
 
     // ---- masks of tile t.  Register r of sub-tile ks in lane group g is key k0 + 32ks + 16(r/8) + 8g + (r%8).
@@ -381,10 +385,14 @@ __global__ __launch_bounds__(256) void flash_fwd_bf16_kernel(const FwdArgs a) {
       __builtin_amdgcn_sched_barrier(0);
     }
 #undef AXL_PV_READ
-    if (do_s) {
-      s[0] = s_nxt[0];
-      s[1] = s_nxt[1];
+  };
+  {
+    int t = t_begin;
+    for (; t + 1 < t_end; t += 2) {
+      tile_step(t, std::integral_constant<int, 0>{}, s_even, s_odd);
+      tile_step(t + 1, std::integral_constant<int, 1>{}, s_odd, s_even);
     }
+    if (t < t_end) tile_step(t, std::integral_constant<int, 0>{}, s_even, s_odd);
   }
 #undef AXL_K_FRAG
 #undef AXL_S_PLAIN
