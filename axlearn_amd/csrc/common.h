@@ -5,6 +5,9 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+#include <utility>
+
 #include "../../include/axl_attn.h"
 
 namespace axl {
@@ -196,6 +199,16 @@ __device__ __forceinline__ void decode_block(int bid, int nqb, int B, int Hq, in
     b = rem / Hq;
     h = rem % Hq;
   }
+}
+
+// f(std::integral_constant<int, 0>{}), ..., f(std::integral_constant<int, N - 1>{}) in order.
+template <class F, int... I>
+__device__ __forceinline__ void for_each_index_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void for_each_index(F&& f) {
+  for_each_index_impl(f, std::make_integer_sequence<int, N>{});
 }
 
 struct Strides3 {

@@ -415,8 +415,10 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
       AXL_AUX_ROW0(h_a, q0_a, bias_t, drop_t)
     }
     __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int n = 0; n < NS; n++) {
+    // One MFMA slot.  The slot number is a compile-time constant (the slots are instantiated one by
+    // one, not produced by a loop unroller, which gives up on bodies of this size).
+    auto slot = [&](auto n_c) __attribute__((always_inline)) {
+      constexpr int n = decltype(n_c)::value;
       // ---- LDS fragments requested ahead of their MFMA
       if (n + kAheadB < NB) AXL_B_READ_AT(b_ad, bfr[n + kAheadB], n + kAheadB)
       if (n + kAheadA >= NB && n + kAheadA - NB < NA) {
@@ -465,7 +467,8 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
       if (n == NS / 2) AXL_READ_STATS_PART(buf_a, 0, lse_n, del_n, seg_n)
       if (n == NS / 2 + 1) AXL_READ_STATS_PART(buf_a, 1, lse_n, del_n, seg_n)
       __builtin_amdgcn_sched_barrier(0);
-    }
+    };
+    for_each_index<NS>(slot);
     // Tile j+3 (requested during the previous iteration) has landed once at most this iteration's
     // loads are outstanding; after the barrier every wavefront's part of it is visible, and nobody
     // reads tile j's buffer any more, which the next iteration refills.  (With a bias or a dropout
@@ -513,10 +516,11 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
     if (a.mask_kind == AXL_MASK_SLIDING_WINDOW)
       u_hi = min(nt - 1, floor_div(a.window + k0 - 31 - a.q_off, Tile::BQ) - t_begin);
   }
-  if (HAS_SEG || AUX) u_lo = nt;  // every tile takes the masked path
   u_lo = min(u_lo, nt);
   u_hi = max(u_hi, u_lo - 1);
-  {
+  if constexpr (HAS_SEG || AUX) {
+    run(0, total, std::true_type{});  // every tile takes the masked path
+  } else {
     int j = 0;
     auto run_to = [&](int e_end, auto masked_c) __attribute__((always_inline)) {
       const int j_end = min(total, e_end - 1);
