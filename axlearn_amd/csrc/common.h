@@ -117,6 +117,16 @@ __device__ __forceinline__ void dma16s(unsigned voff, const void* sbase, unsigne
                : "v"(voff), "s"(sbase), "s"(lds_base)
                : "memory", "m0");
 }
+// The same for lanes 0..7 only (128 bytes).  The load is issued with EXEC narrowed to those lanes and
+// EXEC is then set back to all 64 lanes, so the caller must be in wave-uniform control flow with every
+// lane active (no branch is generated, which keeps the caller's code in one scheduling region).
+__device__ __forceinline__ void dma16s_first8(unsigned voff, const void* sbase, unsigned lds_base) {
+  asm volatile(
+      "s_mov_b64 exec, 0xff\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1\n\ts_mov_b64 exec, -1"
+      :
+      : "v"(voff), "s"(sbase), "s"(lds_base)
+      : "memory", "m0");
+}
 #pragma clang diagnostic pop
 template <int N>
 __device__ __forceinline__ void wait_vmem_le() {

@@ -106,43 +106,51 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
   // global chunk that the swizzle puts there.  Lanes 0..7 of wavefront w also fetch one row of
   // statistics (4 query rows each): w = 0 the scaled lse, 1 delta, 2 the segment ids.
   constexpr int CPR = D / 8;  // 16-byte chunks per row
-  int q_lane[Tile::DMA_PER_WAVE], d_lane[Tile::DMA_PER_WAVE];  // element offsets from the tile's first row
+  constexpr bool PAIRS = Tile::DMA_PER_WAVE == 2;  // the two loads of a tensor go out as one pair
+  static_assert(Tile::DMA_PER_WAVE <= 2, "tile loads per tensor");
+  unsigned q_lane[Tile::DMA_PER_WAVE], d_lane[Tile::DMA_PER_WAVE];  // byte offsets from the tile's first row
 #pragma unroll
   for (int i = 0; i < Tile::DMA_PER_WAVE; i++) {
     const int row = 8 * wave + Tile::RPI * i + lane / CPR;
     const int chunk = (lane % CPR) ^ tile_swizzle<D>(row);
-    q_lane[i] = row * (int)a.qs.s + chunk * 8;
-    d_lane[i] = row * (int)a.dos.s + chunk * 8;
+    // the second load of a pair carries an instruction offset of 1024, which also moves its source
+    q_lane[i] = (unsigned)(row * (int)a.qs.s + chunk * 8) * 2 - (i % 2) * 1024;
+    d_lane[i] = (unsigned)(row * (int)a.dos.s + chunk * 8) * 2 - (i % 2) * 1024;
   }
   const int st_kind = wave;
   // Running source pointers of the prefetch cursor, advanced by wave-uniform steps: no 64-bit
   // multiplies inside the loop.  Tile sequence: query head (outer) x query tile (inner).
   const __bf16* q_src = (const __bf16*)a.q + b * a.qs.b + (int64_t)(hk * G) * a.qs.h + (int64_t)t_begin * Tile::BQ * a.qs.s;
   const __bf16* d_src = (const __bf16*)a.dout + b * a.dos.b + (int64_t)(hk * G) * a.dos.h + (int64_t)t_begin * Tile::BQ * a.dos.s;
-  const int64_t stat_row0 = ((int64_t)b * a.Hq + hk * G) * a.T + (int64_t)t_begin * Tile::BQ + 4 * (lane & 7);
+  const int64_t stat_row0 = ((int64_t)b * a.Hq + hk * G) * a.T + (int64_t)t_begin * Tile::BQ;
   const bool s_is_seg = HAS_SEG && st_kind == 2;
-  const char* s_src = st_kind == 1 ? (const char*)(a.delta + stat_row0) : (const char*)(a.lse2 + stat_row0);
-  if (s_is_seg) s_src = (const char*)(a.seg + (int64_t)b * a.T + (int64_t)t_begin * Tile::BQ + 4 * (lane & 7));
+  const char* s_src = st_kind == 1 ? (const char*)(a.delta + stat_row0) : (const char*)(a.lse2 + stat_row0);  // wave-uniform
+  if (s_is_seg) s_src = (const char*)(a.seg + (int64_t)b * a.T + (int64_t)t_begin * Tile::BQ);
+  const unsigned s_lane = 16 * (lane & 7);  // lanes 0..7 fetch 4 query rows each
   const int64_t q_step = (int64_t)Tile::BQ * a.qs.s, d_step = (int64_t)Tile::BQ * a.dos.s;
   const int64_t q_wrap = a.qs.h - (int64_t)(nt - 1) * q_step;    // last tile of a head -> first of next
   const int64_t d_wrap = a.dos.h - (int64_t)(nt - 1) * d_step;
   const int64_t s_step = Tile::BQ * 4, s_wrap = ((int64_t)a.T - (int64_t)(nt - 1) * Tile::BQ) * 4;
   const int64_t seg_wrap = -(int64_t)(nt - 1) * Tile::BQ * 4;   // segment ids do not depend on the head
   const unsigned lds0 = lds_address(smem);
-  // The k-th of the DMA_PER_TILE loads of the cursor's tile into the buffer at LDS address BUF_.
+  // The k-th group of loads (Q rows, dO rows, statistics) of the cursor's tile into the buffer at LDS
+  // address BUF_; all from scalar bases, no vector instruction forms an address.
+  constexpr int NGRP = 3;
 #define AXL_DMA(BUF_, K_)                                                                          \
   {                                                                                               \
-    if ((K_) < Tile::DMA_PER_WAVE)                                                                \
-      dma16(q_src + q_lane[(K_) % Tile::DMA_PER_WAVE], (BUF_) + wave * (8 * Tile::ROWB) + (K_) * 1024); \
-    else if ((K_) < 2 * Tile::DMA_PER_WAVE)                                                       \
-      dma16(d_src + d_lane[(K_) % Tile::DMA_PER_WAVE],                                            \
-            (BUF_) + Tile::TILE_BYTES + wave * (8 * Tile::ROWB) + ((K_) - Tile::DMA_PER_WAVE) * 1024); \
-    else if (lane < 8)                                                                            \
-      dma16(s_src, (BUF_) + Tile::STAT_BASE + st_kind * (Tile::BQ * 4));                          \
+    if ((K_) == 0) {                                                                              \
+      if constexpr (PAIRS) dma16x2(q_lane[0], q_lane[Tile::DMA_PER_WAVE - 1], q_src, (BUF_) + wave * (8 * Tile::ROWB)); \
+      else dma16s(q_lane[0], q_src, (BUF_) + wave * (8 * Tile::ROWB));                            \
+    } else if ((K_) == 1) {                                                                       \
+      if constexpr (PAIRS) dma16x2(d_lane[0], d_lane[Tile::DMA_PER_WAVE - 1], d_src, (BUF_) + Tile::TILE_BYTES + wave * (8 * Tile::ROWB)); \
+      else dma16s(d_lane[0], d_src, (BUF_) + Tile::TILE_BYTES + wave * (8 * Tile::ROWB));         \
+    } else {                                                                                      \
+      dma16s_first8(s_lane, s_src, (BUF_) + Tile::STAT_BASE + st_kind * (Tile::BQ * 4));          \
+    }                                                                                             \
   }
 #define AXL_DMA_TILE(BUF_)                                                                         \
   {                                                                                               \
-    _Pragma("unroll") for (int k_ = 0; k_ < Tile::DMA_PER_TILE; k_++) AXL_DMA(BUF_, k_)           \
+    AXL_DMA(BUF_, 0) AXL_DMA(BUF_, 1) AXL_DMA(BUF_, 2)                                            \
   }
   // Prefetch cursor; it stops at the last tile (re-fetching that tile is harmless).
   int pf_idx = 0, pf_t = 0, pf_h = 0;  // tile number, query tile within the head, head within the group
@@ -390,8 +398,6 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
     for (int i = 0; i < kAheadB; i++) bfr[i] = bfr_next[i];
     floatx16 s_a, dp_a;
     PackedOperand pb_n, dsb_n;           // tile j + 1, packed as its elements complete
-    floatx4 lse_n[4], del_n[4];          // statistics of tile j + 2
-    intx4 seg_n[4];
     int q0_p = q0_s, h_p = h_s;
     const unsigned lds_s = lds_address(buf_s);
     const char* a_ad[KK];                // this iteration's fragment addresses: stage A in tile j+2,
@@ -462,10 +468,18 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
       if constexpr (AUX) {
         if (n % ESTEP == 0) AXL_AUX_LOAD(bias_t, drop_t, n / ESTEP, braw_n, draw_n)
       }
-      if (n >= LD_SLOT0 && n < LD_SLOT0 + NLD) AXL_DMA(lds_s, n - LD_SLOT0)
-      // ---- statistics of tile j+2 for the next iteration's elementwise stage
-      if (n == NS / 2) AXL_READ_STATS_PART(buf_a, 0, lse_n, del_n, seg_n)
-      if (n == NS / 2 + 1) AXL_READ_STATS_PART(buf_a, 1, lse_n, del_n, seg_n)
+      if (n >= LD_SLOT0 && n < LD_SLOT0 + NGRP) AXL_DMA(lds_s, n - LD_SLOT0)
+      // ---- statistics of tile j+2 for the next iteration's elementwise stage, four query rows at a
+      // time, each group as soon as this iteration's elements are done with the registers
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const char* st_ = buf_a + Tile::STAT_BASE + 8 * g * 4 + 64 * (i / 2) + 16 * (i % 2);
+        if (n == (4 * i + 3) * (NS - 3) / 16 + 1) {
+          lse_v[i] = *(const floatx4*)st_;
+          if (HAS_SEG) seg_v[i] = *(const intx4*)(st_ + 2 * Tile::BQ * 4);
+        }
+        if (n == (4 * i + 3) * (NS - 3) / 16 + 3) del_v[i] = *(const floatx4*)(st_ + Tile::BQ * 4);
+      }
       __builtin_amdgcn_sched_barrier(0);
     };
     for_each_index<NS>(slot);
@@ -486,12 +500,6 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
     dp_e = dp_a;
     pb = pb_n;
     dsb = dsb_n;
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-      lse_v[i] = lse_n[i];
-      del_v[i] = del_n[i];
-      if (HAS_SEG) seg_v[i] = seg_n[i];
-    }
     if constexpr (AUX) {
 #pragma unroll
       for (int r = 0; r < 16; r++) {
