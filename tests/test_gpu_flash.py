@@ -98,6 +98,14 @@ BWD_CASES = [
     (2, 512, 4, 1, 128, "causal", None, True),
     (1, 1024, 4, 2, 128, "sliding", 300, True),
     (2, 512, 2, 2, 64, "sliding", 127, False),
+    # long enough for every kind of loop run in the backward kernels: masked tiles at the window edge,
+    # mask-free interior tiles, masked diagonal tiles; odd and even numbers of 64-key tiles
+    (1, 2048, 2, 1, 128, "sliding", 600, False),
+    (1, 2048, 2, 2, 128, "sliding", 40, False),
+    (1, 1920, 2, 1, 64, "sliding", 777, False),
+    (1, 1536, 4, 2, 128, "none", None, False),
+    (1, 1664, 4, 2, 64, "causal", None, False),
+    (1, 1152, 2, 1, 128, "sliding", 1000, True),
 ]
 
 
@@ -112,6 +120,28 @@ def test_backward_matches_oracle(b, t, hq, hkv, d, mask, window, seg):
     qc, kc, vc, doc = q.cuda(), k.cuda(), v.cuda(), do.cuda()
     out, lse = ops.flash_fwd(qc, kc, vc, softmax_scale=scale, **kw)
     dq, dk, dv = ops.flash_bwd(qc, kc, vc, out, lse, doc, softmax_scale=scale, **kw)
+    _assert_close("dq", dq, wq, dtype)
+    _assert_close("dk", dk, wk, dtype)
+    _assert_close("dv", dv, wv, dtype)
+
+
+@pytest.mark.parametrize("mask,window", [("causal", None), ("sliding", 333)])
+@pytest.mark.parametrize("d", [64, 128])
+def test_backward_with_more_keys_than_queries(mask, window, d):
+    """A chunk of T queries at positions q_off .. q_off+T-1 over S > T keys (gradients of an incremental
+    prefill): dq, dk, dv against the oracle with explicit query positions."""
+    b, t, s_len, hq, hkv, q_off = 1, 256, 1024, 4, 2, 640
+    dtype = torch.bfloat16
+    q, k, v, do = _inputs(b, t, hq, hkv, d, dtype, s=s_len)
+    spec = ref.MaskSpec(causal=mask == "causal", sliding_window=window,
+                        target_positions=torch.arange(q_off, q_off + t)[None], source_positions=torch.arange(s_len)[None])
+    mk = ops.MASK_CAUSAL if mask == "causal" else ops.MASK_SLIDING_WINDOW
+    kw = dict(mask_kind=mk, sliding_window=window or 0, q_pos_offset=q_off, softmax_scale=d ** -0.5)
+    wq, wk, wv = ref.reference_mha_grads(q, k, v, do, spec, softmax_scale=d ** -0.5)
+    qc, kc, vc, doc = q.cuda(), k.cuda(), v.cuda(), do.cuda()
+    out, lse = ops.flash_fwd(qc, kc, vc, **kw)
+    _assert_close("out", out, ref.reference_mha(q, k, v, spec, softmax_scale=d ** -0.5), dtype)
+    dq, dk, dv = ops.flash_bwd(qc, kc, vc, out, lse, doc, **kw)
     _assert_close("dq", dq, wq, dtype)
     _assert_close("dk", dk, wk, dtype)
     _assert_close("dv", dv, wv, dtype)
