@@ -42,6 +42,9 @@ struct DqRing {
   static constexpr int LDS_BYTES = NBUF * BUF_BYTES;
 };
 
+constexpr int kMaxSub = 1024;               // 32-key sub-tiles whose segment ids the dQ kernel classifies
+constexpr int kNotUniform = -0x7fffffff - 1;  // marks a sub-tile with more than one segment id
+
 template <int D, bool HAS_SEG, int NW>
 __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4, NW / 4)))
 void flash_bwd_dq_ring_kernel(const BwdArgs a) {
@@ -401,7 +404,47 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
     e1 = floor_div(qpos_min - 31 - key0, 32) + 1;
     if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) e0 = floor_div(qpos_max - a.window - key0 + 31, 32);
   }
-  if (HAS_SEG) e0 = 0x3fffffff;
+  if (HAS_SEG) {
+    // Sub-tiles whose 32 keys all carry the segment id that all 32 queries of this wavefront carry
+    // need no segment mask either: take the first run [tA, tB) of such sub-tiles (the masked loop is
+    // always correct, so whatever lies outside that run simply stays on it).
+    __shared__ int s_sub[kMaxSub];
+    const int nsub = 2 * trips;
+    int tA = 0, tB = 0;
+    if (nsub <= kMaxSub) {
+      const int32_t* ids = a.seg + (int64_t)b * a.T + key0;
+      for (int i = tid; i < nsub; i += 64 * NW) {
+        const intx4* p = (const intx4*)(ids + 32 * i);
+        const int id0 = ids[32 * i];
+        bool same = true;
+#pragma unroll
+        for (int v = 0; v < 8; v++) {
+          const intx4 x = p[v];
+          same = same && x[0] == id0 && x[1] == id0 && x[2] == id0 && x[3] == id0;
+        }
+        s_sub[i] = same ? id0 : kNotUniform;
+      }
+      __syncthreads();
+      const int wq_id = __builtin_amdgcn_readfirstlane(seg_q);
+      const bool q_uniform = __builtin_amdgcn_ballot_w64(seg_q != wq_id) == 0 && wq_id != kNotUniform;
+      tA = tB = nsub;
+      if (q_uniform) {
+        for (int base = 0; base < nsub && tA == nsub; base += 64) {
+          const int i = base + lane;
+          const uint64_t m = __builtin_amdgcn_ballot_w64(i < nsub && s_sub[i] == wq_id);
+          if (m) tA = base + __builtin_ctzll(m);
+        }
+        for (int base = tA & ~63; base < nsub && tB == nsub; base += 64) {
+          const int i = base + lane;
+          const uint64_t m = __builtin_amdgcn_ballot_w64(i > tA && i < nsub && s_sub[i] != wq_id);
+          if (m) tB = base + __builtin_ctzll(m);
+        }
+      }
+    }
+    e0 = max(e0, tA);
+    e1 = min(e1, tB);
+    if (e1 <= e0) e0 = e1 = 0x3fffffff;
+  }
   // trip t is unmasked iff 2t + 1 >= e0 and 2t + 2 < e1
   const int t0 = min(trips, max(0, e0 >= 0x3fffffff ? trips : floor_div(e0, 2)));
   const int t1 = min(trips, max(t0, e1 >= 0x3fffffff ? trips : floor_div(e1 - 3, 2) + 1));
