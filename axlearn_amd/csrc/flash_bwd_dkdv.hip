@@ -44,6 +44,9 @@ struct DkvTile {
   static constexpr int LDS_BYTES = NBUF * BUF_BYTES;
 };
 
+constexpr int kMaxSubDkv = 1024;                 // query tiles whose segment ids the dK/dV kernel classifies
+constexpr int kNotUniformDkv = -0x7fffffff - 1;  // marks a tile with more than one segment id
+
 template <int D, bool HAS_SEG, bool AUX>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
@@ -524,9 +527,48 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
     if (a.mask_kind == AXL_MASK_SLIDING_WINDOW)
       u_hi = min(nt - 1, floor_div(a.window + k0 - 31 - a.q_off, Tile::BQ) - t_begin);
   }
+  if (HAS_SEG && !AUX) {
+    // Query tiles whose 32 rows all carry the segment id that all 32 keys of this wavefront carry
+    // need no segment mask either: take the first run [tA, tB) of such tiles (the masked loop is
+    // always correct, so whatever lies outside that run simply stays on it).
+    __shared__ int s_sub[kMaxSubDkv];
+    int tA = 0, tB = 0;
+    if (nt <= kMaxSubDkv) {
+      const int32_t* ids = a.seg + (int64_t)b * a.T + (int64_t)t_begin * Tile::BQ;
+      for (int i = tid; i < nt; i += 256) {
+        const intx4* p = (const intx4*)(ids + 32 * i);
+        const int id0 = ids[32 * i];
+        bool same = true;
+#pragma unroll
+        for (int v = 0; v < 8; v++) {
+          const intx4 x = p[v];
+          same = same && x[0] == id0 && x[1] == id0 && x[2] == id0 && x[3] == id0;
+        }
+        s_sub[i] = same ? id0 : kNotUniformDkv;
+      }
+      __syncthreads();
+      const int wk_id = __builtin_amdgcn_readfirstlane(seg_k);
+      const bool k_uniform = __builtin_amdgcn_ballot_w64(seg_k != wk_id) == 0 && wk_id != kNotUniformDkv;
+      tA = tB = nt;
+      if (k_uniform) {
+        for (int base = 0; base < nt && tA == nt; base += 64) {
+          const int i = base + lane;
+          const uint64_t m = __builtin_amdgcn_ballot_w64(i < nt && s_sub[i] == wk_id);
+          if (m) tA = base + __builtin_ctzll(m);
+        }
+        for (int base = tA & ~63; base < nt && tB == nt; base += 64) {
+          const int i = base + lane;
+          const uint64_t m = __builtin_amdgcn_ballot_w64(i > tA && i < nt && s_sub[i] != wk_id);
+          if (m) tB = base + __builtin_ctzll(m);
+        }
+      }
+    }
+    u_lo = max(u_lo, tA);
+    u_hi = min(u_hi, tB - 1);
+  }
   u_lo = min(u_lo, nt);
   u_hi = max(u_hi, u_lo - 1);
-  if constexpr (HAS_SEG || AUX) {
+  if constexpr (AUX) {
     run(0, total, std::true_type{});  // every tile takes the masked path
   } else {
     int j = 0;
