@@ -55,6 +55,9 @@ struct FwdTile {
   __device__ static __forceinline__ int swz(int row) { return tile_swizzle<D>(row); }
 };
 
+constexpr int kMaxSegTiles = 1024;               // key tiles whose segment ids the forward classifies
+constexpr int kSegNotUniform = -0x7fffffff - 1;  // marks a tile with more than one segment id
+
 template <int D, bool AUX>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void flash_fwd_bf16_kernel(const FwdArgs a) {
@@ -96,6 +99,27 @@ void flash_fwd_bf16_kernel(const FwdArgs a) {
   if (seg_k) shrink_to_segment_hull(seg_q, seg_k, tid, k_begin, k_end);
   const int t_begin = k_begin / Tile::BK;
   const int t_end = (k_end + Tile::BK - 1) / Tile::BK;
+  // Key tiles whose 64 keys all carry the segment id that all 32 queries of this wavefront carry need
+  // no segment mask: s_tile_id[t - t_begin] is the tile's id if it has only one.
+  __shared__ int s_tile_id[kMaxSegTiles];
+  bool seg_fast = false;   // this wavefront's queries share one id and the table covers the tiles
+  int wq_id = 0;
+  if (seg_k && t_end - t_begin <= kMaxSegTiles) {
+    for (int i = tid; i < t_end - t_begin; i += 256) {
+      const int32_t* ids = seg_k + (t_begin + i) * Tile::BK;
+      const int id0 = ids[0];
+      bool same = true;
+#pragma unroll
+      for (int v = 0; v < Tile::BK / 4; v++) {
+        const intx4 x = ((const intx4*)ids)[v];
+        same = same && x[0] == id0 && x[1] == id0 && x[2] == id0 && x[3] == id0;
+      }
+      s_tile_id[i] = same ? id0 : kSegNotUniform;
+    }
+    __syncthreads();
+    wq_id = __builtin_amdgcn_readfirstlane(seg_q);
+    seg_fast = __builtin_amdgcn_ballot_w64(seg_q != wq_id) == 0 && wq_id != kSegNotUniform;
+  }
 
   // Dense bias / dropout mask rows of this lane's query (AUX instantiation only).  The bias joins
   // the raw logits as bias / scale, so the scale folded into the exponent applies to both.
@@ -276,7 +300,7 @@ void flash_fwd_bf16_kernel(const FwdArgs a) {
         }
       }
     }
-    if (seg_k) {
+    if (seg_k && !(seg_fast && s_tile_id[t - t_begin] == wq_id)) {
       const char* sg = seg_lds + (t % Tile::NSEG) * (Tile::BK * 4);
 #pragma unroll
       for (int ks = 0; ks < 2; ks++) {
