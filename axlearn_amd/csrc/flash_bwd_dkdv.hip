@@ -429,24 +429,24 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
     auto slot = [&](auto n_c) __attribute__((always_inline)) {
       constexpr int n = decltype(n_c)::value;
       // ---- LDS fragments requested ahead of their MFMA
-      if (n + kAheadB < NB) AXL_B_READ_AT(b_ad, bfr[n + kAheadB], n + kAheadB)
-      if (n + kAheadA >= NB && n + kAheadA - NB < NA) {
-        const int x = n + kAheadA - NB;
+      if constexpr (n + kAheadB < NB) AXL_B_READ_AT(b_ad, bfr[n + kAheadB], n + kAheadB)
+      if constexpr (n + kAheadA >= NB && n + kAheadA - NB < NA) {
+        constexpr int x = n + kAheadA - NB;
         afr[x] = *(const bf16x8*)(a_ad[x / 2] + (x % 2) * Tile::TILE_BYTES);
       }
-      if (n >= NS - kAheadB) AXL_B_READ_AT(e_ad, bfr_next[n - (NS - kAheadB)], n - (NS - kAheadB))
+      if constexpr (n >= NS - kAheadB) AXL_B_READ_AT(e_ad, bfr_next[n - (NS - kAheadB)], n - (NS - kAheadB))
       // ---- the MFMA of this slot.  Stage-B step m = t8 * 2DT + dt * 2 + which (which 0: dV with the
       // dO^T fragment and P, 1: dK with the Q^T fragment and dS); stage-A step x: even -> S chain
       // with Q fragment x/2, odd -> dP chain with dO fragment x/2.
-      if (n < NB) {
-        const int t8 = n / (2 * DT), dt = (n % (2 * DT)) / 2;
-        if (n % 2 == 0)
+      if constexpr (n < NB) {
+        constexpr int t8 = n / (2 * DT), dt = (n % (2 * DT)) / 2;
+        if constexpr (n % 2 == 0)
           dv_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[n].v, pb.v[t8], dv_acc[dt], 0, 0, 0);
         else
           dk_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[n].v, dsb.v[t8], dk_acc[dt], 0, 0, 0);
       } else {
-        const int x = n - NB;
-        if (x % 2 == 0)
+        constexpr int x = n - NB;
+        if constexpr (x % 2 == 0)
           s_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afr[x], kf[x / 2], x == 0 ? zero16 : s_a, 0, 0, 0);
         else
           dp_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afr[x], vf[x / 2], x == 1 ? zero16 : dp_a, 0, 0, 0);
@@ -471,7 +471,7 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
       if constexpr (AUX) {
         if (n % ESTEP == 0) AXL_AUX_LOAD(bias_t, drop_t, n / ESTEP, braw_n, draw_n)
       }
-      if (n >= LD_SLOT0 && n < LD_SLOT0 + NGRP) AXL_DMA(lds_s, n - LD_SLOT0)
+      if constexpr (n >= LD_SLOT0 && n < LD_SLOT0 + NGRP) AXL_DMA(lds_s, n - LD_SLOT0)
       // ---- statistics of tile j+2 for the next iteration's elementwise stage, four query rows at a
       // time, each group as soon as this iteration's elements are done with the registers
 #pragma unroll

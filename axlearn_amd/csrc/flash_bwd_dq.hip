@@ -132,12 +132,12 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
 #define AXL_DMA(BUF_, K_)                                                                          \
   {                                                                                               \
     constexpr int per_ = PAIRS ? 2 : 1;                                                           \
-    if ((K_) < GRP_PER_TENSOR) {                                                                  \
+    if constexpr ((K_) < GRP_PER_TENSOR) {                                                        \
       const unsigned dst_ = (BUF_) + wave * (ROWS_PER_WAVE * Tile::ROWB) + per_ * (K_) * 1024;    \
       if constexpr (PAIRS) dma16x2(k_lane[(2 * (K_)) % Tile::DMA_PER_WAVE], k_lane[(2 * (K_) + 1) % Tile::DMA_PER_WAVE], k_src, dst_); \
       else dma16s(k_lane[(K_) % Tile::DMA_PER_WAVE], k_src, dst_);                                \
-    } else if ((K_) < 2 * GRP_PER_TENSOR) {                                                       \
-      constexpr int kv_ = ((K_) - GRP_PER_TENSOR) % GRP_PER_TENSOR;                               \
+    } else if constexpr ((K_) < 2 * GRP_PER_TENSOR) {                                             \
+      constexpr int kv_ = (K_) - GRP_PER_TENSOR;                                                  \
       const unsigned dst_ = (BUF_) + Tile::TILE_BYTES + wave * (ROWS_PER_WAVE * Tile::ROWB) + per_ * kv_ * 1024; \
       if constexpr (PAIRS) dma16x2(v_lane[(2 * kv_) % Tile::DMA_PER_WAVE], v_lane[(2 * kv_ + 1) % Tile::DMA_PER_WAVE], v_src, dst_); \
       else dma16s(v_lane[kv_ % Tile::DMA_PER_WAVE], v_src, dst_);                                 \
