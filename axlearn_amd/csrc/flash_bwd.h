@@ -29,7 +29,9 @@ struct BwdArgs {
 // reads the dense bias / dropout mask.
 hipError_t launch_bwd_dkdv_bf16(const BwdArgs& a, int head_dim, bool aux, hipStream_t stream);
 
-// Enqueues the dQ kernel (bf16, no dense bias / dropout mask) for head_dim 64 or 128.
-hipError_t launch_bwd_dq_bf16(const BwdArgs& a, int head_dim, hipStream_t stream);
+// Enqueues the dQ kernel (bf16, no dense bias / dropout mask) for head_dim 64 or 128.  With
+// `fuse_delta` it also writes delta and the scaled lse into the workspace (instead of reading them),
+// for a dK/dV kernel enqueued after it.
+hipError_t launch_bwd_dq_bf16(const BwdArgs& a, int head_dim, bool fuse_delta, hipStream_t stream);
 
 }  // namespace axl

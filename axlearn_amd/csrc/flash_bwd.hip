@@ -355,16 +355,26 @@ int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream)
       err = hipGetLastError();                                                                  \
     }                                                                                           \
   } while (0)
+  // All three phases in one call, no bias / dropout mask / sink gradient: the dQ kernel computes delta
+  // on the way (it holds the dO rows anyway) and runs first; the dK/dV kernel reads what it left.
+  const int all = AXL_BWD_DELTA | AXL_BWD_DKDV | AXL_BWD_DQ;
+  if ((phases & all) == all && !aux && !p.d_logit_sink) {
+    err = launch_bwd_dq_bf16(a, p.head_dim, true, stream);
+    if (err == hipSuccess) err = launch_bwd_dkdv_bf16(a, p.head_dim, false, stream);
+    if (err != hipSuccess)
+      return set_error(AXL_ERR_LAUNCH, "axl_flash_bwd: launch failed: %s", hipGetErrorString(err));
+    return AXL_OK;
+  }
   if (p.head_dim == 128) {
     if (phases & AXL_BWD_DELTA) AXL_LAUNCH((bwd_delta_kernel<__bf16, 128>), delta_grid, 0);
     if ((phases & AXL_BWD_DKDV) && err == hipSuccess) err = launch_bwd_dkdv_bf16(a, 128, aux, stream);
     if ((phases & AXL_BWD_DQ) && aux) AXL_LAUNCH((flash_bwd_dq_bf16_kernel<128, true>), dq_grid, DqTile<128>::LDS_BYTES);
-    if ((phases & AXL_BWD_DQ) && !aux && err == hipSuccess) err = launch_bwd_dq_bf16(a, 128, stream);
+    if ((phases & AXL_BWD_DQ) && !aux && err == hipSuccess) err = launch_bwd_dq_bf16(a, 128, false, stream);
   } else {
     if (phases & AXL_BWD_DELTA) AXL_LAUNCH((bwd_delta_kernel<__bf16, 64>), delta_grid, 0);
     if ((phases & AXL_BWD_DKDV) && err == hipSuccess) err = launch_bwd_dkdv_bf16(a, 64, aux, stream);
     if ((phases & AXL_BWD_DQ) && aux) AXL_LAUNCH((flash_bwd_dq_bf16_kernel<64, true>), dq_grid, DqTile<64>::LDS_BYTES);
-    if ((phases & AXL_BWD_DQ) && !aux && err == hipSuccess) err = launch_bwd_dq_bf16(a, 64, stream);
+    if ((phases & AXL_BWD_DQ) && !aux && err == hipSuccess) err = launch_bwd_dq_bf16(a, 64, false, stream);
   }
 #undef AXL_LAUNCH
   if ((phases & AXL_BWD_DELTA) && p.d_logit_sink && err == hipSuccess) {

@@ -45,7 +45,10 @@ struct DqRing {
 constexpr int kMaxSub = 1024;               // 32-key sub-tiles whose segment ids the dQ kernel classifies
 constexpr int kNotUniform = -0x7fffffff - 1;  // marks a sub-tile with more than one segment id
 
-template <int D, bool HAS_SEG, int NW>
+// FUSE_DELTA: the kernel also computes delta = rowsum(out * dO) (gpu_attention.py:653-658) and the
+// scaled lse of its own rows and leaves both in the workspace for the dK/dV kernel, which then has to
+// run after this one; the separate delta pass is not needed.
+template <int D, bool HAS_SEG, int NW, bool FUSE_DELTA>
 __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4, NW / 4)))
 void flash_bwd_dq_ring_kernel(const BwdArgs a) {
   using Tile = DqRing<D, HAS_SEG, NW>;
@@ -75,8 +78,33 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
     dof[kk] = *(const bf16x8*)(dop + 16 * kk + 8 * g);
   }
   const int64_t stat_idx = ((int64_t)b * a.Hq + h) * a.T + q0 + l32;
-  const float off = a.lse2[stat_idx];  // -lse * log2(e)
-  const float delta = a.delta[stat_idx];
+  float off, delta;  // -lse * log2(e), rowsum(out * dO)
+  if constexpr (FUSE_DELTA) {
+    // The lane holds d = 16kk + 8g .. +7 of its query's dO; with the same pieces of out, the two lanes
+    // of a query (g = 0, 1) each sum half of the row.
+    const __bf16* op = (const __bf16*)a.out + b * a.os.b + (int64_t)(q0 + l32) * a.os.s + h * a.os.h;
+    float part = 0.f;
+#pragma unroll
+    for (int kk = 0; kk < KK; kk++) {
+      union {
+        bf16x8 v;
+        bf16x2 p[4];
+      } o, d;
+      o.v = *(const bf16x8*)(op + 16 * kk + 8 * g);
+      d.v = dof[kk];
+#pragma unroll
+      for (int i = 0; i < 4; i++) part = __builtin_amdgcn_fdot2_f32_bf16(o.p[i], d.p[i], part, false);
+    }
+    delta = xor32_sum(part);
+    off = a.lse[stat_idx] * (-kLog2e);
+    if (live && g == 0) {
+      a.delta[stat_idx] = delta;
+      a.lse2[stat_idx] = off;
+    }
+  } else {
+    off = a.lse2[stat_idx];
+    delta = a.delta[stat_idx];
+  }
   const int qpos = q0 + l32 + a.q_off;
   const int qpos_min = q0 + a.q_off, qpos_max = q0 + 31 + a.q_off;  // of the wavefront
   int seg_q = 0;
@@ -490,11 +518,11 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
 #ifndef AXL_DQ_WAVES
 #define AXL_DQ_WAVES 4
 #endif
-template <int D, bool HAS_SEG>
+template <int D, bool HAS_SEG, bool FUSE_DELTA>
 static hipError_t launch_one(const BwdArgs& a, hipStream_t stream) {
   constexpr int NW = AXL_DQ_WAVES;
   using Tile = DqRing<D, HAS_SEG, NW>;
-  auto kernel = flash_bwd_dq_ring_kernel<D, HAS_SEG, NW>;
+  auto kernel = flash_bwd_dq_ring_kernel<D, HAS_SEG, NW, FUSE_DELTA>;
   hipError_t err = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                                        Tile::LDS_BYTES);
   if (err != hipSuccess) return err;
@@ -503,10 +531,14 @@ static hipError_t launch_one(const BwdArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
-hipError_t launch_bwd_dq_bf16(const BwdArgs& a, int head_dim, hipStream_t stream) {
+hipError_t launch_bwd_dq_bf16(const BwdArgs& a, int head_dim, bool fuse_delta, hipStream_t stream) {
   const bool seg = a.seg != nullptr;
-  if (head_dim == 128) return seg ? launch_one<128, true>(a, stream) : launch_one<128, false>(a, stream);
-  return seg ? launch_one<64, true>(a, stream) : launch_one<64, false>(a, stream);
+  if (fuse_delta) {
+    if (head_dim == 128) return seg ? launch_one<128, true, true>(a, stream) : launch_one<128, false, true>(a, stream);
+    return seg ? launch_one<64, true, true>(a, stream) : launch_one<64, false, true>(a, stream);
+  }
+  if (head_dim == 128) return seg ? launch_one<128, true, false>(a, stream) : launch_one<128, false, false>(a, stream);
+  return seg ? launch_one<64, true, false>(a, stream) : launch_one<64, false, false>(a, stream);
 }
 
 }  // namespace axl
