@@ -147,6 +147,42 @@ def test_backward_with_more_keys_than_queries(mask, window, d):
     _assert_close("dv", dv, wv, dtype)
 
 
+@pytest.mark.parametrize("seed", list(range(12)))
+def test_random_shapes_forward_and_backward(seed):
+    """Seeded sweep over sequence lengths (queries and keys), head layouts, head dims, mask kinds,
+    window sizes, query offsets and packings: out, dq, dk, dv against the oracle."""
+    rng = np.random.default_rng(1000 + seed)
+    d = int(rng.choice([64, 128]))
+    hkv = int(rng.choice([1, 2]))
+    hq = hkv * int(rng.choice([1, 2, 4]))
+    t = 128 * int(rng.integers(1, 8))
+    kind = str(rng.choice(["none", "causal", "sliding"]))
+    packed = bool(rng.integers(0, 2))
+    extra = 0 if packed else 128 * int(rng.integers(0, 4))     # segment ids need S == T
+    s_len = t + extra
+    q_off = 0 if kind == "none" else extra                     # the chunk ends where the keys end
+    window = int(rng.integers(0, s_len)) if kind == "sliding" else None
+    dtype = torch.bfloat16
+    q, k, v, do = _inputs(1, t, hq, hkv, d, dtype, s=s_len)
+    segs = ref.packed_segment_ids(seed, 1, t, max_docs=4) if packed else None
+    spec = ref.MaskSpec(causal=kind == "causal", sliding_window=window, segment_ids=segs,
+                        target_positions=torch.arange(q_off, q_off + t)[None],
+                        source_positions=torch.arange(s_len)[None])
+    mk = {"none": ops.MASK_NONE, "causal": ops.MASK_CAUSAL, "sliding": ops.MASK_SLIDING_WINDOW}[kind]
+    kw = dict(mask_kind=mk, sliding_window=window or 0, q_pos_offset=q_off, softmax_scale=d ** -0.5,
+              segment_ids=None if segs is None else segs.cuda())
+    case = f"d={d} hq={hq} hkv={hkv} t={t} s={s_len} {kind} window={window} packed={packed} q_off={q_off}"
+    want = ref.reference_mha(q, k, v, spec, softmax_scale=d ** -0.5)
+    wq, wk, wv = ref.reference_mha_grads(q, k, v, do, spec, softmax_scale=d ** -0.5)
+    qc, kc, vc, doc = q.cuda(), k.cuda(), v.cuda(), do.cuda()
+    out, lse = ops.flash_fwd(qc, kc, vc, **kw)
+    _assert_close("out " + case, out, want, dtype)
+    dq, dk, dv = ops.flash_bwd(qc, kc, vc, out, lse, doc, **kw)
+    _assert_close("dq " + case, dq, wq, dtype)
+    _assert_close("dk " + case, dk, wk, dtype)
+    _assert_close("dv " + case, dv, wv, dtype)
+
+
 @pytest.mark.parametrize("mask,window", [("none", None), ("causal", None), ("sliding", 200)])
 def test_arbitrary_segment_ids_forward_and_backward(mask, window):
     """Segment ids are compared for equality only (attention_bias.py:876-882): ids need not be sorted,
