@@ -480,9 +480,11 @@ template <int D, int GP>
 __global__ __launch_bounds__(256) void decode_combine_kernel(const DecArgs a) {
   __shared__ float sm[kMaxChunks * GP];   // record maxima, then rescale factors
   __shared__ float sl[kMaxChunks * GP];   // record sums
+  __shared__ int s_raw[kMaxChunks];       // the record table row
   __shared__ int s_list[kMaxChunks];      // records of this (sequence, kv head), in chunk order
   __shared__ int s_count;
   __shared__ float s_max[GP], s_inv[GP];
+  __shared__ float4 s_part[256];          // partial sums of the record slices
   const int hk = blockIdx.x, b = blockIdx.y;
   const int tid = threadIdx.x;
   int len = a.lengths[b];
@@ -491,12 +493,13 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecArgs a) {
   live_chunks(a, len, ch0, ch1);
   const int nc = ch1 - ch0;               // live chunks = upper bound on records of this (b, hk)
   const float c = a.scale * kLog2e;
-  if (tid < 64) {  // compact the record table row
-    const int32_t* row = a.ws_tab + ((int64_t)b * a.Hkv + hk) * a.nch;
+  // The whole table row in one round trip, then compacted in chunk order by one wavefront.
+  s_raw[tid] = tid < nc ? a.ws_tab[((int64_t)b * a.Hkv + hk) * a.nch + tid] : -1;
+  __syncthreads();
+  if (tid < 64) {
     int count = 0;
     for (int base = 0; base < nc; base += 64) {
-      const int i = base + tid;
-      const int r = i < nc ? row[i] : -1;
+      const int r = s_raw[base + tid];
       const unsigned long long mask = __builtin_amdgcn_ballot_w64(r >= 0);
       if (r >= 0) s_list[count + __builtin_popcountll(mask & ((1ull << tid) - 1))] = r;
       count += __builtin_popcountll(mask);
@@ -526,12 +529,39 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecArgs a) {
     s_inv[tid] = 1.f / l;
   }
   __syncthreads();
-  for (int idx = tid; idx < a.G * D; idx += 256) {
-    const int gq = idx / D;
-    float acc = 0.f;
-#pragma unroll 8
-    for (int ci = 0; ci < nl; ci++) acc += a.ws_o[(int64_t)s_list[ci] * (GP * D) + idx] * sm[ci * GP + gq];
-    a.out[((int64_t)b * a.Hq + hk * a.G) * D + idx] = (__bf16)(acc * s_inv[gq]);
+  // Output: G*D floats = n4 groups of four.  With fewer groups than threads the records are dealt
+  // to `ways` slices of threads (record ci to slice ci % ways), 16 loads in flight per thread,
+  // and the slices' partial sums are added in slice order.
+  const int n4 = a.G * D / 4;
+  const int per = min(n4, 256);
+  const int ways = 256 / per;
+  for (int base = 0; base < n4; base += per) {
+    const int way = tid / per, col = base + tid % per;
+    const bool live = way < ways && col < n4;
+    const int gq = live ? (4 * col) / D : 0;
+    float4 acc = {0.f, 0.f, 0.f, 0.f};
+    if (live) {
+#pragma unroll 16
+      for (int ci = way; ci < nl; ci += ways) {
+        const float4 o = *(const float4*)(a.ws_o + (int64_t)s_list[ci] * (GP * D) + 4 * col);
+        const float f = sm[ci * GP + gq];
+        acc.x += o.x * f; acc.y += o.y * f; acc.z += o.z * f; acc.w += o.w * f;
+      }
+    }
+    if (base > 0) __syncthreads();  // s_part of the previous pass has been read
+    s_part[tid] = acc;
+    __syncthreads();
+    if (live && way == 0) {
+      for (int w = 1; w < ways; w++) {
+        const float4 p = s_part[w * per + tid];
+        acc.x += p.x; acc.y += p.y; acc.z += p.z; acc.w += p.w;
+      }
+      const float inv = s_inv[gq];
+      union { bf16x2 p[2]; uint2 u; } pk;
+      pk.p[0] = pack_bf16(acc.x * inv, acc.y * inv);
+      pk.p[1] = pack_bf16(acc.z * inv, acc.w * inv);
+      *(uint2*)(a.out + ((int64_t)b * a.Hq + hk * a.G) * D + 4 * col) = pk.u;
+    }
   }
 }
 
