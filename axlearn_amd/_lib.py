@@ -15,7 +15,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libaxl_attn_hip.so")
 
-AXL_BF16, AXL_F32 = 0, 1
+AXL_BF16, AXL_F32, AXL_F16 = 0, 1, 2
 MASK_NONE, MASK_CAUSAL, MASK_SLIDING_WINDOW = 0, 1, 2
 AXL_OK, AXL_ERR_INVALID_ARGUMENT, AXL_ERR_UNSUPPORTED, AXL_ERR_WORKSPACE, AXL_ERR_LAUNCH = 0, -1, -2, -3, -4
 
@@ -195,7 +195,9 @@ def dtype_code(dtype: torch.dtype) -> int:
         return AXL_BF16
     if dtype == torch.float32:
         return AXL_F32
-    raise AxlError(AXL_ERR_UNSUPPORTED, f"dtype {dtype} (supported: bfloat16, float32)")
+    if dtype == torch.float16:
+        return AXL_F16
+    raise AxlError(AXL_ERR_UNSUPPORTED, f"dtype {dtype} (supported: bfloat16, float16, float32)")
 
 
 def strides4(t: torch.Tensor) -> AxlStrides:

@@ -48,7 +48,7 @@ static int check_flash_shapes(const char* who, int batch, int q_len, int kv_len,
                      "%s: num_q_heads %d is not divisible by num_kv_heads %d", who, hq, hkv);
   if (!(scale > 0.f) || !std::isfinite(scale))
     return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: softmax_scale must be finite and > 0", who);
-  if (dtype != AXL_BF16 && dtype != AXL_F32)
+  if (dtype != AXL_BF16 && dtype != AXL_F32 && dtype != AXL_F16)
     return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: unknown dtype %d", who, dtype);
   if (mask_kind < AXL_MASK_NONE || mask_kind > AXL_MASK_SLIDING_WINDOW)
     return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: unknown mask_kind %d", who, mask_kind);
@@ -82,6 +82,8 @@ AuxArgs make_aux_args(const AxlAttnAux& x, float softmax_scale) {
 int check_aux(const char* who, const AxlAttnAux& x, int batch, int hq, int q_len, int kv_len) {
   (void)batch; (void)hq; (void)q_len;
   if (x.bias) {
+    if (x.bias_dtype == AXL_F16)
+      return set_error(AXL_ERR_UNSUPPORTED, "%s: an fp16 bias is not supported (pass it as fp32 or bf16)", who);
     if (x.bias_dtype != AXL_BF16 && x.bias_dtype != AXL_F32)
       return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: unknown bias dtype %d", who, x.bias_dtype);
     const int64_t m = x.bias_dtype == AXL_F32 ? 4 : 8;
@@ -119,7 +121,7 @@ int axl_paged_kv_insert(const AxlPageInsertParams* p, void* stream) {
   if (p->batch <= 0 || p->num_kv_heads <= 0 || p->head_dim <= 0 || p->num_pages <= 0 ||
       p->page_size <= 0 || p->pages_per_seq <= 0)
     return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: non-positive dimension", who);
-  if (p->dtype != AXL_BF16 && p->dtype != AXL_F32)
+  if (p->dtype != AXL_BF16 && p->dtype != AXL_F32 && p->dtype != AXL_F16)
     return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: unknown dtype %d", who, p->dtype);
   if (!p->page_indices || !p->key_positions)
     return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: null page_indices / key_positions", who);
@@ -149,7 +151,7 @@ int axl_flash_fwd(const AxlFlashFwdParams* p, void* stream) {
   if (rc != AXL_OK) return rc;
   if (!p->q || !p->k || !p->v || !p->out)
     return set_error(AXL_ERR_INVALID_ARGUMENT, "axl_flash_fwd: NULL tensor pointer");
-  const int eb = p->dtype == AXL_BF16 ? 2 : 4;
+  const int eb = p->dtype == AXL_F32 ? 4 : 2;
   if (!aligned16(p->q) || !aligned16(p->k) || !aligned16(p->v) || !aligned16(p->out) ||
       !strides_ok(p->q_strides, eb) || !strides_ok(p->k_strides, eb) ||
       !strides_ok(p->v_strides, eb) || !strides_ok(p->out_strides, eb))
@@ -180,7 +182,7 @@ int axl_flash_bwd_phases(const AxlFlashBwdParams* p, int phases, void* stream) {
   if (rc != AXL_OK) return rc;
   if (!p->q || !p->k || !p->v || !p->out || !p->d_out || !p->lse || !p->dq || !p->dk || !p->dv)
     return set_error(AXL_ERR_INVALID_ARGUMENT, "axl_flash_bwd: NULL tensor pointer");
-  const int eb = p->dtype == AXL_BF16 ? 2 : 4;
+  const int eb = p->dtype == AXL_F32 ? 4 : 2;
   const void* ptrs[] = {p->q, p->k, p->v, p->out, p->d_out, p->dq, p->dk, p->dv};
   for (const void* x : ptrs)
     if (!aligned16(x))
@@ -212,8 +214,8 @@ static int check_decode_common(const char* who, int batch, int hq, int hkv, int 
                      "%s: num_q_heads %d is not divisible by num_kv_heads %d", who, hq, hkv);
   if (!(scale > 0.f) || !std::isfinite(scale))
     return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: softmax_scale must be finite and > 0", who);
-  if (dtype != AXL_BF16)
-    return set_error(AXL_ERR_UNSUPPORTED, "%s: only bf16 is supported", who);
+  if (dtype != AXL_BF16 && dtype != AXL_F16)
+    return set_error(AXL_ERR_UNSUPPORTED, "%s: only bf16 and fp16 are supported", who);
   if (d != 128 && d != 64)
     return set_error(AXL_ERR_UNSUPPORTED, "%s: head_dim %d (supported: 64, 128)", who, d);
   if (hq / hkv > 16)

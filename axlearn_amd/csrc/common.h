@@ -56,6 +56,72 @@ __device__ __forceinline__ bf16x8 pack_bf16x8(float a0, float a1, float a2, floa
   return u.v;
 }
 
+typedef __attribute__((__vector_size__(8 * sizeof(_Float16)))) _Float16 halfx8;
+typedef __attribute__((__vector_size__(4 * sizeof(_Float16)))) _Float16 halfx4;
+typedef __attribute__((__vector_size__(2 * sizeof(_Float16)))) _Float16 halfx2;
+
+// Element type of the 16-bit kernels (template parameter E).  Operands travel through global
+// memory, LDS and registers as plain 16-bit patterns in the bf16x2 / bf16x8 / shortx4 carriers
+// whatever the type; only the matrix instructions, the rounding of fp32 results to 16 bits and
+// the widening of single elements differ.  Both roundings are to nearest even.
+struct ElemBf16 {
+  static constexpr int kDtype = AXL_BF16;
+  static __device__ __forceinline__ floatx16 mfma_32x32x16(bf16x8 a, bf16x8 b, floatx16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ floatx4 mfma_16x16x32(bf16x8 a, bf16x8 b, floatx4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ floatx4 mfma_16x16x16(shortx4 a, shortx4 b, floatx4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, b, c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ bf16x2 pack(float a, float b) { return pack_bf16(a, b); }
+  static __device__ __forceinline__ float dot2(bf16x2 a, bf16x2 b, float c) {
+    return __builtin_amdgcn_fdot2_f32_bf16(a, b, c, false);
+  }
+  static __device__ __forceinline__ float widen(__bf16 bits) { return (float)bits; }
+  static __device__ __forceinline__ __bf16 narrow(float x) { return (__bf16)x; }
+};
+struct ElemF16 {
+  static constexpr int kDtype = AXL_F16;
+  static __device__ __forceinline__ floatx16 mfma_32x32x16(bf16x8 a, bf16x8 b, floatx16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, a), __builtin_bit_cast(halfx8, b), c,
+                                                  0, 0, 0);
+  }
+  static __device__ __forceinline__ floatx4 mfma_16x16x32(bf16x8 a, bf16x8 b, floatx4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(halfx8, a), __builtin_bit_cast(halfx8, b), c,
+                                                  0, 0, 0);
+  }
+  static __device__ __forceinline__ floatx4 mfma_16x16x16(shortx4 a, shortx4 b, floatx4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(halfx4, a), __builtin_bit_cast(halfx4, b), c, 0,
+                                                 0, 0);
+  }
+  static __device__ __forceinline__ bf16x2 pack(float a, float b) {
+    floatx2 v = {a, b};
+    return __builtin_bit_cast(bf16x2, __builtin_convertvector(v, halfx2));
+  }
+  static __device__ __forceinline__ float dot2(bf16x2 a, bf16x2 b, float c) {
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(halfx2, a), __builtin_bit_cast(halfx2, b), c, false);
+  }
+  static __device__ __forceinline__ float widen(__bf16 bits) { return (float)__builtin_bit_cast(_Float16, bits); }
+  static __device__ __forceinline__ __bf16 narrow(float x) { return __builtin_bit_cast(__bf16, (_Float16)x); }
+};
+
+// Eight fp32 -> one MFMA operand of element type E.
+template <typename E>
+__device__ __forceinline__ bf16x8 pack8(float a0, float a1, float a2, float a3, float a4, float a5, float a6,
+                                        float a7) {
+  union {
+    bf16x8 v;
+    bf16x2 p[4];
+  } u;
+  u.p[0] = E::pack(a0, a1);
+  u.p[1] = E::pack(a2, a3);
+  u.p[2] = E::pack(a4, a5);
+  u.p[3] = E::pack(a6, a7);
+  return u.v;
+}
+
 // Transposing LDS read (ds_read_b64_tr_b16).  Within each group of 16 lanes, lane j supplies the
 // address of 4 contiguous 16-bit elements; lane i receives, as element e, element (i % 4) of the
 // data addressed by lane 4*e + i/4.  With lane j pointing at row (j / 4), columns 4*(j % 4)..+3 of

@@ -25,13 +25,13 @@ struct BwdArgs {
   AuxArgs aux;  // dense bias / dropout mask (read only by the AUX instantiations)
 };
 
-// Enqueues the dK/dV kernel (bf16) for head_dim 64 or 128; `aux` selects the instantiation that
-// reads the dense bias / dropout mask.
-hipError_t launch_bwd_dkdv_bf16(const BwdArgs& a, int head_dim, bool aux, hipStream_t stream);
+// Enqueues the dK/dV kernel for `dtype` AXL_BF16 or AXL_F16 and head_dim 64 or 128; `aux` selects
+// the instantiation that reads the dense bias / dropout mask.
+hipError_t launch_bwd_dkdv(const BwdArgs& a, int dtype, int head_dim, bool aux, hipStream_t stream);
 
-// Enqueues the dQ kernel (bf16, no dense bias / dropout mask) for head_dim 64 or 128.  With
-// `fuse_delta` it also writes delta and the scaled lse into the workspace (instead of reading them),
-// for a dK/dV kernel enqueued after it.
-hipError_t launch_bwd_dq_bf16(const BwdArgs& a, int head_dim, bool fuse_delta, hipStream_t stream);
+// Enqueues the dQ kernel (no dense bias / dropout mask) for `dtype` AXL_BF16 or AXL_F16 and head_dim
+// 64 or 128.  With `fuse_delta` it also writes delta and the scaled lse into the workspace (instead
+// of reading them), for a dK/dV kernel enqueued after it.
+hipError_t launch_bwd_dq(const BwdArgs& a, int dtype, int head_dim, bool fuse_delta, hipStream_t stream);
 
 }  // namespace axl

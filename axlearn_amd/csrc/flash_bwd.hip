@@ -105,8 +105,8 @@ struct DqTile {
   static constexpr int LDS_BYTES = 4 * TILE_BYTES;  // {K, V} x double buffer
 };
 
-template <int D, bool AUX>
-__global__ __launch_bounds__(256) void flash_bwd_dq_bf16_kernel(const BwdArgs a) {
+template <typename E, int D, bool AUX>
+__global__ __launch_bounds__(256) void flash_bwd_dq_aux_kernel(const BwdArgs a) {
   using Tile = DqTile<D>;
   constexpr int KK = D / 16, DT = D / 32;
   extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -223,12 +223,12 @@ __global__ __launch_bounds__(256) void flash_bwd_dq_bf16_kernel(const BwdArgs a)
 #pragma unroll
         for (int kk = 0; kk < KK; kk++) {
           const bf16x8 kfr = *(const bf16x8*)(ka + kk * 32);
-          s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr, qf[kk], s, 0, 0, 0);
+          s = E::mfma_32x32x16(kfr, qf[kk], s);
         }
 #pragma unroll
         for (int kk = 0; kk < KK; kk++) {
           const bf16x8 vfr = *(const bf16x8*)(va + kk * 32);
-          dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr, dof[kk], dp, 0, 0, 0);
+          dp = E::mfma_32x32x16(vfr, dof[kk], dp);
         }
         // Register r of lane group g is key k0 + 32ks + 16(r/8) + 8g + (r%8); the lane is a query.
         if constexpr (AUX) {
@@ -284,7 +284,7 @@ __global__ __launch_bounds__(256) void flash_bwd_dq_bf16_kernel(const BwdArgs a)
         // dQ^T[d][q] += K^T[d][key] dS^T[key][q].
 #pragma unroll
         for (int t8 = 0; t8 < 2; t8++) {
-          const bf16x8 dsb = pack_bf16x8(dp[8 * t8 + 0], dp[8 * t8 + 1], dp[8 * t8 + 2], dp[8 * t8 + 3],
+          const bf16x8 dsb = pack8<E>(dp[8 * t8 + 0], dp[8 * t8 + 1], dp[8 * t8 + 2], dp[8 * t8 + 3],
                                          dp[8 * t8 + 4], dp[8 * t8 + 5], dp[8 * t8 + 6], dp[8 * t8 + 7]);
           const char* kta = kt + (32 * ks + 16 * t8) * Tile::STRIDE + tr_off;
 #pragma unroll
@@ -292,7 +292,7 @@ __global__ __launch_bounds__(256) void flash_bwd_dq_bf16_kernel(const BwdArgs a)
             union { bf16x8 v; shortx4 hlf[2]; } fa;
             fa.hlf[0] = lds_read_tr16(kta + dt * 64);
             fa.hlf[1] = lds_read_tr16(kta + dt * 64 + 4 * Tile::STRIDE);
-            dq_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa.v, dsb, dq_acc[dt], 0, 0, 0);
+            dq_acc[dt] = E::mfma_32x32x16(fa.v, dsb, dq_acc[dt]);
           }
         }
       }
@@ -311,8 +311,8 @@ __global__ __launch_bounds__(256) void flash_bwd_dq_bf16_kernel(const BwdArgs a)
 #pragma unroll
     for (int rq = 0; rq < 4; rq++) {
       union { bf16x2 p[2]; uint2 u; } w;
-      w.p[0] = pack_bf16(dq_acc[dt][4 * rq + 0] * a.scale, dq_acc[dt][4 * rq + 1] * a.scale);
-      w.p[1] = pack_bf16(dq_acc[dt][4 * rq + 2] * a.scale, dq_acc[dt][4 * rq + 3] * a.scale);
+      w.p[0] = E::pack(dq_acc[dt][4 * rq + 0] * a.scale, dq_acc[dt][4 * rq + 1] * a.scale);
+      w.p[1] = E::pack(dq_acc[dt][4 * rq + 2] * a.scale, dq_acc[dt][4 * rq + 3] * a.scale);
       *(uint2*)(dqp + 32 * dt + 8 * rq + 4 * g) = w.u;
     }
 }
@@ -325,8 +325,9 @@ size_t flash_bwd_workspace_bytes(const AxlFlashBwdParams& p) {
 }
 
 int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream) {
-  if (p.dtype != AXL_BF16)
-    return set_error(AXL_ERR_UNSUPPORTED, "axl_flash_bwd: only bf16 is supported");
+  if (p.dtype != AXL_BF16 && p.dtype != AXL_F16)
+    return set_error(AXL_ERR_UNSUPPORTED, "axl_flash_bwd: only bf16 and fp16 are supported");
+  const int dt = p.dtype;
   BwdArgs a;
   a.q = p.q; a.k = p.k; a.v = p.v; a.out = p.out; a.dout = p.d_out; a.lse = p.lse;
   a.delta = (float*)p.workspace;
@@ -359,23 +360,28 @@ int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream)
   // on the way (it holds the dO rows anyway) and runs first; the dK/dV kernel reads what it left.
   const int all = AXL_BWD_DELTA | AXL_BWD_DKDV | AXL_BWD_DQ;
   if ((phases & all) == all && !aux && !p.d_logit_sink) {
-    err = launch_bwd_dq_bf16(a, p.head_dim, true, stream);
-    if (err == hipSuccess) err = launch_bwd_dkdv_bf16(a, p.head_dim, false, stream);
+    err = launch_bwd_dq(a, dt, p.head_dim, true, stream);
+    if (err == hipSuccess) err = launch_bwd_dkdv(a, dt, p.head_dim, false, stream);
     if (err != hipSuccess)
       return set_error(AXL_ERR_LAUNCH, "axl_flash_bwd: launch failed: %s", hipGetErrorString(err));
     return AXL_OK;
   }
-  if (p.head_dim == 128) {
-    if (phases & AXL_BWD_DELTA) AXL_LAUNCH((bwd_delta_kernel<__bf16, 128>), delta_grid, 0);
-    if ((phases & AXL_BWD_DKDV) && err == hipSuccess) err = launch_bwd_dkdv_bf16(a, 128, aux, stream);
-    if ((phases & AXL_BWD_DQ) && aux) AXL_LAUNCH((flash_bwd_dq_bf16_kernel<128, true>), dq_grid, DqTile<128>::LDS_BYTES);
-    if ((phases & AXL_BWD_DQ) && !aux && err == hipSuccess) err = launch_bwd_dq_bf16(a, 128, false, stream);
+#define AXL_BWD_PHASES(E, T, DD)                                                                  \
+  do {                                                                                            \
+    if (phases & AXL_BWD_DELTA) AXL_LAUNCH((bwd_delta_kernel<T, DD>), delta_grid, 0);             \
+    if ((phases & AXL_BWD_DKDV) && err == hipSuccess) err = launch_bwd_dkdv(a, dt, DD, aux, stream); \
+    if ((phases & AXL_BWD_DQ) && aux)                                                             \
+      AXL_LAUNCH((flash_bwd_dq_aux_kernel<E, DD, true>), dq_grid, DqTile<DD>::LDS_BYTES);         \
+    if ((phases & AXL_BWD_DQ) && !aux && err == hipSuccess) err = launch_bwd_dq(a, dt, DD, false, stream); \
+  } while (0)
+  if (dt == AXL_BF16) {
+    if (p.head_dim == 128) AXL_BWD_PHASES(ElemBf16, __bf16, 128);
+    else AXL_BWD_PHASES(ElemBf16, __bf16, 64);
   } else {
-    if (phases & AXL_BWD_DELTA) AXL_LAUNCH((bwd_delta_kernel<__bf16, 64>), delta_grid, 0);
-    if ((phases & AXL_BWD_DKDV) && err == hipSuccess) err = launch_bwd_dkdv_bf16(a, 64, aux, stream);
-    if ((phases & AXL_BWD_DQ) && aux) AXL_LAUNCH((flash_bwd_dq_bf16_kernel<64, true>), dq_grid, DqTile<64>::LDS_BYTES);
-    if ((phases & AXL_BWD_DQ) && !aux && err == hipSuccess) err = launch_bwd_dq_bf16(a, 64, false, stream);
+    if (p.head_dim == 128) AXL_BWD_PHASES(ElemF16, _Float16, 128);
+    else AXL_BWD_PHASES(ElemF16, _Float16, 64);
   }
+#undef AXL_BWD_PHASES
 #undef AXL_LAUNCH
   if ((phases & AXL_BWD_DELTA) && p.d_logit_sink && err == hipSuccess) {
     hipLaunchKernelGGL(bwd_dsink_kernel, dim3(p.num_q_heads), dim3(256), 0, stream, p.logit_sink,

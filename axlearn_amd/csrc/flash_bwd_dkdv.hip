@@ -47,9 +47,9 @@ struct DkvTile {
 constexpr int kMaxSubDkv = 1024;                 // query tiles whose segment ids the dK/dV kernel classifies
 constexpr int kNotUniformDkv = -0x7fffffff - 1;  // marks a tile with more than one segment id
 
-template <int D, bool HAS_SEG, bool AUX>
+template <typename E, int D, bool HAS_SEG, bool AUX>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
-void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
+void flash_bwd_dkdv_kernel(const BwdArgs a) {
   using Tile = DkvTile<D>;
   constexpr int KK = D / 16, DT = D / 32;
   constexpr int NA = 2 * KK;          // stage-A MFMAs per tile
@@ -286,16 +286,16 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
   }
 #define AXL_PACK_PAIR(PB_, DSB_, I_)                                    \
   {                                                                     \
-    PB_.p[I_] = pack_bf16(s_e[2 * (I_)], s_e[2 * (I_) + 1]);            \
-    DSB_.p[I_] = pack_bf16(dp_e[2 * (I_)], dp_e[2 * (I_) + 1]);         \
+    PB_.p[I_] = E::pack(s_e[2 * (I_)], s_e[2 * (I_) + 1]);            \
+    DSB_.p[I_] = E::pack(dp_e[2 * (I_)], dp_e[2 * (I_) + 1]);         \
   }
   // Stage A of the tile in BUF_ into (S_, DP_), not interleaved with anything (pipeline fill).
 #define AXL_STAGE_A_PLAIN(BUF_, S_, DP_)                                                        \
   _Pragma("unroll") for (int kk = 0; kk < KK; kk++) {                                           \
     const bf16x8 qa_ = AXL_A_FRAG(BUF_, 0, kk);                                                 \
     const bf16x8 da_ = AXL_A_FRAG(BUF_, 1, kk);                                                 \
-    S_ = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa_, kf[kk], S_, 0, 0, 0);                     \
-    DP_ = __builtin_amdgcn_mfma_f32_32x32x16_bf16(da_, vf[kk], DP_, 0, 0, 0);                   \
+    S_ = E::mfma_32x32x16(qa_, kf[kk], S_);                     \
+    DP_ = E::mfma_32x32x16(da_, vf[kk], DP_);                   \
   }
   union TrFrag {
     bf16x8 v;
@@ -441,15 +441,15 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
       if constexpr (n < NB) {
         constexpr int t8 = n / (2 * DT), dt = (n % (2 * DT)) / 2;
         if constexpr (n % 2 == 0)
-          dv_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[n].v, pb.v[t8], dv_acc[dt], 0, 0, 0);
+          dv_acc[dt] = E::mfma_32x32x16(bfr[n].v, pb.v[t8], dv_acc[dt]);
         else
-          dk_acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[n].v, dsb.v[t8], dk_acc[dt], 0, 0, 0);
+          dk_acc[dt] = E::mfma_32x32x16(bfr[n].v, dsb.v[t8], dk_acc[dt]);
       } else {
         constexpr int x = n - NB;
         if constexpr (x % 2 == 0)
-          s_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afr[x], kf[x / 2], x == 0 ? zero16 : s_a, 0, 0, 0);
+          s_a = E::mfma_32x32x16(afr[x], kf[x / 2], x == 0 ? zero16 : s_a);
         else
-          dp_a = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afr[x], vf[x / 2], x == 1 ? zero16 : dp_a, 0, 0, 0);
+          dp_a = E::mfma_32x32x16(afr[x], vf[x / 2], x == 1 ? zero16 : dp_a);
       }
       // ---- elementwise stage of tile j+1: element e starts in slot e (NS-3)/16 and takes three
       // slots; pairs are packed one slot after their second element is complete
@@ -614,20 +614,20 @@ void flash_bwd_dkdv_bf16_kernel(const BwdArgs a) {
         bf16x2 p[2];
         uint2 u;
       } w;
-      w.p[0] = pack_bf16(dk_acc[dt][4 * rq + 0] * a.scale, dk_acc[dt][4 * rq + 1] * a.scale);
-      w.p[1] = pack_bf16(dk_acc[dt][4 * rq + 2] * a.scale, dk_acc[dt][4 * rq + 3] * a.scale);
+      w.p[0] = E::pack(dk_acc[dt][4 * rq + 0] * a.scale, dk_acc[dt][4 * rq + 1] * a.scale);
+      w.p[1] = E::pack(dk_acc[dt][4 * rq + 2] * a.scale, dk_acc[dt][4 * rq + 3] * a.scale);
       *(uint2*)(dkp + 32 * dt + 8 * rq + 4 * g) = w.u;
       const float vs = AUX ? a.aux.keep_scale : 1.0f;  // kept probabilities are P / (1 - rate)
-      w.p[0] = pack_bf16(dv_acc[dt][4 * rq + 0] * vs, dv_acc[dt][4 * rq + 1] * vs);
-      w.p[1] = pack_bf16(dv_acc[dt][4 * rq + 2] * vs, dv_acc[dt][4 * rq + 3] * vs);
+      w.p[0] = E::pack(dv_acc[dt][4 * rq + 0] * vs, dv_acc[dt][4 * rq + 1] * vs);
+      w.p[1] = E::pack(dv_acc[dt][4 * rq + 2] * vs, dv_acc[dt][4 * rq + 3] * vs);
       *(uint2*)(dvp + 32 * dt + 8 * rq + 4 * g) = w.u;
     }
 }
 
-template <int D, bool HAS_SEG, bool AUX>
+template <typename E, int D, bool HAS_SEG, bool AUX>
 static hipError_t launch_one(const BwdArgs& a, hipStream_t stream) {
   using Tile = DkvTile<D>;
-  auto kernel = flash_bwd_dkdv_bf16_kernel<D, HAS_SEG, AUX>;
+  auto kernel = flash_bwd_dkdv_kernel<E, D, HAS_SEG, AUX>;
   hipError_t err = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                                        Tile::LDS_BYTES);
   if (err != hipSuccess) return err;
@@ -636,14 +636,22 @@ static hipError_t launch_one(const BwdArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
-hipError_t launch_bwd_dkdv_bf16(const BwdArgs& a, int head_dim, bool aux, hipStream_t stream) {
+template <typename E>
+static hipError_t launch_for(const BwdArgs& a, int head_dim, bool aux, hipStream_t stream) {
   const bool seg = a.seg != nullptr;
   if (aux) {
-    if (head_dim == 128) return seg ? launch_one<128, true, true>(a, stream) : launch_one<128, false, true>(a, stream);
-    return seg ? launch_one<64, true, true>(a, stream) : launch_one<64, false, true>(a, stream);
+    if (head_dim == 128)
+      return seg ? launch_one<E, 128, true, true>(a, stream) : launch_one<E, 128, false, true>(a, stream);
+    return seg ? launch_one<E, 64, true, true>(a, stream) : launch_one<E, 64, false, true>(a, stream);
   }
-  if (head_dim == 128) return seg ? launch_one<128, true, false>(a, stream) : launch_one<128, false, false>(a, stream);
-  return seg ? launch_one<64, true, false>(a, stream) : launch_one<64, false, false>(a, stream);
+  if (head_dim == 128)
+    return seg ? launch_one<E, 128, true, false>(a, stream) : launch_one<E, 128, false, false>(a, stream);
+  return seg ? launch_one<E, 64, true, false>(a, stream) : launch_one<E, 64, false, false>(a, stream);
+}
+
+hipError_t launch_bwd_dkdv(const BwdArgs& a, int dtype, int head_dim, bool aux, hipStream_t stream) {
+  return dtype == AXL_F16 ? launch_for<ElemF16>(a, head_dim, aux, stream)
+                          : launch_for<ElemBf16>(a, head_dim, aux, stream);
 }
 
 }  // namespace axl

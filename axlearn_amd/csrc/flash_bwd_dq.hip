@@ -48,7 +48,7 @@ constexpr int kNotUniform = -0x7fffffff - 1;  // marks a sub-tile with more than
 // FUSE_DELTA: the kernel also computes delta = rowsum(out * dO) (gpu_attention.py:653-658) and the
 // scaled lse of its own rows and leaves both in the workspace for the dK/dV kernel, which then has to
 // run after this one; the separate delta pass is not needed.
-template <int D, bool HAS_SEG, int NW, bool FUSE_DELTA>
+template <typename E, int D, bool HAS_SEG, int NW, bool FUSE_DELTA>
 __global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(NW / 4, NW / 4)))
 void flash_bwd_dq_ring_kernel(const BwdArgs a) {
   using Tile = DqRing<D, HAS_SEG, NW>;
@@ -93,7 +93,7 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
       o.v = *(const bf16x8*)(op + 16 * kk + 8 * g);
       d.v = dof[kk];
 #pragma unroll
-      for (int i = 0; i < 4; i++) part = __builtin_amdgcn_fdot2_f32_bf16(o.p[i], d.p[i], part, false);
+      for (int i = 0; i < 4; i++) part = E::dot2(o.p[i], d.p[i], part);
     }
     delta = xor32_sum(part);
     off = a.lse[stat_idx] * (-kLog2e);
@@ -283,8 +283,8 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
   _Pragma("unroll") for (int kk = 0; kk < KK; kk++) {                                           \
     const bf16x8 ka_ = *(const bf16x8*)((BUF_) + (SUB_) * Tile::SUB_BYTES + a_off[kk]);         \
     const bf16x8 va_ = *(const bf16x8*)((BUF_) + Tile::TILE_BYTES + (SUB_) * Tile::SUB_BYTES + a_off[kk]); \
-    S_ = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka_, qf[kk], S_, 0, 0, 0);                     \
-    DP_ = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va_, dof[kk], DP_, 0, 0, 0);                  \
+    S_ = E::mfma_32x32x16(ka_, qf[kk], S_);                     \
+    DP_ = E::mfma_32x32x16(va_, dof[kk], DP_);                  \
   }
 
   constexpr int NS = NA + NB;          // MFMAs per step: stage B of sub-tile j, then stage A of sub-tile j+2
@@ -317,7 +317,7 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
 #pragma unroll
     for (int r = 0; r < 16; r++) AXL_ELEM(s1, dp1, sg1, qpos - 8 * g - key0, r, true)
 #pragma unroll
-    for (int i = 0; i < 8; i++) ds0.p[i] = pack_bf16(dp1[2 * i], dp1[2 * i + 1]);
+    for (int i = 0; i < 8; i++) ds0.p[i] = E::pack(dp1[2 * i], dp1[2 * i + 1]);
     AXL_STAGE_A_PLAIN(buf_b, 1, s0, dp0)
     if (HAS_SEG) {
       AXL_READ_SEG_PART(buf_b, 1, 0, sg0)
@@ -354,13 +354,13 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
       /* ---- the MFMA of this slot.  Stage-B step m = t8 * DT + dt; stage-A step x: even -> S chain  \
          with K fragment x/2, odd -> dP chain with V fragment x/2. */                                  \
       if (n < NB) {                                                                                    \
-        dq_acc[n % DT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[n].v, DSB_.v[n / DT], dq_acc[n % DT], 0, 0, 0); \
+        dq_acc[n % DT] = E::mfma_32x32x16(bfr[n].v, DSB_.v[n / DT], dq_acc[n % DT]); \
       } else {                                                                                         \
         const int x = n - NB;                                                                          \
         if (x % 2 == 0)                                                                                \
-          S_A = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afr[x], qf[x / 2], x == 0 ? zero16 : S_A, 0, 0, 0); \
+          S_A = E::mfma_32x32x16(afr[x], qf[x / 2], x == 0 ? zero16 : S_A); \
         else                                                                                           \
-          DP_A = __builtin_amdgcn_mfma_f32_32x32x16_bf16(afr[x], dof[x / 2], x == 1 ? ndelta16 : DP_A, 0, 0, 0); \
+          DP_A = E::mfma_32x32x16(afr[x], dof[x / 2], x == 1 ? ndelta16 : DP_A); \
       }                                                                                                \
       /* ---- first stage-B fragments of sub-tile j+1 (read in the next step's first slots) */         \
       if (n >= NS - kAheadB) {                                                                         \
@@ -375,7 +375,7 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
         if (e * (NS - 3) / 16 == n) AXL_ELEM_1(S_E, SEG_E, diff0, e, MASKED_)                          \
       }                                                                                                \
       _Pragma("unroll") for (int i = 0; i < 8; i++)                                                    \
-        if ((2 * i + 1) * (NS - 3) / 16 + 3 == n) DSB_N.p[i] = pack_bf16(DP_E[2 * i], DP_E[2 * i + 1]); \
+        if ((2 * i + 1) * (NS - 3) / 16 + 3 == n) DSB_N.p[i] = E::pack(DP_E[2 * i], DP_E[2 * i + 1]); \
       /* ---- tile t+3: advance the cursor, then one direct-to-LDS load per slot */                    \
       if ((H_) * NS + n == LD_SLOT0 - 1) AXL_ADVANCE()                                                 \
       if ((H_) * NS + n == LD_SLOT0) AXL_DMA(lds_s, 0)                                                 \
@@ -509,8 +509,8 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
         bf16x2 p[2];
         uint2 u;
       } w;
-      w.p[0] = pack_bf16(dq_acc[dt][4 * rq + 0] * a.scale, dq_acc[dt][4 * rq + 1] * a.scale);
-      w.p[1] = pack_bf16(dq_acc[dt][4 * rq + 2] * a.scale, dq_acc[dt][4 * rq + 3] * a.scale);
+      w.p[0] = E::pack(dq_acc[dt][4 * rq + 0] * a.scale, dq_acc[dt][4 * rq + 1] * a.scale);
+      w.p[1] = E::pack(dq_acc[dt][4 * rq + 2] * a.scale, dq_acc[dt][4 * rq + 3] * a.scale);
       *(uint2*)(dqp + 32 * dt + 8 * rq + 4 * g) = w.u;
     }
 }
@@ -518,11 +518,11 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
 #ifndef AXL_DQ_WAVES
 #define AXL_DQ_WAVES 4
 #endif
-template <int D, bool HAS_SEG, bool FUSE_DELTA>
+template <typename E, int D, bool HAS_SEG, bool FUSE_DELTA>
 static hipError_t launch_one(const BwdArgs& a, hipStream_t stream) {
   constexpr int NW = AXL_DQ_WAVES;
   using Tile = DqRing<D, HAS_SEG, NW>;
-  auto kernel = flash_bwd_dq_ring_kernel<D, HAS_SEG, NW, FUSE_DELTA>;
+  auto kernel = flash_bwd_dq_ring_kernel<E, D, HAS_SEG, NW, FUSE_DELTA>;
   hipError_t err = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
                                        Tile::LDS_BYTES);
   if (err != hipSuccess) return err;
@@ -531,14 +531,22 @@ static hipError_t launch_one(const BwdArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
-hipError_t launch_bwd_dq_bf16(const BwdArgs& a, int head_dim, bool fuse_delta, hipStream_t stream) {
+template <typename E>
+static hipError_t launch_for(const BwdArgs& a, int head_dim, bool fuse_delta, hipStream_t stream) {
   const bool seg = a.seg != nullptr;
   if (fuse_delta) {
-    if (head_dim == 128) return seg ? launch_one<128, true, true>(a, stream) : launch_one<128, false, true>(a, stream);
-    return seg ? launch_one<64, true, true>(a, stream) : launch_one<64, false, true>(a, stream);
+    if (head_dim == 128)
+      return seg ? launch_one<E, 128, true, true>(a, stream) : launch_one<E, 128, false, true>(a, stream);
+    return seg ? launch_one<E, 64, true, true>(a, stream) : launch_one<E, 64, false, true>(a, stream);
   }
-  if (head_dim == 128) return seg ? launch_one<128, true, false>(a, stream) : launch_one<128, false, false>(a, stream);
-  return seg ? launch_one<64, true, false>(a, stream) : launch_one<64, false, false>(a, stream);
+  if (head_dim == 128)
+    return seg ? launch_one<E, 128, true, false>(a, stream) : launch_one<E, 128, false, false>(a, stream);
+  return seg ? launch_one<E, 64, true, false>(a, stream) : launch_one<E, 64, false, false>(a, stream);
+}
+
+hipError_t launch_bwd_dq(const BwdArgs& a, int dtype, int head_dim, bool fuse_delta, hipStream_t stream) {
+  return dtype == AXL_F16 ? launch_for<ElemF16>(a, head_dim, fuse_delta, stream)
+                          : launch_for<ElemBf16>(a, head_dim, fuse_delta, stream);
 }
 
 }  // namespace axl

@@ -58,9 +58,9 @@ struct FwdTile {
 constexpr int kMaxSegTiles = 1024;               // key tiles whose segment ids the forward classifies
 constexpr int kSegNotUniform = -0x7fffffff - 1;  // marks a tile with more than one segment id
 
-template <int D, bool AUX>
+template <typename E, int D, bool AUX>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
-void flash_fwd_bf16_kernel(const FwdArgs a) {
+void flash_fwd_kernel(const FwdArgs a) {
   using Tile = FwdTile<D>;
   constexpr int KK = D / 16;  // MFMA k-steps over head_dim
   constexpr int DT = D / 32;  // 32-row output tiles over head_dim
@@ -219,7 +219,7 @@ void flash_fwd_bf16_kernel(const FwdArgs a) {
       _Pragma("unroll") for (int r = 0; r < 16; r++) S_[ks][r] = 0.f;                                \
     _Pragma("unroll") for (int kk = 0; kk < KK; kk++)                                                \
       _Pragma("unroll") for (int ks = 0; ks < 2; ks++)                                               \
-        S_[ks] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(AXL_K_FRAG(KT_, kk, ks), qf[kk], S_[ks], 0, 0, 0); \
+        S_[ks] = E::mfma_32x32x16(AXL_K_FRAG(KT_, kk, ks), qf[kk], S_[ks]); \
   }
 
   // Pipeline fill: S^T of the first tile.
@@ -361,9 +361,9 @@ void flash_fwd_bf16_kernel(const FwdArgs a) {
         if (n + kAhead < NSL) kfr[n + kAhead] = AXL_K_FRAG(kt, (n + kAhead) / 2, (n + kAhead) % 2);
         if (n < 2) {
           const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-          s_nxt[n % 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr[n], qf[n / 2], zero16, 0, 0, 0);
+          s_nxt[n % 2] = E::mfma_32x32x16(kfr[n], qf[n / 2], zero16);
         } else {
-          s_nxt[n % 2] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfr[n], qf[n / 2], s_nxt[n % 2], 0, 0, 0);
+          s_nxt[n % 2] = E::mfma_32x32x16(kfr[n], qf[n / 2], s_nxt[n % 2]);
         }
 #pragma unroll
         for (int e = 0; e < EPS; e++) {
@@ -372,7 +372,7 @@ void flash_fwd_bf16_kernel(const FwdArgs a) {
           lsum += p;
           const float pu = after_dropout(idx, p);
           s[idx / 16][idx % 16] = pu;
-          if (idx % 2 == 1) pb.p[idx / 2] = pack_bf16(s[idx / 16][idx % 16 - 1], pu);
+          if (idx % 2 == 1) pb.p[idx / 2] = E::pack(s[idx / 16][idx % 16 - 1], pu);
         }
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -383,7 +383,7 @@ void flash_fwd_bf16_kernel(const FwdArgs a) {
         lsum += p;
         const float pu = after_dropout(idx, p);
         s[idx / 16][idx % 16] = pu;
-        if (idx % 2 == 1) pb.p[idx / 2] = pack_bf16(s[idx / 16][idx % 16 - 1], pu);
+        if (idx % 2 == 1) pb.p[idx / 2] = E::pack(s[idx / 16][idx % 16 - 1], pu);
       }
     }
     l_run += lsum;
@@ -405,7 +405,7 @@ void flash_fwd_bf16_kernel(const FwdArgs a) {
 #pragma unroll
     for (int n = 0; n < kPvSteps; n++) {
       if (n + kPvAhead < kPvSteps) AXL_PV_READ(n + kPvAhead)
-      o[n % DT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfr[n].v, pb.v[n / DT], o[n % DT], 0, 0, 0);
+      o[n % DT] = E::mfma_32x32x16(vfr[n].v, pb.v[n / DT], o[n % DT]);
       __builtin_amdgcn_sched_barrier(0);
     }
 #undef AXL_PV_READ
@@ -434,8 +434,8 @@ void flash_fwd_bf16_kernel(const FwdArgs a) {
         bf16x2 p[2];
         uint2 u;
       } w;
-      w.p[0] = pack_bf16(o[dt][4 * rq + 0] * inv_l, o[dt][4 * rq + 1] * inv_l);
-      w.p[1] = pack_bf16(o[dt][4 * rq + 2] * inv_l, o[dt][4 * rq + 3] * inv_l);
+      w.p[0] = E::pack(o[dt][4 * rq + 0] * inv_l, o[dt][4 * rq + 1] * inv_l);
+      w.p[1] = E::pack(o[dt][4 * rq + 2] * inv_l, o[dt][4 * rq + 3] * inv_l);
       *(uint2*)(op + 32 * dt + 8 * rq + 4 * g) = w.u;
     }
   }
@@ -646,18 +646,25 @@ int launch_flash_fwd(const AxlFlashFwdParams& p, hipStream_t stream) {
       err = hipGetLastError();                                                                  \
     }                                                                                           \
   } while (0)
+#define AXL_LAUNCH_FWD16(E)                                                                     \
+  do {                                                                                          \
+    if (p.head_dim == 128) {                                                                    \
+      if (aux) AXL_LAUNCH_FWD((flash_fwd_kernel<E, 128, true>), FwdTile<128>);                  \
+      else AXL_LAUNCH_FWD((flash_fwd_kernel<E, 128, false>), FwdTile<128>);                     \
+    } else {                                                                                    \
+      if (aux) AXL_LAUNCH_FWD((flash_fwd_kernel<E, 64, true>), FwdTile<64>);                    \
+      else AXL_LAUNCH_FWD((flash_fwd_kernel<E, 64, false>), FwdTile<64>);                       \
+    }                                                                                           \
+  } while (0)
   if (p.dtype == AXL_BF16) {
-    if (p.head_dim == 128) {
-      if (aux) AXL_LAUNCH_FWD((flash_fwd_bf16_kernel<128, true>), FwdTile<128>);
-      else AXL_LAUNCH_FWD((flash_fwd_bf16_kernel<128, false>), FwdTile<128>);
-    } else {
-      if (aux) AXL_LAUNCH_FWD((flash_fwd_bf16_kernel<64, true>), FwdTile<64>);
-      else AXL_LAUNCH_FWD((flash_fwd_bf16_kernel<64, false>), FwdTile<64>);
-    }
+    AXL_LAUNCH_FWD16(ElemBf16);
+  } else if (p.dtype == AXL_F16) {
+    AXL_LAUNCH_FWD16(ElemF16);
   } else {
     if (p.head_dim == 128) AXL_LAUNCH_FWD(flash_fwd_f32_kernel<128>, FwdTileF32<128>);
     else AXL_LAUNCH_FWD(flash_fwd_f32_kernel<64>, FwdTileF32<64>);
   }
+#undef AXL_LAUNCH_FWD16
 #undef AXL_LAUNCH_FWD
   if (err != hipSuccess)
     return set_error(AXL_ERR_LAUNCH, "axl_flash_fwd: launch failed: %s", hipGetErrorString(err));

@@ -107,7 +107,7 @@ struct DecTile {
 // in the "transposed" form where lane l owns query head l%16 and the tokens 4*(l/16)..+3 of the
 // page: the accumulator layout of S^T is exactly the B-operand layout of the second product, so
 // probabilities never leave registers, and every softmax statistic is per lane.
-template <int D, int GP, bool PAGED, int NST>
+template <typename E, int D, int GP, bool PAGED, int NST>
 __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
   using Tile = DecTile<D, GP, NST>;
   constexpr int KSTEPS = D / 32;        // MFMA k-steps over head_dim for S^T
@@ -369,7 +369,7 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
     // ---- scores: S^T[token][head]; this lane: head = lane%16, tokens 4kg + r
     floatx4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ks++) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[ks], qf[ks], s, 0, 0, 0);
+    for (int ks = 0; ks < KSTEPS; ks++) s = E::mfma_16x16x32(kf[ks], qf[ks], s);
     // A page that straddles the length (or the window start) holds tokens whose probability is
     // exactly 0; their V rows may be uninitialised pool memory, and 0 * NaN would poison the sum,
     // so those rows are replaced by zeros, as are all rows of a page outside the pool.
@@ -403,8 +403,8 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
     }
     l_run = l_run * corr + psum;
     union { shortx4 v; bf16x2 p[2]; } pf;
-    pf.p[0] = pack_bf16(s[0], s[1]);
-    pf.p[1] = pack_bf16(s[2], s[3]);
+    pf.p[0] = E::pack(s[0], s[1]);
+    pf.p[1] = E::pack(s[2], s[3]);
     if (__builtin_amdgcn_ballot_w64(changed) != 0) {
 #pragma unroll
       for (int nb = 0; nb < NB; nb++) o[nb] *= corr;
@@ -412,7 +412,7 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
     // ---- O^T += V^T P^T
 #pragma unroll
     for (int nb = 0; nb < NB; nb++)
-      o[nb] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf[nb], pf.v, o[nb], 0, 0, 0);
+      o[nb] = E::mfma_16x16x16(vf[nb], pf.v, o[nb]);
     st = (st + 1 == NST) ? 0 : st + 1;
   }
 
@@ -476,7 +476,7 @@ __global__ __launch_bounds__(256) void decode_plan_kernel(int* ticket, int32_t* 
 // (gpu_paged_attention.py:287-296, gpu_decoding.py:277-283).
 constexpr int kMaxChunks = 256;  // per sequence; bounds the combine kernel's LDS tables
 
-template <int D, int GP>
+template <typename E, int D, int GP>
 __global__ __launch_bounds__(256) void decode_combine_kernel(const DecArgs a) {
   __shared__ float sm[kMaxChunks * GP];   // record maxima, then rescale factors
   __shared__ float sl[kMaxChunks * GP];   // record sums
@@ -558,8 +558,8 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecArgs a) {
       }
       const float inv = s_inv[gq];
       union { bf16x2 p[2]; uint2 u; } pk;
-      pk.p[0] = pack_bf16(acc.x * inv, acc.y * inv);
-      pk.p[1] = pack_bf16(acc.z * inv, acc.w * inv);
+      pk.p[0] = E::pack(acc.x * inv, acc.y * inv);
+      pk.p[1] = E::pack(acc.z * inv, acc.w * inv);
       *(uint2*)(a.out + ((int64_t)b * a.Hq + hk * a.G) * D + 4 * col) = pk.u;
     }
   }
@@ -612,7 +612,7 @@ static int cu_count() {
   return n;
 }
 
-template <bool PAGED>
+template <typename E, bool PAGED>
 static int launch_common(DecArgs a, int D, hipStream_t stream, const char* who) {
   const int gp = gp_of(a.G);
   if (a.G > 16) return set_error(AXL_ERR_UNSUPPORTED, "%s: more than 16 query heads per kv head", who);
@@ -635,17 +635,17 @@ static int launch_common(DecArgs a, int D, hipStream_t stream, const char* who) 
   // Two workgroups fit a CU (LDS); the split kernel is persistent and strides over its work items.
   const dim3 grid(2 * cu_count());
   hipError_t err = hipSuccess;
-#define AXL_DEC(DD, GG, NS)                                                                    \
+#define AXL_DEC(E, DD, GG, NS)                                                                  \
   do {                                                                                          \
     using Tile = DecTile<DD, GG, NS>;                                                           \
-    auto kern = decode_split_kernel<DD, GG, PAGED, NS>;                                         \
+    auto kern = decode_split_kernel<E, DD, GG, PAGED, NS>;                                      \
     err = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,    \
                               Tile::LDS_BYTES);                                                 \
     if (err == hipSuccess) {                                                                    \
       hipLaunchKernelGGL(decode_plan_kernel, dim3((n_tab + 255) / 256), dim3(256), 0, stream,   \
                          s.ticket, s.ws_tab, n_tab);                                            \
       hipLaunchKernelGGL(kern, grid, dim3(256), Tile::LDS_BYTES, stream, s);                    \
-      hipLaunchKernelGGL((decode_combine_kernel<DD, GG>), cgrid, dim3(256), 0, stream, s);      \
+      hipLaunchKernelGGL((decode_combine_kernel<E, DD, GG>), cgrid, dim3(256), 0, stream, s);   \
     }                                                                                           \
   } while (0)
   // The kernels keep per-sequence tables in LDS: larger batches go in slices of kMaxBatch.
@@ -663,12 +663,12 @@ static int launch_common(DecArgs a, int D, hipStream_t stream, const char* who) 
     s.ws_tab = a.ws_tab + (size_t)b0 * a.Hkv * a.nch;
     const int n_tab = s.B * a.Hkv * a.nch;
     const dim3 cgrid(a.Hkv, s.B);
-    if (D == 128 && gp == 4) AXL_DEC(128, 4, kStages128);
-    else if (D == 128 && gp == 8) AXL_DEC(128, 8, kStages128);
-    else if (D == 128) AXL_DEC(128, 16, kStages128);
-    else if (gp == 4) AXL_DEC(64, 4, kStages64);
-    else if (gp == 8) AXL_DEC(64, 8, kStages64);
-    else AXL_DEC(64, 16, kStages64);
+    if (D == 128 && gp == 4) AXL_DEC(E, 128, 4, kStages128);
+    else if (D == 128 && gp == 8) AXL_DEC(E, 128, 8, kStages128);
+    else if (D == 128) AXL_DEC(E, 128, 16, kStages128);
+    else if (gp == 4) AXL_DEC(E, 64, 4, kStages64);
+    else if (gp == 8) AXL_DEC(E, 64, 8, kStages64);
+    else AXL_DEC(E, 64, 16, kStages64);
   }
 #undef AXL_DEC
   if (err == hipSuccess) err = hipGetLastError();
@@ -686,7 +686,8 @@ int launch_paged_decode(const AxlPagedDecodeParams& p, hipStream_t stream) {
   a.num_pages = p.num_pages; a.pps = p.pages_per_seq; a.kv_len = p.pages_per_seq * kPage;
   a.window = p.sliding_window < 0 ? -1 : p.sliding_window;
   a.scale = p.softmax_scale;
-  return launch_common<true>(a, p.head_dim, stream, "axl_paged_decode");
+  return p.dtype == AXL_F16 ? launch_common<ElemF16, true>(a, p.head_dim, stream, "axl_paged_decode")
+                            : launch_common<ElemBf16, true>(a, p.head_dim, stream, "axl_paged_decode");
 }
 
 int launch_decode(const AxlDecodeParams& p, hipStream_t stream) {
@@ -700,7 +701,8 @@ int launch_decode(const AxlDecodeParams& p, hipStream_t stream) {
   a.num_pages = 0; a.pps = (p.kv_len + kPage - 1) / kPage; a.kv_len = p.kv_len;
   a.window = p.sliding_window < 0 ? -1 : p.sliding_window;
   a.scale = p.softmax_scale;
-  return launch_common<false>(a, p.head_dim, stream, "axl_decode");
+  return p.dtype == AXL_F16 ? launch_common<ElemF16, false>(a, p.head_dim, stream, "axl_decode")
+                            : launch_common<ElemBf16, false>(a, p.head_dim, stream, "axl_decode");
 }
 
 }  // namespace axl

@@ -257,8 +257,8 @@ class HipFlashAttention(BaseFlashAttention):
         head_dim = query.shape[-1]
         if padded_head_dim(head_dim) is None:  # same limit as gpu_attention.py:954
             return self._log_unsupported(f"{head_dim=} > 128")
-        if query.dtype not in (torch.bfloat16, torch.float32):
-            return self._log_unsupported(f"{query.dtype=} (supported: bfloat16, float32)")
+        if query.dtype not in (torch.bfloat16, torch.float16, torch.float32):
+            return self._log_unsupported(f"{query.dtype=} (supported: bfloat16, float16, float32)")
         if key.dtype != query.dtype or input_batch["value"].dtype != query.dtype:
             return self._log_unsupported("query, key and value dtypes differ")
         logit_sink = input_batch.get("logit_sink", None)

@@ -245,7 +245,42 @@ def test_wide_groups_and_batch_slices():
         assert _ok(got2.cpu(), want), (b, hq, hkv, d)
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("b,s,h,hkv,d,padding,window", [
+    (2, 1024, 16, 2, 128, 111, -1),
+    (4, 512, 48, 48, 64, 0, 127),
+    (3, 2048, 32, 8, 128, 37, -1),
+])
+def test_float16_decode_against_ref(b, s, h, hkv, d, padding, window):
+    """float16 (the reference's decode tests run float32 and float16 on GPU, decoding_test.py:33):
+    same kernels with the f16 matrix instructions; the bar is 8x tighter than bf16's, as the
+    mantissa is."""
+    pps = s // 16
+    q, kp, vp, tables, _ = ref.paged_inputs(11, batch=b, num_heads=h, num_kv_heads=hkv, head_dim=d, page_size=16,
+                                            pages_per_seq=pps, min_len=1, max_len=s, dtype=torch.float16)
+    lengths = torch.full((b,), s - padding, dtype=torch.int32)
+    lengths[0] = max(1, s // 3)
+    scale = d ** -0.5
+    want = ref.reference_decode(q, kp, vp, lengths, softmax_scale=scale, page_tables=tables,
+                                sliding_window=None if window < 0 else window)[:, 0]
+
+    def ok(got):
+        return got.dtype == torch.float16 and (ref.max_abs(got.cpu(), want) <= 2.5e-3 or ref.rel_l2(got.cpu(), want) <= 1.25e-3)
+
+    got = ops.paged_decode(q[:, 0].cuda(), kp.cuda(), vp.cuda(), tables.cuda(), lengths.cuda(),
+                           softmax_scale=scale, sliding_window=window)
+    assert ok(got), (ref.max_abs(got.cpu(), want), ref.rel_l2(got.cpu(), want))
+    kk, vv = ref.reconstruct_kv(tables, kp), ref.reconstruct_kv(tables, vp)
+    got2 = ops.decode(q[:, 0].cuda(), kk.cuda(), vv.cuda(), lengths.cuda(), softmax_scale=scale, sliding_window=window)
+    assert ok(got2), (ref.max_abs(got2.cpu(), want), ref.rel_l2(got2.cpu(), want))
+    with _deterministic():
+        det = ops.paged_decode(q[:, 0].cuda(), kp.cuda(), vp.cuda(), tables.cuda(), lengths.cuda(),
+                               softmax_scale=scale, sliding_window=window)
+        det2 = ops.decode(q[:, 0].cuda(), kk.cuda(), vv.cuda(), lengths.cuda(), softmax_scale=scale,
+                          sliding_window=window)
+    assert ok(det) and torch.equal(det, det2)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("page_size,d", [(16, 128), (8, 64), (32, 128)])
 def test_paged_kv_insert_bit_exact(dtype, page_size, d):
     """Page insert against the oracle, bit for bit: live rows, padding page, positions and pages out of

@@ -19,6 +19,8 @@ from oracle import ref_attention as ref
 pytestmark = pytest.mark.gpu
 
 BF16_MAX_ABS, BF16_REL_L2, FP32_MAX_ABS = 2e-2, 1e-2, 1e-5
+# float16 carries 3 more mantissa bits than bfloat16: its bar is 8x tighter.
+F16_MAX_ABS, F16_REL_L2 = 2.5e-3, 1.25e-3
 
 
 def _ok_bf16(got, want):
@@ -27,9 +29,13 @@ def _ok_bf16(got, want):
 
 def _assert_close(name, got, want, dtype):
     got = got.detach().cpu()
+    assert got.dtype == dtype, f"{name}: {got.dtype}"
     if dtype == torch.float32:
         err = ref.max_abs(got, want)
         assert err <= FP32_MAX_ABS, f"{name}: max-abs {err:.3e}"
+    elif dtype == torch.float16:
+        assert ref.max_abs(got, want) <= F16_MAX_ABS or ref.rel_l2(got, want) <= F16_REL_L2, (
+            f"{name}: max-abs {ref.max_abs(got, want):.3e} rel-L2 {ref.rel_l2(got, want):.3e}")
     else:
         assert _ok_bf16(got, want), f"{name}: max-abs {ref.max_abs(got, want):.3e} rel-L2 {ref.rel_l2(got, want):.3e}"
     assert torch.isfinite(got.float()).all(), name
@@ -61,6 +67,11 @@ FWD_CASES = [
     (1, 1024, 2, 2, 128, torch.bfloat16, "sliding", 129, False),
     (1, 512, 2, 1, 128, torch.bfloat16, "sliding", 0, False),
     (1, 256, 2, 2, 128, torch.bfloat16, "none", None, True),
+    # float16, as the reference's tests run (gpu_attention_test.py:122)
+    (2, 256, 4, 4, 64, torch.float16, "causal", None, False),
+    (1, 384, 8, 2, 128, torch.float16, "causal", None, True),
+    (1, 1024, 4, 2, 128, torch.float16, "sliding", 128, False),
+    (1, 256, 2, 1, 128, torch.float16, "none", None, False),
     (2, 512, 4, 4, 64, torch.float32, "causal", None, False),  # BASELINE config 1
     (1, 256, 4, 2, 128, torch.float32, "sliding", 100, True),
     (1, 256, 2, 2, 64, torch.float32, "none", None, False),
@@ -123,6 +134,38 @@ def test_backward_matches_oracle(b, t, hq, hkv, d, mask, window, seg):
     _assert_close("dq", dq, wq, dtype)
     _assert_close("dk", dk, wk, dtype)
     _assert_close("dv", dv, wv, dtype)
+
+
+@pytest.mark.parametrize("b,t,hq,hkv,d,mask,window,seg", [
+    (2, 256, 4, 4, 64, "causal", None, False),
+    (1, 384, 8, 2, 128, "causal", None, True),
+    (1, 1024, 4, 2, 128, "sliding", 300, True),
+    (1, 1536, 4, 2, 128, "none", None, False),
+    (1, 1920, 2, 1, 64, "sliding", 777, False),
+])
+def test_float16_backward_matches_oracle(b, t, hq, hkv, d, mask, window, seg):
+    """float16 forward + backward (gpu_attention_test.py:197 runs float16 and float32), all phases in
+    one call and phase by phase (the separate delta pre-pass)."""
+    dtype = torch.float16
+    q, k, v, do = _inputs(b, t, hq, hkv, d, dtype)
+    segs = ref.packed_segment_ids(4, b, t, max_docs=5) if seg else None
+    spec, kw = _mask_args(mask, window, segs)
+    scale = d ** -0.5
+    wq, wk, wv = ref.reference_mha_grads(q, k, v, do, spec, softmax_scale=scale)
+    qc, kc, vc, doc = q.cuda(), k.cuda(), v.cuda(), do.cuda()
+    out, lse = ops.flash_fwd(qc, kc, vc, softmax_scale=scale, **kw)
+    _assert_close("out", out, ref.reference_mha(q, k, v, spec, softmax_scale=scale), dtype)
+    dq, dk, dv = ops.flash_bwd(qc, kc, vc, out, lse, doc, softmax_scale=scale, **kw)
+    _assert_close("dq", dq, wq, dtype)
+    _assert_close("dk", dk, wk, dtype)
+    _assert_close("dv", dv, wv, dtype)
+    bufs = (torch.zeros_like(dq), torch.zeros_like(dk), torch.zeros_like(dv),
+            torch.empty((2 * b * hq * t * 4 + 16,), dtype=torch.uint8, device="cuda"))
+    for phase in (1, 2, 4):  # delta, dK/dV, dQ
+        ops.flash_bwd(qc, kc, vc, out, lse, doc, softmax_scale=scale, phases=phase, buffers=bufs, **kw)
+    _assert_close("dq by phases", bufs[0], wq, dtype)
+    _assert_close("dk by phases", bufs[1], wk, dtype)
+    _assert_close("dv by phases", bufs[2], wv, dtype)
 
 
 @pytest.mark.parametrize("mask,window", [("causal", None), ("sliding", 333)])
@@ -377,6 +420,7 @@ def test_dispatch_and_autograd_end_to_end():
     (2, 256, 4, 2, 128, torch.bfloat16, "causal", None, False),
     (1, 512, 4, 4, 64, torch.bfloat16, "sliding", 100, True),
     (1, 384, 2, 1, 128, torch.bfloat16, "none", None, False),
+    (1, 384, 4, 2, 128, torch.float16, "causal", None, True),
     (1, 256, 4, 2, 64, torch.float32, "causal", None, True),
     (1, 128, 2, 2, 128, torch.float32, "none", None, False),
 ])
@@ -394,8 +438,8 @@ def test_logit_sink_forward_and_backward(b, t, hq, hkv, d, dtype, mask, window, 
     # The sink must matter in this test: without it the output differs visibly.
     plain, _ = ops.flash_fwd(q.cuda(), k.cuda(), v.cuda(), softmax_scale=scale, **kw)
     assert ref.max_abs(plain.cpu(), want) > 0.05
-    if dtype != torch.bfloat16:
-        return  # the backward kernels are bf16 only
+    if dtype == torch.float32:
+        return  # the backward kernels are 16-bit only
     wq, wk, wv, ws = ref.reference_mha_grads(q, k, v, do, spec, softmax_scale=scale, logit_sink=sink)
     dq, dk, dv, dsink = ops.flash_bwd(q.cuda(), k.cuda(), v.cuda(), out, lse, do.cuda(), softmax_scale=scale,
                                      logit_sink=sink.cuda(), **kw)
@@ -486,6 +530,9 @@ AUX_CASES = [
     (1, 256, 256, 8, 2, 64, torch.bfloat16, "causal", None, True, "bh", torch.float32, 0.5),
     (1, 256, 256, 2, 2, 64, torch.float32, "causal", None, False, "bh", torch.float32, 0.25),
     (1, 128, 256, 2, 1, 128, torch.float32, "none", None, False, "1h", torch.bfloat16, 0.0),
+    # float16 q/k/v: a float16 bias is handed over as float32 by the wrapper
+    (2, 256, 256, 4, 2, 128, torch.float16, "causal", None, True, "1h", torch.float16, 0.0),
+    (1, 256, 384, 4, 1, 64, torch.float16, "none", None, False, "bh", torch.float32, 0.2),
 ]
 
 
@@ -514,8 +561,8 @@ def test_dense_bias_and_dropout_forward_and_backward(b, t, s, hq, hkv, d, dtype,
     # The optional inputs must matter in this test.
     plain, _ = ops.flash_fwd(q.cuda(), k.cuda(), v.cuda(), softmax_scale=scale, **kw)
     assert ref.max_abs(plain.cpu(), want) > 0.05
-    if dtype != torch.bfloat16:
-        return  # the backward kernels are bf16 only
+    if dtype == torch.float32:
+        return  # the backward kernels are 16-bit only
     wq, wk, wv = ref.reference_mha_grads(q, k, v, do, spec, **okw)
     dq, dk, dv = ops.flash_bwd(q.cuda(), k.cuda(), v.cuda(), out, lse, do.cuda(), **gkw)
     _assert_close("dq", dq, wq, dtype)
