@@ -34,4 +34,8 @@ hipError_t launch_bwd_dkdv(const BwdArgs& a, int dtype, int head_dim, bool aux, 
 // of reading them), for a dK/dV kernel enqueued after it.
 hipError_t launch_bwd_dq(const BwdArgs& a, int dtype, int head_dim, bool fuse_delta, hipStream_t stream);
 
+// Enqueues the fp32 dK/dV and / or dQ kernels (`phases`: AXL_BWD_DKDV, AXL_BWD_DQ) for head_dim 64
+// or 128; they read delta from the workspace and honour the dense bias / dropout mask.
+hipError_t launch_bwd_f32(const BwdArgs& a, int head_dim, int phases, hipStream_t stream);
+
 }  // namespace axl

@@ -325,8 +325,6 @@ size_t flash_bwd_workspace_bytes(const AxlFlashBwdParams& p) {
 }
 
 int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream) {
-  if (p.dtype != AXL_BF16 && p.dtype != AXL_F16)
-    return set_error(AXL_ERR_UNSUPPORTED, "axl_flash_bwd: only bf16 and fp16 are supported");
   const int dt = p.dtype;
   BwdArgs a;
   a.q = p.q; a.k = p.k; a.v = p.v; a.out = p.out; a.dout = p.d_out; a.lse = p.lse;
@@ -359,7 +357,13 @@ int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream)
   // All three phases in one call, no bias / dropout mask / sink gradient: the dQ kernel computes delta
   // on the way (it holds the dO rows anyway) and runs first; the dK/dV kernel reads what it left.
   const int all = AXL_BWD_DELTA | AXL_BWD_DKDV | AXL_BWD_DQ;
-  if ((phases & all) == all && !aux && !p.d_logit_sink) {
+  if (dt == AXL_F32) {
+    if (phases & AXL_BWD_DELTA) {
+      if (p.head_dim == 128) AXL_LAUNCH((bwd_delta_kernel<float, 128>), delta_grid, 0);
+      else AXL_LAUNCH((bwd_delta_kernel<float, 64>), delta_grid, 0);
+    }
+    if (err == hipSuccess) err = launch_bwd_f32(a, p.head_dim, phases, stream);
+  } else if ((phases & all) == all && !aux && !p.d_logit_sink) {
     err = launch_bwd_dq(a, dt, p.head_dim, true, stream);
     if (err == hipSuccess) err = launch_bwd_dkdv(a, dt, p.head_dim, false, stream);
     if (err != hipSuccess)
@@ -374,7 +378,9 @@ int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream)
       AXL_LAUNCH((flash_bwd_dq_aux_kernel<E, DD, true>), dq_grid, DqTile<DD>::LDS_BYTES);         \
     if ((phases & AXL_BWD_DQ) && !aux && err == hipSuccess) err = launch_bwd_dq(a, dt, DD, false, stream); \
   } while (0)
-  if (dt == AXL_BF16) {
+  if (dt == AXL_F32) {
+    // enqueued above
+  } else if (dt == AXL_BF16) {
     if (p.head_dim == 128) AXL_BWD_PHASES(ElemBf16, __bf16, 128);
     else AXL_BWD_PHASES(ElemBf16, __bf16, 64);
   } else {

@@ -168,6 +168,38 @@ def test_float16_backward_matches_oracle(b, t, hq, hkv, d, mask, window, seg):
     _assert_close("dv by phases", bufs[2], wv, dtype)
 
 
+@pytest.mark.parametrize("b,t,s,hq,hkv,d,mask,window,seg", [
+    (2, 512, 512, 4, 4, 64, "causal", None, False),      # BASELINE config 1, with its backward
+    (1, 256, 256, 4, 2, 128, "sliding", 100, True),
+    (1, 384, 384, 8, 2, 128, "causal", None, True),
+    (2, 256, 256, 2, 2, 64, "none", None, False),
+    (1, 128, 384, 2, 1, 128, "none", None, False),
+    (1, 640, 640, 2, 1, 64, "sliding", 33, False),
+    (1, 256, 512, 4, 2, 64, "causal", None, False),
+])
+def test_float32_backward_matches_oracle(b, t, s, hq, hkv, d, mask, window, seg):
+    """float32 forward + backward (gpu_attention_test.py:197 runs float16 and float32; the reference
+    shrinks its backward blocks for float32, gpu_attention.py:645-646), against the float64 oracle at
+    the fp32 bar, all phases in one call and phase by phase (bit-identical: same kernels)."""
+    dtype = torch.float32
+    q, k, v, do = _inputs(b, t, hq, hkv, d, dtype, s=s)
+    segs = ref.packed_segment_ids(4, b, t, max_docs=5) if seg else None
+    spec, kw = _mask_args(mask, window, segs)
+    scale = d ** -0.5
+    wq, wk, wv = ref.reference_mha_grads(q, k, v, do, spec, softmax_scale=scale)
+    qc, kc, vc, doc = q.cuda(), k.cuda(), v.cuda(), do.cuda()
+    out, lse = ops.flash_fwd(qc, kc, vc, softmax_scale=scale, **kw)
+    dq, dk, dv = ops.flash_bwd(qc, kc, vc, out, lse, doc, softmax_scale=scale, **kw)
+    _assert_close("dq", dq, wq, dtype)
+    _assert_close("dk", dk, wk, dtype)
+    _assert_close("dv", dv, wv, dtype)
+    bufs = (torch.zeros_like(dq), torch.zeros_like(dk), torch.zeros_like(dv),
+            torch.empty((2 * b * hq * t * 4 + 16,), dtype=torch.uint8, device="cuda"))
+    for phase in (1, 2, 4):  # delta, dK/dV, dQ
+        ops.flash_bwd(qc, kc, vc, out, lse, doc, softmax_scale=scale, phases=phase, buffers=bufs, **kw)
+    assert torch.equal(bufs[0], dq) and torch.equal(bufs[1], dk) and torch.equal(bufs[2], dv)
+
+
 @pytest.mark.parametrize("mask,window", [("causal", None), ("sliding", 333)])
 @pytest.mark.parametrize("d", [64, 128])
 def test_backward_with_more_keys_than_queries(mask, window, d):
@@ -374,9 +406,10 @@ def test_strided_inputs():
         assert torch.equal(a, c)
 
 
-def test_dispatch_and_autograd_end_to_end():
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_dispatch_and_autograd_end_to_end(dtype):
     b, t, hq, hkv, d = 2, 256, 4, 2, 128
-    q, k, v, do = _inputs(b, t, hq, hkv, d, torch.bfloat16)
+    q, k, v, do = _inputs(b, t, hq, hkv, d, dtype)
     segs = ref.packed_segment_ids(4, b, t, max_docs=3)
     pos = dict(target_positions=torch.arange(t)[None], source_positions=torch.arange(t)[None])
     bias = ab.CompositeAttentionBias([
@@ -388,15 +421,18 @@ def test_dispatch_and_autograd_end_to_end():
     impl = flash_attention_implementation("gpu", query=qd, key=kd, value=vd, bias=bias, softmax_scale=scale)
     assert impl is not None and isinstance(impl.fn, HipFlashAttention)
     out = impl.fn(dict(query=qd, key=kd, value=vd, bias=bias))
-    # Same loss as the reference's tests: mean of the output (gpu_attention_test.py:59-92).
-    out.float().mean().backward()
+    # Same loss as the reference's tests: mean of the output (gpu_attention_test.py:59-92); with
+    # float16 it is scaled up, as float16 training does, so that d_out = 1/numel is a normal number.
+    loss_scale = 2.0 ** 14 if dtype == torch.float16 else 1.0
+    (out.float().mean() * loss_scale).backward()
     spec = ref.MaskSpec(sliding_window=64, segment_ids=segs)
     want = ref.reference_mha(q, k, v, spec, softmax_scale=scale)
-    ones = torch.full_like(want, 1.0 / want.numel())
+    ones = torch.full_like(want, loss_scale / want.numel())
     wq, wk, wv = ref.reference_mha_grads(q, k, v, ones, spec, softmax_scale=scale)
-    _assert_close("out", out, want, torch.bfloat16)
+    _assert_close("out", out, want, dtype)
     for name, got, exp in (("dq", qd.grad, wq), ("dk", kd.grad, wk), ("dv", vd.grad, wv)):
-        assert ref.rel_l2(got.cpu(), exp) < 2e-2, name  # gradients of a mean are ~1e-6: relative check
+        # gradients of a mean are ~1e-6: relative check
+        assert got.dtype == dtype and ref.rel_l2(got.cpu(), exp) < (1e-4 if dtype == torch.float32 else 2e-2), name
     # Function-level entry point with a mask fn.
     o2 = flash_attention(qd, kd, vd, segment_ids=segs.cuda(), softmax_scale=scale,
                          mask_fn=ab.sliding_window_causal_mask(64))
@@ -438,8 +474,6 @@ def test_logit_sink_forward_and_backward(b, t, hq, hkv, d, dtype, mask, window, 
     # The sink must matter in this test: without it the output differs visibly.
     plain, _ = ops.flash_fwd(q.cuda(), k.cuda(), v.cuda(), softmax_scale=scale, **kw)
     assert ref.max_abs(plain.cpu(), want) > 0.05
-    if dtype == torch.float32:
-        return  # the backward kernels are 16-bit only
     wq, wk, wv, ws = ref.reference_mha_grads(q, k, v, do, spec, softmax_scale=scale, logit_sink=sink)
     dq, dk, dv, dsink = ops.flash_bwd(q.cuda(), k.cuda(), v.cuda(), out, lse, do.cuda(), softmax_scale=scale,
                                      logit_sink=sink.cuda(), **kw)
@@ -561,8 +595,6 @@ def test_dense_bias_and_dropout_forward_and_backward(b, t, s, hq, hkv, d, dtype,
     # The optional inputs must matter in this test.
     plain, _ = ops.flash_fwd(q.cuda(), k.cuda(), v.cuda(), softmax_scale=scale, **kw)
     assert ref.max_abs(plain.cpu(), want) > 0.05
-    if dtype == torch.float32:
-        return  # the backward kernels are 16-bit only
     wq, wk, wv = ref.reference_mha_grads(q, k, v, do, spec, **okw)
     dq, dk, dv = ops.flash_bwd(q.cuda(), k.cuda(), v.cuda(), out, lse, do.cuda(), **gkw)
     _assert_close("dq", dq, wq, dtype)
