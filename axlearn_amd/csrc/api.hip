@@ -214,8 +214,8 @@ static int check_decode_common(const char* who, int batch, int hq, int hkv, int 
                      "%s: num_q_heads %d is not divisible by num_kv_heads %d", who, hq, hkv);
   if (!(scale > 0.f) || !std::isfinite(scale))
     return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: softmax_scale must be finite and > 0", who);
-  if (dtype != AXL_BF16 && dtype != AXL_F16)
-    return set_error(AXL_ERR_UNSUPPORTED, "%s: only bf16 and fp16 are supported", who);
+  if (dtype != AXL_BF16 && dtype != AXL_F16 && dtype != AXL_F32)
+    return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: unknown dtype %d", who, dtype);
   if (d != 128 && d != 64)
     return set_error(AXL_ERR_UNSUPPORTED, "%s: head_dim %d (supported: 64, 128)", who, d);
   if (hq / hkv > 16)
@@ -263,7 +263,8 @@ int axl_decode(const AxlDecodeParams* p, void* stream) {
   if (!p->q || !p->k || !p->v || !p->lengths || !p->out)
     return set_error(AXL_ERR_INVALID_ARGUMENT, "axl_decode: NULL tensor pointer");
   if (!aligned16(p->q) || !aligned16(p->k) || !aligned16(p->v) || !aligned16(p->out) ||
-      !strides_ok(p->k_strides, 2) || !strides_ok(p->v_strides, 2))
+      !strides_ok(p->k_strides, p->dtype == AXL_F32 ? 4 : 2) ||
+      !strides_ok(p->v_strides, p->dtype == AXL_F32 ? 4 : 2))
     return set_error(AXL_ERR_UNSUPPORTED, "axl_decode: tensors must be 16-byte aligned rows");
   const size_t need = decode_workspace_bytes(*p);
   if (!p->workspace || p->workspace_bytes < need || !aligned16(p->workspace))

@@ -107,6 +107,11 @@ struct ElemF16 {
   static __device__ __forceinline__ __bf16 narrow(float x) { return __builtin_bit_cast(__bf16, (_Float16)x); }
 };
 
+// Tag of the fp32 kernels where a template is shared with the 16-bit ones.
+struct ElemF32 {
+  static constexpr int kDtype = AXL_F32;
+};
+
 // Eight fp32 -> one MFMA operand of element type E.
 template <typename E>
 __device__ __forceinline__ bf16x8 pack8(float a0, float a1, float a2, float a3, float a4, float a5, float a6,

@@ -557,11 +557,139 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecArgs a) {
         acc.x += p.x; acc.y += p.y; acc.z += p.z; acc.w += p.w;
       }
       const float inv = s_inv[gq];
-      union { bf16x2 p[2]; uint2 u; } pk;
-      pk.p[0] = E::pack(acc.x * inv, acc.y * inv);
-      pk.p[1] = E::pack(acc.z * inv, acc.w * inv);
-      *(uint2*)(a.out + ((int64_t)b * a.Hq + hk * a.G) * D + 4 * col) = pk.u;
+      const int64_t at = ((int64_t)b * a.Hq + hk * a.G) * D + 4 * col;
+      if constexpr (std::is_same_v<E, ElemF32>) {
+        *(float4*)((float*)a.out + at) = float4{acc.x * inv, acc.y * inv, acc.z * inv, acc.w * inv};
+      } else {
+        union { bf16x2 p[2]; uint2 u; } pk;
+        pk.p[0] = E::pack(acc.x * inv, acc.y * inv);
+        pk.p[1] = E::pack(acc.z * inv, acc.w * inv);
+        *(uint2*)(a.out + at) = pk.u;
+      }
     }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// fp32 decode (the reference's decode tests run float32, decoding_test.py:33): plain fp32
+// multiply-adds and the accurate exponential, one workgroup per live block of `chunk_pages` pages of
+// a (sequence, kv head), a fixed decomposition.  A token row is spread over 16 lanes; each 16-lane
+// group keeps a running (m, l, o) per query head over the tokens it visits, the groups are merged at
+// the end and leave one record in the same format as the 16-bit kernel's, for the same merge kernel.
+// For parity with float32 callers, not for speed.
+// ---------------------------------------------------------------------------------------------
+template <int D, int GP, bool PAGED>
+__global__ __launch_bounds__(256) void decode_split_f32_kernel(const DecArgs a) {
+  constexpr int SL = D / 16;  // floats of a row per lane
+  __shared__ float q_lds[GP * D];
+  __shared__ float red_o[4][GP][D];
+  __shared__ float red_m[4][GP], red_l[4][GP];
+  const int c = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, sub = lane >> 4, l16 = lane & 15;
+  int len = a.lengths[b];
+  if (!PAGED) len = min(len, a.kv_len);
+  int ch0, ch1;
+  live_chunks(a, len, ch0, ch1);
+  if (ch0 + c >= ch1) return;
+  const int npages = min((len + kPage - 1) / kPage, a.pps);
+  const int first_page = a.window >= 0 ? max(0, len - 1 - a.window) / kPage : 0;
+  const int p_begin = max((ch0 + c) * a.chunk_pages, first_page);
+  const int p_end = min((ch0 + c + 1) * a.chunk_pages, npages);
+  const float* qg = (const float*)a.q + ((int64_t)b * a.Hq + hk * a.G) * D;
+  for (int i = tid; i < GP * D; i += 256) q_lds[i] = i < a.G * D ? qg[i] : 0.f;
+  __syncthreads();
+
+  float m[GP], l[GP], o[GP][SL];
+#pragma unroll
+  for (int h = 0; h < GP; h++) {
+    m[h] = kNegInf;
+    l[h] = 0.f;
+#pragma unroll
+    for (int i = 0; i < SL; i++) o[h][i] = 0.f;
+  }
+  for (int tok = p_begin * kPage + wave * 4 + sub; tok < p_end * kPage; tok += 16) {
+    const float *kr, *vr;
+    bool valid = true;
+    if (PAGED) {
+      int pg = a.page_tables[(int64_t)b * a.pps + tok / kPage];
+      if (pg < 0) pg += a.num_pages;  // negative indices count from the end, as in the reference's gather
+      valid = (unsigned)pg < (unsigned)a.num_pages;  // a page outside the pool reads as zeros
+      const int64_t off = (((int64_t)hk * a.num_pages + (valid ? pg : 0)) * kPage + tok % kPage) * D;
+      kr = (const float*)a.k + off;
+      vr = (const float*)a.v + off;
+    } else {
+      const int row = min(tok, a.kv_len - 1);  // rows past the cache are masked below
+      kr = (const float*)a.k + b * a.ks.b + (int64_t)row * a.ks.s + hk * a.ks.h;
+      vr = (const float*)a.v + b * a.vs.b + (int64_t)row * a.vs.s + hk * a.vs.h;
+    }
+    bool keep = tok < len;
+    if (a.window >= 0) keep = keep && (len - 1 - tok <= a.window);
+    if (!keep) continue;  // uniform over the 16 lanes of the token
+    float kx[SL], vx[SL];
+#pragma unroll
+    for (int i = 0; i < SL; i += 4) {
+      const float4 x = valid ? *(const float4*)(kr + SL * l16 + i) : float4{0.f, 0.f, 0.f, 0.f};
+      const float4 y = valid ? *(const float4*)(vr + SL * l16 + i) : float4{0.f, 0.f, 0.f, 0.f};
+      kx[i] = x.x; kx[i + 1] = x.y; kx[i + 2] = x.z; kx[i + 3] = x.w;
+      vx[i] = y.x; vx[i + 1] = y.y; vx[i + 2] = y.z; vx[i + 3] = y.w;
+    }
+#pragma unroll
+    for (int h = 0; h < GP; h++) {
+      float dot = 0.f;
+#pragma unroll
+      for (int i = 0; i < SL; i++) dot = __builtin_fmaf(q_lds[h * D + SL * l16 + i], kx[i], dot);
+      dot += __shfl_xor(dot, 1, 64);
+      dot += __shfl_xor(dot, 2, 64);
+      dot += __shfl_xor(dot, 4, 64);
+      dot += __shfl_xor(dot, 8, 64);
+      const float mn = fmaxf(m[h], dot);
+      const float corr = expf((m[h] - mn) * a.scale);
+      const float pr = expf((dot - mn) * a.scale);
+      m[h] = mn;
+      l[h] = l[h] * corr + pr;
+#pragma unroll
+      for (int i = 0; i < SL; i++) o[h][i] = __builtin_fmaf(pr, vx[i], o[h][i] * corr);
+    }
+  }
+  // ---- merge the four 16-lane groups of the wavefront, then the four wavefronts.
+#pragma unroll
+  for (int h = 0; h < GP; h++) {
+    float mw = fmaxf(m[h], __shfl_xor(m[h], 16, 64));
+    mw = fmaxf(mw, __shfl_xor(mw, 32, 64));
+    const float f = expf((m[h] - mw) * a.scale);
+    float lw = l[h] * f;
+    lw += __shfl_xor(lw, 16, 64);
+    lw += __shfl_xor(lw, 32, 64);
+#pragma unroll
+    for (int i = 0; i < SL; i++) {
+      float x = o[h][i] * f;
+      x += __shfl_xor(x, 16, 64);
+      x += __shfl_xor(x, 32, 64);
+      if (sub == 0) red_o[wave][h][SL * l16 + i] = x;
+    }
+    if (lane == 0) {
+      red_m[wave][h] = mw;
+      red_l[wave][h] = lw;
+    }
+  }
+  __syncthreads();
+  const int64_t rec = ((int64_t)b * a.Hkv + hk) * a.nch + c;
+  for (int idx = tid; idx < GP * D; idx += 256) {
+    const int h = idx / D, d = idx % D;
+    const float mw = fmaxf(fmaxf(red_m[0][h], red_m[1][h]), fmaxf(red_m[2][h], red_m[3][h]));
+    float acc = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; w++) acc += red_o[w][h][d] * expf((red_m[w][h] - mw) * a.scale);
+    a.ws_o[rec * (GP * D) + idx] = acc;
+  }
+  if (tid < GP) {
+    const float mw = fmaxf(fmaxf(red_m[0][tid], red_m[1][tid]), fmaxf(red_m[2][tid], red_m[3][tid]));
+    float lw = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; w++) lw += red_l[w][tid] * expf((red_m[w][tid] - mw) * a.scale);
+    a.ws_m[rec * GP + tid] = mw;
+    a.ws_l[rec * GP + tid] = lw;
+    if (tid == 0) a.ws_tab[rec] = (int)rec;
   }
 }
 
@@ -677,6 +805,43 @@ static int launch_common(DecArgs a, int D, hipStream_t stream, const char* who) 
   return AXL_OK;
 }
 
+template <bool PAGED>
+static int launch_f32(DecArgs a, int D, hipStream_t stream, const char* who) {
+  const int gp = gp_of(a.G);
+  a.chunk_pages = pick_chunk_pages(a.pps);
+  if (a.chunk_pages > 256)
+    return set_error(AXL_ERR_UNSUPPORTED, "%s: context longer than %d tokens", who, 256 * kMaxChunks * kPage);
+  if (a.B > 65535) return set_error(AXL_ERR_UNSUPPORTED, "%s: more than 65535 sequences in fp32", who);
+  a.nch = (a.pps + a.chunk_pages - 1) / a.chunk_pages;
+  float* ws = a.ws_o;
+  const size_t n_o = (size_t)a.B * a.Hkv * a.nch * gp * D;
+  const size_t n_s = (size_t)a.B * a.Hkv * a.nch * gp;
+  const size_t n_r = (size_t)a.B * a.Hkv * a.nch;
+  a.ws_m = ws + n_o;
+  a.ws_l = ws + n_o + n_s;
+  a.ws_tab = (int32_t*)(ws + n_o + 2 * n_s);
+  a.ticket = (int*)(ws + n_o + 2 * n_s + n_r);
+  a.deterministic = 1;
+  const int n_tab = (int)n_r;
+  const dim3 grid(a.nch, a.Hkv, a.B), cgrid(a.Hkv, a.B);
+  hipLaunchKernelGGL(decode_plan_kernel, dim3((n_tab + 255) / 256), dim3(256), 0, stream, a.ticket, a.ws_tab, n_tab);
+#define AXL_DEC32(DD, GG)                                                                          \
+  do {                                                                                              \
+    hipLaunchKernelGGL((decode_split_f32_kernel<DD, GG, PAGED>), grid, dim3(256), 0, stream, a);    \
+    hipLaunchKernelGGL((decode_combine_kernel<ElemF32, DD, GG>), cgrid, dim3(256), 0, stream, a);   \
+  } while (0)
+  if (D == 128 && gp == 4) AXL_DEC32(128, 4);
+  else if (D == 128 && gp == 8) AXL_DEC32(128, 8);
+  else if (D == 128) AXL_DEC32(128, 16);
+  else if (gp == 4) AXL_DEC32(64, 4);
+  else if (gp == 8) AXL_DEC32(64, 8);
+  else AXL_DEC32(64, 16);
+#undef AXL_DEC32
+  const hipError_t err = hipGetLastError();
+  if (err != hipSuccess) return set_error(AXL_ERR_LAUNCH, "%s: launch failed: %s", who, hipGetErrorString(err));
+  return AXL_OK;
+}
+
 int launch_paged_decode(const AxlPagedDecodeParams& p, hipStream_t stream) {
   DecArgs a{};
   a.q = (const __bf16*)p.q; a.k = (const __bf16*)p.k_pages; a.v = (const __bf16*)p.v_pages;
@@ -686,6 +851,7 @@ int launch_paged_decode(const AxlPagedDecodeParams& p, hipStream_t stream) {
   a.num_pages = p.num_pages; a.pps = p.pages_per_seq; a.kv_len = p.pages_per_seq * kPage;
   a.window = p.sliding_window < 0 ? -1 : p.sliding_window;
   a.scale = p.softmax_scale;
+  if (p.dtype == AXL_F32) return launch_f32<true>(a, p.head_dim, stream, "axl_paged_decode");
   return p.dtype == AXL_F16 ? launch_common<ElemF16, true>(a, p.head_dim, stream, "axl_paged_decode")
                             : launch_common<ElemBf16, true>(a, p.head_dim, stream, "axl_paged_decode");
 }
@@ -701,6 +867,7 @@ int launch_decode(const AxlDecodeParams& p, hipStream_t stream) {
   a.num_pages = 0; a.pps = (p.kv_len + kPage - 1) / kPage; a.kv_len = p.kv_len;
   a.window = p.sliding_window < 0 ? -1 : p.sliding_window;
   a.scale = p.softmax_scale;
+  if (p.dtype == AXL_F32) return launch_f32<false>(a, p.head_dim, stream, "axl_decode");
   return p.dtype == AXL_F16 ? launch_common<ElemF16, false>(a, p.head_dim, stream, "axl_decode")
                             : launch_common<ElemBf16, false>(a, p.head_dim, stream, "axl_decode");
 }

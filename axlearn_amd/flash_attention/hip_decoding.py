@@ -47,9 +47,9 @@ def _common_checks(self, input_batch: Nested, heads_per_kv: int) -> bool:
     query = input_batch["query"]
     if input_batch.get("logit_sink") is not None:
         return self._log_unsupported("logit_sink is not supported.")
-    if query.dtype not in (torch.bfloat16, torch.float16) or input_batch["key"].dtype != query.dtype:
+    if query.dtype not in (torch.bfloat16, torch.float16, torch.float32) or input_batch["key"].dtype != query.dtype:
         return self._log_unsupported(
-            f"{query.dtype=} / {input_batch['key'].dtype=} (supported: bfloat16 or float16, the same for both)"
+            f"{query.dtype=} / {input_batch['key'].dtype=} (supported: bfloat16, float16 or float32, the same for both)"
         )
     if query.shape[-1] not in (64, 128):
         return self._log_unsupported(f"head_dim {query.shape[-1]} (supported: 64, 128)")

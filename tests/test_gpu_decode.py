@@ -151,10 +151,19 @@ def test_decode_equals_last_row_of_prefill():
     assert _ok(dec.cpu(), full[:, -1].cpu())
 
 
-def test_dispatch_decode_end_to_end():
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_dispatch_decode_end_to_end(dtype):
     b, hq, hkv, d, pps = 4, 16, 2, 64, 32
     q, kp, vp, tables, lengths = ref.paged_inputs(21, batch=b, num_heads=hq, num_kv_heads=hkv, head_dim=d,
-                                                  page_size=16, pages_per_seq=pps, min_len=5, max_len=16 * pps)
+                                                  page_size=16, pages_per_seq=pps, min_len=5, max_len=16 * pps,
+                                                  dtype=dtype)
+
+    def _ok(got, want):  # the bars of the three dtypes
+        if dtype == torch.float32:
+            return got.dtype == dtype and ref.max_abs(got, want) <= 1e-5
+        f = 1.0 if dtype == torch.bfloat16 else 0.125
+        return got.dtype == dtype and (ref.max_abs(got, want) <= 2e-2 * f or ref.rel_l2(got, want) <= 1e-2 * f)
+
     tp = (lengths.long() - 1)[:, None].cuda()
     sp = torch.arange(16 * pps)[None].cuda()
     scale = d ** -0.5
@@ -178,7 +187,7 @@ def test_dispatch_decode_end_to_end():
     assert _ok(got.cpu(), want)
     # Multi-token query with a KV cache is not a decode step: the decode kernel declines and the
     # prefill kernel does not take cached calls either -> None.
-    q2 = torch.zeros(b, 2, hq, d, dtype=torch.bfloat16, device="cuda")
+    q2 = torch.zeros(b, 2, hq, d, dtype=dtype, device="cuda")
     assert flash_attention_implementation("gpu", query=q2, key=kk, value=vv, bias=wbias, kv_cache_type=KVCache) is None
 
 
@@ -278,6 +287,36 @@ def test_float16_decode_against_ref(b, s, h, hkv, d, padding, window):
         det2 = ops.decode(q[:, 0].cuda(), kk.cuda(), vv.cuda(), lengths.cuda(), softmax_scale=scale,
                           sliding_window=window)
     assert ok(det) and torch.equal(det, det2)
+
+
+@pytest.mark.parametrize("b,s,h,hkv,d,padding,window", [
+    (1, 1024, 32, 32, 64, 0, -1),     # shapes of decoding_test.py:95-163
+    (4, 512, 48, 6, 64, 111, -1),
+    (2, 1024, 16, 2, 128, 111, 127),
+    (1, 4096, 8, 1, 128, 0, -1),
+    (3, 640, 12, 4, 128, 5, 33),
+])
+def test_float32_decode_against_ref(b, s, h, hkv, d, padding, window):
+    """float32 (the reference's decode tests run float32 and float16 on GPU, decoding_test.py:33)
+    at the fp32 bar; paged and contiguous agree bit for bit (same arithmetic, fixed decomposition),
+    and a poisoned tail beyond the length changes nothing."""
+    pps = s // 16
+    q, kp, vp, tables, _ = ref.paged_inputs(13, batch=b, num_heads=h, num_kv_heads=hkv, head_dim=d, page_size=16,
+                                            pages_per_seq=pps, min_len=1, max_len=s, dtype=torch.float32)
+    lengths = torch.full((b,), s - padding, dtype=torch.int32)
+    lengths[0] = max(1, s // 3 + 1)
+    scale = d ** -0.5
+    want = ref.reference_decode(q, kp, vp, lengths, softmax_scale=scale, page_tables=tables,
+                                sliding_window=None if window < 0 else window)[:, 0]
+    got = ops.paged_decode(q[:, 0].cuda(), kp.cuda(), vp.cuda(), tables.cuda(), lengths.cuda(),
+                           softmax_scale=scale, sliding_window=window)
+    assert got.dtype == torch.float32 and ref.max_abs(got.cpu(), want) <= 1e-5, ref.max_abs(got.cpu(), want)
+    kk, vv = ref.reconstruct_kv(tables, kp), ref.reconstruct_kv(tables, vp)
+    for bi in range(b):  # rows at and beyond the length are never read into the result
+        kk[bi, int(lengths[bi]):] = float("nan")
+        vv[bi, int(lengths[bi]):] = float("nan")
+    got2 = ops.decode(q[:, 0].cuda(), kk.cuda(), vv.cuda(), lengths.cuda(), softmax_scale=scale, sliding_window=window)
+    assert torch.equal(got2, got)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
