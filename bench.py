@@ -34,7 +34,7 @@ HBM_PEAK_GBS = 8000.0           # MI355X HBM3E
 
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, in KiB; the
 # factors are what the same counters read for a plain 1 GiB copy kernel, `--calibrate-copy`).
-DKDV_TRAFFIC_BYTES = {"c2": 2.82e9}      # flash_bwd_dkdv_bf16_kernel<128>, workload c2
+DKDV_TRAFFIC_BYTES = {"c2": 2.57e9}      # flash_bwd_dkdv_kernel<128>, workload c2
 DECODE_SPLIT_TRAFFIC_BYTES = 4.25e9      # decode_split_kernel<128,4>, workload c4
 
 METRIC = "flash-attn fwd+bwd TFLOP/s; paged-decode HBM GB/s (% roofline), 1 MI355X"
@@ -140,13 +140,13 @@ def bench_flash(cfg, steps, warmup, cpu_baseline):
     result = dict(
         value=tf(fl_fwd + fl_bwd, ms_step), ms_per_step=ms_step,
         kernels={
-            "flash_fwd_bf16_kernel": dict(ms=ms_fwd, tflops=tf(fl_fwd, ms_fwd), algorithmic_tflop=fl_fwd / 1e12),
+            "flash_fwd_kernel": dict(ms=ms_fwd, tflops=tf(fl_fwd, ms_fwd), algorithmic_tflop=fl_fwd / 1e12),
             "bwd_delta_kernel": dict(ms=ms_delta),
-            "flash_bwd_dkdv_bf16_kernel": dict(ms=ms_dkdv, tflops=tf(fl_dkdv, ms_dkdv), algorithmic_tflop=fl_dkdv / 1e12),
-            "flash_bwd_dq_bf16_kernel": dict(ms=ms_dq, tflops=tf(fl_dq, ms_dq), algorithmic_tflop=fl_dq / 1e12),
+            "flash_bwd_dkdv_kernel": dict(ms=ms_dkdv, tflops=tf(fl_dkdv, ms_dkdv), algorithmic_tflop=fl_dkdv / 1e12),
+            "flash_bwd_dq_ring_kernel": dict(ms=ms_dq, tflops=tf(fl_dq, ms_dq), algorithmic_tflop=fl_dq / 1e12),
         },
         roofline=dict(
-            kernel="flash_bwd_dkdv_bf16_kernel", bound="mfma", achieved=tf(fl_dkdv, ms_dkdv),
+            kernel="flash_bwd_dkdv_kernel", bound="mfma", achieved=tf(fl_dkdv, ms_dkdv),
             peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s", frac=tf(fl_dkdv, ms_dkdv) / MFMA_BF16_PEAK_TFLOPS,
             traffic=DKDV_TRAFFIC_BYTES.get(cfg["name"]),
         ),
