@@ -281,6 +281,8 @@ def decode(
     *,
     softmax_scale: float = 1.0,
     sliding_window: int = -1,
+    workspace: Optional[torch.Tensor] = None,
+    out: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """q [B,Hq,D]; k/v [B,S,Hkv,D]; lengths [B] int32 -> [B,Hq,D]."""
     _require_cuda(q, k, v, lengths)
@@ -291,7 +293,8 @@ def decode(
         raise AxlError(_lib.AXL_ERR_UNSUPPORTED, "q must be contiguous")
     if lengths.dtype != torch.int32 or not lengths.is_contiguous():
         raise AxlError(_lib.AXL_ERR_INVALID_ARGUMENT, "lengths must be contiguous int32")
-    out = torch.empty((b, hq, d), dtype=q.dtype, device=q.device)
+    if out is None:
+        out = torch.empty((b, hq, d), dtype=q.dtype, device=q.device)
     p = AxlDecodeParams(
         q=q.data_ptr(), k=k.data_ptr(), v=v.data_ptr(), lengths=lengths.data_ptr(),
         out=out.data_ptr(), k_strides=_lib.strides4(k), v_strides=_lib.strides4(v),
@@ -300,9 +303,10 @@ def decode(
         softmax_scale=float(softmax_scale), workspace=None, workspace_bytes=0,
     )
     need = int(lib.axl_decode_workspace_bytes(ctypes.byref(p)))
-    ws = torch.empty((max(need, 16),), dtype=torch.uint8, device=q.device)
-    p.workspace = ws.data_ptr()
-    p.workspace_bytes = ws.numel()
+    if workspace is None or workspace.numel() * workspace.element_size() < need:
+        workspace = torch.empty((max(need, 16),), dtype=torch.uint8, device=q.device)
+    p.workspace = workspace.data_ptr()
+    p.workspace_bytes = workspace.numel() * workspace.element_size()
     _lib.check(lib.axl_decode(ctypes.byref(p), _lib.current_stream_ptr()))
     return out
 

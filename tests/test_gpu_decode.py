@@ -191,6 +191,45 @@ def test_dispatch_decode_end_to_end(dtype):
     assert flash_attention_implementation("gpu", query=q2, key=kk, value=vv, bias=wbias, kv_cache_type=KVCache) is None
 
 
+def test_decode_replays_from_a_captured_graph():
+    """The decode call enqueues kernels only (no memsets, no allocation inside the library, no
+    synchronisation), so it can be captured into a graph.  Every replay, with eager work between the
+    replays, must equal the eager result bit for bit (fixed decomposition)."""
+    b, hq, hkv, d, pps = 5, 16, 4, 128, 40
+    q, kp, vp, tables, lengths = ref.paged_inputs(31, batch=b, num_heads=hq, num_kv_heads=hkv, head_dim=d,
+                                                  page_size=16, pages_per_seq=pps, min_len=3, max_len=16 * pps)
+    qc, kc, vc, tc, lc = q[:, 0].cuda(), kp.cuda(), vp.cuda(), tables.cuda(), lengths.cuda()
+    kk, vv = ref.reconstruct_kv(tables, kp).cuda(), ref.reconstruct_kv(tables, vp).cuda()
+    with _deterministic():
+        ws = torch.empty((ops.paged_decode_workspace_bytes(b, hq, hkv, d, pps) + 16,), dtype=torch.uint8, device="cuda")
+        ws2 = torch.empty_like(ws)
+        out_g, out_g2 = torch.empty_like(qc), torch.empty_like(qc)
+        eager = ops.paged_decode(qc, kc, vc, tc, lc, softmax_scale=0.1)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):  # warm-up outside the capture
+            ops.paged_decode(qc, kc, vc, tc, lc, softmax_scale=0.1, workspace=ws, out=out_g)
+            ops.decode(qc, kk, vv, lc, softmax_scale=0.1, workspace=ws2, out=out_g2)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            ops.paged_decode(qc, kc, vc, tc, lc, softmax_scale=0.1, workspace=ws, out=out_g)
+            ops.decode(qc, kk, vv, lc, softmax_scale=0.1, workspace=ws2, out=out_g2)
+        for rep in range(3):
+            out_g.zero_()
+            out_g2.zero_()
+            ws.random_(0, 255)  # stale records and counters must not matter
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out_g, eager) and torch.equal(out_g2, eager), rep
+            # eager work of the same kind between the replays
+            again = ops.paged_decode(qc, kc, vc, tc, lc, softmax_scale=0.1)
+            assert torch.equal(again, eager)
+            # new inputs in the captured buffers are picked up by the next replay
+            lc.copy_(torch.clamp(lengths + 7 * (rep + 1), max=16 * pps).cuda())
+            eager = ops.paged_decode(qc, kc, vc, tc, lc, softmax_scale=0.1)
+
+
 def test_baseline_c4_full_size():
     """BASELINE config 4 at full size; the oracle checks a sample of sequences (incl. the shortest
     and the longest), the rest is covered by permutation invariance at full size."""

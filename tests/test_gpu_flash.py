@@ -449,6 +449,33 @@ def test_dispatch_and_autograd_end_to_end(dtype):
     assert ref.max_abs(o3.detach().cpu().float(), out.detach().cpu().float()) < 1e-2
 
 
+def test_forward_and_backward_replay_from_a_captured_graph():
+    """Forward + backward enqueue kernels only, so they can be captured into a graph; every replay,
+    with eager work between the replays, equals the eager result bit for bit."""
+    b, t, hq, hkv, d = 2, 512, 4, 2, 128
+    q, k, v, do = (x.cuda() for x in _inputs(b, t, hq, hkv, d, torch.bfloat16))
+    segs = ref.packed_segment_ids(4, b, t, max_docs=3).cuda()
+    kw = dict(softmax_scale=d ** -0.5, mask_kind=ops.MASK_CAUSAL, segment_ids=segs)
+    out_e, lse_e = ops.flash_fwd(q, k, v, **kw)
+    grads_e = ops.flash_bwd(q, k, v, out_e, lse_e, do, **kw)
+    bufs = (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v),
+            torch.empty((2 * b * hq * t * 4 + 16,), dtype=torch.uint8, device="cuda"))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_g, lse_g = ops.flash_fwd(q, k, v, **kw)
+        ops.flash_bwd(q, k, v, out_g, lse_g, do, buffers=bufs, **kw)
+    for rep in range(3):
+        for x in (out_g, lse_g, *bufs):
+            x.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, out_e) and torch.equal(lse_g, lse_e), rep
+        assert all(torch.equal(g, e) for g, e in zip(bufs[:3], grads_e)), rep
+        q.copy_(q.roll(1, dims=1))  # new inputs in the captured buffers
+        out_e, lse_e = ops.flash_fwd(q, k, v, **kw)
+        grads_e = ops.flash_bwd(q, k, v, out_e, lse_e, do, **kw)
+
+
 # ----------------------------------------------------------------------------- logit sink, head dims
 
 
