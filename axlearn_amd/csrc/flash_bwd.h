@@ -12,7 +12,7 @@ struct BwdArgs {
   const void* out;
   const void* dout;
   const float* lse;
-  float* delta;  // workspace [B, Hq, T]: rowsum(out * dO)
+  float* ndelta; // workspace [B, Hq, T]: -rowsum(out * dO); negated so that a dP accumulator chain can start from it
   float* lse2;   // workspace [B, Hq, T]: -lse * log2(e), the exponent offset of the dK/dV kernel
   void* dq;
   void* dk;

@@ -60,7 +60,7 @@ __global__ __launch_bounds__(256) void bwd_delta_kernel(const BwdArgs a) {
   acc += __shfl_xor(acc, 8, 64);
   if (row < rows && sub == 0) {
     const int64_t idx = ((int64_t)b * a.Hq + h) * a.T + t;
-    a.delta[idx] = acc;
+    a.ndelta[idx] = -acc;
     a.lse2[idx] = a.lse[idx] * (-kLog2e);
   }
 }
@@ -72,7 +72,7 @@ __global__ __launch_bounds__(256) void bwd_delta_kernel(const BwdArgs a) {
 // ---------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void bwd_dsink_kernel(const float* __restrict__ sink,
                                                         const float* __restrict__ lse,
-                                                        const float* __restrict__ delta,
+                                                        const float* __restrict__ ndelta,
                                                         float* __restrict__ d_sink, int B, int Hq,
                                                         int T) {
   __shared__ float red[256];
@@ -81,7 +81,7 @@ __global__ __launch_bounds__(256) void bwd_dsink_kernel(const float* __restrict_
   float acc = 0.f;
   for (int b = 0; b < B; b++) {
     const int64_t base = ((int64_t)b * Hq + h) * T;
-    for (int t = tid; t < T; t += 256) acc -= expf(sk - lse[base + t]) * delta[base + t];
+    for (int t = tid; t < T; t += 256) acc += expf(sk - lse[base + t]) * ndelta[base + t];
   }
   red[tid] = acc;
   __syncthreads();
@@ -136,7 +136,7 @@ __global__ __launch_bounds__(256) void flash_bwd_dq_aux_kernel(const BwdArgs a) 
   }
   const int64_t stat_idx = ((int64_t)b * a.Hq + h) * a.T + q0 + l32;
   const float lse2 = a.lse[stat_idx] * kLog2e;
-  const float delta = a.delta[stat_idx];
+  const float delta = -a.ndelta[stat_idx];
 
   int k_begin = 0, k_end = a.S;
   if (a.mask_kind != AXL_MASK_NONE) {
@@ -328,8 +328,8 @@ int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream)
   const int dt = p.dtype;
   BwdArgs a;
   a.q = p.q; a.k = p.k; a.v = p.v; a.out = p.out; a.dout = p.d_out; a.lse = p.lse;
-  a.delta = (float*)p.workspace;
-  a.lse2 = a.delta + (size_t)p.batch * p.num_q_heads * p.q_len;
+  a.ndelta = (float*)p.workspace;
+  a.lse2 = a.ndelta + (size_t)p.batch * p.num_q_heads * p.q_len;
   a.dq = p.dq; a.dk = p.dk; a.dv = p.dv; a.seg = p.segment_ids;
   a.qs = to_s3(p.q_strides); a.ks = to_s3(p.k_strides); a.vs = to_s3(p.v_strides);
   a.os = to_s3(p.out_strides); a.dos = to_s3(p.d_out_strides); a.dqs = to_s3(p.dq_strides);
@@ -391,7 +391,7 @@ int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream)
 #undef AXL_LAUNCH
   if ((phases & AXL_BWD_DELTA) && p.d_logit_sink && err == hipSuccess) {
     hipLaunchKernelGGL(bwd_dsink_kernel, dim3(p.num_q_heads), dim3(256), 0, stream, p.logit_sink,
-                       p.lse, a.delta, p.d_logit_sink, p.batch, p.num_q_heads, p.q_len);
+                       p.lse, a.ndelta, p.d_logit_sink, p.batch, p.num_q_heads, p.q_len);
     err = hipGetLastError();
   }
   if (err != hipSuccess)

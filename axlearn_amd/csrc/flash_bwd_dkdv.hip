@@ -35,7 +35,7 @@ struct DkvTile {
   static constexpr int ROWB = D * 2;         // bytes per row: unpadded, chunks swizzled (tile_swizzle)
   static constexpr int TILE_BYTES = BQ * ROWB;                   // Q tile, then the dO tile
   static constexpr int STAT_BASE = 2 * TILE_BYTES;
-  static constexpr int STAT_BYTES = 4 * BQ * 4;  // -lse*log2e | delta | segment id | (unused) per query row
+  static constexpr int STAT_BYTES = 4 * BQ * 4;  // -lse*log2e | -delta | segment id | (unused) per query row
   static constexpr int BUF_BYTES = STAT_BASE + STAT_BYTES;
   static constexpr int NBUF = 5;
   static constexpr int RPI = 1024 / ROWB;                        // rows per direct-to-LDS instruction
@@ -127,7 +127,7 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
   const __bf16* d_src = (const __bf16*)a.dout + b * a.dos.b + (int64_t)(hk * G) * a.dos.h + (int64_t)t_begin * Tile::BQ * a.dos.s;
   const int64_t stat_row0 = ((int64_t)b * a.Hq + hk * G) * a.T + (int64_t)t_begin * Tile::BQ;
   const bool s_is_seg = HAS_SEG && st_kind == 2;
-  const char* s_src = st_kind == 1 ? (const char*)(a.delta + stat_row0) : (const char*)(a.lse2 + stat_row0);  // wave-uniform
+  const char* s_src = st_kind == 1 ? (const char*)(a.ndelta + stat_row0) : (const char*)(a.lse2 + stat_row0);  // wave-uniform
   if (s_is_seg) s_src = (const char*)(a.seg + (int64_t)b * a.T + (int64_t)t_begin * Tile::BQ);
   const unsigned s_lane = 16 * (lane & 7);  // lanes 0..7 fetch 4 query rows each
   const int64_t q_step = (int64_t)Tile::BQ * a.qs.s, d_step = (int64_t)Tile::BQ * a.dos.s;
@@ -251,7 +251,8 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
       dpv_ = kept_ ? dpv_ * a.aux.keep_scale : 0.f; /* gpu_attention.py:509-512 */            \
       s_e[r_] = kept_ ? p_ : 0.f; /* P that multiplies dO: dropped entries removed */          \
     }                                                                                          \
-    dp_e[r_] = p_ * (dpv_ - del_v[r_ / 4][r_ % 4]);                                            \
+    if constexpr (AUX) dp_e[r_] = p_ * (dpv_ + del_v[r_ / 4][r_ % 4]); /* del_v holds -delta */ \
+    else dp_e[r_] = p_ * dpv_; /* the dP chain started from -delta */                          \
   }
 #define AXL_ELEM(R_)                                                                           \
   {                                                                                            \
@@ -363,9 +364,13 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
     wait_all_vmem();  // tiles 0..3 have landed; nothing issued before the loop is pending
     __syncthreads();
     // Pipeline fill: stage A and the elementwise stage of tile 0, stage A of tile 1.
-    AXL_STAGE_A_PLAIN(buf_b, s_e, dp_e)
     AXL_READ_STATS_PART(buf_b, 0, lse_v, del_v, seg_v)
     AXL_READ_STATS_PART(buf_b, 1, lse_v, del_v, seg_v)
+    if constexpr (!AUX) {  // the dP chain starts from -delta
+#pragma unroll
+      for (int r = 0; r < 16; r++) dp_e[r] = del_v[r / 4][r % 4];
+    }
+    AXL_STAGE_A_PLAIN(buf_b, s_e, dp_e)
     diff0 = (t_begin * Tile::BQ + a.q_off + 8 * g) - kpos;
 #pragma unroll
     for (int r = 0; r < 16; r++) AXL_ELEM(r)
@@ -373,9 +378,13 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
     for (int i = 0; i < 8; i++) AXL_PACK_PAIR(pb, dsb, i)
 #pragma unroll
     for (int r = 0; r < 16; r++) s_e[r] = dp_e[r] = 0.f;
-    AXL_STAGE_A_PLAIN(buf_e, s_e, dp_e)
     AXL_READ_STATS_PART(buf_e, 0, lse_v, del_v, seg_v)
     AXL_READ_STATS_PART(buf_e, 1, lse_v, del_v, seg_v)
+    if constexpr (!AUX) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) dp_e[r] = del_v[r / 4][r % 4];
+    }
+    AXL_STAGE_A_PLAIN(buf_e, s_e, dp_e)
     if constexpr (AUX) {                 // ... and of tile 1, for the first iteration
       const char* bp_;
       const uint8_t* dp_;
@@ -400,6 +409,7 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
 #pragma unroll
     for (int i = 0; i < kAheadB; i++) bfr[i] = bfr_next[i];
     floatx16 s_a, dp_a;
+    floatx16 dp_start = zero16;          // first operand of the dP chain: -delta without a dropout mask
     PackedOperand pb_n, dsb_n;           // tile j + 1, packed as its elements complete
     int q0_p = q0_s, h_p = h_s;
     const unsigned lds_s = lds_address(buf_s);
@@ -449,7 +459,7 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
         if constexpr (x % 2 == 0)
           s_a = E::mfma_32x32x16(afr[x], kf[x / 2], x == 0 ? zero16 : s_a);
         else
-          dp_a = E::mfma_32x32x16(afr[x], vf[x / 2], x == 1 ? zero16 : dp_a);
+          dp_a = E::mfma_32x32x16(afr[x], vf[x / 2], x == 1 ? dp_start : dp_a);
       }
       // ---- elementwise stage of tile j+1: element e starts in slot e (NS-3)/16 and takes three
       // slots; pairs are packed one slot after their second element is complete
@@ -481,7 +491,15 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
           lse_v[i] = *(const floatx4*)st_;
           if (HAS_SEG) seg_v[i] = *(const intx4*)(st_ + 2 * Tile::BQ * 4);
         }
-        if (n == (4 * i + 3) * (NS - 3) / 16 + 3) del_v[i] = *(const floatx4*)(st_ + Tile::BQ * 4);
+        if constexpr (AUX) {
+          if (n == (4 * i + 3) * (NS - 3) / 16 + 3) del_v[i] = *(const floatx4*)(st_ + Tile::BQ * 4);
+        } else {
+          // -delta of tile j+2's rows: what its dP chain starts from (slot NB + 1)
+          if (n == NB - 4 + i) {
+            const floatx4 d4 = *(const floatx4*)(st_ + Tile::BQ * 4);
+            dp_start[4 * i] = d4[0]; dp_start[4 * i + 1] = d4[1]; dp_start[4 * i + 2] = d4[2]; dp_start[4 * i + 3] = d4[3];
+          }
+        }
       }
       __builtin_amdgcn_sched_barrier(0);
     };

@@ -98,12 +98,12 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
     delta = xor32_sum(part);
     off = a.lse[stat_idx] * (-kLog2e);
     if (live && g == 0) {
-      a.delta[stat_idx] = delta;
+      a.ndelta[stat_idx] = -delta;
       a.lse2[stat_idx] = off;
     }
   } else {
     off = a.lse2[stat_idx];
-    delta = a.delta[stat_idx];
+    delta = -a.ndelta[stat_idx];
   }
   const int qpos = q0 + l32 + a.q_off;
   const int qpos_min = q0 + a.q_off, qpos_max = q0 + 31 + a.q_off;  // of the wavefront

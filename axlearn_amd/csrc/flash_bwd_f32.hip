@@ -72,7 +72,7 @@ __global__ __launch_bounds__(128) void flash_bwd_dq_f32_kernel(const BwdArgs a) 
   const float* kp = (const float*)a.k + b * a.ks.b + hk * a.ks.h;
   const float* vp = (const float*)a.v + b * a.vs.b + hk * a.vs.h;
   const int64_t stat = ((int64_t)b * a.Hq + h) * a.T + q0 + l32;
-  const float lse_q = a.lse[stat], delta_q = a.delta[stat];
+  const float lse_q = a.lse[stat], delta_q = -a.ndelta[stat];
 
   int k_begin = 0, k_end = a.S;
   if (a.mask_kind != AXL_MASK_NONE) {
@@ -224,7 +224,7 @@ __global__ __launch_bounds__(128) void flash_bwd_dkdv_f32_kernel(const BwdArgs a
       stage_rows<D, 128>(do_lds, dop + (int64_t)qt0 * a.dos.s, a.dos.s, Tile::TILE, tid);
       if (tid < Tile::TILE) {
         lse_lds[tid] = a.lse[stat + qt0 + tid];
-        delta_lds[tid] = a.delta[stat + qt0 + tid];
+        delta_lds[tid] = -a.ndelta[stat + qt0 + tid];
       }
       __syncthreads();
       bool skip = false;
