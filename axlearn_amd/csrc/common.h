@@ -267,10 +267,9 @@ __device__ __forceinline__ void decode_block(int bid, int nqb, int B, int Hq, in
   const int npairs = B * Hkv;
   if (npairs % 8 == 0) {
     const int xcd = bid & 7, slot = bid >> 3;
-    const int per_qb = (npairs >> 3) * G;
-    const int qb_rev = slot / per_qb, rem = slot % per_qb;
-    const int pair = xcd + 8 * (rem / G);
-    qb = nqb - 1 - qb_rev;
+    const int per_pair = nqb * G;
+    const int pair = xcd + 8 * (slot / per_pair), rem = slot % per_pair;
+    qb = nqb - 1 - rem / G;
     b = pair / Hkv;
     h = (pair % Hkv) * G + rem % G;
   } else {

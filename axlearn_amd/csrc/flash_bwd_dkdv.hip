@@ -26,6 +26,10 @@
 
 #include "flash_bwd.h"
 
+#ifndef AXL_DKDV_PG
+#define AXL_DKDV_PG 2
+#endif
+
 namespace axl {
 
 template <int D>
@@ -60,11 +64,25 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l32 = lane & 31, g = lane >> 5;
   const int G = a.Hq / a.Hkv;
-  // blockIdx -> (key block, batch, kv head); earliest key blocks (most queries under a causal
-  // mask) first.
-  const int kb = blockIdx.x / (a.B * a.Hkv);
-  const int rem = blockIdx.x % (a.B * a.Hkv);
-  const int b = rem / a.Hkv, hk = rem % a.Hkv;
+  // blockIdx -> (key block, batch, kv head).  When the (batch, kv head) pairs divide evenly over the
+  // 8 XCDs (workgroup i is dispatched to XCD i % 8), an XCD works through one pair after the other,
+  // so the workgroups that run together stream the same Q / dO rows through that XCD's L2; within a
+  // pair the earliest key blocks (most queries under a causal mask) come first.
+  const int npairs = a.B * a.Hkv, nkb = a.S / Tile::BKV;
+  int kb, pair;
+  if (npairs % 8 == 0) {
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int ppx = npairs >> 3;                     // pairs per XCD
+    const int grp = slot / (AXL_DKDV_PG * nkb);      // group of AXL_DKDV_PG pairs worked through together
+    const int r = slot - grp * (AXL_DKDV_PG * nkb);
+    const int pg = min(AXL_DKDV_PG, ppx - grp * AXL_DKDV_PG);
+    pair = xcd + 8 * (grp * AXL_DKDV_PG + r % pg);
+    kb = r / pg;
+  } else {
+    kb = blockIdx.x / npairs;
+    pair = blockIdx.x % npairs;
+  }
+  const int b = pair / a.Hkv, hk = pair % a.Hkv;
   const int k0_wg = kb * Tile::BKV;
   const int k0 = k0_wg + wave * 32;  // this wavefront's keys
 
