@@ -109,7 +109,12 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
   if (HAS_SEG) shrink_to_segment_hull(seg_k, a.seg + (int64_t)b * a.T, tid, q_begin, q_end);
   const int t_begin = q_begin / Tile::BQ;
   const int nt = max(0, (q_end + Tile::BQ - 1) / Tile::BQ - t_begin);
-  const int total = nt * G;  // tiles in processing order: query head (outer) x query tile (inner)
+  // Tiles in processing order: query tile (outer, from the LAST one down to the diagonal) x query head
+  // (inner).  Every workgroup of a (batch, kv head) pair starts at the same last tile and walks down
+  // until it reaches its own diagonal, so the workgroups that run together read the same Q / dO rows
+  // at the same time and all but one of them find them in L2.
+  const int total = nt * G;
+  const int t_first = t_begin + max(nt - 1, 0);  // the tile the sequence starts with
   // keep(q, k)  <=>  (unsigned)(qpos - kpos) <= limit
   const unsigned limit = a.mask_kind == AXL_MASK_NONE             ? 0xffffffffu
                          : a.mask_kind == AXL_MASK_SLIDING_WINDOW ? (unsigned)a.window
@@ -140,19 +145,21 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
   }
   const int st_kind = wave;
   // Running source pointers of the prefetch cursor, advanced by wave-uniform steps: no 64-bit
-  // multiplies inside the loop.  Tile sequence: query head (outer) x query tile (inner).
-  const __bf16* q_src = (const __bf16*)a.q + b * a.qs.b + (int64_t)(hk * G) * a.qs.h + (int64_t)t_begin * Tile::BQ * a.qs.s;
-  const __bf16* d_src = (const __bf16*)a.dout + b * a.dos.b + (int64_t)(hk * G) * a.dos.h + (int64_t)t_begin * Tile::BQ * a.dos.s;
-  const int64_t stat_row0 = ((int64_t)b * a.Hq + hk * G) * a.T + (int64_t)t_begin * Tile::BQ;
+  // multiplies inside the loop.  A step goes to the next head of the same query tile, a wrap from
+  // the last head back to the first head of the tile before.
+  const __bf16* q_src = (const __bf16*)a.q + b * a.qs.b + (int64_t)(hk * G) * a.qs.h + (int64_t)t_first * Tile::BQ * a.qs.s;
+  const __bf16* d_src = (const __bf16*)a.dout + b * a.dos.b + (int64_t)(hk * G) * a.dos.h + (int64_t)t_first * Tile::BQ * a.dos.s;
+  const int64_t stat_row0 = ((int64_t)b * a.Hq + hk * G) * a.T + (int64_t)t_first * Tile::BQ;
   const bool s_is_seg = HAS_SEG && st_kind == 2;
   const char* s_src = st_kind == 1 ? (const char*)(a.ndelta + stat_row0) : (const char*)(a.lse2 + stat_row0);  // wave-uniform
-  if (s_is_seg) s_src = (const char*)(a.seg + (int64_t)b * a.T + (int64_t)t_begin * Tile::BQ);
+  if (s_is_seg) s_src = (const char*)(a.seg + (int64_t)b * a.T + (int64_t)t_first * Tile::BQ);
   const unsigned s_lane = 16 * (lane & 7);  // lanes 0..7 fetch 4 query rows each
-  const int64_t q_step = (int64_t)Tile::BQ * a.qs.s, d_step = (int64_t)Tile::BQ * a.dos.s;
-  const int64_t q_wrap = a.qs.h - (int64_t)(nt - 1) * q_step;    // last tile of a head -> first of next
-  const int64_t d_wrap = a.dos.h - (int64_t)(nt - 1) * d_step;
-  const int64_t s_step = Tile::BQ * 4, s_wrap = ((int64_t)a.T - (int64_t)(nt - 1) * Tile::BQ) * 4;
-  const int64_t seg_wrap = -(int64_t)(nt - 1) * Tile::BQ * 4;   // segment ids do not depend on the head
+  const int64_t q_step = a.qs.h, d_step = a.dos.h;
+  const int64_t q_wrap = -(int64_t)(G - 1) * a.qs.h - (int64_t)Tile::BQ * a.qs.s;
+  const int64_t d_wrap = -(int64_t)(G - 1) * a.dos.h - (int64_t)Tile::BQ * a.dos.s;
+  // statistics rows are [B, Hq, T] fp32; segment ids do not depend on the head
+  const int64_t s_step = s_is_seg ? 0 : (int64_t)a.T * 4;
+  const int64_t s_wrap = s_is_seg ? -(int64_t)Tile::BQ * 4 : (-(int64_t)(G - 1) * a.T - Tile::BQ) * 4;
   const unsigned lds0 = lds_address(smem);
   // The k-th group of loads (Q rows, dO rows, statistics) of the cursor's tile into the buffer at LDS
   // address BUF_; all from scalar bases, no vector instruction forms an address.
@@ -174,17 +181,17 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
     AXL_DMA(BUF_, 0) AXL_DMA(BUF_, 1) AXL_DMA(BUF_, 2)                                            \
   }
   // Prefetch cursor; it stops at the last tile (re-fetching that tile is harmless).
-  int pf_idx = 0, pf_t = 0, pf_h = 0;  // tile number, query tile within the head, head within the group
+  int pf_idx = 0, pf_t = max(nt - 1, 0), pf_h = 0;  // tile number, query tile (from t_begin), head within the group
 #define AXL_ADVANCE()                                                       \
   {                                                                         \
     const bool adv_ = pf_idx + 1 < total;                                   \
-    const bool wrap_ = adv_ && (pf_t + 1 == nt);                            \
+    const bool wrap_ = adv_ && (pf_h + 1 == G);                             \
     pf_idx += adv_ ? 1 : 0;                                                 \
-    pf_t = wrap_ ? 0 : pf_t + (adv_ ? 1 : 0);                               \
-    pf_h += wrap_ ? 1 : 0;                                                  \
+    pf_h = wrap_ ? 0 : pf_h + (adv_ ? 1 : 0);                               \
+    pf_t -= wrap_ ? 1 : 0;                                                  \
     q_src += adv_ ? (wrap_ ? q_wrap : q_step) : 0;                          \
     d_src += adv_ ? (wrap_ ? d_wrap : d_step) : 0;                          \
-    s_src += adv_ ? (wrap_ ? (s_is_seg ? seg_wrap : s_wrap) : s_step) : 0;  \
+    s_src += adv_ ? (wrap_ ? s_wrap : s_step) : 0;                          \
   }
 
   char* buf_b = smem;                         // tile j     (stage B reads)
@@ -353,7 +360,7 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
   constexpr int LD_SLOT0 = 2;                 // one per slot from here on, after the cursor moved in slot 1
   static_assert(LD_SLOT0 + NLD <= NS, "the loads of a tile fit into one iteration");
   TrFrag bfr_next[kAheadB];            // first stage-B fragments of the next iteration
-  int q0_a = t_begin * Tile::BQ, q0_s = q0_a;  // first query of tiles j+2 and j+3
+  int q0_a = t_first * Tile::BQ, q0_s = q0_a;  // first query of tiles j+2 and j+3
   int h_a = 0, h_s = 0;                        // and their heads within the group
 
   if (total > 0) {
@@ -375,7 +382,7 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
     if constexpr (AUX) {                 // bias / dropout columns of tile 0
       const char* bp_;
       const uint8_t* dp_;
-      AXL_AUX_ROW0(0, t_begin * Tile::BQ, bp_, dp_)
+      AXL_AUX_ROW0(0, t_first * Tile::BQ, bp_, dp_)
 #pragma unroll
       for (int r = 0; r < 16; r++) AXL_AUX_LOAD(bp_, dp_, r, braw_v, draw_v)
     }
@@ -389,7 +396,7 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
       for (int r = 0; r < 16; r++) dp_e[r] = del_v[r / 4][r % 4];
     }
     AXL_STAGE_A_PLAIN(buf_b, s_e, dp_e)
-    diff0 = (t_begin * Tile::BQ + a.q_off + 8 * g) - kpos;
+    diff0 = (t_first * Tile::BQ + a.q_off + 8 * g) - kpos;
 #pragma unroll
     for (int r = 0; r < 16; r++) AXL_ELEM(r)
 #pragma unroll
@@ -553,9 +560,9 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
     h_s = h_p;
   }
   };
-  // Tile t (within a head's run of nt tiles) needs no mask for this wavefront's 32 keys when its
-  // queries all see them: t in [u_lo, u_hi].  In processing order (head outer, tile inner) the
-  // elementwise tile of iteration j is e = j + 1.
+  // Query tile t (counted from t_begin) needs no mask for this wavefront's 32 keys when its queries
+  // all see them: t in [u_lo, u_hi].  In processing order tile number e is query tile nt - 1 - e / G
+  // of head e % G, and the elementwise tile of iteration j is e = j + 1.
   auto floor_div = [](int x, int y) { return x >= 0 ? x / y : -((-x + y - 1) / y); };
   int u_lo = 0, u_hi = nt - 1;
   if (a.mask_kind != AXL_MASK_NONE) {
@@ -613,11 +620,9 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
       run(j, j_end, masked_c);
       j = max(j, j_end);
     };
-    for (int hh = 0; hh < G; hh++) {
-      run_to(hh * nt + u_lo, std::true_type{});
-      run_to(hh * nt + u_hi + 1, std::false_type{});
-      run_to((hh + 1) * nt, std::true_type{});
-    }
+    run_to(G * (nt - 1 - u_hi), std::true_type{});   // far end of a sliding window
+    run_to(G * (nt - u_lo), std::false_type{});      // interior
+    run_to(total, std::true_type{});                 // down to the diagonal
     run(j, total, std::true_type{});  // the last iteration (its elementwise tile is past the end)
   }
 #undef AXL_AUX_ROW0
