@@ -34,7 +34,7 @@ HBM_PEAK_GBS = 8000.0           # MI355X HBM3E
 
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, in KiB; the
 # factors are what the same counters read for a plain 1 GiB copy kernel, `--calibrate-copy`).
-DKDV_TRAFFIC_BYTES = {"c2": 2.59e9}      # flash_bwd_dkdv_kernel<128>, workload c2
+DKDV_TRAFFIC_BYTES = {"c2": 0.98e9}      # flash_bwd_dkdv_kernel<128>, workload c2
 DECODE_SPLIT_TRAFFIC_BYTES = 4.25e9      # decode_split_kernel<128,4>, workload c4
 
 METRIC = "flash-attn fwd+bwd TFLOP/s; paged-decode HBM GB/s (% roofline), 1 MI355X"
