@@ -258,6 +258,57 @@ __device__ __forceinline__ void shrink_to_segment_hull(int my_id, const int32_t*
   if (hi < lo) hi = lo;
 }
 
+// One pass over the segment ids of the rows [lo, hi) that a workgroup loops over, in groups of GROUP
+// consecutive rows (GROUP a multiple of 4; ids 16-byte aligned; the row count a multiple of GROUP):
+//   * s_uniform[i], i < cap, gets the id of group lo / GROUP + i if its rows all carry one id, else
+//     `not_uniform` (groups from the one that holds row `lo` on; the return value is that group);
+//   * [lo, hi) is shrunk, in whole groups, to the hull of the groups that hold an id between the
+//     smallest and the largest id of the workgroup's own rows (`my_id`, passed by every thread): only
+//     such a group can hold a row that matches one of them.
+// Called by all NT threads of the workgroup; contains barriers.
+template <int GROUP, int NT>
+__device__ __forceinline__ int classify_segment_groups(int my_id, const int32_t* ids, int tid, int& lo, int& hi,
+                                                       int* s_uniform, int cap, int not_uniform) {
+  __shared__ int s_rng[4];
+  if (tid == 0) {
+    s_rng[0] = 0x7fffffff;       // smallest own id
+    s_rng[1] = -0x7fffffff - 1;  // largest own id
+    s_rng[2] = 0x7fffffff;       // first candidate group
+    s_rng[3] = -1;               // last candidate group
+  }
+  __syncthreads();
+  atomicMin(&s_rng[0], my_id);
+  atomicMax(&s_rng[1], my_id);
+  __syncthreads();
+  const int id_min = s_rng[0], id_max = s_rng[1];
+  const int g0 = lo / GROUP, g1 = (hi + GROUP - 1) / GROUP;
+  int first = 0x7fffffff, last = -1;
+  for (int i = g0 + tid; i < g1; i += NT) {
+    const intx4* p = (const intx4*)(ids + (int64_t)i * GROUP);
+    int mn = 0x7fffffff, mx = -0x7fffffff - 1;
+#pragma unroll
+    for (int v = 0; v < GROUP / 4; v++) {
+      const intx4 x = p[v];
+      mn = min(min(mn, min(x[0], x[1])), min(x[2], x[3]));
+      mx = max(max(mx, max(x[0], x[1])), max(x[2], x[3]));
+    }
+    if (i - g0 < cap) s_uniform[i - g0] = mn == mx ? mn : not_uniform;
+    if (mx >= id_min && mn <= id_max) {
+      first = min(first, i);
+      last = max(last, i);
+    }
+  }
+  if (last >= 0) {
+    atomicMin(&s_rng[2], first);
+    atomicMax(&s_rng[3], last);
+  }
+  __syncthreads();
+  lo = max(lo, s_rng[2] == 0x7fffffff ? hi : s_rng[2] * GROUP);
+  hi = min(hi, (s_rng[3] + 1) * GROUP);
+  if (hi < lo) hi = lo;
+  return g0;
+}
+
 // Decodes blockIdx.x into (query block, batch, query head).  Heaviest query blocks (most visible
 // keys under a causal mask) are issued first; when the (batch, kv head) pairs divide evenly over
 // the 8 XCDs, all workgroups of a pair run on one XCD (workgroup i is dispatched to XCD i % 8).

@@ -96,27 +96,19 @@ void flash_fwd_kernel(const FwdArgs a) {
   }
   const int seg_q = a.seg ? a.seg[(int64_t)b * a.T + q0 + l32] : 0;
   const int32_t* seg_k = a.seg ? a.seg + (int64_t)b * a.T : nullptr;
-  if (seg_k) shrink_to_segment_hull(seg_q, seg_k, tid, k_begin, k_end);
+  // With segment ids: one pass over the ids of the key range shrinks it to the hull of the keys whose
+  // id lies between the smallest and the largest id of this workgroup's queries, and records for
+  // every 64-key tile whether it carries a single id.  A tile whose keys all carry the one id that
+  // all 32 queries of a wavefront carry needs no segment mask.
+  __shared__ int s_tile_id[kMaxSegTiles];
+  int seg_t0 = 0;          // tile that s_tile_id[0] describes
+  if (seg_k) seg_t0 = classify_segment_groups<Tile::BK, 256>(seg_q, seg_k, tid, k_begin, k_end, s_tile_id, kMaxSegTiles,
+                                                            kSegNotUniform);
   const int t_begin = k_begin / Tile::BK;
   const int t_end = (k_end + Tile::BK - 1) / Tile::BK;
-  // Key tiles whose 64 keys all carry the segment id that all 32 queries of this wavefront carry need
-  // no segment mask: s_tile_id[t - t_begin] is the tile's id if it has only one.
-  __shared__ int s_tile_id[kMaxSegTiles];
   bool seg_fast = false;   // this wavefront's queries share one id and the table covers the tiles
   int wq_id = 0;
-  if (seg_k && t_end - t_begin <= kMaxSegTiles) {
-    for (int i = tid; i < t_end - t_begin; i += 256) {
-      const int32_t* ids = seg_k + (t_begin + i) * Tile::BK;
-      const int id0 = ids[0];
-      bool same = true;
-#pragma unroll
-      for (int v = 0; v < Tile::BK / 4; v++) {
-        const intx4 x = ((const intx4*)ids)[v];
-        same = same && x[0] == id0 && x[1] == id0 && x[2] == id0 && x[3] == id0;
-      }
-      s_tile_id[i] = same ? id0 : kSegNotUniform;
-    }
-    __syncthreads();
+  if (seg_k && t_end - seg_t0 <= kMaxSegTiles) {
     wq_id = __builtin_amdgcn_readfirstlane(seg_q);
     seg_fast = __builtin_amdgcn_ballot_w64(seg_q != wq_id) == 0 && wq_id != kSegNotUniform;
   }
@@ -300,7 +292,7 @@ void flash_fwd_kernel(const FwdArgs a) {
         }
       }
     }
-    if (seg_k && !(seg_fast && s_tile_id[t - t_begin] == wq_id)) {
+    if (seg_k && !(seg_fast && s_tile_id[t - seg_t0] == wq_id)) {
       const char* sg = seg_lds + (t % Tile::NSEG) * (Tile::BK * 4);
 #pragma unroll
       for (int ks = 0; ks < 2; ks++) {
