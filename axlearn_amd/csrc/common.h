@@ -260,13 +260,14 @@ __device__ __forceinline__ void shrink_to_segment_hull(int my_id, const int32_t*
 
 // One pass over the segment ids of the rows [lo, hi) that a workgroup loops over, in groups of GROUP
 // consecutive rows (GROUP a multiple of 4; ids 16-byte aligned; the row count a multiple of GROUP):
-//   * s_uniform[i], i < cap, gets the id of group lo / GROUP + i if its rows all carry one id, else
-//     `not_uniform` (groups from the one that holds row `lo` on; the return value is that group);
+//   * s_uniform[i], i < cap, gets the id of group g0 + i if its rows all carry one id, else
+//     `not_uniform`; g0, the return value, is the first group of the ALIGN-row block that holds row
+//     `lo` (ALIGN a multiple of GROUP: the caller's tile size, so that its first tile is covered);
 //   * [lo, hi) is shrunk, in whole groups, to the hull of the groups that hold an id between the
 //     smallest and the largest id of the workgroup's own rows (`my_id`, passed by every thread): only
 //     such a group can hold a row that matches one of them.
 // Called by all NT threads of the workgroup; contains barriers.
-template <int GROUP, int NT>
+template <int GROUP, int NT, int ALIGN = GROUP>
 __device__ __forceinline__ int classify_segment_groups(int my_id, const int32_t* ids, int tid, int& lo, int& hi,
                                                        int* s_uniform, int cap, int not_uniform) {
   __shared__ int s_rng[4];
@@ -281,7 +282,8 @@ __device__ __forceinline__ int classify_segment_groups(int my_id, const int32_t*
   atomicMax(&s_rng[1], my_id);
   __syncthreads();
   const int id_min = s_rng[0], id_max = s_rng[1];
-  const int g0 = lo / GROUP, g1 = (hi + GROUP - 1) / GROUP;
+  // whole ALIGN-row blocks at both ends, so that every group of the caller's first and last tile is described
+  const int g0 = (lo / ALIGN) * (ALIGN / GROUP), g1 = ((hi + ALIGN - 1) / ALIGN) * (ALIGN / GROUP);
   int first = 0x7fffffff, last = -1;
   for (int i = g0 + tid; i < g1; i += NT) {
     const intx4* p = (const intx4*)(ids + (int64_t)i * GROUP);

@@ -117,7 +117,14 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
     k_end = min(a.S, q0_wg + Tile::BQ + a.q_off);
     if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) k_begin = max(0, q0_wg + a.q_off - a.window);
   }
-  if (HAS_SEG) shrink_to_segment_hull(seg_q, a.seg + (int64_t)b * a.T, tid, k_begin, k_end);
+  // With segment ids: one pass over the ids of the key range shrinks it to the hull of the keys whose
+  // id lies between the smallest and the largest id of this workgroup's queries, and records for
+  // every 32-key sub-tile whether it carries a single id.
+  __shared__ int s_sub[HAS_SEG ? kMaxSub : 1];
+  int sub_g0 = 0;  // sub-tile that s_sub[0] describes
+  if (HAS_SEG)
+    sub_g0 = classify_segment_groups<32, 64 * NW, Tile::BK>(seg_q, a.seg + (int64_t)b * a.T, tid, k_begin, k_end,
+                                                           s_sub, kMaxSub, kNotUniform);
   const int t_begin = k_begin / Tile::BK;
   const int trips = max(0, (k_end + Tile::BK - 1) / Tile::BK - t_begin);
   const int key0 = t_begin * Tile::BK;   // first key of sub-tile 0
@@ -436,35 +443,22 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
     // Sub-tiles whose 32 keys all carry the segment id that all 32 queries of this wavefront carry
     // need no segment mask either: take the first run [tA, tB) of such sub-tiles (the masked loop is
     // always correct, so whatever lies outside that run simply stays on it).
-    __shared__ int s_sub[kMaxSub];
     const int nsub = 2 * trips;
+    const int sub0 = key0 / 32 - sub_g0;  // table index of sub-tile 0
     int tA = 0, tB = 0;
-    if (nsub <= kMaxSub) {
-      const int32_t* ids = a.seg + (int64_t)b * a.T + key0;
-      for (int i = tid; i < nsub; i += 64 * NW) {
-        const intx4* p = (const intx4*)(ids + 32 * i);
-        const int id0 = ids[32 * i];
-        bool same = true;
-#pragma unroll
-        for (int v = 0; v < 8; v++) {
-          const intx4 x = p[v];
-          same = same && x[0] == id0 && x[1] == id0 && x[2] == id0 && x[3] == id0;
-        }
-        s_sub[i] = same ? id0 : kNotUniform;
-      }
-      __syncthreads();
+    if (sub0 + nsub <= kMaxSub) {
       const int wq_id = __builtin_amdgcn_readfirstlane(seg_q);
       const bool q_uniform = __builtin_amdgcn_ballot_w64(seg_q != wq_id) == 0 && wq_id != kNotUniform;
       tA = tB = nsub;
       if (q_uniform) {
         for (int base = 0; base < nsub && tA == nsub; base += 64) {
           const int i = base + lane;
-          const uint64_t m = __builtin_amdgcn_ballot_w64(i < nsub && s_sub[i] == wq_id);
+          const uint64_t m = __builtin_amdgcn_ballot_w64(i < nsub && s_sub[sub0 + min(i, nsub - 1)] == wq_id);
           if (m) tA = base + __builtin_ctzll(m);
         }
         for (int base = tA & ~63; base < nsub && tB == nsub; base += 64) {
           const int i = base + lane;
-          const uint64_t m = __builtin_amdgcn_ballot_w64(i > tA && i < nsub && s_sub[i] != wq_id);
+          const uint64_t m = __builtin_amdgcn_ballot_w64(i > tA && i < nsub && s_sub[sub0 + min(i, nsub - 1)] != wq_id);
           if (m) tB = base + __builtin_ctzll(m);
         }
       }
