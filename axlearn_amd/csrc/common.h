@@ -198,6 +198,14 @@ __device__ __forceinline__ void dma16s_first8(unsigned voff, const void* sbase, 
       : "v"(voff), "s"(sbase), "s"(lds_base)
       : "memory", "m0");
 }
+// The same for lanes 0..15 (256 bytes).
+__device__ __forceinline__ void dma16s_first16(unsigned voff, const void* sbase, unsigned lds_base) {
+  asm volatile(
+      "s_mov_b64 exec, 0xffff\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1\n\ts_mov_b64 exec, -1"
+      :
+      : "v"(voff), "s"(sbase), "s"(lds_base)
+      : "memory", "m0");
+}
 #pragma clang diagnostic pop
 template <int N>
 __device__ __forceinline__ void wait_vmem_le() {

@@ -158,7 +158,9 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
   }
   const __bf16* k_src = (const __bf16*)a.k + b * a.ks.b + hk * a.ks.h + (int64_t)key0 * a.ks.s;
   const __bf16* v_src = (const __bf16*)a.v + b * a.vs.b + hk * a.vs.h + (int64_t)key0 * a.vs.s;
-  const int32_t* s_src = HAS_SEG ? a.seg + (int64_t)b * a.T + key0 + 4 * (lane & 15) : nullptr;
+  // segment ids of the tile's 64 keys: lanes 0..15 fetch 4 ids each, from a scalar base
+  const int32_t* s_src = HAS_SEG ? a.seg + (int64_t)b * a.T + key0 : nullptr;
+  const unsigned s_lane = 16 * (lane & 15);
   const int64_t k_step = (int64_t)Tile::BK * a.ks.s, v_step = (int64_t)Tile::BK * a.vs.s;
   // The k-th group of loads (pairs of K loads, pairs of V loads, then the segment ids) of the cursor's
   // tile into the buffer at LDS address BUF_.
@@ -176,8 +178,9 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
       const unsigned dst_ = (BUF_) + Tile::TILE_BYTES + wave * (ROWS_PER_WAVE * Tile::ROWB) + per_ * kv_ * 1024; \
       if constexpr (PAIRS) dma16x2(v_lane[(2 * kv_) % Tile::DMA_PER_WAVE], v_lane[(2 * kv_ + 1) % Tile::DMA_PER_WAVE], v_src, dst_); \
       else dma16s(v_lane[kv_ % Tile::DMA_PER_WAVE], v_src, dst_);                                 \
-    } else if (lane < 16) {                                                                       \
-      dma16(s_src, (BUF_) + Tile::SEG_BASE);                                                      \
+    } else {                                                                                      \
+      /* no branch: the trip stays one scheduling region (all lanes are active here) */            \
+      dma16s_first16(s_lane, s_src, (BUF_) + Tile::SEG_BASE);                                     \
     }                                                                                             \
   }
 #define AXL_DMA_TILE(BUF_)                                                                         \
