@@ -275,6 +275,7 @@ void flash_fwd_kernel(const FwdArgs a) {
       }
     };
     bool need_mask = false;
+    const unsigned mask_limit = a.mask_kind == AXL_MASK_SLIDING_WINDOW ? (unsigned)a.window : 0x7fffffffu;
     if (a.mask_kind != AXL_MASK_NONE) {
       need_mask = k0 + Tile::BK - 1 > qpos_min;
       if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) need_mask = need_mask || (qpos_max - k0 > a.window);
@@ -285,10 +286,9 @@ void flash_fwd_kernel(const FwdArgs a) {
         const int diff0 = qpos - (k0 + 32 * ks + 8 * g);  // qpos - kpos for r == 0
 #pragma unroll
         for (int r = 0; r < 16; r++) {
-          const int diff = diff0 - (16 * (r / 8) + (r % 8));
-          bool keep = diff >= 0;
-          if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) keep = keep && diff <= a.window;
-          s[ks][r] = keep ? s[ks][r] : kMasked;
+          // keep(q, k)  <=>  0 <= qpos - kpos <= window: one unsigned comparison, one select
+          const unsigned diff = (unsigned)(diff0 - (16 * (r / 8) + (r % 8)));
+          s[ks][r] = diff <= mask_limit ? s[ks][r] : kMasked;
         }
       }
     }
