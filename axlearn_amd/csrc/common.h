@@ -319,18 +319,27 @@ __device__ __forceinline__ int classify_segment_groups(int my_id, const int32_t*
   return g0;
 }
 
-// Decodes blockIdx.x into (query block, batch, query head).  Heaviest query blocks (most visible
-// keys under a causal mask) are issued first; when the (batch, kv head) pairs divide evenly over
-// the 8 XCDs, all workgroups of a pair run on one XCD (workgroup i is dispatched to XCD i % 8).
-__device__ __forceinline__ void decode_block(int bid, int nqb, int B, int Hq, int Hkv, int& qb,
+// Decodes blockIdx.x into (query block, batch, query head).  Workgroup i is dispatched to XCD i % 8.
+// When the (batch, kv head) pairs divide evenly over the 8 XCDs, an XCD works through its pairs a
+// group at a time: as few pairs as fill its `slots` resident workgroups (one pair when a pair has
+// that many query blocks x query heads), heaviest query blocks (most visible keys under a causal
+// mask) first across the group.  The workgroups that run together then read the K/V of one or two
+// kv heads, which that XCD's L2 holds, and a group still has enough workgroups to keep every CU busy.
+__device__ __forceinline__ void decode_block(int bid, int nqb, int B, int Hq, int Hkv, int slots, int& qb,
                                              int& b, int& h) {
   const int G = Hq / Hkv;
   const int npairs = B * Hkv;
   if (npairs % 8 == 0) {
     const int xcd = bid & 7, slot = bid >> 3;
+    const int ppx = npairs >> 3;                       // pairs per XCD
     const int per_pair = nqb * G;
-    const int pair = xcd + 8 * (slot / per_pair), rem = slot % per_pair;
-    qb = nqb - 1 - rem / G;
+    const int pgn = max(1, (slots + per_pair - 1) / per_pair);  // pairs per group
+    const int grp = slot / (pgn * per_pair);
+    const int r = slot - grp * (pgn * per_pair);
+    const int pg = min(pgn, ppx - grp * pgn);          // the last group may be smaller
+    const int rem = r % (pg * G);
+    const int pair = xcd + 8 * (grp * pgn + rem / G);
+    qb = nqb - 1 - r / (pg * G);
     b = pair / Hkv;
     h = (pair % Hkv) * G + rem % G;
   } else {

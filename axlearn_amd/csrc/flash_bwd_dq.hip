@@ -60,7 +60,7 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l32 = lane & 31, g = lane >> 5;
   int qb, b, h;
-  decode_block(blockIdx.x, (a.T + Tile::BQ - 1) / Tile::BQ, a.B, a.Hq, a.Hkv, qb, b, h);
+  decode_block(blockIdx.x, (a.T + Tile::BQ - 1) / Tile::BQ, a.B, a.Hq, a.Hkv, 32, qb, b, h);
   const int hk = h / (a.Hq / a.Hkv);
   const int q0_wg = qb * Tile::BQ;
   // This wavefront's queries.  T is a multiple of 128 but not necessarily of BQ: a wavefront past the

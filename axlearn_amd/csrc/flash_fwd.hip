@@ -73,7 +73,7 @@ void flash_fwd_kernel(const FwdArgs a) {
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l32 = lane & 31, g = lane >> 5;
   int qb, b, h;
-  decode_block(blockIdx.x, a.T / Tile::BQ, a.B, a.Hq, a.Hkv, qb, b, h);
+  decode_block(blockIdx.x, a.T / Tile::BQ, a.B, a.Hq, a.Hkv, 64, qb, b, h);
   const int hk = h / (a.Hq / a.Hkv);
   const int q_off = a.q_off + (a.q_offs ? a.q_offs[b] : 0);  // position of this sequence's query row 0
   const int q0_wg = qb * Tile::BQ;
@@ -467,7 +467,8 @@ __global__ __launch_bounds__(256) void flash_fwd_f32_kernel(const FwdArgs a) {
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
   int qb, b, h;
-  decode_block(blockIdx.x, a.T / Tile::BQ, a.B, a.Hq, a.Hkv, qb, b, h);
+  // all pairs of an XCD in one group: query blocks in the globally longest-first order
+  decode_block(blockIdx.x, a.T / Tile::BQ, a.B, a.Hq, a.Hkv, 1 << 20, qb, b, h);
   const int hk = h / (a.Hq / a.Hkv);
   const int q_off = a.q_off + (a.q_offs ? a.q_offs[b] : 0);  // position of this sequence's query row 0
   const int q0_wg = qb * Tile::BQ;
