@@ -258,6 +258,39 @@ def test_random_shapes_forward_and_backward(seed):
     _assert_close("dv " + case, dv, wv, dtype)
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_random_shapes_with_pairs_spread_over_xcds(seed):
+    """Shapes whose (batch x kv head) pairs are a multiple of 8, which the kernels work through in
+    per-XCD groups (including a last group smaller than the others): out, dq, dk, dv against the
+    oracle, bf16 and fp16, every mask kind, with and without packing."""
+    rng = np.random.default_rng(5000 + seed)
+    d = int(rng.choice([64, 128]))
+    b, hkv = [(1, 8), (2, 4), (3, 8), (8, 1), (2, 8), (5, 8)][int(rng.integers(0, 6))]
+    hq = hkv * int(rng.choice([1, 2, 4]))
+    t = 128 * int(rng.integers(1, 10))
+    kind = str(rng.choice(["none", "causal", "sliding"]))
+    packed = bool(rng.integers(0, 2))
+    dtype = [torch.bfloat16, torch.float16][int(rng.integers(0, 2))]
+    window = int(rng.integers(0, t)) if kind == "sliding" else None
+    q, k, v, do = _inputs(b, t, hq, hkv, d, dtype, s=t)
+    segs = ref.packed_segment_ids(seed, b, t, max_docs=4) if packed else None
+    spec = ref.MaskSpec(causal=kind == "causal", sliding_window=window, segment_ids=segs,
+                        target_positions=torch.arange(t)[None], source_positions=torch.arange(t)[None])
+    mk = {"none": ops.MASK_NONE, "causal": ops.MASK_CAUSAL, "sliding": ops.MASK_SLIDING_WINDOW}[kind]
+    kw = dict(mask_kind=mk, sliding_window=window or 0, q_pos_offset=0, softmax_scale=d ** -0.5,
+              segment_ids=None if segs is None else segs.cuda())
+    case = f"b={b} d={d} hq={hq} hkv={hkv} t={t} {kind} window={window} packed={packed} {dtype}"
+    want = ref.reference_mha(q, k, v, spec, softmax_scale=d ** -0.5)
+    wq, wk, wv = ref.reference_mha_grads(q, k, v, do, spec, softmax_scale=d ** -0.5)
+    qc, kc, vc, doc = q.cuda(), k.cuda(), v.cuda(), do.cuda()
+    out, lse = ops.flash_fwd(qc, kc, vc, **kw)
+    _assert_close("out " + case, out, want, dtype)
+    dq, dk, dv = ops.flash_bwd(qc, kc, vc, out, lse, doc, **kw)
+    _assert_close("dq " + case, dq, wq, dtype)
+    _assert_close("dk " + case, dk, wk, dtype)
+    _assert_close("dv " + case, dv, wv, dtype)
+
+
 @pytest.mark.parametrize("mask,window", [("none", None), ("causal", None), ("sliding", 200)])
 def test_arbitrary_segment_ids_forward_and_backward(mask, window):
     """Segment ids are compared for equality only (attention_bias.py:876-882): ids need not be sorted,
