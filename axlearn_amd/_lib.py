@@ -17,10 +17,11 @@ LIB_PATH = os.path.join(_HERE, "libaxl_attn_hip.so")
 
 AXL_BF16, AXL_F32, AXL_F16 = 0, 1, 2
 MASK_NONE, MASK_CAUSAL, MASK_SLIDING_WINDOW = 0, 1, 2
+DECODE_DETERMINISTIC, DECODE_WORKSPACE_REUSED = 1, 2  # AXL_DECODE_* flags
 AXL_OK, AXL_ERR_INVALID_ARGUMENT, AXL_ERR_UNSUPPORTED, AXL_ERR_WORKSPACE, AXL_ERR_LAUNCH = 0, -1, -2, -3, -4
 
 
-ABI_VERSION = 4  # AXL_ATTN_ABI_VERSION of include/axl_attn.h these structures mirror
+ABI_VERSION = 5  # AXL_ATTN_ABI_VERSION of include/axl_attn.h these structures mirror
 
 
 class AxlError(RuntimeError):
@@ -97,6 +98,7 @@ class AxlPagedDecodeParams(ctypes.Structure):
         ("dtype", ctypes.c_int32), ("sliding_window", ctypes.c_int32),
         ("softmax_scale", ctypes.c_float),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
+        ("flags", ctypes.c_int32),
     ]
 
 
@@ -110,6 +112,7 @@ class AxlDecodeParams(ctypes.Structure):
         ("dtype", ctypes.c_int32), ("sliding_window", ctypes.c_int32),
         ("softmax_scale", ctypes.c_float),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
+        ("flags", ctypes.c_int32),
     ]
 
 

@@ -3,6 +3,8 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cmath>
+#include <mutex>
+#include <unordered_map>
 
 #include "common.h"
 
@@ -26,6 +28,29 @@ size_t paged_decode_workspace_bytes(const AxlPagedDecodeParams& p);
 int launch_decode(const AxlDecodeParams& p, hipStream_t stream);
 size_t decode_workspace_bytes(const AxlDecodeParams& p);
 int launch_page_insert(const AxlPageInsertParams& p, hipStream_t stream);
+
+hipError_t allow_dynamic_lds(const void* kernel, int bytes) {
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return err;
+  const uint64_t key = (uint64_t)reinterpret_cast<uintptr_t>(kernel) ^ ((uint64_t)(dev + 1) << 56);
+  // The pair this thread set (or found set) last: repeated launches of one kernel take no lock.
+  static thread_local uint64_t last_key = 0;
+  static thread_local int last_bytes = 0;
+  if (last_key == key && last_bytes >= bytes) return hipSuccess;
+  static std::mutex mu;
+  static std::unordered_map<uint64_t, int> granted;  // (kernel, device) -> limit already set
+  std::lock_guard<std::mutex> lock(mu);
+  auto it = granted.find(key);
+  if (it == granted.end() || it->second < bytes) {
+    err = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (err != hipSuccess) return err;
+    granted[key] = bytes;
+  }
+  last_key = key;
+  last_bytes = bytes;
+  return hipSuccess;
+}
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 

@@ -409,4 +409,8 @@ __device__ __forceinline__ void load_bias(const char* row, int col, int is_f32, 
 
 int set_error(int code, const char* fmt, ...);
 
+// Raises a kernel's dynamic LDS limit to `bytes` (hipFuncAttributeMaxDynamicSharedMemorySize) the
+// first time the kernel is launched on the current device; later launches only look the pair up.
+hipError_t allow_dynamic_lds(const void* kernel, int bytes);
+
 }  // namespace axl

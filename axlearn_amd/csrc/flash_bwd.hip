@@ -347,8 +347,7 @@ int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream)
 #define AXL_LAUNCH(KERNEL, GRID, LDS)                                                           \
   do {                                                                                          \
     if (err == hipSuccess && (LDS) > 0)                                                         \
-      err = hipFuncSetAttribute((const void*)KERNEL, hipFuncAttributeMaxDynamicSharedMemorySize, \
-                                (LDS));                                                         \
+      err = allow_dynamic_lds((const void*)KERNEL, (LDS));                                      \
     if (err == hipSuccess) {                                                                    \
       hipLaunchKernelGGL(KERNEL, dim3(GRID), dim3(256), (LDS), stream, a);                      \
       err = hipGetLastError();                                                                  \

@@ -669,8 +669,7 @@ template <typename E, int D, bool HAS_SEG, bool AUX>
 static hipError_t launch_one(const BwdArgs& a, hipStream_t stream) {
   using Tile = DkvTile<D>;
   auto kernel = flash_bwd_dkdv_kernel<E, D, HAS_SEG, AUX>;
-  hipError_t err = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       Tile::LDS_BYTES);
+  hipError_t err = allow_dynamic_lds((const void*)kernel, Tile::LDS_BYTES);
   if (err != hipSuccess) return err;
   const int grid = (a.S / Tile::BKV) * a.B * a.Hkv;
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), Tile::LDS_BYTES, stream, a);

@@ -520,8 +520,7 @@ static hipError_t launch_one(const BwdArgs& a, hipStream_t stream) {
   constexpr int NW = AXL_DQ_WAVES;
   using Tile = DqRing<D, HAS_SEG, NW>;
   auto kernel = flash_bwd_dq_ring_kernel<E, D, HAS_SEG, NW, FUSE_DELTA>;
-  hipError_t err = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       Tile::LDS_BYTES);
+  hipError_t err = allow_dynamic_lds((const void*)kernel, Tile::LDS_BYTES);
   if (err != hipSuccess) return err;
   const int grid = ((a.T + Tile::BQ - 1) / Tile::BQ) * a.B * a.Hq;
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(64 * NW), Tile::LDS_BYTES, stream, a);

@@ -301,7 +301,7 @@ static hipError_t launch_f32(const BwdArgs& a, int phases, hipStream_t stream) {
   hipError_t err = hipSuccess;
   if (phases & AXL_BWD_DKDV) {
     auto kernel = flash_bwd_dkdv_f32_kernel<D>;
-    err = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, Tile::LDS_BYTES);
+    err = allow_dynamic_lds((const void*)kernel, Tile::LDS_BYTES);
     if (err != hipSuccess) return err;
     hipLaunchKernelGGL(kernel, dim3((a.S / Tile::ROWS) * a.B * a.Hkv), dim3(128), Tile::LDS_BYTES, stream, a);
     err = hipGetLastError();
@@ -309,7 +309,7 @@ static hipError_t launch_f32(const BwdArgs& a, int phases, hipStream_t stream) {
   }
   if (phases & AXL_BWD_DQ) {
     auto kernel = flash_bwd_dq_f32_kernel<D>;
-    err = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, Tile::LDS_BYTES);
+    err = allow_dynamic_lds((const void*)kernel, Tile::LDS_BYTES);
     if (err != hipSuccess) return err;
     hipLaunchKernelGGL(kernel, dim3((a.T / Tile::ROWS) * a.B * a.Hq), dim3(128), Tile::LDS_BYTES, stream, a);
     err = hipGetLastError();

@@ -632,8 +632,7 @@ int launch_flash_fwd(const AxlFlashFwdParams& p, hipStream_t stream) {
   hipError_t err = hipSuccess;
 #define AXL_LAUNCH_FWD(KERNEL, TILE)                                                            \
   do {                                                                                          \
-    err = hipFuncSetAttribute((const void*)KERNEL, hipFuncAttributeMaxDynamicSharedMemorySize,  \
-                              TILE::LDS_BYTES);                                                 \
+    err = allow_dynamic_lds((const void*)KERNEL, TILE::LDS_BYTES);                              \
     if (err == hipSuccess) {                                                                    \
       hipLaunchKernelGGL(KERNEL, dim3(grid), dim3(256), TILE::LDS_BYTES, stream, a);            \
       err = hipGetLastError();                                                                  \

@@ -23,9 +23,10 @@
 //     workspace (the reference stores partial o in the query dtype, gpu_paged_attention.py:272)
 //     and a second small kernel merges the records of a (sequence, kv head) in context order.
 // Work is handed out by timing, so the grouping of the fp32 partial sums - not the set of keys -
-// can differ between two calls; AXL_DECODE_DETERMINISTIC=1 in the environment selects a fixed
-// decomposition (one block per record, pages dealt round-robin) whose result is reproducible bit
-// for bit.
+// can differ between two calls; the AXL_DECODE_DETERMINISTIC flag of the call (or
+// AXL_DECODE_DETERMINISTIC=1 in the environment, read once, as the default for every call) selects
+// a fixed decomposition (one block per record, pages dealt round-robin) whose result is
+// reproducible bit for bit.
 // Keys at index >= length are masked (gpu_paged_attention.py:100, gpu_decoding.py:109); the query
 // position is length-1, so a sliding window w also masks keys with (length-1) - j > w.  A page
 // index outside the pool reads as zeros and a negative one counts from the end of the pool, as the
@@ -44,7 +45,8 @@ struct DecArgs {
   float* ws_o;                 // [records, GP, D]; at most B * Hkv * NCH records
   float* ws_m;                 // [records, GP]
   float* ws_l;                 // [records, GP]
-  int32_t* ws_tab;             // [B, Hkv, NCH]: record that starts at this chunk, or -1
+  int32_t* ws_tab;             // [B, Hkv, NCH]: record that starts at this live chunk, or -1; every live
+                               // chunk's entry is written by the workgroup that streams the chunk
   Strides3 ks, vs;             // contiguous only
   int B, Hq, Hkv, G;
   int num_pages, pps;          // pool pages; logical pages per sequence (ceil(S/16) if contiguous)
@@ -52,7 +54,8 @@ struct DecArgs {
   int chunk_pages, nch;
   int window;
   float scale;
-  int* ticket;                 // [0] blocks handed out, [1] records written (zeroed by decode_plan_kernel)
+  int* ticket;                 // [0] blocks handed out: zero when the split kernel starts (zeroed by
+                               // decode_plan_kernel, or left at zero by the previous call's combine kernel)
   int deterministic;           // fixed work decomposition: results reproducible bit for bit
 };
 
@@ -83,6 +86,12 @@ __device__ __forceinline__ void live_chunks(const DecArgs& a, int len, int& ch0,
   const int first_page = a.window >= 0 ? max(0, len - 1 - a.window) / kPage : 0;
   ch0 = first_page / a.chunk_pages;
   ch1 = max(ch0, (npages + a.chunk_pages - 1) / a.chunk_pages);
+}
+
+// Lengths outside [0, capacity] are clamped: a sequence cannot hold more keys than its page table
+// (or its cache rows) can address, and a non-positive length is an empty context.
+__device__ __forceinline__ int clamp_length(const DecArgs& a, int len) {
+  return max(0, min(len, a.kv_len));
 }
 
 template <int D, int GP, int NST>
@@ -135,8 +144,7 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
       const int bi = tid * PER + i;
       int n = 0;
       if (bi < a.B) {
-        int l = a.lengths[bi];
-        if (!PAGED) l = min(l, a.kv_len);
+        const int l = clamp_length(a, a.lengths[bi]);
         lens[bi] = l;
         int c0, c1;
         live_chunks(a, l, c0, c1);
@@ -208,15 +216,13 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
   // the 4 wavefronts finish together however unevenly the memory system serves them.
   const int n_pg = c_end - c_begin;
 
-  // Draw the next run and this segment's record slot; the round trips overlap the loads of Q and
-  // of the page ids below.
-  int rec = 0;
-  if (tid == 0) {
-    if (first_segment) {
-      next_n = min(max_run, max(1, (n_blocks - handed) / (4 * n_wg)));
-      next_e = atomicAdd(&a.ticket[0], next_n);
-    }
-    rec = atomicAdd(&a.ticket[1], 1);
+  // Draw the next run; the round trip overlaps the loads of Q and of the page ids below.  The
+  // segment's record slot is the number of its first block: unique, and below the B * Hkv * NCH
+  // records the workspace holds.
+  const int rec = run_e;
+  if (tid == 0 && first_segment) {
+    next_n = min(max_run, max(1, (n_blocks - handed) / (4 * n_wg)));
+    next_e = atomicAdd(&a.ticket[0], next_n);
   }
   first_segment = false;
 
@@ -423,7 +429,6 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
     red_m[wave][head] = m_run;
     red_l[wave][head] = l_run;
   }
-  if (tid == 0) s_next[2] = rec;
   __syncthreads();  // also: every wavefront is done with its ring, which red_o aliases
   {
     const float mw = fmaxf(fmaxf(red_m[0][head], red_m[1][head]), fmaxf(red_m[2][head], red_m[3][head]));
@@ -436,7 +441,7 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
     }
   }
   __syncthreads();
-  const int64_t slot = s_next[2];
+  const int64_t slot = rec;
   float* out_ws = a.ws_o + slot * (GP * D);
   for (int idx = tid; idx < GP * D; idx += 256) {
     const int gq = idx / D, d = idx % D;
@@ -449,8 +454,9 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
     for (int w = 0; w < 4; w++) lw += red_l[w][tid] * fast_exp2((red_m[w][tid] - mw) * c);
     a.ws_m[slot * GP + tid] = mw;
     a.ws_l[slot * GP + tid] = lw;
-    if (tid == 0) a.ws_tab[((int64_t)b * a.Hkv + hk) * a.nch + cl] = (int)slot;
   }
+  // Table entries of the segment's chunks: the record at its first chunk, "none" at the others.
+  for (int i = tid; i < seg; i += 256) a.ws_tab[((int64_t)b * a.Hkv + hk) * a.nch + cl + i] = i == 0 ? (int)slot : -1;
   if (tid == 0) *s_page = 4 * NST;
   __syncthreads();  // the ring (and red_m/red_l) are reused by the next segment
   run_e += seg;
@@ -464,12 +470,11 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
   }  // runs
 }
 
-// Resets the work counters and the record table ahead of the split kernel (a kernel rather than
-// memsets so that the sequence can be captured into a graph).
-__global__ __launch_bounds__(256) void decode_plan_kernel(int* ticket, int32_t* tab, int n_tab) {
-  const int i = blockIdx.x * 256 + threadIdx.x;
-  if (i < 2) ticket[i] = 0;
-  if (i < n_tab) tab[i] = -1;
+// Zeroes the work counter ahead of the split kernel when the workspace comes with unknown contents
+// (a kernel rather than a memset so that the sequence can be captured into a graph).  A workspace
+// that the caller declares reused skips it: the combine kernel leaves the counter at zero.
+__global__ __launch_bounds__(64) void decode_plan_kernel(int* ticket) {
+  if (threadIdx.x == 0) ticket[0] = 0;
 }
 
 // Merges the per-chunk partials of one (sequence, kv head): the "final round of flash"
@@ -487,11 +492,12 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecArgs a) {
   __shared__ float4 s_part[256];          // partial sums of the record slices
   const int hk = blockIdx.x, b = blockIdx.y;
   const int tid = threadIdx.x;
-  int len = a.lengths[b];
-  if (a.page_tables == nullptr) len = min(len, a.kv_len);
+  const int len = clamp_length(a, a.lengths[b]);
   int ch0, ch1;
   live_chunks(a, len, ch0, ch1);
   const int nc = ch1 - ch0;               // live chunks = upper bound on records of this (b, hk)
+  // The split kernel has finished: leave the work counter at zero for the next call on this workspace.
+  if (hk == 0 && b == 0 && tid == 0) a.ticket[0] = 0;
   const float c = a.scale * kLog2e;
   // The whole table row in one round trip, then compacted in chunk order by one wavefront.
   s_raw[tid] = tid < nc ? a.ws_tab[((int64_t)b * a.Hkv + hk) * a.nch + tid] : -1;
@@ -526,7 +532,9 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecArgs a) {
   if (tid < GP) {
     float l = 0.f;
     for (int i = tid; i < n; i += GP) l += sl[i] * sm[i];
-    s_inv[tid] = 1.f / l;
+    // An empty context (length 0, or no key inside the window) has no record: the output is zeros,
+    // as with the reference's o / (l + eps) (gpu_decoding.py:282, gpu_paged_attention.py:291-293).
+    s_inv[tid] = l > 0.f ? 1.f / l : 0.f;
   }
   __syncthreads();
   // Output: G*D floats = n4 groups of four.  With fewer groups than threads the records are dealt
@@ -586,8 +594,7 @@ __global__ __launch_bounds__(256) void decode_split_f32_kernel(const DecArgs a) 
   __shared__ float red_m[4][GP], red_l[4][GP];
   const int c = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, sub = lane >> 4, l16 = lane & 15;
-  int len = a.lengths[b];
-  if (!PAGED) len = min(len, a.kv_len);
+  const int len = clamp_length(a, a.lengths[b]);
   int ch0, ch1;
   live_chunks(a, len, ch0, ch1);
   if (ch0 + c >= ch1) return;
@@ -706,8 +713,10 @@ static int pick_chunk_pages(int pps) {
   return cp < 4 ? 4 : cp;
 }
 
+constexpr int kWsHeaderFloats = 64;  // 256 bytes ahead of the records: the work counter
+
 static size_t ws_bytes(int B, int Hkv, int nch, int gp, int D) {
-  return (size_t)B * Hkv * nch * ((size_t)gp * D + 2 * gp + 1) * sizeof(float) + 256;  // + headers, counters
+  return (size_t)B * Hkv * nch * ((size_t)gp * D + 2 * gp + 1) * sizeof(float) + kWsHeaderFloats * sizeof(float);
 }
 
 static int gp_of(int G) { return G <= 4 ? 4 : (G <= 8 ? 8 : 16); }
@@ -740,43 +749,51 @@ static int cu_count() {
   return n;
 }
 
+// AXL_DECODE_DETERMINISTIC in the environment, read once: the default for calls that do not set the flag.
+static bool deterministic_by_default() {
+  static const bool v = [] {
+    const char* det = getenv("AXL_DECODE_DETERMINISTIC");
+    return det && det[0] != '\0' && det[0] != '0';
+  }();
+  return v;
+}
+
 template <typename E, bool PAGED>
-static int launch_common(DecArgs a, int D, hipStream_t stream, const char* who) {
+static int launch_common(DecArgs a, int D, int flags, hipStream_t stream, const char* who) {
   const int gp = gp_of(a.G);
   if (a.G > 16) return set_error(AXL_ERR_UNSUPPORTED, "%s: more than 16 query heads per kv head", who);
   a.chunk_pages = pick_chunk_pages(a.pps);
   if (a.chunk_pages > 256)
     return set_error(AXL_ERR_UNSUPPORTED, "%s: context longer than %d tokens", who, 256 * kMaxChunks * kPage);
   a.nch = (a.pps + a.chunk_pages - 1) / a.chunk_pages;
+  // Workspace: a 256-byte header (the work counter, at the same place whatever the shapes), then the
+  // records, their statistics and the record table.
+  a.ticket = (int*)a.ws_o;
+  a.ws_o += kWsHeaderFloats;
   float* ws = a.ws_o;
   const size_t n_o = (size_t)a.B * a.Hkv * a.nch * gp * D;
   const size_t n_s = (size_t)a.B * a.Hkv * a.nch * gp;
   a.ws_m = ws + n_o;
   a.ws_l = ws + n_o + n_s;
-  const size_t n_r = (size_t)a.B * a.Hkv * a.nch;
   a.ws_tab = (int32_t*)(ws + n_o + 2 * n_s);
-  {
-    const char* det = getenv("AXL_DECODE_DETERMINISTIC");
-    a.deterministic = det && det[0] != '\0' && det[0] != '0';
-  }
-  a.ticket = (int*)(ws + n_o + 2 * n_s + n_r);
+  a.deterministic = (flags & AXL_DECODE_DETERMINISTIC) != 0 || deterministic_by_default();
   // Two workgroups fit a CU (LDS); the split kernel is persistent and strides over its work items.
   const dim3 grid(2 * cu_count());
   hipError_t err = hipSuccess;
+  if (!(flags & AXL_DECODE_WORKSPACE_REUSED))
+    hipLaunchKernelGGL(decode_plan_kernel, dim3(1), dim3(64), 0, stream, a.ticket);
 #define AXL_DEC(E, DD, GG, NS)                                                                  \
   do {                                                                                          \
     using Tile = DecTile<DD, GG, NS>;                                                           \
     auto kern = decode_split_kernel<E, DD, GG, PAGED, NS>;                                      \
-    err = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,    \
-                              Tile::LDS_BYTES);                                                 \
+    err = allow_dynamic_lds((const void*)kern, Tile::LDS_BYTES);                                \
     if (err == hipSuccess) {                                                                    \
-      hipLaunchKernelGGL(decode_plan_kernel, dim3((n_tab + 255) / 256), dim3(256), 0, stream,   \
-                         s.ticket, s.ws_tab, n_tab);                                            \
       hipLaunchKernelGGL(kern, grid, dim3(256), Tile::LDS_BYTES, stream, s);                    \
       hipLaunchKernelGGL((decode_combine_kernel<E, DD, GG>), cgrid, dim3(256), 0, stream, s);   \
     }                                                                                           \
   } while (0)
-  // The kernels keep per-sequence tables in LDS: larger batches go in slices of kMaxBatch.
+  // The kernels keep per-sequence tables in LDS: larger batches go in slices of kMaxBatch (each
+  // slice's combine kernel leaves the shared work counter at zero for the next slice).
   for (int b0 = 0; b0 < a.B && err == hipSuccess; b0 += kMaxBatch) {
     DecArgs s = a;
     s.B = a.B - b0 < kMaxBatch ? a.B - b0 : kMaxBatch;
@@ -789,7 +806,6 @@ static int launch_common(DecArgs a, int D, hipStream_t stream, const char* who) 
     s.ws_m = a.ws_m + (size_t)b0 * a.Hkv * a.nch * gp;
     s.ws_l = a.ws_l + (size_t)b0 * a.Hkv * a.nch * gp;
     s.ws_tab = a.ws_tab + (size_t)b0 * a.Hkv * a.nch;
-    const int n_tab = s.B * a.Hkv * a.nch;
     const dim3 cgrid(a.Hkv, s.B);
     if (D == 128 && gp == 4) AXL_DEC(E, 128, 4, kStages128);
     else if (D == 128 && gp == 8) AXL_DEC(E, 128, 8, kStages128);
@@ -813,18 +829,18 @@ static int launch_f32(DecArgs a, int D, hipStream_t stream, const char* who) {
     return set_error(AXL_ERR_UNSUPPORTED, "%s: context longer than %d tokens", who, 256 * kMaxChunks * kPage);
   if (a.B > 65535) return set_error(AXL_ERR_UNSUPPORTED, "%s: more than 65535 sequences in fp32", who);
   a.nch = (a.pps + a.chunk_pages - 1) / a.chunk_pages;
+  a.ticket = (int*)a.ws_o;
+  a.ws_o += kWsHeaderFloats;
   float* ws = a.ws_o;
   const size_t n_o = (size_t)a.B * a.Hkv * a.nch * gp * D;
   const size_t n_s = (size_t)a.B * a.Hkv * a.nch * gp;
-  const size_t n_r = (size_t)a.B * a.Hkv * a.nch;
   a.ws_m = ws + n_o;
   a.ws_l = ws + n_o + n_s;
   a.ws_tab = (int32_t*)(ws + n_o + 2 * n_s);
-  a.ticket = (int*)(ws + n_o + 2 * n_s + n_r);
   a.deterministic = 1;
-  const int n_tab = (int)n_r;
+  // One workgroup per live chunk writes that chunk's table entry; the work counter is not used (the
+  // combine kernel still leaves it at zero).
   const dim3 grid(a.nch, a.Hkv, a.B), cgrid(a.Hkv, a.B);
-  hipLaunchKernelGGL(decode_plan_kernel, dim3((n_tab + 255) / 256), dim3(256), 0, stream, a.ticket, a.ws_tab, n_tab);
 #define AXL_DEC32(DD, GG)                                                                          \
   do {                                                                                              \
     hipLaunchKernelGGL((decode_split_f32_kernel<DD, GG, PAGED>), grid, dim3(256), 0, stream, a);    \
@@ -852,8 +868,8 @@ int launch_paged_decode(const AxlPagedDecodeParams& p, hipStream_t stream) {
   a.window = p.sliding_window < 0 ? -1 : p.sliding_window;
   a.scale = p.softmax_scale;
   if (p.dtype == AXL_F32) return launch_f32<true>(a, p.head_dim, stream, "axl_paged_decode");
-  return p.dtype == AXL_F16 ? launch_common<ElemF16, true>(a, p.head_dim, stream, "axl_paged_decode")
-                            : launch_common<ElemBf16, true>(a, p.head_dim, stream, "axl_paged_decode");
+  return p.dtype == AXL_F16 ? launch_common<ElemF16, true>(a, p.head_dim, p.flags, stream, "axl_paged_decode")
+                            : launch_common<ElemBf16, true>(a, p.head_dim, p.flags, stream, "axl_paged_decode");
 }
 
 int launch_decode(const AxlDecodeParams& p, hipStream_t stream) {
@@ -868,8 +884,8 @@ int launch_decode(const AxlDecodeParams& p, hipStream_t stream) {
   a.window = p.sliding_window < 0 ? -1 : p.sliding_window;
   a.scale = p.softmax_scale;
   if (p.dtype == AXL_F32) return launch_f32<false>(a, p.head_dim, stream, "axl_decode");
-  return p.dtype == AXL_F16 ? launch_common<ElemF16, false>(a, p.head_dim, stream, "axl_decode")
-                            : launch_common<ElemBf16, false>(a, p.head_dim, stream, "axl_decode");
+  return p.dtype == AXL_F16 ? launch_common<ElemF16, false>(a, p.head_dim, p.flags, stream, "axl_decode")
+                            : launch_common<ElemBf16, false>(a, p.head_dim, p.flags, stream, "axl_decode");
 }
 
 }  // namespace axl

@@ -37,9 +37,50 @@ __all__ = [
 
 
 def _require_cuda(*tensors):
+    dev = None
     for t in tensors:
-        if t is not None and not t.is_cuda:
+        if t is None:
+            continue
+        if not t.is_cuda:
             raise AxlError(_lib.AXL_ERR_INVALID_ARGUMENT, "all tensors must live on the GPU")
+        if dev is not None and t.device != dev:
+            raise AxlError(_lib.AXL_ERR_INVALID_ARGUMENT, f"tensors live on different devices ({dev} and {t.device})")
+        dev = t.device
+
+
+def _bad(msg: str) -> AxlError:
+    return AxlError(_lib.AXL_ERR_INVALID_ARGUMENT, msg)
+
+
+def _want_shape(name: str, t: torch.Tensor, shape) -> None:
+    if tuple(t.shape) != tuple(shape):
+        raise _bad(f"{name} must have shape {list(shape)}, got {list(t.shape)}")
+
+
+def _check_qkv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor):
+    """The kernels take every extent from these shapes and read raw pointers: anything that does not
+    fit together is rejected here, before a parameter block is built."""
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        raise _bad(f"q, k, v must be 4-d [batch, seq, heads, head_dim], got {list(q.shape)}, {list(k.shape)}, {list(v.shape)}")
+    b, t, hq, d = q.shape
+    if k.shape[0] != b or k.shape[3] != d:
+        raise _bad(f"k {list(k.shape)} does not match q {list(q.shape)} in batch / head_dim")
+    if tuple(v.shape) != tuple(k.shape):
+        raise _bad(f"v {list(v.shape)} must have the shape of k {list(k.shape)}")
+    hkv = k.shape[2]
+    if hkv <= 0 or hq % hkv != 0:
+        raise _bad(f"num_q_heads {hq} is not divisible by num_kv_heads {hkv}")
+    if k.dtype != q.dtype or v.dtype != q.dtype:
+        raise AxlError(_lib.AXL_ERR_UNSUPPORTED, "q, k, v must share one dtype")
+    return b, t, hq, d, k.shape[1], hkv
+
+
+def _check_segment_ids(segment_ids: Optional[torch.Tensor], b: int, t: int, s: int) -> None:
+    if segment_ids is None:
+        return
+    if t != s:
+        raise _bad(f"segment_ids need q_len == kv_len (got {t} vs {s})")
+    _want_shape("segment_ids", segment_ids, (b, t))
 
 
 def _sink(logit_sink: Optional[torch.Tensor], num_heads: int) -> Optional[torch.Tensor]:
@@ -116,14 +157,14 @@ def flash_fwd(
     logit_sink [Hq]: optional per-head sink logit (joins the softmax and lse, carries no value).
     bias [B|1,Hq|1,T,S] bf16/fp32: dense additive logit bias.  dropout_mask [B,Hq,T,S] bool/uint8
     (True = dropped) with dropout_rate: kept probabilities are scaled by 1 / (1 - rate)."""
+    b, t, hq, d, s, hkv = _check_qkv(q, k, v)
+    _check_segment_ids(segment_ids, b, t, s)
+    if q_pos_offsets is not None:
+        _want_shape("q_pos_offsets", q_pos_offsets, (b,))
     _require_cuda(q, k, v, segment_ids, logit_sink, bias, dropout_mask, q_pos_offsets)
     lib = _lib.load()
-    b, t, hq, d = q.shape
     if q_pos_offsets is not None:
-        if tuple(q_pos_offsets.shape) != (b,):
-            raise AxlError(_lib.AXL_ERR_INVALID_ARGUMENT, f"q_pos_offsets must have shape [{b}]")
         q_pos_offsets = q_pos_offsets.to(torch.int32).contiguous()
-    s, hkv = k.shape[1], k.shape[2]
     out = torch.empty((b, t, hq, d), dtype=q.dtype, device=q.device)
     lse = torch.empty((b, hq, t), dtype=torch.float32, device=q.device) if return_lse else None
     seg = _seg(segment_ids)
@@ -139,8 +180,6 @@ def flash_fwd(
         q_pos_offset=int(q_pos_offset), softmax_scale=float(softmax_scale),
         logit_sink=_lib.ptr(sink), aux=aux, q_pos_offsets=_lib.ptr(q_pos_offsets),
     )
-    if k.dtype != q.dtype or v.dtype != q.dtype:
-        raise AxlError(_lib.AXL_ERR_UNSUPPORTED, "q, k, v must share one dtype")
     _lib.check(lib.axl_flash_fwd(ctypes.byref(p), _lib.current_stream_ptr()))
     return out, lse
 
@@ -172,14 +211,25 @@ def flash_bwd(
     = (dq, dk, dv, workspace) reuses caller-provided outputs instead of allocating.  bias,
     dropout_mask and dropout_rate must be the ones the forward was given (the bias gets no gradient,
     as in gpu_attention.py:786)."""
-    _require_cuda(q, k, v, out, lse, d_out, segment_ids, logit_sink, bias, dropout_mask)
-    lib = _lib.load()
-    b, t, hq, d = q.shape
-    s, hkv = k.shape[1], k.shape[2]
+    b, t, hq, d, s, hkv = _check_qkv(q, k, v)
+    _check_segment_ids(segment_ids, b, t, s)
+    _want_shape("out", out, q.shape)
+    _want_shape("d_out", d_out, q.shape)
+    _want_shape("lse", lse, (b, hq, t))
+    if out.dtype != q.dtype or d_out.dtype != q.dtype:
+        raise AxlError(_lib.AXL_ERR_UNSUPPORTED, "out and d_out must have the dtype of q")
     ws = None
     if buffers is not None:
         dq, dk, dv, ws = buffers
-    else:
+        _want_shape("buffers dq", dq, q.shape)
+        _want_shape("buffers dk", dk, k.shape)
+        _want_shape("buffers dv", dv, v.shape)
+        if dq.dtype != q.dtype or dk.dtype != q.dtype or dv.dtype != q.dtype:
+            raise AxlError(_lib.AXL_ERR_UNSUPPORTED, "buffers dq, dk, dv must have the dtype of q")
+    _require_cuda(q, k, v, out, lse, d_out, segment_ids, logit_sink, bias, dropout_mask,
+                  *(buffers if buffers is not None else ()))
+    lib = _lib.load()
+    if buffers is None:
         dq = torch.empty((b, t, hq, d), dtype=q.dtype, device=q.device)
         dk = torch.empty((b, s, hkv, d), dtype=k.dtype, device=q.device)
         dv = torch.empty((b, s, hkv, d), dtype=v.dtype, device=q.device)
@@ -220,6 +270,19 @@ def flash_bwd_buffers(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor):
     return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), ws
 
 
+def _decode_flags(deterministic: bool, workspace_reused: bool) -> int:
+    return (_lib.DECODE_DETERMINISTIC if deterministic else 0) | (_lib.DECODE_WORKSPACE_REUSED if workspace_reused else 0)
+
+
+def _check_decode_out_ws(q, out, workspace):
+    if out is not None:
+        _want_shape("out", out, q.shape)
+        if out.dtype != q.dtype or not out.is_contiguous():
+            raise _bad("out must be contiguous and have the dtype of q")
+    if workspace is not None and (workspace.dtype != torch.uint8 or not workspace.is_contiguous()):
+        raise _bad("workspace must be a contiguous uint8 tensor")
+
+
 def paged_decode(
     q: torch.Tensor,
     k_pages: torch.Tensor,
@@ -231,17 +294,38 @@ def paged_decode(
     sliding_window: int = -1,
     workspace: Optional[torch.Tensor] = None,
     out: Optional[torch.Tensor] = None,
+    deterministic: bool = False,
+    workspace_reused: bool = False,
 ) -> torch.Tensor:
-    """q [B,Hq,D]; pools [Hkv,P,page,D]; page_tables [B,pps] int32; lengths [B] int32 -> [B,Hq,D]."""
-    _require_cuda(q, k_pages, v_pages, page_tables, lengths)
-    lib = _lib.load()
+    """q [B,Hq,D]; pools [Hkv,P,page,D]; page_tables [B,pps] int32; lengths [B] int32 -> [B,Hq,D].
+
+    Lengths are clamped to [0, pps * page]; a sequence of length 0 yields zeros.  `deterministic`
+    fixes the work decomposition (bit-reproducible); `workspace_reused` promises that `workspace` was
+    last touched by an earlier decode call (skips the launch that zeroes its work counter)."""
+    if q.dim() != 3 or k_pages.dim() != 4:
+        raise _bad(f"q must be [B,Hq,D] and k_pages [Hkv,P,page,D], got {list(q.shape)}, {list(k_pages.shape)}")
     b, hq, d = q.shape
-    hkv, num_pages, page_size, _ = k_pages.shape
+    hkv, num_pages, page_size, dk = k_pages.shape
+    if dk != d:
+        raise _bad(f"head_dim of k_pages ({dk}) differs from q's ({d})")
+    _want_shape("v_pages", v_pages, k_pages.shape)
+    if hkv <= 0 or hq % hkv != 0:
+        raise _bad(f"num_q_heads {hq} is not divisible by num_kv_heads {hkv}")
+    if page_tables.dim() != 2 or page_tables.shape[0] != b:
+        raise _bad(f"page_tables must be [{b}, pages_per_seq], got {list(page_tables.shape)}")
+    _want_shape("lengths", lengths, (b,))
+    if page_tables.dtype != torch.int32 or lengths.dtype != torch.int32:
+        raise AxlError(_lib.AXL_ERR_INVALID_ARGUMENT, "page_tables and lengths must be int32")
+    if k_pages.dtype != q.dtype or v_pages.dtype != q.dtype:
+        raise AxlError(_lib.AXL_ERR_UNSUPPORTED, "q and the pools must share one dtype")
     for name, x in (("q", q), ("k_pages", k_pages), ("v_pages", v_pages), ("page_tables", page_tables), ("lengths", lengths)):
         if not x.is_contiguous():
             raise AxlError(_lib.AXL_ERR_UNSUPPORTED, f"{name} must be contiguous")
-    if page_tables.dtype != torch.int32 or lengths.dtype != torch.int32:
-        raise AxlError(_lib.AXL_ERR_INVALID_ARGUMENT, "page_tables and lengths must be int32")
+    _check_decode_out_ws(q, out, workspace)
+    if workspace_reused and workspace is None:
+        raise _bad("workspace_reused needs the workspace of the earlier call")
+    _require_cuda(q, k_pages, v_pages, page_tables, lengths, out, workspace)
+    lib = _lib.load()
     if out is None:
         out = torch.empty((b, hq, d), dtype=q.dtype, device=q.device)
     p = AxlPagedDecodeParams(
@@ -251,12 +335,15 @@ def paged_decode(
         page_size=page_size, pages_per_seq=page_tables.shape[1],
         dtype=_lib.dtype_code(q.dtype), sliding_window=int(sliding_window),
         softmax_scale=float(softmax_scale), workspace=None, workspace_bytes=0,
+        flags=_decode_flags(deterministic, workspace_reused),
     )
     need = int(lib.axl_paged_decode_workspace_bytes(ctypes.byref(p)))
-    if workspace is None or workspace.numel() * workspace.element_size() < need:
+    if workspace is None or workspace.numel() < need:
+        if workspace_reused:
+            raise AxlError(_lib.AXL_ERR_WORKSPACE, f"workspace needs {need} bytes, got {workspace.numel()}")
         workspace = torch.empty((max(need, 16),), dtype=torch.uint8, device=q.device)
     p.workspace = workspace.data_ptr()
-    p.workspace_bytes = workspace.numel() * workspace.element_size()
+    p.workspace_bytes = workspace.numel()
     _lib.check(lib.axl_paged_decode(ctypes.byref(p), _lib.current_stream_ptr()))
     return out
 
@@ -283,16 +370,32 @@ def decode(
     sliding_window: int = -1,
     workspace: Optional[torch.Tensor] = None,
     out: Optional[torch.Tensor] = None,
+    deterministic: bool = False,
+    workspace_reused: bool = False,
 ) -> torch.Tensor:
-    """q [B,Hq,D]; k/v [B,S,Hkv,D]; lengths [B] int32 -> [B,Hq,D]."""
-    _require_cuda(q, k, v, lengths)
-    lib = _lib.load()
+    """q [B,Hq,D]; k/v [B,S,Hkv,D]; lengths [B] int32 -> [B,Hq,D].  Lengths are clamped to [0, S]; a
+    sequence of length 0 yields zeros.  `deterministic` / `workspace_reused`: see `paged_decode`."""
+    if q.dim() != 3 or k.dim() != 4:
+        raise _bad(f"q must be [B,Hq,D] and k [B,S,Hkv,D], got {list(q.shape)}, {list(k.shape)}")
     b, hq, d = q.shape
     s, hkv = k.shape[1], k.shape[2]
+    if k.shape[0] != b or k.shape[3] != d:
+        raise _bad(f"k {list(k.shape)} does not match q {list(q.shape)} in batch / head_dim")
+    _want_shape("v", v, k.shape)
+    if hkv <= 0 or hq % hkv != 0:
+        raise _bad(f"num_q_heads {hq} is not divisible by num_kv_heads {hkv}")
+    _want_shape("lengths", lengths, (b,))
+    if k.dtype != q.dtype or v.dtype != q.dtype:
+        raise AxlError(_lib.AXL_ERR_UNSUPPORTED, "q, k, v must share one dtype")
     if not q.is_contiguous():
         raise AxlError(_lib.AXL_ERR_UNSUPPORTED, "q must be contiguous")
     if lengths.dtype != torch.int32 or not lengths.is_contiguous():
         raise AxlError(_lib.AXL_ERR_INVALID_ARGUMENT, "lengths must be contiguous int32")
+    _check_decode_out_ws(q, out, workspace)
+    if workspace_reused and workspace is None:
+        raise _bad("workspace_reused needs the workspace of the earlier call")
+    _require_cuda(q, k, v, lengths, out, workspace)
+    lib = _lib.load()
     if out is None:
         out = torch.empty((b, hq, d), dtype=q.dtype, device=q.device)
     p = AxlDecodeParams(
@@ -301,12 +404,15 @@ def decode(
         batch=b, kv_len=s, num_q_heads=hq, num_kv_heads=hkv, head_dim=d,
         dtype=_lib.dtype_code(q.dtype), sliding_window=int(sliding_window),
         softmax_scale=float(softmax_scale), workspace=None, workspace_bytes=0,
+        flags=_decode_flags(deterministic, workspace_reused),
     )
     need = int(lib.axl_decode_workspace_bytes(ctypes.byref(p)))
-    if workspace is None or workspace.numel() * workspace.element_size() < need:
+    if workspace is None or workspace.numel() < need:
+        if workspace_reused:
+            raise AxlError(_lib.AXL_ERR_WORKSPACE, f"workspace needs {need} bytes, got {workspace.numel()}")
         workspace = torch.empty((max(need, 16),), dtype=torch.uint8, device=q.device)
     p.workspace = workspace.data_ptr()
-    p.workspace_bytes = workspace.numel() * workspace.element_size()
+    p.workspace_bytes = workspace.numel()
     _lib.check(lib.axl_decode(ctypes.byref(p), _lib.current_stream_ptr()))
     return out
 
@@ -329,6 +435,10 @@ def paged_kv_insert(
         raise AxlError(_lib.AXL_ERR_INVALID_ARGUMENT, "nothing to insert")
     _require_cuda(pool, proj, page_indices, key_positions)
     lib = _lib.load()
+    if pool.dim() != 4 or page_indices.dim() != 2:
+        raise _bad(f"pools must be [Hkv,P,page,D] and page_indices [B,pps], got {list(pool.shape)}, {list(page_indices.shape)}")
+    if k_pages is not None and v_pages is not None and tuple(k_pages.shape) != tuple(v_pages.shape):
+        raise _bad(f"k_pages {list(k_pages.shape)} and v_pages {list(v_pages.shape)} differ")
     hkv, num_pages, page_size, d = pool.shape
     b = page_indices.shape[0]
     for name, x in (("k_pages", k_pages), ("v_pages", v_pages), ("page_indices", page_indices),

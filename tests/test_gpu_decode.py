@@ -3,13 +3,13 @@
 Shapes follow the reference's decoding tests (decoding_test.py:95-163, :187-269): (B, S, H, D) in
 {(1,1024,32,64), (4,512,48,64), (2,1024,16,128), (1,4096,8,128)}, padding in {0, 111},
 kv_head_factor in {1, 8}, window in {-1, 127}, page size 16.  Page-table and length masking are
-checked bit-exactly (permutation invariance, poison) with AXL_DECODE_DETERMINISTIC=1, which fixes
-the work decomposition; by default work is handed out dynamically and two calls agree only up to the
-rounding of the fp32 partial sums, which is checked too.
+checked bit-exactly (permutation invariance, poison) with the AXL_DECODE_DETERMINISTIC flag of the
+call, which fixes the work decomposition; by default work is handed out dynamically and two calls
+agree only up to the rounding of the fp32 partial sums, which is checked too.
 """
 
 import contextlib
-import os
+import functools
 
 import numpy as np
 import pytest
@@ -28,16 +28,15 @@ pytestmark = pytest.mark.gpu
 
 @contextlib.contextmanager
 def _deterministic():
-    """Fixed work decomposition: the result does not depend on timing."""
-    old = os.environ.get("AXL_DECODE_DETERMINISTIC")
-    os.environ["AXL_DECODE_DETERMINISTIC"] = "1"
+    """Fixed work decomposition (every decode call inside carries the AXL_DECODE_DETERMINISTIC flag):
+    the result does not depend on timing."""
+    paged, contiguous = ops.paged_decode, ops.decode
+    ops.paged_decode = functools.partial(paged, deterministic=True)
+    ops.decode = functools.partial(contiguous, deterministic=True)
     try:
         yield
     finally:
-        if old is None:
-            del os.environ["AXL_DECODE_DETERMINISTIC"]
-        else:
-            os.environ["AXL_DECODE_DETERMINISTIC"] = old
+        ops.paged_decode, ops.decode = paged, contiguous
 
 
 def _ok(got, want):
@@ -228,6 +227,85 @@ def test_decode_replays_from_a_captured_graph():
             # new inputs in the captured buffers are picked up by the next replay
             lc.copy_(torch.clamp(lengths + 7 * (rep + 1), max=16 * pps).cuda())
             eager = ops.paged_decode(qc, kc, vc, tc, lc, softmax_scale=0.1)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("window", [-1, 40])
+def test_empty_and_out_of_range_lengths(dtype, window):
+    """A sequence without a visible key gets zeros (the reference's combine divides by l + eps,
+    gpu_decoding.py:282, gpu_paged_attention.py:291-293); lengths beyond the capacity are clamped to
+    it; negative lengths count as 0.  The other rows are unaffected and finite."""
+    b, hq, hkv, d, pps = 6, 8, 2, 128, 12
+    q, kp, vp, tables, lengths = ref.paged_inputs(17, batch=b, num_heads=hq, num_kv_heads=hkv, head_dim=d,
+                                                  page_size=16, pages_per_seq=pps, min_len=5, max_len=16 * pps,
+                                                  dtype=dtype)
+    cap = 16 * pps
+    lengths[1], lengths[3], lengths[4] = 0, cap + 1000, -7
+    clamped = lengths.clamp(0, cap)
+    live = [i for i in range(b) if int(clamped[i]) > 0]
+    want = ref.reference_decode(q[live], kp, vp, clamped[live], softmax_scale=0.1, page_tables=tables[live],
+                                sliding_window=None if window < 0 else window)[:, 0]
+    kk, vv = ref.reconstruct_kv(tables, kp), ref.reconstruct_kv(tables, vp)
+    tol = dict(atol=1e-5) if dtype == torch.float32 else None
+    for det in (False, True):
+        got = ops.paged_decode(q[:, 0].cuda(), kp.cuda(), vp.cuda(), tables.cuda(), lengths.cuda(), softmax_scale=0.1,
+                               sliding_window=window, deterministic=det).cpu()
+        got2 = ops.decode(q[:, 0].cuda(), kk.cuda(), vv.cuda(), lengths.cuda(), softmax_scale=0.1,
+                          sliding_window=window, deterministic=det).cpu()
+        for out in (got, got2):
+            assert torch.isfinite(out.float()).all()
+            assert (out[1] == 0).all() and (out[4] == 0).all()
+            if tol:
+                assert ref.max_abs(out[live], want) <= 1e-5
+            else:
+                assert _ok(out[live], want), (ref.max_abs(out[live], want), ref.rel_l2(out[live], want))
+    # every sequence empty
+    zero = torch.zeros((b,), dtype=torch.int32)
+    out = ops.paged_decode(q[:, 0].cuda(), kp.cuda(), vp.cuda(), tables.cuda(), zero.cuda(), softmax_scale=0.1,
+                           sliding_window=window)
+    assert (out == 0).all()
+
+
+def test_reused_workspace_skips_the_counter_reset():
+    """With AXL_DECODE_WORKSPACE_REUSED the call relies on the counter its predecessor left at zero:
+    eager calls of different shapes on one workspace and graph replays all equal the plain call."""
+    b, hq, hkv, d, pps = 7, 16, 4, 128, 48
+    q, kp, vp, tables, lengths = ref.paged_inputs(33, batch=b, num_heads=hq, num_kv_heads=hkv, head_dim=d,
+                                                  page_size=16, pages_per_seq=pps, min_len=3, max_len=16 * pps)
+    qc, kc, vc, tc, lc = q[:, 0].cuda(), kp.cuda(), vp.cuda(), tables.cuda(), lengths.cuda()
+    kk, vv = ref.reconstruct_kv(tables, kp).cuda(), ref.reconstruct_kv(tables, vp).cuda()
+    want = ops.paged_decode(qc, kc, vc, tc, lc, softmax_scale=0.1, deterministic=True)
+    ws = torch.empty((ops.paged_decode_workspace_bytes(b, hq, hkv, d, pps) + 64,), dtype=torch.uint8, device="cuda")
+    ws.random_(0, 255)
+    first = ops.paged_decode(qc, kc, vc, tc, lc, softmax_scale=0.1, deterministic=True, workspace=ws)  # resets
+    assert torch.equal(first, want)
+    for rep in range(3):
+        again = ops.paged_decode(qc, kc, vc, tc, lc, softmax_scale=0.1, deterministic=True, workspace=ws,
+                                 workspace_reused=True)
+        assert torch.equal(again, want), rep
+        # another shape (fewer sequences, contiguous cache, dynamic hand-out) in between
+        other = ops.decode(qc[:3], kk[:3], vv[:3], lc[:3], softmax_scale=0.1, workspace=ws, workspace_reused=True)
+        assert ref.max_abs(other.cpu(), want[:3].cpu().float()) <= 2e-3
+        dyn = ops.paged_decode(qc, kc, vc, tc, lc, softmax_scale=0.1, workspace=ws, workspace_reused=True)
+        assert ref.max_abs(dyn.cpu(), want.cpu().float()) <= 2e-3
+    out_g = torch.empty_like(qc)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        ops.paged_decode(qc, kc, vc, tc, lc, softmax_scale=0.1, deterministic=True, workspace=ws, out=out_g,
+                         workspace_reused=True)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ops.paged_decode(qc, kc, vc, tc, lc, softmax_scale=0.1, deterministic=True, workspace=ws, out=out_g,
+                         workspace_reused=True)
+    for rep in range(3):
+        out_g.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, want), rep
+        eager = ops.paged_decode(qc, kc, vc, tc, lc, softmax_scale=0.1, deterministic=True)
+        assert torch.equal(eager, want)
 
 
 def test_baseline_c4_full_size():

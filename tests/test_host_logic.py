@@ -353,3 +353,58 @@ def test_abi_validation_without_gpu():
     assert lib.axl_paged_decode_workspace_bytes(ctypes.byref(dp)) > 0
     dp.num_q_heads = 64
     assert lib.axl_paged_decode(ctypes.byref(dp), None) == _lib.AXL_ERR_UNSUPPORTED  # 32 heads per kv head
+
+
+def test_ops_reject_mismatched_shapes_before_any_launch():
+    """The tensor-level wrappers hand raw pointers to the kernels, so every extent that the kernels
+    take from q / k alone is checked against the other tensors first.  CPU tensors suffice: the shape
+    checks come before the device check and before the library is touched."""
+    from axlearn_amd import ops
+
+    bf = torch.bfloat16
+    q = torch.zeros((2, 128, 4, 64), dtype=bf)
+    k = torch.zeros((2, 128, 2, 64), dtype=bf)
+
+    def raises(fn, *args, **kw):
+        with pytest.raises(_lib.AxlError) as e:
+            fn(*args, **kw)
+        return e.value
+
+    assert raises(ops.flash_fwd, q, k[:1], k[:1]).code == _lib.AXL_ERR_INVALID_ARGUMENT       # batch
+    assert raises(ops.flash_fwd, q, k, k[:, :64]).code == _lib.AXL_ERR_INVALID_ARGUMENT       # v vs k
+    assert raises(ops.flash_fwd, q, k[..., :32], k[..., :32]).code == _lib.AXL_ERR_INVALID_ARGUMENT  # head_dim
+    assert raises(ops.flash_fwd, q[:, :, :3], k, k).code == _lib.AXL_ERR_INVALID_ARGUMENT     # 3 heads over 2
+    assert raises(ops.flash_fwd, q, k.float(), k.float()).code == _lib.AXL_ERR_UNSUPPORTED    # dtypes differ
+    seg = torch.zeros((2, 64), dtype=torch.int32)
+    assert "segment_ids" in str(raises(ops.flash_fwd, q, k, k, segment_ids=seg))
+    assert "q_pos_offsets" in str(raises(ops.flash_fwd, q, k, k, q_pos_offsets=torch.zeros(3, dtype=torch.int32)))
+    # all shapes right: the next thing to fail is the device check
+    assert "GPU" in str(raises(ops.flash_fwd, q, k, k, segment_ids=torch.zeros((2, 128), dtype=torch.int32)))
+
+    lse = torch.zeros((2, 4, 128))
+    assert "lse" in str(raises(ops.flash_bwd, q, k, k, q, lse[:, :2], q))
+    assert "out" in str(raises(ops.flash_bwd, q, k, k, q[:, :64], lse, q))
+    assert "d_out" in str(raises(ops.flash_bwd, q, k, k, q, lse, q[:1]))
+    bufs = (torch.zeros_like(q), torch.zeros_like(k)[:, :64], torch.zeros_like(k), None)
+    assert "buffers dk" in str(raises(ops.flash_bwd, q, k, k, q, lse, q, buffers=bufs))
+    assert "GPU" in str(raises(ops.flash_bwd, q, k, k, q, lse, q))
+
+    dq = torch.zeros((3, 8, 128), dtype=bf)
+    pool = torch.zeros((2, 40, 16, 128), dtype=bf)
+    tables = torch.zeros((3, 10), dtype=torch.int32)
+    lengths = torch.zeros((3,), dtype=torch.int32)
+    assert "page_tables" in str(raises(ops.paged_decode, dq, pool, pool, tables[:2], lengths))
+    assert "lengths" in str(raises(ops.paged_decode, dq, pool, pool, tables, lengths[:2]))
+    assert "v_pages" in str(raises(ops.paged_decode, dq, pool, pool[:, :39], tables, lengths))
+    assert "head_dim" in str(raises(ops.paged_decode, dq[..., :64], pool, pool, tables, lengths))
+    assert "int32" in str(raises(ops.paged_decode, dq, pool, pool, tables.long(), lengths))
+    assert "out" in str(raises(ops.paged_decode, dq, pool, pool, tables, lengths, out=torch.zeros((3, 8, 64), dtype=bf)))
+    assert "workspace" in str(raises(ops.paged_decode, dq, pool, pool, tables, lengths, workspace=torch.zeros(8)))
+    assert "workspace_reused" in str(raises(ops.paged_decode, dq, pool, pool, tables, lengths, workspace_reused=True))
+    assert "GPU" in str(raises(ops.paged_decode, dq, pool, pool, tables, lengths))
+
+    kc = torch.zeros((3, 160, 2, 128), dtype=bf)
+    assert "does not match" in str(raises(ops.decode, dq, kc[:2], kc[:2], lengths))
+    assert "v" in str(raises(ops.decode, dq, kc, kc[:, :100], lengths))
+    assert "lengths" in str(raises(ops.decode, dq, kc, kc, lengths[:1]))
+    assert "GPU" in str(raises(ops.decode, dq, kc, kc, lengths))
