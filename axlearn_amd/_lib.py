@@ -136,6 +136,7 @@ EXPORTED_SYMBOLS = (
     "axl_flash_bwd_workspace_bytes",
     "axl_paged_decode",
     "axl_paged_decode_workspace_bytes",
+    "axl_paged_decode_static",
     "axl_decode",
     "axl_decode_workspace_bytes",
     "axl_paged_kv_insert",
@@ -168,6 +169,7 @@ def load() -> ctypes.CDLL:
         ("axl_flash_fwd", AxlFlashFwdParams),
         ("axl_flash_bwd", AxlFlashBwdParams),
         ("axl_paged_decode", AxlPagedDecodeParams),
+        ("axl_paged_decode_static", AxlPagedDecodeParams),
         ("axl_decode", AxlDecodeParams),
         ("axl_paged_kv_insert", AxlPageInsertParams),
     ):

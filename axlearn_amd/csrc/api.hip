@@ -25,6 +25,7 @@ int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream)
 size_t flash_bwd_workspace_bytes(const AxlFlashBwdParams& p);
 int launch_paged_decode(const AxlPagedDecodeParams& p, hipStream_t stream);
 size_t paged_decode_workspace_bytes(const AxlPagedDecodeParams& p);
+int launch_paged_decode_static(const AxlPagedDecodeParams& p, hipStream_t stream);
 int launch_decode(const AxlDecodeParams& p, hipStream_t stream);
 size_t decode_workspace_bytes(const AxlDecodeParams& p);
 int launch_page_insert(const AxlPageInsertParams& p, hipStream_t stream);
@@ -253,20 +254,32 @@ size_t axl_paged_decode_workspace_bytes(const AxlPagedDecodeParams* p) {
   return paged_decode_workspace_bytes(*p);
 }
 
-int axl_paged_decode(const AxlPagedDecodeParams* p, void* stream) {
-  if (!p) return set_error(AXL_ERR_INVALID_ARGUMENT, "axl_paged_decode: params is NULL");
-  int rc = check_decode_common("axl_paged_decode", p->batch, p->num_q_heads, p->num_kv_heads,
-                               p->head_dim, p->dtype, p->softmax_scale);
+// Everything axl_paged_decode checks except the workspace.
+static int check_paged_decode(const char* who, const AxlPagedDecodeParams* p) {
+  if (!p) return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: params is NULL", who);
+  int rc = check_decode_common(who, p->batch, p->num_q_heads, p->num_kv_heads, p->head_dim, p->dtype,
+                               p->softmax_scale);
   if (rc != AXL_OK) return rc;
   if (p->num_pages <= 0 || p->page_size <= 0 || p->pages_per_seq <= 0)
-    return set_error(AXL_ERR_INVALID_ARGUMENT, "axl_paged_decode: non-positive page geometry");
+    return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: non-positive page geometry", who);
   if (!p->q || !p->k_pages || !p->v_pages || !p->page_tables || !p->lengths || !p->out)
-    return set_error(AXL_ERR_INVALID_ARGUMENT, "axl_paged_decode: NULL tensor pointer");
+    return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: NULL tensor pointer", who);
   if (p->page_size != 16)
-    return set_error(AXL_ERR_UNSUPPORTED, "axl_paged_decode: page_size %d (supported: 16)",
-                     p->page_size);
+    return set_error(AXL_ERR_UNSUPPORTED, "%s: page_size %d (supported: 16)", who, p->page_size);
   if (!aligned16(p->q) || !aligned16(p->k_pages) || !aligned16(p->v_pages) || !aligned16(p->out))
-    return set_error(AXL_ERR_UNSUPPORTED, "axl_paged_decode: tensors must be 16-byte aligned");
+    return set_error(AXL_ERR_UNSUPPORTED, "%s: tensors must be 16-byte aligned", who);
+  return AXL_OK;
+}
+
+int axl_paged_decode_static(const AxlPagedDecodeParams* p, void* stream) {
+  const int rc = check_paged_decode("axl_paged_decode_static", p);
+  if (rc != AXL_OK) return rc;
+  return launch_paged_decode_static(*p, (hipStream_t)stream);
+}
+
+int axl_paged_decode(const AxlPagedDecodeParams* p, void* stream) {
+  const int rc = check_paged_decode("axl_paged_decode", p);
+  if (rc != AXL_OK) return rc;
   const size_t need = paged_decode_workspace_bytes(*p);
   if (!p->workspace || p->workspace_bytes < need || !aligned16(p->workspace))
     return set_error(AXL_ERR_WORKSPACE, "axl_paged_decode: workspace needs %zu bytes, got %zu",

@@ -31,6 +31,8 @@
 // position is length-1, so a sliding window w also masks keys with (length-1) - j > w.  A page
 // index outside the pool reads as zeros and a negative one counts from the end of the pool, as the
 // reference's gather does (kv_cache/paged_kv_cache.py:32).
+#include <mutex>
+
 #include "common.h"
 
 namespace axl {
@@ -870,6 +872,56 @@ int launch_paged_decode(const AxlPagedDecodeParams& p, hipStream_t stream) {
   if (p.dtype == AXL_F32) return launch_f32<true>(a, p.head_dim, stream, "axl_paged_decode");
   return p.dtype == AXL_F16 ? launch_common<ElemF16, true>(a, p.head_dim, p.flags, stream, "axl_paged_decode")
                             : launch_common<ElemBf16, true>(a, p.head_dim, p.flags, stream, "axl_paged_decode");
+}
+
+// ---------------------------------------------------------------------------------------------
+// Allocation-free variant of the paged decode: the split-K workspace (partial records, record table,
+// work counter) is this file-scope device array instead of caller memory.  Every GPU the library runs
+// on holds its own copy until the process ends; `scratch` itself is a host-side stand-in, the device
+// address comes from hipGetSymbolAddress, once per device.
+// ---------------------------------------------------------------------------------------------
+constexpr size_t kStaticScratchBytes = AXL_PAGED_DECODE_STATIC_MAX_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mu;
+static void* g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each device, once resolved
+
+// Device address of this device's copy of `scratch` (the current device is the one the call runs on).
+static int static_scratch(void** ptr, const char* who) {
+  int dev = 0;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return set_error(AXL_ERR_LAUNCH, "%s: hipGetDevice: %s", who, hipGetErrorString(err));
+  if (dev < 0 || dev >= kMaxDevices) return set_error(AXL_ERR_UNSUPPORTED, "%s: device index %d", who, dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (err != hipSuccess || !p)
+      return set_error(AXL_ERR_LAUNCH, "%s: hipGetSymbolAddress(scratch): %s", who, hipGetErrorString(err));
+    g_scratch_ptr[dev] = p;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return AXL_OK;
+}
+
+int launch_paged_decode_static(const AxlPagedDecodeParams& p, hipStream_t stream) {
+  const char* who = "axl_paged_decode_static";
+  const size_t need = paged_decode_workspace_bytes(p);
+  if (need > kStaticScratchBytes)
+    return set_error(AXL_ERR_WORKSPACE,
+                     "%s: these shapes need %zu bytes of split-K scratch, the built-in buffer holds %zu "
+                     "(use axl_paged_decode with a caller workspace)", who, need, kStaticScratchBytes);
+  void* ws = nullptr;
+  const int rc = static_scratch(&ws, who);
+  if (rc != AXL_OK) return rc;
+  AxlPagedDecodeParams q = p;
+  q.workspace = ws;  // the resolved device address, never the array's name
+  q.workspace_bytes = kStaticScratchBytes;
+  // The buffer keeps the previous call's contents (possibly of other shapes, possibly of a call that
+  // was captured and never replayed): the work counter is zeroed by a kernel on every call.
+  q.flags &= ~AXL_DECODE_WORKSPACE_REUSED;
+  return launch_paged_decode(q, stream);
 }
 
 int launch_decode(const AxlDecodeParams& p, hipStream_t stream) {
