@@ -206,6 +206,17 @@ __device__ __forceinline__ void dma16s_first16(unsigned voff, const void* sbase,
       : "v"(voff), "s"(sbase), "s"(lds_base)
       : "memory", "m0");
 }
+// Two 16-byte-per-lane global stores from one scalar base: lane l's pieces go to sbase + voff and
+// sbase + voff + 1024.  Issued through inline assembly like the tile loads, so the compiler's wait
+// counts never involve them (vector memory stores count in vmcnt as well).  The data is written once
+// and read by a later kernel: streaming policy (write through, no reuse), which costs the issuing
+// kernel least (measured against the default and the single-modifier policies).
+__device__ __forceinline__ void store16x2(unsigned voff, void* sbase, bf16x8 d0, bf16x8 d1) {
+  asm volatile("global_store_dwordx4 %0, %1, %3 sc0 sc1 nt\n\tglobal_store_dwordx4 %0, %2, %3 offset:1024 sc0 sc1 nt"
+               :
+               : "v"(voff), "v"(d0), "v"(d1), "s"(sbase)
+               : "memory");
+}
 #pragma clang diagnostic pop
 template <int N>
 __device__ __forceinline__ void wait_vmem_le() {

@@ -319,9 +319,32 @@ __global__ __launch_bounds__(256) void flash_bwd_dq_aux_kernel(const BwdArgs a) 
 
 static Strides3 to_s3(const AxlStrides& s) { return Strides3{s.batch, s.seq, s.head}; }
 
+// delta and lse2, [B, Hq, T] fp32 each, rounded up to 256 bytes.
+static size_t stats_bytes(const AxlFlashBwdParams& p) {
+  return (2 * (size_t)p.batch * p.num_q_heads * p.q_len * sizeof(float) + 255) & ~(size_t)255;
+}
+
+// The dS-spill path: the dK/dV kernel stores dS and the dQ kernel becomes one streaming GEMM
+// (5 executed GEMMs instead of 7).  Plain causal attention over equal lengths only.
+static bool spill_eligible(const AxlFlashBwdParams& p) {
+  return (p.dtype == AXL_BF16 || p.dtype == AXL_F16) && p.mask_kind == AXL_MASK_CAUSAL && p.q_pos_offset == 0 &&
+         p.q_len == p.kv_len && !p.segment_ids && !p.aux.bias && !p.aux.dropout_mask &&
+         !(p.flags & AXL_BWD_NO_SPILL);
+}
+
+static size_t spill_bytes(const AxlFlashBwdParams& p) {
+  return (size_t)p.batch * p.num_q_heads * (size_t)ds_blocks_per_head(p.q_len) * kDsBlockBytes;
+}
+
+// Above this size the dS workspace is not asked for (the caller can still pass one: a workspace that
+// holds it selects the spill path whatever its size).
+constexpr size_t kSpillAskCap = (size_t)8 << 30;
+
+size_t flash_bwd_min_workspace_bytes(const AxlFlashBwdParams& p) { return stats_bytes(p); }
+
 size_t flash_bwd_workspace_bytes(const AxlFlashBwdParams& p) {
-  // delta and lse2, [B, Hq, T] fp32 each.
-  return 2 * (size_t)p.batch * p.num_q_heads * p.q_len * sizeof(float);
+  if (spill_eligible(p) && spill_bytes(p) <= kSpillAskCap) return stats_bytes(p) + spill_bytes(p);
+  return stats_bytes(p);
 }
 
 int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream) {
@@ -331,6 +354,9 @@ int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream)
   a.ndelta = (float*)p.workspace;
   a.lse2 = a.ndelta + (size_t)p.batch * p.num_q_heads * p.q_len;
   a.dq = p.dq; a.dk = p.dk; a.dv = p.dv; a.seg = p.segment_ids;
+  // A workspace that also holds dS selects the spill path.
+  const bool spill = spill_eligible(p) && p.workspace_bytes >= stats_bytes(p) + spill_bytes(p);
+  a.ds = spill ? (char*)p.workspace + stats_bytes(p) : nullptr;
   a.qs = to_s3(p.q_strides); a.ks = to_s3(p.k_strides); a.vs = to_s3(p.v_strides);
   a.os = to_s3(p.out_strides); a.dos = to_s3(p.d_out_strides); a.dqs = to_s3(p.dq_strides);
   a.dks = to_s3(p.dk_strides); a.dvs = to_s3(p.dv_strides);
@@ -362,6 +388,29 @@ int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream)
       else AXL_LAUNCH((bwd_delta_kernel<float, 64>), delta_grid, 0);
     }
     if (err == hipSuccess) err = launch_bwd_f32(a, p.head_dim, phases, stream);
+  } else if (spill) {
+    // delta, then the dK/dV kernel (which leaves dS behind), then dq = scale * dS k.
+    if (phases & AXL_BWD_DELTA) {
+      if (dt == AXL_BF16) {
+        if (p.head_dim == 128) AXL_LAUNCH((bwd_delta_kernel<__bf16, 128>), delta_grid, 0);
+        else AXL_LAUNCH((bwd_delta_kernel<__bf16, 64>), delta_grid, 0);
+      } else {
+        if (p.head_dim == 128) AXL_LAUNCH((bwd_delta_kernel<_Float16, 128>), delta_grid, 0);
+        else AXL_LAUNCH((bwd_delta_kernel<_Float16, 64>), delta_grid, 0);
+      }
+    }
+    if ((phases & AXL_BWD_DKDV) && err == hipSuccess) err = launch_bwd_dkdv(a, dt, p.head_dim, false, stream);
+    if ((phases & AXL_BWD_DQ) && err == hipSuccess) err = launch_bwd_dq_stream(a, dt, p.head_dim, stream);
+    phases &= AXL_BWD_DELTA;  // what is left for the code below: the sink gradient
+    phases = (phases & AXL_BWD_DELTA) && p.d_logit_sink ? AXL_BWD_DELTA : 0;
+    if (phases) {
+      hipLaunchKernelGGL(bwd_dsink_kernel, dim3(p.num_q_heads), dim3(256), 0, stream, p.logit_sink,
+                         p.lse, a.ndelta, p.d_logit_sink, p.batch, p.num_q_heads, p.q_len);
+      if (err == hipSuccess) err = hipGetLastError();
+    }
+    if (err != hipSuccess)
+      return set_error(AXL_ERR_LAUNCH, "axl_flash_bwd: launch failed: %s", hipGetErrorString(err));
+    return AXL_OK;
   } else if ((phases & all) == all && !aux && !p.d_logit_sink) {
     err = launch_bwd_dq(a, dt, p.head_dim, true, stream);
     if (err == hipSuccess) err = launch_bwd_dkdv(a, dt, p.head_dim, false, stream);

@@ -9,19 +9,21 @@
 // those keys (128 registers), and loops over ALL query heads of the kv head's group and all query
 // tiles that can see the keys, so dK/dV need neither atomics nor a pass that sums repeated KV
 // heads.  Query tiles (32 rows of Q and dO plus their scaled lse / delta / segment ids) stream
-// through a five-deep LDS ring, filled by direct global->LDS loads: no staging registers and no LDS
+// through a six-deep LDS ring, filled by direct global->LDS loads: no staging registers and no LDS
 // store instructions, one unpadded XOR-swizzled copy per tile that serves both the row-per-lane
 // fragment reads of stage A and the transposing reads of stage B without bank conflicts.
 //
 // Register pressure allows one wavefront per SIMD, so nobody else can cover this wavefront's
-// latencies; the loop is software pipelined by hand instead.  Iteration j runs
-//   stage A of tile j+1:  S = Q K^T and dP = dO V^T   (2*D/16 MFMAs, lane = key, registers = queries)
-//   stage B of tile j:    P = exp2(S*c - lse), dS = P * (dP - delta) elementwise, then
-//                         dV^T += dO^T P and dK^T += Q^T dS   (D/4 MFMAs, A operands from
-//                         transposing LDS reads of the same dO / Q tiles)
-// and the elementwise work of stage B is issued BETWEEN the MFMAs of stage A, one slice per MFMA, so
-// the VALU and the matrix pipe run at the same time.  Masks are evaluated arithmetically on every
-// tile (no branches inside the loop body: a branch would end the scheduling region).
+// latencies; the loop is software pipelined by hand instead, with three tiles in flight.  Iteration j
+// runs
+//   stage A of tile j+2:      S = Q K^T and dP = dO V^T   (2*D/16 MFMAs, lane = key, registers = queries)
+//   elementwise of tile j+1:  P = exp2(S*c - lse), dS = P * (dP - delta), packed to 16 bits
+//   stage B of tile j:        dV^T += dO^T P and dK^T += Q^T dS   (D/4 MFMAs, A operands from
+//                             transposing LDS reads of the same dO / Q tiles)
+// while tile j+3 is awaited and tiles j+4, j+5 are in flight from HBM / L2.  Everything that is not
+// an MFMA is dealt out over the MFMA slots of the iteration.  Tiles that no mask touches run a copy
+// of the loop without mask arithmetic; the choice is made per run of tiles, never inside an iteration
+// (a branch would end the scheduling region).
 #include <type_traits>
 
 #include "flash_bwd.h"
@@ -41,7 +43,7 @@ struct DkvTile {
   static constexpr int STAT_BASE = 2 * TILE_BYTES;
   static constexpr int STAT_BYTES = 4 * BQ * 4;  // -lse*log2e | -delta | segment id | (unused) per query row
   static constexpr int BUF_BYTES = STAT_BASE + STAT_BYTES;
-  static constexpr int NBUF = 5;
+  static constexpr int NBUF = 6;
   static constexpr int RPI = 1024 / ROWB;                        // rows per direct-to-LDS instruction
   static constexpr int DMA_PER_WAVE = BQ / 4 / RPI;              // per tensor per tile (8 rows per wavefront)
   static constexpr int DMA_PER_TILE = 2 * DMA_PER_WAVE + 1;      // Q, dO and one row of statistics
@@ -51,9 +53,12 @@ struct DkvTile {
 constexpr int kMaxSubDkv = 1024;                 // query tiles whose segment ids the dK/dV kernel classifies
 constexpr int kNotUniformDkv = -0x7fffffff - 1;  // marks a tile with more than one segment id
 
-template <typename E, int D, bool HAS_SEG, bool AUX>
+// SPILL: the kernel also stores every tile's dS (rounded to the input dtype, as it enters the dK
+// product) into the a.ds workspace, for the streaming dQ kernel.  Causal mask with q_off 0 and T == S.
+template <typename E, int D, bool HAS_SEG, bool AUX, bool SPILL = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void flash_bwd_dkdv_kernel(const BwdArgs a) {
+  static_assert(!SPILL || (!HAS_SEG && !AUX), "the spill path has no segment ids, bias or dropout mask");
   using Tile = DkvTile<D>;
   constexpr int KK = D / 16, DT = D / 32;
   constexpr int NA = 2 * KK;          // stage-A MFMAs per tile
@@ -115,6 +120,14 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
   // at the same time and all but one of them find them in L2.
   const int total = nt * G;
   const int t_first = t_begin + max(nt - 1, 0);  // the tile the sequence starts with
+  // dS store cursor (SPILL): block of this wavefront's 32 keys in the run of the tile whose stage B
+  // the iteration executes; it walks the tiles in processing order.  A lane stores its two packed
+  // operand registers at [query half][key l32][8 g .. 8 g + 7].
+  char* ds_ptr = nullptr;
+  int st_t = t_first, st_h = 0;
+  const unsigned ds_lane = (unsigned)(l32 * 32 + g * 16);
+  if constexpr (SPILL)
+    ds_ptr = (char*)a.ds + (ds_run_start(pair, a.T, G, t_first, 0) + 4 * kb + wave) * kDsBlockBytes;
   // keep(q, k)  <=>  (unsigned)(qpos - kpos) <= limit
   const unsigned limit = a.mask_kind == AXL_MASK_NONE             ? 0xffffffffu
                          : a.mask_kind == AXL_MASK_SLIDING_WINDOW ? (unsigned)a.window
@@ -197,8 +210,9 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
   char* buf_b = smem;                         // tile j     (stage B reads)
   char* buf_e = smem + Tile::BUF_BYTES;       // tile j + 1 (next stage B; its statistics are in registers)
   char* buf_a = smem + 2 * Tile::BUF_BYTES;   // tile j + 2 (stage A reads)
-  char* buf_n = smem + 3 * Tile::BUF_BYTES;   // tile j + 3 (requested one iteration ago, awaited at the end of this one)
-  char* buf_s = smem + 4 * Tile::BUF_BYTES;   // tile j + 4 (requested during this iteration)
+  char* buf_n = smem + 3 * Tile::BUF_BYTES;   // tile j + 3 (requested two iterations ago, awaited at the end of this one)
+  char* buf_s = smem + 4 * Tile::BUF_BYTES;   // tile j + 4 (requested one iteration ago)
+  char* buf_s2 = smem + 5 * Tile::BUF_BYTES;  // tile j + 5 (requested during this iteration)
 
   // Per-lane read offsets (bytes) into a swizzled tile.  Stage A: row swap_bits_2_3(l32), logical
   // chunk 2kk + g.  Stage B (transposing reads): row 8g + j16/4 (+4 for the second half, +16 for the
@@ -360,8 +374,8 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
   constexpr int LD_SLOT0 = 2;                 // one per slot from here on, after the cursor moved in slot 1
   static_assert(LD_SLOT0 + NLD <= NS, "the loads of a tile fit into one iteration");
   TrFrag bfr_next[kAheadB];            // first stage-B fragments of the next iteration
-  int q0_a = t_first * Tile::BQ, q0_s = q0_a;  // first query of tiles j+2 and j+3
-  int h_a = 0, h_s = 0;                        // and their heads within the group
+  int q0_a = t_first * Tile::BQ, q0_s = q0_a, q0_s2 = q0_a;  // first query of tiles j+2, j+3 and j+4
+  int h_a = 0, h_s = 0, h_s2 = 0;                            // and their heads within the group
 
   if (total > 0) {
     // Everything the compiler tracks (stationary fragments, segment ids) has landed before the first
@@ -379,6 +393,10 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
     q0_s = (t_begin + pf_t) * Tile::BQ;
     h_s = pf_h;
     AXL_DMA_TILE(lds_address(buf_n))
+    AXL_ADVANCE()
+    q0_s2 = (t_begin + pf_t) * Tile::BQ;
+    h_s2 = pf_h;
+    AXL_DMA_TILE(lds_address(buf_s))
     if constexpr (AUX) {                 // bias / dropout columns of tile 0
       const char* bp_;
       const uint8_t* dp_;
@@ -436,8 +454,8 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
     floatx16 s_a, dp_a;
     floatx16 dp_start = zero16;          // first operand of the dP chain: -delta without a dropout mask
     PackedOperand pb_n, dsb_n;           // tile j + 1, packed as its elements complete
-    int q0_p = q0_s, h_p = h_s;
-    const unsigned lds_s = lds_address(buf_s);
+    int q0_p = q0_s2, h_p = h_s2;
+    const unsigned lds_s = lds_address(buf_s2);
     const char* a_ad[KK];                // this iteration's fragment addresses: stage A in tile j+2,
     const char* b_ad[2][DT];             // stage B in tile j,
     const char* e_ad[2][DT];             // and the first stage-B fragments of tile j+1
@@ -457,6 +475,18 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
 #pragma unroll
       for (int r = 0; r < 16; r++) braw_n[r] = draw_n[r] = 0;
       AXL_AUX_ROW0(h_a, q0_a, bias_t, drop_t)
+    }
+    if constexpr (SPILL) {
+      // dS of tile j (this iteration's stage-B operand), ahead of the iteration's tile loads: by the
+      // end of the iteration the stores have long been accepted.
+      store16x2(ds_lane, ds_ptr, dsb.v[0], dsb.v[1]);
+      // next head of the same tile (one run further), or head 0 of the tile before (G runs of that
+      // tile back from head 0 of this one)
+      const bool wrap_ = st_h + 1 == G;
+      const int run_ = 4 * ((st_t >> 2) + 1) * kDsBlockBytes, run_prev_ = 4 * (((st_t - 1) >> 2) + 1) * kDsBlockBytes;
+      ds_ptr += wrap_ ? -(int64_t)((G - 1) * run_ + G * run_prev_) : (int64_t)run_;
+      st_h = wrap_ ? 0 : st_h + 1;
+      st_t -= wrap_ ? 1 : 0;
     }
     __builtin_amdgcn_sched_barrier(0);
     // One MFMA slot.  The slot number is a compile-time constant (the slots are instantiated one by
@@ -529,19 +559,22 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
       __builtin_amdgcn_sched_barrier(0);
     };
     for_each_index<NS>(slot);
-    // Tile j+3 (requested during the previous iteration) has landed once at most this iteration's
-    // loads are outstanding; after the barrier every wavefront's part of it is visible, and nobody
-    // reads tile j's buffer any more, which the next iteration refills.  (With a bias or a dropout
-    // mask, at least 27 of their element loads - 11 of the previous iteration, 16 of this one - are
-    // younger than tile j+3's loads as well; 24 leaves a margin.)
-    wait_vmem_le<NLD + (AUX ? 24 : 0)>();
+    // Tile j+3 (requested two iterations ago) has landed once at most the loads of the last two
+    // iterations are outstanding (loads complete in issue order; the dS stores of the spill path may
+    // complete out of order with them, which only makes the count stricter); after the barrier every
+    // wavefront's part of it is visible, and nobody reads tile j's buffer any more, which the next
+    // iteration refills.  (With a bias or a dropout mask, at least 43 of their element loads - 11 of
+    // the iteration before last, 16 of each iteration since - are younger than tile j+3's loads as
+    // well; 40 leaves a margin.)
+    wait_vmem_le<2 * NLD + (AUX ? 40 : 0)>();
     __syncthreads();
     char* const tmp = buf_b;
     buf_b = buf_e;
     buf_e = buf_a;
     buf_a = buf_n;
     buf_n = buf_s;
-    buf_s = tmp;
+    buf_s = buf_s2;
+    buf_s2 = tmp;
     s_e = s_a;
     dp_e = dp_a;
     pb = pb_n;
@@ -555,9 +588,11 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
     }
     diff0 = (q0_a + a.q_off + 8 * g) - kpos;
     q0_a = q0_s;
-    q0_s = q0_p;
+    q0_s = q0_s2;
+    q0_s2 = q0_p;
     h_a = h_s;
-    h_s = h_p;
+    h_s = h_s2;
+    h_s2 = h_p;
   }
   };
   // Query tile t (counted from t_begin) needs no mask for this wavefront's 32 keys when its queries
@@ -665,10 +700,10 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
     }
 }
 
-template <typename E, int D, bool HAS_SEG, bool AUX>
+template <typename E, int D, bool HAS_SEG, bool AUX, bool SPILL = false>
 static hipError_t launch_one(const BwdArgs& a, hipStream_t stream) {
   using Tile = DkvTile<D>;
-  auto kernel = flash_bwd_dkdv_kernel<E, D, HAS_SEG, AUX>;
+  auto kernel = flash_bwd_dkdv_kernel<E, D, HAS_SEG, AUX, SPILL>;
   hipError_t err = allow_dynamic_lds((const void*)kernel, Tile::LDS_BYTES);
   if (err != hipSuccess) return err;
   const int grid = (a.S / Tile::BKV) * a.B * a.Hkv;
@@ -684,6 +719,9 @@ static hipError_t launch_for(const BwdArgs& a, int head_dim, bool aux, hipStream
       return seg ? launch_one<E, 128, true, true>(a, stream) : launch_one<E, 128, false, true>(a, stream);
     return seg ? launch_one<E, 64, true, true>(a, stream) : launch_one<E, 64, false, true>(a, stream);
   }
+  if (a.ds && !seg)
+    return head_dim == 128 ? launch_one<E, 128, false, false, true>(a, stream)
+                           : launch_one<E, 64, false, false, true>(a, stream);
   if (head_dim == 128)
     return seg ? launch_one<E, 128, true, false>(a, stream) : launch_one<E, 128, false, false>(a, stream);
   return seg ? launch_one<E, 64, true, false>(a, stream) : launch_one<E, 64, false, false>(a, stream);

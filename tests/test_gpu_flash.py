@@ -803,10 +803,18 @@ def test_backward_without_saved_residuals_is_bit_identical():
 # ----------------------------------------------------------------------------- BASELINE sizes
 
 
-def _sampled_fwd_bwd_check(B, T, Hq, Hkv, D, mask, window, seg, samples, dq_rows):
+def _rel_ok(got, want):
+    """The relative-L2 arm of the bf16 bar alone: on late rows of a long sequence outputs and
+    gradients are small (rms ~ 0.03), so the max-abs arm would pass errors of tens of percent."""
+    return ref.rel_l2(got, want) <= BF16_REL_L2
+
+
+def _sampled_fwd_bwd_check(B, T, Hq, Hkv, D, mask, window, seg, samples, dq_rows, key_blocks=(), spill=True):
     """Full-size run on the GPU; the oracle checks sampled (batch, kv head) groups on query-row
-    windows (a causal row only needs the keys before it), and size-independent identities check
-    the rest: sum_s dV == sum_t dO and sum_s dK == 0 for every (batch, kv head)."""
+    windows (a causal row only needs the keys before it) and on key blocks (dK/dV of a key block
+    only needs the query rows that can see it, each with all the keys it normalises over), and
+    size-independent identities check the rest: sum_s dV == sum_t dO and sum_s dK == 0 for every
+    (batch, kv head)."""
     dev = "cuda"
     gen = torch.Generator(device=dev).manual_seed(0)
     mk = lambda h: torch.randn((B, T, h, D), device=dev, generator=gen).to(torch.bfloat16)
@@ -816,11 +824,30 @@ def _sampled_fwd_bwd_check(B, T, Hq, Hkv, D, mask, window, seg, samples, dq_rows
     _, kw = _mask_args(mask, window, segs)
     scale = D ** -0.5
     out, lse = ops.flash_fwd(q, k, v, softmax_scale=scale, **kw)
-    dq, dk, dv = ops.flash_bwd(q, k, v, out, lse, do, softmax_scale=scale, **kw)
+    dq, dk, dv = ops.flash_bwd(q, k, v, out, lse, do, softmax_scale=scale, spill=spill, **kw)
     torch.cuda.synchronize()
     G = Hq // Hkv
+    w = window if mask == "sliding" else None
     for (b, hk) in samples:
         hs = slice(hk * G, (hk + 1) * G)
+        for (k0, k1) in key_blocks:
+            # dK/dV of keys [k0, k1): contributions come from query rows [k0, r_hi) only, and those rows
+            # normalise over keys [s_lo, r_hi).
+            r_hi = T if w is None else min(T, k1 + w)
+            s_lo = 0 if w is None else max(0, k0 - w)
+            qs, dos = q[b:b + 1, k0:r_hi, hs].cpu(), do[b:b + 1, k0:r_hi, hs].cpu()
+            ks, vs = k[b:b + 1, s_lo:r_hi, hk:hk + 1].cpu(), v[b:b + 1, s_lo:r_hi, hk:hk + 1].cpu()
+            sub = ref.MaskSpec(**spec_kw, target_positions=torch.arange(k0, r_hi)[None],
+                               source_positions=torch.arange(s_lo, r_hi)[None])
+            if segs is not None:
+                keep = segs[b:b + 1, k0:r_hi, None] == segs[b:b + 1, None, s_lo:r_hi]
+                sub.dense_bias = ref.bool_to_bias(keep)[:, None]
+            _, wk, wv = ref.reference_mha_grads(qs, ks, vs, dos, sub, softmax_scale=scale, row_block=128)
+            sl = slice(k0 - s_lo, k1 - s_lo)
+            assert _rel_ok(dk[b:b + 1, k0:k1, hk:hk + 1].cpu(), wk[:, sl]), (
+                "dk", b, hk, k0, ref.rel_l2(dk[b:b + 1, k0:k1, hk:hk + 1].cpu(), wk[:, sl]))
+            assert _rel_ok(dv[b:b + 1, k0:k1, hk:hk + 1].cpu(), wv[:, sl]), (
+                "dv", b, hk, k0, ref.rel_l2(dv[b:b + 1, k0:k1, hk:hk + 1].cpu(), wv[:, sl]))
         for (r0, r1) in dq_rows:
             # Query rows [r0, r1) against keys [0, r1): exact for causal / sliding masks.
             qs, ks, vs = q[b:b + 1, r0:r1, hs].cpu(), k[b:b + 1, :r1, hk:hk + 1].cpu(), v[b:b + 1, :r1, hk:hk + 1].cpu()
@@ -832,10 +859,10 @@ def _sampled_fwd_bwd_check(B, T, Hq, Hkv, D, mask, window, seg, samples, dq_rows
                 keep = segs[b:b + 1, r0:r1, None] == segs[b:b + 1, None, :r1]
                 sub.dense_bias = ref.bool_to_bias(keep)[:, None]
             want = ref.reference_mha(qs, ks, vs, sub, softmax_scale=scale, row_block=128)
-            assert _ok_bf16(out[b:b + 1, r0:r1, hs].cpu(), want), ("out", b, hk, r0)
+            assert _rel_ok(out[b:b + 1, r0:r1, hs].cpu(), want), ("out", b, hk, r0)
             # dq of these rows only depends on these rows.
             wq, _, _ = ref.reference_mha_grads(qs, ks, vs, do[b:b + 1, r0:r1, hs].cpu(), sub, softmax_scale=scale, row_block=128)
-            assert _ok_bf16(dq[b:b + 1, r0:r1, hs].cpu(), wq), ("dq", b, hk, r0)
+            assert _rel_ok(dq[b:b + 1, r0:r1, hs].cpu(), wq), ("dq", b, hk, r0)
     # Identities over the whole tensors (fp32 sums of bf16 values).
     dv_sum = dv.float().sum(dim=1)                                   # [B, Hkv, D]
     do_sum = do.float().sum(dim=1).reshape(B, Hkv, G, D).sum(dim=2)
@@ -845,9 +872,14 @@ def _sampled_fwd_bwd_check(B, T, Hq, Hkv, D, mask, window, seg, samples, dq_rows
     return out, dq, dk, dv
 
 
-def test_baseline_c2_full_size():
+@pytest.mark.parametrize("spill", [True, False])
+def test_baseline_c2_full_size(spill):
+    """C2 at full size (32 (batch, kv head) pairs: the per-XCD grouped block order), through the
+    dS-workspace backward and through the one that recomputes dS for dq.  Key blocks: the first, one
+    in the middle and a late one that only 256 query rows see."""
     _sampled_fwd_bwd_check(4, 4096, 32, 8, 128, "causal", None, False,
-                           samples=[(0, 0), (3, 7)], dq_rows=[(0, 128), (1920, 2048), (3968, 4096)])
+                           samples=[(0, 0), (3, 7)], dq_rows=[(0, 128), (1920, 2048), (3968, 4096)],
+                           key_blocks=[(0, 128), (2048, 2176), (3840, 3968)], spill=spill)
 
 
 def test_baseline_c2_dkdv_sampled():
@@ -864,11 +896,27 @@ def test_baseline_c2_dkdv_sampled():
         _assert_close(name, got, want, torch.bfloat16)
 
 
+def _doc_boundary(seed, batch, seq_len, b):
+    """First position of row b's second document (or the middle of the row if it has one document)."""
+    ids = ref.packed_segment_ids(seed, batch, seq_len)[b]
+    change = torch.nonzero(ids[1:] != ids[:-1]).flatten()
+    return int(change[0]) + 1 if len(change) else seq_len // 2
+
+
 def test_baseline_c3_full_size():
-    _sampled_fwd_bwd_check(8, 8192, 16, 16, 128, "sliding", 4096, True,
-                           samples=[(0, 0), (5, 11)], dq_rows=[(0, 128), (4096, 4224), (8064, 8192)])
+    """C3 at full size (128 pairs).  Key blocks per sampled row: one that straddles a document
+    boundary, one whose last visible query rows sit at the window edge (key + 4096 < T), a late one."""
+    B, T = 8, 8192
+    for b, hk in ((0, 0), (5, 11)):
+        cut = _doc_boundary(4, B, T, b)
+        straddle = (cut // 128) * 128 if cut % 128 else cut - 64  # 128 keys with the boundary inside
+        straddle = max(0, min(T - 128, straddle))
+        _sampled_fwd_bwd_check(B, T, 16, 16, 128, "sliding", 4096, True, samples=[(b, hk)],
+                               dq_rows=[(0, 128), (4096, 4224), (8064, 8192)],
+                               key_blocks=[(straddle, straddle + 128), (1024, 1152), (7936, 8064)])
 
 
 def test_baseline_c5_full_size():
     _sampled_fwd_bwd_check(1, 32768, 64, 8, 128, "causal", None, False,
-                           samples=[(0, 3)], dq_rows=[(0, 128), (16384, 16512), (32640, 32768)])
+                           samples=[(0, 3)], dq_rows=[(0, 128), (16384, 16512), (32640, 32768)],
+                           key_blocks=[(32384, 32512), (32000, 32128)])
