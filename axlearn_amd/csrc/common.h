@@ -34,6 +34,14 @@ constexpr float kMasked = -__builtin_inff();
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
+// Exponent offset -lse * log2(e) of the backward kernels (p = exp2(s * c + offset)).  A query row with
+// no visible key leaves the forward with lse = -inf (and out = 0); its probabilities are all zero, so
+// the offset is a large negative number instead of +inf, which would turn s * c + offset into inf or,
+// for a masked s = -inf, NaN.
+__device__ __forceinline__ float lse_to_exp2_offset(float lse) {
+  return lse == -__builtin_inff() ? -1e30f : lse * -1.4426950408889634f;
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 

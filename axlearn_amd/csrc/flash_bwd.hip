@@ -61,7 +61,7 @@ __global__ __launch_bounds__(256) void bwd_delta_kernel(const BwdArgs a) {
   if (row < rows && sub == 0) {
     const int64_t idx = ((int64_t)b * a.Hq + h) * a.T + t;
     a.ndelta[idx] = -acc;
-    a.lse2[idx] = a.lse[idx] * (-kLog2e);
+    a.lse2[idx] = lse_to_exp2_offset(a.lse[idx]);
   }
 }
 
@@ -135,7 +135,7 @@ __global__ __launch_bounds__(256) void flash_bwd_dq_aux_kernel(const BwdArgs a) 
     dof[kk] = *(const bf16x8*)(dop + 16 * kk + 8 * g);
   }
   const int64_t stat_idx = ((int64_t)b * a.Hq + h) * a.T + q0 + l32;
-  const float lse2 = a.lse[stat_idx] * kLog2e;
+  const float lse2 = -lse_to_exp2_offset(a.lse[stat_idx]);
   const float delta = -a.ndelta[stat_idx];
 
   int k_begin = 0, k_end = a.S;

@@ -96,7 +96,7 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
       for (int i = 0; i < 4; i++) part = E::dot2(o.p[i], d.p[i], part);
     }
     delta = xor32_sum(part);
-    off = a.lse[stat_idx] * (-kLog2e);
+    off = lse_to_exp2_offset(a.lse[stat_idx]);
     if (live && g == 0) {
       a.ndelta[stat_idx] = -delta;
       a.lse2[stat_idx] = off;

@@ -800,6 +800,31 @@ def test_backward_without_saved_residuals_is_bit_identical():
             assert torch.equal(x, y)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_rows_without_a_visible_key(dtype):
+    """Causal rows at negative positions see no key: out = 0, lse = -inf, and the backward leaves dq of
+    those rows at zero and every gradient finite; the other rows match the oracle on the sub-problem
+    without the empty rows."""
+    b, t, hq, hkv, d, off = 2, 256, 4, 2, 128, -100
+    q, k, v, do = _inputs(b, t, hq, hkv, d, dtype)
+    kw = dict(softmax_scale=d ** -0.5, mask_kind=ops.MASK_CAUSAL, q_pos_offset=off)
+    out, lse = ops.flash_fwd(q.cuda(), k.cuda(), v.cuda(), **kw)
+    dq, dk, dv = ops.flash_bwd(q.cuda(), k.cuda(), v.cuda(), out, lse, do.cuda(), **kw)
+    e = -off
+    assert (out[:, :e] == 0).all() and torch.isinf(lse[:, :, :e]).all() and (lse[:, :, :e] < 0).all()
+    assert (dq[:, :e] == 0).all()
+    for x in (out, dq, dk, dv):
+        assert torch.isfinite(x.float()).all()
+    assert torch.isfinite(lse[:, :, e:]).all()
+    spec = ref.MaskSpec(causal=True, target_positions=torch.arange(t - e)[None], source_positions=torch.arange(t)[None])
+    want = ref.reference_mha(q[:, e:], k, v, spec, softmax_scale=d ** -0.5)
+    wq, wk, wv = ref.reference_mha_grads(q[:, e:], k, v, do[:, e:], spec, softmax_scale=d ** -0.5)
+    _assert_close("out", out[:, e:], want, dtype)
+    _assert_close("dq", dq[:, e:], wq, dtype)
+    _assert_close("dk", dk, wk, dtype)
+    _assert_close("dv", dv, wv, dtype)
+
+
 # ----------------------------------------------------------------------------- BASELINE sizes
 
 

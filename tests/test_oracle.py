@@ -379,6 +379,69 @@ def test_reconstruct_kv_loop():
                 assert torch.equal(got[bi, j, h], want)
 
 
+def test_reconstruct_kv_negative_and_out_of_pool_indices_loop():
+    """`pages.at[:, page_tables].get(mode="fill", fill_value=0)` (kv_cache/paged_kv_cache.py:32) is
+    jax.numpy indexing (jax 0.8.3, pyproject.toml:25; not under the reference tree): a signed index
+    is first normalised the numpy way, i + size if i < 0, and only what is still outside [0, size)
+    afterwards is out of bounds and reads the fill value.  Spelled out element by element."""
+    hkv, total, page, d, pps = 2, 5, 2, 3, 7
+    pages = torch.arange(1, 1 + hkv * total * page * d, dtype=torch.float32).reshape(hkv, total, page, d)
+    tables = torch.tensor([[-1, -5, -6, 4, 5, 0, -2], [2, -total, total, -total - 1, 1, -3, 3]], dtype=torch.int32)
+    got = ref.reconstruct_kv(tables, pages)
+    assert got.shape == (2, pps * page, hkv, d)
+    for bi in range(2):
+        for j in range(pps * page):
+            idx = int(tables[bi, j // page])
+            if idx < 0:
+                idx += total            # -1 is the last page, -total the first
+            for h in range(hkv):
+                if 0 <= idx < total:
+                    assert torch.equal(got[bi, j, h], pages[h, idx, j % page]), (bi, j, h)
+                else:                   # below -total or at / above total: the fill value
+                    assert torch.equal(got[bi, j, h], torch.zeros(d)), (bi, j, h)
+    # the entries above cover: wrap to the last / first page, one past either end, and plain indices
+    assert int((got == 0).all(dim=-1).sum()) == 4 * page * hkv
+
+
+def _bf16_round(x: float) -> float:
+    """Round-to-nearest-even of a double to bfloat16, by bit manipulation of its float32 pattern
+    (independent of torch's conversion)."""
+    import struct
+
+    bits = struct.unpack("<I", struct.pack("<f", x))[0]
+    bits = (bits + 0x7FFF + ((bits >> 16) & 1)) & 0xFFFF0000
+    return struct.unpack("<f", struct.pack("<I", bits))[0]
+
+
+def test_faithful_mode_rounding_points_by_hand():
+    """The "faithful" mode keeps ReferenceMHA's rounding points for bf16 inputs (q * scale in bf16,
+    flash_attention/common.py:505; logits in bf16, :510; fp32 softmax rounded back to bf16,
+    attention.py:604-625; context in bf16, common.py:519).  Two keys, head_dim 1, numbers chosen so
+    that every rounding point moves the result by more than a bf16 step: worked with python floats."""
+    import math
+
+    scale, q, k0, k1, v0, v1 = 0.3, 1.0, 100.0, 99.0, 1.0, 0.0
+    qs = _bf16_round(q * scale)                                         # 0.30078125
+    assert qs == 0.30078125
+    l0, l1 = _bf16_round(qs * k0), _bf16_round(qs * k1)                # 30.125, 29.75
+    assert (l0, l1) == (30.125, 29.75)
+    p0 = 1.0 / (1.0 + math.exp(l1 - l0))
+    p0r, p1r = _bf16_round(p0), _bf16_round(1.0 - p0)
+    want = _bf16_round(p0r * v0 + p1r * v1)                             # 0.59375
+    assert want == 0.59375
+    # what the result would be with the rounding of q * scale left out, for contrast
+    no_q_round = _bf16_round(_bf16_round(1.0 / (1.0 + math.exp(_bf16_round(0.3 * k1) - _bf16_round(0.3 * k0)))))
+    assert no_q_round == 0.5625 and no_q_round != want
+    qt = torch.tensor([[[[q]]]], dtype=torch.bfloat16)                 # [B=1, T=1, H=1, D=1]
+    kt = torch.tensor([[[[k0]], [[k1]]]], dtype=torch.bfloat16)        # [1, S=2, 1, 1]
+    vt = torch.tensor([[[[v0]], [[v1]]]], dtype=torch.bfloat16)
+    got = ref.reference_mha(qt, kt, vt, ref.MaskSpec(), softmax_scale=scale, mode="faithful")
+    assert got.dtype == torch.bfloat16 and float(got[0, 0, 0, 0]) == want
+    # the high-precision mode rounds nowhere: sigmoid(0.3) exactly
+    hp = ref.reference_mha(qt, kt, vt, ref.MaskSpec(), softmax_scale=scale)
+    assert abs(float(hp[0, 0, 0, 0]) - 1.0 / (1.0 + math.exp(-0.3))) < 1e-12
+
+
 def test_scatter_update_pages_loop():
     """The oracle's page insert against the element-wise loop documented in
     kv_cache/paged_kv_cache.py:156-165, with the GPU kernel's guards (paged_kv_cache_gpu_kernel.py:26,31):
