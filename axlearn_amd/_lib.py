@@ -18,7 +18,7 @@ LIB_PATH = os.path.join(_HERE, "libaxl_attn_hip.so")
 AXL_BF16, AXL_F32, AXL_F16 = 0, 1, 2
 MASK_NONE, MASK_CAUSAL, MASK_SLIDING_WINDOW = 0, 1, 2
 DECODE_DETERMINISTIC, DECODE_WORKSPACE_REUSED = 1, 2  # AXL_DECODE_* flags
-BWD_NO_SPILL = 1  # AXL_BWD_NO_SPILL
+BWD_DS_WORKSPACE = 1  # AXL_BWD_DS_WORKSPACE
 AXL_OK, AXL_ERR_INVALID_ARGUMENT, AXL_ERR_UNSUPPORTED, AXL_ERR_WORKSPACE, AXL_ERR_LAUNCH = 0, -1, -2, -3, -4
 
 
@@ -136,7 +136,6 @@ EXPORTED_SYMBOLS = (
     "axl_flash_bwd",
     "axl_flash_bwd_phases",
     "axl_flash_bwd_workspace_bytes",
-    "axl_flash_bwd_min_workspace_bytes",
     "axl_paged_decode",
     "axl_paged_decode_workspace_bytes",
     "axl_paged_decode_static",
@@ -183,7 +182,6 @@ def load() -> ctypes.CDLL:
     lib.axl_flash_bwd_phases.argtypes = [ctypes.POINTER(AxlFlashBwdParams), ctypes.c_int, ctypes.c_void_p]
     for name, ptype in (
         ("axl_flash_bwd_workspace_bytes", AxlFlashBwdParams),
-        ("axl_flash_bwd_min_workspace_bytes", AxlFlashBwdParams),
         ("axl_paged_decode_workspace_bytes", AxlPagedDecodeParams),
         ("axl_decode_workspace_bytes", AxlDecodeParams),
     ):

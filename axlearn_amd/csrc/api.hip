@@ -23,7 +23,6 @@ int set_error(int code, const char* fmt, ...) {
 int launch_flash_fwd(const AxlFlashFwdParams& p, hipStream_t stream);
 int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream);
 size_t flash_bwd_workspace_bytes(const AxlFlashBwdParams& p);
-size_t flash_bwd_min_workspace_bytes(const AxlFlashBwdParams& p);
 int launch_paged_decode(const AxlPagedDecodeParams& p, hipStream_t stream);
 size_t paged_decode_workspace_bytes(const AxlPagedDecodeParams& p);
 int launch_paged_decode_static(const AxlPagedDecodeParams& p, hipStream_t stream);
@@ -195,10 +194,6 @@ size_t axl_flash_bwd_workspace_bytes(const AxlFlashBwdParams* p) {
   return flash_bwd_workspace_bytes(*p);
 }
 
-size_t axl_flash_bwd_min_workspace_bytes(const AxlFlashBwdParams* p) {
-  if (!p) return 0;
-  return flash_bwd_min_workspace_bytes(*p);
-}
 
 int axl_flash_bwd(const AxlFlashBwdParams* p, void* stream) {
   return axl_flash_bwd_phases(p, AXL_BWD_DELTA | AXL_BWD_DKDV | AXL_BWD_DQ, stream);
@@ -230,11 +225,10 @@ int axl_flash_bwd_phases(const AxlFlashBwdParams* p, int phases, void* stream) {
   if (rc != AXL_OK) return rc;
   if (p->d_logit_sink && !p->logit_sink)
     return set_error(AXL_ERR_INVALID_ARGUMENT, "axl_flash_bwd: d_logit_sink without logit_sink");
-  const size_t need = flash_bwd_min_workspace_bytes(*p);
+  const size_t need = flash_bwd_workspace_bytes(*p);
   if (!p->workspace || p->workspace_bytes < need || (reinterpret_cast<uintptr_t>(p->workspace) & 255))
-    return set_error(AXL_ERR_WORKSPACE,
-                     "axl_flash_bwd: workspace needs at least %zu bytes, 256-byte aligned (got %zu)", need,
-                     p->workspace ? p->workspace_bytes : (size_t)0);
+    return set_error(AXL_ERR_WORKSPACE, "axl_flash_bwd: workspace needs %zu bytes, 256-byte aligned (got %zu)",
+                     need, p->workspace ? p->workspace_bytes : (size_t)0);
   return launch_flash_bwd(*p, phases, (hipStream_t)stream);
 }
 

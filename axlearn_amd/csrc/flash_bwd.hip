@@ -329,22 +329,15 @@ static size_t stats_bytes(const AxlFlashBwdParams& p) {
 static bool spill_eligible(const AxlFlashBwdParams& p) {
   return (p.dtype == AXL_BF16 || p.dtype == AXL_F16) && p.mask_kind == AXL_MASK_CAUSAL && p.q_pos_offset == 0 &&
          p.q_len == p.kv_len && !p.segment_ids && !p.aux.bias && !p.aux.dropout_mask &&
-         !(p.flags & AXL_BWD_NO_SPILL);
+         (p.flags & AXL_BWD_DS_WORKSPACE);
 }
 
 static size_t spill_bytes(const AxlFlashBwdParams& p) {
   return (size_t)p.batch * p.num_q_heads * (size_t)ds_blocks_per_head(p.q_len) * kDsBlockBytes;
 }
 
-// Above this size the dS workspace is not asked for (the caller can still pass one: a workspace that
-// holds it selects the spill path whatever its size).
-constexpr size_t kSpillAskCap = (size_t)8 << 30;
-
-size_t flash_bwd_min_workspace_bytes(const AxlFlashBwdParams& p) { return stats_bytes(p); }
-
 size_t flash_bwd_workspace_bytes(const AxlFlashBwdParams& p) {
-  if (spill_eligible(p) && spill_bytes(p) <= kSpillAskCap) return stats_bytes(p) + spill_bytes(p);
-  return stats_bytes(p);
+  return stats_bytes(p) + (spill_eligible(p) ? spill_bytes(p) : 0);
 }
 
 int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream) {
@@ -354,8 +347,7 @@ int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream)
   a.ndelta = (float*)p.workspace;
   a.lse2 = a.ndelta + (size_t)p.batch * p.num_q_heads * p.q_len;
   a.dq = p.dq; a.dk = p.dk; a.dv = p.dv; a.seg = p.segment_ids;
-  // A workspace that also holds dS selects the spill path.
-  const bool spill = spill_eligible(p) && p.workspace_bytes >= stats_bytes(p) + spill_bytes(p);
+  const bool spill = spill_eligible(p);  // the entry point has checked that the workspace holds dS as well
   a.ds = spill ? (char*)p.workspace + stats_bytes(p) : nullptr;
   a.qs = to_s3(p.q_strides); a.ks = to_s3(p.k_strides); a.vs = to_s3(p.v_strides);
   a.os = to_s3(p.out_strides); a.dos = to_s3(p.d_out_strides); a.dqs = to_s3(p.dq_strides);

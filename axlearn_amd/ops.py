@@ -203,7 +203,7 @@ def flash_bwd(
     bias: Optional[torch.Tensor] = None,
     dropout_mask: Optional[torch.Tensor] = None,
     dropout_rate: float = 0.0,
-    spill: bool = True,
+    ds_workspace: bool = False,
 ):
     """Returns (dq [B,T,Hq,D], dk [B,S,Hkv,D], dv [B,S,Hkv,D]) in the dtype of q, followed by
     d_logit_sink [Hq] fp32 when `logit_sink` (the one the forward was given) is passed.
@@ -211,8 +211,8 @@ def flash_bwd(
     `phases` selects a subset of {1: delta, 2: dK/dV, 4: dQ} (timing / profiling only); `buffers`
     = (dq, dk, dv, workspace) reuses caller-provided outputs instead of allocating.  bias,
     dropout_mask and dropout_rate must be the ones the forward was given (the bias gets no gradient,
-    as in gpu_attention.py:786).  `spill=False` (AXL_BWD_NO_SPILL) keeps the backward on the kernels
-    that recompute dS for dq even where the dS workspace would be used (plain causal attention)."""
+    as in gpu_attention.py:786).  `ds_workspace=True` (AXL_BWD_DS_WORKSPACE; plain causal attention
+    only, ignored otherwise) keeps dS in a larger workspace instead of recomputing it for dq."""
     b, t, hq, d, s, hkv = _check_qkv(q, k, v)
     _check_segment_ids(segment_ids, b, t, s)
     _want_shape("out", out, q.shape)
@@ -252,13 +252,13 @@ def flash_bwd(
         dtype=_lib.dtype_code(q.dtype), mask_kind=mask_kind, sliding_window=int(sliding_window),
         q_pos_offset=int(q_pos_offset), softmax_scale=float(softmax_scale),
         workspace=None, workspace_bytes=0, logit_sink=_lib.ptr(sink), d_logit_sink=_lib.ptr(d_sink),
-        aux=aux, flags=0 if spill else _lib.BWD_NO_SPILL,
+        aux=aux, flags=_lib.BWD_DS_WORKSPACE if ds_workspace else 0,
     )
+    need = int(lib.axl_flash_bwd_workspace_bytes(ctypes.byref(p)))
     if ws is None:
-        need = lib.axl_flash_bwd_workspace_bytes(ctypes.byref(p))
-        ws = torch.empty((max(int(need), 256),), dtype=torch.uint8, device=q.device)
-    elif ws.numel() * ws.element_size() < lib.axl_flash_bwd_min_workspace_bytes(ctypes.byref(p)):
-        raise AxlError(_lib.AXL_ERR_WORKSPACE, "buffers workspace is too small")
+        ws = torch.empty((max(need, 256),), dtype=torch.uint8, device=q.device)
+    elif ws.numel() * ws.element_size() < need:
+        raise AxlError(_lib.AXL_ERR_WORKSPACE, f"buffers workspace holds {ws.numel() * ws.element_size()} bytes, {need} needed")
     p.workspace = ws.data_ptr()
     p.workspace_bytes = ws.numel() * ws.element_size()
     _lib.check(lib.axl_flash_bwd_phases(ctypes.byref(p), int(phases), _lib.current_stream_ptr()))
@@ -268,28 +268,19 @@ def flash_bwd(
 
 
 def flash_bwd_buffers(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, mask_kind: int = MASK_NONE,
-                      spill: bool = True, workspace_bytes: Optional[int] = None, **_unused):
+                      ds_workspace: bool = False):
     """Pre-allocates (dq, dk, dv, workspace) for repeated `flash_bwd(..., buffers=...)` calls.
 
-    The workspace always holds delta and the scaled lse (fp32 [B,Hq,T] each).  For a plain causal
-    mask (`mask_kind=MASK_CAUSAL`, equal lengths, no offsets / segment ids / bias / dropout) and
-    `spill=True` it also holds dS, T*S bytes per (batch, head), up to the 8 GiB the library asks for;
-    `workspace_bytes` overrides the size (a workspace that holds dS selects that path at any size)."""
+    The workspace holds delta and the scaled lse (fp32 [B,Hq,T] each); with `ds_workspace=True` and
+    `mask_kind=MASK_CAUSAL` (equal lengths, no offsets / segment ids / bias / dropout) also dS, about
+    T*S bytes per (batch, head), for `flash_bwd(..., ds_workspace=True)`."""
     b, t, hq, d = q.shape
-    if workspace_bytes is None:
-        p = AxlFlashBwdParams(batch=b, q_len=t, kv_len=k.shape[1], num_q_heads=hq, num_kv_heads=k.shape[2],
-                              head_dim=d, dtype=_lib.dtype_code(q.dtype), mask_kind=mask_kind,
-                              flags=0 if spill else _lib.BWD_NO_SPILL)
-        workspace_bytes = int(_lib.load().axl_flash_bwd_workspace_bytes(ctypes.byref(p)))
-    ws = torch.empty((max(int(workspace_bytes), 256),), dtype=torch.uint8, device=q.device)
+    p = AxlFlashBwdParams(batch=b, q_len=t, kv_len=k.shape[1], num_q_heads=hq, num_kv_heads=k.shape[2],
+                          head_dim=d, dtype=_lib.dtype_code(q.dtype), mask_kind=mask_kind,
+                          flags=_lib.BWD_DS_WORKSPACE if ds_workspace else 0)
+    nbytes = int(_lib.load().axl_flash_bwd_workspace_bytes(ctypes.byref(p)))
+    ws = torch.empty((max(nbytes, 256),), dtype=torch.uint8, device=q.device)
     return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), ws
-
-
-def flash_bwd_spill_workspace_bytes(batch: int, q_len: int, num_q_heads: int) -> int:
-    """Bytes of a workspace that holds delta, the scaled lse and dS for plain causal attention."""
-    a = q_len // 128
-    stats = (2 * batch * num_q_heads * q_len * 4 + 255) // 256 * 256
-    return stats + batch * num_q_heads * 8 * a * (a + 1) * 2048
 
 
 def _decode_flags(deterministic: bool, workspace_reused: bool) -> int:

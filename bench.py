@@ -1,16 +1,24 @@
 """Benchmark of the MI355X attention kernel path (one GPU).
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c5] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|c1|c2|c3|c4|c5] [--no-cpu-baseline]
 
-Default workload (BASELINE.json configs[1], "C2"): causal GQA flash attention forward + backward,
-bf16, batch 4, 32 query heads / 8 kv heads, seq 4096, head_dim 128.  A step is one forward
+The headline workload (BASELINE.json configs[1], "C2") is causal GQA flash attention forward +
+backward, bf16, batch 4, 32 query heads / 8 kv heads, seq 4096, head_dim 128: a step is one forward
 (axl_flash_fwd) plus one backward (axl_flash_bwd) over one synthetic batch already resident in HBM.
 The paged-decode half of the metric (configs[3], "C4") is measured in the same run and reported in
-the `paged_decode` object of the same JSON line.
+the `paged_decode` object of the same JSON line.  With the default `--workload all` the line also
+carries `c1` (configs[0]: the fp32 case the reference itself runs on CPU), `c3` (sliding window +
+packed segments) and `c5` (one GPU's share of a 32768-token sequence), each with its own `roofline`
+and `cpu_baseline`.
+
+Inputs follow one seeding scheme, the same the parity tests use: numpy `default_rng(seed)`,
+`standard_normal` in fp32, rounded to the element type; q = seed 0, k = 1, v = 2, dO = 3, segment
+ids = 4, decode lengths = 5, page permutation = 6.
 
 Prints ONE JSON line.  `value` = algorithmic TFLOP/s of fwd+bwd (4*B*Hq*T^2*D/2 forward, 2.5x that
-backward).  `roofline` describes the dominant kernel (the dK/dV backward kernel), timed with device
-events around its own launches on the stream it runs on.  `cpu_baseline` times the CPU oracle
+backward; with segment ids the exact count of unmasked (query, key) pairs replaces T^2/2).
+`roofline` describes the dominant kernel (the dK/dV backward kernel), timed with device events
+around its own launches on the stream it runs on.  `cpu_baseline` times the CPU oracle
 (oracle/ref_attention.py, a restatement of the reference's XLA attention) on a bounded slice of the
 same workload on this machine's host cores.
 """
@@ -30,14 +38,34 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
+MFMA_F32_PEAK_TFLOPS = 157.3    # MI355X dense fp32 matrix
 HBM_PEAK_GBS = 8000.0           # MI355X HBM3E
 
-# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, in KiB; the
-# factors are what the same counters read for a plain 1 GiB copy kernel, `--calibrate-copy`).
-DKDV_TRAFFIC_BYTES = {"c2": 0.98e9}      # flash_bwd_dkdv_kernel<128>, workload c2
-DECODE_SPLIT_TRAFFIC_BYTES = 4.25e9      # decode_split_kernel<128,4>, workload c4
+# HBM bytes per launch of each workload's dominant kernel, measured with rocprofv3 --pmc (FETCH_SIZE x
+# 2.0 + WRITE_SIZE x 1.0, in KiB; the factors are what the same counters read for a plain 1 GiB copy
+# kernel, `--calibrate-copy`).  Constants from the committed profile named next to each: the run
+# that prints them does not read the counters itself.
+TRAFFIC = {
+    "c2": dict(bytes=None, source="profiles/flash_counters.md (flash_bwd_dkdv_kernel)"),
+    "c3": dict(bytes=None, source="profiles/flash_counters.md (flash_bwd_dkdv_kernel, segment ids)"),
+    "c5": dict(bytes=None, source="profiles/flash_counters.md (flash_bwd_dkdv_kernel)"),
+    "c4": dict(bytes=4.25e9, source="profiles/bench_c2_c4_counters.md (decode_split_kernel)"),
+}
 
 METRIC = "flash-attn fwd+bwd TFLOP/s; paged-decode HBM GB/s (% roofline), 1 MI355X"
+
+
+def normal_tensor(seed, shape, dtype, device):
+    """iid N(0,1) from numpy's default_rng(seed), generated in fp32, rounded to `dtype`, moved to the GPU
+    in slices (bounds the host staging buffer)."""
+    rng = np.random.default_rng(seed)
+    out = torch.empty(shape, dtype=dtype, device=device)
+    flat = out.view(-1)
+    n, step = flat.numel(), 1 << 26
+    for i in range(0, n, step):
+        m = min(step, n - i)
+        flat[i:i + m] = torch.from_numpy(rng.standard_normal(size=m, dtype=np.float32)).to(device).to(dtype)
+    return out
 
 
 def _events(n):
@@ -98,17 +126,21 @@ def count_pairs(seg, window):
     return total
 
 
+def _traffic(name):
+    t = TRAFFIC.get(name)
+    return (None, None) if t is None else (t["bytes"], t["source"])
+
+
 def bench_flash(cfg, steps, warmup, cpu_baseline):
     from axlearn_amd import ops
 
     dev = torch.device("cuda:0")
     B, T, Hq, Hkv, D = cfg["B"], cfg["T"], cfg["Hq"], cfg["Hkv"], cfg["D"]
-    gen = torch.Generator(device=dev).manual_seed(0)
     bf = torch.bfloat16
-    q = torch.randn((B, T, Hq, D), device=dev, dtype=torch.float32, generator=gen).to(bf)
-    k = torch.randn((B, T, Hkv, D), device=dev, dtype=torch.float32, generator=gen).to(bf)
-    v = torch.randn((B, T, Hkv, D), device=dev, dtype=torch.float32, generator=gen).to(bf)
-    do = torch.randn((B, T, Hq, D), device=dev, dtype=torch.float32, generator=gen).to(bf)
+    q = normal_tensor(0, (B, T, Hq, D), bf, dev)
+    k = normal_tensor(1, (B, T, Hkv, D), bf, dev)
+    v = normal_tensor(2, (B, T, Hkv, D), bf, dev)
+    do = normal_tensor(3, (B, T, Hq, D), bf, dev)
     seg = None
     pairs = None
     if cfg["seg"]:
@@ -116,19 +148,21 @@ def bench_flash(cfg, steps, warmup, cpu_baseline):
         pairs = count_pairs(seg, cfg["window"])
     mask_kind = {"none": ops.MASK_NONE, "causal": ops.MASK_CAUSAL, "sliding": ops.MASK_SLIDING_WINDOW}[cfg["mask"]]
     kw = dict(softmax_scale=D ** -0.5, mask_kind=mask_kind, sliding_window=cfg["window"], segment_ids=seg)
-    bufs = ops.flash_bwd_buffers(q, k, v)
+    spill = bool(cfg.get("ds_workspace"))
+    bufs = ops.flash_bwd_buffers(q, k, v, mask_kind=mask_kind, ds_workspace=spill)
+    kw_b = dict(kw, ds_workspace=spill)
     out, lse = ops.flash_fwd(q, k, v, **kw)
 
     def step():
         o, l = ops.flash_fwd(q, k, v, **kw)
-        ops.flash_bwd(q, k, v, o, l, do, buffers=bufs, **kw)
+        ops.flash_bwd(q, k, v, o, l, do, buffers=bufs, **kw_b)
 
     ms_step = _time_region(step, steps, warmup)
     # Per-kernel durations, each kernel timed over its own launches.
     ms_fwd = _time_region(lambda: ops.flash_fwd(q, k, v, **kw), steps, 1)
-    ms_delta = _time_region(lambda: ops.flash_bwd(q, k, v, out, lse, do, buffers=bufs, phases=1, **kw), steps, 1)
-    ms_dkdv = _time_region(lambda: ops.flash_bwd(q, k, v, out, lse, do, buffers=bufs, phases=2, **kw), steps, 1)
-    ms_dq = _time_region(lambda: ops.flash_bwd(q, k, v, out, lse, do, buffers=bufs, phases=4, **kw), steps, 1)
+    ms_delta = _time_region(lambda: ops.flash_bwd(q, k, v, out, lse, do, buffers=bufs, phases=1, **kw_b), steps, 1)
+    ms_dkdv = _time_region(lambda: ops.flash_bwd(q, k, v, out, lse, do, buffers=bufs, phases=2, **kw_b), steps, 1)
+    ms_dq = _time_region(lambda: ops.flash_bwd(q, k, v, out, lse, do, buffers=bufs, phases=4, **kw_b), steps, 1)
 
     if pairs is None:
         gemm = 2.0 * B * Hq * (T * T / 2.0) * D  # one [T,T,D] causal GEMM (the 1/2 convention)
@@ -137,27 +171,34 @@ def bench_flash(cfg, steps, warmup, cpu_baseline):
     fl_fwd, fl_bwd = 2 * gemm, 5 * gemm
     fl_dkdv, fl_dq = 4 * gemm, 1 * gemm           # S, dP, dV, dK | dQ
     tf = lambda fl, ms: fl / (ms * 1e-3) / 1e12
+    dq_name = "flash_bwd_dq_stream_kernel" if spill else "flash_bwd_dq_ring_kernel"
+    traffic, traffic_src = _traffic(cfg["name"])
     result = dict(
-        value=tf(fl_fwd + fl_bwd, ms_step), ms_per_step=ms_step,
+        workload=cfg["label"], value=tf(fl_fwd + fl_bwd, ms_step), unit="TFLOP/s", ms_per_step=ms_step,
+        backward="dS workspace: delta, dK/dV (stores dS), dq = dS k" if spill else "dQ (recomputes dS, computes delta), dK/dV",
         kernels={
             "flash_fwd_kernel": dict(ms=ms_fwd, tflops=tf(fl_fwd, ms_fwd), algorithmic_tflop=fl_fwd / 1e12),
-            "bwd_delta_kernel": dict(ms=ms_delta),
+            "bwd_delta_kernel": dict(ms=ms_delta, in_step=spill),
             "flash_bwd_dkdv_kernel": dict(ms=ms_dkdv, tflops=tf(fl_dkdv, ms_dkdv), algorithmic_tflop=fl_dkdv / 1e12),
-            "flash_bwd_dq_ring_kernel": dict(ms=ms_dq, tflops=tf(fl_dq, ms_dq), algorithmic_tflop=fl_dq / 1e12),
+            dq_name: dict(ms=ms_dq, tflops=tf(fl_dq, ms_dq), algorithmic_tflop=fl_dq / 1e12),
         },
         roofline=dict(
             kernel="flash_bwd_dkdv_kernel", bound="mfma", achieved=tf(fl_dkdv, ms_dkdv),
             peak=MFMA_BF16_PEAK_TFLOPS, unit="TFLOP/s", frac=tf(fl_dkdv, ms_dkdv) / MFMA_BF16_PEAK_TFLOPS,
-            traffic=DKDV_TRAFFIC_BYTES.get(cfg["name"]),
+            traffic=traffic, traffic_source=traffic_src,
         ),
         step_frac_of_mfma_peak=tf(fl_fwd + fl_bwd, ms_step) / MFMA_BF16_PEAK_TFLOPS,
     )
+    if pairs is not None:
+        result["unmasked_pairs"] = pairs
     if cpu_baseline:
         result["cpu_baseline"] = cpu_baseline_flash(cfg)
+    del q, k, v, do, out, lse, bufs
+    torch.cuda.empty_cache()
     return result
 
 
-def cpu_baseline_flash(cfg):
+def cpu_baseline_flash(cfg, budget_s=8.0):
     """Times the oracle's fwd+bwd (reverse-mode autodiff of the ReferenceMHA restatement, fp32 math
     on bf16-rounded inputs) on a slice of the workload: batch element 0, kv heads [0, nkv)."""
     from oracle import ref_attention as ref
@@ -181,7 +222,7 @@ def cpu_baseline_flash(cfg):
         ref.reference_mha_grads(q, k, v, do, spec, softmax_scale=D ** -0.5, row_block=512, dtype=torch.float32)
         reps += 1
         dt = time.perf_counter() - t0
-        if dt > 12.0 or reps >= 64:
+        if dt > budget_s or reps >= 64:
             break
     pairs = ref.count_unmasked_pairs(spec, 1, t_cap, t_cap) if cfg["seg"] else t_cap * t_cap / 2.0
     flops = 7.0 * 2.0 * (nkv * G) * pairs * D  # fwd (2 GEMMs) + bwd (5 GEMMs), algorithmic
@@ -192,6 +233,49 @@ def cpu_baseline_flash(cfg):
     )
 
 
+def bench_c1(steps, warmup, cpu_baseline):
+    """C1 (configs[0]): causal MHA forward, fp32, B2 H4 T512 D64, scale 1/8.  The CPU oracle is the
+    subject (timed in full); the fp32 forward kernel is timed, and checked against it, beside it."""
+    from axlearn_amd import ops
+
+    dev = torch.device("cuda:0")
+    B, T, H, D = 2, 512, 4, 64
+    q, k, v = (normal_tensor(s, (B, T, H, D), torch.float32, dev) for s in (0, 1, 2))
+    kw = dict(softmax_scale=0.125, mask_kind=ops.MASK_CAUSAL)
+    ms = _time_region(lambda: ops.flash_fwd(q, k, v, **kw), max(steps, 50), warmup)
+    flops = 4.0 * B * H * T * T * D / 2.0
+    tfl = flops / (ms * 1e-3) / 1e12
+    res = dict(
+        workload="C1: causal MHA forward, fp32, B2 H4 T512 D64", value=tfl, unit="TFLOP/s", ms_per_step=ms,
+        algorithmic_gflop=flops / 1e9,
+        roofline=dict(kernel="flash_fwd_f32_kernel", bound="mfma", achieved=tfl, peak=MFMA_F32_PEAK_TFLOPS,
+                      unit="TFLOP/s", frac=tfl / MFMA_F32_PEAK_TFLOPS, traffic=None,
+                      traffic_source="not measured: 32 workgroups, 0.27 GFLOP, bound by launch latency"),
+    )
+    if cpu_baseline:
+        from oracle import ref_attention as ref
+
+        cores = min(os.cpu_count() or 1, 16)
+        torch.set_num_threads(cores)
+        qc, kc, vc = q.cpu(), k.cpu(), v.cpu()
+        spec = ref.MaskSpec(causal=True)
+        want = ref.reference_mha(qc, kc, vc, spec, softmax_scale=0.125)
+        t0 = time.perf_counter()
+        reps = 0
+        while time.perf_counter() - t0 < 2.0:
+            ref.reference_mha(qc, kc, vc, spec, softmax_scale=0.125, mode="faithful")
+            reps += 1
+        dt = time.perf_counter() - t0
+        out, _ = ops.flash_fwd(q, k, v, **kw)
+        res["max_abs_vs_oracle"] = float((out.cpu().double() - want.double()).abs().max())
+        res["cpu_baseline"] = dict(
+            value=flops * reps / dt / 1e12, unit="TFLOP/s", ms_per_step=dt / reps * 1e3, cores=cores, kind="port",
+            sample=f"oracle ReferenceMHA restatement (fp32, the reference's rounding points), the whole of C1, "
+                   f"{reps} repetitions in {dt:.1f} s",
+        )
+    return res
+
+
 def bench_paged_decode(steps, warmup, cpu_baseline):
     """C4: B64, Hq32/Hkv8, D128, page 16, pool of 64*2048 pages, lengths U[512, 32768]."""
     from axlearn_amd import ops
@@ -199,14 +283,10 @@ def bench_paged_decode(steps, warmup, cpu_baseline):
     dev = torch.device("cuda:0")
     B, Hq, Hkv, D, page, pps = 64, 32, 8, 128, 16, 2048
     P = B * pps
-    gen = torch.Generator(device=dev).manual_seed(1)
     bf = torch.bfloat16
-    kp = torch.empty((Hkv, P, page, D), device=dev, dtype=bf)
-    vp = torch.empty((Hkv, P, page, D), device=dev, dtype=bf)
-    for h in range(Hkv):  # generate per head to bound the fp32 staging buffer
-        kp[h] = torch.randn((P, page, D), device=dev, dtype=torch.float32, generator=gen).to(bf)
-        vp[h] = torch.randn((P, page, D), device=dev, dtype=torch.float32, generator=gen).to(bf)
-    q = torch.randn((B, Hq, D), device=dev, dtype=torch.float32, generator=gen).to(bf)
+    kp = normal_tensor(1, (Hkv, P, page, D), bf, dev)
+    vp = normal_tensor(2, (Hkv, P, page, D), bf, dev)
+    q = normal_tensor(0, (B, Hq, D), bf, dev)
     lengths_cpu = torch.from_numpy(np.random.default_rng(5).integers(512, 32769, size=B).astype(np.int32))
     tables_cpu = torch.from_numpy(np.random.default_rng(6).permutation(P).astype(np.int32)).reshape(B, pps)
     lengths, tables = lengths_cpu.to(dev), tables_cpu.to(dev)
@@ -223,11 +303,12 @@ def bench_paged_decode(steps, warmup, cpu_baseline):
     # Algorithmic bytes: every live K and V page once, its page-table entry, q and out.
     algo_bytes = live_pages * page * Hkv * D * 2 * 2 + live_pages * 4 + 2 * B * Hq * D * 2
     gbs = algo_bytes / (ms * 1e-3) / 1e9
+    traffic, traffic_src = _traffic("c4")
     res = dict(
         workload="C4: paged decode, bf16, B64 Hq32/Hkv8 D128, page 16, ctx U[512,32768]",
         value=gbs, unit="GB/s", ms_per_step=ms, algorithmic_gb=algo_bytes / 1e9,
         roofline=dict(kernel="decode_split_kernel", bound="hbm", achieved=gbs, peak=HBM_PEAK_GBS, unit="GB/s",
-                      frac=gbs / HBM_PEAK_GBS, traffic=DECODE_SPLIT_TRAFFIC_BYTES),
+                      frac=gbs / HBM_PEAK_GBS, traffic=traffic, traffic_source=traffic_src),
     )
     if cpu_baseline:
         from oracle import ref_attention as ref
@@ -246,6 +327,8 @@ def bench_paged_decode(steps, warmup, cpu_baseline):
             sample=f"oracle ReferenceMHA restatement (page gather + dense attention) on sequences 0..{nb - 1}, {dt:.2f} s",
         )
         del kc, vc
+    del kp, vp
+    torch.cuda.empty_cache()
     return res
 
 
@@ -254,7 +337,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c2", choices=["c2", "c3", "c4", "c5"])
+    ap.add_argument("--workload", default="all", choices=["all", "c1", "c2", "c3", "c4", "c5"],
+                    help="all: headline C2 + C4, with C1, C3 and C5 as extra keys of the same line")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true", help="skip the paged-decode half of the metric")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -285,19 +369,35 @@ def main():
         if "cpu_baseline" in dec:
             line["cpu_baseline"] = dec["cpu_baseline"]
         line["paged_decode"] = dec
+    elif args.workload == "c1":
+        res = bench_c1(args.steps, args.warmup, cpu_base)
+        line.update(value=res["value"], unit="TFLOP/s", ms_per_step=res["ms_per_step"], dtype="f32",
+                    config=dict(workload=res["workload"]), roofline=res["roofline"])
+        if "cpu_baseline" in res:
+            line["cpu_baseline"] = res["cpu_baseline"]
+        line["c1"] = res
     else:
-        cfg = _flash_workload(args.workload)
+        cfg = _flash_workload("c2" if args.workload == "all" else args.workload)
         res = bench_flash(cfg, args.steps, args.warmup, cpu_base)
         line.update(value=res["value"], unit="TFLOP/s", ms_per_step=res["ms_per_step"],
                     config=dict(workload=cfg["label"], batch=cfg["B"], seq_len=cfg["T"], num_q_heads=cfg["Hq"],
                                 num_kv_heads=cfg["Hkv"], head_dim=cfg["D"], mask=cfg["mask"], window=cfg["window"],
-                                segment_ids=cfg["seg"]),
+                                segment_ids=cfg["seg"], backward=res["backward"]),
                     roofline=res["roofline"], kernels=res["kernels"],
                     step_frac_of_mfma_peak=res["step_frac_of_mfma_peak"])
+        if "unmasked_pairs" in res:
+            line["unmasked_pairs"] = res["unmasked_pairs"]
         if "cpu_baseline" in res:
             line["cpu_baseline"] = res["cpu_baseline"]
         if not args.no_decode:
             line["paged_decode"] = bench_paged_decode(args.steps, args.warmup, cpu_base)
+        if args.workload == "all":
+            # The other BASELINE configs, fewer repetitions: they are reported, not the headline.
+            # The same C2 step through the backward that keeps dS in a workspace (AXL_BWD_DS_WORKSPACE).
+            line["c2_ds_workspace"] = bench_flash(dict(cfg, ds_workspace=True), args.steps, args.warmup, False)
+            line["c1"] = bench_c1(args.steps, args.warmup, cpu_base)
+            line["c3"] = bench_flash(_flash_workload("c3"), max(5, args.steps // 2), 2, cpu_base)
+            line["c5"] = bench_flash(_flash_workload("c5"), max(3, args.steps // 4), 1, cpu_base)
     print(json.dumps(line))
 
 

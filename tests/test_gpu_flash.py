@@ -825,6 +825,36 @@ def test_rows_without_a_visible_key(dtype):
     _assert_close("dv", dv, wv, dtype)
 
 
+@pytest.mark.parametrize("b,t,hq,hkv,d,dtype", [
+    (1, 256, 4, 2, 128, torch.bfloat16), (2, 512, 8, 2, 128, torch.bfloat16), (1, 1024, 4, 1, 64, torch.bfloat16),
+    (2, 384, 6, 6, 128, torch.float16), (8, 1152, 8, 2, 128, torch.bfloat16), (3, 640, 10, 5, 64, torch.float16),
+])
+def test_ds_workspace_backward_matches_oracle(b, t, hq, hkv, d, dtype):
+    """The backward that keeps dS in the workspace (AXL_BWD_DS_WORKSPACE): dq, dk, dv against the
+    oracle, dv bit-identical to the recompute path's (same arithmetic up to dS), also with a logit sink."""
+    q, k, v, do = _inputs(b, t, hq, hkv, d, dtype)
+    spec = ref.MaskSpec(causal=True)
+    scale = d ** -0.5
+    sink = torch.linspace(-1.0, 1.0, hq)
+    for sk in (None, sink):
+        kw = dict(softmax_scale=scale, mask_kind=ops.MASK_CAUSAL, logit_sink=None if sk is None else sk.cuda())
+        out, lse = ops.flash_fwd(q.cuda(), k.cuda(), v.cuda(), **kw)
+        got = ops.flash_bwd(q.cuda(), k.cuda(), v.cuda(), out, lse, do.cuda(), ds_workspace=True, **kw)
+        base = ops.flash_bwd(q.cuda(), k.cuda(), v.cuda(), out, lse, do.cuda(), **kw)
+        want = ref.reference_mha_grads(q, k, v, do, spec, softmax_scale=scale, logit_sink=sk)
+        for name, x, w in zip(("dq", "dk", "dv"), got, want):
+            _assert_close(name, x, w, dtype)
+        assert torch.equal(got[2], base[2])
+        if sk is not None:
+            assert ref.max_abs(got[3].cpu(), want[3]) <= 2e-2 * max(1.0, float(want[3].abs().max()))
+    # the flag is ignored where the path does not apply (here: a sliding window)
+    kw = dict(softmax_scale=scale, mask_kind=ops.MASK_SLIDING_WINDOW, sliding_window=100)
+    out, lse = ops.flash_fwd(q.cuda(), k.cuda(), v.cuda(), **kw)
+    a = ops.flash_bwd(q.cuda(), k.cuda(), v.cuda(), out, lse, do.cuda(), ds_workspace=True, **kw)
+    c = ops.flash_bwd(q.cuda(), k.cuda(), v.cuda(), out, lse, do.cuda(), **kw)
+    assert all(torch.equal(x, y) for x, y in zip(a, c))
+
+
 # ----------------------------------------------------------------------------- BASELINE sizes
 
 
@@ -834,7 +864,7 @@ def _rel_ok(got, want):
     return ref.rel_l2(got, want) <= BF16_REL_L2
 
 
-def _sampled_fwd_bwd_check(B, T, Hq, Hkv, D, mask, window, seg, samples, dq_rows, key_blocks=(), spill=True):
+def _sampled_fwd_bwd_check(B, T, Hq, Hkv, D, mask, window, seg, samples, dq_rows, key_blocks=(), ds_workspace=False):
     """Full-size run on the GPU; the oracle checks sampled (batch, kv head) groups on query-row
     windows (a causal row only needs the keys before it) and on key blocks (dK/dV of a key block
     only needs the query rows that can see it, each with all the keys it normalises over), and
@@ -849,7 +879,7 @@ def _sampled_fwd_bwd_check(B, T, Hq, Hkv, D, mask, window, seg, samples, dq_rows
     _, kw = _mask_args(mask, window, segs)
     scale = D ** -0.5
     out, lse = ops.flash_fwd(q, k, v, softmax_scale=scale, **kw)
-    dq, dk, dv = ops.flash_bwd(q, k, v, out, lse, do, softmax_scale=scale, spill=spill, **kw)
+    dq, dk, dv = ops.flash_bwd(q, k, v, out, lse, do, softmax_scale=scale, ds_workspace=ds_workspace, **kw)
     torch.cuda.synchronize()
     G = Hq // Hkv
     w = window if mask == "sliding" else None
@@ -897,14 +927,14 @@ def _sampled_fwd_bwd_check(B, T, Hq, Hkv, D, mask, window, seg, samples, dq_rows
     return out, dq, dk, dv
 
 
-@pytest.mark.parametrize("spill", [True, False])
-def test_baseline_c2_full_size(spill):
+@pytest.mark.parametrize("ds_workspace", [False, True])
+def test_baseline_c2_full_size(ds_workspace):
     """C2 at full size (32 (batch, kv head) pairs: the per-XCD grouped block order), through the
-    dS-workspace backward and through the one that recomputes dS for dq.  Key blocks: the first, one
+    backward that recomputes dS for dq and through the one that keeps dS in the workspace.  Key blocks: the first, one
     in the middle and a late one that only 256 query rows see."""
     _sampled_fwd_bwd_check(4, 4096, 32, 8, 128, "causal", None, False,
                            samples=[(0, 0), (3, 7)], dq_rows=[(0, 128), (1920, 2048), (3968, 4096)],
-                           key_blocks=[(0, 128), (2048, 2176), (3840, 3968)], spill=spill)
+                           key_blocks=[(0, 128), (2048, 2176), (3840, 3968)], ds_workspace=ds_workspace)
 
 
 def test_baseline_c2_dkdv_sampled():

@@ -340,15 +340,14 @@ def test_abi_validation_without_gpu():
                                 kv_len=256, num_q_heads=4, num_kv_heads=2, head_dim=128, dtype=0, mask_kind=1,
                                 sliding_window=0, q_pos_offset=0, softmax_scale=1.0, workspace=256, workspace_bytes=16)
     stats = 2 * (2 * 4 * 256 * 4)  # delta and scaled lse, fp32 [B, Hq, T] each
-    assert lib.axl_flash_bwd_min_workspace_bytes(ctypes.byref(bp)) == stats
-    # plain causal attention: the dS workspace on top, A = T / 128 = 2 -> 8 A (A + 1) blocks of 2 KB per head
-    assert lib.axl_flash_bwd_workspace_bytes(ctypes.byref(bp)) == stats + 2 * 4 * 48 * 2048
-    bp.flags = _lib.BWD_NO_SPILL
     assert lib.axl_flash_bwd_workspace_bytes(ctypes.byref(bp)) == stats
-    bp.flags = 0
-    bp.mask_kind = 2  # a sliding window has no dS workspace
+    # plain causal attention with the dS workspace: A = T / 128 = 2 -> 8 A (A + 1) blocks of 2 KB per head
+    bp.flags = _lib.BWD_DS_WORKSPACE
+    assert lib.axl_flash_bwd_workspace_bytes(ctypes.byref(bp)) == stats + 2 * 4 * 48 * 2048
+    bp.mask_kind = 2  # a sliding window has no dS workspace: the flag is ignored
     assert lib.axl_flash_bwd_workspace_bytes(ctypes.byref(bp)) == stats
     bp.mask_kind = 1
+    bp.flags = 0
     assert lib.axl_flash_bwd(ctypes.byref(bp), None) == _lib.AXL_ERR_WORKSPACE
     assert lib.axl_flash_bwd_phases(ctypes.byref(bp), 0, None) == _lib.AXL_ERR_INVALID_ARGUMENT
     # Paged decode geometry.
