@@ -1,0 +1,254 @@
+"""JAX side of the XLA FFI binding (csrc/ffi_shim.cc): what an AXLearn maintainer adds next to
+axlearn/common/flash_attention/gpu_attention.py to put the HIP kernels behind
+`flash_attention_implementation`.
+
+This module needs jax and the FFI library `libaxl_attn_ffi.so` (built from csrc/ffi_shim.cc against
+jaxlib's `xla/ffi/api/ffi.h`).  Neither exists in this repository's environment, so nothing here is
+imported by the package or exercised by its tests: it is the source of the reference-side binding,
+kept next to the torch host mirror (`hip_attention.py`, `hip_decoding.py`) whose behaviour it repeats
+call for call.
+
+It mirrors, name for name:
+  * `flash_attention` with its `jax.custom_vjp` and residuals `(q, k, v, bias, segment_ids, prng_key,
+    out, lse)` (gpu_attention.py:247-287, :420-424, :789): `out` and `lse` carry
+    `checkpoint_name(..., f"gpu_attention.{FLASH_ATTN_RESIDUAL_NAME}")`, the name the remat policy
+    `save_and_offload_only_these_names_regex` matches (axlearn/common/flash_attention/remat.py:9-58);
+  * `PallasGPUFlashAttention` (gpu_attention.py:929-992) as `HipFlashAttention`, `GPUDecoding`
+    (gpu_decoding.py:286-352) as `HipDecoding`, `GPUPagedAttention` (gpu_paged_attention.py:299-379)
+    as `HipPagedAttention`, to be listed first in `BACKENDS["gpu"]` / `PAGED_ATTN_BACKENDS["gpu"]`
+    (flash_attention/utils.py:31-58);
+  * `gpu_scatter_update_pages_shmap_fn` (kv_cache/paged_kv_cache_gpu_kernel.py:36-60) as
+    `hip_scatter_update_pages`.
+"""
+
+# pylint: disable=import-error,too-many-arguments
+from __future__ import annotations
+
+import ctypes
+import functools
+import os
+
+import jax
+import jax.numpy as jnp
+import numpy as np
+from jax.ad_checkpoint import checkpoint_name
+
+from axlearn.common.attention_bias import (  # the reference's own types: this file lives in its tree
+    BaseAttentionBias,
+    CausalAttentionBias,
+    MaskFnAttentionBias,
+    SegmentIdAttentionBias,
+    SlidingWindowAttentionBias,
+    split,
+)
+from axlearn.common.flash_attention.common import (
+    BaseFlashAttention,
+    BasePagedAttention,
+    BaseSingleStepDecoding,
+    repeat_kv_heads,  # noqa: F401  (NOT used: K/V go to the kernels with their own Hkv heads)
+)
+from axlearn.common.flash_attention.remat import FLASH_ATTN_RESIDUAL_NAME
+from axlearn.common.utils import Nested, Tensor
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_FFI_LIB = ctypes.CDLL(os.path.join(_HERE, "..", "libaxl_attn_ffi.so"))
+_CORE_LIB = ctypes.CDLL(os.path.join(_HERE, "..", "libaxl_attn_hip.so"))
+
+for _name in ("AxlFlashFwd", "AxlFlashBwd", "AxlDecode", "AxlPagedDecode", "AxlPagedKvInsert"):
+    jax.ffi.register_ffi_target(_name, jax.ffi.pycapsule(getattr(_FFI_LIB, _name)), platform="ROCM")
+
+MASK_NONE, MASK_CAUSAL, MASK_SLIDING_WINDOW = 0, 1, 2
+DECODE_DETERMINISTIC = 1
+
+
+def _empty(dtype) -> Tensor:
+    """Stand-in for an absent optional operand (XLA FFI has no optional buffers)."""
+    return jnp.zeros((0,), dtype)
+
+
+def _mask_of(bias: BaseAttentionBias):
+    """(mask_kind, window, segment_ids, dense bias or None): the structured parts the kernels evaluate
+    arithmetically, as `PallasGPUFlashAttention.__call__` splits them (gpu_attention.py:972-974)."""
+    mask, segment_ids, explicit = split(bias, MaskFnAttentionBias, SegmentIdAttentionBias)
+    kind, window = MASK_NONE, 0
+    if isinstance(mask, SlidingWindowAttentionBias):
+        kind, window = MASK_SLIDING_WINDOW, int(mask.sliding_window_size)
+    elif isinstance(mask, CausalAttentionBias):
+        kind = MASK_CAUSAL
+    elif mask.has_value():
+        explicit = explicit + mask  # an arbitrary mask_fn: materialised as a bias, once
+    seg = segment_ids.segment_ids if segment_ids.has_value() else None
+    return kind, window, seg, (explicit.value() if explicit.has_value() else None)
+
+
+def _bwd_workspace_bytes(b, t, s, hq, hkv, d, dtype_code, mask_kind, has_seg, flags) -> int:
+    """axl_flash_bwd_workspace_bytes for these shapes (a host-side size query of the core library)."""
+    from axlearn_amd._lib import AxlFlashBwdParams  # the ctypes mirror of include/axl_attn.h
+
+    p = AxlFlashBwdParams(batch=b, q_len=t, kv_len=s, num_q_heads=hq, num_kv_heads=hkv, head_dim=d,
+                          dtype=dtype_code, mask_kind=mask_kind, segment_ids=1 if has_seg else None, flags=flags)
+    _CORE_LIB.axl_flash_bwd_workspace_bytes.restype = ctypes.c_size_t
+    return int(_CORE_LIB.axl_flash_bwd_workspace_bytes(ctypes.byref(p)))
+
+
+_DTYPE_CODE = {jnp.dtype(jnp.bfloat16): 0, jnp.dtype(jnp.float32): 1, jnp.dtype(jnp.float16): 2}
+
+
+@functools.partial(jax.custom_vjp, nondiff_argnums=(6, 7, 8, 9, 10))
+def flash_attention(query, key, value, bias, segment_ids, dropout_mask, softmax_scale, mask_kind,
+                    sliding_window, dropout_rate, logit_sink_present):
+    """Same contract as gpu_attention.py:250-287 with the block-size / warp arguments gone (the kernels
+    pick their own tiles) and the dropout mask instead of the prng key (drawn by the caller with
+    `jax.random.bernoulli(prng_key, dropout_rate, [B,H,T,S])`, as :374-385 does before its kernel)."""
+    del logit_sink_present
+    out, _ = _fwd_call(query, key, value, bias, segment_ids, dropout_mask, None, softmax_scale, mask_kind,
+                       sliding_window, dropout_rate)
+    return out
+
+
+def _fwd_call(query, key, value, bias, segment_ids, dropout_mask, logit_sink, softmax_scale, mask_kind,
+              sliding_window, dropout_rate, q_pos_offsets=None):
+    b, t, hq, _ = query.shape
+    out_type = jax.ShapeDtypeStruct(query.shape, query.dtype)
+    lse_type = jax.ShapeDtypeStruct((b, hq, t), jnp.float32)
+    return jax.ffi.ffi_call("AxlFlashFwd", (out_type, lse_type))(
+        query, key, value,
+        _empty(jnp.int32) if segment_ids is None else segment_ids.astype(jnp.int32),
+        _empty(jnp.float32) if logit_sink is None else logit_sink.astype(jnp.float32),
+        _empty(jnp.float32) if bias is None else bias,
+        _empty(jnp.uint8) if dropout_mask is None else dropout_mask.astype(jnp.uint8),
+        _empty(jnp.int32) if q_pos_offsets is None else q_pos_offsets.astype(jnp.int32),
+        softmax_scale=np.float32(softmax_scale), mask_kind=np.int32(mask_kind),
+        sliding_window=np.int32(sliding_window), q_pos_offset=np.int32(0), dropout_rate=np.float32(dropout_rate))
+
+
+def _flash_fwd(query, key, value, bias, segment_ids, dropout_mask, softmax_scale, mask_kind, sliding_window,
+               dropout_rate, logit_sink_present):
+    del logit_sink_present
+    out, lse = _fwd_call(query, key, value, bias, segment_ids, dropout_mask, None, softmax_scale, mask_kind,
+                         sliding_window, dropout_rate)
+    # The names the remat policy looks for (remat.py:13-58): saving or offloading exactly these two
+    # tensors lets the backward skip the forward kernel.
+    out = checkpoint_name(out, f"gpu_attention.{FLASH_ATTN_RESIDUAL_NAME}")
+    lse = checkpoint_name(lse, f"gpu_attention.{FLASH_ATTN_RESIDUAL_NAME}")
+    return out, (query, key, value, bias, segment_ids, dropout_mask, out, lse)
+
+
+def _flash_bwd(softmax_scale, mask_kind, sliding_window, dropout_rate, logit_sink_present, res, d_out):
+    del logit_sink_present
+    query, key, value, bias, segment_ids, dropout_mask, out, lse = res
+    b, t, hq, d = query.shape
+    s, hkv = key.shape[1], key.shape[2]
+    flags = 0
+    ws_bytes = _bwd_workspace_bytes(b, t, s, hq, hkv, d, _DTYPE_CODE[jnp.dtype(query.dtype)], mask_kind,
+                                    segment_ids is not None, flags)
+    dq, dk, dv, _, _ = jax.ffi.ffi_call(
+        "AxlFlashBwd",
+        (jax.ShapeDtypeStruct(query.shape, query.dtype), jax.ShapeDtypeStruct(key.shape, key.dtype),
+         jax.ShapeDtypeStruct(value.shape, value.dtype), jax.ShapeDtypeStruct((0,), jnp.float32),
+         jax.ShapeDtypeStruct((ws_bytes,), jnp.uint8)),
+    )(query, key, value, out, d_out, lse,
+      _empty(jnp.int32) if segment_ids is None else segment_ids.astype(jnp.int32), _empty(jnp.float32),
+      _empty(jnp.float32) if bias is None else bias,
+      _empty(jnp.uint8) if dropout_mask is None else dropout_mask.astype(jnp.uint8),
+      softmax_scale=np.float32(softmax_scale), mask_kind=np.int32(mask_kind), sliding_window=np.int32(sliding_window),
+      q_pos_offset=np.int32(0), dropout_rate=np.float32(dropout_rate), flags=np.int32(flags))
+    # No gradient for bias, segment ids or the dropout mask, as `_mha_backward` returns (:786).
+    return dq, dk, dv, None, None, None
+
+
+flash_attention.defvjp(_flash_fwd, _flash_bwd)
+
+
+class HipFlashAttention(BaseFlashAttention):
+    """Stands where `PallasGPUFlashAttention` does (gpu_attention.py:929-992)."""
+
+    def is_supported(self, input_batch: Nested[Tensor | BaseAttentionBias], kv_cache_type=None) -> bool:
+        if not super().is_supported(input_batch=input_batch, kv_cache_type=kv_cache_type):
+            return False
+        query, key = input_batch["query"], input_batch["key"]
+        if query.dtype not in (jnp.bfloat16, jnp.float16, jnp.float32) or key.dtype != query.dtype:
+            return self._log_unsupported(f"{query.dtype=} / {key.dtype=}")
+        if not self._check_block_size(input_batch=input_batch, block_size=128):
+            return False
+        if query.shape[-1] not in (64, 128):
+            return self._log_unsupported(f"head_dim {query.shape[-1]} (supported: 64, 128)")
+        return True
+
+    @functools.partial(jax.jit, static_argnames=["self"])
+    def __call__(self, input_batch: Nested[Tensor | BaseAttentionBias]) -> Tensor:
+        cfg = self.config
+        query, key, value = input_batch["query"], input_batch["key"], input_batch["value"]
+        mask_kind, window, segment_ids, dense = _mask_of(input_batch["bias"])
+        dropout_mask = None
+        if cfg.dropout_rate > 0.0:
+            b, t, hq, _ = query.shape
+            dropout_mask = jax.random.bernoulli(input_batch["prng_key"], cfg.dropout_rate, (b, hq, t, key.shape[1]))
+        # K / V keep their Hkv heads: no repeat_kv_heads (gpu_attention.py:975-976 repeats them).
+        return flash_attention(query, key, value, dense, segment_ids, dropout_mask, cfg.softmax_scale, mask_kind,
+                               window, cfg.dropout_rate, False)
+
+
+def _lengths(bias: BaseAttentionBias, batch: int) -> Tensor:
+    mask, _ = split(bias, MaskFnAttentionBias)
+    if mask is None or mask.target_positions is None:
+        raise ValueError("Cannot retrieve MaskFnAttentionBias or target_positions.")
+    return jnp.broadcast_to(mask.target_positions[:, -1] + 1, (batch,)).astype(jnp.int32)  # gpu_decoding.py:314
+
+
+def _decode_window(bias: BaseAttentionBias) -> int:
+    kind, window, _, _ = _mask_of(bias)
+    return window if kind == MASK_SLIDING_WINDOW else -1
+
+
+class HipDecoding(BaseSingleStepDecoding):
+    """Stands where `GPUDecoding` does (gpu_decoding.py:286-352)."""
+
+    @functools.partial(jax.jit, static_argnames=["self"])
+    def __call__(self, input_batch: Nested[Tensor | BaseAttentionBias]) -> Tensor:
+        query, key, value = input_batch["query"], input_batch["key"], input_batch["value"]
+        b, _, hq, d = query.shape
+        ws = _decode_workspace_bytes(b, hq, key.shape[2], d, key.shape[1])
+        out, _ = jax.ffi.ffi_call(
+            "AxlDecode", (jax.ShapeDtypeStruct((b, hq, d), query.dtype), jax.ShapeDtypeStruct((ws,), jnp.uint8)),
+        )(query.reshape(b, hq, d), key, value, _lengths(input_batch["bias"], b),
+          softmax_scale=np.float32(self.config.softmax_scale), sliding_window=np.int32(_decode_window(input_batch["bias"])),
+          flags=np.int32(0))
+        return out.reshape(b, 1, hq, d)
+
+
+class HipPagedAttention(BasePagedAttention):
+    """Stands where `GPUPagedAttention` does (gpu_paged_attention.py:299-379)."""
+
+    @functools.partial(jax.jit, static_argnames=["self"])
+    def __call__(self, input_batch: Nested[Tensor | BaseAttentionBias]) -> Tensor:
+        query, key, value = input_batch["query"], input_batch["key"], input_batch["value"]
+        page_tables = input_batch["page_tables"]
+        b, _, hq, d = query.shape
+        ws = _decode_workspace_bytes(b, hq, key.shape[0], d, page_tables.shape[1] * key.shape[2])
+        out, _ = jax.ffi.ffi_call(
+            "AxlPagedDecode", (jax.ShapeDtypeStruct((b, hq, d), query.dtype), jax.ShapeDtypeStruct((ws,), jnp.uint8)),
+        )(query.reshape(b, hq, d), key, value, page_tables.astype(jnp.int32), _lengths(input_batch["bias"], b),
+          softmax_scale=np.float32(self.config.softmax_scale), sliding_window=np.int32(_decode_window(input_batch["bias"])),
+          flags=np.int32(0))
+        return out.reshape(b, 1, hq, d)
+
+
+def _decode_workspace_bytes(b, hq, hkv, d, kv_len) -> int:
+    from axlearn_amd._lib import AxlDecodeParams
+
+    p = AxlDecodeParams(batch=b, kv_len=kv_len, num_q_heads=hq, num_kv_heads=hkv, head_dim=d, dtype=0)
+    _CORE_LIB.axl_decode_workspace_bytes.restype = ctypes.c_size_t
+    return int(_CORE_LIB.axl_decode_workspace_bytes(ctypes.byref(p)))  # same size rule as the paged entry point
+
+
+def hip_scatter_update_pages(k_pages: Tensor, v_pages: Tensor, k_proj: Tensor, v_proj: Tensor,
+                             page_indices: Tensor, key_positions: Tensor):
+    """`gpu_scatter_update_pages_shmap_fn` (paged_kv_cache_gpu_kernel.py:36-60) for the K and the V pool
+    in one call; pools [Hkv,P,page,D], projections [Hkv,B,1,D].  The pools are donated and updated in
+    place (`input_output_aliases`, as :57).  Returns the updated (k_pages, v_pages)."""
+    return jax.ffi.ffi_call(
+        "AxlPagedKvInsert",
+        (jax.ShapeDtypeStruct(k_pages.shape, k_pages.dtype), jax.ShapeDtypeStruct(v_pages.shape, v_pages.dtype)),
+        input_output_aliases={0: 0, 1: 1},
+    )(k_pages, v_pages, k_proj, v_proj, page_indices.astype(jnp.int32), key_positions.reshape(-1).astype(jnp.int32))

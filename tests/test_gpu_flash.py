@@ -855,6 +855,52 @@ def test_ds_workspace_backward_matches_oracle(b, t, hq, hkv, d, dtype):
     assert all(torch.equal(x, y) for x, y in zip(a, c))
 
 
+def test_layer_compute_attention_end_to_end():
+    """The layer-level calling sequence (layer.py:218-376) over the HIP kernels: bias cast to the query
+    dtype, softmax_scale 1.0 by default with the scale folded into q beforehand, `(context, probs)` with
+    probs a shape without contents, prefill and both decode paths, autograd through the context."""
+    from axlearn_amd.flash_attention.layer import FlashAttention
+    from axlearn_amd.kv_cache import KVCache, PagedKVCache
+
+    b, t, hq, hkv, d = 2, 256, 8, 2, 128
+    q, k, v, do = _inputs(b, t, hq, hkv, d, torch.bfloat16)
+    scale = d ** -0.5
+    q_scaled = (q.float() * scale).to(torch.bfloat16)   # `scale_query` happens before the layer calls the kernels
+    pos = dict(target_positions=torch.arange(t)[None], source_positions=torch.arange(t)[None])
+    bias = ab.CompositeAttentionBias([ab.CausalAttentionBias(**pos)])
+    layer = FlashAttention.default_config().instantiate()
+    qd, kd, vd = (x.cuda().requires_grad_(True) for x in (q_scaled, k, v))
+    ctx, probs = layer.compute_attention(q_proj=qd, k_proj=kd, v_proj=vd, attention_logit_biases=bias)
+    assert probs.device.type == "meta" and tuple(probs.shape) == (b, hq, t, t)
+    spec = ref.MaskSpec(causal=True)
+    want = ref.reference_mha(q_scaled, k, v, spec, softmax_scale=1.0)
+    _assert_close("context", ctx, want, torch.bfloat16)
+    ctx.backward(do.cuda())
+    wq, wk, wv = ref.reference_mha_grads(q_scaled, k, v, do, spec, softmax_scale=1.0)
+    _assert_close("dq", qd.grad, wq, torch.bfloat16)
+    _assert_close("dk", kd.grad, wk, torch.bfloat16)
+    _assert_close("dv", vd.grad, wv, torch.bfloat16)
+    # an explicit softmax_scale is passed through
+    layer2 = FlashAttention.default_config().set(softmax_scale=scale).instantiate()
+    ctx2, _ = layer2.compute_attention(q_proj=q.cuda(), k_proj=k.cuda(), v_proj=v.cuda(), attention_logit_biases=bias)
+    _assert_close("context (scale in the kernel)", ctx2, ref.reference_mha(q, k, v, spec, softmax_scale=scale), torch.bfloat16)
+    # decode: contiguous cache, then paged pools with page_indices
+    qq, kp, vp, tables, lengths = ref.paged_inputs(5, batch=3, num_heads=hq, num_kv_heads=hkv, head_dim=d, page_size=16,
+                                                   pages_per_seq=8, min_len=10, max_len=128)
+    dbias = ab.CompositeAttentionBias([ab.CausalAttentionBias(
+        target_positions=(lengths.long() - 1)[:, None], source_positions=torch.arange(128)[None])])
+    want_d = ref.reference_decode(qq, kp, vp, lengths, softmax_scale=1.0, page_tables=tables)
+    got_p, probs_p = layer.compute_attention(q_proj=qq.cuda(), k_proj=kp.cuda(), v_proj=vp.cuda(),
+                                             attention_logit_biases=dbias, page_indices=tables.cuda(),
+                                             kv_cache_type=PagedKVCache)
+    assert tuple(probs_p.shape) == (3, hq, 1, 128)
+    _assert_close("paged decode", got_p, want_d, torch.bfloat16)
+    kk, vv = ref.reconstruct_kv(tables, kp), ref.reconstruct_kv(tables, vp)
+    got_c, _ = layer.compute_attention(q_proj=qq.cuda(), k_proj=kk.cuda(), v_proj=vv.cuda(),
+                                       attention_logit_biases=dbias, kv_cache_type=KVCache)
+    _assert_close("contiguous decode", got_c, want_d, torch.bfloat16)
+
+
 # ----------------------------------------------------------------------------- BASELINE sizes
 
 

@@ -416,3 +416,63 @@ def test_ops_reject_mismatched_shapes_before_any_launch():
     assert "v" in str(raises(ops.decode, dq, kc, kc[:, :100], lengths))
     assert "lengths" in str(raises(ops.decode, dq, kc, kc, lengths[:1]))
     assert "GPU" in str(raises(ops.decode, dq, kc, kc, lengths))
+
+
+def test_config_modifiers_rewrite_every_flash_config_in_a_tree():
+    """FlashBlockSizeModifier / BackendOverrideModifier (layer.py:434-496): every FlashAttention config in
+    the tree is rewritten; overrides are merged, falsy override values are not inserted."""
+    import dataclasses
+
+    from axlearn_amd.flash_attention.layer import BackendOverrideModifier, FlashAttention, FlashBlockSizeModifier
+
+    @dataclasses.dataclass
+    class Layer:
+        attention: object
+        other: int = 3
+
+    @dataclasses.dataclass
+    class Model:
+        layers: list
+        extra: dict
+
+    a = FlashAttention.default_config()
+    b = FlashAttention.default_config().set(backend_overrides=dict(save_residuals=True))
+    c = FlashAttention.default_config()
+    model = Model(layers=[Layer(a), Layer(b)], extra=dict(decoder=(Layer(c),), n=1))
+    out = FlashBlockSizeModifier.default_config().set(tpu_block_size=1024, gpu_block_size=64).instantiate()(model)
+    assert out is model
+    for cfg in (a, b, c):
+        assert (cfg.tpu_block_size, cfg.gpu_block_size) == (1024, 64)
+    mod = BackendOverrideModifier.default_config().set(
+        backend_overrides=dict(splash_block_q=2048, save_residuals=None)).instantiate()
+    mod(model)
+    assert a.backend_overrides == dict(splash_block_q=2048)
+    assert b.backend_overrides == dict(save_residuals=True, splash_block_q=2048)   # merged, None not inserted
+    BackendOverrideModifier.default_config().instantiate()(model)                  # no overrides: nothing changes
+    assert c.backend_overrides == dict(splash_block_q=2048)
+
+
+def test_layer_falls_back_when_no_kernel_supports_the_request():
+    """`compute_attention` (layer.py:218-376): the bias reaches the dispatch cast to the query dtype
+    (:253); when no kernel accepts the request (here: tensors on the CPU) the caller's standard attention
+    runs with the ORIGINAL projections and the cast bias (:278-285); without one the call raises."""
+    from axlearn_amd.flash_attention.layer import FlashAttention
+
+    t = 128
+    q = torch.zeros((1, t, 2, 64), dtype=torch.bfloat16)
+    k = torch.zeros((1, t, 2, 64), dtype=torch.bfloat16)
+    pos = dict(target_positions=torch.arange(t)[None], source_positions=torch.arange(t)[None])
+    bias = ab.CompositeAttentionBias([ab.CausalAttentionBias(**pos)])
+    assert bias.dtype is None
+    layer = FlashAttention.default_config().instantiate()
+    seen = {}
+
+    def standard_attention(**kw):
+        seen.update(kw)
+        return "context", "probs"
+
+    assert layer.compute_attention(q_proj=q, k_proj=k, v_proj=k, attention_logit_biases=bias,
+                                   fallback=standard_attention) == ("context", "probs")
+    assert seen["q_proj"] is q and seen["k_proj"] is k and seen["attention_logit_biases"].dtype == torch.bfloat16
+    with pytest.raises(NotImplementedError):
+        layer.compute_attention(q_proj=q, k_proj=k, v_proj=k, attention_logit_biases=bias)
