@@ -439,6 +439,12 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
 #pragma unroll
     for (int i = 0; i < kAheadB; i++) AXL_B_READ_FROM(buf_b, bfr_next[i], i)
   }
+  // On every path into the loops below, including the one around the block above, nothing the
+  // compiler tracks is pending any more.  Without this its wait-count pass carries the loads of the
+  // stationary K / V fragments into the loop and covers each fragment's first use there with a
+  // vmcnt wait, down to vmcnt(0): every iteration would then wait for the tile loads it has just
+  // issued, which the pass cannot see and which are meant to stay in flight for two more iterations.
+  wait_all_vmem();
 
   const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   // Iterations [j_from, j_to); MASKED_C says whether their elementwise tiles (j + 1) need mask
