@@ -77,6 +77,24 @@ struct ElemBf16 {
   static __device__ __forceinline__ floatx16 mfma_32x32x16(bf16x8 a, bf16x8 b, floatx16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
+  // The same instruction with its accumulator in VECTOR registers whatever form the compiler picks
+  // for the function's other MFMAs (inline assembly; `_zero` starts a chain from 0).  For chains whose
+  // result vector ALU code reads: in a kernel compiled with accumulators in AGPRs that saves one
+  // v_accvgpr_read per element.  The compiler does not know what the assembly is, so the CALLER keeps
+  // the distance the hardware wants between the last MFMA of a chain and the first vector ALU read of
+  // its result (12 wait states for this 8-pass MFMA; two later MFMAs in between are enough, the matrix
+  // pipe takes them one after the other), and keeps register pressure low enough that the compiler
+  // has no reason to copy the accumulator elsewhere right after the chain.  `_last` ends a chain whose
+  // result is read right away: the wait states are part of the same statement.
+  static __device__ __forceinline__ void mfma_32x32x16_vgpr(bf16x8 a, bf16x8 b, floatx16& c) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void mfma_32x32x16_vgpr_last(bf16x8 a, bf16x8 b, floatx16& c) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0\n\ts_nop 15\n\ts_nop 3" : "+v"(c) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void mfma_32x32x16_vgpr_zero(bf16x8 a, bf16x8 b, floatx16& c) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
+  }
   static __device__ __forceinline__ floatx4 mfma_16x16x32(bf16x8 a, bf16x8 b, floatx4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
   }
@@ -95,6 +113,15 @@ struct ElemF16 {
   static __device__ __forceinline__ floatx16 mfma_32x32x16(bf16x8 a, bf16x8 b, floatx16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, a), __builtin_bit_cast(halfx8, b), c,
                                                   0, 0, 0);
+  }
+  static __device__ __forceinline__ void mfma_32x32x16_vgpr(bf16x8 a, bf16x8 b, floatx16& c) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(c) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void mfma_32x32x16_vgpr_last(bf16x8 a, bf16x8 b, floatx16& c) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0\n\ts_nop 15\n\ts_nop 3" : "+v"(c) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void mfma_32x32x16_vgpr_zero(bf16x8 a, bf16x8 b, floatx16& c) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(c) : "v"(a), "v"(b));
   }
   static __device__ __forceinline__ floatx4 mfma_16x16x32(bf16x8 a, bf16x8 b, floatx4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(halfx8, a), __builtin_bit_cast(halfx8, b), c,

@@ -234,12 +234,16 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
   // that is not an MFMA - elementwise arithmetic, operand packing, LDS fragment reads, tile load
   // requests, pointer updates - is dealt out over the MFMA slots of the iteration, so the matrix
   // pipe never waits for it.
-  floatx16 s_e, dp_e;          // tile j + 1: logits / dP, then P / dS
+  // Two register sets that swap roles from iteration to iteration, so nothing is copied: in an
+  // iteration one holds tile j + 1 (logits / dP, turned into P / dS) and tile j's packed operands,
+  // the other receives the stage-A accumulators of tile j + 2 and tile j + 1's packed operands.
+  // (s_e, dp_e, pb, dsb) is the first kind on entry to every run of iterations.
+  floatx16 s_e, dp_e, s_x, dp_x;
   union PackedOperand {
     bf16x8 v[2];
     bf16x2 p[8];
   };
-  PackedOperand pb, dsb;       // tile j: P and dS as MFMA operands
+  PackedOperand pb, dsb, pb_x, dsb_x;
 #pragma unroll
   for (int r = 0; r < 16; r++) s_e[r] = dp_e[r] = 0.f;
 
@@ -334,8 +338,16 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
   _Pragma("unroll") for (int kk = 0; kk < KK; kk++) {                                           \
     const bf16x8 qa_ = AXL_A_FRAG(BUF_, 0, kk);                                                 \
     const bf16x8 da_ = AXL_A_FRAG(BUF_, 1, kk);                                                 \
-    S_ = E::mfma_32x32x16(qa_, kf[kk], S_);                     \
-    DP_ = E::mfma_32x32x16(da_, vf[kk], DP_);                   \
+    if constexpr (AUX) {                                                                        \
+      S_ = E::mfma_32x32x16(qa_, kf[kk], S_);                                                   \
+      DP_ = E::mfma_32x32x16(da_, vf[kk], DP_);                                                 \
+    } else if (kk + 1 < KK) {                                                                   \
+      E::mfma_32x32x16_vgpr(qa_, kf[kk], S_);                                                   \
+      E::mfma_32x32x16_vgpr(da_, vf[kk], DP_);                                                  \
+    } else {                                                                                    \
+      E::mfma_32x32x16_vgpr_last(qa_, kf[kk], S_);                                              \
+      E::mfma_32x32x16_vgpr_last(da_, vf[kk], DP_);                                             \
+    }                                                                                           \
   }
   union TrFrag {
     bf16x8 v;
@@ -452,14 +464,19 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
   // inside one loop.
   auto run = [&](int j_from, int j_to, auto masked_c) __attribute__((always_inline)) {
     constexpr bool MASKED = decltype(masked_c)::value;
-  for (int j = j_from; j < j_to; j++) {
+  // One iteration.  (s_e, dp_e): tile j + 1; (pb, dsb): tile j, packed; (s_a, dp_a): the stage-A
+  // accumulators of tile j + 2; (pb_n, dsb_n): tile j + 1, packed as its elements complete.
+  // Without a bias / dropout mask the stage-A chains accumulate in vector registers
+  // (mfma_32x32x16_vgpr): the next iteration's elementwise stage reads them where they are.  Its first
+  // read of s comes after that iteration's first MFMA and after the last MFMA of the dP chain, its
+  // first read of dp two slots later.  The bias / dropout instantiations, which run out of vector
+  // registers, keep the compiler's own form.
+  auto iter = [&](floatx16& s_e, floatx16& dp_e, PackedOperand& pb, PackedOperand& dsb, floatx16& s_a, floatx16& dp_a,
+                  PackedOperand& pb_n, PackedOperand& dsb_n) __attribute__((always_inline)) {
     bf16x8 afr[NA];
     TrFrag bfr[NB];
 #pragma unroll
     for (int i = 0; i < kAheadB; i++) bfr[i] = bfr_next[i];
-    floatx16 s_a, dp_a;
-    floatx16 dp_start = zero16;          // first operand of the dP chain: -delta without a dropout mask
-    PackedOperand pb_n, dsb_n;           // tile j + 1, packed as its elements complete
     int q0_p = q0_s2, h_p = h_s2;
     const unsigned lds_s = lds_address(buf_s2);
     const char* a_ad[KK];                // this iteration's fragment addresses: stage A in tile j+2,
@@ -517,11 +534,18 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
           dk_acc[dt] = E::mfma_32x32x16(bfr[n].v, dsb.v[t8], dk_acc[dt]);
       } else {
         constexpr int x = n - NB;
-        if constexpr (x % 2 == 0)
-          s_a = E::mfma_32x32x16(afr[x], kf[x / 2], x == 0 ? zero16 : s_a);
-        else
-          dp_a = E::mfma_32x32x16(afr[x], vf[x / 2], x == 1 ? dp_start : dp_a);
+        if constexpr (AUX) {
+          if constexpr (x % 2 == 0) s_a = E::mfma_32x32x16(afr[x], kf[x / 2], x == 0 ? zero16 : s_a);
+          else dp_a = E::mfma_32x32x16(afr[x], vf[x / 2], x == 1 ? zero16 : dp_a);
+        } else {
+          if constexpr (x == 0) E::mfma_32x32x16_vgpr_zero(afr[x], kf[x / 2], s_a);
+          else if constexpr (x % 2 == 0) E::mfma_32x32x16_vgpr(afr[x], kf[x / 2], s_a);
+          else E::mfma_32x32x16_vgpr(afr[x], vf[x / 2], dp_a);  // the chain starts from -delta
+        }
       }
+      // The first elementwise read of (s_e, dp_e) stays behind this slot's MFMA: two MFMAs then lie
+      // between it and the last MFMA of the S chain, whatever the barrier in between took.
+      if constexpr (n == 0) __builtin_amdgcn_sched_barrier(0);
       // ---- elementwise stage of tile j+1: element e starts in slot e (NS-3)/16 and takes three
       // slots; pairs are packed one slot after their second element is complete
 #pragma unroll
@@ -555,10 +579,11 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
         if constexpr (AUX) {
           if (n == (4 * i + 3) * (NS - 3) / 16 + 3) del_v[i] = *(const floatx4*)(st_ + Tile::BQ * 4);
         } else {
-          // -delta of tile j+2's rows: what its dP chain starts from (slot NB + 1)
+          // -delta of tile j+2's rows: what its dP chain starts from (slot NB + 1), loaded into the
+          // accumulator itself (the register set is idle until then)
           if (n == NB - 4 + i) {
             const floatx4 d4 = *(const floatx4*)(st_ + Tile::BQ * 4);
-            dp_start[4 * i] = d4[0]; dp_start[4 * i + 1] = d4[1]; dp_start[4 * i + 2] = d4[2]; dp_start[4 * i + 3] = d4[3];
+            dp_a[4 * i] = d4[0]; dp_a[4 * i + 1] = d4[1]; dp_a[4 * i + 2] = d4[2]; dp_a[4 * i + 3] = d4[3];
           }
         }
       }
@@ -581,10 +606,6 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
     buf_n = buf_s;
     buf_s = buf_s2;
     buf_s2 = tmp;
-    s_e = s_a;
-    dp_e = dp_a;
-    pb = pb_n;
-    dsb = dsb_n;
     if constexpr (AUX) {
 #pragma unroll
       for (int r = 0; r < 16; r++) {
@@ -599,7 +620,21 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
     h_a = h_s;
     h_s = h_s2;
     h_s2 = h_p;
-  }
+  };
+    int j = j_from;
+    for (; j + 1 < j_to; j += 2) {
+      iter(s_e, dp_e, pb, dsb, s_x, dp_x, pb_x, dsb_x);
+      iter(s_x, dp_x, pb_x, dsb_x, s_e, dp_e, pb, dsb);
+    }
+    if (j < j_to) {
+      // odd count: one more iteration, then the sets go back to their roles with one copy per run
+      iter(s_e, dp_e, pb, dsb, s_x, dp_x, pb_x, dsb_x);
+      if constexpr (!AUX) asm volatile("s_nop 15\n\ts_nop 3" : "+v"(s_x), "+v"(dp_x));  // the chains have just ended
+      s_e = s_x;
+      dp_e = dp_x;
+      pb = pb_x;
+      dsb = dsb_x;
+    }
   };
   // Query tile t (counted from t_begin) needs no mask for this wavefront's 32 keys when its queries
   // all see them: t in [u_lo, u_hi].  In processing order tile number e is query tile nt - 1 - e / G
