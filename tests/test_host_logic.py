@@ -476,3 +476,36 @@ def test_layer_falls_back_when_no_kernel_supports_the_request():
     assert seen["q_proj"] is q and seen["k_proj"] is k and seen["attention_logit_biases"].dtype == torch.bfloat16
     with pytest.raises(NotImplementedError):
         layer.compute_attention(q_proj=q, k_proj=k, v_proj=k, attention_logit_biases=bias)
+
+
+def test_dkdv_kernel_keeps_its_vector_register_accumulators_in_place():
+    """The plain dK/dV instantiations accumulate S and dP in vector registers through inline-assembly
+    MFMAs, whose hazards the compiler does not see: their correctness rests on the compiler not copying
+    those registers right after a chain.  It has no reason to while nothing spills, so a build whose
+    plain instantiations use AGPRs for anything but the dK / dV accumulators (head_dim of them), or
+    scratch memory, fails here rather than on the GPU."""
+    import re
+    import shutil
+    import subprocess
+
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("hipcc not available")
+    csrc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "axlearn_amd", "csrc")
+    cmd = [hipcc, "-O3", "-std=c++17", "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang",
+           "-packed-fp32-ops", "-Wno-unused-value", "-Wno-unknown-attributes", "--cuda-device-only", "-S",
+           "-Rpass-analysis=kernel-resource-usage", "-o", os.devnull, os.path.join(csrc, "flash_bwd_dkdv.hip")]
+    out = subprocess.run(cmd, capture_output=True, text=True, cwd=csrc, timeout=600)
+    assert out.returncode == 0, out.stderr[-2000:]
+    seen = 0
+    for block in out.stderr.split("Function Name: ")[1:]:
+        name = block.split()[0]
+        m = re.match(r"_ZN3axl21flash_bwd_dkdv_kernelINS_\d+Elem\w+ELi(\d+)ELb([01])ELb([01])ELb([01])EEE", name)
+        if not m or m.group(3) == "1":  # other kernels; bias / dropout instantiations use the compiler's own form
+            continue
+        agprs = int(re.search(r"AGPRs: (\d+)", block).group(1))
+        scratch = int(re.search(r"ScratchSize \[bytes/lane\]: (\d+)", block).group(1))
+        assert agprs == int(m.group(1)), f"{name}: {agprs} AGPRs"
+        assert scratch == 0, f"{name}: scratch {scratch}"
+        seen += 1
+    assert seen == 12  # {bf16, f16} x {64, 128} x {plain, segment ids, dS workspace}
