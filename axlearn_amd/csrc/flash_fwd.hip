@@ -41,16 +41,20 @@ struct FwdArgs {
   float scale;
 };
 
-template <int D>
+// NW wavefronts of 32 query rows each.  The kernels are launched with 4 (two workgroups per CU); 8
+// (one workgroup per CU, twice as many query rows sharing every K / V tile that comes in from L2) was
+// measured and is not used: -4 % on causal MHA at 8192 tokens, +1 to +3 % on the GQA and windowed shapes.
+template <int D, int NW = 4>
 struct FwdTile {
-  static constexpr int BQ = 128;              // query rows per workgroup
+  static constexpr int BQ = 32 * NW;          // query rows per workgroup
   static constexpr int BK = 64;               // keys per LDS tile
   static constexpr int ROWB = D * 2;          // bytes per K / V row in LDS: unpadded
   static constexpr int TILE_BYTES = BK * ROWB;
   static constexpr int NSEG = 4;              // ring of segment-id rows (a tile's ids outlive its K buffer)
   static constexpr int SEG_BASE = 4 * TILE_BYTES;            // {K, V} x double buffer, then the ids
   static constexpr int LDS_BYTES = SEG_BASE + NSEG * BK * 4;
-  static constexpr int DMA_PER_WAVE = TILE_BYTES / 1024 / 4;  // direct-to-LDS loads per wavefront per tile
+  static constexpr int WROWS = BK / NW;       // tile rows that one wavefront fetches
+  static constexpr int DMA_PER_WAVE = TILE_BYTES / 1024 / NW;  // direct-to-LDS loads per wavefront per tile
   // Tiles arrive by direct global->LDS loads: unpadded rows, chunks XOR-swizzled (tile_swizzle).
   __device__ static __forceinline__ int swz(int row) { return tile_swizzle<D>(row); }
 };
@@ -58,10 +62,10 @@ struct FwdTile {
 constexpr int kMaxSegTiles = 1024;               // key tiles whose segment ids the forward classifies
 constexpr int kSegNotUniform = -0x7fffffff - 1;  // marks a tile with more than one segment id
 
-template <typename E, int D, bool AUX>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+template <typename E, int D, bool AUX, int NW = 4>
+__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void flash_fwd_kernel(const FwdArgs a) {
-  using Tile = FwdTile<D>;
+  using Tile = FwdTile<D, NW>;
   constexpr int KK = D / 16;  // MFMA k-steps over head_dim
   constexpr int DT = D / 32;  // 32-row output tiles over head_dim
   constexpr int CPR = D / 8;  // 16-byte chunks per row
@@ -73,7 +77,7 @@ void flash_fwd_kernel(const FwdArgs a) {
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l32 = lane & 31, g = lane >> 5;
   int qb, b, h;
-  decode_block(blockIdx.x, a.T / Tile::BQ, a.B, a.Hq, a.Hkv, 64, qb, b, h);
+  decode_block(blockIdx.x, a.T / Tile::BQ, a.B, a.Hq, a.Hkv, 256 / NW, qb, b, h);
   const int hk = h / (a.Hq / a.Hkv);
   const int q_off = a.q_off + (a.q_offs ? a.q_offs[b] : 0);  // position of this sequence's query row 0
   const int q0_wg = qb * Tile::BQ;
@@ -102,7 +106,7 @@ void flash_fwd_kernel(const FwdArgs a) {
   // all 32 queries of a wavefront carry needs no segment mask.
   __shared__ int s_tile_id[kMaxSegTiles];
   int seg_t0 = 0;          // tile that s_tile_id[0] describes
-  if (seg_k) seg_t0 = classify_segment_groups<Tile::BK, 256>(seg_q, seg_k, tid, k_begin, k_end, s_tile_id, kMaxSegTiles,
+  if (seg_k) seg_t0 = classify_segment_groups<Tile::BK, 64 * NW>(seg_q, seg_k, tid, k_begin, k_end, s_tile_id, kMaxSegTiles,
                                                             kSegNotUniform);
   const int t_begin = k_begin / Tile::BK;
   const int t_end = (k_end + Tile::BK - 1) / Tile::BK;
@@ -153,7 +157,7 @@ void flash_fwd_kernel(const FwdArgs a) {
   unsigned k_src[Tile::DMA_PER_WAVE], v_src[Tile::DMA_PER_WAVE];  // byte offsets from the tile's first row
 #pragma unroll
   for (int i = 0; i < Tile::DMA_PER_WAVE; i++) {
-    const int row = 16 * wave + RPI * i + lane / CPR;
+    const int row = Tile::WROWS * wave + RPI * i + lane / CPR;
     const int chunk = (lane % CPR) ^ Tile::swz(row);
     // the second load of a pair carries an instruction offset of 1024, which also moves its source
     k_src[i] = (unsigned)(row * (int)a.ks.s + chunk * 8) * 2 - (i % 2) * 1024;
@@ -162,15 +166,24 @@ void flash_fwd_kernel(const FwdArgs a) {
   const unsigned lds0 = lds_address(smem);
   auto issue_k = [&](int t, int buf) {
     const __bf16* src = kp + (int64_t)t * Tile::BK * a.ks.s;
-    const unsigned dst = lds0 + buf * Tile::TILE_BYTES + wave * (16 * Tile::ROWB);
+    const unsigned dst = lds0 + buf * Tile::TILE_BYTES + wave * (Tile::WROWS * Tile::ROWB);
 #pragma unroll
     for (int i = 0; i < Tile::DMA_PER_WAVE; i += 2) dma16x2(k_src[i], k_src[i + 1], src, dst + i * 1024);
     if (seg_k && wave == 0 && lane < Tile::BK / 4)  // 64 ids = 16 lanes x 16 bytes
       dma16(seg_k + t * Tile::BK + 4 * lane, lds0 + Tile::SEG_BASE + (t % Tile::NSEG) * (Tile::BK * 4));
   };
+  // One pair of a tile's loads (FAST tiles deal the pairs out over their MFMA slots).
+  auto issue_k_pair = [&](int t, int buf, int i) __attribute__((always_inline)) {
+    const __bf16* src = kp + (int64_t)t * Tile::BK * a.ks.s;
+    dma16x2(k_src[i], k_src[i + 1], src, lds0 + buf * Tile::TILE_BYTES + wave * (Tile::WROWS * Tile::ROWB) + i * 1024);
+  };
+  auto issue_v_pair = [&](int t, int buf, int i) __attribute__((always_inline)) {
+    const __bf16* src = vp + (int64_t)t * Tile::BK * a.vs.s;
+    dma16x2(v_src[i], v_src[i + 1], src, lds0 + (2 + buf) * Tile::TILE_BYTES + wave * (Tile::WROWS * Tile::ROWB) + i * 1024);
+  };
   auto issue_v = [&](int t, int buf) {
     const __bf16* src = vp + (int64_t)t * Tile::BK * a.vs.s;
-    const unsigned dst = lds0 + (2 + buf) * Tile::TILE_BYTES + wave * (16 * Tile::ROWB);
+    const unsigned dst = lds0 + (2 + buf) * Tile::TILE_BYTES + wave * (Tile::WROWS * Tile::ROWB);
 #pragma unroll
     for (int i = 0; i < Tile::DMA_PER_WAVE; i += 2) dma16x2(v_src[i], v_src[i + 1], src, dst + i * 1024);
   };
@@ -221,18 +234,30 @@ void flash_fwd_kernel(const FwdArgs a) {
 
   // One tile: softmax and P V of tile t (logits in s), S^T of tile t+1 (into s_nxt).  buf_c is the
   // parity of the tile, i.e. which half of the double buffers holds it.
-  auto tile_step = [&](int t, auto buf_c, floatx16 (&s)[2], floatx16 (&s_nxt)[2]) __attribute__((always_inline)) {
+  // Lane-local maximum of the logits that the last FAST tile left in its s_nxt (taken between its P V
+  // MFMAs); a FAST tile starts from it instead of scanning its 32 logits.
+  float mx_carry = kNegInf;
+  auto tile_step = [&](int t, auto buf_c, floatx16 (&s)[2], floatx16 (&s_nxt)[2], auto fast_c) __attribute__((always_inline)) {
     constexpr int buf = decltype(buf_c)::value;
+    // FAST: a tile in the interior of this wavefront's range - its softmax needs no mask of any kind
+    // and the tile after it is processed too - so every test below is decided at compile time.
+    constexpr bool FAST = decltype(fast_c)::value;
     // K(t+1) and V(t) (requested one iteration ago) become visible to the whole workgroup and every
     // wavefront is done with S(t) and PV(t-1); the buffers those were read from are then refilled
     // with K(t+2) and V(t+1).
     wait_vmem_le<0>();
     __syncthreads();
-    if (t + 2 < t_end) issue_k(t + 2, buf);
-    if (t + 1 < t_end) issue_v(t + 1, buf ^ 1);
+    if constexpr (!FAST) {
+      if (t + 2 < t_end) issue_k(t + 2, buf);
+      if (t + 1 < t_end) issue_v(t + 1, buf ^ 1);
+    }
+    // FAST tiles issue the same loads one pair per MFMA slot further down, where their issue time
+    // overlaps the matrix pipe's work; K(t+2) may not exist (t + 2 == t_end), then the last tile is
+    // fetched again into a buffer that nobody reads any more.
+    const int t_k2 = min(t + 2, t_end - 1);
 
-    const bool do_sm = t >= tw_begin && t < tw_end;          // softmax and PV of tile t
-    const bool do_s = t + 1 >= tw_begin && t + 1 < tw_end;   // S of tile t + 1
+    const bool do_sm = FAST || (t >= tw_begin && t < tw_end);          // softmax and PV of tile t
+    const bool do_s = FAST || (t + 1 >= tw_begin && t + 1 < tw_end);   // S of tile t + 1
     const char* kt = k_lds + (buf ^ 1) * Tile::TILE_BYTES;   // K(t+1)
     const char* vt = v_lds + buf * Tile::TILE_BYTES;         // V(t)
     const int k0 = t * Tile::BK;
@@ -243,7 +268,7 @@ void flash_fwd_kernel(const FwdArgs a) {
 
     // ---- masks of tile t.  Register r of sub-tile ks in lane group g is key k0 + 32ks + 16(r/8) + 8g + (r%8).
     uint2 dm[2][2] = {};  // dropout bytes of the lane's 4 runs of 8 keys
-    if constexpr (AUX) {
+    if constexpr (AUX && !FAST) {
       if (bias_row) {
 #pragma unroll
         for (int ks = 0; ks < 2; ks++)
@@ -276,7 +301,7 @@ void flash_fwd_kernel(const FwdArgs a) {
     };
     bool need_mask = false;
     const unsigned mask_limit = a.mask_kind == AXL_MASK_SLIDING_WINDOW ? (unsigned)a.window : 0x7fffffffu;
-    if (a.mask_kind != AXL_MASK_NONE) {
+    if (!FAST && a.mask_kind != AXL_MASK_NONE) {
       need_mask = k0 + Tile::BK - 1 > qpos_min;
       if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) need_mask = need_mask || (qpos_max - k0 > a.window);
     }
@@ -292,7 +317,7 @@ void flash_fwd_kernel(const FwdArgs a) {
         }
       }
     }
-    if (seg_k && !(seg_fast && s_tile_id[t - seg_t0] == wq_id)) {
+    if (!FAST && seg_k && !(seg_fast && s_tile_id[t - seg_t0] == wq_id)) {
       const char* sg = seg_lds + (t % Tile::NSEG) * (Tile::BK * 4);
 #pragma unroll
       for (int ks = 0; ks < 2; ks++) {
@@ -313,10 +338,14 @@ void flash_fwd_kernel(const FwdArgs a) {
     // moves when the new max exceeds it by more than 2^kLazyLog2 in the exponent; until then exp2 is
     // taken against the stale max, which scales numerator and denominator alike.
     float mx = m_run;
+    if constexpr (FAST) {
+      mx = fmaxf(mx, mx_carry);
+    } else {
 #pragma unroll
-    for (int ks = 0; ks < 2; ks++)
+      for (int ks = 0; ks < 2; ks++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[ks][r]);
+        for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[ks][r]);
+    }
     mx = xor32_max(mx);
     constexpr float kLazyLog2 = 8.0f;
     const bool move = (mx - m_run) * c > kLazyLog2;
@@ -351,7 +380,20 @@ void flash_fwd_kernel(const FwdArgs a) {
 #pragma unroll
       for (int n = 0; n < NSL; n++) {
         if (n + kAhead < NSL) kfr[n + kAhead] = AXL_K_FRAG(kt, (n + kAhead) / 2, (n + kAhead) % 2);
-        if (n < 2) {
+        if constexpr (FAST) {
+          constexpr int kPairs = Tile::DMA_PER_WAVE / 2;
+          if (n % 2 == 0 && n / 2 < kPairs) issue_k_pair(t_k2, buf, n);
+          if (n % 2 == 0 && n / 2 >= kPairs && n / 2 < 2 * kPairs) issue_v_pair(t + 1, buf ^ 1, n - 2 * kPairs);
+          // the ids of tile t+2 for a general tile that may follow (every wavefront fetches the same
+          // 256 bytes: no branch on the wavefront number inside the slot sequence)
+          if (n == 4 * kPairs && seg_k)
+            dma16s_first16(16 * (lane & 15), seg_k + t_k2 * Tile::BK, lds0 + Tile::SEG_BASE + (t_k2 % Tile::NSEG) * (Tile::BK * 4));
+          // The chain in vector registers where the next tile's softmax reads it, started from a
+          // literal zero: no register is cleared and none is copied.  (The 16 P V MFMAs of this tile lie
+          // between the end of the chain and the first read of its result.)
+          if (n < 2) E::mfma_32x32x16_vgpr_zero(kfr[n], qf[n / 2], s_nxt[n % 2]);
+          else E::mfma_32x32x16_vgpr(kfr[n], qf[n / 2], s_nxt[n % 2]);
+        } else if (n < 2) {
           const floatx16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
           s_nxt[n % 2] = E::mfma_32x32x16(kfr[n], qf[n / 2], zero16);
         } else {
@@ -394,21 +436,81 @@ void flash_fwd_kernel(const FwdArgs a) {
 #pragma unroll
     for (int n = 0; n < kPvAhead; n++) AXL_PV_READ(n)
     __builtin_amdgcn_sched_barrier(0);
+    float pm[4] = {kMasked, kMasked, kMasked, kMasked};
 #pragma unroll
     for (int n = 0; n < kPvSteps; n++) {
       if (n + kPvAhead < kPvSteps) AXL_PV_READ(n + kPvAhead)
       o[n % DT] = E::mfma_32x32x16(vfr[n].v, pb.v[n / DT], o[n % DT]);
+      if constexpr (FAST) {
+        // Row maximum of the next tile's logits, two per slot from slot 2 on: by then two MFMAs have
+        // been issued after the last one of the S chains, whose results these reads therefore find
+        // complete.  Four independent partial maxima keep the chains short.
+#pragma unroll
+        for (int j = 0; j < 16; j++)
+          if (2 + j * (kPvSteps - 2) / 16 == n)
+            pm[j % 4] = fmaxf(fmaxf(pm[j % 4], s_nxt[(2 * j) / 16][(2 * j) % 16]), s_nxt[(2 * j + 1) / 16][(2 * j + 1) % 16]);
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
+    if constexpr (FAST) mx_carry = fmaxf(fmaxf(pm[0], pm[1]), fmaxf(pm[2], pm[3]));
 #undef AXL_PV_READ
   };
   {
-    int t = t_begin;
-    for (; t + 1 < t_end; t += 2) {
-      tile_step(t, std::integral_constant<int, 0>{}, s_even, s_odd);
-      tile_step(t + 1, std::integral_constant<int, 1>{}, s_odd, s_even);
+    // Tiles [f_lo, f_hi) of this wavefront take the FAST form: inside its own range, the tile after
+    // them inside it too, no positional mask (every key of the tile at or before the wavefront's first
+    // query and, under a sliding window, within the window of its last query), no segment ids, no bias
+    // or dropout mask.  f_lo has the parity of t_begin so that a pair of FAST tiles uses the register
+    // sets and the buffers in the order (even, odd).
+    const std::integral_constant<int, 0> c0{};
+    const std::integral_constant<int, 1> c1{};
+    int f_lo = t_end, f_hi = t_end;
+    if (!AUX && (!seg_k || seg_fast)) {
+      f_lo = tw_begin;
+      f_hi = tw_end - 1;
+      if (a.mask_kind != AXL_MASK_NONE) {
+        f_hi = min(f_hi, qpos_min >= Tile::BK - 1 ? (qpos_min - (Tile::BK - 1)) / Tile::BK + 1 : 0);
+        if (a.mask_kind == AXL_MASK_SLIDING_WINDOW)
+          f_lo = max(f_lo, qpos_max - a.window > 0 ? (qpos_max - a.window + Tile::BK - 1) / Tile::BK : 0);
+      }
+      if (seg_k) {
+        // ... and, with segment ids, only the run of tiles that ends at f_hi and whose keys all carry the
+        // one id that all of this wavefront's queries carry (lane j looks at tile base - j; the lowest
+        // set bit of the ballot is the last tile that breaks the run).
+        for (int base = f_hi - 1; base >= f_lo; base -= 64) {
+          const int i = base - lane;
+          const uint64_t m = __builtin_amdgcn_ballot_w64(i >= f_lo && s_tile_id[i - seg_t0] != wq_id);
+          if (m) {
+            f_lo = base - __builtin_ctzll(m) + 1;
+            break;
+          }
+        }
+      }
+      f_lo += (f_lo - t_begin) & 1;
     }
-    if (t < t_end) tile_step(t, std::integral_constant<int, 0>{}, s_even, s_odd);
+    int t = t_begin;
+    // Pairs of tiles in the general form up to tile t_to (t and t_to have the parity of t_begin).
+    auto generic_pairs_to = [&](int t_to) __attribute__((always_inline)) {
+      for (; t + 1 < t_to; t += 2) {
+        tile_step(t, c0, s_even, s_odd, std::false_type{});
+        tile_step(t + 1, c1, s_odd, s_even, std::false_type{});
+      }
+    };
+    if constexpr (!AUX) {
+      generic_pairs_to(min(f_lo, t_end));
+      if (t + 1 < f_hi) {  // the first FAST tile's lane-local maximum (later ones get theirs from the tile before)
+        mx_carry = kMasked;
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) mx_carry = fmaxf(mx_carry, s_even[ks][r]);
+      }
+      for (; t + 1 < f_hi; t += 2) {
+        tile_step(t, c0, s_even, s_odd, std::true_type{});
+        tile_step(t + 1, c1, s_odd, s_even, std::true_type{});
+      }
+    }
+    generic_pairs_to(t_end);
+    if (t < t_end) tile_step(t, c0, s_even, s_odd, std::false_type{});
   }
 #undef AXL_K_FRAG
 #undef AXL_S_PLAIN
@@ -628,13 +730,13 @@ int launch_flash_fwd(const AxlFlashFwdParams& p, hipStream_t stream) {
   a.mask_kind = p.mask_kind; a.window = p.sliding_window; a.q_off = p.q_pos_offset;
   a.q_offs = p.q_pos_offsets;
   a.scale = p.softmax_scale;
-  const int grid = (p.q_len / 128) * p.batch * p.num_q_heads;
   hipError_t err = hipSuccess;
 #define AXL_LAUNCH_FWD(KERNEL, TILE)                                                            \
   do {                                                                                          \
     err = allow_dynamic_lds((const void*)KERNEL, TILE::LDS_BYTES);                              \
     if (err == hipSuccess) {                                                                    \
-      hipLaunchKernelGGL(KERNEL, dim3(grid), dim3(256), TILE::LDS_BYTES, stream, a);            \
+      const int grid = (p.q_len / TILE::BQ) * p.batch * p.num_q_heads;                          \
+      hipLaunchKernelGGL(KERNEL, dim3(grid), dim3(2 * TILE::BQ), TILE::LDS_BYTES, stream, a);   \
       err = hipGetLastError();                                                                  \
     }                                                                                           \
   } while (0)
