@@ -14,33 +14,38 @@
 // the 128 query rows of block a can see.  A block is 2 KB: [q half 2][key 32][16 queries] in the input
 // dtype, i.e. the dK/dV kernel's packed dS operand registers written lane by lane.
 //
-// Mapping.  A workgroup owns 128 query rows of one (batch, query head); wavefront w owns query tile
-// 4 qb + w and the fp32 dQ^T accumulators of its 32 rows.  Per trip of 64 keys the K tile (shared,
-// XOR-swizzled) and each wavefront's own 4 KB of ds arrive by direct global->LDS loads through a
-// five-deep ring; dQ^T += K^T dS^T with both operands from transposing LDS reads.
+// Mapping.  A workgroup of NW wavefronts owns 32 NW query rows of one (batch, query head); wavefront w
+// owns query tile NW qb + w and the fp32 dQ^T accumulators of its 32 rows.  Per trip of 64 keys the K
+// tile (shared, XOR-swizzled) and each wavefront's own 4 KB of ds arrive by direct global->LDS loads
+// through a ring of buffers; dQ^T += K^T dS^T with both operands from transposing LDS reads.  The
+// kernel issues 2.5 LDS reads and half a tile load per MFMA, each of which holds up the wavefront that
+// issues it, so it runs with two wavefronts per SIMD where the shape allows (NW = 8, one workgroup of
+// 256 rows per CU, three buffers; a wavefront of the upper 128 rows has two trips more than one of
+// the lower 128) and with NW = 4 (five buffers) otherwise.
 #include "flash_bwd.h"
 
 namespace axl {
 
-template <int D>
+template <int D, int NW>
 struct DqStream {
-  static constexpr int BQ = 128;             // query rows per workgroup (32 per wavefront)
+  static constexpr int BQ = 32 * NW;         // query rows per workgroup (32 per wavefront)
   static constexpr int BK = 64;              // keys per trip
   static constexpr int ROWB = D * 2;         // bytes per K row: unpadded, chunks swizzled (tile_swizzle)
   static constexpr int K_BYTES = BK * ROWB;
   static constexpr int DS_WAVE_BYTES = 2 * kDsBlockBytes;          // two 32-key blocks per wavefront per trip
   static constexpr int DS_BASE = K_BYTES;
-  static constexpr int BUF_BYTES = K_BYTES + 4 * DS_WAVE_BYTES;
-  static constexpr int NBUF = 5;
+  static constexpr int BUF_BYTES = K_BYTES + NW * DS_WAVE_BYTES;
+  static constexpr int NBUF = NW == 8 ? 3 : 5;
+  static constexpr int WROWS = BK / NW;                            // K rows that one wavefront fetches
   static constexpr int RPI = 1024 / ROWB;                          // K rows per direct-to-LDS instruction
-  static constexpr int K_DMA_PER_WAVE = BK / 4 / RPI;              // 16 K rows per wavefront
+  static constexpr int K_DMA_PER_WAVE = WROWS / RPI;
   static constexpr int NLD = K_DMA_PER_WAVE + DS_WAVE_BYTES / 1024;  // loads per wavefront per trip
   static constexpr int LDS_BYTES = NBUF * BUF_BYTES;
 };
 
-template <typename E, int D>
-__global__ __launch_bounds__(256) void flash_bwd_dq_stream_kernel(const BwdArgs a) {
-  using Tile = DqStream<D>;
+template <typename E, int D, int NW>
+__global__ __launch_bounds__(64 * NW) void flash_bwd_dq_stream_kernel(const BwdArgs a) {
+  using Tile = DqStream<D, NW>;
   constexpr int DT = D / 32;
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
@@ -50,7 +55,9 @@ __global__ __launch_bounds__(256) void flash_bwd_dq_stream_kernel(const BwdArgs 
   decode_block(blockIdx.x, a.T / Tile::BQ, a.B, a.Hq, a.Hkv, 32, qb, b, h);
   const int hk = h / (a.Hq / a.Hkv);
   const int q0 = qb * Tile::BQ + wave * 32;
-  const int trips = 2 * (qb + 1);            // 64-key tiles up to and including the diagonal block
+  const int t_q = NW * qb + wave;            // this wavefront's query tile
+  const int trips = 2 * ((NW * qb + NW - 1) / 4 + 1);  // 64-key tiles up to and including the last diagonal block
+  const int my_trips = __builtin_amdgcn_readfirstlane(2 * (t_q / 4 + 1));  // ... of this wavefront's own 128-row block
 
   floatx16 dq_acc[DT];
 #pragma unroll
@@ -64,7 +71,7 @@ __global__ __launch_bounds__(256) void flash_bwd_dq_stream_kernel(const BwdArgs 
   unsigned k_lane[Tile::K_DMA_PER_WAVE];
 #pragma unroll
   for (int i = 0; i < Tile::K_DMA_PER_WAVE; i++) {
-    const int row = 16 * wave + Tile::RPI * i + lane / CPR;
+    const int row = Tile::WROWS * wave + Tile::RPI * i + lane / CPR;
     const int chunk = (lane % CPR) ^ tile_swizzle<D>(row);
     // the second load of a pair carries an instruction offset of 1024, which also moves its source
     k_lane[i] = (unsigned)(row * (int)a.ks.s + chunk * 8) * 2 - (i % 2) * 1024;
@@ -72,28 +79,28 @@ __global__ __launch_bounds__(256) void flash_bwd_dq_stream_kernel(const BwdArgs 
   static_assert(Tile::K_DMA_PER_WAVE % 2 == 0, "K loads are issued in pairs");
   const __bf16* k_src = (const __bf16*)a.k + b * a.ks.b + hk * a.ks.h;
   const int64_t k_step = (int64_t)Tile::BK * a.ks.s;
-  const int t_q = 4 * qb + wave;             // this wavefront's query tile
   const int G = a.Hq / a.Hkv;
   const char* ds_src = (const char*)a.ds + ds_run_start((int64_t)b * a.Hkv + hk, a.T, G, t_q, h - hk * G) * kDsBlockBytes;
   const unsigned ds_lane = 16 * lane;
   const unsigned lds0 = lds_address(smem);
 #define AXL_DMA_TRIP(BUF_)                                                                         \
   {                                                                                               \
-    const unsigned kdst_ = lds0 + (BUF_) * Tile::BUF_BYTES + wave * (16 * Tile::ROWB);            \
+    const unsigned kdst_ = lds0 + (BUF_) * Tile::BUF_BYTES + wave * (Tile::WROWS * Tile::ROWB);   \
     _Pragma("unroll") for (int i = 0; i < Tile::K_DMA_PER_WAVE; i += 2)                           \
       dma16x2(k_lane[i], k_lane[i + 1], k_src, kdst_ + i * 1024);                                 \
     const unsigned ddst_ = lds0 + (BUF_) * Tile::BUF_BYTES + Tile::DS_BASE + wave * Tile::DS_WAVE_BYTES; \
     _Pragma("unroll") for (int i = 0; i < Tile::DS_WAVE_BYTES / 2048; i++)                        \
       dma16x2(ds_lane, ds_lane, ds_src + i * 2048, ddst_ + i * 2048);                             \
   }
-  // Prefetch cursor; it stops at the last trip (re-fetching that trip is harmless).
+  // Prefetch cursor; it stops at the last trip (re-fetching that trip is harmless), the dS part of it
+  // at the last trip of this wavefront's own run of blocks.
   int pf = 0;
 #define AXL_ADVANCE()                                                       \
   {                                                                         \
     const bool adv_ = pf + 1 < trips;                                       \
+    ds_src += __builtin_amdgcn_readfirstlane(pf + 1 < my_trips ? Tile::DS_WAVE_BYTES : 0); \
     pf += adv_ ? 1 : 0;                                                     \
     k_src += adv_ ? k_step : 0;                                             \
-    ds_src += adv_ ? Tile::DS_WAVE_BYTES : 0;                               \
   }
 
   // ---- per-lane LDS read offsets.  K^T fragments (A operands): transposing reads of the swizzled K
@@ -119,26 +126,27 @@ __global__ __launch_bounds__(256) void flash_bwd_dq_stream_kernel(const BwdArgs 
 
   // Everything the compiler tracks has landed before the first untracked load.
   wait_all_vmem();
+  constexpr int PF = Tile::NBUF - 1;   // trips in flight ahead of the one being computed
   AXL_DMA_TRIP(0)
-  AXL_ADVANCE()
-  AXL_DMA_TRIP(1)
-  AXL_ADVANCE()
-  AXL_DMA_TRIP(2)
-  AXL_ADVANCE()
-  AXL_DMA_TRIP(3)
-  wait_vmem_le<3 * Tile::NLD>();   // trip 0 has landed
+#pragma unroll
+  for (int i = 1; i < PF; i++) {
+    AXL_ADVANCE()
+    AXL_DMA_TRIP(i)
+  }
+  wait_vmem_le<(PF - 1) * Tile::NLD>();   // trip 0 has landed
   __syncthreads();
 
   constexpr int NM = 4 * DT;          // MFMAs per trip: (32-key block, 16-key group) x dt
   constexpr int kAhead = 4;
-  int buf = 0, buf_pf = 4;          // ring slots of trip t and of trip t+4
+  int buf = 0, buf_pf = PF;         // ring slots of trip t and of trip t + PF
   for (int t = 0; t < trips; t++) {
     const char* kt = smem + buf * Tile::BUF_BYTES;
-    // Trip t+4 into the buffer that trip t-1 was read from (every wavefront passed the barrier after it).
+    // Trip t + PF into the buffer that trip t-1 was read from (every wavefront passed the barrier after it).
     AXL_ADVANCE()
     AXL_DMA_TRIP(buf_pf)
     buf = buf == Tile::NBUF - 1 ? 0 : buf + 1;
     buf_pf = buf_pf == Tile::NBUF - 1 ? 0 : buf_pf + 1;
+    if (t < my_trips) {
     TrFrag dsf[4], kfr[NM];
 #pragma unroll
     for (int s = 0; s < 4; s++) {     // s = 2 * block + 16-key group
@@ -162,9 +170,10 @@ __global__ __launch_bounds__(256) void flash_bwd_dq_stream_kernel(const BwdArgs 
       __builtin_amdgcn_sched_barrier(0);
     }
 #undef AXL_K_READ
-    // Trip t+1 has landed once at most the loads of trips t+2 .. t+4 are outstanding; after the
-    // barrier every wavefront's part of it is visible and nobody reads trip t's buffer any more.
-    wait_vmem_le<3 * Tile::NLD>();
+    }
+    // Trip t+1 has landed once at most the loads of the PF - 1 trips after it are outstanding; after
+    // the barrier every wavefront's part of it is visible and nobody reads trip t's buffer any more.
+    wait_vmem_le<(PF - 1) * Tile::NLD>();
     __syncthreads();
   }
   // The cursor re-requests the last trip during the final trips; none of those loads may still be in
@@ -188,15 +197,22 @@ __global__ __launch_bounds__(256) void flash_bwd_dq_stream_kernel(const BwdArgs 
     }
 }
 
-template <typename E, int D>
-static hipError_t launch_one(const BwdArgs& a, hipStream_t stream) {
-  using Tile = DqStream<D>;
-  auto kernel = flash_bwd_dq_stream_kernel<E, D>;
+template <typename E, int D, int NW>
+static hipError_t launch_nw(const BwdArgs& a, hipStream_t stream) {
+  using Tile = DqStream<D, NW>;
+  auto kernel = flash_bwd_dq_stream_kernel<E, D, NW>;
   hipError_t err = allow_dynamic_lds((const void*)kernel, Tile::LDS_BYTES);
   if (err != hipSuccess) return err;
   const int grid = (a.T / Tile::BQ) * a.B * a.Hq;
-  hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), Tile::LDS_BYTES, stream, a);
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(64 * NW), Tile::LDS_BYTES, stream, a);
   return hipGetLastError();
+}
+
+template <typename E, int D>
+static hipError_t launch_one(const BwdArgs& a, hipStream_t stream) {
+  // 8 wavefronts need two K loads per wavefront (head_dim 128) and 256-row blocks
+  if (D == 128 && a.T % 256 == 0) return launch_nw<E, D, D == 128 ? 8 : 4>(a, stream);
+  return launch_nw<E, D, 4>(a, stream);
 }
 
 hipError_t launch_bwd_dq_stream(const BwdArgs& a, int dtype, int head_dim, hipStream_t stream) {

@@ -5,6 +5,9 @@
 The headline workload (BASELINE.json configs[1], "C2") is causal GQA flash attention forward +
 backward, bf16, batch 4, 32 query heads / 8 kv heads, seq 4096, head_dim 128: a step is one forward
 (axl_flash_fwd) plus one backward (axl_flash_bwd) over one synthetic batch already resident in HBM.
+The backward of the headline step keeps dS in a workspace the caller provides (AXL_BWD_DS_WORKSPACE);
+`c2_recompute` in the same line is the same step through the backward that recomputes dS instead
+(`--recompute` makes that one the headline).
 The paged-decode half of the metric (configs[3], "C4") is measured in the same run and reported in
 the `paged_decode` object of the same JSON line.  With the default `--workload all` the line also
 carries `c1` (configs[0]: the fp32 case the reference itself runs on CPU), `c3` (sliding window +
@@ -332,6 +335,29 @@ def bench_paged_decode(steps, warmup, cpu_baseline):
     return res
 
 
+def calibrate_mfma(n=8192, reps=20):
+    """What the matrix cores of this machine sustain on a plain library GEMM (torch.matmul, bf16,
+    n^3) with N(0,1) operands and with all-zero operands: the clock is set by the power the operands'
+    bit activity draws, so the two differ, and the first is the practical ceiling for any kernel whose
+    MFMAs see random data.  Calibration only, like --calibrate-copy; no part of the measured path."""
+    dev = torch.device("cuda:0")
+    out = {}
+    for kind in ("normal", "zeros"):
+        if kind == "normal":
+            a = normal_tensor(7, (n, n), torch.bfloat16, dev)
+            b = normal_tensor(8, (n, n), torch.bfloat16, dev)
+        else:
+            a = torch.zeros((n, n), dtype=torch.bfloat16, device=dev)
+            b = torch.zeros((n, n), dtype=torch.bfloat16, device=dev)
+        c = torch.empty((n, n), dtype=torch.bfloat16, device=dev)
+        ms = _time_region(lambda: torch.matmul(a, b, out=c), reps, 10)
+        out[f"gemm_bf16_{n}_{kind}_tflops"] = 2.0 * n ** 3 / (ms * 1e-3) / 1e12
+        del a, b, c
+    out["note"] = "torch.matmul (hipBLASLt) bf16 GEMM, calibration of the power-limited matrix-core rate"
+    torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -341,6 +367,8 @@ def main():
                     help="all: headline C2 + C4, with C1, C3 and C5 as extra keys of the same line")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true", help="skip the paged-decode half of the metric")
+    ap.add_argument("--recompute", action="store_true",
+                    help="C2 through the backward whose dQ kernel recomputes dS (no dS workspace)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (known traffic) for scaling rocprofv3 byte counters")
     args = ap.parse_args()
@@ -378,6 +406,10 @@ def main():
         line["c1"] = res
     else:
         cfg = _flash_workload("c2" if args.workload == "all" else args.workload)
+        if cfg["name"] == "c2" and not args.recompute:
+            # The headline step runs the backward that keeps dS in a caller-provided workspace
+            # (AXL_BWD_DS_WORKSPACE: 5 executed GEMMs instead of 7; plain causal attention only).
+            cfg = dict(cfg, ds_workspace=True)
         res = bench_flash(cfg, args.steps, args.warmup, cpu_base)
         line.update(value=res["value"], unit="TFLOP/s", ms_per_step=res["ms_per_step"],
                     config=dict(workload=cfg["label"], batch=cfg["B"], seq_len=cfg["T"], num_q_heads=cfg["Hq"],
@@ -393,8 +425,10 @@ def main():
             line["paged_decode"] = bench_paged_decode(args.steps, args.warmup, cpu_base)
         if args.workload == "all":
             # The other BASELINE configs, fewer repetitions: they are reported, not the headline.
-            # The same C2 step through the backward that keeps dS in a workspace (AXL_BWD_DS_WORKSPACE).
-            line["c2_ds_workspace"] = bench_flash(dict(cfg, ds_workspace=True), args.steps, args.warmup, False)
+            # The same C2 step through the other backward (the dQ kernel recomputes dS; no dS workspace).
+            line["c2_recompute" if cfg.get("ds_workspace") else "c2_ds_workspace"] = bench_flash(
+                dict(cfg, ds_workspace=not cfg.get("ds_workspace")), args.steps, args.warmup, False)
+            line["machine"] = calibrate_mfma()
             line["c1"] = bench_c1(args.steps, args.warmup, cpu_base)
             line["c3"] = bench_flash(_flash_workload("c3"), max(5, args.steps // 2), 2, cpu_base)
             line["c5"] = bench_flash(_flash_workload("c5"), max(3, args.steps // 4), 1, cpu_base)
