@@ -324,45 +324,122 @@ __device__ __forceinline__ void shrink_to_segment_hull(int my_id, const int32_t*
 template <int GROUP, int NT, int ALIGN = GROUP>
 __device__ __forceinline__ int classify_segment_groups(int my_id, const int32_t* ids, int tid, int& lo, int& hi,
                                                        int* s_uniform, int cap, int not_uniform) {
-  __shared__ int s_rng[4];
-  if (tid == 0) {
-    s_rng[0] = 0x7fffffff;       // smallest own id
-    s_rng[1] = -0x7fffffff - 1;  // largest own id
-    s_rng[2] = 0x7fffffff;       // first candidate group
-    s_rng[3] = -1;               // last candidate group
+  // Reductions go lane to lane inside a wavefront and through one LDS slot per wavefront between
+  // them: no atomics (256 threads updating one LDS word take turns).
+  __shared__ int s_rng[4 * (NT / 64)];
+  const int lane = tid & 63, wave = tid >> 6;
+  int id_min = my_id, id_max = my_id;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    id_min = min(id_min, __shfl_xor(id_min, o));
+    id_max = max(id_max, __shfl_xor(id_max, o));
+  }
+  if (lane == 0) {
+    s_rng[4 * wave] = id_min;
+    s_rng[4 * wave + 1] = id_max;
   }
   __syncthreads();
-  atomicMin(&s_rng[0], my_id);
-  atomicMax(&s_rng[1], my_id);
-  __syncthreads();
-  const int id_min = s_rng[0], id_max = s_rng[1];
+#pragma unroll
+  for (int w = 0; w < NT / 64; w++) {
+    id_min = min(id_min, s_rng[4 * w]);
+    id_max = max(id_max, s_rng[4 * w + 1]);
+  }
   // whole ALIGN-row blocks at both ends, so that every group of the caller's first and last tile is described
   const int g0 = (lo / ALIGN) * (ALIGN / GROUP), g1 = ((hi + ALIGN - 1) / ALIGN) * (ALIGN / GROUP);
-  int first = 0x7fffffff, last = -1;
-  for (int i = g0 + tid; i < g1; i += NT) {
-    const intx4* p = (const intx4*)(ids + (int64_t)i * GROUP);
-    int mn = 0x7fffffff, mx = -0x7fffffff - 1;
+  int first = 0x7fffffff, last = -1;   // wave-uniform
+  for (int base = g0 + wave * 64; base < g1; base += NT) {
+    const int i = base + lane;
+    bool cand = false;
+    if (i < g1) {
+      const intx4* p = (const intx4*)(ids + (int64_t)i * GROUP);
+      int mn = 0x7fffffff, mx = -0x7fffffff - 1;
 #pragma unroll
-    for (int v = 0; v < GROUP / 4; v++) {
-      const intx4 x = p[v];
-      mn = min(min(mn, min(x[0], x[1])), min(x[2], x[3]));
-      mx = max(max(mx, max(x[0], x[1])), max(x[2], x[3]));
+      for (int v = 0; v < GROUP / 4; v++) {
+        const intx4 x = p[v];
+        mn = min(min(mn, min(x[0], x[1])), min(x[2], x[3]));
+        mx = max(max(mx, max(x[0], x[1])), max(x[2], x[3]));
+      }
+      if (i - g0 < cap) s_uniform[i - g0] = mn == mx ? mn : not_uniform;
+      cand = mx >= id_min && mn <= id_max;
     }
-    if (i - g0 < cap) s_uniform[i - g0] = mn == mx ? mn : not_uniform;
-    if (mx >= id_min && mn <= id_max) {
-      first = min(first, i);
-      last = max(last, i);
+    const uint64_t m = __builtin_amdgcn_ballot_w64(cand);   // lane j looks at group base + j
+    if (m) {
+      first = min(first, base + (int)__builtin_ctzll(m));
+      last = max(last, base + 63 - (int)__builtin_clzll(m));
     }
   }
-  if (last >= 0) {
-    atomicMin(&s_rng[2], first);
-    atomicMax(&s_rng[3], last);
+  if (lane == 0) {
+    s_rng[4 * wave + 2] = first;
+    s_rng[4 * wave + 3] = last;
   }
   __syncthreads();
-  lo = max(lo, s_rng[2] == 0x7fffffff ? hi : s_rng[2] * GROUP);
-  hi = min(hi, (s_rng[3] + 1) * GROUP);
+#pragma unroll
+  for (int w = 0; w < NT / 64; w++) {
+    first = min(first, s_rng[4 * w + 2]);
+    last = max(last, s_rng[4 * w + 3]);
+  }
+  lo = max(lo, first == 0x7fffffff ? hi : first * GROUP);
+  hi = min(hi, (last + 1) * GROUP);
   if (hi < lo) hi = lo;
-  return g0;
+  // the same in every lane: say so, the callers form scalar addresses from them
+  lo = __builtin_amdgcn_readfirstlane(lo);
+  hi = __builtin_amdgcn_readfirstlane(hi);
+  return __builtin_amdgcn_readfirstlane(g0);
+}
+
+// The same classification from a table that one small kernel has filled beforehand (the backward has a
+// workspace for it): `tbl` holds, for every group of 32 consecutive rows of this sequence, the
+// smallest and the largest segment id in the group.  The workgroup's own rows are the `own_n` groups
+// from `own_g0` on, so their id range comes from the table as well: one global load per thread, one
+// barrier, no atomics - instead of a pass over the ids themselves whose latencies nothing overlaps
+// when a CU holds a single workgroup.  Semantics as classify_segment_groups with GROUP = 32.
+// Called by all NT threads of the workgroup (whole wavefronts); contains a barrier.
+constexpr int kSegGroupRows = 32;
+template <int NT, int ALIGN = kSegGroupRows>
+__device__ __forceinline__ int classify_segment_groups_tbl(const int2* tbl, int own_g0, int own_n, int tid, int& lo,
+                                                           int& hi, int* s_uniform, int cap, int not_uniform) {
+  constexpr int GROUP = kSegGroupRows;
+  __shared__ int s_rng[2 * (NT / 64)];
+  int id_min = 0x7fffffff, id_max = -0x7fffffff - 1;
+  for (int i = 0; i < own_n; i++) {
+    const int2 e = tbl[own_g0 + i];
+    id_min = min(id_min, e.x);
+    id_max = max(id_max, e.y);
+  }
+  const int g0 = (lo / ALIGN) * (ALIGN / GROUP), g1 = ((hi + ALIGN - 1) / ALIGN) * (ALIGN / GROUP);
+  const int lane = tid & 63, wave = tid >> 6;
+  int first = 0x7fffffff, last = -1;   // wave-uniform
+  for (int base = g0 + wave * 64; base < g1; base += NT) {
+    const int i = base + lane;
+    bool cand = false;
+    if (i < g1) {
+      const int2 e = tbl[i];
+      if (i - g0 < cap) s_uniform[i - g0] = e.x == e.y ? e.x : not_uniform;
+      cand = e.y >= id_min && e.x <= id_max;
+    }
+    const uint64_t m = __builtin_amdgcn_ballot_w64(cand);   // lane j looks at group base + j
+    if (m) {
+      first = min(first, base + (int)__builtin_ctzll(m));
+      last = max(last, base + 63 - (int)__builtin_clzll(m));
+    }
+  }
+  if (lane == 0) {
+    s_rng[2 * wave] = first;
+    s_rng[2 * wave + 1] = last;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int w = 0; w < NT / 64; w++) {
+    first = min(first, s_rng[2 * w]);
+    last = max(last, s_rng[2 * w + 1]);
+  }
+  lo = max(lo, first == 0x7fffffff ? hi : first * GROUP);
+  hi = min(hi, (last + 1) * GROUP);
+  if (hi < lo) hi = lo;
+  // the same in every lane: say so, the callers form scalar addresses from them
+  lo = __builtin_amdgcn_readfirstlane(lo);
+  hi = __builtin_amdgcn_readfirstlane(hi);
+  return __builtin_amdgcn_readfirstlane(g0);
 }
 
 // Decodes blockIdx.x into (query block, batch, query head).  Workgroup i is dispatched to XCD i % 8.

@@ -19,6 +19,7 @@ struct BwdArgs {
   void* dk;
   void* dv;
   const int32_t* seg;
+  const int2* seg_tbl;  // workspace [B, T / 32]: smallest and largest segment id of every 32 rows (with seg)
   Strides3 qs, ks, vs, os, dos, dqs, dks, dvs;
   int B, T, S, Hq, Hkv;
   int mask_kind, window, q_off;

@@ -317,6 +317,23 @@ __global__ __launch_bounds__(256) void flash_bwd_dq_aux_kernel(const BwdArgs a) 
     }
 }
 
+// Smallest and largest segment id of every group of 32 consecutive rows ([B, T / 32] groups in all):
+// what the dQ and dK/dV kernels classify their loop ranges from (classify_segment_groups_tbl).  One
+// thread per group.
+__global__ __launch_bounds__(256) void seg_group_table_kernel(const int32_t* seg, int2* tbl, int groups) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= groups) return;
+  const intx4* p = (const intx4*)(seg + (int64_t)i * kSegGroupRows);
+  int mn = 0x7fffffff, mx = -0x7fffffff - 1;
+#pragma unroll
+  for (int v = 0; v < kSegGroupRows / 4; v++) {
+    const intx4 x = p[v];
+    mn = min(min(mn, min(x[0], x[1])), min(x[2], x[3]));
+    mx = max(max(mx, max(x[0], x[1])), max(x[2], x[3]));
+  }
+  tbl[i] = make_int2(mn, mx);
+}
+
 static Strides3 to_s3(const AxlStrides& s) { return Strides3{s.batch, s.seq, s.head}; }
 
 // delta and lse2, [B, Hq, T] fp32 each, rounded up to 256 bytes.
@@ -336,8 +353,14 @@ static size_t spill_bytes(const AxlFlashBwdParams& p) {
   return (size_t)p.batch * p.num_q_heads * (size_t)ds_blocks_per_head(p.q_len) * kDsBlockBytes;
 }
 
+// With segment ids: the table of per-group id ranges (seg_group_table_kernel), 256-byte rounded.
+static size_t seg_table_bytes(const AxlFlashBwdParams& p) {
+  if (!p.segment_ids) return 0;
+  return ((size_t)p.batch * (p.q_len / kSegGroupRows) * sizeof(int2) + 255) & ~(size_t)255;
+}
+
 size_t flash_bwd_workspace_bytes(const AxlFlashBwdParams& p) {
-  return stats_bytes(p) + (spill_eligible(p) ? spill_bytes(p) : 0);
+  return stats_bytes(p) + seg_table_bytes(p) + (spill_eligible(p) ? spill_bytes(p) : 0);
 }
 
 int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream) {
@@ -348,7 +371,8 @@ int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream)
   a.lse2 = a.ndelta + (size_t)p.batch * p.num_q_heads * p.q_len;
   a.dq = p.dq; a.dk = p.dk; a.dv = p.dv; a.seg = p.segment_ids;
   const bool spill = spill_eligible(p);  // the entry point has checked that the workspace holds dS as well
-  a.ds = spill ? (char*)p.workspace + stats_bytes(p) : nullptr;
+  a.seg_tbl = p.segment_ids ? (const int2*)((char*)p.workspace + stats_bytes(p)) : nullptr;
+  a.ds = spill ? (char*)p.workspace + stats_bytes(p) + seg_table_bytes(p) : nullptr;
   a.qs = to_s3(p.q_strides); a.ks = to_s3(p.k_strides); a.vs = to_s3(p.v_strides);
   a.os = to_s3(p.out_strides); a.dos = to_s3(p.d_out_strides); a.dqs = to_s3(p.dq_strides);
   a.dks = to_s3(p.dk_strides); a.dvs = to_s3(p.dv_strides);
@@ -374,6 +398,13 @@ int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream)
   // All three phases in one call, no bias / dropout mask / sink gradient: the dQ kernel computes delta
   // on the way (it holds the dO rows anyway) and runs first; the dK/dV kernel reads what it left.
   const int all = AXL_BWD_DELTA | AXL_BWD_DKDV | AXL_BWD_DQ;
+  if (a.seg_tbl && dt != AXL_F32 && (phases & (AXL_BWD_DKDV | AXL_BWD_DQ))) {
+    // every call fills the table it reads: the phases may be enqueued one by one on a fresh workspace
+    const int groups = p.batch * (p.q_len / kSegGroupRows);
+    hipLaunchKernelGGL(seg_group_table_kernel, dim3((groups + 255) / 256), dim3(256), 0, stream, p.segment_ids,
+                       (int2*)a.seg_tbl, groups);
+    err = hipGetLastError();
+  }
   if (dt == AXL_F32) {
     if (phases & AXL_BWD_DELTA) {
       if (p.head_dim == 128) AXL_LAUNCH((bwd_delta_kernel<float, 128>), delta_grid, 0);

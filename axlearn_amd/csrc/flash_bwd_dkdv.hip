@@ -111,7 +111,16 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
     if (a.mask_kind == AXL_MASK_SLIDING_WINDOW)
       q_end = min(a.T, k0_wg + Tile::BKV - 1 + a.window - a.q_off + 1);
   }
-  if (HAS_SEG) shrink_to_segment_hull(seg_k, a.seg + (int64_t)b * a.T, tid, q_begin, q_end);
+  // With segment ids: the query range shrinks to the hull of the 32-row groups that hold an id
+  // between the smallest and the largest id of this workgroup's keys, and s_sub records for every query
+  // tile from sub_g0 on whether its rows carry a single id (both from the table of per-group id ranges
+  // that a small kernel leaves in the workspace).
+  __shared__ int s_sub[HAS_SEG && !AUX ? kMaxSubDkv : 1];
+  int sub_g0 = 0;
+  if (HAS_SEG)
+    sub_g0 = classify_segment_groups_tbl<256>(a.seg_tbl + (int64_t)b * (a.T / kSegGroupRows), k0_wg / kSegGroupRows,
+                                              Tile::BKV / kSegGroupRows, tid, q_begin, q_end, s_sub,
+                                              AUX ? 0 : kMaxSubDkv, kNotUniformDkv);
   const int t_begin = q_begin / Tile::BQ;
   const int nt = max(0, (q_end + Tile::BQ - 1) / Tile::BQ - t_begin);
   // Tiles in processing order: query tile (outer, from the LAST one down to the diagonal) x query head
@@ -650,34 +659,21 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
     // Query tiles whose 32 rows all carry the segment id that all 32 keys of this wavefront carry
     // need no segment mask either: take the first run [tA, tB) of such tiles (the masked loop is
     // always correct, so whatever lies outside that run simply stays on it).
-    __shared__ int s_sub[kMaxSubDkv];
     int tA = 0, tB = 0;
-    if (nt <= kMaxSubDkv) {
-      const int32_t* ids = a.seg + (int64_t)b * a.T + (int64_t)t_begin * Tile::BQ;
-      for (int i = tid; i < nt; i += 256) {
-        const intx4* p = (const intx4*)(ids + 32 * i);
-        const int id0 = ids[32 * i];
-        bool same = true;
-#pragma unroll
-        for (int v = 0; v < 8; v++) {
-          const intx4 x = p[v];
-          same = same && x[0] == id0 && x[1] == id0 && x[2] == id0 && x[3] == id0;
-        }
-        s_sub[i] = same ? id0 : kNotUniformDkv;
-      }
-      __syncthreads();
+    const int sub0 = t_begin - sub_g0;   // table index of query tile t_begin
+    if (sub0 + nt <= kMaxSubDkv) {
       const int wk_id = __builtin_amdgcn_readfirstlane(seg_k);
       const bool k_uniform = __builtin_amdgcn_ballot_w64(seg_k != wk_id) == 0 && wk_id != kNotUniformDkv;
       tA = tB = nt;
       if (k_uniform) {
         for (int base = 0; base < nt && tA == nt; base += 64) {
           const int i = base + lane;
-          const uint64_t m = __builtin_amdgcn_ballot_w64(i < nt && s_sub[i] == wk_id);
+          const uint64_t m = __builtin_amdgcn_ballot_w64(i < nt && s_sub[sub0 + min(i, nt - 1)] == wk_id);
           if (m) tA = base + __builtin_ctzll(m);
         }
         for (int base = tA & ~63; base < nt && tB == nt; base += 64) {
           const int i = base + lane;
-          const uint64_t m = __builtin_amdgcn_ballot_w64(i > tA && i < nt && s_sub[i] != wk_id);
+          const uint64_t m = __builtin_amdgcn_ballot_w64(i > tA && i < nt && s_sub[sub0 + min(i, nt - 1)] != wk_id);
           if (m) tB = base + __builtin_ctzll(m);
         }
       }

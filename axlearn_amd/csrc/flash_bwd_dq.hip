@@ -123,8 +123,9 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
   __shared__ int s_sub[HAS_SEG ? kMaxSub : 1];
   int sub_g0 = 0;  // sub-tile that s_sub[0] describes
   if (HAS_SEG)
-    sub_g0 = classify_segment_groups<32, 64 * NW, Tile::BK>(seg_q, a.seg + (int64_t)b * a.T, tid, k_begin, k_end,
-                                                           s_sub, kMaxSub, kNotUniform);
+    sub_g0 = classify_segment_groups_tbl<64 * NW, Tile::BK>(a.seg_tbl + (int64_t)b * (a.T / kSegGroupRows),
+                                                           q0_wg / kSegGroupRows, min(Tile::BQ, a.T - q0_wg) / kSegGroupRows, tid, k_begin,
+                                                           k_end, s_sub, kMaxSub, kNotUniform);
   const int t_begin = k_begin / Tile::BK;
   const int trips = max(0, (k_end + Tile::BK - 1) / Tile::BK - t_begin);
   const int key0 = t_begin * Tile::BK;   // first key of sub-tile 0

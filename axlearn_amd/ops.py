@@ -268,15 +268,17 @@ def flash_bwd(
 
 
 def flash_bwd_buffers(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, mask_kind: int = MASK_NONE,
-                      ds_workspace: bool = False):
+                      ds_workspace: bool = False, segment_ids: Optional[torch.Tensor] = None):
     """Pre-allocates (dq, dk, dv, workspace) for repeated `flash_bwd(..., buffers=...)` calls.
 
-    The workspace holds delta and the scaled lse (fp32 [B,Hq,T] each); with `ds_workspace=True` and
+    The workspace holds delta and the scaled lse (fp32 [B,Hq,T] each); with `segment_ids` (the ones the
+    calls will pass) also the table of id ranges per 32 rows; with `ds_workspace=True` and
     `mask_kind=MASK_CAUSAL` (equal lengths, no offsets / segment ids / bias / dropout) also dS, about
     T*S bytes per (batch, head), for `flash_bwd(..., ds_workspace=True)`."""
     b, t, hq, d = q.shape
     p = AxlFlashBwdParams(batch=b, q_len=t, kv_len=k.shape[1], num_q_heads=hq, num_kv_heads=k.shape[2],
                           head_dim=d, dtype=_lib.dtype_code(q.dtype), mask_kind=mask_kind,
+                          segment_ids=_lib.ptr(_seg(segment_ids)),
                           flags=_lib.BWD_DS_WORKSPACE if ds_workspace else 0)
     nbytes = int(_lib.load().axl_flash_bwd_workspace_bytes(ctypes.byref(p)))
     ws = torch.empty((max(nbytes, 256),), dtype=torch.uint8, device=q.device)

@@ -152,7 +152,7 @@ def bench_flash(cfg, steps, warmup, cpu_baseline):
     mask_kind = {"none": ops.MASK_NONE, "causal": ops.MASK_CAUSAL, "sliding": ops.MASK_SLIDING_WINDOW}[cfg["mask"]]
     kw = dict(softmax_scale=D ** -0.5, mask_kind=mask_kind, sliding_window=cfg["window"], segment_ids=seg)
     spill = bool(cfg.get("ds_workspace"))
-    bufs = ops.flash_bwd_buffers(q, k, v, mask_kind=mask_kind, ds_workspace=spill)
+    bufs = ops.flash_bwd_buffers(q, k, v, mask_kind=mask_kind, ds_workspace=spill, segment_ids=seg)
     kw_b = dict(kw, ds_workspace=spill)
     out, lse = ops.flash_fwd(q, k, v, **kw)
 

@@ -160,7 +160,7 @@ def test_float16_backward_matches_oracle(b, t, hq, hkv, d, mask, window, seg):
     _assert_close("dk", dk, wk, dtype)
     _assert_close("dv", dv, wv, dtype)
     bufs = (torch.zeros_like(dq), torch.zeros_like(dk), torch.zeros_like(dv),
-            torch.empty((2 * b * hq * t * 4 + 16,), dtype=torch.uint8, device="cuda"))
+            ops.flash_bwd_buffers(qc, kc, vc, mask_kind=kw["mask_kind"], segment_ids=kw.get("segment_ids"))[3])
     for phase in (1, 2, 4):  # delta, dK/dV, dQ
         ops.flash_bwd(qc, kc, vc, out, lse, doc, softmax_scale=scale, phases=phase, buffers=bufs, **kw)
     _assert_close("dq by phases", bufs[0], wq, dtype)
@@ -194,7 +194,7 @@ def test_float32_backward_matches_oracle(b, t, s, hq, hkv, d, mask, window, seg)
     _assert_close("dk", dk, wk, dtype)
     _assert_close("dv", dv, wv, dtype)
     bufs = (torch.zeros_like(dq), torch.zeros_like(dk), torch.zeros_like(dv),
-            torch.empty((2 * b * hq * t * 4 + 16,), dtype=torch.uint8, device="cuda"))
+            ops.flash_bwd_buffers(qc, kc, vc, mask_kind=kw["mask_kind"], segment_ids=kw.get("segment_ids"))[3])
     for phase in (1, 2, 4):  # delta, dK/dV, dQ
         ops.flash_bwd(qc, kc, vc, out, lse, doc, softmax_scale=scale, phases=phase, buffers=bufs, **kw)
     assert torch.equal(bufs[0], dq) and torch.equal(bufs[1], dk) and torch.equal(bufs[2], dv)
@@ -492,7 +492,7 @@ def test_forward_and_backward_replay_from_a_captured_graph():
     out_e, lse_e = ops.flash_fwd(q, k, v, **kw)
     grads_e = ops.flash_bwd(q, k, v, out_e, lse_e, do, **kw)
     bufs = (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v),
-            torch.empty((2 * b * hq * t * 4 + 16,), dtype=torch.uint8, device="cuda"))
+            ops.flash_bwd_buffers(q, k, v, mask_kind=kw["mask_kind"], segment_ids=kw.get("segment_ids"))[3])
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
         out_g, lse_g = ops.flash_fwd(q, k, v, **kw)
