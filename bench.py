@@ -49,10 +49,11 @@ HBM_PEAK_GBS = 8000.0           # MI355X HBM3E
 # kernel, `--calibrate-copy`).  Constants from the committed profile named next to each: the run
 # that prints them does not read the counters itself.
 TRAFFIC = {
-    "c2": dict(bytes=None, source="profiles/flash_counters.md (flash_bwd_dkdv_kernel)"),
-    "c3": dict(bytes=None, source="profiles/flash_counters.md (flash_bwd_dkdv_kernel, segment ids)"),
-    "c5": dict(bytes=None, source="profiles/flash_counters.md (flash_bwd_dkdv_kernel)"),
-    "c4": dict(bytes=4.25e9, source="profiles/bench_c2_c4_counters.md (decode_split_kernel)"),
+    "c2": dict(bytes=3.205e9, source="profiles/flash_c2_trace_counters.md (flash_bwd_dkdv_kernel, dS-workspace step)"),
+    "c2_recompute": dict(bytes=0.983e9, source="profiles/flash_c2_trace_counters.md (flash_bwd_dkdv_kernel, --recompute)"),
+    "c3": dict(bytes=1.902e9, source="profiles/flash_c3_c5_trace_counters.md (flash_bwd_dkdv_kernel, segment ids)"),
+    "c5": dict(bytes=24.44e9, source="profiles/flash_c3_c5_trace_counters.md (flash_bwd_dkdv_kernel)"),
+    "c4": dict(bytes=4.254e9, source="profiles/paged_decode_c4_trace_counters.md (decode_split_kernel)"),
 }
 
 METRIC = "flash-attn fwd+bwd TFLOP/s; paged-decode HBM GB/s (% roofline), 1 MI355X"
@@ -175,7 +176,7 @@ def bench_flash(cfg, steps, warmup, cpu_baseline):
     fl_dkdv, fl_dq = 4 * gemm, 1 * gemm           # S, dP, dV, dK | dQ
     tf = lambda fl, ms: fl / (ms * 1e-3) / 1e12
     dq_name = "flash_bwd_dq_stream_kernel" if spill else "flash_bwd_dq_ring_kernel"
-    traffic, traffic_src = _traffic(cfg["name"])
+    traffic, traffic_src = _traffic(cfg["name"] if (spill or cfg["name"] != "c2") else "c2_recompute")
     result = dict(
         workload=cfg["label"], value=tf(fl_fwd + fl_bwd, ms_step), unit="TFLOP/s", ms_per_step=ms_step,
         backward="dS workspace: delta, dK/dV (stores dS), dq = dS k" if spill else "dQ (recomputes dS, computes delta), dK/dV",
