@@ -513,12 +513,12 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
     }
 }
 
-#ifndef AXL_DQ_WAVES
-#define AXL_DQ_WAVES 4
-#endif
+// Wavefronts per workgroup: at head_dim 64 the kernel fits 256 registers, and eight wavefronts (two per
+// SIMD, 256 query rows share every K / V tile) are 4 % faster than four; at head_dim 128 they spill
+// (+40 %).
 template <typename E, int D, bool HAS_SEG, bool FUSE_DELTA>
 static hipError_t launch_one(const BwdArgs& a, hipStream_t stream) {
-  constexpr int NW = AXL_DQ_WAVES;
+  constexpr int NW = D == 64 ? 8 : 4;
   using Tile = DqRing<D, HAS_SEG, NW>;
   auto kernel = flash_bwd_dq_ring_kernel<E, D, HAS_SEG, NW, FUSE_DELTA>;
   hipError_t err = allow_dynamic_lds((const void*)kernel, Tile::LDS_BYTES);
