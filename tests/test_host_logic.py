@@ -348,6 +348,10 @@ def test_abi_validation_without_gpu():
     assert lib.axl_flash_bwd_workspace_bytes(ctypes.byref(bp)) == stats
     bp.mask_kind = 1
     bp.flags = 0
+    # with segment ids: the table of id ranges per 32 rows, [B, T / 32] pairs of int32, rounded to 256 bytes
+    bp.segment_ids = 256
+    assert lib.axl_flash_bwd_workspace_bytes(ctypes.byref(bp)) == stats + 256
+    bp.segment_ids = None
     assert lib.axl_flash_bwd(ctypes.byref(bp), None) == _lib.AXL_ERR_WORKSPACE
     assert lib.axl_flash_bwd_phases(ctypes.byref(bp), 0, None) == _lib.AXL_ERR_INVALID_ARGUMENT
     # Paged decode geometry.
