@@ -499,6 +499,10 @@ struct AuxArgs {
   float keep_scale;     // 1 / (1 - dropout_rate)
 };
 
+// Template argument of the kernels that are compiled once per combination of these inputs: which
+// of them there are and the element type of the bias (0 = the plain kernel).
+constexpr int kAuxBias16 = 1, kAuxBias32 = 2, kAuxDrop = 4;
+
 AuxArgs make_aux_args(const AxlAttnAux& x, float softmax_scale);
 int check_aux(const char* who, const AxlAttnAux& x, int batch, int hq, int q_len, int kv_len);
 

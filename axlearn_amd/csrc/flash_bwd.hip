@@ -183,9 +183,44 @@ __global__ __launch_bounds__(256) void flash_bwd_dq_aux_kernel(const BwdArgs a) 
     *(u32x4*)(k_st + (BUF_) * Tile::TILE_BYTES + i * ROWS_PER_PASS * Tile::STRIDE) = kreg[i];   \
     *(u32x4*)(v_st + (BUF_) * Tile::TILE_BYTES + i * ROWS_PER_PASS * Tile::STRIDE) = vreg[i];   \
   }
+  // AUX: raw bias words and dropout bytes of the lane's 4 runs of 8 keys of a tile (run i = keys
+  // 32(i/2) + 16(i%2) + 8g .. +7; an fp32 bias fills both vectors of a run, a bf16 bias repeats its one
+  // load), requested one tile ahead, together with that tile's K / V rows.  The presence tests are
+  // on the arguments, which are uniform (the row pointers differ by lane).
+  const bool has_bias = AUX && a.aux.bias != nullptr, has_drop = AUX && a.aux.drop != nullptr;
+  const int bias_shift = a.aux.bias_f32 ? 2 : 1, bias_second = a.aux.bias_f32 ? 16 : 0;
+  u32x4 bias_nx[AUX ? 8 : 1], bias_cur[AUX ? 8 : 1];
+  uint2 drop_nx[AUX ? 4 : 1], drop_cur[AUX ? 4 : 1];
+  auto aux_request = [&](int t) __attribute__((always_inline)) {
+    if constexpr (AUX) {
+      const int key0 = t * Tile::BK + 8 * g;
+      if (has_bias) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const char* p = bias_row + ((int64_t)(key0 + 32 * (i / 2) + 16 * (i % 2)) << bias_shift);
+          bias_nx[2 * i] = *(const u32x4*)p;
+          bias_nx[2 * i + 1] = *(const u32x4*)(p + bias_second);
+        }
+      }
+      if (has_drop) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) drop_nx[i] = *(const uint2*)(drop_row + key0 + 32 * (i / 2) + 16 * (i % 2));
+      }
+    }
+  };
+  auto aux_rotate = [&]() __attribute__((always_inline)) {
+    if constexpr (AUX) {
+#pragma unroll
+      for (int i = 0; i < 8; i++) bias_cur[i] = bias_nx[i];
+#pragma unroll
+      for (int i = 0; i < 4; i++) drop_cur[i] = drop_nx[i];
+    }
+  };
   if (t_begin < t_end) {
     AXL_LOAD_TILE(t_begin)
+    aux_request(t_begin);
     AXL_STORE_TILE(0)
+    aux_rotate();
   }
   wait_all_vmem();  // stationary fragments have landed: nothing issued before the loop is pending
   __syncthreads();
@@ -199,6 +234,7 @@ __global__ __launch_bounds__(256) void flash_bwd_dq_aux_kernel(const BwdArgs a) 
     const bool has_next = t + 1 < t_end;
     if (has_next) {
       AXL_LOAD_TILE(t + 1)
+      aux_request(t + 1);
     }
     const int k0 = t * Tile::BK;
     bool skip = false, need_mask = false;
@@ -234,19 +270,33 @@ __global__ __launch_bounds__(256) void flash_bwd_dq_aux_kernel(const BwdArgs a) 
         if constexpr (AUX) {
           // logits = scale * qk + bias, kept in raw units as qk + bias / scale; a dropped element
           // has dP = 0, a kept one dP / (1 - rate) (gpu_attention.py:601-603).
-          if (bias_row) {
+          if (has_bias) {
 #pragma unroll
             for (int t8 = 0; t8 < 2; t8++) {
+              const u32x4 w0 = bias_cur[2 * (2 * ks + t8)], w1 = bias_cur[2 * (2 * ks + t8) + 1];
               float bv[8];
-              load_bias<8>(bias_row, k0 + 32 * ks + 16 * t8 + 8 * g, a.aux.bias_f32, bv);
+              if (a.aux.bias_f32) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                  const unsigned lo = w0[j], hi = w1[j];
+                  bv[j] = __builtin_bit_cast(float, lo);
+                  bv[4 + j] = __builtin_bit_cast(float, hi);
+                }
+              } else {
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                  bv[2 * j] = __builtin_bit_cast(float, w0[j] << 16);
+                  bv[2 * j + 1] = __builtin_bit_cast(float, w0[j] & 0xffff0000u);
+                }
+              }
 #pragma unroll
               for (int j = 0; j < 8; j++) s[8 * t8 + j] = __builtin_fmaf(bv[j], a.aux.inv_scale, s[8 * t8 + j]);
             }
           }
-          if (drop_row) {
+          if (has_drop) {
 #pragma unroll
             for (int t8 = 0; t8 < 2; t8++) {
-              const uint2 w = *(const uint2*)(drop_row + k0 + 32 * ks + 16 * t8 + 8 * g);
+              const uint2 w = drop_cur[2 * ks + t8];
 #pragma unroll
               for (int j = 0; j < 8; j++) {
                 const unsigned byte = ((j < 4 ? w.x : w.y) >> (8 * (j % 4))) & 0xffu;
@@ -299,6 +349,7 @@ __global__ __launch_bounds__(256) void flash_bwd_dq_aux_kernel(const BwdArgs a) 
     }
     if (has_next) {
       AXL_STORE_TILE(buf ^ 1)
+      aux_rotate();
     }
     __syncthreads();
   }

@@ -55,11 +55,13 @@ constexpr int kNotUniformDkv = -0x7fffffff - 1;  // marks a tile with more than 
 
 // SPILL: the kernel also stores every tile's dS (rounded to the input dtype, as it enters the dK
 // product) into the a.ds workspace, for the streaming dQ kernel.  Causal mask with q_off 0 and T == S.
-template <typename E, int D, bool HAS_SEG, bool AUX, bool SPILL = false>
+template <typename E, int D, bool HAS_SEG, int AUX, bool SPILL = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void flash_bwd_dkdv_kernel(const BwdArgs a) {
   static_assert(!SPILL || (!HAS_SEG && !AUX), "the spill path has no segment ids, bias or dropout mask");
   using Tile = DkvTile<D>;
+  constexpr bool HAS_BIAS = (AUX & (kAuxBias16 | kAuxBias32)) != 0, BIAS_F32 = (AUX & kAuxBias32) != 0;
+  constexpr bool HAS_DROP = (AUX & kAuxDrop) != 0;
   constexpr int KK = D / 16, DT = D / 32;
   constexpr int NA = 2 * KK;          // stage-A MFMAs per tile
   constexpr int NB = 4 * DT;          // stage-B MFMAs per tile
@@ -286,9 +288,14 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
       if (HAS_SEG) sv_ = seg_v[r_ / 4][r_ % 4] == seg_k ? sv_ : kMasked;                       \
     }                                                                                          \
     float off_ = lse_v[r_ / 4][r_ % 4]; /* -lse * log2 e */                                    \
-    if constexpr (AUX) {                                                                       \
-      /* bias raw bits: fp32 as loaded, bf16 in the low half; zero when there is no bias */    \
-      off_ = __builtin_fmaf(__builtin_bit_cast(float, braw_v[r_] << bias_shift), kLog2e, off_); \
+    if constexpr (HAS_BIAS) {                                                                  \
+      /* bias raw bits: fp32 as loaded, bf16 in the low half.  The empty statement keeps the    \
+         first use of the loaded register here, an iteration after its load: without it the     \
+         shift (and the test of the dropout byte below) moves up to the load and waits there    \
+         for everything in flight. */                                                           \
+      uint32_t bw_ = braw_v[r_];                                                               \
+      asm volatile("" : "+v"(bw_));                                                            \
+      off_ = __builtin_fmaf(__builtin_bit_cast(float, bw_ << (BIAS_F32 ? 0 : 16)), kLog2e, off_); \
     }                                                                                          \
     s_e[r_] = __builtin_fmaf(sv_, c, off_);                                                    \
   }
@@ -298,8 +305,10 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
     const int r_ = (R_);                                                                       \
     const float p_ = s_e[r_];                                                                  \
     float dpv_ = dp_e[r_];                                                                     \
-    if constexpr (AUX) {                                                                       \
-      const bool kept_ = draw_v[r_] == 0;                                                      \
+    if constexpr (HAS_DROP) {                                                                  \
+      uint32_t dw_ = draw_v[r_];                                                               \
+      asm volatile("" : "+v"(dw_));                                                            \
+      const bool kept_ = dw_ == 0;                                                             \
       dpv_ = kept_ ? dpv_ * a.aux.keep_scale : 0.f; /* gpu_attention.py:509-512 */            \
       s_e[r_] = kept_ ? p_ : 0.f; /* P that multiplies dO: dropped entries removed */          \
     }                                                                                          \
@@ -313,29 +322,32 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
     AXL_ELEM_3(R_)                                                                             \
   }
   // Dense bias / dropout mask (AUX): this lane's key column of the 16 query rows of a tile, one
-  // element per register, requested a whole iteration before the elementwise stage consumes it.
-  uint32_t braw_v[16], draw_v[16];
+  // element per register, requested a whole iteration before the elementwise stage consumes it.  Two
+  // register sets swap roles from iteration to iteration (a copy would have to wait for the loads).
+  // Which inputs there are and the bias element type are template arguments, so the requests are
+  // straight-line code and the compiler's wait counts for them stay exact.
+  uint32_t braw_v[16], draw_v[16], braw_w[16], draw_w[16];
 #pragma unroll
-  for (int r = 0; r < 16; r++) braw_v[r] = draw_v[r] = 0;
-  const int bias_shift = a.aux.bias_f32 ? 0 : 16;
-  const int bias_es = a.aux.bias_f32 ? 4 : 2;
+  for (int r = 0; r < 16; r++) braw_v[r] = draw_v[r] = braw_w[r] = draw_w[r] = 0;
+  constexpr int bias_es = BIAS_F32 ? 4 : 2;
 #define AXL_AUX_ROW0(H_, Q0_, BP_, DP_)                                                              \
   {                                                                                                  \
     const int64_t head_ = hk * G + (H_), row_ = (Q0_) + 8 * g;                                       \
-    BP_ = a.aux.bias ? a.aux.bias + b * a.aux.bias_sb + head_ * a.aux.bias_sh + row_ * a.aux.bias_sr + \
-                           (int64_t)kpos * bias_es                                                   \
-                     : nullptr;                                                                      \
-    DP_ = a.aux.drop ? a.aux.drop + b * a.aux.drop_sb + head_ * a.aux.drop_sh + row_ * a.aux.drop_sr + kpos \
-                     : nullptr;                                                                      \
+    BP_ = HAS_BIAS ? a.aux.bias + b * a.aux.bias_sb + head_ * a.aux.bias_sh + row_ * a.aux.bias_sr + \
+                         (int64_t)kpos * bias_es                                                     \
+                   : nullptr;                                                                        \
+    DP_ = HAS_DROP ? a.aux.drop + b * a.aux.drop_sb + head_ * a.aux.drop_sh + row_ * a.aux.drop_sr + kpos \
+                   : nullptr;                                                                        \
   }
 #define AXL_AUX_LOAD(BP_, DP_, R_, BDST_, DDST_)                                                     \
   {                                                                                                  \
     const int64_t rr_ = 16 * ((R_) / 8) + ((R_) % 8);                                                \
-    if (BP_) {                                                                                       \
+    if constexpr (HAS_BIAS) {                                                                        \
       const char* e_ = (BP_) + rr_ * a.aux.bias_sr;                                                  \
-      BDST_[R_] = a.aux.bias_f32 ? *(const uint32_t*)e_ : (uint32_t)*(const uint16_t*)e_;            \
+      if constexpr (BIAS_F32) BDST_[R_] = *(const uint32_t*)e_;                                      \
+      else BDST_[R_] = *(const uint16_t*)e_;                                                         \
     }                                                                                                \
-    if (DP_) DDST_[R_] = *((DP_) + rr_ * a.aux.drop_sr);                                             \
+    if constexpr (HAS_DROP) DDST_[R_] = *((DP_) + rr_ * a.aux.drop_sr);                              \
   }
 #define AXL_PACK_PAIR(PB_, DSB_, I_)                                    \
   {                                                                     \
@@ -481,7 +493,8 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
   // first read of dp two slots later.  The bias / dropout instantiations, which run out of vector
   // registers, keep the compiler's own form.
   auto iter = [&](floatx16& s_e, floatx16& dp_e, PackedOperand& pb, PackedOperand& dsb, floatx16& s_a, floatx16& dp_a,
-                  PackedOperand& pb_n, PackedOperand& dsb_n) __attribute__((always_inline)) {
+                  PackedOperand& pb_n, PackedOperand& dsb_n, uint32_t (&braw_v)[16], uint32_t (&draw_v)[16],
+                  uint32_t (&braw_n)[16], uint32_t (&draw_n)[16]) __attribute__((always_inline)) {
     bf16x8 afr[NA];
     TrFrag bfr[NB];
 #pragma unroll
@@ -500,14 +513,9 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
       e_ad[0][dt] = buf_e + tb_off[0][dt];
       e_ad[1][dt] = buf_e + tb_off[1][dt];
     }
-    uint32_t braw_n[16], draw_n[16];     // bias / dropout columns of tile j + 2
-    const char* bias_t = nullptr;
+    const char* bias_t = nullptr;        // bias / dropout columns of tile j + 2 go to (braw_n, draw_n)
     const uint8_t* drop_t = nullptr;
-    if constexpr (AUX) {
-#pragma unroll
-      for (int r = 0; r < 16; r++) braw_n[r] = draw_n[r] = 0;
-      AXL_AUX_ROW0(h_a, q0_a, bias_t, drop_t)
-    }
+    if constexpr (AUX) AXL_AUX_ROW0(h_a, q0_a, bias_t, drop_t)
     if constexpr (SPILL) {
       // dS of tile j (this iteration's stage-B operand), ahead of the iteration's tile loads: by the
       // end of the iteration the stores have long been accepted.
@@ -615,13 +623,6 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
     buf_n = buf_s;
     buf_s = buf_s2;
     buf_s2 = tmp;
-    if constexpr (AUX) {
-#pragma unroll
-      for (int r = 0; r < 16; r++) {
-        braw_v[r] = braw_n[r];
-        draw_v[r] = draw_n[r];
-      }
-    }
     diff0 = (q0_a + a.q_off + 8 * g) - kpos;
     q0_a = q0_s;
     q0_s = q0_s2;
@@ -632,17 +633,24 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
   };
     int j = j_from;
     for (; j + 1 < j_to; j += 2) {
-      iter(s_e, dp_e, pb, dsb, s_x, dp_x, pb_x, dsb_x);
-      iter(s_x, dp_x, pb_x, dsb_x, s_e, dp_e, pb, dsb);
+      iter(s_e, dp_e, pb, dsb, s_x, dp_x, pb_x, dsb_x, braw_v, draw_v, braw_w, draw_w);
+      iter(s_x, dp_x, pb_x, dsb_x, s_e, dp_e, pb, dsb, braw_w, draw_w, braw_v, draw_v);
     }
     if (j < j_to) {
       // odd count: one more iteration, then the sets go back to their roles with one copy per run
-      iter(s_e, dp_e, pb, dsb, s_x, dp_x, pb_x, dsb_x);
+      iter(s_e, dp_e, pb, dsb, s_x, dp_x, pb_x, dsb_x, braw_v, draw_v, braw_w, draw_w);
       if constexpr (!AUX) asm volatile("s_nop 15\n\ts_nop 3" : "+v"(s_x), "+v"(dp_x));  // the chains have just ended
       s_e = s_x;
       dp_e = dp_x;
       pb = pb_x;
       dsb = dsb_x;
+      if constexpr (AUX) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          braw_v[r] = braw_w[r];
+          draw_v[r] = draw_w[r];
+        }
+      }
     }
   };
   // Query tile t (counted from t_begin) needs no mask for this wavefront's 32 keys when its queries
@@ -737,7 +745,7 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
     }
 }
 
-template <typename E, int D, bool HAS_SEG, bool AUX, bool SPILL = false>
+template <typename E, int D, bool HAS_SEG, int AUX, bool SPILL = false>
 static hipError_t launch_one(const BwdArgs& a, hipStream_t stream) {
   using Tile = DkvTile<D>;
   auto kernel = flash_bwd_dkdv_kernel<E, D, HAS_SEG, AUX, SPILL>;
@@ -748,20 +756,32 @@ static hipError_t launch_one(const BwdArgs& a, hipStream_t stream) {
   return hipGetLastError();
 }
 
+template <typename E, int D, int AUX>
+static hipError_t launch_seg(const BwdArgs& a, hipStream_t stream) {
+  return a.seg ? launch_one<E, D, true, AUX>(a, stream) : launch_one<E, D, false, AUX>(a, stream);
+}
+
+template <typename E, int D>
+static hipError_t launch_aux(const BwdArgs& a, hipStream_t stream) {
+  const int bias = a.aux.bias ? (a.aux.bias_f32 ? kAuxBias32 : kAuxBias16) : 0;
+  const int mode = bias | (a.aux.drop ? kAuxDrop : 0);
+  switch (mode) {
+    case kAuxBias16: return launch_seg<E, D, kAuxBias16>(a, stream);
+    case kAuxBias32: return launch_seg<E, D, kAuxBias32>(a, stream);
+    case kAuxDrop: return launch_seg<E, D, kAuxDrop>(a, stream);
+    case kAuxBias16 | kAuxDrop: return launch_seg<E, D, kAuxBias16 | kAuxDrop>(a, stream);
+    default: return launch_seg<E, D, kAuxBias32 | kAuxDrop>(a, stream);
+  }
+}
+
 template <typename E>
 static hipError_t launch_for(const BwdArgs& a, int head_dim, bool aux, hipStream_t stream) {
   const bool seg = a.seg != nullptr;
-  if (aux) {
-    if (head_dim == 128)
-      return seg ? launch_one<E, 128, true, true>(a, stream) : launch_one<E, 128, false, true>(a, stream);
-    return seg ? launch_one<E, 64, true, true>(a, stream) : launch_one<E, 64, false, true>(a, stream);
-  }
+  if (aux) return head_dim == 128 ? launch_aux<E, 128>(a, stream) : launch_aux<E, 64>(a, stream);
   if (a.ds && !seg)
-    return head_dim == 128 ? launch_one<E, 128, false, false, true>(a, stream)
-                           : launch_one<E, 64, false, false, true>(a, stream);
-  if (head_dim == 128)
-    return seg ? launch_one<E, 128, true, false>(a, stream) : launch_one<E, 128, false, false>(a, stream);
-  return seg ? launch_one<E, 64, true, false>(a, stream) : launch_one<E, 64, false, false>(a, stream);
+    return head_dim == 128 ? launch_one<E, 128, false, 0, true>(a, stream)
+                           : launch_one<E, 64, false, 0, true>(a, stream);
+  return head_dim == 128 ? launch_seg<E, 128, 0>(a, stream) : launch_seg<E, 64, 0>(a, stream);
 }
 
 hipError_t launch_bwd_dkdv(const BwdArgs& a, int dtype, int head_dim, bool aux, hipStream_t stream) {

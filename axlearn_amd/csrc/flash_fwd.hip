@@ -63,7 +63,7 @@ constexpr int kMaxSegTiles = 1024;               // key tiles whose segment ids 
 constexpr int kSegNotUniform = -0x7fffffff - 1;  // marks a tile with more than one segment id
 
 template <typename E, int D, bool AUX, int NW = 4>
-__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(2, 2)))
+__global__ __launch_bounds__(64 * NW) __attribute__((amdgpu_waves_per_eu(AUX ? 1 : 2, AUX ? 1 : 2)))
 void flash_fwd_kernel(const FwdArgs a) {
   using Tile = FwdTile<D, NW>;
   constexpr int KK = D / 16;  // MFMA k-steps over head_dim
@@ -227,6 +227,34 @@ void flash_fwd_kernel(const FwdArgs a) {
         S_[ks] = E::mfma_32x32x16(AXL_K_FRAG(KT_, kk, ks), qf[kk], S_[ks]); \
   }
 
+  // AUX: raw bias words and dropout bytes of the lane's 4 runs of 8 keys, requested one tile ahead
+  // with ordinary (compiler-tracked) loads.  Run i covers keys 32(i/2) + 16(i%2) + 8g .. +7 of the tile;
+  // an fp32 bias fills both vectors of a run, a bf16 bias the first.
+  u32x4 bias_nx[AUX ? 8 : 1];
+  uint2 drop_nx[AUX ? 4 : 1];
+  // Both tests are uniform (the row pointers are not: they differ by lane).  A bf16 bias repeats its
+  // one load so that the request is the same straight-line code for both element types.
+  const bool has_bias = AUX && a.aux.bias != nullptr, has_drop = AUX && a.aux.drop != nullptr;
+  const int bias_shift = a.aux.bias_f32 ? 2 : 1, bias_second = a.aux.bias_f32 ? 16 : 0;
+  auto aux_request = [&](int t) __attribute__((always_inline)) {
+    if constexpr (AUX) {
+      const int k0 = t * Tile::BK + 8 * g;
+      if (has_bias) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const char* p = bias_row + ((int64_t)(k0 + 32 * (i / 2) + 16 * (i % 2)) << bias_shift);
+          bias_nx[2 * i] = *(const u32x4*)p;
+          bias_nx[2 * i + 1] = *(const u32x4*)(p + bias_second);
+        }
+      }
+      if (has_drop) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) drop_nx[i] = *(const uint2*)(drop_row + k0 + 32 * (i / 2) + 16 * (i % 2));
+      }
+    }
+  };
+  if (t_begin < t_end && t_begin >= tw_begin && t_begin < tw_end) aux_request(t_begin);
+
   // Pipeline fill: S^T of the first tile.
   wait_vmem_le<0>();
   __syncthreads();
@@ -247,17 +275,54 @@ void flash_fwd_kernel(const FwdArgs a) {
     // with K(t+2) and V(t+1).
     wait_vmem_le<0>();
     __syncthreads();
-    if constexpr (!FAST) {
-      if (t + 2 < t_end) issue_k(t + 2, buf);
-      if (t + 1 < t_end) issue_v(t + 1, buf ^ 1);
-    }
-    // FAST tiles issue the same loads one pair per MFMA slot further down, where their issue time
+    // FAST tiles issue the tile loads one pair per MFMA slot further down, where their issue time
     // overlaps the matrix pipe's work; K(t+2) may not exist (t + 2 == t_end), then the last tile is
     // fetched again into a buffer that nobody reads any more.
     const int t_k2 = min(t + 2, t_end - 1);
 
     const bool do_sm = FAST || (t >= tw_begin && t < tw_end);          // softmax and PV of tile t
     const bool do_s = FAST || (t + 1 >= tw_begin && t + 1 < tw_end);   // S of tile t + 1
+    // Bias and dropout bytes of tile t arrived with the wait above (they were requested one tile
+    // ago, ahead of that tile's K / V loads); they are consumed here, before anything else is
+    // requested, so the compiler's own wait for them finds the counter at zero already.
+    uint2 dm[2][2] = {};  // dropout bytes of the lane's 4 runs of 8 keys
+    if constexpr (AUX && !FAST) {
+      if (do_sm) {
+        if (has_bias) {
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            float bv[8];
+            if (a.aux.bias_f32) {
+#pragma unroll
+              for (int j = 0; j < 4; j++) {
+                // (copies first: a bit cast applied to the vector element itself reads element 0)
+                const unsigned w0 = bias_nx[2 * i][j], w1 = bias_nx[2 * i + 1][j];
+                bv[j] = __builtin_bit_cast(float, w0);
+                bv[4 + j] = __builtin_bit_cast(float, w1);
+              }
+            } else {
+#pragma unroll
+              for (int j = 0; j < 4; j++) {
+                bv[2 * j] = __builtin_bit_cast(float, bias_nx[2 * i][j] << 16);
+                bv[2 * j + 1] = __builtin_bit_cast(float, bias_nx[2 * i][j] & 0xffff0000u);
+              }
+            }
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+              s[i / 2][8 * (i % 2) + j] = __builtin_fmaf(bv[j], a.aux.inv_scale, s[i / 2][8 * (i % 2) + j]);
+          }
+        }
+        if (has_drop) {
+#pragma unroll
+          for (int i = 0; i < 4; i++) dm[i / 2][i % 2] = drop_nx[i];
+        }
+      }
+      if (do_s) aux_request(t + 1);
+    }
+    if constexpr (!FAST) {
+      if (t + 2 < t_end) issue_k(t + 2, buf);
+      if (t + 1 < t_end) issue_v(t + 1, buf ^ 1);
+    }
     const char* kt = k_lds + (buf ^ 1) * Tile::TILE_BYTES;   // K(t+1)
     const char* vt = v_lds + buf * Tile::TILE_BYTES;         // V(t)
     const int k0 = t * Tile::BK;
@@ -267,28 +332,6 @@ void flash_fwd_kernel(const FwdArgs a) {
     }
 
     // ---- masks of tile t.  Register r of sub-tile ks in lane group g is key k0 + 32ks + 16(r/8) + 8g + (r%8).
-    uint2 dm[2][2] = {};  // dropout bytes of the lane's 4 runs of 8 keys
-    if constexpr (AUX && !FAST) {
-      if (bias_row) {
-#pragma unroll
-        for (int ks = 0; ks < 2; ks++)
-#pragma unroll
-          for (int t8 = 0; t8 < 2; t8++) {
-            float bv[8];
-            load_bias<8>(bias_row, k0 + 32 * ks + 16 * t8 + 8 * g, a.aux.bias_f32, bv);
-#pragma unroll
-            for (int j = 0; j < 8; j++)
-              s[ks][8 * t8 + j] = __builtin_fmaf(bv[j], a.aux.inv_scale, s[ks][8 * t8 + j]);
-          }
-      }
-      if (drop_row) {
-#pragma unroll
-        for (int ks = 0; ks < 2; ks++)
-#pragma unroll
-          for (int t8 = 0; t8 < 2; t8++)
-            dm[ks][t8] = *(const uint2*)(drop_row + k0 + 32 * ks + 16 * t8 + 8 * g);
-      }
-    }
     // Probability that enters P V: zero where the dropout mask says so (the row sum keeps it).
     auto after_dropout = [&](int idx, float p) {
       if constexpr (AUX) {

@@ -504,8 +504,8 @@ def test_dkdv_kernel_keeps_its_vector_register_accumulators_in_place():
     seen = 0
     for block in out.stderr.split("Function Name: ")[1:]:
         name = block.split()[0]
-        m = re.match(r"_ZN3axl21flash_bwd_dkdv_kernelINS_\d+Elem\w+ELi(\d+)ELb([01])ELb([01])ELb([01])EEE", name)
-        if not m or m.group(3) == "1":  # other kernels; bias / dropout instantiations use the compiler's own form
+        m = re.match(r"_ZN3axl21flash_bwd_dkdv_kernelINS_\d+Elem\w+ELi(\d+)ELb([01])ELi(\d+)ELb([01])EEE", name)
+        if not m or m.group(3) != "0":  # other kernels; bias / dropout instantiations use the compiler's own form
             continue
         agprs = int(re.search(r"AGPRs: (\d+)", block).group(1))
         scratch = int(re.search(r"ScratchSize \[bytes/lane\]: (\d+)", block).group(1))
