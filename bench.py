@@ -7,7 +7,8 @@ backward, bf16, batch 4, 32 query heads / 8 kv heads, seq 4096, head_dim 128: a 
 (axl_flash_fwd) plus one backward (axl_flash_bwd) over one synthetic batch already resident in HBM.
 The backward of the headline step keeps dS in a workspace the caller provides (AXL_BWD_DS_WORKSPACE);
 `c2_recompute` in the same line is the same step through the backward that recomputes dS instead
-(`--recompute` makes that one the headline).
+(`--recompute` makes that one the headline).  `c5`, the other plain causal workload, is reported the
+same way (`c5` with the workspace, 69 GB at that length, and `c5_recompute`).
 The paged-decode half of the metric (configs[3], "C4") is measured in the same run and reported in
 the `paged_decode` object of the same JSON line.  With the default `--workload all` the line also
 carries `c1` (configs[0]: the fp32 case the reference itself runs on CPU), `c3` (sliding window +
@@ -52,9 +53,14 @@ TRAFFIC = {
     "c2": dict(bytes=3.205e9, source="profiles/flash_c2_trace_counters.md (flash_bwd_dkdv_kernel, dS-workspace step)"),
     "c2_recompute": dict(bytes=0.983e9, source="profiles/flash_c2_trace_counters.md (flash_bwd_dkdv_kernel, --recompute)"),
     "c3": dict(bytes=1.902e9, source="profiles/flash_c3_c5_trace_counters.md (flash_bwd_dkdv_kernel, segment ids)"),
-    "c5": dict(bytes=24.44e9, source="profiles/flash_c3_c5_trace_counters.md (flash_bwd_dkdv_kernel)"),
+    "c5": dict(bytes=24.44e9, source="profiles/flash_c3_c5_trace_counters.md (flash_bwd_dkdv_kernel, dS-workspace step)"),
+    "c5_recompute": dict(bytes=24.44e9, source="profiles/flash_c3_c5_trace_counters.md (flash_bwd_dkdv_kernel, --recompute)"),
     "c4": dict(bytes=4.254e9, source="profiles/paged_decode_c4_trace_counters.md (decode_split_kernel)"),
 }
+
+# Plain causal workloads: their default step runs the backward that keeps dS in a caller-provided
+# workspace (AXL_BWD_DS_WORKSPACE: 5 executed GEMMs instead of 7; 2.1 GB for C2, 69 GB for C5).
+DS_WORKSPACE_WORKLOADS = ("c2", "c5")
 
 METRIC = "flash-attn fwd+bwd TFLOP/s; paged-decode HBM GB/s (% roofline), 1 MI355X"
 
@@ -176,7 +182,7 @@ def bench_flash(cfg, steps, warmup, cpu_baseline):
     fl_dkdv, fl_dq = 4 * gemm, 1 * gemm           # S, dP, dV, dK | dQ
     tf = lambda fl, ms: fl / (ms * 1e-3) / 1e12
     dq_name = "flash_bwd_dq_stream_kernel" if spill else "flash_bwd_dq_ring_kernel"
-    traffic, traffic_src = _traffic(cfg["name"] if (spill or cfg["name"] != "c2") else "c2_recompute")
+    traffic, traffic_src = _traffic(cfg["name"] + ("_recompute" if cfg["name"] in DS_WORKSPACE_WORKLOADS and not spill else ""))
     result = dict(
         workload=cfg["label"], value=tf(fl_fwd + fl_bwd, ms_step), unit="TFLOP/s", ms_per_step=ms_step,
         backward="dS workspace: delta, dK/dV (stores dS), dq = dS k" if spill else "dQ (recomputes dS, computes delta), dK/dV",
@@ -407,9 +413,7 @@ def main():
         line["c1"] = res
     else:
         cfg = _flash_workload("c2" if args.workload == "all" else args.workload)
-        if cfg["name"] == "c2" and not args.recompute:
-            # The headline step runs the backward that keeps dS in a caller-provided workspace
-            # (AXL_BWD_DS_WORKSPACE: 5 executed GEMMs instead of 7; plain causal attention only).
+        if cfg["name"] in DS_WORKSPACE_WORKLOADS and not args.recompute:
             cfg = dict(cfg, ds_workspace=True)
         res = bench_flash(cfg, args.steps, args.warmup, cpu_base)
         line.update(value=res["value"], unit="TFLOP/s", ms_per_step=res["ms_per_step"],
@@ -432,7 +436,10 @@ def main():
             line["machine"] = calibrate_mfma()
             line["c1"] = bench_c1(args.steps, args.warmup, cpu_base)
             line["c3"] = bench_flash(_flash_workload("c3"), max(5, args.steps // 2), 2, cpu_base)
-            line["c5"] = bench_flash(_flash_workload("c5"), max(3, args.steps // 4), 1, cpu_base)
+            c5 = dict(_flash_workload("c5"), ds_workspace=not args.recompute)
+            line["c5"] = bench_flash(c5, max(3, args.steps // 4), 1, cpu_base)
+            line["c5_recompute" if c5["ds_workspace"] else "c5_ds_workspace"] = bench_flash(
+                dict(c5, ds_workspace=not c5["ds_workspace"]), max(3, args.steps // 4), 1, False)
     print(json.dumps(line))
 
 
