@@ -53,8 +53,8 @@ TRAFFIC = {
     "c2": dict(bytes=3.205e9, source="profiles/flash_c2_trace_counters.md (flash_bwd_dkdv_kernel, dS-workspace step)"),
     "c2_recompute": dict(bytes=0.983e9, source="profiles/flash_c2_trace_counters.md (flash_bwd_dkdv_kernel, --recompute)"),
     "c3": dict(bytes=1.902e9, source="profiles/flash_c3_c5_trace_counters.md (flash_bwd_dkdv_kernel, segment ids)"),
-    "c5": dict(bytes=24.44e9, source="profiles/flash_c3_c5_trace_counters.md (flash_bwd_dkdv_kernel, dS-workspace step)"),
-    "c5_recompute": dict(bytes=24.44e9, source="profiles/flash_c3_c5_trace_counters.md (flash_bwd_dkdv_kernel, --recompute)"),
+    "c5": dict(bytes=88.15e9, source="profiles/flash_c3_c5_trace_counters.md (flash_bwd_dkdv_kernel, dS-workspace step)"),
+    "c5_recompute": dict(bytes=24.17e9, source="profiles/flash_c3_c5_trace_counters.md (flash_bwd_dkdv_kernel, --recompute)"),
     "c4": dict(bytes=4.254e9, source="profiles/paged_decode_c4_trace_counters.md (decode_split_kernel)"),
 }
 
