@@ -20,6 +20,8 @@ struct BwdArgs {
   void* dv;
   const int32_t* seg;
   const int2* seg_tbl;  // workspace [B, T / 32]: smallest and largest segment id of every 32 rows (with seg)
+  int2* kb_tbl;         // workspace [B, S / 128]: the query tiles [first, end) whose dS each key block's dK/dV
+                        // workgroups store (spill path under a sliding window or segment ids), or nullptr
   Strides3 qs, ks, vs, os, dos, dqs, dks, dvs;
   int B, T, S, Hq, Hkv;
   int mask_kind, window, q_off;
@@ -27,7 +29,10 @@ struct BwdArgs {
   AuxArgs aux;  // dense bias / dropout mask (read only by the AUX instantiations)
 };
 
-// dS workspace of the spill path (causal mask, q_pos_offset 0, q_len == kv_len).  A block is the dS
+// Most key blocks (of 128 keys) the spill path handles when the stored tiles depend on the key block.
+constexpr int kMaxKbRanged = 512;
+
+// dS workspace of the spill path (causal or sliding-window mask, q_pos_offset 0, q_len == kv_len).  A block is the dS
 // of 32 queries x 32 keys as [query half 2][key 32][16 queries] in the input dtype: 2 KB.  Query tile
 // t = 4a + r (32 rows) of a head has a run of ds_run_blocks(t) = 4(a+1) blocks, one per 32 keys that the
 // 128 query rows of block a can see.  Per (batch, kv head) pair the runs are ordered by tile, then by
@@ -51,11 +56,12 @@ __host__ __device__ inline int64_t ds_run_start(int64_t pair, int T, int G, int 
 
 // Enqueues the dK/dV kernel for `dtype` AXL_BF16 or AXL_F16 and head_dim 64 or 128; `aux` selects
 // the instantiation that reads the dense bias / dropout mask.  With a.ds set (and no bias / dropout
-// mask / segment ids, causal mask, q_off 0, T == S) the kernel also stores dS for
-// launch_bwd_dq_stream.
+// mask, causal or sliding-window mask, q_off 0, T == S) the kernel also stores dS for
+// launch_bwd_dq_stream, and with a.kb_tbl set the range of query tiles each key block stored.
 hipError_t launch_bwd_dkdv(const BwdArgs& a, int dtype, int head_dim, bool aux, hipStream_t stream);
 
-// Enqueues the streaming dQ kernel, dq = scale * dS k from the dS blocks in a.ds.
+// Enqueues the streaming dQ kernel, dq = scale * dS k from the dS blocks in a.ds (with a.kb_tbl set:
+// from the blocks that table says were stored).
 hipError_t launch_bwd_dq_stream(const BwdArgs& a, int dtype, int head_dim, hipStream_t stream);
 
 // Enqueues the dQ kernel (no dense bias / dropout mask) for `dtype` AXL_BF16 or AXL_F16 and head_dim

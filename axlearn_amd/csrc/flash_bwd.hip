@@ -393,11 +393,17 @@ static size_t stats_bytes(const AxlFlashBwdParams& p) {
 }
 
 // The dS-spill path: the dK/dV kernel stores dS and the dQ kernel becomes one streaming GEMM
-// (5 executed GEMMs instead of 7).  Plain causal attention over equal lengths only.
+// (5 executed GEMMs instead of 7).  Causal or sliding-window attention over equal lengths, with or
+// without segment ids.
+static bool spill_ranged(const AxlFlashBwdParams& p) {
+  return p.mask_kind == AXL_MASK_SLIDING_WINDOW || p.segment_ids;
+}
 static bool spill_eligible(const AxlFlashBwdParams& p) {
-  return (p.dtype == AXL_BF16 || p.dtype == AXL_F16) && p.mask_kind == AXL_MASK_CAUSAL && p.q_pos_offset == 0 &&
-         p.q_len == p.kv_len && !p.segment_ids && !p.aux.bias && !p.aux.dropout_mask &&
-         (p.flags & AXL_BWD_DS_WORKSPACE);
+  return (p.dtype == AXL_BF16 || p.dtype == AXL_F16) &&
+         (p.mask_kind == AXL_MASK_CAUSAL || p.mask_kind == AXL_MASK_SLIDING_WINDOW) && p.q_pos_offset == 0 &&
+         p.q_len == p.kv_len && !p.aux.bias && !p.aux.dropout_mask && (p.flags & AXL_BWD_DS_WORKSPACE) &&
+         // the ranged kernel keeps the table in LDS beside its ring: 256-row blocks at head_dim 128
+         (!spill_ranged(p) || (p.kv_len / 128 <= kMaxKbRanged && (p.head_dim != 128 || p.q_len % 256 == 0)));
 }
 
 static size_t spill_bytes(const AxlFlashBwdParams& p) {
@@ -410,8 +416,14 @@ static size_t seg_table_bytes(const AxlFlashBwdParams& p) {
   return ((size_t)p.batch * (p.q_len / kSegGroupRows) * sizeof(int2) + 255) & ~(size_t)255;
 }
 
+// Spill path under a sliding window or with segment ids: the query tiles each key block stored dS for.
+static size_t kb_table_bytes(const AxlFlashBwdParams& p) {
+  if (!spill_eligible(p) || !spill_ranged(p)) return 0;
+  return ((size_t)p.batch * (p.kv_len / 128) * sizeof(int2) + 255) & ~(size_t)255;
+}
+
 size_t flash_bwd_workspace_bytes(const AxlFlashBwdParams& p) {
-  return stats_bytes(p) + seg_table_bytes(p) + (spill_eligible(p) ? spill_bytes(p) : 0);
+  return stats_bytes(p) + seg_table_bytes(p) + kb_table_bytes(p) + (spill_eligible(p) ? spill_bytes(p) : 0);
 }
 
 int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream) {
@@ -423,7 +435,8 @@ int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream)
   a.dq = p.dq; a.dk = p.dk; a.dv = p.dv; a.seg = p.segment_ids;
   const bool spill = spill_eligible(p);  // the entry point has checked that the workspace holds dS as well
   a.seg_tbl = p.segment_ids ? (const int2*)((char*)p.workspace + stats_bytes(p)) : nullptr;
-  a.ds = spill ? (char*)p.workspace + stats_bytes(p) + seg_table_bytes(p) : nullptr;
+  a.kb_tbl = kb_table_bytes(p) ? (int2*)((char*)p.workspace + stats_bytes(p) + seg_table_bytes(p)) : nullptr;
+  a.ds = spill ? (char*)p.workspace + stats_bytes(p) + seg_table_bytes(p) + kb_table_bytes(p) : nullptr;
   a.qs = to_s3(p.q_strides); a.ks = to_s3(p.k_strides); a.vs = to_s3(p.v_strides);
   a.os = to_s3(p.out_strides); a.dos = to_s3(p.d_out_strides); a.dqs = to_s3(p.dq_strides);
   a.dks = to_s3(p.dk_strides); a.dvs = to_s3(p.dv_strides);

@@ -54,11 +54,12 @@ constexpr int kMaxSubDkv = 1024;                 // query tiles whose segment id
 constexpr int kNotUniformDkv = -0x7fffffff - 1;  // marks a tile with more than one segment id
 
 // SPILL: the kernel also stores every tile's dS (rounded to the input dtype, as it enters the dK
-// product) into the a.ds workspace, for the streaming dQ kernel.  Causal mask with q_off 0 and T == S.
+// product) into the a.ds workspace, for the streaming dQ kernel.  Causal or sliding-window mask with
+// q_off 0 and T == S; masked elements are stored as the zeros they are.
 template <typename E, int D, bool HAS_SEG, int AUX, bool SPILL = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
 void flash_bwd_dkdv_kernel(const BwdArgs a) {
-  static_assert(!SPILL || (!HAS_SEG && !AUX), "the spill path has no segment ids, bias or dropout mask");
+  static_assert(!SPILL || !AUX, "the spill path has no bias or dropout mask");
   using Tile = DkvTile<D>;
   constexpr bool HAS_BIAS = (AUX & (kAuxBias16 | kAuxBias32)) != 0, BIAS_F32 = (AUX & kAuxBias32) != 0;
   constexpr bool HAS_DROP = (AUX & kAuxDrop) != 0;
@@ -125,6 +126,10 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
                                               AUX ? 0 : kMaxSubDkv, kNotUniformDkv);
   const int t_begin = q_begin / Tile::BQ;
   const int nt = max(0, (q_end + Tile::BQ - 1) / Tile::BQ - t_begin);
+  if constexpr (SPILL) {
+    // which tiles' dS this key block stores, for the streaming dQ kernel (the same for every kv head)
+    if (a.kb_tbl && hk == 0 && tid == 0) a.kb_tbl[b * nkb + kb] = make_int2(t_begin, t_begin + nt);
+  }
   // Tiles in processing order: query tile (outer, from the LAST one down to the diagonal) x query head
   // (inner).  Every workgroup of a (batch, kv head) pair starts at the same last tile and walks down
   // until it reaches its own diagonal, so the workgroups that run together read the same Q / dO rows
@@ -778,9 +783,11 @@ template <typename E>
 static hipError_t launch_for(const BwdArgs& a, int head_dim, bool aux, hipStream_t stream) {
   const bool seg = a.seg != nullptr;
   if (aux) return head_dim == 128 ? launch_aux<E, 128>(a, stream) : launch_aux<E, 64>(a, stream);
-  if (a.ds && !seg)
-    return head_dim == 128 ? launch_one<E, 128, false, 0, true>(a, stream)
-                           : launch_one<E, 64, false, 0, true>(a, stream);
+  if (a.ds) {
+    if (head_dim == 128)
+      return seg ? launch_one<E, 128, true, 0, true>(a, stream) : launch_one<E, 128, false, 0, true>(a, stream);
+    return seg ? launch_one<E, 64, true, 0, true>(a, stream) : launch_one<E, 64, false, 0, true>(a, stream);
+  }
   return head_dim == 128 ? launch_seg<E, 128, 0>(a, stream) : launch_seg<E, 64, 0>(a, stream);
 }
 

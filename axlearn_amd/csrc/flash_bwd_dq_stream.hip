@@ -43,7 +43,10 @@ struct DqStream {
   static constexpr int LDS_BYTES = NBUF * BUF_BYTES;
 };
 
-template <typename E, int D, int NW>
+// RANGED: under a sliding window or with segment ids a key block's dK/dV workgroups store the dS of
+// the query tiles [first, end) that a.kb_tbl records for it; the other blocks of the workspace hold
+// nothing and are skipped (their loads are pointed at the first block, their MFMAs left out).
+template <typename E, int D, int NW, bool RANGED>
 __global__ __launch_bounds__(64 * NW) void flash_bwd_dq_stream_kernel(const BwdArgs a) {
   using Tile = DqStream<D, NW>;
   constexpr int DT = D / 32;
@@ -56,8 +59,52 @@ __global__ __launch_bounds__(64 * NW) void flash_bwd_dq_stream_kernel(const BwdA
   const int hk = h / (a.Hq / a.Hkv);
   const int q0 = qb * Tile::BQ + wave * 32;
   const int t_q = NW * qb + wave;            // this wavefront's query tile
-  const int trips = 2 * ((NW * qb + NW - 1) / 4 + 1);  // 64-key tiles up to and including the last diagonal block
+  int trips = 2 * ((NW * qb + NW - 1) / 4 + 1);  // 64-key tiles up to and including the last diagonal block
   const int my_trips = __builtin_amdgcn_readfirstlane(2 * (t_q / 4 + 1));  // ... of this wavefront's own 128-row block
+  int trip0 = 0;                                 // first 64-key tile that any of the workgroup's query tiles has dS for
+  __shared__ int2 s_rng[RANGED ? kMaxKbRanged : 1];
+  __shared__ int s_first[RANGED ? NW : 1], s_last[RANGED ? NW : 1];
+  if constexpr (RANGED) {
+    const int nkb = trips / 2;
+    const int2* tbl = a.kb_tbl + (int64_t)b * (a.S / 128);
+    int first = 0x7fffffff, last = -1;
+    for (int i = tid; i < nkb; i += 64 * NW) {
+      const int2 r = tbl[i];
+      s_rng[i] = r;
+      if (r.x < NW * qb + NW && r.y > NW * qb) {   // [r.x, r.y) meets the workgroup's tiles
+        first = min(first, i);
+        last = max(last, i);
+      }
+    }
+#pragma unroll
+    for (int off = 32; off; off >>= 1) {
+      first = min(first, __shfl_xor(first, off));
+      last = max(last, __shfl_xor(last, off));
+    }
+    if (lane == 0) {
+      s_first[wave] = first;
+      s_last[wave] = last;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int w = 0; w < NW; w++) {
+      first = min(first, s_first[w]);
+      last = max(last, s_last[w]);
+    }
+    first = __builtin_amdgcn_readfirstlane(first);
+    last = __builtin_amdgcn_readfirstlane(last);
+    trip0 = last < 0 ? 0 : 2 * first;
+    trips = last < 0 ? 0 : 2 * (last + 1);
+  }
+  // Does this wavefront's query tile have dS for the key block of 64-key tile `trip`?
+  auto has_ds = [&](int trip) __attribute__((always_inline)) {
+    if constexpr (RANGED) {
+      const int2 r = s_rng[trip >> 1];
+      return __builtin_amdgcn_readfirstlane((int)(r.x <= t_q && t_q < r.y)) != 0;
+    } else {
+      return true;
+    }
+  };
 
   floatx16 dq_acc[DT];
 #pragma unroll
@@ -77,10 +124,11 @@ __global__ __launch_bounds__(64 * NW) void flash_bwd_dq_stream_kernel(const BwdA
     k_lane[i] = (unsigned)(row * (int)a.ks.s + chunk * 8) * 2 - (i % 2) * 1024;
   }
   static_assert(Tile::K_DMA_PER_WAVE % 2 == 0, "K loads are issued in pairs");
-  const __bf16* k_src = (const __bf16*)a.k + b * a.ks.b + hk * a.ks.h;
   const int64_t k_step = (int64_t)Tile::BK * a.ks.s;
+  const __bf16* k_src = (const __bf16*)a.k + b * a.ks.b + hk * a.ks.h + trip0 * k_step;
   const int G = a.Hq / a.Hkv;
-  const char* ds_src = (const char*)a.ds + ds_run_start((int64_t)b * a.Hkv + hk, a.T, G, t_q, h - hk * G) * kDsBlockBytes;
+  const char* ds_src = (const char*)a.ds + ds_run_start((int64_t)b * a.Hkv + hk, a.T, G, t_q, h - hk * G) * kDsBlockBytes +
+                       (int64_t)trip0 * Tile::DS_WAVE_BYTES;
   const unsigned ds_lane = 16 * lane;
   const unsigned lds0 = lds_address(smem);
 #define AXL_DMA_TRIP(BUF_)                                                                         \
@@ -89,12 +137,13 @@ __global__ __launch_bounds__(64 * NW) void flash_bwd_dq_stream_kernel(const BwdA
     _Pragma("unroll") for (int i = 0; i < Tile::K_DMA_PER_WAVE; i += 2)                           \
       dma16x2(k_lane[i], k_lane[i + 1], k_src, kdst_ + i * 1024);                                 \
     const unsigned ddst_ = lds0 + (BUF_) * Tile::BUF_BYTES + Tile::DS_BASE + wave * Tile::DS_WAVE_BYTES; \
+    const char* dsrc_ = has_ds(pf) ? ds_src : (const char*)a.ds;                                  \
     _Pragma("unroll") for (int i = 0; i < Tile::DS_WAVE_BYTES / 2048; i++)                        \
-      dma16x2(ds_lane, ds_lane, ds_src + i * 2048, ddst_ + i * 2048);                             \
+      dma16x2(ds_lane, ds_lane, dsrc_ + i * 2048, ddst_ + i * 2048);                              \
   }
   // Prefetch cursor; it stops at the last trip (re-fetching that trip is harmless), the dS part of it
   // at the last trip of this wavefront's own run of blocks.
-  int pf = 0;
+  int pf = trip0;
 #define AXL_ADVANCE()                                                       \
   {                                                                         \
     const bool adv_ = pf + 1 < trips;                                       \
@@ -139,14 +188,14 @@ __global__ __launch_bounds__(64 * NW) void flash_bwd_dq_stream_kernel(const BwdA
   constexpr int NM = 4 * DT;          // MFMAs per trip: (32-key block, 16-key group) x dt
   constexpr int kAhead = 4;
   int buf = 0, buf_pf = PF;         // ring slots of trip t and of trip t + PF
-  for (int t = 0; t < trips; t++) {
+  for (int t = trip0; t < trips; t++) {
     const char* kt = smem + buf * Tile::BUF_BYTES;
     // Trip t + PF into the buffer that trip t-1 was read from (every wavefront passed the barrier after it).
     AXL_ADVANCE()
     AXL_DMA_TRIP(buf_pf)
     buf = buf == Tile::NBUF - 1 ? 0 : buf + 1;
     buf_pf = buf_pf == Tile::NBUF - 1 ? 0 : buf_pf + 1;
-    if (t < my_trips) {
+    if (t < my_trips && has_ds(t)) {
     TrFrag dsf[4], kfr[NM];
 #pragma unroll
     for (int s = 0; s < 4; s++) {     // s = 2 * block + 16-key group
@@ -197,10 +246,10 @@ __global__ __launch_bounds__(64 * NW) void flash_bwd_dq_stream_kernel(const BwdA
     }
 }
 
-template <typename E, int D, int NW>
+template <typename E, int D, int NW, bool RANGED>
 static hipError_t launch_nw(const BwdArgs& a, hipStream_t stream) {
   using Tile = DqStream<D, NW>;
-  auto kernel = flash_bwd_dq_stream_kernel<E, D, NW>;
+  auto kernel = flash_bwd_dq_stream_kernel<E, D, NW, RANGED>;
   hipError_t err = allow_dynamic_lds((const void*)kernel, Tile::LDS_BYTES);
   if (err != hipSuccess) return err;
   const int grid = (a.T / Tile::BQ) * a.B * a.Hq;
@@ -211,8 +260,10 @@ static hipError_t launch_nw(const BwdArgs& a, hipStream_t stream) {
 template <typename E, int D>
 static hipError_t launch_one(const BwdArgs& a, hipStream_t stream) {
   // 8 wavefronts need two K loads per wavefront (head_dim 128) and 256-row blocks
-  if (D == 128 && a.T % 256 == 0) return launch_nw<E, D, D == 128 ? 8 : 4>(a, stream);
-  return launch_nw<E, D, 4>(a, stream);
+  constexpr int NW8 = D == 128 ? 8 : 4;
+  if (D == 128 && a.T % 256 == 0)
+    return a.kb_tbl ? launch_nw<E, D, NW8, true>(a, stream) : launch_nw<E, D, NW8, false>(a, stream);
+  return a.kb_tbl ? launch_nw<E, D, 4, true>(a, stream) : launch_nw<E, D, 4, false>(a, stream);
 }
 
 hipError_t launch_bwd_dq_stream(const BwdArgs& a, int dtype, int head_dim, hipStream_t stream) {

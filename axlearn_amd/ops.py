@@ -211,8 +211,9 @@ def flash_bwd(
     `phases` selects a subset of {1: delta, 2: dK/dV, 4: dQ} (timing / profiling only); `buffers`
     = (dq, dk, dv, workspace) reuses caller-provided outputs instead of allocating.  bias,
     dropout_mask and dropout_rate must be the ones the forward was given (the bias gets no gradient,
-    as in gpu_attention.py:786).  `ds_workspace=True` (AXL_BWD_DS_WORKSPACE; plain causal attention
-    only, ignored otherwise) keeps dS in a larger workspace instead of recomputing it for dq."""
+    as in gpu_attention.py:786).  `ds_workspace=True` (AXL_BWD_DS_WORKSPACE; causal or sliding-window
+    attention over equal lengths without offsets, bias or dropout; ignored otherwise) keeps dS in a
+    larger workspace instead of recomputing it for dq."""
     b, t, hq, d, s, hkv = _check_qkv(q, k, v)
     _check_segment_ids(segment_ids, b, t, s)
     _want_shape("out", out, q.shape)
@@ -272,9 +273,9 @@ def flash_bwd_buffers(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, mask
     """Pre-allocates (dq, dk, dv, workspace) for repeated `flash_bwd(..., buffers=...)` calls.
 
     The workspace holds delta and the scaled lse (fp32 [B,Hq,T] each); with `segment_ids` (the ones the
-    calls will pass) also the table of id ranges per 32 rows; with `ds_workspace=True` and
-    `mask_kind=MASK_CAUSAL` (equal lengths, no offsets / segment ids / bias / dropout) also dS, about
-    T*S bytes per (batch, head), for `flash_bwd(..., ds_workspace=True)`."""
+    calls will pass) also the table of id ranges per 32 rows; with `ds_workspace=True` and a causal or
+    sliding-window `mask_kind` (equal lengths, no offsets / bias / dropout) also dS, about T*S bytes per
+    (batch, head), for `flash_bwd(..., ds_workspace=True)`."""
     b, t, hq, d = q.shape
     p = AxlFlashBwdParams(batch=b, q_len=t, kv_len=k.shape[1], num_q_heads=hq, num_kv_heads=k.shape[2],
                           head_dim=d, dtype=_lib.dtype_code(q.dtype), mask_kind=mask_kind,

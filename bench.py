@@ -7,8 +7,8 @@ backward, bf16, batch 4, 32 query heads / 8 kv heads, seq 4096, head_dim 128: a 
 (axl_flash_fwd) plus one backward (axl_flash_bwd) over one synthetic batch already resident in HBM.
 The backward of the headline step keeps dS in a workspace the caller provides (AXL_BWD_DS_WORKSPACE);
 `c2_recompute` in the same line is the same step through the backward that recomputes dS instead
-(`--recompute` makes that one the headline).  `c5`, the other plain causal workload, is reported the
-same way (`c5` with the workspace, 69 GB at that length, and `c5_recompute`).
+(`--recompute` makes that one the headline).  `c3` and `c5` are reported the same way (with the
+workspace, 8.7 GB and 69 GB, and as `c3_recompute`, `c5_recompute`).
 The paged-decode half of the metric (configs[3], "C4") is measured in the same run and reported in
 the `paged_decode` object of the same JSON line.  With the default `--workload all` the line also
 carries `c1` (configs[0]: the fp32 case the reference itself runs on CPU), `c3` (sliding window +
@@ -52,15 +52,16 @@ HBM_PEAK_GBS = 8000.0           # MI355X HBM3E
 TRAFFIC = {
     "c2": dict(bytes=3.205e9, source="profiles/flash_c2_trace_counters.md (flash_bwd_dkdv_kernel, dS-workspace step)"),
     "c2_recompute": dict(bytes=0.983e9, source="profiles/flash_c2_trace_counters.md (flash_bwd_dkdv_kernel, --recompute)"),
-    "c3": dict(bytes=1.902e9, source="profiles/flash_c3_c5_trace_counters.md (flash_bwd_dkdv_kernel, segment ids)"),
+    "c3": dict(bytes=1.902e9, source="profiles/flash_c3_c5_trace_counters.md (flash_bwd_dkdv_kernel, segment ids, dS-workspace step)"),
+    "c3_recompute": dict(bytes=1.902e9, source="profiles/flash_c3_c5_trace_counters.md (flash_bwd_dkdv_kernel, segment ids, --recompute)"),
     "c5": dict(bytes=88.15e9, source="profiles/flash_c3_c5_trace_counters.md (flash_bwd_dkdv_kernel, dS-workspace step)"),
     "c5_recompute": dict(bytes=24.17e9, source="profiles/flash_c3_c5_trace_counters.md (flash_bwd_dkdv_kernel, --recompute)"),
     "c4": dict(bytes=4.254e9, source="profiles/paged_decode_c4_trace_counters.md (decode_split_kernel)"),
 }
 
-# Plain causal workloads: their default step runs the backward that keeps dS in a caller-provided
-# workspace (AXL_BWD_DS_WORKSPACE: 5 executed GEMMs instead of 7; 2.1 GB for C2, 69 GB for C5).
-DS_WORKSPACE_WORKLOADS = ("c2", "c5")
+# Workloads whose default step runs the backward that keeps dS in a caller-provided workspace
+# (AXL_BWD_DS_WORKSPACE: 5 executed GEMMs instead of 7; 2.1 GB for C2, 8.7 GB for C3, 69 GB for C5).
+DS_WORKSPACE_WORKLOADS = ("c2", "c3", "c5")
 
 METRIC = "flash-attn fwd+bwd TFLOP/s; paged-decode HBM GB/s (% roofline), 1 MI355X"
 
@@ -435,7 +436,10 @@ def main():
                 dict(cfg, ds_workspace=not cfg.get("ds_workspace")), args.steps, args.warmup, False)
             line["machine"] = calibrate_mfma()
             line["c1"] = bench_c1(args.steps, args.warmup, cpu_base)
-            line["c3"] = bench_flash(_flash_workload("c3"), max(5, args.steps // 2), 2, cpu_base)
+            c3 = dict(_flash_workload("c3"), ds_workspace=not args.recompute)
+            line["c3"] = bench_flash(c3, max(5, args.steps // 2), 2, cpu_base)
+            line["c3_recompute" if c3["ds_workspace"] else "c3_ds_workspace"] = bench_flash(
+                dict(c3, ds_workspace=not c3["ds_workspace"]), max(5, args.steps // 2), 2, False)
             c5 = dict(_flash_workload("c5"), ds_workspace=not args.recompute)
             line["c5"] = bench_flash(c5, max(3, args.steps // 4), 1, cpu_base)
             line["c5_recompute" if c5["ds_workspace"] else "c5_ds_workspace"] = bench_flash(

@@ -847,12 +847,49 @@ def test_ds_workspace_backward_matches_oracle(b, t, hq, hkv, d, dtype):
         assert torch.equal(got[2], base[2])
         if sk is not None:
             assert ref.max_abs(got[3].cpu(), want[3]) <= 2e-2 * max(1.0, float(want[3].abs().max()))
-    # the flag is ignored where the path does not apply (here: a sliding window)
-    kw = dict(softmax_scale=scale, mask_kind=ops.MASK_SLIDING_WINDOW, sliding_window=100)
+    # the flag is ignored where the path does not apply (here: no mask)
+    kw = dict(softmax_scale=scale, mask_kind=ops.MASK_NONE)
     out, lse = ops.flash_fwd(q.cuda(), k.cuda(), v.cuda(), **kw)
     a = ops.flash_bwd(q.cuda(), k.cuda(), v.cuda(), out, lse, do.cuda(), ds_workspace=True, **kw)
     c = ops.flash_bwd(q.cuda(), k.cuda(), v.cuda(), out, lse, do.cuda(), **kw)
     assert all(torch.equal(x, y) for x, y in zip(a, c))
+
+
+@pytest.mark.parametrize("b,t,hq,hkv,d,dtype,mask,window,seg", [
+    (1, 512, 4, 2, 128, torch.bfloat16, "causal", None, "packed"),
+    (2, 512, 4, 2, 128, torch.bfloat16, "sliding", 100, None),
+    (2, 1024, 8, 2, 128, torch.bfloat16, "sliding", 300, "packed"),
+    (1, 1024, 4, 1, 64, torch.bfloat16, "sliding", 200, "packed"),
+    (3, 640, 10, 5, 64, torch.float16, "sliding", 31, "packed"),
+    # ids that come back later in the row: the key blocks that hold dS for a query tile are then not one run
+    (2, 768, 6, 6, 128, torch.float16, "causal", None, "unsorted"),
+    # head_dim 128 with a length that is not a multiple of 256: the flag falls back to the recomputing path
+    (1, 384, 4, 4, 128, torch.bfloat16, "sliding", 64, "packed"),
+])
+def test_ds_workspace_backward_under_window_and_segments(b, t, hq, hkv, d, dtype, mask, window, seg):
+    """AXL_BWD_DS_WORKSPACE under a sliding window and / or segment ids: the dK/dV kernel records which
+    query tiles each key block stored dS for and the streaming dQ kernel reads only those.  Against the
+    oracle, and dv bit-identical to the recomputing path's."""
+    q, k, v, do = _inputs(b, t, hq, hkv, d, dtype)
+    segs = None
+    if seg is not None:
+        segs = ref.packed_segment_ids(4, b, t, max_docs=4)
+        if seg == "unsorted":
+            segs = (segs * 7) % 5 + 1
+    spec, kw = _mask_args(mask, window, segs)
+    scale = d ** -0.5
+    out, lse = ops.flash_fwd(q.cuda(), k.cuda(), v.cuda(), softmax_scale=scale, **kw)
+    bufs = ops.flash_bwd_buffers(q.cuda(), k.cuda(), v.cuda(), mask_kind=kw["mask_kind"], ds_workspace=True,
+                                 segment_ids=kw["segment_ids"])
+    bufs[3].fill_(0xff)   # blocks nobody stores must not be read: as NaN patterns they would show
+    got = ops.flash_bwd(q.cuda(), k.cuda(), v.cuda(), out, lse, do.cuda(), softmax_scale=scale, ds_workspace=True,
+                        buffers=bufs, **kw)
+    base = ops.flash_bwd(q.cuda(), k.cuda(), v.cuda(), out, lse, do.cuda(), softmax_scale=scale, **kw)
+    want = ref.reference_mha_grads(q, k, v, do, spec, softmax_scale=scale)
+    for name, x, w in zip(("dq", "dk", "dv"), got, want):
+        _assert_close(name, x, w, dtype)
+    assert torch.equal(got[2], base[2])
+    assert ref.rel_l2(got[0].cpu(), base[0].cpu().float()) < 1e-4
 
 
 def test_layer_compute_attention_end_to_end():
@@ -1004,9 +1041,11 @@ def _doc_boundary(seed, batch, seq_len, b):
     return int(change[0]) + 1 if len(change) else seq_len // 2
 
 
-def test_baseline_c3_full_size():
-    """C3 at full size (128 pairs).  Key blocks per sampled row: one that straddles a document
-    boundary, one whose last visible query rows sit at the window edge (key + 4096 < T), a late one."""
+@pytest.mark.parametrize("ds_workspace", [False, True])
+def test_baseline_c3_full_size(ds_workspace):
+    """C3 at full size (128 pairs), through both backward paths.  Key blocks per sampled row: one that
+    straddles a document boundary, one whose last visible query rows sit at the window edge
+    (key + 4096 < T), a late one."""
     B, T = 8, 8192
     for b, hk in ((0, 0), (5, 11)):
         cut = _doc_boundary(4, B, T, b)
@@ -1014,10 +1053,12 @@ def test_baseline_c3_full_size():
         straddle = max(0, min(T - 128, straddle))
         _sampled_fwd_bwd_check(B, T, 16, 16, 128, "sliding", 4096, True, samples=[(b, hk)],
                                dq_rows=[(0, 128), (4096, 4224), (8064, 8192)],
-                               key_blocks=[(straddle, straddle + 128), (1024, 1152), (7936, 8064)])
+                               key_blocks=[(straddle, straddle + 128), (1024, 1152), (7936, 8064)],
+                               ds_workspace=ds_workspace)
 
 
-def test_baseline_c5_full_size():
+@pytest.mark.parametrize("ds_workspace", [False, True])
+def test_baseline_c5_full_size(ds_workspace):
     _sampled_fwd_bwd_check(1, 32768, 64, 8, 128, "causal", None, False,
                            samples=[(0, 3)], dq_rows=[(0, 128), (16384, 16512), (32640, 32768)],
-                           key_blocks=[(32384, 32512), (32000, 32128)])
+                           key_blocks=[(32384, 32512), (32000, 32128)], ds_workspace=ds_workspace)

@@ -344,7 +344,17 @@ def test_abi_validation_without_gpu():
     # plain causal attention with the dS workspace: A = T / 128 = 2 -> 8 A (A + 1) blocks of 2 KB per head
     bp.flags = _lib.BWD_DS_WORKSPACE
     assert lib.axl_flash_bwd_workspace_bytes(ctypes.byref(bp)) == stats + 2 * 4 * 48 * 2048
-    bp.mask_kind = 2  # a sliding window has no dS workspace: the flag is ignored
+    # under a sliding window (or with segment ids): also which query tiles each 128-key block stored,
+    # [B, S / 128] pairs of int32, rounded to 256 bytes
+    bp.mask_kind = 2
+    assert lib.axl_flash_bwd_workspace_bytes(ctypes.byref(bp)) == stats + 256 + 2 * 4 * 48 * 2048
+    bp.segment_ids = 256
+    assert lib.axl_flash_bwd_workspace_bytes(ctypes.byref(bp)) == stats + 256 + 256 + 2 * 4 * 48 * 2048
+    bp.segment_ids = None
+    bp.q_len = bp.kv_len = 384  # ... which at head_dim 128 needs 256-row blocks: the flag is ignored
+    assert lib.axl_flash_bwd_workspace_bytes(ctypes.byref(bp)) == 2 * (2 * 4 * 384 * 4)
+    bp.q_len = bp.kv_len = 256
+    bp.mask_kind = 0  # no mask: no dS workspace
     assert lib.axl_flash_bwd_workspace_bytes(ctypes.byref(bp)) == stats
     bp.mask_kind = 1
     bp.flags = 0
@@ -512,4 +522,4 @@ def test_dkdv_kernel_keeps_its_vector_register_accumulators_in_place():
         assert agprs == int(m.group(1)), f"{name}: {agprs} AGPRs"
         assert scratch == 0, f"{name}: scratch {scratch}"
         seen += 1
-    assert seen == 12  # {bf16, f16} x {64, 128} x {plain, segment ids, dS workspace}
+    assert seen == 16  # {bf16, f16} x {64, 128} x {plain, segment ids} x {recomputing, dS workspace}
