@@ -50,11 +50,11 @@ HBM_PEAK_GBS = 8000.0           # MI355X HBM3E
 # kernel, `--calibrate-copy`).  Constants from the committed profile named next to each: the run
 # that prints them does not read the counters itself.
 TRAFFIC = {
-    "c2": dict(bytes=3.205e9, source="profiles/flash_c2_trace_counters.md (flash_bwd_dkdv_kernel, dS-workspace step)"),
-    "c2_recompute": dict(bytes=0.983e9, source="profiles/flash_c2_trace_counters.md (flash_bwd_dkdv_kernel, --recompute)"),
-    "c3": dict(bytes=1.902e9, source="profiles/flash_c3_c5_trace_counters.md (flash_bwd_dkdv_kernel, segment ids, dS-workspace step)"),
+    "c2": dict(bytes=3.204e9, source="profiles/flash_c2_trace_counters.md (flash_bwd_dkdv_kernel, dS-workspace step)"),
+    "c2_recompute": dict(bytes=0.982e9, source="profiles/flash_c2_trace_counters.md (flash_bwd_dkdv_kernel, --recompute)"),
+    "c3": dict(bytes=5.666e9, source="profiles/flash_c3_c5_trace_counters.md (flash_bwd_dkdv_kernel, segment ids, dS-workspace step)"),
     "c3_recompute": dict(bytes=1.902e9, source="profiles/flash_c3_c5_trace_counters.md (flash_bwd_dkdv_kernel, segment ids, --recompute)"),
-    "c5": dict(bytes=88.15e9, source="profiles/flash_c3_c5_trace_counters.md (flash_bwd_dkdv_kernel, dS-workspace step)"),
+    "c5": dict(bytes=91.89e9, source="profiles/flash_c3_c5_trace_counters.md (flash_bwd_dkdv_kernel, dS-workspace step)"),
     "c5_recompute": dict(bytes=24.17e9, source="profiles/flash_c3_c5_trace_counters.md (flash_bwd_dkdv_kernel, --recompute)"),
     "c4": dict(bytes=4.254e9, source="profiles/paged_decode_c4_trace_counters.md (decode_split_kernel)"),
 }
