@@ -892,6 +892,38 @@ def test_ds_workspace_backward_under_window_and_segments(b, t, hq, hkv, d, dtype
     assert ref.rel_l2(got[0].cpu(), base[0].cpu().float()) < 1e-4
 
 
+@pytest.mark.parametrize("seed", range(10))
+def test_ds_workspace_sweep_against_the_recomputing_path(seed):
+    """Seeded sweep at sizes the oracle would take long for: lengths up to 4096, batch x kv heads spread
+    over the XCDs or not, windows from a few keys to the whole row, 1..6 documents per row.  The two
+    backward paths share everything up to dS, so dv is bit-identical, dk differs only through delta's
+    summation order and dq through its own; the workspace starts out as NaN patterns."""
+    rng = np.random.default_rng(4000 + seed)
+    d = int(rng.choice([64, 128]))
+    dtype = [torch.bfloat16, torch.float16][int(rng.integers(0, 2))]
+    hkv = int(rng.choice([1, 2, 4, 8]))
+    hq = hkv * int(rng.choice([1, 2, 4]))
+    b = int(rng.choice([1, 2, 4]))
+    t = 256 * int(rng.integers(1, 17))
+    kind = str(rng.choice(["causal", "sliding"]))
+    window = int(rng.choice([7, 100, t // 3, t - 1, 2 * t])) if kind == "sliding" else None
+    packed = bool(rng.integers(0, 2))
+    q, k, v, do = (x.cuda() for x in _inputs(b, t, hq, hkv, d, dtype))
+    segs = ref.packed_segment_ids(seed, b, t).cuda() if packed else None
+    mk = ops.MASK_CAUSAL if kind == "causal" else ops.MASK_SLIDING_WINDOW
+    kw = dict(mask_kind=mk, sliding_window=window or 0, softmax_scale=d ** -0.5, segment_ids=segs)
+    case = f"b={b} t={t} hq={hq} hkv={hkv} d={d} {dtype} {kind} window={window} packed={packed}"
+    out, lse = ops.flash_fwd(q, k, v, **kw)
+    bufs = ops.flash_bwd_buffers(q, k, v, mask_kind=mk, ds_workspace=True, segment_ids=segs)
+    bufs[3].fill_(0xff)
+    dq, dk, dv = ops.flash_bwd(q, k, v, out, lse, do, ds_workspace=True, buffers=bufs, **kw)
+    bq, bk, bv = ops.flash_bwd(q, k, v, out, lse, do, **kw)
+    assert torch.equal(dv, bv), case
+    for name, x, y in (("dq", dq, bq), ("dk", dk, bk)):
+        assert torch.isfinite(x.float()).all(), f"{name} {case}"
+        assert ref.rel_l2(x.cpu(), y.cpu().float()) < 1e-4, f"{name} {case}: {ref.rel_l2(x.cpu(), y.cpu().float()):.3e}"
+
+
 def test_layer_compute_attention_end_to_end():
     """The layer-level calling sequence (layer.py:218-376) over the HIP kernels: bias cast to the query
     dtype, softmax_scale 1.0 by default with the scale folded into q beforehand, `(context, probs)` with
