@@ -482,21 +482,25 @@ def test_dispatch_and_autograd_end_to_end(dtype):
     assert ref.max_abs(o3.detach().cpu().float(), out.detach().cpu().float()) < 1e-2
 
 
-def test_forward_and_backward_replay_from_a_captured_graph():
+@pytest.mark.parametrize("mask,window,ds_workspace", [("causal", None, False), ("causal", None, True),
+                                                      ("sliding", 200, True)])
+def test_forward_and_backward_replay_from_a_captured_graph(mask, window, ds_workspace):
     """Forward + backward enqueue kernels only, so they can be captured into a graph; every replay,
-    with eager work between the replays, equals the eager result bit for bit."""
+    with eager work between the replays, equals the eager result bit for bit.  Both backward paths
+    (the dS-workspace one with its table of stored tiles as well)."""
     b, t, hq, hkv, d = 2, 512, 4, 2, 128
     q, k, v, do = (x.cuda() for x in _inputs(b, t, hq, hkv, d, torch.bfloat16))
     segs = ref.packed_segment_ids(4, b, t, max_docs=3).cuda()
-    kw = dict(softmax_scale=d ** -0.5, mask_kind=ops.MASK_CAUSAL, segment_ids=segs)
+    mk = ops.MASK_CAUSAL if mask == "causal" else ops.MASK_SLIDING_WINDOW
+    kw = dict(softmax_scale=d ** -0.5, mask_kind=mk, sliding_window=window or 0, segment_ids=segs)
     out_e, lse_e = ops.flash_fwd(q, k, v, **kw)
-    grads_e = ops.flash_bwd(q, k, v, out_e, lse_e, do, **kw)
+    grads_e = ops.flash_bwd(q, k, v, out_e, lse_e, do, ds_workspace=ds_workspace, **kw)
     bufs = (torch.empty_like(q), torch.empty_like(k), torch.empty_like(v),
-            ops.flash_bwd_buffers(q, k, v, mask_kind=kw["mask_kind"], segment_ids=kw.get("segment_ids"))[3])
+            ops.flash_bwd_buffers(q, k, v, mask_kind=mk, segment_ids=segs, ds_workspace=ds_workspace)[3])
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
         out_g, lse_g = ops.flash_fwd(q, k, v, **kw)
-        ops.flash_bwd(q, k, v, out_g, lse_g, do, buffers=bufs, **kw)
+        ops.flash_bwd(q, k, v, out_g, lse_g, do, buffers=bufs, ds_workspace=ds_workspace, **kw)
     for rep in range(3):
         for x in (out_g, lse_g, *bufs):
             x.zero_()
@@ -506,7 +510,7 @@ def test_forward_and_backward_replay_from_a_captured_graph():
         assert all(torch.equal(g, e) for g, e in zip(bufs[:3], grads_e)), rep
         q.copy_(q.roll(1, dims=1))  # new inputs in the captured buffers
         out_e, lse_e = ops.flash_fwd(q, k, v, **kw)
-        grads_e = ops.flash_bwd(q, k, v, out_e, lse_e, do, **kw)
+        grads_e = ops.flash_bwd(q, k, v, out_e, lse_e, do, ds_workspace=ds_workspace, **kw)
 
 
 # ----------------------------------------------------------------------------- logit sink, head dims
