@@ -506,31 +506,24 @@ constexpr int kAuxBias16 = 1, kAuxBias32 = 2, kAuxDrop = 4;
 AuxArgs make_aux_args(const AxlAttnAux& x, float softmax_scale);
 int check_aux(const char* who, const AxlAttnAux& x, int batch, int hq, int q_len, int kv_len);
 
-// N consecutive bias elements (N = 4 or 8) starting at byte offset `off` of the ELEMENT index, i.e.
-// p points at the row, `col` is the first key; returns them as fp32.
+// 4 consecutive bias elements of a row, starting at key `col`, as fp32 (the fp32 kernels' bias read;
+// the 16-bit kernels fetch raw words a tile ahead and convert at the use).
 template <int N>
 __device__ __forceinline__ void load_bias(const char* row, int col, int is_f32, float (&out)[N]) {
+  static_assert(N == 4, "four elements per call");
   if (is_f32) {
+    const floatx4 v = *(const floatx4*)(row + (int64_t)col * 4);
 #pragma unroll
-    for (int i = 0; i < N / 4; i++) {
-      const floatx4 v = *(const floatx4*)(row + (int64_t)col * 4 + 16 * i);
-#pragma unroll
-      for (int j = 0; j < 4; j++) out[4 * i + j] = v[j];
-    }
+    for (int j = 0; j < 4; j++) out[j] = v[j];
   } else {
     union {
-      uint32_t u[N / 2];
-      __bf16 e[N];
+      uint32_t u[2];
+      __bf16 e[4];
     } w;
-    if constexpr (N == 8) {
-      const u32x4 v = *(const u32x4*)(row + (int64_t)col * 2);
-      w.u[0] = v[0]; w.u[1] = v[1]; w.u[2] = v[2]; w.u[3] = v[3];
-    } else {
-      const uint2 v = *(const uint2*)(row + (int64_t)col * 2);
-      w.u[0] = v.x; w.u[1] = v.y;
-    }
+    const uint2 v = *(const uint2*)(row + (int64_t)col * 2);
+    w.u[0] = v.x; w.u[1] = v.y;
 #pragma unroll
-    for (int i = 0; i < N; i++) out[i] = (float)w.e[i];
+    for (int i = 0; i < 4; i++) out[i] = (float)w.e[i];
   }
 }
 
