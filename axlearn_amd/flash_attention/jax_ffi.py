@@ -81,6 +81,14 @@ def _mask_of(bias: BaseAttentionBias):
     return kind, window, seg, (explicit.value() if explicit.has_value() else None)
 
 
+# True: the backward keeps dS in its workspace where the library has that path (AXL_BWD_DS_WORKSPACE in
+# include/axl_attn.h: about T*S bytes per (batch, head) of scratch that XLA allocates for the call, for a
+# backward of 5 GEMMs instead of 7).  The size query below sees the same flag, so the scratch result of the
+# custom call grows with it.
+BWD_DS_WORKSPACE = False
+_AXL_BWD_DS_WORKSPACE = 1
+
+
 def _bwd_workspace_bytes(b, t, s, hq, hkv, d, dtype_code, mask_kind, has_seg, flags) -> int:
     """axl_flash_bwd_workspace_bytes for these shapes (a host-side size query of the core library)."""
     from axlearn_amd._lib import AxlFlashBwdParams  # the ctypes mirror of include/axl_attn.h
@@ -139,7 +147,7 @@ def _flash_bwd(softmax_scale, mask_kind, sliding_window, dropout_rate, logit_sin
     query, key, value, bias, segment_ids, dropout_mask, out, lse = res
     b, t, hq, d = query.shape
     s, hkv = key.shape[1], key.shape[2]
-    flags = 0
+    flags = _AXL_BWD_DS_WORKSPACE if BWD_DS_WORKSPACE else 0
     ws_bytes = _bwd_workspace_bytes(b, t, s, hq, hkv, d, _DTYPE_CODE[jnp.dtype(query.dtype)], mask_kind,
                                     segment_ids is not None, flags)
     dq, dk, dv, _, _ = jax.ffi.ffi_call(
