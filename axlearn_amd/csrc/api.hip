@@ -223,12 +223,12 @@ int axl_flash_bwd_phases(const AxlFlashBwdParams* p, int phases, void* stream) {
     return set_error(AXL_ERR_UNSUPPORTED, "axl_flash_bwd: segment_ids must be 16-byte aligned");
   rc = check_aux("axl_flash_bwd", p->aux, p->batch, p->num_q_heads, p->q_len, p->kv_len);
   if (rc != AXL_OK) return rc;
+  const size_t need = flash_bwd_workspace_bytes(*p);
+  if (!p->workspace || p->workspace_bytes < need || !aligned16(p->workspace))
+    return set_error(AXL_ERR_WORKSPACE, "axl_flash_bwd: workspace needs %zu bytes, 16-byte aligned (got %zu)",
+                     need, p->workspace ? p->workspace_bytes : (size_t)0);
   if (p->d_logit_sink && !p->logit_sink)
     return set_error(AXL_ERR_INVALID_ARGUMENT, "axl_flash_bwd: d_logit_sink without logit_sink");
-  const size_t need = flash_bwd_workspace_bytes(*p);
-  if (!p->workspace || p->workspace_bytes < need || (reinterpret_cast<uintptr_t>(p->workspace) & 255))
-    return set_error(AXL_ERR_WORKSPACE, "axl_flash_bwd: workspace needs %zu bytes, 256-byte aligned (got %zu)",
-                     need, p->workspace ? p->workspace_bytes : (size_t)0);
   return launch_flash_bwd(*p, phases, (hipStream_t)stream);
 }
 

@@ -422,21 +422,27 @@ static size_t kb_table_bytes(const AxlFlashBwdParams& p) {
   return ((size_t)p.batch * (p.kv_len / 128) * sizeof(int2) + 255) & ~(size_t)255;
 }
 
+// The parts of the workspace start on 256-byte boundaries; the caller's pointer only has to be
+// 16-byte aligned (allocators that slice one arena, XLA's buffer assignment among them, promise less
+// than 256), so the size includes the slack for rounding it up.
+constexpr size_t kWsAlign = 256;
 size_t flash_bwd_workspace_bytes(const AxlFlashBwdParams& p) {
-  return stats_bytes(p) + seg_table_bytes(p) + kb_table_bytes(p) + (spill_eligible(p) ? spill_bytes(p) : 0);
+  return stats_bytes(p) + seg_table_bytes(p) + kb_table_bytes(p) + (spill_eligible(p) ? spill_bytes(p) : 0) +
+         (kWsAlign - 16);
 }
 
 int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream) {
   const int dt = p.dtype;
   BwdArgs a;
   a.q = p.q; a.k = p.k; a.v = p.v; a.out = p.out; a.dout = p.d_out; a.lse = p.lse;
-  a.ndelta = (float*)p.workspace;
+  char* const ws = (char*)((reinterpret_cast<uintptr_t>(p.workspace) + (kWsAlign - 1)) & ~(uintptr_t)(kWsAlign - 1));
+  a.ndelta = (float*)ws;
   a.lse2 = a.ndelta + (size_t)p.batch * p.num_q_heads * p.q_len;
   a.dq = p.dq; a.dk = p.dk; a.dv = p.dv; a.seg = p.segment_ids;
   const bool spill = spill_eligible(p);  // the entry point has checked that the workspace holds dS as well
-  a.seg_tbl = p.segment_ids ? (const int2*)((char*)p.workspace + stats_bytes(p)) : nullptr;
-  a.kb_tbl = kb_table_bytes(p) ? (int2*)((char*)p.workspace + stats_bytes(p) + seg_table_bytes(p)) : nullptr;
-  a.ds = spill ? (char*)p.workspace + stats_bytes(p) + seg_table_bytes(p) + kb_table_bytes(p) : nullptr;
+  a.seg_tbl = p.segment_ids ? (const int2*)(ws + stats_bytes(p)) : nullptr;
+  a.kb_tbl = kb_table_bytes(p) ? (int2*)(ws + stats_bytes(p) + seg_table_bytes(p)) : nullptr;
+  a.ds = spill ? ws + stats_bytes(p) + seg_table_bytes(p) + kb_table_bytes(p) : nullptr;
   a.qs = to_s3(p.q_strides); a.ks = to_s3(p.k_strides); a.vs = to_s3(p.v_strides);
   a.os = to_s3(p.out_strides); a.dos = to_s3(p.d_out_strides); a.dqs = to_s3(p.dq_strides);
   a.dks = to_s3(p.dk_strides); a.dvs = to_s3(p.dv_strides);

@@ -39,9 +39,9 @@ namespace axl {
 
 struct DecArgs {
   const __bf16* q;        // [B, Hq, D]
-  const __bf16* k;        // paged: [Hkv, P, 16, D]; contiguous: [B, S, Hkv, D] (strided)
+  const __bf16* k;        // paged: [Hkv, P, page_size, D]; contiguous: [B, S, Hkv, D] (strided)
   const __bf16* v;
-  const int32_t* page_tables;  // [B, pps] (paged only)
+  const int32_t* page_tables;  // [B, pt_stride] (paged only)
   const int32_t* lengths;      // [B]
   __bf16* out;                 // [B, Hq, D]
   float* ws_o;                 // [records, GP, D]; at most B * Hkv * NCH records
@@ -51,8 +51,16 @@ struct DecArgs {
                                // chunk's entry is written by the workgroup that streams the chunk
   Strides3 ks, vs;             // contiguous only
   int B, Hq, Hkv, G;
-  int num_pages, pps;          // pool pages; logical pages per sequence (ceil(S/16) if contiguous)
-  int kv_len;                  // contiguous only
+  int ngrp, Hv;                // groups of 16 query heads per kv head; Hv = Hkv * ngrp "virtual" kv heads:
+                               // a kv head with more than 16 query heads is streamed once per group
+  int num_pages, pps;          // pool pages; 16-token tiles per sequence (ceil(S/16) if contiguous)
+  int page_shift, pt_stride;   // a pool page holds 16 << page_shift tokens; entries per page-table row
+  int d_real;                  // head_dim of the tensors (a multiple of 8, <= the compiled width D)
+  int kv_len;                  // key positions a sequence can address (cache rows / table capacity)
+  const char* bias;            // [B|1, Hq|1, kv_len] additive logit bias, bf16 or fp32, or nullptr
+  int64_t bias_sb, bias_sh;    // BYTES per batch / query head (0 broadcasts)
+  int bias_f32;
+  float inv_scale;             // 1 / scale: the bias joins the raw (unscaled) logits
   int chunk_pages, nch;
   int window;
   float scale;
@@ -61,7 +69,18 @@ struct DecArgs {
   int deterministic;           // fixed work decomposition: results reproducible bit for bit
 };
 
+// Tokens per tile: the unit the kernels stream and compute on.  A pool page of 16 << page_shift
+// tokens is that many consecutive tiles (the reference gathers gpu_block_size / page_size pages per
+// compute block, gpu_paged_attention.py:91-94; here the compute block is a tile and a page spans
+// several).
 constexpr int kPage = 16;
+
+// One element of the bias row of (sequence b, query head h) at key position t, in raw-logit units.
+__device__ __forceinline__ float decode_bias_at(const DecArgs& a, int b, int h, int t) {
+  const char* row = a.bias + b * a.bias_sb + h * a.bias_sh;
+  const float x = a.bias_f32 ? ((const float*)row)[t] : (float)((const __bf16*)row)[t];
+  return x * a.inv_scale;
+}
 
 // XOR swizzle of the 16-byte chunks of a K row inside an LDS tile, so that 16 lanes reading the
 // same logical chunk of 16 different rows hit 16 different bank groups.
@@ -118,7 +137,7 @@ struct DecTile {
 // in the "transposed" form where lane l owns query head l%16 and the tokens 4*(l/16)..+3 of the
 // page: the accumulator layout of S^T is exactly the B-operand layout of the second product, so
 // probabilities never leave registers, and every softmax statistic is per lane.
-template <typename E, int D, int GP, bool PAGED, int NST>
+template <typename E, int D, int GP, bool PAGED, int NST, bool BIAS>
 __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
   using Tile = DecTile<D, GP, NST>;
   constexpr int KSTEPS = D / 32;        // MFMA k-steps over head_dim for S^T
@@ -181,7 +200,7 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
   // single blocks at the end (guided self-scheduling) - so that workgroups on CUs that get more
   // of the memory system take more of the work.  The part of a run inside one (sequence, kv head)
   // is a segment: one contiguous page range, streamed without a break, one partial record.
-  const int n_blocks = pfx[a.B] * a.Hkv;
+  const int n_blocks = pfx[a.B] * a.Hv;
   const int n_wg = gridDim.x;
   // The ids of at most 256 pages are kept in registers.  A fixed decomposition (one block per
   // record, pages dealt round-robin) makes the result independent of timing.
@@ -199,15 +218,20 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
   int next_e = 0, next_n = 0;
   while (run_e < run_end) {
   int b = 0;
-  for (int hi = a.B; hi - b > 1;) {  // last b with Hkv * pfx[b] <= run_e
+  for (int hi = a.B; hi - b > 1;) {  // last b with Hv * pfx[b] <= run_e
     const int mid = (b + hi) >> 1;
-    if (pfx[mid] * a.Hkv <= run_e) b = mid; else hi = mid;
+    if (pfx[mid] * a.Hv <= run_e) b = mid; else hi = mid;
   }
   const int len = lens[b];
   int ch0, ch1;
   live_chunks(a, len, ch0, ch1);
-  const int rem = run_e - pfx[b] * a.Hkv;
-  const int hk = rem / (ch1 - ch0), cl = rem % (ch1 - ch0);
+  const int rem = run_e - pfx[b] * a.Hv;
+  const int hv = rem / (ch1 - ch0), cl = rem % (ch1 - ch0);
+  // Virtual head -> kv head and group of (at most) 16 of its query heads.
+  const int hk = a.ngrp == 1 ? hv : hv / a.ngrp;
+  const int grp = hv - hk * a.ngrp;
+  const int gcount = min(16, a.G - 16 * grp);
+  const int hbase = hk * a.G + 16 * grp;
   const int seg = min(run_end - run_e, ch1 - ch0 - cl);
   int first_page = 0;
   if (a.window >= 0) first_page = max(0, (len - 1 - a.window)) / kPage;
@@ -233,19 +257,20 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
   bf16x8 qf[KSTEPS];
 #pragma unroll
   for (int s = 0; s < KSTEPS; s++) {
-    if (head < a.G) {
-      qf[s] = *(const bf16x8*)(a.q + ((int64_t)b * a.Hq + hk * a.G + head) * D + 32 * s + 8 * kg);
+    if (head < gcount && 32 * s + 8 * kg < a.d_real) {
+      qf[s] = *(const bf16x8*)(a.q + ((int64_t)b * a.Hq + hbase + head) * a.d_real + 32 * s + 8 * kg);
     } else {
 #pragma unroll
       for (int e = 0; e < 8; e++) qf[s][e] = (__bf16)0.f;
     }
   }
-  // Page ids of the segment (at most 256): register r, lane l holds page 64r + l.
+  // Pool page of each tile of the segment (at most 256 tiles): register r, lane l holds tile 64r + l.
   int seg_pages[4] = {0, 0, 0, 0};
   if (PAGED) {
 #pragma unroll
     for (int r = 0; r < 4; r++)
-      if (64 * r + lane < n_pg) seg_pages[r] = a.page_tables[(int64_t)b * a.pps + c_begin + 64 * r + lane];
+      if (64 * r + lane < n_pg)
+        seg_pages[r] = a.page_tables[(int64_t)b * a.pt_stride + ((c_begin + 64 * r + lane) >> a.page_shift)];
   }
   auto page_id = [&](int idx) -> int {
     int pg = __builtin_amdgcn_readlane(seg_pages[0], idx & 63);
@@ -269,14 +294,19 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
   // Both tiles are stored with their 16-byte chunks XOR-swizzled by a function of the row, which
   // makes the K reads (16 lanes = 16 rows, same chunk) and the transposing V reads (rows 0..7 of
   // the same 32-byte column window) hit distinct banks.
-  const int64_t k_row_stride = PAGED ? D : a.ks.s;
-  const int64_t v_row_stride = PAGED ? D : a.vs.s;
+  const int64_t k_row_stride = PAGED ? a.d_real : a.ks.s;
+  const int64_t v_row_stride = PAGED ? a.d_real : a.vs.s;
+  // A head_dim below the compiled width: the slices past it are fetched from slice 0 of the same row
+  // instead.  Those LDS columns then hold finite copies of real data; the Q columns they meet are
+  // zero, and the output rows they produce are never written.
+  const int real_slices = a.d_real >> 3;
   int k_src[NLOAD], v_src[NLOAD];
 #pragma unroll
   for (int i = 0; i < NLOAD; i++) {
     const int row = TPL * i + vtok;
-    k_src[i] = (vslice ^ k_swizzle<D>(row)) * 8;     // + row * stride, added per page
-    v_src[i] = (vslice ^ v_swizzle<D>(row)) * 8;
+    const int ksl = vslice ^ k_swizzle<D>(row), vsl = vslice ^ v_swizzle<D>(row);
+    k_src[i] = (ksl < real_slices ? ksl : 0) * 8;     // + row * stride, added per page
+    v_src[i] = (vsl < real_slices ? vsl : 0) * 8;
   }
   int k_rd[KSTEPS];
 #pragma unroll
@@ -300,7 +330,9 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
     if (PAGED) {
       int pg = page_id(idx);
       if ((unsigned)pg >= (unsigned)a.num_pages) pg = 0;  // reads as zeros: see `valid` below
-      const int64_t off = ((int64_t)hk * a.num_pages + pg) * (kPage * D);
+      // tile (j mod tiles-per-page) of pool page pg of kv head hk
+      const int64_t tile = ((((int64_t)hk * a.num_pages + pg) << a.page_shift) + (j & ((1 << a.page_shift) - 1)));
+      const int64_t off = tile * (kPage * a.d_real);
       kb = a.k + off;
       vb = a.v + off;
     } else {
@@ -378,6 +410,15 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
     floatx4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ks++) s = E::mfma_16x16x32(kf[ks], qf[ks], s);
+    if constexpr (BIAS) {
+      // logits = scale * q.k + bias (gpu_decoding.py:117-121, gpu_paged_attention.py:103-106): in raw
+      // units, bias / scale.  Positions past the row's end are masked below; their reads are clamped.
+      if (head < gcount) {
+#pragma unroll
+        for (int r = 0; r < 4; r++)
+          s[r] += decode_bias_at(a, b, hbase + head, min(j * kPage + 4 * kg + r, a.kv_len - 1));
+      }
+    }
     // A page that straddles the length (or the window start) holds tokens whose probability is
     // exactly 0; their V rows may be uninitialised pool memory, and 0 * NaN would poison the sum,
     // so those rows are replaced by zeros, as are all rows of a page outside the pool.
@@ -458,7 +499,7 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
     a.ws_l[slot * GP + tid] = lw;
   }
   // Table entries of the segment's chunks: the record at its first chunk, "none" at the others.
-  for (int i = tid; i < seg; i += 256) a.ws_tab[((int64_t)b * a.Hkv + hk) * a.nch + cl + i] = i == 0 ? (int)slot : -1;
+  for (int i = tid; i < seg; i += 256) a.ws_tab[((int64_t)b * a.Hv + hv) * a.nch + cl + i] = i == 0 ? (int)slot : -1;
   if (tid == 0) *s_page = 4 * NST;
   __syncthreads();  // the ring (and red_m/red_l) are reused by the next segment
   run_e += seg;
@@ -492,17 +533,20 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecArgs a) {
   __shared__ int s_count;
   __shared__ float s_max[GP], s_inv[GP];
   __shared__ float4 s_part[256];          // partial sums of the record slices
-  const int hk = blockIdx.x, b = blockIdx.y;
+  const int hv = blockIdx.x, b = blockIdx.y;
+  const int hk = hv / a.ngrp, grp = hv - hk * a.ngrp;
+  const int gcount = min(16, a.G - 16 * grp);   // query heads of this group
+  const int hbase = hk * a.G + 16 * grp;
   const int tid = threadIdx.x;
   const int len = clamp_length(a, a.lengths[b]);
   int ch0, ch1;
   live_chunks(a, len, ch0, ch1);
   const int nc = ch1 - ch0;               // live chunks = upper bound on records of this (b, hk)
   // The split kernel has finished: leave the work counter at zero for the next call on this workspace.
-  if (hk == 0 && b == 0 && tid == 0) a.ticket[0] = 0;
+  if (hv == 0 && b == 0 && tid == 0) a.ticket[0] = 0;
   const float c = a.scale * kLog2e;
   // The whole table row in one round trip, then compacted in chunk order by one wavefront.
-  s_raw[tid] = tid < nc ? a.ws_tab[((int64_t)b * a.Hkv + hk) * a.nch + tid] : -1;
+  s_raw[tid] = tid < nc ? a.ws_tab[((int64_t)b * a.Hv + hv) * a.nch + tid] : -1;
   __syncthreads();
   if (tid < 64) {
     int count = 0;
@@ -542,7 +586,7 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecArgs a) {
   // Output: G*D floats = n4 groups of four.  With fewer groups than threads the records are dealt
   // to `ways` slices of threads (record ci to slice ci % ways), 16 loads in flight per thread,
   // and the slices' partial sums are added in slice order.
-  const int n4 = a.G * D / 4;
+  const int n4 = gcount * D / 4;
   const int per = min(n4, 256);
   const int ways = 256 / per;
   for (int base = 0; base < n4; base += per) {
@@ -567,14 +611,17 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecArgs a) {
         acc.x += p.x; acc.y += p.y; acc.z += p.z; acc.w += p.w;
       }
       const float inv = s_inv[gq];
-      const int64_t at = ((int64_t)b * a.Hq + hk * a.G) * D + 4 * col;
-      if constexpr (std::is_same_v<E, ElemF32>) {
-        *(float4*)((float*)a.out + at) = float4{acc.x * inv, acc.y * inv, acc.z * inv, acc.w * inv};
-      } else {
-        union { bf16x2 p[2]; uint2 u; } pk;
-        pk.p[0] = E::pack(acc.x * inv, acc.y * inv);
-        pk.p[1] = E::pack(acc.z * inv, acc.w * inv);
-        *(uint2*)(a.out + at) = pk.u;
+      const int dcol = 4 * col - gq * D;   // column inside the head: the ones past head_dim are padding
+      const int64_t at = ((int64_t)b * a.Hq + hbase + gq) * a.d_real + dcol;
+      if (dcol < a.d_real) {
+        if constexpr (std::is_same_v<E, ElemF32>) {
+          *(float4*)((float*)a.out + at) = float4{acc.x * inv, acc.y * inv, acc.z * inv, acc.w * inv};
+        } else {
+          union { bf16x2 p[2]; uint2 u; } pk;
+          pk.p[0] = E::pack(acc.x * inv, acc.y * inv);
+          pk.p[1] = E::pack(acc.z * inv, acc.w * inv);
+          *(uint2*)(a.out + at) = pk.u;
+        }
       }
     }
   }

@@ -106,7 +106,8 @@ def mask_fn_as_bias(mask_fn: MaskFn, q_len: int, kv_len: int, device, q_pos_offs
 
 
 def _attend(query, key, value, segment_ids, softmax_scale, mask_kind, window, logit_sink=None,
-            bias=None, dropout_mask=None, dropout_rate=0.0, save_residuals=True, bwd_ds_workspace=False):
+            bias=None, dropout_mask=None, dropout_rate=0.0, save_residuals=True, bwd_ds_workspace=None,
+            bwd_workspace_limit_bytes=None):
     """Pads the head dim if needed and runs the differentiable kernel pair."""
     head_dim = query.shape[-1]
     width = padded_head_dim(head_dim)
@@ -115,7 +116,7 @@ def _attend(query, key, value, segment_ids, softmax_scale, mask_kind, window, lo
     out = _FlashAttentionFn.apply(
         _pad_last(query, width), _pad_last(key, width), _pad_last(value, width), segment_ids,
         softmax_scale, mask_kind, window, logit_sink, bias, dropout_mask, dropout_rate, save_residuals,
-        bwd_ds_workspace,
+        bwd_ds_workspace, bwd_workspace_limit_bytes,
     )
     return out if width == head_dim else out[..., :head_dim]
 
@@ -128,11 +129,14 @@ class _FlashAttentionFn(torch.autograd.Function):
     backward re-runs the forward kernel on the saved q, k, v first, trading one forward pass for
     [B,T,Hq,D] + [B,Hq,T] of memory, and produces bit-identical gradients.  bwd_ds_workspace=True
     asks the backward to keep dS in its workspace (AXL_BWD_DS_WORKSPACE: about T*S bytes per (batch,
-    head) more, 5 GEMMs instead of 7; ignored where that path does not apply)."""
+    head) more, 5 GEMMs instead of 7; ignored where that path does not apply), False to recompute dS
+    in the dQ kernel, None to take the dS workspace whenever it fits bwd_workspace_limit_bytes (None:
+    a sixteenth of the device's memory)."""
 
     @staticmethod
     def forward(ctx, query, key, value, segment_ids, softmax_scale, mask_kind, window, logit_sink,
-                bias, dropout_mask, dropout_rate, save_residuals, bwd_ds_workspace=False):
+                bias, dropout_mask, dropout_rate, save_residuals, bwd_ds_workspace=None,
+                bwd_workspace_limit_bytes=None):
         aux = dict(bias=bias, dropout_mask=dropout_mask, dropout_rate=dropout_rate)
         out, lse = ops.flash_fwd(
             query, key, value, softmax_scale=softmax_scale, mask_kind=mask_kind,
@@ -145,7 +149,8 @@ class _FlashAttentionFn(torch.autograd.Function):
         ctx.segment_ids = segment_ids
         ctx.aux = aux  # not differentiated: the bias gets no gradient (gpu_attention.py:786)
         ctx.args = (softmax_scale, mask_kind, window)
-        ctx.bwd_ds_workspace = bool(bwd_ds_workspace)
+        ctx.bwd_ds_workspace = None if bwd_ds_workspace is None else bool(bwd_ds_workspace)
+        ctx.bwd_workspace_limit_bytes = bwd_workspace_limit_bytes
         return out
 
     @staticmethod
@@ -162,10 +167,10 @@ class _FlashAttentionFn(torch.autograd.Function):
         grads = ops.flash_bwd(
             query, key, value, out, lse, d_out, softmax_scale=softmax_scale, mask_kind=mask_kind,
             sliding_window=window, segment_ids=ctx.segment_ids, logit_sink=logit_sink,
-            ds_workspace=ctx.bwd_ds_workspace, **ctx.aux,
+            ds_workspace=ctx.bwd_ds_workspace, ds_workspace_limit=ctx.bwd_workspace_limit_bytes, **ctx.aux,
         )
         d_sink = grads[3].to(logit_sink.dtype) if logit_sink is not None else None
-        return grads[0], grads[1], grads[2], None, None, None, None, d_sink, None, None, None, None, None
+        return grads[0], grads[1], grads[2], None, None, None, None, d_sink, None, None, None, None, None, None
 
 
 # pylint: disable-next=too-many-positional-arguments
@@ -228,10 +233,15 @@ class HipFlashAttention(BaseFlashAttention):
         # False: do not keep (out, lse) for the backward, recompute them there instead; the
         # counterpart of leaving `flash_residuals` out of the remat policy's saved names.
         save_residuals: bool = True
-        # True: the backward keeps dS in its workspace (AXL_BWD_DS_WORKSPACE) where that path
-        # applies: about T*S bytes per (batch, head) of transient memory for a backward that runs 5
-        # GEMMs instead of 7.  Also settable through backend_overrides["bwd_ds_workspace"].
-        bwd_ds_workspace: bool = False
+        # The backward can keep dS in its workspace (AXL_BWD_DS_WORKSPACE) where that path applies:
+        # about T*S bytes per (batch, head) of transient memory for a backward that runs 5 GEMMs
+        # instead of 7.  None (default): do so whenever that workspace fits bwd_workspace_limit_bytes;
+        # True / False force the choice.  Also settable through backend_overrides["bwd_ds_workspace"].
+        bwd_ds_workspace: Optional[bool] = None
+        # Largest backward workspace the automatic choice may take; None = a sixteenth of the device's
+        # memory (18 GB on an MI355X: C2 and C3 of the benchmark take the dS workspace, the 69 GB of a
+        # 32768-token sequence do not).  Also settable through backend_overrides.
+        bwd_workspace_limit_bytes: Optional[int] = None
 
     _kv_cache_type = None
 
@@ -335,5 +345,7 @@ class HipFlashAttention(BaseFlashAttention):
             query, key, value, seg, float(self.cfg.softmax_scale), kind[0], kind[1],
             input_batch.get("logit_sink", None), bias=dense, dropout_mask=dropout_mask, dropout_rate=rate,
             save_residuals=bool(self.get_backend_overrides("save_residuals", self.cfg.save_residuals)),
-            bwd_ds_workspace=bool(self.get_backend_overrides("bwd_ds_workspace", self.cfg.bwd_ds_workspace)),
+            bwd_ds_workspace=self.get_backend_overrides("bwd_ds_workspace", self.cfg.bwd_ds_workspace),
+            bwd_workspace_limit_bytes=self.get_backend_overrides(
+                "bwd_workspace_limit_bytes", self.cfg.bwd_workspace_limit_bytes),
         )

@@ -81,11 +81,14 @@ def _mask_of(bias: BaseAttentionBias):
     return kind, window, seg, (explicit.value() if explicit.has_value() else None)
 
 
-# True: the backward keeps dS in its workspace where the library has that path (AXL_BWD_DS_WORKSPACE in
+# The backward can keep dS in its workspace where the library has that path (AXL_BWD_DS_WORKSPACE in
 # include/axl_attn.h: about T*S bytes per (batch, head) of scratch that XLA allocates for the call, for a
-# backward of 5 GEMMs instead of 7).  The size query below sees the same flag, so the scratch result of the
-# custom call grows with it.
-BWD_DS_WORKSPACE = False
+# backward of 5 GEMMs instead of 7).  None: do so whenever that scratch fits BWD_WORKSPACE_LIMIT_BYTES
+# (the same rule as HipFlashAttention.Config.bwd_ds_workspace / bwd_workspace_limit_bytes on the torch
+# side); True / False force the choice.  The size query below sees the flag that was chosen, so the
+# scratch result of the custom call grows with it.
+BWD_DS_WORKSPACE = None
+BWD_WORKSPACE_LIMIT_BYTES = 18 << 30  # a sixteenth of an MI355X's 288 GB
 _AXL_BWD_DS_WORKSPACE = 1
 
 
@@ -147,9 +150,12 @@ def _flash_bwd(softmax_scale, mask_kind, sliding_window, dropout_rate, logit_sin
     query, key, value, bias, segment_ids, dropout_mask, out, lse = res
     b, t, hq, d = query.shape
     s, hkv = key.shape[1], key.shape[2]
-    flags = _AXL_BWD_DS_WORKSPACE if BWD_DS_WORKSPACE else 0
-    ws_bytes = _bwd_workspace_bytes(b, t, s, hq, hkv, d, _DTYPE_CODE[jnp.dtype(query.dtype)], mask_kind,
-                                    segment_ids is not None, flags)
+    size_args = (b, t, s, hq, hkv, d, _DTYPE_CODE[jnp.dtype(query.dtype)], mask_kind, segment_ids is not None)
+    flags = _AXL_BWD_DS_WORKSPACE if BWD_DS_WORKSPACE or BWD_DS_WORKSPACE is None else 0
+    ws_bytes = _bwd_workspace_bytes(*size_args, flags)
+    if BWD_DS_WORKSPACE is None and flags and ws_bytes > BWD_WORKSPACE_LIMIT_BYTES:
+        flags = 0  # too large for the automatic choice: the recomputing pair
+        ws_bytes = _bwd_workspace_bytes(*size_args, flags)
     dq, dk, dv, _, _ = jax.ffi.ffi_call(
         "AxlFlashBwd",
         (jax.ShapeDtypeStruct(query.shape, query.dtype), jax.ShapeDtypeStruct(key.shape, key.dtype),

@@ -31,6 +31,8 @@ __all__ = [
     "flash_fwd",
     "flash_bwd",
     "flash_bwd_buffers",
+    "flash_bwd_ds_workspace_bytes",
+    "default_bwd_workspace_limit",
     "paged_decode",
     "decode",
 ]
@@ -203,7 +205,8 @@ def flash_bwd(
     bias: Optional[torch.Tensor] = None,
     dropout_mask: Optional[torch.Tensor] = None,
     dropout_rate: float = 0.0,
-    ds_workspace: bool = False,
+    ds_workspace: Optional[bool] = False,
+    ds_workspace_limit: Optional[int] = None,
 ):
     """Returns (dq [B,T,Hq,D], dk [B,S,Hkv,D], dv [B,S,Hkv,D]) in the dtype of q, followed by
     d_logit_sink [Hq] fp32 when `logit_sink` (the one the forward was given) is passed.
@@ -213,9 +216,15 @@ def flash_bwd(
     dropout_mask and dropout_rate must be the ones the forward was given (the bias gets no gradient,
     as in gpu_attention.py:786).  `ds_workspace=True` (AXL_BWD_DS_WORKSPACE; causal or sliding-window
     attention over equal lengths without offsets, bias or dropout; ignored otherwise) keeps dS in a
-    larger workspace instead of recomputing it for dq."""
+    larger workspace instead of recomputing it for dq.  `ds_workspace=None` decides by size: the dS
+    workspace is used when that path applies and fits `ds_workspace_limit` bytes (default:
+    `default_bwd_workspace_limit`, a sixteenth of the device's memory)."""
     b, t, hq, d, s, hkv = _check_qkv(q, k, v)
     _check_segment_ids(segment_ids, b, t, s)
+    if ds_workspace is None:
+        ds_workspace = (phases == 7 and bias is None and dropout_mask is None and q_pos_offset == 0
+                        and select_ds_workspace(q, k, mask_kind=mask_kind, segment_ids=segment_ids,
+                                                limit=ds_workspace_limit))
     _want_shape("out", out, q.shape)
     _want_shape("d_out", d_out, q.shape)
     _want_shape("lse", lse, (b, hq, t))
@@ -284,6 +293,38 @@ def flash_bwd_buffers(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, mask
     nbytes = int(_lib.load().axl_flash_bwd_workspace_bytes(ctypes.byref(p)))
     ws = torch.empty((max(nbytes, 256),), dtype=torch.uint8, device=q.device)
     return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), ws
+
+
+def flash_bwd_ds_workspace_bytes(q: torch.Tensor, k: torch.Tensor, *, mask_kind: int,
+                                 segment_ids: Optional[torch.Tensor] = None) -> Tuple[int, int]:
+    """(bytes with AXL_BWD_DS_WORKSPACE, bytes without) of backward workspace for these shapes and
+    this mask; the two are equal where the dS-workspace path does not apply (the flag is ignored)."""
+    b, t, hq, d = q.shape
+    p = AxlFlashBwdParams(batch=b, q_len=t, kv_len=k.shape[1], num_q_heads=hq, num_kv_heads=k.shape[2],
+                          head_dim=d, dtype=_lib.dtype_code(q.dtype), mask_kind=mask_kind,
+                          segment_ids=None if segment_ids is None else 256, flags=_lib.BWD_DS_WORKSPACE)
+    lib = _lib.load()
+    with_ds = int(lib.axl_flash_bwd_workspace_bytes(ctypes.byref(p)))
+    p.flags = 0
+    return with_ds, int(lib.axl_flash_bwd_workspace_bytes(ctypes.byref(p)))
+
+
+def default_bwd_workspace_limit(device) -> int:
+    """Transient bytes the backward may take for dS when the caller states no limit: a sixteenth of the
+    device's memory (18 GB of an MI355X's 288 GB)."""
+    return torch.cuda.get_device_properties(device).total_memory // 16
+
+
+def select_ds_workspace(q: torch.Tensor, k: torch.Tensor, *, mask_kind: int,
+                        segment_ids: Optional[torch.Tensor] = None, limit: Optional[int] = None) -> bool:
+    """The backward's default policy: keep dS in the workspace (5 executed GEMMs instead of 7) when
+    that path applies to these shapes and its workspace fits `limit` bytes."""
+    with_ds, without = flash_bwd_ds_workspace_bytes(q, k, mask_kind=mask_kind, segment_ids=segment_ids)
+    if with_ds == without:
+        return False
+    if limit is None:
+        limit = default_bwd_workspace_limit(q.device)
+    return with_ds <= int(limit)
 
 
 def _decode_flags(deterministic: bool, workspace_reused: bool) -> int:

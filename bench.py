@@ -4,11 +4,15 @@
 
 The headline workload (BASELINE.json configs[1], "C2") is causal GQA flash attention forward +
 backward, bf16, batch 4, 32 query heads / 8 kv heads, seq 4096, head_dim 128: a step is one forward
-(axl_flash_fwd) plus one backward (axl_flash_bwd) over one synthetic batch already resident in HBM.
-The backward of the headline step keeps dS in a workspace the caller provides (AXL_BWD_DS_WORKSPACE);
-`c2_recompute` in the same line is the same step through the backward that recomputes dS instead
-(`--recompute` makes that one the headline).  `c3` and `c5` are reported the same way (with the
-workspace, 8.7 GB and 69 GB, and as `c3_recompute`, `c5_recompute`).
+plus one backward over one synthetic batch already resident in HBM, obtained the way a caller of the
+library obtains them: `flash_attention_implementation("gpu", ...)` with the default configuration, the
+returned kernel object applied to the batch, autograd's backward with a given dO (`c_abi_ms_per_step`
+in the same object is the same pair of C-ABI calls with buffers allocated once).  The default
+configuration keeps dS in the backward's workspace when that workspace fits a sixteenth of the
+device's memory (C2: 2.15 GB, C3: 8.7 GB) and recomputes dS in the dQ kernel when it does not (C5:
+69 GB); `backward` and `backward_chosen_by` say which ran.  `c2_recompute` / `c3_recompute` /
+`c5_ds_workspace` in the same line are the same steps with the other backward forced through
+`backend_overrides` (`--recompute` / `--ds-workspace` force it for the headline).
 The paged-decode half of the metric (configs[3], "C4") is measured in the same run and reported in
 the `paged_decode` object of the same JSON line.  With the default `--workload all` the line also
 carries `c1` (configs[0]: the fp32 case the reference itself runs on CPU), `c3` (sliding window +
@@ -45,23 +49,19 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16
 MFMA_F32_PEAK_TFLOPS = 157.3    # MI355X dense fp32 matrix
 HBM_PEAK_GBS = 8000.0           # MI355X HBM3E
 
-# HBM bytes per launch of each workload's dominant kernel, measured with rocprofv3 --pmc (FETCH_SIZE x
-# 2.0 + WRITE_SIZE x 1.0, in KiB; the factors are what the same counters read for a plain 1 GiB copy
-# kernel, `--calibrate-copy`).  Constants from the committed profile named next to each: the run
-# that prints them does not read the counters itself.
-TRAFFIC = {
-    "c2": dict(bytes=3.204e9, source="profiles/flash_c2_trace_counters.md (flash_bwd_dkdv_kernel, dS-workspace step)"),
-    "c2_recompute": dict(bytes=0.982e9, source="profiles/flash_c2_trace_counters.md (flash_bwd_dkdv_kernel, --recompute)"),
-    "c3": dict(bytes=5.666e9, source="profiles/flash_c3_c5_trace_counters.md (flash_bwd_dkdv_kernel, segment ids, dS-workspace step)"),
-    "c3_recompute": dict(bytes=1.902e9, source="profiles/flash_c3_c5_trace_counters.md (flash_bwd_dkdv_kernel, segment ids, --recompute)"),
-    "c5": dict(bytes=91.89e9, source="profiles/flash_c3_c5_trace_counters.md (flash_bwd_dkdv_kernel, dS-workspace step)"),
-    "c5_recompute": dict(bytes=24.17e9, source="profiles/flash_c3_c5_trace_counters.md (flash_bwd_dkdv_kernel, --recompute)"),
-    "c4": dict(bytes=4.254e9, source="profiles/paged_decode_c4_trace_counters.md (decode_split_kernel)"),
-}
+# HBM bytes per launch of each workload's dominant kernel come from profiles/traffic.json, which is
+# written next to the rocprofv3 --pmc summaries it is taken from (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0,
+# in KiB; the factors are what the same counters read for a plain 1 GiB copy kernel,
+# `--calibrate-copy`): the run that prints them does not read the counters itself.
+def _load_traffic():
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            return json.load(f)
+    except (OSError, ValueError):
+        return {}
 
-# Workloads whose default step runs the backward that keeps dS in a caller-provided workspace
-# (AXL_BWD_DS_WORKSPACE: 5 executed GEMMs instead of 7; 2.1 GB for C2, 8.7 GB for C3, 69 GB for C5).
-DS_WORKSPACE_WORKLOADS = ("c2", "c3", "c5")
+
+TRAFFIC = _load_traffic()
 
 METRIC = "flash-attn fwd+bwd TFLOP/s; paged-decode HBM GB/s (% roofline), 1 MI355X"
 
@@ -142,15 +142,36 @@ def _traffic(name):
     return (None, None) if t is None else (t["bytes"], t["source"])
 
 
+def _dispatch_bias(cfg, seg, T, dev):
+    """The attention bias a layer would hand to the dispatch for this workload."""
+    from axlearn_amd import attention_bias as ab
+
+    pos = dict(target_positions=torch.arange(T, device=dev)[None], source_positions=torch.arange(T, device=dev)[None])
+    parts = []
+    if cfg["mask"] == "causal":
+        parts.append(ab.CausalAttentionBias(**pos))
+    elif cfg["mask"] == "sliding":
+        parts.append(ab.SlidingWindowAttentionBias(ab.sliding_window_causal_mask(cfg["window"]),
+                                                   sliding_window_size=cfg["window"], **pos))
+    if seg is not None:
+        parts.append(ab.SegmentIdAttentionBias(seg))
+    return ab.CompositeAttentionBias(parts)
+
+
 def bench_flash(cfg, steps, warmup, cpu_baseline):
+    """One fwd+bwd step = what a caller of `flash_attention_implementation("gpu", ...)` gets: the
+    returned kernel object applied to the batch, then autograd's backward with a given dO.
+    cfg["ds_workspace"]: None = the plugin's default (dS workspace when it fits the default limit, a
+    sixteenth of the device's memory), True / False = forced through backend_overrides."""
     from axlearn_amd import ops
+    from axlearn_amd.flash_attention.utils import flash_attention_implementation
 
     dev = torch.device("cuda:0")
     B, T, Hq, Hkv, D = cfg["B"], cfg["T"], cfg["Hq"], cfg["Hkv"], cfg["D"]
     bf = torch.bfloat16
-    q = normal_tensor(0, (B, T, Hq, D), bf, dev)
-    k = normal_tensor(1, (B, T, Hkv, D), bf, dev)
-    v = normal_tensor(2, (B, T, Hkv, D), bf, dev)
+    q = normal_tensor(0, (B, T, Hq, D), bf, dev).requires_grad_(True)
+    k = normal_tensor(1, (B, T, Hkv, D), bf, dev).requires_grad_(True)
+    v = normal_tensor(2, (B, T, Hkv, D), bf, dev).requires_grad_(True)
     do = normal_tensor(3, (B, T, Hq, D), bf, dev)
     seg = None
     pairs = None
@@ -158,22 +179,46 @@ def bench_flash(cfg, steps, warmup, cpu_baseline):
         seg = packed_segment_ids(4, B, T).to(dev)
         pairs = count_pairs(seg, cfg["window"])
     mask_kind = {"none": ops.MASK_NONE, "causal": ops.MASK_CAUSAL, "sliding": ops.MASK_SLIDING_WINDOW}[cfg["mask"]]
-    kw = dict(softmax_scale=D ** -0.5, mask_kind=mask_kind, sliding_window=cfg["window"], segment_ids=seg)
-    spill = bool(cfg.get("ds_workspace"))
-    bufs = ops.flash_bwd_buffers(q, k, v, mask_kind=mask_kind, ds_workspace=spill, segment_ids=seg)
-    kw_b = dict(kw, ds_workspace=spill)
-    out, lse = ops.flash_fwd(q, k, v, **kw)
+    forced = cfg.get("ds_workspace")
+    if forced is None:
+        spill = ops.select_ds_workspace(q, k, mask_kind=mask_kind, segment_ids=seg)
+        chosen = "default config (by workspace size)"
+    else:
+        spill = bool(forced)
+        chosen = f"backend_overrides bwd_ds_workspace={spill}"
+    ws_need, _ = ops.flash_bwd_ds_workspace_bytes(q, k, mask_kind=mask_kind, segment_ids=seg)
+    bias = _dispatch_bias(cfg, seg, T, dev)
+    impl = flash_attention_implementation(
+        "gpu", query=q, key=k, value=v, bias=bias, softmax_scale=D ** -0.5,
+        backend_overrides=None if forced is None else dict(bwd_ds_workspace=spill))
+    if impl is None:
+        sys.exit("bench.py: the dispatch found no kernel for " + cfg["label"])
+    batch = dict(query=q, key=k, value=v, bias=bias)
 
     def step():
-        o, l = ops.flash_fwd(q, k, v, **kw)
-        ops.flash_bwd(q, k, v, o, l, do, buffers=bufs, **kw_b)
+        q.grad = k.grad = v.grad = None
+        impl.fn(batch).backward(do)
 
     ms_step = _time_region(step, steps, warmup)
-    # Per-kernel durations, each kernel timed over its own launches.
-    ms_fwd = _time_region(lambda: ops.flash_fwd(q, k, v, **kw), steps, 1)
-    ms_delta = _time_region(lambda: ops.flash_bwd(q, k, v, out, lse, do, buffers=bufs, phases=1, **kw_b), steps, 1)
-    ms_dkdv = _time_region(lambda: ops.flash_bwd(q, k, v, out, lse, do, buffers=bufs, phases=2, **kw_b), steps, 1)
-    ms_dq = _time_region(lambda: ops.flash_bwd(q, k, v, out, lse, do, buffers=bufs, phases=4, **kw_b), steps, 1)
+    q.grad = k.grad = v.grad = None
+    # The same kernels through the C ABI with buffers allocated once (no allocator, no autograd).
+    qd, kd, vd = q.detach(), k.detach(), v.detach()
+    kw = dict(softmax_scale=D ** -0.5, mask_kind=mask_kind, sliding_window=cfg["window"], segment_ids=seg)
+    bufs = ops.flash_bwd_buffers(qd, kd, vd, mask_kind=mask_kind, ds_workspace=spill, segment_ids=seg)
+    kw_b = dict(kw, ds_workspace=spill)
+    out, lse = ops.flash_fwd(qd, kd, vd, **kw)
+
+    def abi_step():
+        o, l = ops.flash_fwd(qd, kd, vd, **kw)
+        ops.flash_bwd(qd, kd, vd, o, l, do, buffers=bufs, **kw_b)
+
+    ms_abi = _time_region(abi_step, steps, 2)
+    # Per-kernel durations, each kernel timed over its own launches (device events on the stream the
+    # launches go to).  With the dS workspace the dq phase reads what the dK/dV phase before it left.
+    ms_fwd = _time_region(lambda: ops.flash_fwd(qd, kd, vd, **kw), steps, 1)
+    ms_delta = _time_region(lambda: ops.flash_bwd(qd, kd, vd, out, lse, do, buffers=bufs, phases=1, **kw_b), steps, 1)
+    ms_dkdv = _time_region(lambda: ops.flash_bwd(qd, kd, vd, out, lse, do, buffers=bufs, phases=2, **kw_b), steps, 1)
+    ms_dq = _time_region(lambda: ops.flash_bwd(qd, kd, vd, out, lse, do, buffers=bufs, phases=4, **kw_b), steps, 1)
 
     if pairs is None:
         gemm = 2.0 * B * Hq * (T * T / 2.0) * D  # one [T,T,D] causal GEMM (the 1/2 convention)
@@ -183,10 +228,13 @@ def bench_flash(cfg, steps, warmup, cpu_baseline):
     fl_dkdv, fl_dq = 4 * gemm, 1 * gemm           # S, dP, dV, dK | dQ
     tf = lambda fl, ms: fl / (ms * 1e-3) / 1e12
     dq_name = "flash_bwd_dq_stream_kernel" if spill else "flash_bwd_dq_ring_kernel"
-    traffic, traffic_src = _traffic(cfg["name"] + ("_recompute" if cfg["name"] in DS_WORKSPACE_WORKLOADS and not spill else ""))
+    traffic, traffic_src = _traffic(cfg["name"] + ("" if spill else "_recompute"))
     result = dict(
         workload=cfg["label"], value=tf(fl_fwd + fl_bwd, ms_step), unit="TFLOP/s", ms_per_step=ms_step,
+        entry="flash_attention_implementation('gpu', ...).fn(batch) + autograd backward",
         backward="dS workspace: delta, dK/dV (stores dS), dq = dS k" if spill else "dQ (recomputes dS, computes delta), dK/dV",
+        backward_chosen_by=chosen, ds_workspace_bytes=ws_need if spill else 0,
+        c_abi_ms_per_step=ms_abi,
         kernels={
             "flash_fwd_kernel": dict(ms=ms_fwd, tflops=tf(fl_fwd, ms_fwd), algorithmic_tflop=fl_fwd / 1e12),
             "bwd_delta_kernel": dict(ms=ms_delta, in_step=spill),
@@ -204,7 +252,7 @@ def bench_flash(cfg, steps, warmup, cpu_baseline):
         result["unmasked_pairs"] = pairs
     if cpu_baseline:
         result["cpu_baseline"] = cpu_baseline_flash(cfg)
-    del q, k, v, do, out, lse, bufs
+    del q, k, v, qd, kd, vd, do, out, lse, bufs, batch, impl
     torch.cuda.empty_cache()
     return result
 
@@ -304,12 +352,15 @@ def bench_paged_decode(steps, warmup, cpu_baseline):
     out = torch.empty((B, Hq, D), device=dev, dtype=bf)
     ws = torch.empty((ops.paged_decode_workspace_bytes(B, Hq, Hkv, D, pps),), device=dev, dtype=torch.uint8)
     scale = D ** -0.5
-    # A serving loop keeps one workspace: the first call zeroes its work counter, every later call
-    # finds it at zero (AXL_DECODE_WORKSPACE_REUSED) and launches the split and merge kernels only.
-    ops.paged_decode(q, kp, vp, tables, lengths, softmax_scale=scale, workspace=ws, out=out)
-    fn = lambda: ops.paged_decode(q, kp, vp, tables, lengths, softmax_scale=scale, workspace=ws, out=out,
-                                  workspace_reused=True)
+    # The timed call is what a caller whose scratch memory comes from an allocator per call (XLA) gets:
+    # the library zeroes the work counter of a workspace it knows nothing about (one extra one-thread
+    # launch).  A serving loop that keeps one workspace sets AXL_DECODE_WORKSPACE_REUSED from its second
+    # call on and launches the split and merge kernels only: reported beside it.
+    fn = lambda: ops.paged_decode(q, kp, vp, tables, lengths, softmax_scale=scale, workspace=ws, out=out)
     ms = _time_region(fn, steps, warmup)
+    fn_reused = lambda: ops.paged_decode(q, kp, vp, tables, lengths, softmax_scale=scale, workspace=ws, out=out,
+                                         workspace_reused=True)
+    ms_reused = _time_region(fn_reused, steps, 2)
     live_pages = int(((lengths_cpu.long() + page - 1) // page).sum())
     # Algorithmic bytes: every live K and V page once, its page-table entry, q and out.
     algo_bytes = live_pages * page * Hkv * D * 2 * 2 + live_pages * 4 + 2 * B * Hq * D * 2
@@ -318,6 +369,7 @@ def bench_paged_decode(steps, warmup, cpu_baseline):
     res = dict(
         workload="C4: paged decode, bf16, B64 Hq32/Hkv8 D128, page 16, ctx U[512,32768]",
         value=gbs, unit="GB/s", ms_per_step=ms, algorithmic_gb=algo_bytes / 1e9,
+        workspace_reused=dict(ms_per_step=ms_reused, value=algo_bytes / (ms_reused * 1e-3) / 1e9, unit="GB/s"),
         roofline=dict(kernel="decode_split_kernel", bound="hbm", achieved=gbs, peak=HBM_PEAK_GBS, unit="GB/s",
                       frac=gbs / HBM_PEAK_GBS, traffic=traffic, traffic_source=traffic_src),
     )
@@ -376,7 +428,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true", help="skip the paged-decode half of the metric")
     ap.add_argument("--recompute", action="store_true",
-                    help="C2 through the backward whose dQ kernel recomputes dS (no dS workspace)")
+                    help="force the backward whose dQ kernel recomputes dS (no dS workspace)")
+    ap.add_argument("--ds-workspace", action="store_true",
+                    help="force the backward that keeps dS in its workspace, whatever its size")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (known traffic) for scaling rocprofv3 byte counters")
     args = ap.parse_args()
@@ -414,14 +468,15 @@ def main():
         line["c1"] = res
     else:
         cfg = _flash_workload("c2" if args.workload == "all" else args.workload)
-        if cfg["name"] in DS_WORKSPACE_WORKLOADS and not args.recompute:
-            cfg = dict(cfg, ds_workspace=True)
+        forced = False if args.recompute else (True if args.ds_workspace else None)
+        cfg = dict(cfg, ds_workspace=forced)
         res = bench_flash(cfg, args.steps, args.warmup, cpu_base)
         line.update(value=res["value"], unit="TFLOP/s", ms_per_step=res["ms_per_step"],
                     config=dict(workload=cfg["label"], batch=cfg["B"], seq_len=cfg["T"], num_q_heads=cfg["Hq"],
                                 num_kv_heads=cfg["Hkv"], head_dim=cfg["D"], mask=cfg["mask"], window=cfg["window"],
-                                segment_ids=cfg["seg"], backward=res["backward"]),
-                    roofline=res["roofline"], kernels=res["kernels"],
+                                segment_ids=cfg["seg"], entry=res["entry"], backward=res["backward"],
+                                backward_chosen_by=res["backward_chosen_by"]),
+                    roofline=res["roofline"], kernels=res["kernels"], c_abi_ms_per_step=res["c_abi_ms_per_step"],
                     step_frac_of_mfma_peak=res["step_frac_of_mfma_peak"])
         if "unmasked_pairs" in res:
             line["unmasked_pairs"] = res["unmasked_pairs"]
@@ -431,19 +486,19 @@ def main():
             line["paged_decode"] = bench_paged_decode(args.steps, args.warmup, cpu_base)
         if args.workload == "all":
             # The other BASELINE configs, fewer repetitions: they are reported, not the headline.
-            # The same C2 step through the other backward (the dQ kernel recomputes dS; no dS workspace).
-            line["c2_recompute" if cfg.get("ds_workspace") else "c2_ds_workspace"] = bench_flash(
-                dict(cfg, ds_workspace=not cfg.get("ds_workspace")), args.steps, args.warmup, False)
+            def other(name, first, n_steps, n_warm):
+                # the same step with the backward the default did not pick, forced through backend_overrides
+                took_ds = first["backward"].startswith("dS workspace")
+                key = name + ("_recompute" if took_ds else "_ds_workspace")
+                line[key] = bench_flash(dict(_flash_workload(name), ds_workspace=not took_ds), n_steps, n_warm, False)
+
+            other("c2", res, args.steps, args.warmup)
             line["machine"] = calibrate_mfma()
             line["c1"] = bench_c1(args.steps, args.warmup, cpu_base)
-            c3 = dict(_flash_workload("c3"), ds_workspace=not args.recompute)
-            line["c3"] = bench_flash(c3, max(5, args.steps // 2), 2, cpu_base)
-            line["c3_recompute" if c3["ds_workspace"] else "c3_ds_workspace"] = bench_flash(
-                dict(c3, ds_workspace=not c3["ds_workspace"]), max(5, args.steps // 2), 2, False)
-            c5 = dict(_flash_workload("c5"), ds_workspace=not args.recompute)
-            line["c5"] = bench_flash(c5, max(3, args.steps // 4), 1, cpu_base)
-            line["c5_recompute" if c5["ds_workspace"] else "c5_ds_workspace"] = bench_flash(
-                dict(c5, ds_workspace=not c5["ds_workspace"]), max(3, args.steps // 4), 1, False)
+            line["c3"] = bench_flash(dict(_flash_workload("c3"), ds_workspace=forced), max(5, args.steps // 2), 2, cpu_base)
+            other("c3", line["c3"], max(5, args.steps // 2), 2)
+            line["c5"] = bench_flash(dict(_flash_workload("c5"), ds_workspace=forced), max(3, args.steps // 4), 1, cpu_base)
+            other("c5", line["c5"], max(3, args.steps // 4), 1)
     print(json.dumps(line))
 
 

@@ -40,7 +40,10 @@ def _deterministic():
 
 
 def _ok(got, want):
-    return ref.max_abs(got, want) <= 2e-2 or ref.rel_l2(got, want) <= 1e-2
+    """The relative-L2 arm of the bf16 bar alone (as decoding_test.py:53-71 uses relative
+    tolerances): a decode output over n keys has rms ~ sqrt(1/n), far below 2e-2 at long contexts,
+    so the max-abs arm would pass a dropped page or a mis-merged split record."""
+    return ref.rel_l2(got, want) <= 1e-2
 
 
 @pytest.mark.parametrize("b,s,h,d", [(1, 1024, 32, 64), (4, 512, 48, 64), (2, 1024, 16, 128), (1, 4096, 8, 128)])
@@ -161,7 +164,7 @@ def test_dispatch_decode_end_to_end(dtype):
         if dtype == torch.float32:
             return got.dtype == dtype and ref.max_abs(got, want) <= 1e-5
         f = 1.0 if dtype == torch.bfloat16 else 0.125
-        return got.dtype == dtype and (ref.max_abs(got, want) <= 2e-2 * f or ref.rel_l2(got, want) <= 1e-2 * f)
+        return got.dtype == dtype and ref.rel_l2(got, want) <= 1e-2 * f
 
     tp = (lengths.long() - 1)[:, None].cuda()
     sp = torch.arange(16 * pps)[None].cuda()
@@ -390,7 +393,7 @@ def test_float16_decode_against_ref(b, s, h, hkv, d, padding, window):
                                 sliding_window=None if window < 0 else window)[:, 0]
 
     def ok(got):
-        return got.dtype == torch.float16 and (ref.max_abs(got.cpu(), want) <= 2.5e-3 or ref.rel_l2(got.cpu(), want) <= 1.25e-3)
+        return got.dtype == torch.float16 and ref.rel_l2(got.cpu(), want) <= 1.25e-3
 
     got = ops.paged_decode(q[:, 0].cuda(), kp.cuda(), vp.cuda(), tables.cuda(), lengths.cuda(),
                            softmax_scale=scale, sliding_window=window)

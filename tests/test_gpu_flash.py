@@ -806,15 +806,24 @@ def test_backward_without_saved_residuals_is_bit_identical():
 
 def test_ds_workspace_backward_through_the_plugin_config():
     """`bwd_ds_workspace` (config field or backend override) reaches the backward: dv is bit-identical
-    to the default path's, dq and dk agree to summation order, and the gradients match the kernel
-    called directly with the flag."""
+    to the recomputing path's, dq and dk agree to summation order, and the gradients match the kernel
+    called directly with the flag.  Left at its default (None) the choice goes by size: the dS
+    workspace where it fits `bwd_workspace_limit_bytes` (default a sixteenth of the device's memory),
+    the recomputing pair where it does not."""
     b, t, hq, hkv, d = 2, 512, 4, 2, 128
     q, k, v, do = _inputs(b, t, hq, hkv, d, torch.bfloat16)
     pos = dict(target_positions=torch.arange(t)[None], source_positions=torch.arange(t)[None])
     bias = ab.CompositeAttentionBias([
         ab.SlidingWindowAttentionBias(ab.sliding_window_causal_mask(100), sliding_window_size=100, **pos)])
     grads = []
-    for cfg in (dict(), dict(bwd_ds_workspace=True), dict(backend_overrides=dict(bwd_ds_workspace=True))):
+    need, plain = ops.flash_bwd_ds_workspace_bytes(q.cuda(), k.cuda(), mask_kind=ops.MASK_SLIDING_WINDOW)
+    assert plain < need < ops.default_bwd_workspace_limit(torch.device("cuda:0"))
+    for cfg in (dict(bwd_ds_workspace=False), dict(bwd_ds_workspace=True),
+                dict(backend_overrides=dict(bwd_ds_workspace=True)),
+                dict(),                                                # fits the default limit: dS workspace
+                dict(bwd_workspace_limit_bytes=need),                  # just fits
+                dict(bwd_workspace_limit_bytes=need - 1),              # does not: recomputing pair
+                dict(backend_overrides=dict(bwd_workspace_limit_bytes=plain))):
         qd, kd, vd = (x.cuda().requires_grad_(True) for x in (q, k, v))
         fa = HipFlashAttention.default_config().set(softmax_scale=d ** -0.5, **cfg).instantiate()
         out = fa(dict(query=qd, key=kd, value=vd, bias=bias))
@@ -823,11 +832,13 @@ def test_ds_workspace_backward_through_the_plugin_config():
     kw = dict(softmax_scale=d ** -0.5, mask_kind=ops.MASK_SLIDING_WINDOW, sliding_window=100)
     out, lse = ops.flash_fwd(q.cuda(), k.cuda(), v.cuda(), **kw)
     direct = ops.flash_bwd(q.cuda(), k.cuda(), v.cuda(), out, lse, do.cuda(), ds_workspace=True, **kw)
-    for g in grads[1:]:
+    for g in grads[1:5]:
         assert torch.equal(g[0], grads[0][0]) and torch.equal(g[3], grads[0][3])
         assert all(torch.equal(x, y) for x, y in zip(g[1:], direct))
         assert not torch.equal(g[1], grads[0][1])  # a different dq kernel ran
         assert ref.rel_l2(g[1].cpu(), grads[0][1].cpu().float()) < 1e-4
+    for g in grads[5:]:
+        assert all(torch.equal(x, y) for x, y in zip(g, grads[0]))
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])

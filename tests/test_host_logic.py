@@ -339,7 +339,8 @@ def test_abi_validation_without_gpu():
                                 d_out_strides=s, dq_strides=s, dk_strides=s, dv_strides=s, batch=2, q_len=256,
                                 kv_len=256, num_q_heads=4, num_kv_heads=2, head_dim=128, dtype=0, mask_kind=1,
                                 sliding_window=0, q_pos_offset=0, softmax_scale=1.0, workspace=256, workspace_bytes=16)
-    stats = 2 * (2 * 4 * 256 * 4)  # delta and scaled lse, fp32 [B, Hq, T] each
+    # delta and scaled lse, fp32 [B, Hq, T] each, plus the slack for rounding a 16-byte aligned pointer up to 256
+    stats = 2 * (2 * 4 * 256 * 4) + 240
     assert lib.axl_flash_bwd_workspace_bytes(ctypes.byref(bp)) == stats
     # plain causal attention with the dS workspace: A = T / 128 = 2 -> 8 A (A + 1) blocks of 2 KB per head
     bp.flags = _lib.BWD_DS_WORKSPACE
@@ -352,7 +353,7 @@ def test_abi_validation_without_gpu():
     assert lib.axl_flash_bwd_workspace_bytes(ctypes.byref(bp)) == stats + 256 + 256 + 2 * 4 * 48 * 2048
     bp.segment_ids = None
     bp.q_len = bp.kv_len = 384  # ... which at head_dim 128 needs 256-row blocks: the flag is ignored
-    assert lib.axl_flash_bwd_workspace_bytes(ctypes.byref(bp)) == 2 * (2 * 4 * 384 * 4)
+    assert lib.axl_flash_bwd_workspace_bytes(ctypes.byref(bp)) == 2 * (2 * 4 * 384 * 4) + 240
     bp.q_len = bp.kv_len = 256
     bp.mask_kind = 0  # no mask: no dS workspace
     assert lib.axl_flash_bwd_workspace_bytes(ctypes.byref(bp)) == stats
@@ -363,6 +364,16 @@ def test_abi_validation_without_gpu():
     assert lib.axl_flash_bwd_workspace_bytes(ctypes.byref(bp)) == stats + 256
     bp.segment_ids = None
     assert lib.axl_flash_bwd(ctypes.byref(bp), None) == _lib.AXL_ERR_WORKSPACE
+    # a pointer that is not 256-byte aligned is fine as long as the size covers the query (which
+    # includes the rounding slack): the check that follows is the next one, not the workspace's
+    bp.workspace, bp.workspace_bytes = 256 + 128, stats
+    bp.d_logit_sink = 256
+    assert lib.axl_flash_bwd(ctypes.byref(bp), None) == _lib.AXL_ERR_INVALID_ARGUMENT  # d_logit_sink without sink
+    assert b"d_logit_sink" in lib.axl_last_error()
+    bp.d_logit_sink = None
+    bp.workspace = 256 + 8
+    assert lib.axl_flash_bwd(ctypes.byref(bp), None) == _lib.AXL_ERR_WORKSPACE  # not 16-byte aligned
+    bp.workspace, bp.workspace_bytes = 256, 16
     assert lib.axl_flash_bwd_phases(ctypes.byref(bp), 0, None) == _lib.AXL_ERR_INVALID_ARGUMENT
     # Paged decode geometry.
     dp = _lib.AxlPagedDecodeParams(q=256, k_pages=256, v_pages=256, page_tables=256, lengths=256, out=256, batch=2,
