@@ -22,7 +22,7 @@ BWD_DS_WORKSPACE = 1  # AXL_BWD_DS_WORKSPACE
 AXL_OK, AXL_ERR_INVALID_ARGUMENT, AXL_ERR_UNSUPPORTED, AXL_ERR_WORKSPACE, AXL_ERR_LAUNCH = 0, -1, -2, -3, -4
 
 
-ABI_VERSION = 5  # AXL_ATTN_ABI_VERSION of include/axl_attn.h these structures mirror
+ABI_VERSION = 6  # AXL_ATTN_ABI_VERSION of include/axl_attn.h these structures mirror
 
 
 class AxlError(RuntimeError):
@@ -89,6 +89,13 @@ class AxlFlashBwdParams(ctypes.Structure):
     ]
 
 
+class AxlDecodeBias(ctypes.Structure):
+    _fields_ = [
+        ("bias", ctypes.c_void_p), ("batch_stride", ctypes.c_int64), ("head_stride", ctypes.c_int64),
+        ("dtype", ctypes.c_int32),
+    ]
+
+
 class AxlPagedDecodeParams(ctypes.Structure):
     _fields_ = [
         ("q", ctypes.c_void_p), ("k_pages", ctypes.c_void_p), ("v_pages", ctypes.c_void_p),
@@ -101,6 +108,7 @@ class AxlPagedDecodeParams(ctypes.Structure):
         ("softmax_scale", ctypes.c_float),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
         ("flags", ctypes.c_int32),
+        ("bias", AxlDecodeBias),
     ]
 
 
@@ -115,6 +123,7 @@ class AxlDecodeParams(ctypes.Structure):
         ("softmax_scale", ctypes.c_float),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
         ("flags", ctypes.c_int32),
+        ("bias", AxlDecodeBias),
     ]
 
 

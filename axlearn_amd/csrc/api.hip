@@ -233,7 +233,7 @@ int axl_flash_bwd_phases(const AxlFlashBwdParams* p, int phases, void* stream) {
 }
 
 static int check_decode_common(const char* who, int batch, int hq, int hkv, int d, int dtype,
-                               float scale) {
+                               float scale, const AxlDecodeBias& bias) {
   if (batch <= 0 || hq <= 0 || hkv <= 0 || d <= 0)
     return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: non-positive dimension", who);
   if (hq % hkv != 0)
@@ -243,10 +243,16 @@ static int check_decode_common(const char* who, int batch, int hq, int hkv, int 
     return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: softmax_scale must be finite and > 0", who);
   if (dtype != AXL_BF16 && dtype != AXL_F16 && dtype != AXL_F32)
     return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: unknown dtype %d", who, dtype);
-  if (d != 128 && d != 64)
-    return set_error(AXL_ERR_UNSUPPORTED, "%s: head_dim %d (supported: 64, 128)", who, d);
-  if (hq / hkv > 16)
-    return set_error(AXL_ERR_UNSUPPORTED, "%s: more than 16 query heads per kv head", who);
+  if (d > 128 || d % 8 != 0)
+    return set_error(AXL_ERR_UNSUPPORTED, "%s: head_dim %d (supported: multiples of 8 up to 128)", who, d);
+  if (bias.bias) {
+    if (bias.dtype != AXL_BF16 && bias.dtype != AXL_F32)
+      return set_error(AXL_ERR_UNSUPPORTED, "%s: bias dtype %d (supported: bf16, fp32)", who, bias.dtype);
+    if (bias.batch_stride < 0 || bias.head_stride < 0)
+      return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: bias strides must be >= 0", who);
+    if (reinterpret_cast<uintptr_t>(bias.bias) % (bias.dtype == AXL_F32 ? 4 : 2))
+      return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: bias is not aligned to its element type", who);
+  }
   return AXL_OK;
 }
 
@@ -259,14 +265,16 @@ size_t axl_paged_decode_workspace_bytes(const AxlPagedDecodeParams* p) {
 static int check_paged_decode(const char* who, const AxlPagedDecodeParams* p) {
   if (!p) return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: params is NULL", who);
   int rc = check_decode_common(who, p->batch, p->num_q_heads, p->num_kv_heads, p->head_dim, p->dtype,
-                               p->softmax_scale);
+                               p->softmax_scale, p->bias);
   if (rc != AXL_OK) return rc;
   if (p->num_pages <= 0 || p->page_size <= 0 || p->pages_per_seq <= 0)
     return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: non-positive page geometry", who);
   if (!p->q || !p->k_pages || !p->v_pages || !p->page_tables || !p->lengths || !p->out)
     return set_error(AXL_ERR_INVALID_ARGUMENT, "%s: NULL tensor pointer", who);
-  if (p->page_size != 16)
-    return set_error(AXL_ERR_UNSUPPORTED, "%s: page_size %d (supported: 16)", who, p->page_size);
+  if (p->page_size < 16 || (p->page_size & (p->page_size - 1)) != 0)
+    return set_error(AXL_ERR_UNSUPPORTED, "%s: page_size %d (supported: 16 times a power of two)", who, p->page_size);
+  if ((int64_t)p->page_size * p->pages_per_seq > (int64_t)1 << 30)
+    return set_error(AXL_ERR_UNSUPPORTED, "%s: page_size * pages_per_seq above 2^30", who);
   if (!aligned16(p->q) || !aligned16(p->k_pages) || !aligned16(p->v_pages) || !aligned16(p->out))
     return set_error(AXL_ERR_UNSUPPORTED, "%s: tensors must be 16-byte aligned", who);
   return AXL_OK;
@@ -296,7 +304,7 @@ size_t axl_decode_workspace_bytes(const AxlDecodeParams* p) {
 int axl_decode(const AxlDecodeParams* p, void* stream) {
   if (!p) return set_error(AXL_ERR_INVALID_ARGUMENT, "axl_decode: params is NULL");
   int rc = check_decode_common("axl_decode", p->batch, p->num_q_heads, p->num_kv_heads,
-                               p->head_dim, p->dtype, p->softmax_scale);
+                               p->head_dim, p->dtype, p->softmax_scale, p->bias);
   if (rc != AXL_OK) return rc;
   if (p->kv_len <= 0) return set_error(AXL_ERR_INVALID_ARGUMENT, "axl_decode: kv_len <= 0");
   if (!p->q || !p->k || !p->v || !p->lengths || !p->out)

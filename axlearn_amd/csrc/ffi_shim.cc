@@ -156,13 +156,30 @@ ffi::Error FlashBwd(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi:
   return rc == AXL_OK ? ffi::Error::Success() : Fail("axl_flash_bwd", rc);
 }
 
+// Decode bias operand: [B|1, Hq|1, S] bf16 / f32, or an empty buffer for none.
+ffi::Error FillDecodeBias(const char* who, const ffi::AnyBuffer& bias, AxlDecodeBias* out) {
+  *out = AxlDecodeBias{};
+  if (bias.element_count() == 0) return ffi::Error::Success();
+  auto d = bias.dimensions();
+  if (d.size() != 3) return ffi::Error(ffi::ErrorCode::kInvalidArgument, std::string(who) + ": bias must be [B|1, Hq|1, S]");
+  const int dt = DtypeOf(bias.element_type());
+  if (dt != AXL_BF16 && dt != AXL_F32)
+    return ffi::Error(ffi::ErrorCode::kUnimplemented, std::string(who) + ": bias must be bf16 or f32");
+  out->bias = bias.untyped_data();
+  out->dtype = dt;
+  out->head_stride = d[1] == 1 ? 0 : d[2];
+  out->batch_stride = d[0] == 1 ? 0 : d[1] * d[2];
+  return ffi::Error::Success();
+}
+
 // ---------------------------------------------------------------------------------------------
-// Contiguous-cache decode.  Operands: q [B,Hq,D], k, v [B,S,Hkv,D], lengths [B] s32.  Results: out
-// [B,Hq,D], workspace (u8).
+// Contiguous-cache decode.  Operands: q [B,Hq,D], k, v [B,S,Hkv,D], lengths [B] s32, bias [B|1,Hq|1,S]
+// | [0].  Results: out [B,Hq,D], workspace (u8, sized by axl_decode_workspace_bytes with the same
+// bias presence).
 // ---------------------------------------------------------------------------------------------
 ffi::Error Decode(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi::AnyBuffer v, ffi::AnyBuffer lengths,
-                  ffi::Result<ffi::AnyBuffer> out, ffi::Result<ffi::AnyBuffer> workspace, float softmax_scale,
-                  int32_t sliding_window, int32_t flags) {
+                  ffi::AnyBuffer bias, ffi::Result<ffi::AnyBuffer> out, ffi::Result<ffi::AnyBuffer> workspace,
+                  float softmax_scale, int32_t sliding_window, int32_t flags) {
   auto qd = q.dimensions(), kd = k.dimensions();
   if (qd.size() != 3 || kd.size() != 4)
     return ffi::Error(ffi::ErrorCode::kInvalidArgument, "axl_decode: q must be [B,Hq,D], k / v [B,S,Hkv,D]");
@@ -178,18 +195,19 @@ ffi::Error Decode(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k, ffi::A
   p.workspace = workspace->untyped_data(); p.workspace_bytes = workspace->size_bytes();
   // XLA hands out a fresh scratch buffer per call: never AXL_DECODE_WORKSPACE_REUSED.
   p.flags = flags & AXL_DECODE_DETERMINISTIC;
+  if (auto e = FillDecodeBias("axl_decode", bias, &p.bias); e.failure()) return e;
   const int rc = axl_decode(&p, stream);
   return rc == AXL_OK ? ffi::Error::Success() : Fail("axl_decode", rc);
 }
 
 // ---------------------------------------------------------------------------------------------
 // Paged decode.  Operands: q [B,Hq,D], k_pages, v_pages [Hkv,P,page,D], page_tables [B,pps] s32,
-// lengths [B] s32.  Results: out [B,Hq,D], workspace (u8).
+// lengths [B] s32, bias [B|1,Hq|1,pps*page] | [0].  Results: out [B,Hq,D], workspace (u8).
 // ---------------------------------------------------------------------------------------------
 ffi::Error PagedDecode(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k_pages, ffi::AnyBuffer v_pages,
-                       ffi::AnyBuffer page_tables, ffi::AnyBuffer lengths, ffi::Result<ffi::AnyBuffer> out,
-                       ffi::Result<ffi::AnyBuffer> workspace, float softmax_scale, int32_t sliding_window,
-                       int32_t flags) {
+                       ffi::AnyBuffer page_tables, ffi::AnyBuffer lengths, ffi::AnyBuffer bias,
+                       ffi::Result<ffi::AnyBuffer> out, ffi::Result<ffi::AnyBuffer> workspace, float softmax_scale,
+                       int32_t sliding_window, int32_t flags) {
   auto qd = q.dimensions(), pd = k_pages.dimensions(), td = page_tables.dimensions();
   if (qd.size() != 3 || pd.size() != 4 || td.size() != 2)
     return ffi::Error(ffi::ErrorCode::kInvalidArgument,
@@ -206,6 +224,7 @@ ffi::Error PagedDecode(hipStream_t stream, ffi::AnyBuffer q, ffi::AnyBuffer k_pa
   p.sliding_window = sliding_window; p.softmax_scale = softmax_scale;
   p.workspace = workspace->untyped_data(); p.workspace_bytes = workspace->size_bytes();
   p.flags = flags & AXL_DECODE_DETERMINISTIC;
+  if (auto e = FillDecodeBias("axl_paged_decode", bias, &p.bias); e.failure()) return e;
   const int rc = axl_paged_decode(&p, stream);
   return rc == AXL_OK ? ffi::Error::Success() : Fail("axl_paged_decode", rc);
 }
@@ -299,6 +318,7 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(AxlDecode, Decode,
                                   .Arg<ffi::AnyBuffer>()  // k
                                   .Arg<ffi::AnyBuffer>()  // v
                                   .Arg<ffi::AnyBuffer>()  // lengths
+                                  .Arg<ffi::AnyBuffer>()  // bias | [0]
                                   .Ret<ffi::AnyBuffer>()  // out
                                   .Ret<ffi::AnyBuffer>()  // workspace
                                   .Attr<float>("softmax_scale")
@@ -313,6 +333,7 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(AxlPagedDecode, PagedDecode,
                                   .Arg<ffi::AnyBuffer>()  // v_pages
                                   .Arg<ffi::AnyBuffer>()  // page_tables
                                   .Arg<ffi::AnyBuffer>()  // lengths
+                                  .Arg<ffi::AnyBuffer>()  // bias | [0]
                                   .Ret<ffi::AnyBuffer>()  // out
                                   .Ret<ffi::AnyBuffer>()  // workspace
                                   .Attr<float>("softmax_scale")

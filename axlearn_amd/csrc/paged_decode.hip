@@ -641,7 +641,10 @@ __global__ __launch_bounds__(256) void decode_split_f32_kernel(const DecArgs a) 
   __shared__ float q_lds[GP * D];
   __shared__ float red_o[4][GP][D];
   __shared__ float red_m[4][GP], red_l[4][GP];
-  const int c = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
+  const int c = blockIdx.x, hv = blockIdx.y, b = blockIdx.z;
+  const int hk = hv / a.ngrp, grp = hv - hk * a.ngrp;
+  const int gcount = min(16, a.G - 16 * grp);   // query heads of this group
+  const int hbase = hk * a.G + 16 * grp;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, sub = lane >> 4, l16 = lane & 15;
   const int len = clamp_length(a, a.lengths[b]);
   int ch0, ch1;
@@ -651,8 +654,11 @@ __global__ __launch_bounds__(256) void decode_split_f32_kernel(const DecArgs a) 
   const int first_page = a.window >= 0 ? max(0, len - 1 - a.window) / kPage : 0;
   const int p_begin = max((ch0 + c) * a.chunk_pages, first_page);
   const int p_end = min((ch0 + c + 1) * a.chunk_pages, npages);
-  const float* qg = (const float*)a.q + ((int64_t)b * a.Hq + hk * a.G) * D;
-  for (int i = tid; i < GP * D; i += 256) q_lds[i] = i < a.G * D ? qg[i] : 0.f;
+  const float* qg = (const float*)a.q + ((int64_t)b * a.Hq + hbase) * a.d_real;
+  for (int i = tid; i < GP * D; i += 256) {
+    const int h = i / D, d = i % D;   // columns past head_dim and heads past the group are zero
+    q_lds[i] = (h < gcount && d < a.d_real) ? qg[h * a.d_real + d] : 0.f;
+  }
   __syncthreads();
 
   float m[GP], l[GP], o[GP][SL];
@@ -667,10 +673,11 @@ __global__ __launch_bounds__(256) void decode_split_f32_kernel(const DecArgs a) 
     const float *kr, *vr;
     bool valid = true;
     if (PAGED) {
-      int pg = a.page_tables[(int64_t)b * a.pps + tok / kPage];
+      const int page_tokens = kPage << a.page_shift;
+      int pg = a.page_tables[(int64_t)b * a.pt_stride + tok / page_tokens];
       if (pg < 0) pg += a.num_pages;  // negative indices count from the end, as in the reference's gather
       valid = (unsigned)pg < (unsigned)a.num_pages;  // a page outside the pool reads as zeros
-      const int64_t off = (((int64_t)hk * a.num_pages + (valid ? pg : 0)) * kPage + tok % kPage) * D;
+      const int64_t off = (((int64_t)hk * a.num_pages + (valid ? pg : 0)) * page_tokens + tok % page_tokens) * a.d_real;
       kr = (const float*)a.k + off;
       vr = (const float*)a.v + off;
     } else {
@@ -684,8 +691,9 @@ __global__ __launch_bounds__(256) void decode_split_f32_kernel(const DecArgs a) 
     float kx[SL], vx[SL];
 #pragma unroll
     for (int i = 0; i < SL; i += 4) {
-      const float4 x = valid ? *(const float4*)(kr + SL * l16 + i) : float4{0.f, 0.f, 0.f, 0.f};
-      const float4 y = valid ? *(const float4*)(vr + SL * l16 + i) : float4{0.f, 0.f, 0.f, 0.f};
+      const bool in = valid && SL * l16 + i < a.d_real;   // head_dim is a multiple of 8: whole groups of 4
+      const float4 x = in ? *(const float4*)(kr + SL * l16 + i) : float4{0.f, 0.f, 0.f, 0.f};
+      const float4 y = in ? *(const float4*)(vr + SL * l16 + i) : float4{0.f, 0.f, 0.f, 0.f};
       kx[i] = x.x; kx[i + 1] = x.y; kx[i + 2] = x.z; kx[i + 3] = x.w;
       vx[i] = y.x; vx[i + 1] = y.y; vx[i + 2] = y.z; vx[i + 3] = y.w;
     }
@@ -698,6 +706,7 @@ __global__ __launch_bounds__(256) void decode_split_f32_kernel(const DecArgs a) 
       dot += __shfl_xor(dot, 2, 64);
       dot += __shfl_xor(dot, 4, 64);
       dot += __shfl_xor(dot, 8, 64);
+      if (a.bias && h < gcount) dot += decode_bias_at(a, b, hbase + h, tok);
       const float mn = fmaxf(m[h], dot);
       const float corr = expf((m[h] - mn) * a.scale);
       const float pr = expf((dot - mn) * a.scale);
@@ -729,7 +738,7 @@ __global__ __launch_bounds__(256) void decode_split_f32_kernel(const DecArgs a) 
     }
   }
   __syncthreads();
-  const int64_t rec = ((int64_t)b * a.Hkv + hk) * a.nch + c;
+  const int64_t rec = ((int64_t)b * a.Hv + hv) * a.nch + c;
   for (int idx = tid; idx < GP * D; idx += 256) {
     const int h = idx / D, d = idx % D;
     const float mw = fmaxf(fmaxf(red_m[0][h], red_m[1][h]), fmaxf(red_m[2][h], red_m[3][h]));
@@ -768,21 +777,46 @@ static size_t ws_bytes(int B, int Hkv, int nch, int gp, int D) {
   return (size_t)B * Hkv * nch * ((size_t)gp * D + 2 * gp + 1) * sizeof(float) + kWsHeaderFloats * sizeof(float);
 }
 
-static int gp_of(int G) { return G <= 4 ? 4 : (G <= 8 ? 8 : 16); }
+// Query-head columns a record holds: the heads of a group padded to 4 / 8 / 16.  The kernels that add
+// a bias are compiled for 16 only.
+static int gp_of(int G, bool bias) { return bias || G > 8 ? 16 : (G <= 4 ? 4 : 8); }
+// Groups of at most 16 query heads per kv head ("virtual" kv heads per kv head).
+static int groups_of(int G) { return (G + 15) / 16; }
+// Compiled head_dim width that serves a head_dim (a multiple of 8, at most 128).
+static int width_of(int d) { return d <= 64 ? 64 : 128; }
+// log2(page_size / 16), or -1 if the page size is not 16 times a power of two.
+static int page_shift_of(int page_size) {
+  for (int sh = 0; sh < 16; sh++)
+    if (page_size == (kPage << sh)) return sh;
+  return -1;
+}
+
+static size_t ws_bytes_for(int batch, int hq, int hkv, int d, int tiles, bool bias) {
+  const int G = hq / hkv;
+  const int cp = pick_chunk_pages(tiles);
+  const int nch = (tiles + cp - 1) / cp;
+  return ws_bytes(batch, hkv * groups_of(G), nch, gp_of(G, bias), width_of(d));
+}
 
 size_t paged_decode_workspace_bytes(const AxlPagedDecodeParams& p) {
-  if (p.pages_per_seq <= 0 || p.num_kv_heads <= 0) return 0;
-  const int cp = pick_chunk_pages(p.pages_per_seq);
-  const int nch = (p.pages_per_seq + cp - 1) / cp;
-  return ws_bytes(p.batch, p.num_kv_heads, nch, gp_of(p.num_q_heads / p.num_kv_heads), p.head_dim);
+  const int sh = page_shift_of(p.page_size);
+  if (p.pages_per_seq <= 0 || p.num_kv_heads <= 0 || p.num_q_heads < p.num_kv_heads || sh < 0) return 0;
+  return ws_bytes_for(p.batch, p.num_q_heads, p.num_kv_heads, p.head_dim, p.pages_per_seq << sh, p.bias.bias != nullptr);
 }
 
 size_t decode_workspace_bytes(const AxlDecodeParams& p) {
-  if (p.kv_len <= 0 || p.num_kv_heads <= 0) return 0;
-  const int pps = (p.kv_len + kPage - 1) / kPage;
-  const int cp = pick_chunk_pages(pps);
-  const int nch = (pps + cp - 1) / cp;
-  return ws_bytes(p.batch, p.num_kv_heads, nch, gp_of(p.num_q_heads / p.num_kv_heads), p.head_dim);
+  if (p.kv_len <= 0 || p.num_kv_heads <= 0 || p.num_q_heads < p.num_kv_heads) return 0;
+  return ws_bytes_for(p.batch, p.num_q_heads, p.num_kv_heads, p.head_dim, (p.kv_len + kPage - 1) / kPage,
+                      p.bias.bias != nullptr);
+}
+
+static void set_bias(DecArgs& a, const AxlDecodeBias& x, float scale) {
+  const int es = x.dtype == AXL_F32 ? 4 : 2;
+  a.bias = (const char*)x.bias;
+  a.bias_sb = x.batch_stride * es;
+  a.bias_sh = x.head_stride * es;
+  a.bias_f32 = x.dtype == AXL_F32;
+  a.inv_scale = 1.0f / scale;
 }
 
 static int cu_count() {
@@ -808,9 +842,12 @@ static bool deterministic_by_default() {
 }
 
 template <typename E, bool PAGED>
-static int launch_common(DecArgs a, int D, int flags, hipStream_t stream, const char* who) {
-  const int gp = gp_of(a.G);
-  if (a.G > 16) return set_error(AXL_ERR_UNSUPPORTED, "%s: more than 16 query heads per kv head", who);
+static int launch_common(DecArgs a, int flags, hipStream_t stream, const char* who) {
+  const int D = width_of(a.d_real);
+  const bool bias = a.bias != nullptr;
+  const int gp = gp_of(a.G, bias);
+  a.ngrp = groups_of(a.G);
+  a.Hv = a.Hkv * a.ngrp;
   a.chunk_pages = pick_chunk_pages(a.pps);
   if (a.chunk_pages > 256)
     return set_error(AXL_ERR_UNSUPPORTED, "%s: context longer than %d tokens", who, 256 * kMaxChunks * kPage);
@@ -820,8 +857,8 @@ static int launch_common(DecArgs a, int D, int flags, hipStream_t stream, const 
   a.ticket = (int*)a.ws_o;
   a.ws_o += kWsHeaderFloats;
   float* ws = a.ws_o;
-  const size_t n_o = (size_t)a.B * a.Hkv * a.nch * gp * D;
-  const size_t n_s = (size_t)a.B * a.Hkv * a.nch * gp;
+  const size_t n_o = (size_t)a.B * a.Hv * a.nch * gp * D;
+  const size_t n_s = (size_t)a.B * a.Hv * a.nch * gp;
   a.ws_m = ws + n_o;
   a.ws_l = ws + n_o + n_s;
   a.ws_tab = (int32_t*)(ws + n_o + 2 * n_s);
@@ -831,10 +868,10 @@ static int launch_common(DecArgs a, int D, int flags, hipStream_t stream, const 
   hipError_t err = hipSuccess;
   if (!(flags & AXL_DECODE_WORKSPACE_REUSED))
     hipLaunchKernelGGL(decode_plan_kernel, dim3(1), dim3(64), 0, stream, a.ticket);
-#define AXL_DEC(E, DD, GG, NS)                                                                  \
+#define AXL_DEC(E, DD, GG, NS, BB)                                                              \
   do {                                                                                          \
     using Tile = DecTile<DD, GG, NS>;                                                           \
-    auto kern = decode_split_kernel<E, DD, GG, PAGED, NS>;                                      \
+    auto kern = decode_split_kernel<E, DD, GG, PAGED, NS, BB>;                                  \
     err = allow_dynamic_lds((const void*)kern, Tile::LDS_BYTES);                                \
     if (err == hipSuccess) {                                                                    \
       hipLaunchKernelGGL(kern, grid, dim3(256), Tile::LDS_BYTES, stream, s);                    \
@@ -846,22 +883,25 @@ static int launch_common(DecArgs a, int D, int flags, hipStream_t stream, const 
   for (int b0 = 0; b0 < a.B && err == hipSuccess; b0 += kMaxBatch) {
     DecArgs s = a;
     s.B = a.B - b0 < kMaxBatch ? a.B - b0 : kMaxBatch;
-    s.q = a.q + (size_t)b0 * a.Hq * D;
-    s.out = a.out + (size_t)b0 * a.Hq * D;
+    s.q = a.q + (size_t)b0 * a.Hq * a.d_real;
+    s.out = a.out + (size_t)b0 * a.Hq * a.d_real;
     s.lengths = a.lengths + b0;
-    if (PAGED) s.page_tables = a.page_tables + (size_t)b0 * a.pps;
+    if (PAGED) s.page_tables = a.page_tables + (size_t)b0 * a.pt_stride;
     else { s.k = a.k + b0 * a.ks.b; s.v = a.v + b0 * a.vs.b; }
-    s.ws_o = a.ws_o + (size_t)b0 * a.Hkv * a.nch * gp * D;
-    s.ws_m = a.ws_m + (size_t)b0 * a.Hkv * a.nch * gp;
-    s.ws_l = a.ws_l + (size_t)b0 * a.Hkv * a.nch * gp;
-    s.ws_tab = a.ws_tab + (size_t)b0 * a.Hkv * a.nch;
-    const dim3 cgrid(a.Hkv, s.B);
-    if (D == 128 && gp == 4) AXL_DEC(E, 128, 4, kStages128);
-    else if (D == 128 && gp == 8) AXL_DEC(E, 128, 8, kStages128);
-    else if (D == 128) AXL_DEC(E, 128, 16, kStages128);
-    else if (gp == 4) AXL_DEC(E, 64, 4, kStages64);
-    else if (gp == 8) AXL_DEC(E, 64, 8, kStages64);
-    else AXL_DEC(E, 64, 16, kStages64);
+    if (bias) s.bias = a.bias + b0 * a.bias_sb;
+    s.ws_o = a.ws_o + (size_t)b0 * a.Hv * a.nch * gp * D;
+    s.ws_m = a.ws_m + (size_t)b0 * a.Hv * a.nch * gp;
+    s.ws_l = a.ws_l + (size_t)b0 * a.Hv * a.nch * gp;
+    s.ws_tab = a.ws_tab + (size_t)b0 * a.Hv * a.nch;
+    const dim3 cgrid(a.Hv, s.B);
+    if (bias && D == 128) AXL_DEC(E, 128, 16, kStages128, true);
+    else if (bias) AXL_DEC(E, 64, 16, kStages64, true);
+    else if (D == 128 && gp == 4) AXL_DEC(E, 128, 4, kStages128, false);
+    else if (D == 128 && gp == 8) AXL_DEC(E, 128, 8, kStages128, false);
+    else if (D == 128) AXL_DEC(E, 128, 16, kStages128, false);
+    else if (gp == 4) AXL_DEC(E, 64, 4, kStages64, false);
+    else if (gp == 8) AXL_DEC(E, 64, 8, kStages64, false);
+    else AXL_DEC(E, 64, 16, kStages64, false);
   }
 #undef AXL_DEC
   if (err == hipSuccess) err = hipGetLastError();
@@ -871,8 +911,11 @@ static int launch_common(DecArgs a, int D, int flags, hipStream_t stream, const 
 }
 
 template <bool PAGED>
-static int launch_f32(DecArgs a, int D, hipStream_t stream, const char* who) {
-  const int gp = gp_of(a.G);
+static int launch_f32(DecArgs a, hipStream_t stream, const char* who) {
+  const int D = width_of(a.d_real);
+  const int gp = gp_of(a.G, a.bias != nullptr);
+  a.ngrp = groups_of(a.G);
+  a.Hv = a.Hkv * a.ngrp;
   a.chunk_pages = pick_chunk_pages(a.pps);
   if (a.chunk_pages > 256)
     return set_error(AXL_ERR_UNSUPPORTED, "%s: context longer than %d tokens", who, 256 * kMaxChunks * kPage);
@@ -881,15 +924,15 @@ static int launch_f32(DecArgs a, int D, hipStream_t stream, const char* who) {
   a.ticket = (int*)a.ws_o;
   a.ws_o += kWsHeaderFloats;
   float* ws = a.ws_o;
-  const size_t n_o = (size_t)a.B * a.Hkv * a.nch * gp * D;
-  const size_t n_s = (size_t)a.B * a.Hkv * a.nch * gp;
+  const size_t n_o = (size_t)a.B * a.Hv * a.nch * gp * D;
+  const size_t n_s = (size_t)a.B * a.Hv * a.nch * gp;
   a.ws_m = ws + n_o;
   a.ws_l = ws + n_o + n_s;
   a.ws_tab = (int32_t*)(ws + n_o + 2 * n_s);
   a.deterministic = 1;
   // One workgroup per live chunk writes that chunk's table entry; the work counter is not used (the
   // combine kernel still leaves it at zero).
-  const dim3 grid(a.nch, a.Hkv, a.B), cgrid(a.Hkv, a.B);
+  const dim3 grid(a.nch, a.Hv, a.B), cgrid(a.Hv, a.B);
 #define AXL_DEC32(DD, GG)                                                                          \
   do {                                                                                              \
     hipLaunchKernelGGL((decode_split_f32_kernel<DD, GG, PAGED>), grid, dim3(256), 0, stream, a);    \
@@ -913,12 +956,16 @@ int launch_paged_decode(const AxlPagedDecodeParams& p, hipStream_t stream) {
   a.page_tables = p.page_tables; a.lengths = p.lengths; a.out = (__bf16*)p.out;
   a.ws_o = (float*)p.workspace;
   a.B = p.batch; a.Hq = p.num_q_heads; a.Hkv = p.num_kv_heads; a.G = p.num_q_heads / p.num_kv_heads;
-  a.num_pages = p.num_pages; a.pps = p.pages_per_seq; a.kv_len = p.pages_per_seq * kPage;
+  a.page_shift = page_shift_of(p.page_size);   // the entry point has checked the page size
+  a.pt_stride = p.pages_per_seq;
+  a.num_pages = p.num_pages; a.pps = p.pages_per_seq << a.page_shift; a.kv_len = p.pages_per_seq * p.page_size;
+  a.d_real = p.head_dim;
   a.window = p.sliding_window < 0 ? -1 : p.sliding_window;
   a.scale = p.softmax_scale;
-  if (p.dtype == AXL_F32) return launch_f32<true>(a, p.head_dim, stream, "axl_paged_decode");
-  return p.dtype == AXL_F16 ? launch_common<ElemF16, true>(a, p.head_dim, p.flags, stream, "axl_paged_decode")
-                            : launch_common<ElemBf16, true>(a, p.head_dim, p.flags, stream, "axl_paged_decode");
+  set_bias(a, p.bias, p.softmax_scale);
+  if (p.dtype == AXL_F32) return launch_f32<true>(a, stream, "axl_paged_decode");
+  return p.dtype == AXL_F16 ? launch_common<ElemF16, true>(a, p.flags, stream, "axl_paged_decode")
+                            : launch_common<ElemBf16, true>(a, p.flags, stream, "axl_paged_decode");
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -980,11 +1027,14 @@ int launch_decode(const AxlDecodeParams& p, hipStream_t stream) {
   a.vs = Strides3{p.v_strides.batch, p.v_strides.seq, p.v_strides.head};
   a.B = p.batch; a.Hq = p.num_q_heads; a.Hkv = p.num_kv_heads; a.G = p.num_q_heads / p.num_kv_heads;
   a.num_pages = 0; a.pps = (p.kv_len + kPage - 1) / kPage; a.kv_len = p.kv_len;
+  a.page_shift = 0; a.pt_stride = 0;
+  a.d_real = p.head_dim;
   a.window = p.sliding_window < 0 ? -1 : p.sliding_window;
   a.scale = p.softmax_scale;
-  if (p.dtype == AXL_F32) return launch_f32<false>(a, p.head_dim, stream, "axl_decode");
-  return p.dtype == AXL_F16 ? launch_common<ElemF16, false>(a, p.head_dim, p.flags, stream, "axl_decode")
-                            : launch_common<ElemBf16, false>(a, p.head_dim, p.flags, stream, "axl_decode");
+  set_bias(a, p.bias, p.softmax_scale);
+  if (p.dtype == AXL_F32) return launch_f32<false>(a, stream, "axl_decode");
+  return p.dtype == AXL_F16 ? launch_common<ElemF16, false>(a, p.flags, stream, "axl_decode")
+                            : launch_common<ElemBf16, false>(a, p.flags, stream, "axl_decode");
 }
 
 }  // namespace axl

@@ -34,6 +34,7 @@ import numpy as np
 from jax.ad_checkpoint import checkpoint_name
 
 from axlearn.common.attention_bias import (  # the reference's own types: this file lives in its tree
+    NEG_INF,
     BaseAttentionBias,
     CausalAttentionBias,
     MaskFnAttentionBias,
@@ -210,9 +211,21 @@ def _lengths(bias: BaseAttentionBias, batch: int) -> Tensor:
     return jnp.broadcast_to(mask.target_positions[:, -1] + 1, (batch,)).astype(jnp.int32)  # gpu_decoding.py:314
 
 
-def _decode_window(bias: BaseAttentionBias) -> int:
-    kind, window, _, _ = _mask_of(bias)
-    return window if kind == MASK_SLIDING_WINDOW else -1
+def _decode_mask_and_bias(bias: BaseAttentionBias, lengths: Tensor, kv_len: int):
+    """(sliding window for the kernel or -1, bias [B|1, Hq|1, kv_len] or None).  Causal and sliding-window
+    masks are evaluated inside the kernel; any other mask fn is evaluated here as the reference's kernels
+    evaluate it, `mask_fn(kv_len - 1, key positions)` per sequence (gpu_decoding.py:110,
+    gpu_paged_attention.py:108), and handed over as a row of 0 / NEG_INF beside the explicit bias
+    [B|1, Hq|1, 1, S] (gpu_decoding.py:327-336)."""
+    mask, explicit = split(bias, MaskFnAttentionBias)
+    dense = explicit.value()[:, :, 0] if explicit.has_value() else None
+    if isinstance(mask, SlidingWindowAttentionBias):
+        return int(mask.sliding_window_size), dense
+    if isinstance(mask, CausalAttentionBias) or mask.mask is None:
+        return -1, dense
+    keep = mask.mask((lengths - 1)[:, None], jnp.arange(kv_len)[None, :])
+    row = jnp.where(keep, 0.0, NEG_INF).astype(jnp.float32)[:, None, :]
+    return -1, row if dense is None else dense.astype(jnp.float32) + row
 
 
 class HipDecoding(BaseSingleStepDecoding):
@@ -222,12 +235,14 @@ class HipDecoding(BaseSingleStepDecoding):
     def __call__(self, input_batch: Nested[Tensor | BaseAttentionBias]) -> Tensor:
         query, key, value = input_batch["query"], input_batch["key"], input_batch["value"]
         b, _, hq, d = query.shape
-        ws = _decode_workspace_bytes(b, hq, key.shape[2], d, key.shape[1])
+        lengths = _lengths(input_batch["bias"], b)
+        window, dense = _decode_mask_and_bias(input_batch["bias"], lengths, key.shape[1])
+        ws = _decode_workspace_bytes(b, hq, key.shape[2], d, key.shape[1], dense is not None)
         out, _ = jax.ffi.ffi_call(
             "AxlDecode", (jax.ShapeDtypeStruct((b, hq, d), query.dtype), jax.ShapeDtypeStruct((ws,), jnp.uint8)),
-        )(query.reshape(b, hq, d), key, value, _lengths(input_batch["bias"], b),
-          softmax_scale=np.float32(self.config.softmax_scale), sliding_window=np.int32(_decode_window(input_batch["bias"])),
-          flags=np.int32(0))
+        )(query.reshape(b, hq, d), key.astype(query.dtype), value.astype(query.dtype), lengths,
+          _empty(jnp.float32) if dense is None else dense,
+          softmax_scale=np.float32(self.config.softmax_scale), sliding_window=np.int32(window), flags=np.int32(0))
         return out.reshape(b, 1, hq, d)
 
 
@@ -239,19 +254,23 @@ class HipPagedAttention(BasePagedAttention):
         query, key, value = input_batch["query"], input_batch["key"], input_batch["value"]
         page_tables = input_batch["page_tables"]
         b, _, hq, d = query.shape
-        ws = _decode_workspace_bytes(b, hq, key.shape[0], d, page_tables.shape[1] * key.shape[2])
+        kv_len = page_tables.shape[1] * key.shape[2]
+        lengths = _lengths(input_batch["bias"], b)
+        window, dense = _decode_mask_and_bias(input_batch["bias"], lengths, kv_len)
+        ws = _decode_workspace_bytes(b, hq, key.shape[0], d, kv_len, dense is not None)
         out, _ = jax.ffi.ffi_call(
             "AxlPagedDecode", (jax.ShapeDtypeStruct((b, hq, d), query.dtype), jax.ShapeDtypeStruct((ws,), jnp.uint8)),
-        )(query.reshape(b, hq, d), key, value, page_tables.astype(jnp.int32), _lengths(input_batch["bias"], b),
-          softmax_scale=np.float32(self.config.softmax_scale), sliding_window=np.int32(_decode_window(input_batch["bias"])),
-          flags=np.int32(0))
+        )(query.reshape(b, hq, d), key.astype(query.dtype), value.astype(query.dtype), page_tables.astype(jnp.int32),
+          lengths, _empty(jnp.float32) if dense is None else dense,
+          softmax_scale=np.float32(self.config.softmax_scale), sliding_window=np.int32(window), flags=np.int32(0))
         return out.reshape(b, 1, hq, d)
 
 
-def _decode_workspace_bytes(b, hq, hkv, d, kv_len) -> int:
-    from axlearn_amd._lib import AxlDecodeParams
+def _decode_workspace_bytes(b, hq, hkv, d, kv_len, with_bias) -> int:
+    from axlearn_amd._lib import AxlDecodeBias, AxlDecodeParams
 
-    p = AxlDecodeParams(batch=b, kv_len=kv_len, num_q_heads=hq, num_kv_heads=hkv, head_dim=d, dtype=0)
+    p = AxlDecodeParams(batch=b, kv_len=kv_len, num_q_heads=hq, num_kv_heads=hkv, head_dim=d, dtype=0,
+                        bias=AxlDecodeBias(bias=256 if with_bias else None))
     _CORE_LIB.axl_decode_workspace_bytes.restype = ctypes.c_size_t
     return int(_CORE_LIB.axl_decode_workspace_bytes(ctypes.byref(p)))  # same size rule as the paged entry point
 

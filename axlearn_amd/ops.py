@@ -16,6 +16,7 @@ from axlearn_amd._lib import (
     MASK_CAUSAL,
     MASK_NONE,
     MASK_SLIDING_WINDOW,
+    AxlDecodeBias,
     AxlDecodeParams,
     AxlError,
     AxlFlashBwdParams,
@@ -340,6 +341,24 @@ def _check_decode_out_ws(q, out, workspace):
         raise _bad("workspace must be a contiguous uint8 tensor")
 
 
+def _decode_bias(bias: Optional[torch.Tensor], b: int, hq: int, kv_len: int):
+    """The AxlDecodeBias block for a bias `[B|1, Hq|1, kv_len]`; returns it with the tensor it points at."""
+    blk = AxlDecodeBias()
+    if bias is None:
+        return blk, None
+    if bias.dim() != 3 or bias.shape[0] not in (1, b) or bias.shape[1] not in (1, hq) or bias.shape[2] != kv_len:
+        raise _bad(f"bias must be [{b}|1, {hq}|1, {kv_len}], got {list(bias.shape)}")
+    if bias.dtype not in (torch.bfloat16, torch.float32):
+        bias = bias.to(torch.float32)
+    if bias.stride(-1) != 1:
+        bias = bias.contiguous()
+    blk.bias = bias.data_ptr()
+    blk.batch_stride = bias.stride(0) if bias.shape[0] > 1 else 0
+    blk.head_stride = bias.stride(1) if bias.shape[1] > 1 else 0
+    blk.dtype = _lib.dtype_code(bias.dtype)
+    return blk, bias
+
+
 def paged_decode(
     q: torch.Tensor,
     k_pages: torch.Tensor,
@@ -353,12 +372,14 @@ def paged_decode(
     out: Optional[torch.Tensor] = None,
     deterministic: bool = False,
     workspace_reused: bool = False,
+    bias: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """q [B,Hq,D]; pools [Hkv,P,page,D]; page_tables [B,pps] int32; lengths [B] int32 -> [B,Hq,D].
 
     Lengths are clamped to [0, pps * page]; a sequence of length 0 yields zeros.  `deterministic`
     fixes the work decomposition (bit-reproducible); `workspace_reused` promises that `workspace` was
-    last touched by an earlier decode call (skips the launch that zeroes its work counter)."""
+    last touched by an earlier decode call (skips the launch that zeroes its work counter).
+    bias [B|1,Hq|1,pps*page] bf16/fp32: additive logit bias per key position."""
     if q.dim() != 3 or k_pages.dim() != 4:
         raise _bad(f"q must be [B,Hq,D] and k_pages [Hkv,P,page,D], got {list(q.shape)}, {list(k_pages.shape)}")
     b, hq, d = q.shape
@@ -381,10 +402,11 @@ def paged_decode(
     _check_decode_out_ws(q, out, workspace)
     if workspace_reused and workspace is None:
         raise _bad("workspace_reused needs the workspace of the earlier call")
-    _require_cuda(q, k_pages, v_pages, page_tables, lengths, out, workspace)
+    _require_cuda(q, k_pages, v_pages, page_tables, lengths, out, workspace, bias)
     lib = _lib.load()
     if out is None:
         out = torch.empty((b, hq, d), dtype=q.dtype, device=q.device)
+    bias_blk, _keep = _decode_bias(bias, b, hq, page_size * page_tables.shape[1])
     p = AxlPagedDecodeParams(
         q=q.data_ptr(), k_pages=k_pages.data_ptr(), v_pages=v_pages.data_ptr(),
         page_tables=page_tables.data_ptr(), lengths=lengths.data_ptr(), out=out.data_ptr(),
@@ -392,7 +414,7 @@ def paged_decode(
         page_size=page_size, pages_per_seq=page_tables.shape[1],
         dtype=_lib.dtype_code(q.dtype), sliding_window=int(sliding_window),
         softmax_scale=float(softmax_scale), workspace=None, workspace_bytes=0,
-        flags=_decode_flags(deterministic, workspace_reused),
+        flags=_decode_flags(deterministic, workspace_reused), bias=bias_blk,
     )
     need = int(lib.axl_paged_decode_workspace_bytes(ctypes.byref(p)))
     if workspace is None or workspace.numel() < need:
@@ -406,13 +428,14 @@ def paged_decode(
 
 
 def paged_decode_workspace_bytes(batch: int, num_q_heads: int, num_kv_heads: int, head_dim: int,
-                                 pages_per_seq: int, page_size: int = 16) -> int:
+                                 pages_per_seq: int, page_size: int = 16, with_bias: bool = False) -> int:
     """Bytes of device workspace `paged_decode` needs for these shapes (bf16)."""
     lib = _lib.load()
     p = AxlPagedDecodeParams(
         batch=batch, num_q_heads=num_q_heads, num_kv_heads=num_kv_heads, head_dim=head_dim,
         num_pages=batch * pages_per_seq, page_size=page_size, pages_per_seq=pages_per_seq,
         dtype=_lib.dtype_code(torch.bfloat16), sliding_window=-1, softmax_scale=1.0,
+        bias=AxlDecodeBias(bias=256 if with_bias else None),
     )
     return int(lib.axl_paged_decode_workspace_bytes(ctypes.byref(p)))
 
@@ -429,9 +452,11 @@ def decode(
     out: Optional[torch.Tensor] = None,
     deterministic: bool = False,
     workspace_reused: bool = False,
+    bias: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """q [B,Hq,D]; k/v [B,S,Hkv,D]; lengths [B] int32 -> [B,Hq,D].  Lengths are clamped to [0, S]; a
-    sequence of length 0 yields zeros.  `deterministic` / `workspace_reused`: see `paged_decode`."""
+    sequence of length 0 yields zeros.  `deterministic` / `workspace_reused`: see `paged_decode`.
+    bias [B|1,Hq|1,S] bf16/fp32: additive logit bias per key position."""
     if q.dim() != 3 or k.dim() != 4:
         raise _bad(f"q must be [B,Hq,D] and k [B,S,Hkv,D], got {list(q.shape)}, {list(k.shape)}")
     b, hq, d = q.shape
@@ -451,17 +476,18 @@ def decode(
     _check_decode_out_ws(q, out, workspace)
     if workspace_reused and workspace is None:
         raise _bad("workspace_reused needs the workspace of the earlier call")
-    _require_cuda(q, k, v, lengths, out, workspace)
+    _require_cuda(q, k, v, lengths, out, workspace, bias)
     lib = _lib.load()
     if out is None:
         out = torch.empty((b, hq, d), dtype=q.dtype, device=q.device)
+    bias_blk, _keep = _decode_bias(bias, b, hq, s)
     p = AxlDecodeParams(
         q=q.data_ptr(), k=k.data_ptr(), v=v.data_ptr(), lengths=lengths.data_ptr(),
         out=out.data_ptr(), k_strides=_lib.strides4(k), v_strides=_lib.strides4(v),
         batch=b, kv_len=s, num_q_heads=hq, num_kv_heads=hkv, head_dim=d,
         dtype=_lib.dtype_code(q.dtype), sliding_window=int(sliding_window),
         softmax_scale=float(softmax_scale), workspace=None, workspace_bytes=0,
-        flags=_decode_flags(deterministic, workspace_reused),
+        flags=_decode_flags(deterministic, workspace_reused), bias=bias_blk,
     )
     need = int(lib.axl_decode_workspace_bytes(ctypes.byref(p)))
     if workspace is None or workspace.numel() < need:

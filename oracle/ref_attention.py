@@ -391,11 +391,14 @@ def reference_decode(
     sliding_window: Optional[int] = None,
     page_tables: Optional[torch.Tensor] = None,
     mode: str = "highprec",
+    dense_bias: Optional[torch.Tensor] = None,
 ):
     """Single-token decode through `ReferenceMHA` with a causal bias whose only query position is
     `lengths - 1` (decoding_test.py:131: `query_offset = seq_len - padding - 1`).
 
-    query [B,1,Hq,D]; key/value [B,S,Hkv,D] or page pools + page_tables; lengths [B] int.
+    query [B,1,Hq,D]; key/value [B,S,Hkv,D] or page pools + page_tables; lengths [B] int;
+    dense_bias [1|B, 1|Hq, 1, S]: an explicit bias summed with the causal one, as the composite bias
+    of a decode call sums its members (attention_bias.py:243-246; decoding_test.py:118-127 builds it).
     """
     b = query.shape[0]
     if page_tables is not None:
@@ -408,6 +411,7 @@ def reference_decode(
         sliding_window=sliding_window,
         target_positions=tp,
         source_positions=torch.arange(kv_len, dtype=torch.int64)[None],
+        dense_bias=dense_bias,
     )
     return reference_mha(
         query, key, value, spec, softmax_scale=softmax_scale, mode=mode, page_tables=page_tables

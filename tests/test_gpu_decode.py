@@ -521,3 +521,254 @@ def test_decode_edge_lengths_and_random_shapes():
         got = ops.paged_decode(q[:, 0].cuda(), kp.cuda(), vp.cuda(), tables.cuda(), lengths.cuda(),
                                softmax_scale=d ** -0.5, sliding_window=window)
         assert _ok(got.cpu(), want), (b, hkv, g, d, pps, window, ref.max_abs(got.cpu(), want))
+
+
+# ----------------------------------------------------------------------------- the reference's full decode contract
+
+
+def _bar(got, want, dtype):
+    """The bars of the three dtypes: fp32 1e-5 max-abs; bf16 1e-2 relative L2, float16 an eighth of it."""
+    if dtype == torch.float32:
+        return got.dtype == dtype and ref.max_abs(got, want) <= 1e-5
+    return got.dtype == dtype and ref.rel_l2(got, want) <= (1e-2 if dtype == torch.bfloat16 else 1.25e-3)
+
+
+def _repage(tables, pool, page_size):
+    """The same sequences laid out in pages of `page_size` tokens (a multiple of the 16 of `pool`): the
+    new pool's page p of sequence b holds the old logical pages [p * r, (p + 1) * r) of b, the new
+    table is a seeded permutation again.  Returns (new pool builder, new tables)."""
+    r = page_size // 16
+    b, pps = tables.shape
+    assert pps % r == 0
+    new_pps = pps // r
+    perm = torch.from_numpy(np.random.default_rng(11).permutation(b * new_pps).astype(np.int32)).reshape(b, new_pps)
+
+    def build(old):
+        hkv, _, _, d = old.shape
+        new = torch.empty((hkv, b * new_pps, page_size, d), dtype=old.dtype)
+        gathered = old[:, tables.long()]                        # [hkv, b, pps, 16, d]
+        new[:, perm.long().reshape(-1)] = gathered.reshape(hkv, b * new_pps, page_size, d)
+        return new
+
+    return build, perm
+
+
+@pytest.mark.parametrize("page_size", [32, 64, 128])
+@pytest.mark.parametrize("b,s,h,d", [(1, 1024, 32, 64), (4, 512, 48, 64), (2, 1024, 16, 128), (1, 4096, 8, 128)])
+@pytest.mark.parametrize("padding", [0, 111])
+@pytest.mark.parametrize("kv_head_factor", [1, 8])
+@pytest.mark.parametrize("window", [-1, 127])
+def test_paged_decode_page_sizes(page_size, b, s, h, d, padding, kv_head_factor, window):
+    """The page sizes the reference admits at its compute block of 128 keys besides 16
+    (gpu_paged_attention.py:313-321), on the grid of decoding_test.py:95-163: against the oracle, and -
+    with the fixed decomposition - bit for bit against the same tokens in 16-token pages and in a
+    contiguous cache (the kernels stream the same 16-token tiles in the same order)."""
+    hkv = h // kv_head_factor
+    q, kp, vp, tables, _ = ref.paged_inputs(3, batch=b, num_heads=h, num_kv_heads=hkv, head_dim=d, page_size=16,
+                                            pages_per_seq=s // 16, min_len=1, max_len=s)
+    build, tables2 = _repage(tables, kp, page_size)
+    kp2, vp2 = build(kp), build(vp)
+    assert torch.equal(ref.reconstruct_kv(tables2, kp2), ref.reconstruct_kv(tables, kp))
+    lengths = torch.full((b,), s - padding, dtype=torch.int32)
+    scale = d ** -0.5
+    want = ref.reference_decode(q, kp2, vp2, lengths, softmax_scale=scale, page_tables=tables2,
+                                sliding_window=None if window < 0 else window)[:, 0]
+    got = ops.paged_decode(q[:, 0].cuda(), kp2.cuda(), vp2.cuda(), tables2.cuda(), lengths.cuda(),
+                           softmax_scale=scale, sliding_window=window)
+    assert _ok(got.cpu(), want), ref.rel_l2(got.cpu(), want)
+    with _deterministic():
+        det = ops.paged_decode(q[:, 0].cuda(), kp2.cuda(), vp2.cuda(), tables2.cuda(), lengths.cuda(),
+                               softmax_scale=scale, sliding_window=window)
+        det16 = ops.paged_decode(q[:, 0].cuda(), kp.cuda(), vp.cuda(), tables.cuda(), lengths.cuda(),
+                                 softmax_scale=scale, sliding_window=window)
+    assert torch.equal(det, det16)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_paged_decode_page_sizes_ragged_poison_and_dispatch(dtype):
+    """Ragged lengths over 64-token pages: tokens past a sequence's length inside its last page, and
+    whole pages past it, are never read into the result (NaN poison); the dispatch accepts the pool."""
+    b, hq, hkv, d, page, pps = 5, 8, 2, 128, 64, 6
+    q, kp, vp, tables, lengths = ref.paged_inputs(19, batch=b, num_heads=hq, num_kv_heads=hkv, head_dim=d,
+                                                  page_size=page, pages_per_seq=pps, min_len=1, max_len=page * pps,
+                                                  dtype=dtype)
+    lengths[0], lengths[1], lengths[2] = 1, page, page + 1
+    want = ref.reference_decode(q, kp, vp, lengths, softmax_scale=0.1, page_tables=tables)
+    kpo, vpo = kp.clone(), vp.clone()
+    for bi in range(b):
+        n = int(lengths[bi])
+        for j in range(pps):
+            lo = max(0, n - j * page)
+            if lo < page:
+                kpo[:, int(tables[bi, j]), lo:] = float("nan")
+                vpo[:, int(tables[bi, j]), lo:] = float("nan")
+    tp = (lengths.long() - 1)[:, None].cuda()
+    bias = ab.CompositeAttentionBias([ab.CausalAttentionBias(target_positions=tp,
+                                                             source_positions=torch.arange(page * pps)[None].cuda())])
+    args = dict(query=q.cuda(), key=kpo.cuda(), value=vpo.cuda(), bias=bias)
+    impl = flash_attention_implementation("gpu", **args, softmax_scale=0.1, kv_cache_type=PagedKVCache,
+                                          page_tables=tables.cuda())
+    assert impl is not None and isinstance(impl.fn, HipPagedAttention)
+    got = impl.fn(dict(**args, page_tables=tables.cuda()))
+    assert torch.isfinite(got.float()).all() and _bar(got.cpu(), want, dtype)
+    # the reference's gate: fewer than 16 pages per compute block, the block a multiple of the page
+    small = HipPagedAttention.default_config().set(softmax_scale=0.1, gpu_block_size=32).instantiate()
+    assert not small.is_supported(dict(**args, page_tables=tables.cuda()), kv_cache_type=PagedKVCache)  # 32 % 64
+
+
+@pytest.mark.parametrize("g,hkv", [(24, 2), (32, 1), (64, 1), (17, 3)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_decode_more_than_16_query_heads_per_kv_head(g, hkv, dtype):
+    """gpu_decoding.py:341 pads its head block to the next power of two, so MQA with 32 or 64 query
+    heads runs there; here a kv head's query heads are served in groups of 16."""
+    b, d, pps = 3, 128, 24
+    hq = g * hkv
+    q, kp, vp, tables, lengths = ref.paged_inputs(23, batch=b, num_heads=hq, num_kv_heads=hkv, head_dim=d,
+                                                  page_size=16, pages_per_seq=pps, min_len=1, max_len=16 * pps,
+                                                  dtype=dtype)
+    want = ref.reference_decode(q, kp, vp, lengths, softmax_scale=0.09, page_tables=tables)[:, 0]
+    got = ops.paged_decode(q[:, 0].cuda(), kp.cuda(), vp.cuda(), tables.cuda(), lengths.cuda(), softmax_scale=0.09)
+    assert _bar(got.cpu(), want, dtype), ref.rel_l2(got.cpu(), want)
+    kk, vv = ref.reconstruct_kv(tables, kp).cuda(), ref.reconstruct_kv(tables, vp).cuda()
+    got2 = ops.decode(q[:, 0].cuda(), kk, vv, lengths.cuda(), softmax_scale=0.09, sliding_window=-1)
+    assert _bar(got2.cpu(), want, dtype)
+    # a group's result does not depend on the other groups: heads [16, 2 * 16) alone, as their own call
+    if g >= 32 and hkv == 1:
+        sub = ops.paged_decode(q[:, 0, 16:32].contiguous().cuda(), kp.cuda(), vp.cuda(), tables.cuda(), lengths.cuda(),
+                               softmax_scale=0.09, deterministic=True)
+        full = ops.paged_decode(q[:, 0].cuda(), kp.cuda(), vp.cuda(), tables.cuda(), lengths.cuda(),
+                                softmax_scale=0.09, deterministic=True)
+        assert torch.equal(sub, full[:, 16:32])
+
+
+@pytest.mark.parametrize("d", [8, 40, 72, 80, 96, 120])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_decode_head_dims_between_the_compiled_widths(d, dtype):
+    """Any head_dim that is a multiple of 8 up to 128, on the tensors as they are (no padded copies):
+    paged pool rows and contiguous cache rows of d elements."""
+    b, hq, hkv, pps = 4, 8, 2, 20
+    q, kp, vp, tables, lengths = ref.paged_inputs(29, batch=b, num_heads=hq, num_kv_heads=hkv, head_dim=d,
+                                                  page_size=16, pages_per_seq=pps, min_len=1, max_len=16 * pps,
+                                                  dtype=dtype)
+    scale = d ** -0.5
+    for window in (-1, 33):
+        want = ref.reference_decode(q, kp, vp, lengths, softmax_scale=scale, page_tables=tables,
+                                    sliding_window=None if window < 0 else window)[:, 0]
+        got = ops.paged_decode(q[:, 0].cuda(), kp.cuda(), vp.cuda(), tables.cuda(), lengths.cuda(),
+                               softmax_scale=scale, sliding_window=window)
+        assert got.shape == (b, hq, d) and _bar(got.cpu(), want, dtype), (window, ref.rel_l2(got.cpu(), want))
+        kk, vv = ref.reconstruct_kv(tables, kp).cuda(), ref.reconstruct_kv(tables, vp).cuda()
+        got2 = ops.decode(q[:, 0].cuda(), kk, vv, lengths.cuda(), softmax_scale=scale, sliding_window=window)
+        assert _bar(got2.cpu(), want, dtype), window
+    # NaNs in the columns of a wider tensor that the call does not cover never reach the result
+    wide = torch.full((b, 16 * pps, hkv, d + 8), float("nan"), dtype=dtype)
+    wide[..., :d] = ref.reconstruct_kv(tables, kp)
+    wide_v = torch.full_like(wide, float("nan"))
+    wide_v[..., :d] = ref.reconstruct_kv(tables, vp)
+    got3 = ops.decode(q[:, 0].cuda(), wide.cuda()[..., :d], wide_v.cuda()[..., :d], lengths.cuda(),
+                      softmax_scale=scale, sliding_window=33)
+    assert _bar(got3.cpu(), want, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("bias_shape", ["bh", "1h", "b1"])
+@pytest.mark.parametrize("bias_dtype", [torch.float32, torch.bfloat16])
+def test_decode_with_an_explicit_bias(dtype, bias_shape, bias_dtype):
+    """An explicit bias [B|1, Hq|1, 1, S] beside the causal mask (gpu_decoding.py:327-336,
+    gpu_paged_attention.py:346-348), kernel level and through both dispatch classes."""
+    b, hq, hkv, d, pps = 3, 8, 2, 128, 18
+    s = 16 * pps
+    q, kp, vp, tables, lengths = ref.paged_inputs(31, batch=b, num_heads=hq, num_kv_heads=hkv, head_dim=d,
+                                                  page_size=16, pages_per_seq=pps, min_len=1, max_len=s, dtype=dtype)
+    lengths[0] = s - 5  # a last tile that straddles the length
+    shape = dict(bh=(b, hq, 1, s), **{"1h": (1, hq, 1, s), "b1": (b, 1, 1, s)})[bias_shape]
+    dense = (2.0 * ref.normal_tensor(37, shape, torch.float32)).to(bias_dtype)
+    want = ref.reference_decode(q, kp, vp, lengths, softmax_scale=0.1, page_tables=tables, dense_bias=dense.float())
+    plain = ref.reference_decode(q, kp, vp, lengths, softmax_scale=0.1, page_tables=tables)
+    assert ref.rel_l2(plain, want) > 0.1  # the bias matters
+    got = ops.paged_decode(q[:, 0].cuda(), kp.cuda(), vp.cuda(), tables.cuda(), lengths.cuda(), softmax_scale=0.1,
+                           bias=dense[:, :, 0].cuda())
+    assert _bar(got.cpu(), want[:, 0], dtype), ref.rel_l2(got.cpu(), want[:, 0])
+    kk, vv = ref.reconstruct_kv(tables, kp).cuda(), ref.reconstruct_kv(tables, vp).cuda()
+    got2 = ops.decode(q[:, 0].cuda(), kk, vv, lengths.cuda(), softmax_scale=0.1, bias=dense[:, :, 0].cuda())
+    assert _bar(got2.cpu(), want[:, 0], dtype)
+    # through the dispatch
+    tp = (lengths.long() - 1)[:, None].cuda()
+    bias = ab.CompositeAttentionBias([
+        ab.CausalAttentionBias(target_positions=tp, source_positions=torch.arange(s)[None].cuda()),
+        ab.TensorAttentionBias(dense.cuda()),
+    ])
+    impl = flash_attention_implementation("gpu", query=q.cuda(), key=kk, value=vv, bias=bias, softmax_scale=0.1,
+                                          kv_cache_type=KVCache)
+    assert impl is not None and isinstance(impl.fn, HipDecoding)
+    assert _bar(impl.fn(dict(query=q.cuda(), key=kk, value=vv, bias=bias)).cpu(), want, dtype)
+    pargs = dict(query=q.cuda(), key=kp.cuda(), value=vp.cuda(), bias=bias)
+    impl = flash_attention_implementation("gpu", **pargs, softmax_scale=0.1, kv_cache_type=PagedKVCache,
+                                          page_tables=tables.cuda())
+    assert impl is not None and isinstance(impl.fn, HipPagedAttention)
+    assert _bar(impl.fn(dict(**pargs, page_tables=tables.cuda())).cpu(), want, dtype)
+
+
+def test_decode_with_an_arbitrary_mask_fn():
+    """Any mask fn, not only the causal and sliding-window ones (gpu_decoding.py:110,
+    gpu_paged_attention.py:108: `mask_fn(kv_len - 1, indices)`): here a strided causal mask."""
+    b, hq, hkv, d, pps = 4, 8, 4, 64, 16
+    s = 16 * pps
+    q, kp, vp, tables, lengths = ref.paged_inputs(41, batch=b, num_heads=hq, num_kv_heads=hkv, head_dim=d,
+                                                  page_size=16, pages_per_seq=pps, min_len=8, max_len=s)
+    strided = lambda qp, kp_: (qp >= kp_) & ((qp - kp_) % 3 != 1)
+    qpos = (lengths.long() - 1)[:, None]
+    keep = strided(qpos, torch.arange(s)[None])                       # [B, S]
+    dense = ref.bool_to_bias(keep)[:, None, None, :]                  # [B, 1, 1, S]
+    want = ref.reference_decode(q, kp, vp, lengths, softmax_scale=0.2, page_tables=tables, dense_bias=dense)
+    tp = qpos.cuda()
+    bias = ab.CompositeAttentionBias([ab.MaskFnAttentionBias(strided, target_positions=tp,
+                                                             source_positions=torch.arange(s)[None].cuda())])
+    kk, vv = ref.reconstruct_kv(tables, kp).cuda(), ref.reconstruct_kv(tables, vp).cuda()
+    impl = flash_attention_implementation("gpu", query=q.cuda(), key=kk, value=vv, bias=bias, softmax_scale=0.2,
+                                          kv_cache_type=KVCache)
+    assert impl is not None and isinstance(impl.fn, HipDecoding)
+    got = impl.fn(dict(query=q.cuda(), key=kk, value=vv, bias=bias))
+    assert _ok(got.cpu(), want), ref.rel_l2(got.cpu(), want)
+    pargs = dict(query=q.cuda(), key=kp.cuda(), value=vp.cuda(), bias=bias)
+    impl = flash_attention_implementation("gpu", **pargs, softmax_scale=0.2, kv_cache_type=PagedKVCache,
+                                          page_tables=tables.cuda())
+    assert impl is not None and isinstance(impl.fn, HipPagedAttention)
+    assert _ok(impl.fn(dict(**pargs, page_tables=tables.cuda())).cpu(), want)
+    # masking is exact: poison in every key the mask drops changes nothing (fixed decomposition)
+    kpo, vpo = ref.reconstruct_kv(tables, kp).clone(), ref.reconstruct_kv(tables, vp).clone()
+    for bi in range(b):
+        kpo[bi, ~keep[bi]] = 1e4
+        vpo[bi, ~keep[bi]] = -1e4
+    with _deterministic():
+        a = impl_decode = HipDecoding.default_config().set(softmax_scale=0.2).instantiate()
+        base = a(dict(query=q.cuda(), key=kk, value=vv, bias=bias))
+        poisoned = impl_decode(dict(query=q.cuda(), key=kpo.cuda(), value=vpo.cuda(), bias=bias))
+    assert torch.equal(base, poisoned)
+
+
+@pytest.mark.parametrize("q_dtype,kv_dtype", [(torch.bfloat16, torch.float32), (torch.float32, torch.bfloat16),
+                                              (torch.bfloat16, torch.float16)])
+def test_decode_kv_dtype_other_than_the_query_dtype(q_dtype, kv_dtype):
+    """K/V are cast to the query's dtype (gpu_decoding.py:115,133), so a cache kept in another precision
+    is accepted; the result is that of the cast tensors."""
+    b, hq, hkv, d, pps = 3, 8, 2, 128, 10
+    s = 16 * pps
+    q, kp, vp, tables, lengths = ref.paged_inputs(43, batch=b, num_heads=hq, num_kv_heads=hkv, head_dim=d,
+                                                  page_size=16, pages_per_seq=pps, min_len=1, max_len=s, dtype=kv_dtype)
+    q = q.to(q_dtype)
+    want = ref.reference_decode(q, kp.to(q_dtype), vp.to(q_dtype), lengths, softmax_scale=0.1, page_tables=tables)
+    tp = (lengths.long() - 1)[:, None].cuda()
+    bias = ab.CompositeAttentionBias([ab.CausalAttentionBias(target_positions=tp,
+                                                             source_positions=torch.arange(s)[None].cuda())])
+    pargs = dict(query=q.cuda(), key=kp.cuda(), value=vp.cuda(), bias=bias)
+    impl = flash_attention_implementation("gpu", **pargs, softmax_scale=0.1, kv_cache_type=PagedKVCache,
+                                          page_tables=tables.cuda())
+    assert impl is not None and isinstance(impl.fn, HipPagedAttention)
+    got = impl.fn(dict(**pargs, page_tables=tables.cuda()))
+    assert _bar(got.cpu(), want, q_dtype)
+    kk, vv = ref.reconstruct_kv(tables, kp).cuda(), ref.reconstruct_kv(tables, vp).cuda()
+    impl = flash_attention_implementation("gpu", query=q.cuda(), key=kk, value=vv, bias=bias, softmax_scale=0.1,
+                                          kv_cache_type=KVCache)
+    assert impl is not None and isinstance(impl.fn, HipDecoding)
+    assert _bar(impl.fn(dict(query=q.cuda(), key=kk, value=vv, bias=bias)).cpu(), want, q_dtype)

@@ -290,8 +290,8 @@ def test_library_exports_every_declared_symbol():
 def test_struct_layouts_match_header():
     """Field order of the ctypes mirrors equals the order in the header."""
     text = open(os.path.join(ROOT, "include", "axl_attn.h")).read()
-    for cls in (_lib.AxlAttnAux, _lib.AxlFlashFwdParams, _lib.AxlFlashBwdParams, _lib.AxlPagedDecodeParams,
-                _lib.AxlDecodeParams, _lib.AxlPageInsertParams):
+    for cls in (_lib.AxlAttnAux, _lib.AxlFlashFwdParams, _lib.AxlFlashBwdParams, _lib.AxlDecodeBias,
+                _lib.AxlPagedDecodeParams, _lib.AxlDecodeParams, _lib.AxlPageInsertParams):
         body = re.search(r"typedef struct %s \{(.*?)\} %s;" % (cls.__name__, cls.__name__), text, flags=re.S).group(1)
         body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
         names = []
@@ -377,15 +377,35 @@ def test_abi_validation_without_gpu():
     assert lib.axl_flash_bwd_phases(ctypes.byref(bp), 0, None) == _lib.AXL_ERR_INVALID_ARGUMENT
     # Paged decode geometry.
     dp = _lib.AxlPagedDecodeParams(q=256, k_pages=256, v_pages=256, page_tables=256, lengths=256, out=256, batch=2,
-                                   num_q_heads=8, num_kv_heads=2, head_dim=128, num_pages=64, page_size=32,
+                                   num_q_heads=8, num_kv_heads=2, head_dim=128, num_pages=64, page_size=48,
                                    pages_per_seq=32, dtype=0, sliding_window=-1, softmax_scale=1.0, workspace=None,
                                    workspace_bytes=0)
-    assert lib.axl_paged_decode(ctypes.byref(dp), None) == _lib.AXL_ERR_UNSUPPORTED  # page size 32
+    assert lib.axl_paged_decode(ctypes.byref(dp), None) == _lib.AXL_ERR_UNSUPPORTED  # 48 is not 16 * 2^k
+    dp.page_size = 8
+    assert lib.axl_paged_decode(ctypes.byref(dp), None) == _lib.AXL_ERR_UNSUPPORTED
+    sizes = {}
+    for page in (16, 32, 64, 128):  # what gpu_paged_attention.py:313-321 admits at its block of 128
+        dp.page_size = page
+        assert lib.axl_paged_decode(ctypes.byref(dp), None) == _lib.AXL_ERR_WORKSPACE
+        sizes[page] = lib.axl_paged_decode_workspace_bytes(ctypes.byref(dp))
+        assert sizes[page] > 0
+    assert sizes[16] < sizes[32] < sizes[64]  # the split-K records follow the context the table can address
     dp.page_size = 16
+    base = sizes[16]
+    dp.num_q_heads = 64  # 32 query heads per kv head: two groups of 16, each with records of its own
     assert lib.axl_paged_decode(ctypes.byref(dp), None) == _lib.AXL_ERR_WORKSPACE
-    assert lib.axl_paged_decode_workspace_bytes(ctypes.byref(dp)) > 0
-    dp.num_q_heads = 64
-    assert lib.axl_paged_decode(ctypes.byref(dp), None) == _lib.AXL_ERR_UNSUPPORTED  # 32 heads per kv head
+    assert lib.axl_paged_decode_workspace_bytes(ctypes.byref(dp)) > 2 * base
+    dp.num_q_heads = 8
+    dp.head_dim = 80   # between the compiled widths: served at 128
+    assert lib.axl_paged_decode_workspace_bytes(ctypes.byref(dp)) == base
+    dp.head_dim = 76   # not a multiple of 8
+    assert lib.axl_paged_decode(ctypes.byref(dp), None) == _lib.AXL_ERR_UNSUPPORTED
+    dp.head_dim = 128
+    dp.bias = _lib.AxlDecodeBias(bias=256, batch_stride=0, head_stride=0, dtype=_lib.AXL_F16)
+    assert lib.axl_paged_decode(ctypes.byref(dp), None) == _lib.AXL_ERR_UNSUPPORTED  # bias must be bf16 / fp32
+    dp.bias.dtype = _lib.AXL_F32
+    assert lib.axl_paged_decode_workspace_bytes(ctypes.byref(dp)) > base  # records padded to 16 head columns
+    assert lib.axl_paged_decode(ctypes.byref(dp), None) == _lib.AXL_ERR_WORKSPACE
 
 
 def test_ops_reject_mismatched_shapes_before_any_launch():
