@@ -6,7 +6,7 @@ The headline workload (BASELINE.json configs[1], "C2") is causal GQA flash atten
 backward, bf16, batch 4, 32 query heads / 8 kv heads, seq 4096, head_dim 128: a step is one forward
 plus one backward over one synthetic batch already resident in HBM, obtained the way a caller of the
 library obtains them: `flash_attention_implementation("gpu", ...)` with the default configuration, the
-returned kernel object applied to the batch, autograd's backward with a given dO (`c_abi_ms_per_step`
+returned kernel object applied to the batch, `torch.autograd.grad` with a given dO (`c_abi_ms_per_step`
 in the same object is the same pair of C-ABI calls with buffers allocated once).  The default
 configuration keeps dS in the backward's workspace when that workspace fits a sixteenth of the
 device's memory (C2: 2.15 GB, C3: 8.7 GB) and recomputes dS in the dQ kernel when it does not (C5:
@@ -196,11 +196,12 @@ def bench_flash(cfg, steps, warmup, cpu_baseline):
     batch = dict(query=q, key=k, value=v, bias=bias)
 
     def step():
-        q.grad = k.grad = v.grad = None
-        impl.fn(batch).backward(do)
+        # gradients handed back to the caller, as they are to the layer below attention in a model (a
+        # .backward() into leaf tensors would add a copy of every gradient: autograd clones what it
+        # accumulates into a leaf)
+        torch.autograd.grad(impl.fn(batch), (q, k, v), do)
 
     ms_step = _time_region(step, steps, warmup)
-    q.grad = k.grad = v.grad = None
     # The same kernels through the C ABI with buffers allocated once (no allocator, no autograd).
     qd, kd, vd = q.detach(), k.detach(), v.detach()
     kw = dict(softmax_scale=D ** -0.5, mask_kind=mask_kind, sliding_window=cfg["window"], segment_ids=seg)
@@ -231,7 +232,7 @@ def bench_flash(cfg, steps, warmup, cpu_baseline):
     traffic, traffic_src = _traffic(cfg["name"] + ("" if spill else "_recompute"))
     result = dict(
         workload=cfg["label"], value=tf(fl_fwd + fl_bwd, ms_step), unit="TFLOP/s", ms_per_step=ms_step,
-        entry="flash_attention_implementation('gpu', ...).fn(batch) + autograd backward",
+        entry="flash_attention_implementation('gpu', ...).fn(batch) + torch.autograd.grad(out, (q, k, v), dO)",
         backward="dS workspace: delta, dK/dV (stores dS), dq = dS k" if spill else "dQ (recomputes dS, computes delta), dK/dV",
         backward_chosen_by=chosen, ds_workspace_bytes=ws_need if spill else 0,
         c_abi_ms_per_step=ms_abi,
