@@ -621,6 +621,11 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
     // well; 40 leaves a margin.)
     wait_vmem_le<2 * NLD + (AUX ? 40 : 0)>();
     __syncthreads();
+    // The stage-A chains of the last slots were issued through inline assembly, so the compiler places
+    // no wait states behind them; where a run of iterations ends it may move values into their
+    // registers a few instructions after this barrier.  Eight wait states here bring every such write
+    // to at least the 12 the hardware wants after the last MFMA of a chain, whatever the barrier took.
+    if constexpr (!AUX) asm volatile("s_nop 7");
     char* const tmp = buf_b;
     buf_b = buf_e;
     buf_e = buf_a;

@@ -362,6 +362,19 @@ def bench_paged_decode(steps, warmup, cpu_baseline):
     fn_reused = lambda: ops.paged_decode(q, kp, vp, tables, lengths, softmax_scale=scale, workspace=ws, out=out,
                                          workspace_reused=True)
     ms_reused = _time_region(fn_reused, steps, 2)
+    # The fixed work decomposition (AXL_DECODE_DETERMINISTIC: bit-reproducible results).
+    fn_det = lambda: ops.paged_decode(q, kp, vp, tables, lengths, softmax_scale=scale, workspace=ws, out=out,
+                                      deterministic=True)
+    ms_det = _time_region(fn_det, steps, 2)
+    # The same sequences in 64-token pages (one of the page sizes the reference admits besides 16): the
+    # pools are re-viewed, so every 64-token page is four of the old ones that happen to be adjacent, and
+    # the table is a permutation of those.
+    kp64, vp64 = kp.view(Hkv, P // 4, 64, D), vp.view(Hkv, P // 4, 64, D)
+    tables64 = torch.from_numpy(np.random.default_rng(6).permutation(P // 4).astype(np.int32)).reshape(B, pps // 4).to(dev)
+    fn64 = lambda: ops.paged_decode(q, kp64, vp64, tables64, lengths, softmax_scale=scale, workspace=ws, out=out)
+    ms64 = _time_region(fn64, steps, 2)
+    live64 = int(((lengths_cpu.long() + 63) // 64).sum())
+    bytes64 = live64 * 64 * Hkv * D * 2 * 2 + live64 * 4 + 2 * B * Hq * D * 2
     live_pages = int(((lengths_cpu.long() + page - 1) // page).sum())
     # Algorithmic bytes: every live K and V page once, its page-table entry, q and out.
     algo_bytes = live_pages * page * Hkv * D * 2 * 2 + live_pages * 4 + 2 * B * Hq * D * 2
@@ -371,6 +384,9 @@ def bench_paged_decode(steps, warmup, cpu_baseline):
         workload="C4: paged decode, bf16, B64 Hq32/Hkv8 D128, page 16, ctx U[512,32768]",
         value=gbs, unit="GB/s", ms_per_step=ms, algorithmic_gb=algo_bytes / 1e9,
         workspace_reused=dict(ms_per_step=ms_reused, value=algo_bytes / (ms_reused * 1e-3) / 1e9, unit="GB/s"),
+        deterministic=dict(ms_per_step=ms_det, value=algo_bytes / (ms_det * 1e-3) / 1e9, unit="GB/s"),
+        page_size_64=dict(ms_per_step=ms64, value=bytes64 / (ms64 * 1e-3) / 1e9, unit="GB/s",
+                          algorithmic_gb=bytes64 / 1e9),
         roofline=dict(kernel="decode_split_kernel", bound="hbm", achieved=gbs, peak=HBM_PEAK_GBS, unit="GB/s",
                       frac=gbs / HBM_PEAK_GBS, traffic=traffic, traffic_source=traffic_src),
     )

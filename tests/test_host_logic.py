@@ -523,27 +523,52 @@ def test_layer_falls_back_when_no_kernel_supports_the_request():
         layer.compute_attention(q_proj=q, k_proj=k, v_proj=k, attention_logit_biases=bias)
 
 
-def test_dkdv_kernel_keeps_its_vector_register_accumulators_in_place():
-    """The plain dK/dV instantiations accumulate S and dP in vector registers through inline-assembly
-    MFMAs, whose hazards the compiler does not see: their correctness rests on the compiler not copying
-    those registers right after a chain.  It has no reason to while nothing spills, so a build whose
-    plain instantiations use AGPRs for anything but the dK / dV accumulators (head_dim of them), or
-    scratch memory, fails here rather than on the GPU."""
-    import re
+def _device_asm(source, extra=()):
+    """(assembly text, compiler remarks) of one kernel file, compiled as the Makefile compiles it."""
     import shutil
     import subprocess
+    import tempfile
 
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(hipcc):
         pytest.skip("hipcc not available")
     csrc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "axlearn_amd", "csrc")
-    cmd = [hipcc, "-O3", "-std=c++17", "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang",
-           "-packed-fp32-ops", "-Wno-unused-value", "-Wno-unknown-attributes", "--cuda-device-only", "-S",
-           "-Rpass-analysis=kernel-resource-usage", "-o", os.devnull, os.path.join(csrc, "flash_bwd_dkdv.hip")]
-    out = subprocess.run(cmd, capture_output=True, text=True, cwd=csrc, timeout=600)
-    assert out.returncode == 0, out.stderr[-2000:]
+    with tempfile.TemporaryDirectory() as tmp:
+        out_s = os.path.join(tmp, "kernel.s")
+        cmd = [hipcc, "-O3", "-std=c++17", "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang",
+               "-packed-fp32-ops", "-Wno-unused-value", "-Wno-unknown-attributes", "--cuda-device-only", "-S",
+               "-Rpass-analysis=kernel-resource-usage", *extra, "-o", out_s, os.path.join(csrc, source)]
+        out = subprocess.run(cmd, capture_output=True, text=True, cwd=csrc, timeout=900)
+        assert out.returncode == 0, out.stderr[-2000:]
+        return open(out_s).read(), out.stderr
+
+
+def _assert_asm_mfma_distances(asm, pattern, want_kernels):
+    """Every inline-assembly MFMA chain of the kernels whose name matches `pattern`: 12 wait states
+    or two further MFMAs before anything else touches its registers, on every path."""
+    import isa_hazards  # tests/isa_hazards.py (pytest puts the test directory on sys.path)
+
+    checked = 0
+    for name, lines in isa_hazards.split_functions(asm).items():
+        if not re.match(pattern, name):
+            continue
+        chains = sum(1 for l in lines if l.startswith("@v_mfma_"))
+        bad = isa_hazards.check_function(lines)
+        assert not bad, f"{name}: {len(bad)} hazards, first {bad[0]}"
+        checked += chains > 0
+    assert checked == want_kernels, checked
+
+
+def test_dkdv_kernel_keeps_its_vector_register_accumulators_in_place():
+    """The plain dK/dV instantiations accumulate S and dP in vector registers through inline-assembly
+    MFMAs, whose hazards the compiler does not see.  Two checks on what the compiler produced: nothing
+    spills (a build whose plain instantiations use AGPRs for anything but the dK / dV accumulators,
+    head_dim of them, or scratch memory, has started copying registers around), and on every path
+    through every such kernel the first instruction that touches a chain's registers comes 12 wait
+    states or two MFMAs after the chain's last MFMA."""
+    asm, remarks = _device_asm("flash_bwd_dkdv.hip")
     seen = 0
-    for block in out.stderr.split("Function Name: ")[1:]:
+    for block in remarks.split("Function Name: ")[1:]:
         name = block.split()[0]
         m = re.match(r"_ZN3axl21flash_bwd_dkdv_kernelINS_\d+Elem\w+ELi(\d+)ELb([01])ELi(\d+)ELb([01])EEE", name)
         if not m or m.group(3) != "0":  # other kernels; bias / dropout instantiations use the compiler's own form
@@ -554,3 +579,14 @@ def test_dkdv_kernel_keeps_its_vector_register_accumulators_in_place():
         assert scratch == 0, f"{name}: scratch {scratch}"
         seen += 1
     assert seen == 16  # {bf16, f16} x {64, 128} x {plain, segment ids} x {recomputing, dS workspace}
+    _assert_asm_mfma_distances(asm, r"_ZN3axl21flash_bwd_dkdv_kernel", 16)
+
+
+def test_forward_kernel_keeps_the_distance_behind_its_assembly_mfma_chains():
+    """The same for the forward's interior tiles, whose S^T chains of the next tile are inline-assembly
+    MFMAs read by the softmax of the next step: the hazard distance on every path of the four
+    instantiations that have such tiles ({bf16, f16} x {64, 128}, no bias / dropout).  (Any register
+    the compiler spilled or copied right behind a chain would show up here as the first instruction
+    that touches it.)"""
+    asm, _ = _device_asm("flash_fwd.hip", extra=("-mllvm", "-amdgpu-mfma-vgpr-form"))
+    _assert_asm_mfma_distances(asm, r"_ZN3axl16flash_fwd_kernel", 4)
