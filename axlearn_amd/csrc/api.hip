@@ -3,6 +3,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cmath>
+#include <initializer_list>
 #include <mutex>
 #include <unordered_map>
 
@@ -83,11 +84,27 @@ static int check_flash_shapes(const char* who, int batch, int q_len, int kv_len,
   if (seg && q_len != kv_len)
     return set_error(AXL_ERR_INVALID_ARGUMENT,
                      "%s: segment_ids need q_len == kv_len (got %d vs %d)", who, q_len, kv_len);
-  if (d != 64 && d != 128)
-    return set_error(AXL_ERR_UNSUPPORTED, "%s: head_dim %d (supported: 64, 128)", who, d);
+  if (dtype == AXL_F32 ? (d != 64 && d != 128) : (d > 128 || d % 8 != 0))
+    return set_error(AXL_ERR_UNSUPPORTED, "%s: head_dim %d (supported: 64 and 128; in bf16 / f16 any multiple of 8 up to 128)",
+                     who, d);
   if (q_len % 128 != 0 || kv_len % 128 != 0)
     return set_error(AXL_ERR_UNSUPPORTED, "%s: q_len %d / kv_len %d not divisible by 128", who,
                      q_len, kv_len);
+  return AXL_OK;
+}
+
+// A head_dim between the compiled widths (16-bit kernels): the kernels run at the next width on the
+// tensors as they are.  Their tile loads address a second 1 KB group of rows relative to the first,
+// which needs rows at least as far apart as the compiled width, and the bias / dropout instantiations
+// have no such form.
+static int check_odd_head_dim(const char* who, int d, bool aux, std::initializer_list<const AxlStrides*> tensors) {
+  if (d == 64 || d == 128) return AXL_OK;
+  if (aux)
+    return set_error(AXL_ERR_UNSUPPORTED, "%s: head_dim %d with a bias or dropout mask (supported: 64, 128)", who, d);
+  const int width = d <= 64 ? 64 : 128;
+  for (const AxlStrides* s : tensors)
+    if (s->seq < width)
+      return set_error(AXL_ERR_UNSUPPORTED, "%s: head_dim %d needs rows at least %d elements apart", who, d, width);
   return AXL_OK;
 }
 
@@ -186,6 +203,9 @@ int axl_flash_fwd(const AxlFlashFwdParams* p, void* stream) {
     return set_error(AXL_ERR_UNSUPPORTED, "axl_flash_fwd: segment_ids must be 16-byte aligned");
   rc = check_aux("axl_flash_fwd", p->aux, p->batch, p->num_q_heads, p->q_len, p->kv_len);
   if (rc != AXL_OK) return rc;
+  rc = check_odd_head_dim("axl_flash_fwd", p->head_dim, p->aux.bias || p->aux.dropout_mask,
+                          {&p->q_strides, &p->k_strides, &p->v_strides, &p->out_strides});
+  if (rc != AXL_OK) return rc;
   return launch_flash_fwd(*p, (hipStream_t)stream);
 }
 
@@ -222,6 +242,10 @@ int axl_flash_bwd_phases(const AxlFlashBwdParams* p, int phases, void* stream) {
   if (p->segment_ids && !aligned16(p->segment_ids))
     return set_error(AXL_ERR_UNSUPPORTED, "axl_flash_bwd: segment_ids must be 16-byte aligned");
   rc = check_aux("axl_flash_bwd", p->aux, p->batch, p->num_q_heads, p->q_len, p->kv_len);
+  if (rc != AXL_OK) return rc;
+  rc = check_odd_head_dim("axl_flash_bwd", p->head_dim, p->aux.bias || p->aux.dropout_mask,
+                          {&p->q_strides, &p->k_strides, &p->v_strides, &p->out_strides, &p->d_out_strides,
+                           &p->dq_strides, &p->dk_strides, &p->dv_strides});
   if (rc != AXL_OK) return rc;
   const size_t need = flash_bwd_workspace_bytes(*p);
   if (!p->workspace || p->workspace_bytes < need || !aligned16(p->workspace))

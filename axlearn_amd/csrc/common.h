@@ -484,6 +484,13 @@ __device__ __forceinline__ void for_each_index(F&& f) {
   for_each_index_impl(f, std::make_integer_sequence<int, N>{});
 }
 
+// Eight consecutive 16-bit elements of a row, or zeros where the row (of d_real elements, a multiple
+// of 8) has already ended: the operand fragments of a head_dim below the compiled width.
+__device__ __forceinline__ bf16x8 load8_within(const __bf16* row, int col, int d_real) {
+  const bf16x8 zero8 = {};
+  return col < d_real ? *(const bf16x8*)(row + col) : zero8;
+}
+
 struct Strides3 {
   int64_t b, s, h;
 };

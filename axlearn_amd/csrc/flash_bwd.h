@@ -26,6 +26,10 @@ struct BwdArgs {
   int B, T, S, Hq, Hkv;
   int mask_kind, window, q_off;
   float scale;
+  int d_real;   // head_dim of the tensors: a multiple of 8, at most the compiled width (16-bit kernels without
+                // bias / dropout mask).  Operand fragments are zero past it, tile loads fetch slice 0 of the row in
+                // place of the slices past it (finite values that only ever meet those zeros or end up in
+                // output columns that are not stored), stores leave the columns past it out.
   AuxArgs aux;  // dense bias / dropout mask (read only by the AUX instantiations)
 };
 

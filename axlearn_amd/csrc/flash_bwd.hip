@@ -45,7 +45,7 @@ __global__ __launch_bounds__(256) void bwd_delta_kernel(const BwdArgs a) {
 #pragma unroll
     for (int s = 0; s < (STEPS > 0 ? STEPS : 1); s++) {
       const int off = (s * 16 + sub) * VEC;
-      if (off < D) {
+      if (off < a.d_real) {
         union { uint4 u; T e[VEC]; } x, y;
         x.u = *(const uint4*)(o + off);
         y.u = *(const uint4*)(d + off);
@@ -403,7 +403,7 @@ static bool spill_eligible(const AxlFlashBwdParams& p) {
          (p.mask_kind == AXL_MASK_CAUSAL || p.mask_kind == AXL_MASK_SLIDING_WINDOW) && p.q_pos_offset == 0 &&
          p.q_len == p.kv_len && !p.aux.bias && !p.aux.dropout_mask && (p.flags & AXL_BWD_DS_WORKSPACE) &&
          // the ranged kernel keeps the table in LDS beside its ring: 256-row blocks at head_dim 128
-         (!spill_ranged(p) || (p.kv_len / 128 <= kMaxKbRanged && (p.head_dim != 128 || p.q_len % 256 == 0)));
+         (!spill_ranged(p) || (p.kv_len / 128 <= kMaxKbRanged && (p.head_dim <= 64 || p.q_len % 256 == 0)));
 }
 
 static size_t spill_bytes(const AxlFlashBwdParams& p) {
@@ -449,6 +449,8 @@ int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream)
   a.B = p.batch; a.T = p.q_len; a.S = p.kv_len; a.Hq = p.num_q_heads; a.Hkv = p.num_kv_heads;
   a.mask_kind = p.mask_kind; a.window = p.sliding_window; a.q_off = p.q_pos_offset;
   a.scale = p.softmax_scale;
+  a.d_real = p.head_dim;
+  const int width = p.head_dim <= 64 ? 64 : 128;   // the compiled width that serves this head_dim
   a.aux = make_aux_args(p.aux, p.softmax_scale);
   const bool aux = p.aux.bias || p.aux.dropout_mask;
   hipError_t err = hipSuccess;
@@ -477,23 +479,23 @@ int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream)
   }
   if (dt == AXL_F32) {
     if (phases & AXL_BWD_DELTA) {
-      if (p.head_dim == 128) AXL_LAUNCH((bwd_delta_kernel<float, 128>), delta_grid, 0);
+      if (width == 128) AXL_LAUNCH((bwd_delta_kernel<float, 128>), delta_grid, 0);
       else AXL_LAUNCH((bwd_delta_kernel<float, 64>), delta_grid, 0);
     }
-    if (err == hipSuccess) err = launch_bwd_f32(a, p.head_dim, phases, stream);
+    if (err == hipSuccess) err = launch_bwd_f32(a, width, phases, stream);
   } else if (spill) {
     // delta, then the dK/dV kernel (which leaves dS behind), then dq = scale * dS k.
     if (phases & AXL_BWD_DELTA) {
       if (dt == AXL_BF16) {
-        if (p.head_dim == 128) AXL_LAUNCH((bwd_delta_kernel<__bf16, 128>), delta_grid, 0);
+        if (width == 128) AXL_LAUNCH((bwd_delta_kernel<__bf16, 128>), delta_grid, 0);
         else AXL_LAUNCH((bwd_delta_kernel<__bf16, 64>), delta_grid, 0);
       } else {
-        if (p.head_dim == 128) AXL_LAUNCH((bwd_delta_kernel<_Float16, 128>), delta_grid, 0);
+        if (width == 128) AXL_LAUNCH((bwd_delta_kernel<_Float16, 128>), delta_grid, 0);
         else AXL_LAUNCH((bwd_delta_kernel<_Float16, 64>), delta_grid, 0);
       }
     }
-    if ((phases & AXL_BWD_DKDV) && err == hipSuccess) err = launch_bwd_dkdv(a, dt, p.head_dim, false, stream);
-    if ((phases & AXL_BWD_DQ) && err == hipSuccess) err = launch_bwd_dq_stream(a, dt, p.head_dim, stream);
+    if ((phases & AXL_BWD_DKDV) && err == hipSuccess) err = launch_bwd_dkdv(a, dt, width, false, stream);
+    if ((phases & AXL_BWD_DQ) && err == hipSuccess) err = launch_bwd_dq_stream(a, dt, width, stream);
     phases &= AXL_BWD_DELTA;  // what is left for the code below: the sink gradient
     phases = (phases & AXL_BWD_DELTA) && p.d_logit_sink ? AXL_BWD_DELTA : 0;
     if (phases) {
@@ -505,8 +507,8 @@ int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream)
       return set_error(AXL_ERR_LAUNCH, "axl_flash_bwd: launch failed: %s", hipGetErrorString(err));
     return AXL_OK;
   } else if ((phases & all) == all && !aux && !p.d_logit_sink) {
-    err = launch_bwd_dq(a, dt, p.head_dim, true, stream);
-    if (err == hipSuccess) err = launch_bwd_dkdv(a, dt, p.head_dim, false, stream);
+    err = launch_bwd_dq(a, dt, width, true, stream);
+    if (err == hipSuccess) err = launch_bwd_dkdv(a, dt, width, false, stream);
     if (err != hipSuccess)
       return set_error(AXL_ERR_LAUNCH, "axl_flash_bwd: launch failed: %s", hipGetErrorString(err));
     return AXL_OK;
@@ -522,10 +524,10 @@ int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream)
   if (dt == AXL_F32) {
     // enqueued above
   } else if (dt == AXL_BF16) {
-    if (p.head_dim == 128) AXL_BWD_PHASES(ElemBf16, __bf16, 128);
+    if (width == 128) AXL_BWD_PHASES(ElemBf16, __bf16, 128);
     else AXL_BWD_PHASES(ElemBf16, __bf16, 64);
   } else {
-    if (p.head_dim == 128) AXL_BWD_PHASES(ElemF16, _Float16, 128);
+    if (width == 128) AXL_BWD_PHASES(ElemF16, _Float16, 128);
     else AXL_BWD_PHASES(ElemF16, _Float16, 64);
   }
 #undef AXL_BWD_PHASES

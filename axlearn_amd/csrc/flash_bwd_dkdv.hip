@@ -100,8 +100,8 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
   bf16x8 kf[KK], vf[KK];
 #pragma unroll
   for (int kk = 0; kk < KK; kk++) {
-    kf[kk] = *(const bf16x8*)(kp + 16 * kk + 8 * g);
-    vf[kk] = *(const bf16x8*)(vp + 16 * kk + 8 * g);
+    kf[kk] = load8_within(kp, 16 * kk + 8 * g, a.d_real);
+    vf[kk] = load8_within(vp, 16 * kk + 8 * g, a.d_real);
   }
   const int kpos = k0 + l32;
   int seg_k = 0;
@@ -167,7 +167,8 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
 #pragma unroll
   for (int i = 0; i < Tile::DMA_PER_WAVE; i++) {
     const int row = 8 * wave + Tile::RPI * i + lane / CPR;
-    const int chunk = (lane % CPR) ^ tile_swizzle<D>(row);
+    const int slot_chunk = (lane % CPR) ^ tile_swizzle<D>(row);
+    const int chunk = slot_chunk * 8 < a.d_real ? slot_chunk : 0;
     // the second load of a pair carries an instruction offset of 1024, which also moves its source
     q_lane[i] = (unsigned)(row * (int)a.qs.s + chunk * 8) * 2 - (i % 2) * 1024;
     d_lane[i] = (unsigned)(row * (int)a.dos.s + chunk * 8) * 2 - (i % 2) * 1024;
@@ -747,11 +748,12 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
       } w;
       w.p[0] = E::pack(dk_acc[dt][4 * rq + 0] * a.scale, dk_acc[dt][4 * rq + 1] * a.scale);
       w.p[1] = E::pack(dk_acc[dt][4 * rq + 2] * a.scale, dk_acc[dt][4 * rq + 3] * a.scale);
-      *(uint2*)(dkp + 32 * dt + 8 * rq + 4 * g) = w.u;
+      const bool in_row = 32 * dt + 8 * rq + 4 * g < a.d_real;
+      if (in_row) *(uint2*)(dkp + 32 * dt + 8 * rq + 4 * g) = w.u;
       const float vs = AUX ? a.aux.keep_scale : 1.0f;  // kept probabilities are P / (1 - rate)
       w.p[0] = E::pack(dv_acc[dt][4 * rq + 0] * vs, dv_acc[dt][4 * rq + 1] * vs);
       w.p[1] = E::pack(dv_acc[dt][4 * rq + 2] * vs, dv_acc[dt][4 * rq + 3] * vs);
-      *(uint2*)(dvp + 32 * dt + 8 * rq + 4 * g) = w.u;
+      if (in_row) *(uint2*)(dvp + 32 * dt + 8 * rq + 4 * g) = w.u;
     }
 }
 

@@ -74,8 +74,8 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
   bf16x8 qf[KK], dof[KK];
 #pragma unroll
   for (int kk = 0; kk < KK; kk++) {
-    qf[kk] = *(const bf16x8*)(qp + 16 * kk + 8 * g);
-    dof[kk] = *(const bf16x8*)(dop + 16 * kk + 8 * g);
+    qf[kk] = load8_within(qp, 16 * kk + 8 * g, a.d_real);
+    dof[kk] = load8_within(dop, 16 * kk + 8 * g, a.d_real);
   }
   const int64_t stat_idx = ((int64_t)b * a.Hq + h) * a.T + q0 + l32;
   float off, delta;  // -lse * log2(e), rowsum(out * dO)
@@ -90,7 +90,7 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
         bf16x8 v;
         bf16x2 p[4];
       } o, d;
-      o.v = *(const bf16x8*)(op + 16 * kk + 8 * g);
+      o.v = load8_within(op, 16 * kk + 8 * g, a.d_real);
       d.v = dof[kk];
 #pragma unroll
       for (int i = 0; i < 4; i++) part = E::dot2(o.p[i], d.p[i], part);
@@ -152,7 +152,8 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
 #pragma unroll
   for (int i = 0; i < Tile::DMA_PER_WAVE; i++) {
     const int row = ROWS_PER_WAVE * wave + Tile::RPI * i + lane / CPR;
-    const int chunk = (lane % CPR) ^ tile_swizzle<D>(row);
+    const int slot_chunk = (lane % CPR) ^ tile_swizzle<D>(row);
+    const int chunk = slot_chunk * 8 < a.d_real ? slot_chunk : 0;
     // the second load of a pair carries an instruction offset of 1024, which also moves its source
     k_lane[i] = (unsigned)(row * (int)a.ks.s + chunk * 8) * 2 - (PAIRS ? (i % 2) * 1024 : 0);
     v_lane[i] = (unsigned)(row * (int)a.vs.s + chunk * 8) * 2 - (PAIRS ? (i % 2) * 1024 : 0);
@@ -509,7 +510,7 @@ void flash_bwd_dq_ring_kernel(const BwdArgs a) {
       } w;
       w.p[0] = E::pack(dq_acc[dt][4 * rq + 0] * a.scale, dq_acc[dt][4 * rq + 1] * a.scale);
       w.p[1] = E::pack(dq_acc[dt][4 * rq + 2] * a.scale, dq_acc[dt][4 * rq + 3] * a.scale);
-      *(uint2*)(dqp + 32 * dt + 8 * rq + 4 * g) = w.u;
+      if (32 * dt + 8 * rq + 4 * g < a.d_real) *(uint2*)(dqp + 32 * dt + 8 * rq + 4 * g) = w.u;
     }
 }
 

@@ -119,7 +119,8 @@ __global__ __launch_bounds__(64 * NW) void flash_bwd_dq_stream_kernel(const BwdA
 #pragma unroll
   for (int i = 0; i < Tile::K_DMA_PER_WAVE; i++) {
     const int row = Tile::WROWS * wave + Tile::RPI * i + lane / CPR;
-    const int chunk = (lane % CPR) ^ tile_swizzle<D>(row);
+    const int slot_chunk = (lane % CPR) ^ tile_swizzle<D>(row);
+    const int chunk = slot_chunk * 8 < a.d_real ? slot_chunk : 0;
     // the second load of a pair carries an instruction offset of 1024, which also moves its source
     k_lane[i] = (unsigned)(row * (int)a.ks.s + chunk * 8) * 2 - (i % 2) * 1024;
   }
@@ -242,7 +243,7 @@ __global__ __launch_bounds__(64 * NW) void flash_bwd_dq_stream_kernel(const BwdA
       } w;
       w.p[0] = E::pack(dq_acc[dt][4 * rq + 0] * a.scale, dq_acc[dt][4 * rq + 1] * a.scale);
       w.p[1] = E::pack(dq_acc[dt][4 * rq + 2] * a.scale, dq_acc[dt][4 * rq + 3] * a.scale);
-      *(uint2*)(dqp + 32 * dt + 8 * rq + 4 * g) = w.u;
+      if (32 * dt + 8 * rq + 4 * g < a.d_real) *(uint2*)(dqp + 32 * dt + 8 * rq + 4 * g) = w.u;
     }
 }
 

@@ -39,6 +39,7 @@ struct FwdArgs {
   int B, T, S, Hq, Hkv;
   int mask_kind, window, q_off;
   float scale;
+  int d_real;  // head_dim of the tensors: a multiple of 8, at most the compiled width D (16-bit kernels)
 };
 
 // NW wavefronts of 32 query rows each.  The kernels are launched with 4 (two workgroups per CU); 8
@@ -88,9 +89,15 @@ void flash_fwd_kernel(const FwdArgs a) {
   const __bf16* vp = (const __bf16*)a.v + b * a.vs.b + hk * a.vs.h;
 
   // Q fragments: B operand of S^T = K Q^T; lane (query l32, k-group g) holds d = 16kk + 8g .. +7.
+  // (A head_dim below the compiled width: the columns past it are zeros here, so whatever the K tile
+  // holds in them adds nothing to the logits; the V columns past it make output columns that are not
+  // stored.  The tiles fetch slice 0 of the row in their place: finite values, no padded copies.)
   bf16x8 qf[KK];
 #pragma unroll
-  for (int kk = 0; kk < KK; kk++) qf[kk] = *(const bf16x8*)(qp + 16 * kk + 8 * g);
+  for (int kk = 0; kk < KK; kk++) {
+    const bf16x8 zero8 = {};
+    qf[kk] = 16 * kk + 8 * g < a.d_real ? *(const bf16x8*)(qp + 16 * kk + 8 * g) : zero8;
+  }
 
   // Visible key range of this workgroup.
   int k_begin = 0, k_end = a.S;
@@ -158,7 +165,8 @@ void flash_fwd_kernel(const FwdArgs a) {
 #pragma unroll
   for (int i = 0; i < Tile::DMA_PER_WAVE; i++) {
     const int row = Tile::WROWS * wave + RPI * i + lane / CPR;
-    const int chunk = (lane % CPR) ^ Tile::swz(row);
+    const int slot_chunk = (lane % CPR) ^ Tile::swz(row);
+    const int chunk = slot_chunk * 8 < a.d_real ? slot_chunk : 0;
     // the second load of a pair carries an instruction offset of 1024, which also moves its source
     k_src[i] = (unsigned)(row * (int)a.ks.s + chunk * 8) * 2 - (i % 2) * 1024;
     v_src[i] = (unsigned)(row * (int)a.vs.s + chunk * 8) * 2 - (i % 2) * 1024;
@@ -573,7 +581,7 @@ void flash_fwd_kernel(const FwdArgs a) {
       } w;
       w.p[0] = E::pack(o[dt][4 * rq + 0] * inv_l, o[dt][4 * rq + 1] * inv_l);
       w.p[1] = E::pack(o[dt][4 * rq + 2] * inv_l, o[dt][4 * rq + 3] * inv_l);
-      *(uint2*)(op + 32 * dt + 8 * rq + 4 * g) = w.u;
+      if (32 * dt + 8 * rq + 4 * g < a.d_real) *(uint2*)(op + 32 * dt + 8 * rq + 4 * g) = w.u;
     }
   }
   if (a.lse && g == 0) {
@@ -773,6 +781,8 @@ int launch_flash_fwd(const AxlFlashFwdParams& p, hipStream_t stream) {
   a.mask_kind = p.mask_kind; a.window = p.sliding_window; a.q_off = p.q_pos_offset;
   a.q_offs = p.q_pos_offsets;
   a.scale = p.softmax_scale;
+  a.d_real = p.head_dim;
+  const int width = p.head_dim <= 64 ? 64 : 128;  // the compiled width that serves this head_dim
   hipError_t err = hipSuccess;
 #define AXL_LAUNCH_FWD(KERNEL, TILE)                                                            \
   do {                                                                                          \
@@ -785,7 +795,7 @@ int launch_flash_fwd(const AxlFlashFwdParams& p, hipStream_t stream) {
   } while (0)
 #define AXL_LAUNCH_FWD16(E)                                                                     \
   do {                                                                                          \
-    if (p.head_dim == 128) {                                                                    \
+    if (width == 128) {                                                                         \
       if (aux) AXL_LAUNCH_FWD((flash_fwd_kernel<E, 128, true>), FwdTile<128>);                  \
       else AXL_LAUNCH_FWD((flash_fwd_kernel<E, 128, false>), FwdTile<128>);                     \
     } else {                                                                                    \

@@ -66,16 +66,30 @@ def classify_mask_bias(mask: BaseAttentionBias) -> Optional[Tuple[int, int]]:
 
 
 def padded_head_dim(head_dim: int) -> Optional[int]:
-    """Head dim the kernels run at for a given model head dim (None if it does not fit).
+    """Compiled width the kernels run a given head dim at (None if it does not fit).
 
     The Pallas kernel pads the head dim to the next power of two inside its blocks and masks the
-    extra columns (gpu_attention.py:172-176, :328); here the tensors are zero-padded to the next
-    compiled width instead: zero columns of q/k add nothing to the logits and zero columns of v
-    give zero output columns, which are sliced off again."""
+    extra columns (gpu_attention.py:172-176, :328).  The 16-bit HIP kernels do the same on the tensors
+    as they are for any multiple of 8 (`runs_at_native_head_dim`); what they do not take that way is
+    zero-padded to the width by `_pad_last` instead: zero columns of q/k add nothing to the logits and
+    zero columns of v give zero output columns, which are sliced off again."""
     for width in (64, 128):
         if head_dim <= width:
             return width
     return None
+
+
+def runs_at_native_head_dim(query: Tensor, key: Tensor, value: Tensor, *, aux: bool) -> bool:
+    """Whether the kernels take these tensors without padded copies: head dims 64 and 128 always;
+    other multiples of 8 in bf16 / f16 without a bias or dropout mask, rows at least one compiled
+    width apart (the kernels' tile loads assume that much; a single head of 72 columns is not)."""
+    head_dim = query.shape[-1]
+    if head_dim in (64, 128):
+        return True
+    width = padded_head_dim(head_dim)
+    if width is None or head_dim % 8 != 0 or aux or query.dtype == torch.float32:
+        return False
+    return all(x.stride(1) >= width and x.shape[2] * head_dim >= width for x in (query, key, value))
 
 
 def _pad_last(x: Tensor, width: int) -> Tensor:
@@ -113,6 +127,8 @@ def _attend(query, key, value, segment_ids, softmax_scale, mask_kind, window, lo
     width = padded_head_dim(head_dim)
     if width is None:
         raise NotImplementedError(f"{head_dim=} > 128 is not supported by the HIP kernels.")
+    if runs_at_native_head_dim(query, key, value, aux=bias is not None or dropout_mask is not None):
+        width = head_dim
     out = _FlashAttentionFn.apply(
         _pad_last(query, width), _pad_last(key, width), _pad_last(value, width), segment_ids,
         softmax_scale, mask_kind, window, logit_sink, bias, dropout_mask, dropout_rate, save_residuals,
@@ -308,7 +324,7 @@ class HipFlashAttention(BaseFlashAttention):
         consecutive = positions[:, :1] + torch.arange(t, device=query.device)[None]
         if not torch.equal(positions, consecutive.to(positions.dtype)):
             raise NotImplementedError("target_positions of a chunk must be consecutive.")
-        width = padded_head_dim(head_dim)
+        width = head_dim if runs_at_native_head_dim(query, key, value, aux=False) else padded_head_dim(head_dim)
         rows = -(-t // 128) * 128
         q = torch.nn.functional.pad(query.detach(), (0, width - head_dim, 0, 0, 0, rows - t))
         out, _ = ops.flash_fwd(

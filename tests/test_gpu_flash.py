@@ -579,12 +579,73 @@ def test_logit_sink_through_dispatch_with_autograd():
     assert sd.grad.shape == (hq,) and ref.rel_l2(sd.grad.cpu(), ws) < 1e-2
 
 
-@pytest.mark.parametrize("d", [32, 80, 96, 120])
-def test_head_dims_between_the_compiled_widths(d):
-    # Any head dim up to 128 is accepted, as by the Pallas kernel (gpu_attention.py:172-176, :954):
-    # the host zero-pads to 64 or 128 and slices the result; gradients flow through the padding.
-    b, t, hq, hkv = 1, 256, 4, 2
+@pytest.mark.parametrize("d", [32, 72, 80, 96, 120])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_head_dims_between_the_compiled_widths(d, dtype, monkeypatch):
+    """Any head dim up to 128 is accepted, as by the Pallas kernel (gpu_attention.py:172-176, :954).  In
+    bf16 / f16 a multiple of 8 runs on the tensors as they are: no padded copy of q, k, v or dO is made
+    (the padding helper must not be called), forward and both backward paths."""
+    from axlearn_amd.flash_attention import hip_attention
+
+    def no_padding(x, width):
+        assert x.shape[-1] == width, "a padded copy was made"
+        return x
+
+    monkeypatch.setattr(hip_attention, "_pad_last", no_padding)
+    b, t, hq, hkv = 2, 512, 4, 2
+    q, k, v, do = _inputs(b, t, hq, hkv, d, dtype)
+    scale = d ** -0.5
+    segs = ref.packed_segment_ids(4, b, t, max_docs=3)
+    pos = dict(target_positions=torch.arange(t)[None], source_positions=torch.arange(t)[None])
+    for window, seg, ds in ((None, False, True), (None, False, False), (100, True, True), (100, True, False)):
+        qd, kd, vd = (x.cuda().requires_grad_(True) for x in (q, k, v))
+        mask = ab.CausalAttentionBias(**pos) if window is None else ab.SlidingWindowAttentionBias(
+            ab.sliding_window_causal_mask(window), sliding_window_size=window, **pos)
+        bias = ab.CompositeAttentionBias([mask] + ([ab.SegmentIdAttentionBias(segs.cuda())] if seg else []))
+        fa = HipFlashAttention.default_config().set(softmax_scale=scale, bwd_ds_workspace=ds).instantiate()
+        batch = dict(query=qd, key=kd, value=vd, bias=bias)
+        assert fa.is_supported(batch, kv_cache_type=None)
+        out = fa(batch)
+        assert out.shape == (b, t, hq, d)
+        (out.float() * do.cuda().float()).sum().backward()
+        spec = ref.MaskSpec(causal=window is None, sliding_window=window, segment_ids=segs if seg else None)
+        want = ref.reference_mha(q, k, v, spec, softmax_scale=scale)
+        wq, wk, wv = ref.reference_mha_grads(q, k, v, do, spec, softmax_scale=scale)
+        _assert_close("out", out, want, dtype)
+        for name, got, exp in (("dq", qd.grad, wq), ("dk", kd.grad, wk), ("dv", vd.grad, wv)):
+            assert got.shape == exp.shape and got.is_contiguous()
+            _assert_close(name, got, exp, dtype)
+
+
+def test_head_dim_columns_past_the_end_are_never_used():
+    """head_dim 72 as a view of wider tensors whose other columns hold NaN: neither the forward nor the
+    backward lets one of them into a result (the tile loads stay inside the 72 columns)."""
+    b, t, hq, hkv, d, wide = 1, 256, 4, 2, 72, 128
     q, k, v, do = _inputs(b, t, hq, hkv, d, torch.bfloat16)
+
+    def widen(x):
+        w = torch.full(x.shape[:-1] + (wide,), float("nan"), dtype=x.dtype, device="cuda")
+        w[..., :d] = x.cuda()
+        return w[..., :d]
+
+    kw = dict(softmax_scale=d ** -0.5, mask_kind=ops.MASK_CAUSAL)
+    out, lse = ops.flash_fwd(widen(q), widen(k), widen(v), **kw)
+    base, base_lse = ops.flash_fwd(q.cuda(), k.cuda(), v.cuda(), **kw)
+    assert torch.equal(out, base) and torch.equal(lse, base_lse)
+    for ds in (False, True):
+        got = ops.flash_bwd(widen(q), widen(k), widen(v), widen(out.cpu()), lse, widen(do), ds_workspace=ds, **kw)
+        want = ops.flash_bwd(q.cuda(), k.cuda(), v.cuda(), base, base_lse, do.cuda(), ds_workspace=ds, **kw)
+        for x, y in zip(got, want):
+            assert torch.isfinite(x.float()).all() and torch.equal(x, y)
+
+
+@pytest.mark.parametrize("d,dtype,hq,hkv", [(36, torch.bfloat16, 4, 2), (80, torch.float32, 4, 2), (72, torch.bfloat16, 1, 1),
+                                             (8, torch.bfloat16, 4, 2)])
+def test_head_dims_that_take_the_padded_path(d, dtype, hq, hkv):
+    """What the kernels do not take as it is - a head dim that is not a multiple of 8, float32, rows
+    closer together than the compiled width - is zero-padded by the host mirror and sliced."""
+    b, t = 1, 256
+    q, k, v, do = _inputs(b, t, hq, hkv, d, dtype)
     qd, kd, vd = (x.cuda().requires_grad_(True) for x in (q, k, v))
     scale = d ** -0.5
     out = flash_attention(qd, kd, vd, softmax_scale=scale, mask_fn=ab.causal_mask)
@@ -593,16 +654,10 @@ def test_head_dims_between_the_compiled_widths(d):
     spec = ref.MaskSpec(causal=True)
     want = ref.reference_mha(q, k, v, spec, softmax_scale=scale)
     wq, wk, wv = ref.reference_mha_grads(q, k, v, do, spec, softmax_scale=scale)
-    _assert_close("out", out, want, torch.bfloat16)
+    _assert_close("out", out, want, dtype)
     for name, got, exp in (("dq", qd.grad, wq), ("dk", kd.grad, wk), ("dv", vd.grad, wv)):
         assert got.shape == exp.shape
-        _assert_close(name, got, exp, torch.bfloat16)
-    pos = dict(target_positions=torch.arange(t)[None], source_positions=torch.arange(t)[None])
-    bias = ab.CompositeAttentionBias([ab.CausalAttentionBias(**pos)])
-    fa = HipFlashAttention.default_config().set(softmax_scale=scale).instantiate()
-    batch = dict(query=qd.detach(), key=kd.detach(), value=vd.detach(), bias=bias)
-    assert fa.is_supported(batch, kv_cache_type=None)
-    assert torch.equal(fa(batch), out.detach())
+        _assert_close(name, got, exp, dtype)
 
 
 # ----------------------------------------------------------------------------- dense bias, dropout

@@ -316,8 +316,19 @@ def test_abi_validation_without_gpu():
     assert lib.axl_flash_fwd(ctypes.byref(p), None) == _lib.AXL_ERR_INVALID_ARGUMENT
     assert b"divisible" in lib.axl_last_error()
     p.num_q_heads = 4
-    p.head_dim = 72
+    p.head_dim = 76   # bf16: multiples of 8 up to 128 run on the tensors as they are, others do not
     assert lib.axl_flash_fwd(ctypes.byref(p), None) == _lib.AXL_ERR_UNSUPPORTED
+    p.head_dim = 72   # ... if the rows lie at least one compiled width (128) apart
+    p.k_strides = _lib.AxlStrides(1 << 20, 72, 72)
+    assert lib.axl_flash_fwd(ctypes.byref(p), None) == _lib.AXL_ERR_UNSUPPORTED
+    assert b"128 elements apart" in lib.axl_last_error()
+    p.k_strides = s
+    p.aux = _lib.AxlAttnAux(bias=256, bias_batch_stride=0, bias_head_stride=0, bias_row_stride=128, bias_dtype=1)
+    assert lib.axl_flash_fwd(ctypes.byref(p), None) == _lib.AXL_ERR_UNSUPPORTED  # no such form with a bias
+    p.aux = _lib.AxlAttnAux()
+    p.dtype = 1       # float32: the compiled widths only
+    assert lib.axl_flash_fwd(ctypes.byref(p), None) == _lib.AXL_ERR_UNSUPPORTED
+    p.dtype = 0
     p.head_dim = 128
     p.q_len = 100
     assert lib.axl_flash_fwd(ctypes.byref(p), None) == _lib.AXL_ERR_UNSUPPORTED
