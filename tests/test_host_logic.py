@@ -601,3 +601,58 @@ def test_forward_kernel_keeps_the_distance_behind_its_assembly_mfma_chains():
     that touches it.)"""
     asm, _ = _device_asm("flash_fwd.hip", extra=("-mllvm", "-amdgpu-mfma-vgpr-form"))
     _assert_asm_mfma_distances(asm, r"_ZN3axl16flash_fwd_kernel", 4)
+
+
+def test_ffi_shim_and_jax_side_stay_in_step_with_the_abi():
+    """csrc/ffi_shim.cc and flash_attention/jax_ffi.py cannot be compiled or imported here (no jaxlib
+    headers, no jax), so an ABI change could leave them behind unnoticed.  Checked from their text:
+    every field the shim fills exists in the header's structure of that name (through the ctypes mirror,
+    itself checked against the header), every handler binds as many operands, results and attributes -
+    by name - as the JAX side passes to `jax.ffi.ffi_call`, and every registered target has a handler."""
+    import ast
+
+    pkg = os.path.join(ROOT, "axlearn_amd")
+    shim = open(os.path.join(pkg, "csrc", "ffi_shim.cc")).read()
+    shim_code = re.sub(r"//[^\n]*", "", shim)
+    structs = {c.__name__: {f[0] for f in c._fields_} for c in (
+        _lib.AxlFlashFwdParams, _lib.AxlFlashBwdParams, _lib.AxlDecodeParams, _lib.AxlPagedDecodeParams,
+        _lib.AxlPageInsertParams, _lib.AxlAttnAux, _lib.AxlDecodeBias, _lib.AxlStrides)}
+    # ---- fields filled through `T p{}` / `T* name` variables
+    funcs = re.split(r"\nffi::Error (\w+)\(", shim_code)
+    filled = 0
+    for name, body in zip(funcs[1::2], funcs[2::2]):
+        body = body[:body.find("\n}\n")]
+        local = {v: t for t, v in re.findall(r"\b(Axl\w+)\s+(\w+)\{\}", body)}  # AxlDecodeParams p{}
+        local.update({v: t for t, v in re.findall(r"\b(Axl\w+)\*\s+(\w+)\b", body)})  # AxlAttnAux* aux
+        for var, typ in list(local.items()):
+            if typ not in structs:
+                continue
+            for fld in re.findall(r"\b%s(?:\.|->)(\w+)\s*=[^=]" % re.escape(var), body):
+                assert fld in structs[typ], f"{name}: {typ} has no field {fld}"
+                filled += 1
+    assert filled > 80
+    # ---- bindings
+    bound = {}
+    for m in re.finditer(r"XLA_FFI_DEFINE_HANDLER_SYMBOL\((\w+),\s*(\w+),(.*?)\);[ \t]*\n", shim_code, flags=re.S):
+        target, func, bind = m.groups()
+        assert re.search(r"\nffi::Error %s\(" % func, shim_code), func
+        bound[target] = (len(re.findall(r"\.Arg<", bind)), len(re.findall(r"\.Ret<", bind)),
+                         re.findall(r'\.Attr<\w+>\("(\w+)"\)', bind))
+    # ---- the JAX side's calls
+    tree = ast.parse(open(os.path.join(pkg, "flash_attention", "jax_ffi.py")).read())
+    called = {}
+    registered = None
+    for node in ast.walk(tree):
+        if isinstance(node, ast.Call) and isinstance(node.func, ast.Call) and ast.unparse(node.func.func).endswith("ffi_call"):
+            inner = node.func
+            results = inner.args[1]
+            assert isinstance(results, (ast.Tuple, ast.List))
+            called[inner.args[0].value] = (len(node.args), len(results.elts), [k.arg for k in node.keywords])
+        if isinstance(node, ast.For) and "register_ffi_target" in ast.unparse(node):
+            registered = [e.value for e in node.iter.elts]
+    assert registered is not None and set(registered) == set(bound) == set(called)
+    for target, (n_args, n_rets, attrs) in bound.items():
+        assert called[target] == (n_args, n_rets, attrs), (target, called[target], (n_args, n_rets, attrs))
+    # the version the shim and the binding were written against
+    assert _lib.ABI_VERSION == int(re.search(r"#define AXL_ATTN_ABI_VERSION (\d+)",
+                                             open(os.path.join(ROOT, "include", "axl_attn.h")).read()).group(1))
