@@ -359,6 +359,25 @@ def test_baseline_c4_full_size():
     with _deterministic():
         det2 = ops.paged_decode(q, kp2, vp2, tables2.to(dev), lengths.to(dev), softmax_scale=scale)
     assert torch.equal(det, det2)
+    # The same pools read as 64-token pages (four adjacent 16-token pages each) under a table of their
+    # own: the oracle checks the sampled sequences again, and the result does not depend on which page
+    # size the same tokens are addressed through (fixed decomposition: bit for bit).
+    kp64, vp64 = kp2.view(Hkv, P // 4, 64, D), vp2.view(Hkv, P // 4, 64, D)
+    tables64 = torch.from_numpy(np.random.default_rng(8).permutation(P // 4).astype(np.int32)).reshape(B, pps // 4)
+    out64 = ops.paged_decode(q, kp64, vp64, tables64.to(dev), lengths.to(dev), softmax_scale=scale)
+    for bi in sample:
+        n_pages = (int(lengths[bi]) + 63) // 64
+        idx = tables64[bi, :n_pages].long().to(dev)
+        local = torch.arange(n_pages, dtype=torch.int32)[None]
+        want = ref.reference_decode(q[bi:bi + 1].cpu().unsqueeze(1), kp64[:, idx].cpu(), vp64[:, idx].cpu(),
+                                    lengths[bi:bi + 1], softmax_scale=scale, page_tables=local)[:, 0]
+        assert _ok(out64[bi:bi + 1].cpu(), want), bi
+    # ... 16-token tables that spell out the same physical tokens
+    tables16 = (4 * tables64[:, :, None] + torch.arange(4, dtype=torch.int32)[None, None, :]).reshape(B, pps)
+    with _deterministic():
+        a64 = ops.paged_decode(q, kp64, vp64, tables64.to(dev), lengths.to(dev), softmax_scale=scale)
+        a16 = ops.paged_decode(q, kp2, vp2, tables16.to(dev), lengths.to(dev), softmax_scale=scale)
+    assert torch.equal(a64, a16)
 
 
 def test_wide_groups_and_batch_slices():
