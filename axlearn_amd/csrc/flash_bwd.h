@@ -30,6 +30,7 @@ struct BwdArgs {
                 // bias / dropout mask).  Operand fragments are zero past it, tile loads fetch slice 0 of the row in
                 // place of the slices past it (finite values that only ever meet those zeros or end up in
                 // output columns that are not stored), stores leave the columns past it out.
+  int kb_per_wg;  // key blocks (of 128 keys) a dK/dV workgroup works through: 1, or 2 (a block and its mirror image)
   AuxArgs aux;  // dense bias / dropout mask (read only by the AUX instantiations)
 };
 

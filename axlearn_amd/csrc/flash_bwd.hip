@@ -450,6 +450,13 @@ int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream)
   a.mask_kind = p.mask_kind; a.window = p.sliding_window; a.q_off = p.q_pos_offset;
   a.scale = p.softmax_scale;
   a.d_real = p.head_dim;
+  {
+    // Two key blocks per dK/dV workgroup under a causal mask, where a block and its mirror image see
+    // complementary shares of the queries (an even number of blocks); AXL_DKDV_KB_PER_WG=1 in the
+    // environment (read once) keeps one block per workgroup.
+    static const bool single = [] { const char* e = getenv("AXL_DKDV_KB_PER_WG"); return e && e[0] == '1'; }();
+    a.kb_per_wg = (!single && p.mask_kind == AXL_MASK_CAUSAL && (p.kv_len / 128) % 2 == 0) ? 2 : 1;
+  }
   const int width = p.head_dim <= 64 ? 64 : 128;   // the compiled width that serves this head_dim
   a.aux = make_aux_args(p.aux, p.softmax_scale);
   const bool aux = p.aux.bias || p.aux.dropout_mask;

@@ -69,28 +69,42 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
   static_assert(Tile::BQ == 32, "tiling");
   extern __shared__ __attribute__((aligned(16))) char smem[];
 
-  const int tid = threadIdx.x;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l32 = lane & 31, g = lane >> 5;
   const int G = a.Hq / a.Hkv;
   // blockIdx -> (key block, batch, kv head).  When the (batch, kv head) pairs divide evenly over the
   // 8 XCDs (workgroup i is dispatched to XCD i % 8), an XCD works through one pair after the other,
   // so the workgroups that run together stream the same Q / dO rows through that XCD's L2; within a
   // pair the earliest key blocks (most queries under a causal mask) come first.
+  // With a.kb_per_wg == 2 a workgroup works through TWO key blocks of its pair, one after the other:
+  // block kb0 of the first half and its mirror image nkb - 1 - kb0.  Under a causal mask the two see
+  // complementary shares of the queries, so every workgroup of the launch walks the same number of
+  // tiles: the workgroups of a pair that start together stay in step down their first blocks (one of
+  // them brings a Q / dO tile into L2, the others find it there), half as many workgroups start and
+  // end, and the launch divides evenly over the CUs.
   const int npairs = a.B * a.Hkv, nkb = a.S / Tile::BKV;
-  int kb, pair;
+  const int nkb_wg = nkb / a.kb_per_wg;              // key blocks the blockIdx mapping numbers
+  int kb0, pair;
   if (npairs % 8 == 0) {
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
     const int ppx = npairs >> 3;                     // pairs per XCD
-    const int grp = slot / (AXL_DKDV_PG * nkb);      // group of AXL_DKDV_PG pairs worked through together
-    const int r = slot - grp * (AXL_DKDV_PG * nkb);
+    const int grp = slot / (AXL_DKDV_PG * nkb_wg);   // group of AXL_DKDV_PG pairs worked through together
+    const int r = slot - grp * (AXL_DKDV_PG * nkb_wg);
     const int pg = min(AXL_DKDV_PG, ppx - grp * AXL_DKDV_PG);
     pair = xcd + 8 * (grp * AXL_DKDV_PG + r % pg);
-    kb = r / pg;
+    kb0 = r / pg;
   } else {
-    kb = blockIdx.x / npairs;
+    kb0 = blockIdx.x / npairs;
     pair = blockIdx.x % npairs;
   }
   const int b = pair / a.Hkv, hk = pair % a.Hkv;
+  for (int pass = 0; pass < a.kb_per_wg; pass++) {
+  // Everything a key block needs is derived again from the thread index inside its pass (the empty
+  // statement hides the index's origin from the compiler): hoisted out of the pass loop, the lane
+  // offsets of the prologue and the epilogue would stay live through the main loops, which have no
+  // register to spare.
+  int tid = threadIdx.x;
+  asm volatile("" : "+v"(tid));
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+  const int kb = pass == 0 ? kb0 : nkb - 1 - kb0;
   const int k0_wg = kb * Tile::BKV;
   const int k0 = k0_wg + wave * 32;  // this wavefront's keys
 
@@ -133,9 +147,13 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
   // Tiles in processing order: query tile (outer, from the LAST one down to the diagonal) x query head
   // (inner).  Every workgroup of a (batch, kv head) pair starts at the same last tile and walks down
   // until it reaches its own diagonal, so the workgroups that run together read the same Q / dO rows
-  // at the same time and all but one of them find them in L2.
+  // at the same time and all but one of them find them in L2.  The second key block of a workgroup is
+  // walked the other way, from its diagonal UP to the last tile: a workgroup that took nkb - kb0
+  // steps down its first block starts its second at tile nkb - 1 - kb0, so at any moment the
+  // workgroups that started together are again all at the same tile, and they end together.
   const int total = nt * G;
-  const int t_first = t_begin + max(nt - 1, 0);  // the tile the sequence starts with
+  const int dir = pass == 0 ? -1 : 1;
+  const int t_first = t_begin + (dir < 0 ? max(nt - 1, 0) : 0);  // the tile the sequence starts with
   // dS store cursor (SPILL): block of this wavefront's 32 keys in the run of the tile whose stage B
   // the iteration executes; it walks the tiles in processing order.  A lane stores its two packed
   // operand registers at [query half][key l32][8 g .. 8 g + 7].
@@ -176,7 +194,7 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
   const int st_kind = wave;
   // Running source pointers of the prefetch cursor, advanced by wave-uniform steps: no 64-bit
   // multiplies inside the loop.  A step goes to the next head of the same query tile, a wrap from
-  // the last head back to the first head of the tile before.
+  // the last head back to the first head of the tile before (dir < 0) or after it.
   const __bf16* q_src = (const __bf16*)a.q + b * a.qs.b + (int64_t)(hk * G) * a.qs.h + (int64_t)t_first * Tile::BQ * a.qs.s;
   const __bf16* d_src = (const __bf16*)a.dout + b * a.dos.b + (int64_t)(hk * G) * a.dos.h + (int64_t)t_first * Tile::BQ * a.dos.s;
   const int64_t stat_row0 = ((int64_t)b * a.Hq + hk * G) * a.T + (int64_t)t_first * Tile::BQ;
@@ -185,11 +203,11 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
   if (s_is_seg) s_src = (const char*)(a.seg + (int64_t)b * a.T + (int64_t)t_first * Tile::BQ);
   const unsigned s_lane = 16 * (lane & 7);  // lanes 0..7 fetch 4 query rows each
   const int64_t q_step = a.qs.h, d_step = a.dos.h;
-  const int64_t q_wrap = -(int64_t)(G - 1) * a.qs.h - (int64_t)Tile::BQ * a.qs.s;
-  const int64_t d_wrap = -(int64_t)(G - 1) * a.dos.h - (int64_t)Tile::BQ * a.dos.s;
+  const int64_t q_wrap = -(int64_t)(G - 1) * a.qs.h + dir * (int64_t)Tile::BQ * a.qs.s;
+  const int64_t d_wrap = -(int64_t)(G - 1) * a.dos.h + dir * (int64_t)Tile::BQ * a.dos.s;
   // statistics rows are [B, Hq, T] fp32; segment ids do not depend on the head
   const int64_t s_step = s_is_seg ? 0 : (int64_t)a.T * 4;
-  const int64_t s_wrap = s_is_seg ? -(int64_t)Tile::BQ * 4 : (-(int64_t)(G - 1) * a.T - Tile::BQ) * 4;
+  const int64_t s_wrap = s_is_seg ? dir * (int64_t)Tile::BQ * 4 : (-(int64_t)(G - 1) * a.T + dir * Tile::BQ) * 4;
   const unsigned lds0 = lds_address(smem);
   // The k-th group of loads (Q rows, dO rows, statistics) of the cursor's tile into the buffer at LDS
   // address BUF_; all from scalar bases, no vector instruction forms an address.
@@ -211,14 +229,14 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
     AXL_DMA(BUF_, 0) AXL_DMA(BUF_, 1) AXL_DMA(BUF_, 2)                                            \
   }
   // Prefetch cursor; it stops at the last tile (re-fetching that tile is harmless).
-  int pf_idx = 0, pf_t = max(nt - 1, 0), pf_h = 0;  // tile number, query tile (from t_begin), head within the group
+  int pf_idx = 0, pf_t = t_first - t_begin, pf_h = 0;  // tile number, query tile (from t_begin), head within the group
 #define AXL_ADVANCE()                                                       \
   {                                                                         \
     const bool adv_ = pf_idx + 1 < total;                                   \
     const bool wrap_ = adv_ && (pf_h + 1 == G);                             \
     pf_idx += adv_ ? 1 : 0;                                                 \
     pf_h = wrap_ ? 0 : pf_h + (adv_ ? 1 : 0);                               \
-    pf_t -= wrap_ ? 1 : 0;                                                  \
+    pf_t += wrap_ ? dir : 0;                                                \
     q_src += adv_ ? (wrap_ ? q_wrap : q_step) : 0;                          \
     d_src += adv_ ? (wrap_ ? d_wrap : d_step) : 0;                          \
     s_src += adv_ ? (wrap_ ? s_wrap : s_step) : 0;                          \
@@ -527,12 +545,12 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
       // end of the iteration the stores have long been accepted.
       store16x2(ds_lane, ds_ptr, dsb.v[0], dsb.v[1]);
       // next head of the same tile (one run further), or head 0 of the tile before (G runs of that
-      // tile back from head 0 of this one)
+      // tile back from head 0 of this one) or of the tile after (which is the next run as well)
       const bool wrap_ = st_h + 1 == G;
       const int run_ = 4 * ((st_t >> 2) + 1) * kDsBlockBytes, run_prev_ = 4 * (((st_t - 1) >> 2) + 1) * kDsBlockBytes;
-      ds_ptr += wrap_ ? -(int64_t)((G - 1) * run_ + G * run_prev_) : (int64_t)run_;
+      ds_ptr += wrap_ && dir < 0 ? -(int64_t)((G - 1) * run_ + G * run_prev_) : (int64_t)run_;
       st_h = wrap_ ? 0 : st_h + 1;
-      st_t -= wrap_ ? 1 : 0;
+      st_t += wrap_ ? dir : 0;
     }
     __builtin_amdgcn_sched_barrier(0);
     // One MFMA slot.  The slot number is a compile-time constant (the slots are instantiated one by
@@ -666,7 +684,8 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
   };
   // Query tile t (counted from t_begin) needs no mask for this wavefront's 32 keys when its queries
   // all see them: t in [u_lo, u_hi].  In processing order tile number e is query tile nt - 1 - e / G
-  // of head e % G, and the elementwise tile of iteration j is e = j + 1.
+  // (walking down) or e / G (walking up) of head e % G, and the elementwise tile of iteration j is
+  // e = j + 1.
   auto floor_div = [](int x, int y) { return x >= 0 ? x / y : -((-x + y - 1) / y); };
   int u_lo = 0, u_hi = nt - 1;
   if (a.mask_kind != AXL_MASK_NONE) {
@@ -711,9 +730,10 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
       run(j, j_end, masked_c);
       j = max(j, j_end);
     };
-    run_to(G * (nt - 1 - u_hi), std::true_type{});   // far end of a sliding window
-    run_to(G * (nt - u_lo), std::false_type{});      // interior
-    run_to(total, std::true_type{});                 // down to the diagonal
+    // walking down: far end of a sliding window, interior, down to the diagonal; walking up: the reverse
+    run_to(dir < 0 ? G * (nt - 1 - u_hi) : G * u_lo, std::true_type{});
+    run_to(dir < 0 ? G * (nt - u_lo) : G * (u_hi + 1), std::false_type{});
+    run_to(total, std::true_type{});
     run(j, total, std::true_type{});  // the last iteration (its elementwise tile is past the end)
   }
 #undef AXL_AUX_ROW0
@@ -755,6 +775,8 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
       w.p[1] = E::pack(dv_acc[dt][4 * rq + 2] * vs, dv_acc[dt][4 * rq + 3] * vs);
       if (in_row) *(uint2*)(dvp + 32 * dt + 8 * rq + 4 * g) = w.u;
     }
+  __syncthreads();  // every wavefront is done with the ring before the next key block's first tiles arrive
+  }  // key blocks of this workgroup
 }
 
 template <typename E, int D, bool HAS_SEG, int AUX, bool SPILL = false>
@@ -763,7 +785,7 @@ static hipError_t launch_one(const BwdArgs& a, hipStream_t stream) {
   auto kernel = flash_bwd_dkdv_kernel<E, D, HAS_SEG, AUX, SPILL>;
   hipError_t err = allow_dynamic_lds((const void*)kernel, Tile::LDS_BYTES);
   if (err != hipSuccess) return err;
-  const int grid = (a.S / Tile::BKV) * a.B * a.Hkv;
+  const int grid = (a.S / Tile::BKV) * a.B * a.Hkv / a.kb_per_wg;
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), Tile::LDS_BYTES, stream, a);
   return hipGetLastError();
 }
