@@ -378,6 +378,13 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
     PB_.p[I_] = E::pack(s_e[2 * (I_)], s_e[2 * (I_) + 1]);            \
     DSB_.p[I_] = E::pack(dp_e[2 * (I_)], dp_e[2 * (I_) + 1]);         \
   }
+  // Ahead of the inline-assembly chains of a pipeline-fill tile, whose accumulators vector ALU
+  // instructions have just set (zeros, -delta): a matrix instruction that reads, as its addend, a
+  // register which a vector ALU instruction wrote right before it gets a stale value, and the
+  // compiler, which keeps that distance for its own MFMAs, does not know what the assembly is.  The
+  // wait below is placed after whatever wrote the registers and before the first MFMA.
+#define AXL_CHAIN_START(S_, DP_) \
+  if constexpr (!AUX) asm volatile("s_nop 7" : "+v"(S_), "+v"(DP_));
   // Stage A of the tile in BUF_ into (S_, DP_), not interleaved with anything (pipeline fill).
 #define AXL_STAGE_A_PLAIN(BUF_, S_, DP_)                                                        \
   _Pragma("unroll") for (int kk = 0; kk < KK; kk++) {                                           \
@@ -470,6 +477,7 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
 #pragma unroll
       for (int r = 0; r < 16; r++) dp_e[r] = del_v[r / 4][r % 4];
     }
+    AXL_CHAIN_START(s_e, dp_e)
     AXL_STAGE_A_PLAIN(buf_b, s_e, dp_e)
     diff0 = (t_first * Tile::BQ + a.q_off + 8 * g) - kpos;
 #pragma unroll
@@ -484,6 +492,7 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
 #pragma unroll
       for (int r = 0; r < 16; r++) dp_e[r] = del_v[r / 4][r % 4];
     }
+    AXL_CHAIN_START(s_e, dp_e)
     AXL_STAGE_A_PLAIN(buf_e, s_e, dp_e)
     if constexpr (AUX) {                 // ... and of tile 1, for the first iteration
       const char* bp_;
@@ -749,6 +758,7 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
 #undef AXL_ELEM_3
 #undef AXL_PACK_PAIR
 #undef AXL_STAGE_A_PLAIN
+#undef AXL_CHAIN_START
 #undef AXL_B_READ_FROM
 #undef AXL_B_READ_AT
 #undef AXL_DMA

@@ -114,3 +114,37 @@ def check_function(lines, need_mfma=2, need_nops=12):
                     todo.append((labels[x.split()[1]], nm, nn))
                 pc += 1
     return bad
+
+
+def check_sources(lines, need=8):
+    """Every inline-assembly MFMA: none of its vector-register operands (the two factors and the addend)
+    is written by a vector ALU instruction within `need` wait states before it, counted back along the
+    instruction stream (labels are walked through as fall-through: a branch into the stretch can only
+    come from further away).  The hardware wants a distance between such a write and a matrix
+    instruction that reads the register; for its own MFMAs the compiler keeps it, behind a register that
+    assembly reads it does not.  Loads (LDS, global) are not meant here: the compiler waits for them
+    before the assembly statement that names their register.  Returns the violations."""
+    from_asm = [l.startswith("@") for l in lines]
+    lines = [l.lstrip("@") for l in lines]
+    bad = []
+    for i, ins in enumerate(lines):
+        if not from_asm[i] or not ins.startswith("v_mfma_"):
+            continue
+        ops = [o.strip() for o in ins.split(None, 1)[1].split(",")]
+        R = vregs(ops[1]) | vregs(ops[2]) | vregs(ops[3])
+        waited, j = 0, i - 1
+        while j >= 0 and waited < need:
+            x = lines[j]
+            j -= 1
+            if x.endswith(":"):
+                continue
+            op = x.split()[0]
+            if op == "s_nop":
+                waited += int(x.split()[1], 0) + 1
+                continue
+            if op.startswith("v_") and not op.startswith("v_mfma_") and not op.startswith("v_cmp"):
+                if vregs(x.split(None, 1)[1].split(",")[0]) & R:
+                    bad.append((i, ins, j + 1, x, waited))
+                    break
+            waited += 1
+    return bad

@@ -556,7 +556,8 @@ def _device_asm(source, extra=()):
 
 def _assert_asm_mfma_distances(asm, pattern, want_kernels):
     """Every inline-assembly MFMA chain of the kernels whose name matches `pattern`: 12 wait states
-    or two further MFMAs before anything else touches its registers, on every path."""
+    or two further MFMAs before anything else touches its registers, on every path; and no vector ALU
+    write to a register an inline-assembly MFMA reads within the 8 wait states before it."""
     import isa_hazards  # tests/isa_hazards.py (pytest puts the test directory on sys.path)
 
     checked = 0
@@ -566,6 +567,8 @@ def _assert_asm_mfma_distances(asm, pattern, want_kernels):
         chains = sum(1 for l in lines if l.startswith("@v_mfma_"))
         bad = isa_hazards.check_function(lines)
         assert not bad, f"{name}: {len(bad)} hazards, first {bad[0]}"
+        bad = isa_hazards.check_sources(lines)
+        assert not bad, f"{name}: {len(bad)} operands written right before their MFMA, first {bad[0]}"
         checked += chains > 0
     assert checked == want_kernels, checked
 
