@@ -22,7 +22,7 @@ BWD_DS_WORKSPACE = 1  # AXL_BWD_DS_WORKSPACE
 AXL_OK, AXL_ERR_INVALID_ARGUMENT, AXL_ERR_UNSUPPORTED, AXL_ERR_WORKSPACE, AXL_ERR_LAUNCH = 0, -1, -2, -3, -4
 
 
-ABI_VERSION = 6  # AXL_ATTN_ABI_VERSION of include/axl_attn.h these structures mirror
+ABI_VERSION = 7  # AXL_ATTN_ABI_VERSION of include/axl_attn.h these structures mirror
 
 
 class AxlError(RuntimeError):

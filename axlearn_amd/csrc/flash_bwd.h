@@ -24,6 +24,8 @@ struct BwdArgs {
                         // workgroups store (spill path under a sliding window or segment ids), or nullptr
   Strides3 qs, ks, vs, os, dos, dqs, dks, dvs;
   int B, T, S, Hq, Hkv;
+  int stat_hq;  // query heads of the [B, heads, T] statistics (ndelta, lse2): Hq, or more when the
+                // launch covers a slice of the heads and the pointers start at the slice's first head
   int mask_kind, window, q_off;
   float scale;
   int d_real;   // head_dim of the tensors: a multiple of 8, at most the compiled width (16-bit kernels without

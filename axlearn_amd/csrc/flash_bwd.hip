@@ -406,8 +406,15 @@ static bool spill_eligible(const AxlFlashBwdParams& p) {
          (!spill_ranged(p) || (p.kv_len / 128 <= kMaxKbRanged && (p.head_dim <= 64 || p.q_len % 256 == 0)));
 }
 
+// kv heads whose dS the workspace holds at a time (AXL_BWD_DS_SLICE_KV_HEADS in the flags; all of them
+// by default): the dK/dV and dQ kernels of the path run once per slice of that many kv heads.
+static int spill_slice_heads(const AxlFlashBwdParams& p) {
+  const int n = (p.flags >> 8) & 0xffff;
+  return n > 0 && n < p.num_kv_heads ? n : p.num_kv_heads;
+}
 static size_t spill_bytes(const AxlFlashBwdParams& p) {
-  return (size_t)p.batch * p.num_q_heads * (size_t)ds_blocks_per_head(p.q_len) * kDsBlockBytes;
+  const int heads = spill_slice_heads(p) * (p.num_q_heads / p.num_kv_heads);
+  return (size_t)p.batch * heads * (size_t)ds_blocks_per_head(p.q_len) * kDsBlockBytes;
 }
 
 // With segment ids: the table of per-group id ranges (seg_group_table_kernel), 256-byte rounded.
@@ -450,6 +457,7 @@ int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream)
   a.mask_kind = p.mask_kind; a.window = p.sliding_window; a.q_off = p.q_pos_offset;
   a.scale = p.softmax_scale;
   a.d_real = p.head_dim;
+  a.stat_hq = p.num_q_heads;
   {
     // Two key blocks per dK/dV workgroup under a causal mask, where a block and its mirror image see
     // complementary shares of the queries (an even number of blocks); AXL_DKDV_KB_PER_WG=1 in the
@@ -492,6 +500,10 @@ int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream)
     if (err == hipSuccess) err = launch_bwd_f32(a, width, phases, stream);
   } else if (spill) {
     // delta, then the dK/dV kernel (which leaves dS behind), then dq = scale * dS k.
+    if (spill_slice_heads(p) < p.num_kv_heads && (phases & AXL_BWD_DKDV) != 0 && (phases & AXL_BWD_DQ) == 0)
+      return set_error(AXL_ERR_UNSUPPORTED,
+                       "axl_flash_bwd_phases: with dS slices (AXL_BWD_DS_SLICE_KV_HEADS) a slice's dS lives only "
+                       "until the next slice's dK/dV kernel: run the DKDV and DQ phases in one call");
     if (phases & AXL_BWD_DELTA) {
       if (dt == AXL_BF16) {
         if (width == 128) AXL_LAUNCH((bwd_delta_kernel<__bf16, 128>), delta_grid, 0);
@@ -501,8 +513,26 @@ int launch_flash_bwd(const AxlFlashBwdParams& p, int phases, hipStream_t stream)
         else AXL_LAUNCH((bwd_delta_kernel<_Float16, 64>), delta_grid, 0);
       }
     }
-    if ((phases & AXL_BWD_DKDV) && err == hipSuccess) err = launch_bwd_dkdv(a, dt, width, false, stream);
-    if ((phases & AXL_BWD_DQ) && err == hipSuccess) err = launch_bwd_dq_stream(a, dt, width, stream);
+    // One slice of kv heads after the other: the kernels see a problem of that many heads (tensors
+    // and statistics offset to the slice's first head) and the same dS workspace.
+    const int slice = spill_slice_heads(p), G = p.num_q_heads / p.num_kv_heads, es = 2;
+    for (int h0 = 0; h0 < p.num_kv_heads && err == hipSuccess; h0 += slice) {
+      BwdArgs s = a;
+      s.Hkv = min(slice, p.num_kv_heads - h0);
+      s.Hq = s.Hkv * G;
+      const int64_t hq0 = (int64_t)h0 * G;
+      s.q = (const char*)a.q + hq0 * a.qs.h * es;
+      s.dout = (const char*)a.dout + hq0 * a.dos.h * es;
+      s.dq = (char*)a.dq + hq0 * a.dqs.h * es;
+      s.k = (const char*)a.k + h0 * a.ks.h * es;
+      s.v = (const char*)a.v + h0 * a.vs.h * es;
+      s.dk = (char*)a.dk + h0 * a.dks.h * es;
+      s.dv = (char*)a.dv + h0 * a.dvs.h * es;
+      s.ndelta = a.ndelta + hq0 * p.q_len;
+      s.lse2 = a.lse2 + hq0 * p.q_len;
+      if (phases & AXL_BWD_DKDV) err = launch_bwd_dkdv(s, dt, width, false, stream);
+      if ((phases & AXL_BWD_DQ) && err == hipSuccess) err = launch_bwd_dq_stream(s, dt, width, stream);
+    }
     phases &= AXL_BWD_DELTA;  // what is left for the code below: the sink gradient
     phases = (phases & AXL_BWD_DELTA) && p.d_logit_sink ? AXL_BWD_DELTA : 0;
     if (phases) {

@@ -197,7 +197,7 @@ void flash_bwd_dkdv_kernel(const BwdArgs a) {
   // the last head back to the first head of the tile before (dir < 0) or after it.
   const __bf16* q_src = (const __bf16*)a.q + b * a.qs.b + (int64_t)(hk * G) * a.qs.h + (int64_t)t_first * Tile::BQ * a.qs.s;
   const __bf16* d_src = (const __bf16*)a.dout + b * a.dos.b + (int64_t)(hk * G) * a.dos.h + (int64_t)t_first * Tile::BQ * a.dos.s;
-  const int64_t stat_row0 = ((int64_t)b * a.Hq + hk * G) * a.T + (int64_t)t_first * Tile::BQ;
+  const int64_t stat_row0 = ((int64_t)b * a.stat_hq + hk * G) * a.T + (int64_t)t_first * Tile::BQ;
   const bool s_is_seg = HAS_SEG && st_kind == 2;
   const char* s_src = st_kind == 1 ? (const char*)(a.ndelta + stat_row0) : (const char*)(a.lse2 + stat_row0);  // wave-uniform
   if (s_is_seg) s_src = (const char*)(a.seg + (int64_t)b * a.T + (int64_t)t_first * Tile::BQ);

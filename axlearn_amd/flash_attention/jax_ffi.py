@@ -84,9 +84,9 @@ def _mask_of(bias: BaseAttentionBias):
 
 # The backward can keep dS in its workspace where the library has that path (AXL_BWD_DS_WORKSPACE in
 # include/axl_attn.h: about T*S bytes per (batch, head) of scratch that XLA allocates for the call, for a
-# backward of 5 GEMMs instead of 7).  None: do so whenever that scratch fits BWD_WORKSPACE_LIMIT_BYTES
-# (the same rule as HipFlashAttention.Config.bwd_ds_workspace / bwd_workspace_limit_bytes on the torch
-# side); True / False force the choice.  The size query below sees the flag that was chosen, so the
+# backward of 5 GEMMs instead of 7).  None: do so whenever that scratch fits BWD_WORKSPACE_LIMIT_BYTES,
+# whole or a few kv heads at a time (the same rule as HipFlashAttention.Config.bwd_ds_workspace /
+# bwd_workspace_limit_bytes on the torch side, ops.select_ds_slice); True / False force the choice.  The size query below sees the flag that was chosen, so the
 # scratch result of the custom call grows with it.
 BWD_DS_WORKSPACE = None
 BWD_WORKSPACE_LIMIT_BYTES = 18 << 30  # a sixteenth of an MI355X's 288 GB
@@ -155,7 +155,14 @@ def _flash_bwd(softmax_scale, mask_kind, sliding_window, dropout_rate, logit_sin
     flags = _AXL_BWD_DS_WORKSPACE if BWD_DS_WORKSPACE or BWD_DS_WORKSPACE is None else 0
     ws_bytes = _bwd_workspace_bytes(*size_args, flags)
     if BWD_DS_WORKSPACE is None and flags and ws_bytes > BWD_WORKSPACE_LIMIT_BYTES:
-        flags = 0  # too large for the automatic choice: the recomputing pair
+        # Too large for the automatic choice in one piece: the dS of as many kv heads at a time as fit
+        # (AXL_BWD_DS_SLICE_KV_HEADS(n) = n << 8 in the flags; the kernels then run slice after slice),
+        # if a slice still gives each of the 256 CUs a dK/dV workgroup; else the recomputing pair.
+        per_head = b * (s // 128) // (2 if mask_kind == 1 else 1)   # AXL_MASK_CAUSAL: two key blocks per workgroup
+        heads = hkv - 1
+        while heads >= 1 and _bwd_workspace_bytes(*size_args, flags | (heads << 8)) > BWD_WORKSPACE_LIMIT_BYTES:
+            heads -= 1
+        flags = flags | (heads << 8) if heads >= 1 and heads * per_head >= 256 else 0
         ws_bytes = _bwd_workspace_bytes(*size_args, flags)
     dq, dk, dv, _, _ = jax.ffi.ffi_call(
         "AxlFlashBwd",

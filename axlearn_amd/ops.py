@@ -208,6 +208,7 @@ def flash_bwd(
     dropout_rate: float = 0.0,
     ds_workspace: Optional[bool] = False,
     ds_workspace_limit: Optional[int] = None,
+    ds_slice_kv_heads: int = 0,
 ):
     """Returns (dq [B,T,Hq,D], dk [B,S,Hkv,D], dv [B,S,Hkv,D]) in the dtype of q, followed by
     d_logit_sink [Hq] fp32 when `logit_sink` (the one the forward was given) is passed.
@@ -217,15 +218,19 @@ def flash_bwd(
     dropout_mask and dropout_rate must be the ones the forward was given (the bias gets no gradient,
     as in gpu_attention.py:786).  `ds_workspace=True` (AXL_BWD_DS_WORKSPACE; causal or sliding-window
     attention over equal lengths without offsets, bias or dropout; ignored otherwise) keeps dS in a
-    larger workspace instead of recomputing it for dq.  `ds_workspace=None` decides by size: the dS
+    larger workspace instead of recomputing it for dq; with `ds_slice_kv_heads=n` the workspace holds
+    the dS of n kv heads at a time and the two kernels run slice after slice
+    (AXL_BWD_DS_SLICE_KV_HEADS).  `ds_workspace=None` decides by size (`select_ds_slice`): the dS
     workspace is used when that path applies and fits `ds_workspace_limit` bytes (default:
-    `default_bwd_workspace_limit`, a sixteenth of the device's memory)."""
+    `default_bwd_workspace_limit`, a sixteenth of the device's memory), whole or in slices of kv
+    heads that still fill the GPU."""
     b, t, hq, d, s, hkv = _check_qkv(q, k, v)
     _check_segment_ids(segment_ids, b, t, s)
     if ds_workspace is None:
-        ds_workspace = (phases == 7 and bias is None and dropout_mask is None and q_pos_offset == 0
-                        and select_ds_workspace(q, k, mask_kind=mask_kind, segment_ids=segment_ids,
-                                                limit=ds_workspace_limit))
+        ds_workspace, ds_slice_kv_heads = False, 0
+        if phases == 7 and bias is None and dropout_mask is None and q_pos_offset == 0:
+            ds_workspace, ds_slice_kv_heads = select_ds_slice(q, k, mask_kind=mask_kind, segment_ids=segment_ids,
+                                                              limit=ds_workspace_limit)
     _want_shape("out", out, q.shape)
     _want_shape("d_out", d_out, q.shape)
     _want_shape("lse", lse, (b, hq, t))
@@ -263,7 +268,7 @@ def flash_bwd(
         dtype=_lib.dtype_code(q.dtype), mask_kind=mask_kind, sliding_window=int(sliding_window),
         q_pos_offset=int(q_pos_offset), softmax_scale=float(softmax_scale),
         workspace=None, workspace_bytes=0, logit_sink=_lib.ptr(sink), d_logit_sink=_lib.ptr(d_sink),
-        aux=aux, flags=_lib.BWD_DS_WORKSPACE if ds_workspace else 0,
+        aux=aux, flags=_bwd_flags(ds_workspace, ds_slice_kv_heads),
     )
     need = int(lib.axl_flash_bwd_workspace_bytes(ctypes.byref(p)))
     if ws is None:
@@ -278,32 +283,45 @@ def flash_bwd(
     return dq, dk, dv
 
 
+def _bwd_flags(ds_workspace: bool, ds_slice_kv_heads: int = 0) -> int:
+    if not ds_workspace:
+        return 0
+    if not 0 <= int(ds_slice_kv_heads) < 65536:
+        raise _bad(f"ds_slice_kv_heads must be in [0, 65535], got {ds_slice_kv_heads}")
+    return _lib.BWD_DS_WORKSPACE | (int(ds_slice_kv_heads) << 8)  # AXL_BWD_DS_SLICE_KV_HEADS(n)
+
+
 def flash_bwd_buffers(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, *, mask_kind: int = MASK_NONE,
-                      ds_workspace: bool = False, segment_ids: Optional[torch.Tensor] = None):
+                      ds_workspace: bool = False, segment_ids: Optional[torch.Tensor] = None,
+                      ds_slice_kv_heads: int = 0):
     """Pre-allocates (dq, dk, dv, workspace) for repeated `flash_bwd(..., buffers=...)` calls.
 
     The workspace holds delta and the scaled lse (fp32 [B,Hq,T] each); with `segment_ids` (the ones the
     calls will pass) also the table of id ranges per 32 rows; with `ds_workspace=True` and a causal or
     sliding-window `mask_kind` (equal lengths, no offsets / bias / dropout) also dS, about T*S bytes per
-    (batch, head), for `flash_bwd(..., ds_workspace=True)`."""
+    (batch, head), for `flash_bwd(..., ds_workspace=True)` - of `ds_slice_kv_heads` kv heads at a time if that
+    is given (the calls must pass the same number)."""
     b, t, hq, d = q.shape
     p = AxlFlashBwdParams(batch=b, q_len=t, kv_len=k.shape[1], num_q_heads=hq, num_kv_heads=k.shape[2],
                           head_dim=d, dtype=_lib.dtype_code(q.dtype), mask_kind=mask_kind,
                           segment_ids=_lib.ptr(_seg(segment_ids)),
-                          flags=_lib.BWD_DS_WORKSPACE if ds_workspace else 0)
+                          flags=_bwd_flags(ds_workspace, ds_slice_kv_heads))
     nbytes = int(_lib.load().axl_flash_bwd_workspace_bytes(ctypes.byref(p)))
     ws = torch.empty((max(nbytes, 256),), dtype=torch.uint8, device=q.device)
     return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), ws
 
 
 def flash_bwd_ds_workspace_bytes(q: torch.Tensor, k: torch.Tensor, *, mask_kind: int,
-                                 segment_ids: Optional[torch.Tensor] = None) -> Tuple[int, int]:
+                                 segment_ids: Optional[torch.Tensor] = None,
+                                 ds_slice_kv_heads: int = 0) -> Tuple[int, int]:
     """(bytes with AXL_BWD_DS_WORKSPACE, bytes without) of backward workspace for these shapes and
-    this mask; the two are equal where the dS-workspace path does not apply (the flag is ignored)."""
+    this mask; the two are equal where the dS-workspace path does not apply (the flag is ignored).
+    `ds_slice_kv_heads`: with the dS of that many kv heads at a time (0: all)."""
     b, t, hq, d = q.shape
     p = AxlFlashBwdParams(batch=b, q_len=t, kv_len=k.shape[1], num_q_heads=hq, num_kv_heads=k.shape[2],
                           head_dim=d, dtype=_lib.dtype_code(q.dtype), mask_kind=mask_kind,
-                          segment_ids=None if segment_ids is None else 256, flags=_lib.BWD_DS_WORKSPACE)
+                          segment_ids=None if segment_ids is None else 256,
+                          flags=_bwd_flags(True, ds_slice_kv_heads))
     lib = _lib.load()
     with_ds = int(lib.axl_flash_bwd_workspace_bytes(ctypes.byref(p)))
     p.flags = 0
@@ -316,16 +334,36 @@ def default_bwd_workspace_limit(device) -> int:
     return torch.cuda.get_device_properties(device).total_memory // 16
 
 
-def select_ds_workspace(q: torch.Tensor, k: torch.Tensor, *, mask_kind: int,
-                        segment_ids: Optional[torch.Tensor] = None, limit: Optional[int] = None) -> bool:
-    """The backward's default policy: keep dS in the workspace (5 executed GEMMs instead of 7) when
-    that path applies to these shapes and its workspace fits `limit` bytes."""
+def select_ds_slice(q: torch.Tensor, k: torch.Tensor, *, mask_kind: int,
+                    segment_ids: Optional[torch.Tensor] = None, limit: Optional[int] = None) -> Tuple[bool, int]:
+    """The backward's default policy, as (ds_workspace, ds_slice_kv_heads): keep dS in the workspace (5
+    executed GEMMs instead of 7) when that path applies to these shapes and its workspace fits `limit`
+    bytes - whole (slice 0), or of as many kv heads at a time as fit, provided a slice still gives every
+    CU a dK/dV workgroup (batch * heads * kv_len / 256 of them under a causal mask, twice that under a
+    window); else the recomputing pair."""
     with_ds, without = flash_bwd_ds_workspace_bytes(q, k, mask_kind=mask_kind, segment_ids=segment_ids)
     if with_ds == without:
-        return False
+        return False, 0
     if limit is None:
         limit = default_bwd_workspace_limit(q.device)
-    return with_ds <= int(limit)
+    if with_ds <= int(limit):
+        return True, 0
+    b, hkv, s = q.shape[0], k.shape[2], k.shape[1]
+    heads = min(hkv - 1, (int(limit) - without) * hkv // (with_ds - without) + 1)   # kv heads whose dS fits
+    while heads >= 1 and flash_bwd_ds_workspace_bytes(q, k, mask_kind=mask_kind, segment_ids=segment_ids,
+                                                      ds_slice_kv_heads=heads)[0] > int(limit):
+        heads -= 1
+    per_head = b * (s // 128) // (2 if mask_kind == MASK_CAUSAL else 1)   # dK/dV workgroups per kv head
+    cus = torch.cuda.get_device_properties(q.device).multi_processor_count
+    if heads < 1 or heads * per_head < cus:
+        return False, 0
+    return True, int(heads)
+
+
+def select_ds_workspace(q: torch.Tensor, k: torch.Tensor, *, mask_kind: int,
+                        segment_ids: Optional[torch.Tensor] = None, limit: Optional[int] = None) -> bool:
+    """Whether `select_ds_slice` takes the dS workspace for these shapes (whole or in slices)."""
+    return select_ds_slice(q, k, mask_kind=mask_kind, segment_ids=segment_ids, limit=limit)[0]
 
 
 def _decode_flags(deterministic: bool, workspace_reused: bool) -> int:

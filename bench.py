@@ -171,7 +171,8 @@ def bench_flash(cfg, steps, warmup, cpu_baseline):
     """One fwd+bwd step = what a caller of `flash_attention_implementation("gpu", ...)` gets: the
     returned kernel object applied to the batch, then autograd's backward with a given dO.
     cfg["ds_workspace"]: None = the plugin's default (dS workspace when it fits the default limit, a
-    sixteenth of the device's memory), True / False = forced through backend_overrides."""
+    sixteenth of the device's memory - whole, or the dS of a few kv heads at a time), True / False =
+    forced through backend_overrides (True: the whole dS at once)."""
     from axlearn_amd import ops
     from axlearn_amd.flash_attention.utils import flash_attention_implementation
 
@@ -189,13 +190,15 @@ def bench_flash(cfg, steps, warmup, cpu_baseline):
         pairs = count_pairs(seg, cfg["window"])
     mask_kind = {"none": ops.MASK_NONE, "causal": ops.MASK_CAUSAL, "sliding": ops.MASK_SLIDING_WINDOW}[cfg["mask"]]
     forced = cfg.get("ds_workspace")
+    slice_heads = 0   # kv heads whose dS the workspace holds at a time (0: all)
     if forced is None:
-        spill = ops.select_ds_workspace(q, k, mask_kind=mask_kind, segment_ids=seg)
+        spill, slice_heads = ops.select_ds_slice(q, k, mask_kind=mask_kind, segment_ids=seg)
         chosen = "default config (by workspace size)"
     else:
         spill = bool(forced)
         chosen = f"backend_overrides bwd_ds_workspace={spill}"
-    ws_need, _ = ops.flash_bwd_ds_workspace_bytes(q, k, mask_kind=mask_kind, segment_ids=seg)
+    ws_need, _ = ops.flash_bwd_ds_workspace_bytes(q, k, mask_kind=mask_kind, segment_ids=seg,
+                                                  ds_slice_kv_heads=slice_heads)
     bias = _dispatch_bias(cfg, seg, T, dev)
     impl = flash_attention_implementation(
         "gpu", query=q, key=k, value=v, bias=bias, softmax_scale=D ** -0.5,
@@ -214,8 +217,9 @@ def bench_flash(cfg, steps, warmup, cpu_baseline):
     # The same kernels through the C ABI with buffers allocated once (no allocator, no autograd).
     qd, kd, vd = q.detach(), k.detach(), v.detach()
     kw = dict(softmax_scale=D ** -0.5, mask_kind=mask_kind, sliding_window=cfg["window"], segment_ids=seg)
-    bufs = ops.flash_bwd_buffers(qd, kd, vd, mask_kind=mask_kind, ds_workspace=spill, segment_ids=seg)
-    kw_b = dict(kw, ds_workspace=spill)
+    bufs = ops.flash_bwd_buffers(qd, kd, vd, mask_kind=mask_kind, ds_workspace=spill, segment_ids=seg,
+                                 ds_slice_kv_heads=slice_heads)
+    kw_b = dict(kw, ds_workspace=spill, ds_slice_kv_heads=slice_heads)
     out, lse = ops.flash_fwd(qd, kd, vd, **kw)
 
     def abi_step():
@@ -227,8 +231,26 @@ def bench_flash(cfg, steps, warmup, cpu_baseline):
     # launches go to).  With the dS workspace the dq phase reads what the dK/dV phase before it left.
     ms_fwd = _time_region(lambda: ops.flash_fwd(qd, kd, vd, **kw), steps, 1)
     ms_delta = _time_region(lambda: ops.flash_bwd(qd, kd, vd, out, lse, do, buffers=bufs, phases=1, **kw_b), steps, 1)
-    ms_dkdv = _time_region(lambda: ops.flash_bwd(qd, kd, vd, out, lse, do, buffers=bufs, phases=2, **kw_b), steps, 1)
-    ms_dq = _time_region(lambda: ops.flash_bwd(qd, kd, vd, out, lse, do, buffers=bufs, phases=4, **kw_b), steps, 1)
+    n_slices = 1
+    if slice_heads:
+        # The dK/dV and dQ kernels run once per slice of kv heads, every launch on the same amount of work:
+        # one slice's launch of each is timed on its own (the first slice's heads as a problem of their
+        # own, which is what the library enqueues), the step holds n_slices of them.
+        n_slices = -(-Hkv // slice_heads)
+        hq_s = slice_heads * (Hq // Hkv)
+        qs, ks, vs, dos, outs = qd[:, :, :hq_s], kd[:, :, :slice_heads], vd[:, :, :slice_heads], do[:, :, :hq_s], out[:, :, :hq_s]
+        lses = lse[:, :hq_s].contiguous()
+        kw_s = dict(kw, ds_workspace=True)
+        bufs_s = ops.flash_bwd_buffers(qs, ks, vs, mask_kind=mask_kind, ds_workspace=True, segment_ids=seg)
+        ops.flash_bwd(qs, ks, vs, outs, lses, dos, buffers=bufs_s, **kw_s)
+        ms_dkdv = n_slices * _time_region(
+            lambda: ops.flash_bwd(qs, ks, vs, outs, lses, dos, buffers=bufs_s, phases=2, **kw_s), steps, 1)
+        ms_dq = n_slices * _time_region(
+            lambda: ops.flash_bwd(qs, ks, vs, outs, lses, dos, buffers=bufs_s, phases=4, **kw_s), steps, 1)
+        del bufs_s
+    else:
+        ms_dkdv = _time_region(lambda: ops.flash_bwd(qd, kd, vd, out, lse, do, buffers=bufs, phases=2, **kw_b), steps, 1)
+        ms_dq = _time_region(lambda: ops.flash_bwd(qd, kd, vd, out, lse, do, buffers=bufs, phases=4, **kw_b), steps, 1)
 
     if pairs is None:
         gemm = 2.0 * B * Hq * (T * T / 2.0) * D  # one [T,T,D] causal GEMM (the 1/2 convention)
@@ -242,8 +264,10 @@ def bench_flash(cfg, steps, warmup, cpu_baseline):
     result = dict(
         workload=cfg["label"], value=tf(fl_fwd + fl_bwd, ms_step), unit="TFLOP/s", ms_per_step=ms_step,
         entry="flash_attention_implementation('gpu', ...).fn(batch) + torch.autograd.grad(out, (q, k, v), dO)",
-        backward="dS workspace: delta, dK/dV (stores dS), dq = dS k" if spill else "dQ (recomputes dS, computes delta), dK/dV",
-        backward_chosen_by=chosen, ds_workspace_bytes=ws_need if spill else 0,
+        backward=("dS workspace: delta, dK/dV (stores dS), dq = dS k"
+                  + (f", the last two once per slice of {slice_heads} kv heads ({n_slices} slices)" if slice_heads else "")
+                  if spill else "dQ (recomputes dS, computes delta), dK/dV"),
+        backward_chosen_by=chosen, ds_workspace_bytes=ws_need if spill else 0, ds_slice_kv_heads=slice_heads,
         c_abi_ms_per_step=ms_abi,
         kernels={
             "flash_fwd_kernel": dict(ms=ms_fwd, tflops=tf(fl_fwd, ms_fwd), algorithmic_tflop=fl_fwd / 1e12),

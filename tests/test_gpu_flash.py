@@ -10,7 +10,7 @@ import pytest
 import torch
 
 from axlearn_amd import attention_bias as ab
-from axlearn_amd import ops
+from axlearn_amd import _lib, ops
 from axlearn_amd.flash_attention.hip_attention import HipFlashAttention, flash_attention
 from axlearn_amd.flash_attention.utils import flash_attention_implementation
 from oracle import brute
@@ -1018,6 +1018,47 @@ def test_ds_workspace_sweep_against_the_recomputing_path(seed):
     for name, x, y in (("dq", dq, bq), ("dk", dk, bk)):
         assert torch.isfinite(x.float()).all(), f"{name} {case}"
         assert ref.rel_l2(x.cpu(), y.cpu().float()) < 1e-4, f"{name} {case}: {ref.rel_l2(x.cpu(), y.cpu().float()):.3e}"
+
+
+@pytest.mark.parametrize("b,t,hq,hkv,d,kind,window,packed", [
+    (2, 512, 8, 4, 128, "causal", None, False),
+    (1, 768, 6, 3, 64, "causal", None, True),
+    (2, 512, 4, 4, 128, "sliding", 200, True),
+    (1, 1024, 10, 5, 64, "sliding", 77, False),
+])
+def test_ds_workspace_in_slices_of_kv_heads_is_bit_identical(b, t, hq, hkv, d, kind, window, packed):
+    """AXL_BWD_DS_SLICE_KV_HEADS: the workspace holds the dS of n kv heads at a time and the dK/dV and dQ
+    kernels run slice after slice (every n from 1 to hkv - 1, so uneven last slices too).  A slice's
+    kernels do what the whole launch does for those heads, so dq, dk and dv are bit-identical to the
+    unsliced path; the workspace shrinks by the dS of the heads left out; the dK/dV phase without the
+    dQ phase is refused (the next slice would overwrite what it left); the automatic choice takes the
+    largest slice that fits its limit, or the recomputing pair when a slice would not fill the GPU."""
+    q, k, v, do = (x.cuda() for x in _inputs(b, t, hq, hkv, d, torch.bfloat16))
+    segs = ref.packed_segment_ids(7, b, t).cuda() if packed else None
+    mk = ops.MASK_CAUSAL if kind == "causal" else ops.MASK_SLIDING_WINDOW
+    kw = dict(mask_kind=mk, sliding_window=window or 0, softmax_scale=d ** -0.5, segment_ids=segs)
+    out, lse = ops.flash_fwd(q, k, v, **kw)
+    whole = ops.flash_bwd(q, k, v, out, lse, do, ds_workspace=True, **kw)
+    full, plain = ops.flash_bwd_ds_workspace_bytes(q, k, mask_kind=mk, segment_ids=segs)
+    for n in range(1, hkv):
+        need, _ = ops.flash_bwd_ds_workspace_bytes(q, k, mask_kind=mk, segment_ids=segs, ds_slice_kv_heads=n)
+        assert abs((need - plain) - (full - plain) * n // hkv) <= 512, n   # dS of n heads (+ the table of stored tiles)
+        bufs = ops.flash_bwd_buffers(q, k, v, mask_kind=mk, ds_workspace=True, segment_ids=segs, ds_slice_kv_heads=n)
+        assert bufs[3].numel() == max(need, 256)
+        bufs[3].fill_(0xff)
+        got = ops.flash_bwd(q, k, v, out, lse, do, ds_workspace=True, ds_slice_kv_heads=n, buffers=bufs, **kw)
+        for name, x, y in zip(("dq", "dk", "dv"), got, whole):
+            assert torch.equal(x, y), f"{name} with slices of {n}"
+        with pytest.raises(ops.AxlError) as err:
+            ops.flash_bwd(q, k, v, out, lse, do, ds_workspace=True, ds_slice_kv_heads=n, buffers=bufs, phases=2, **kw)
+        assert err.value.code == _lib.AXL_ERR_UNSUPPORTED
+    # the automatic choice: whole where it fits; slices where they fit and fill the CUs; else recompute
+    assert ops.select_ds_slice(q, k, mask_kind=mk, segment_ids=segs, limit=full) == (True, 0)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    per_head = b * (t // 128) // (2 if kind == "causal" else 1)
+    use, n = ops.select_ds_slice(q, k, mask_kind=mk, segment_ids=segs, limit=full - 1)
+    assert (use, n) == ((True, hkv - 1) if (hkv - 1) * per_head >= cus else (False, 0))
+    assert ops.select_ds_slice(q, k, mask_kind=mk, segment_ids=segs, limit=plain) == (False, 0)
 
 
 def test_layer_compute_attention_end_to_end():

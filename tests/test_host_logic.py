@@ -356,6 +356,14 @@ def test_abi_validation_without_gpu():
     # plain causal attention with the dS workspace: A = T / 128 = 2 -> 8 A (A + 1) blocks of 2 KB per head
     bp.flags = _lib.BWD_DS_WORKSPACE
     assert lib.axl_flash_bwd_workspace_bytes(ctypes.byref(bp)) == stats + 2 * 4 * 48 * 2048
+    # ... of one of the two kv heads (2 query heads each) at a time: half of that; 2 or more heads is all of them
+    bp.flags = _lib.BWD_DS_WORKSPACE | (1 << 8)   # AXL_BWD_DS_SLICE_KV_HEADS(1)
+    assert lib.axl_flash_bwd_workspace_bytes(ctypes.byref(bp)) == stats + 2 * 2 * 48 * 2048
+    bp.flags = _lib.BWD_DS_WORKSPACE | (2 << 8)
+    assert lib.axl_flash_bwd_workspace_bytes(ctypes.byref(bp)) == stats + 2 * 4 * 48 * 2048
+    bp.flags = 1 << 8                             # without AXL_BWD_DS_WORKSPACE the slice count means nothing
+    assert lib.axl_flash_bwd_workspace_bytes(ctypes.byref(bp)) == stats
+    bp.flags = _lib.BWD_DS_WORKSPACE
     # under a sliding window (or with segment ids): also which query tiles each 128-key block stored,
     # [B, S / 128] pairs of int32, rounded to 256 bytes
     bp.mask_kind = 2

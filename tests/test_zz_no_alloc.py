@@ -6,6 +6,7 @@ max-abs arm says nothing about outputs this small) otherwise.  Two calls in a ro
 stale records, table entries and counters of the first call must not leak into the second."""
 
 import ctypes
+import gc
 
 import pytest
 import torch
@@ -71,7 +72,10 @@ def test_static_scratch_decode_matches_workspace_decode():
                 resolved = True
             torch.cuda.synchronize()
             # "allocates nothing": neither through torch's caching allocator nor behind its back (the
-            # driver's count of free device memory, which a hipMalloc / hipFree inside the library moves)
+            # driver's count of free device memory, which a hipMalloc / hipFree inside the library moves).
+            # Garbage that earlier tests left in reference cycles goes first: the collector would otherwise
+            # be free to return its tensors in the middle of the measured call.
+            gc.collect()
             before, free_before = torch.cuda.memory_allocated(dev), torch.cuda.mem_get_info(dev)[0]
             _lib.check(lib.axl_paged_decode_static(ctypes.byref(ps), stream))
             torch.cuda.synchronize()
