@@ -8,54 +8,95 @@
 //   dp = dO v^T, zeroed where dropped and scaled by 1/(1-rate)   (:508-512, :600-603)
 //   ds = p * (dp - delta)                                   (:514, :604)
 //   dv += (p after dropout)^T dO,  dk += scale * ds^T q,  dq += scale * ds k   (:513, :518, :608)
-// This path is for parity, not speed: tiles are staged through LDS by ordinary loads, one 32-row
-// tile per step, nothing is pipelined.  The mapping is the forward's (flash_fwd.hip, fp32 kernel):
-// an accumulator register r of lane (l32, g) is row 8(r/4) + 4g + (r%4), column l32, so a product
-// whose reduction runs over the accumulator's rows takes register r itself as the B operand of
-// MFMA r ("one reduction index per lane group per MFMA").
+//
+// A workgroup of 4 wavefronts owns 128 rows (queries in the dQ kernel, keys in the dK/dV kernel), 32
+// per wavefront, one wavefront per SIMD.  A lane keeps the half of its own row that its MFMAs read
+// (elements 2 d2 + g of the row: the fp32 matrix instruction takes one element per lane and step) in
+// registers for the whole kernel, next to the fp32 accumulators (the dK/dV kernel, whose two accumulator
+// sets leave less room, keeps its V rows in LDS instead); the 32-row tiles it loops over come
+// through a double-buffered LDS copy whose next tile is on its way from global memory while the
+// current one is multiplied, with one barrier per tile.  The mapping is the forward's (flash_fwd.hip,
+// fp32 kernel): an accumulator register r of lane (l32, g) is row 8(r/4) + 4g + (r%4), column l32, so
+// a product whose reduction runs over the accumulator's rows takes register r itself as the B operand
+// of MFMA r ("one reduction index per lane group per MFMA").
 #include "flash_bwd.h"
 
 namespace axl {
 
 template <int D>
 struct BwdTileF32 {
-  static constexpr int ROWS = 64;              // rows owned by a workgroup (2 wavefronts x 32)
+  static constexpr int NT = 256;               // threads of a workgroup
+  static constexpr int ROWS = 128;             // rows owned by a workgroup (4 wavefronts x 32)
   static constexpr int TILE = 32;              // rows of the tiles it loops over
   static constexpr int PS = D + 1;             // words per LDS row: lanes read a column of rows
-  static constexpr int LDS_BYTES = (2 * ROWS + 2 * TILE) * PS * 4 + 2 * TILE * 4;
+  static constexpr int TILE_WORDS = TILE * PS;
+  static constexpr int BUF_WORDS = 2 * TILE_WORDS + 2 * TILE;   // two tensors' tiles, two rows of statistics
+  static constexpr int LDS_BYTES = 2 * BUF_WORDS * 4;
+  static constexpr int OWN_WORDS = ROWS * PS;                   // one owned tensor kept in LDS (dK/dV kernel: V)
+  static constexpr int LDS_BYTES_DKDV = LDS_BYTES + OWN_WORDS * 4;
+  static constexpr int LD4 = TILE * (D / 4) / NT;               // float4 loads per thread and tensor tile
+  static_assert(TILE * (D / 4) % NT == 0, "a tile divides evenly over the threads");
+  static_assert(4 * TILE_WORDS <= 2 * BUF_WORDS, "the owned rows pass through the ring, 128 at a time");
 };
-
-// rows x D floats from global (row stride `stride` elements) into LDS rows of PS words.
-template <int D, int NT>
-__device__ __forceinline__ void stage_rows(float* lds, const float* src, int64_t stride, int rows, int tid) {
-  constexpr int PS = D + 1;
-  for (int i = tid; i < rows * (D / 4); i += NT) {
-    const int row = i / (D / 4), c4 = i % (D / 4);
-    const float4 x = *(const float4*)(src + (int64_t)row * stride + c4 * 4);
-    float* dst = lds + row * PS + c4 * 4;
-    dst[0] = x.x; dst[1] = x.y; dst[2] = x.z; dst[3] = x.w;
-  }
-}
 
 __device__ __forceinline__ float bias_at(const AuxArgs& x, const char* row, int col) {
   if (x.bias_f32) return *(const float*)(row + (int64_t)col * 4);
   return (float)*(const __bf16*)(row + (int64_t)col * 2);
 }
 
+// The 32 x D tile at `src` (row stride `stride` elements) into this thread's registers, and from there
+// into LDS rows of PS words.
+template <int D>
+__device__ __forceinline__ void tile_request(float4 (&x)[BwdTileF32<D>::LD4], const float* src, int64_t stride, int tid) {
+  using Tile = BwdTileF32<D>;
+#pragma unroll
+  for (int i = 0; i < Tile::LD4; i++) {
+    const int e = tid + i * Tile::NT, row = e / (D / 4), c4 = e % (D / 4);
+    x[i] = *(const float4*)(src + (int64_t)row * stride + c4 * 4);
+  }
+}
+template <int D>
+__device__ __forceinline__ void tile_deposit(float* lds, const float4 (&x)[BwdTileF32<D>::LD4], int tid) {
+  using Tile = BwdTileF32<D>;
+#pragma unroll
+  for (int i = 0; i < Tile::LD4; i++) {
+    const int e = tid + i * Tile::NT, row = e / (D / 4), c4 = e % (D / 4);
+    float* dst = lds + row * Tile::PS + c4 * 4;
+    dst[0] = x[i].x; dst[1] = x[i].y; dst[2] = x[i].z; dst[3] = x[i].w;
+  }
+}
+
+// The workgroup's 128 owned rows of one tensor pass through LDS once (`lds`: 128 rows of PS words) and
+// every lane keeps elements 2 d2 + g of its row.  Called by all threads; contains barriers.
+template <int D>
+__device__ __forceinline__ void own_rows(float (&mine)[D / 2], float* lds, const float* src, int64_t stride, int tid) {
+  using Tile = BwdTileF32<D>;
+  __syncthreads();  // whoever read this memory before is done
+  for (int i = tid; i < Tile::ROWS * (D / 4); i += Tile::NT) {
+    const int row = i / (D / 4), c4 = i % (D / 4);
+    const float4 x = *(const float4*)(src + (int64_t)row * stride + c4 * 4);
+    float* dst = lds + row * Tile::PS + c4 * 4;
+    dst[0] = x.x; dst[1] = x.y; dst[2] = x.z; dst[3] = x.w;
+  }
+  __syncthreads();
+  const int lane = tid & 63, g = lane >> 5;
+  const float* row = lds + ((tid >> 6) * 32 + (lane & 31)) * Tile::PS;
+#pragma unroll
+  for (int d2 = 0; d2 < D / 2; d2++) mine[d2] = row[2 * d2 + g];
+}
+
 // ---------------------------------------------------------------------------------------------
-// dQ: a workgroup owns 64 query rows of one head and loops over 32-key tiles.
+// dQ: a workgroup owns 128 query rows of one head and loops over 32-key tiles.
 //   S^T[key][q] = K Q^T and dP^T[key][q] = V dO^T (A = K / V row l32, B = Q / dO row l32), so lane
 //   (l32, g) holds query l32 and keys 8(r/4) + 4g + (r%4); dQ^T[d][q] += K^T[d][key] dS^T[key][q].
 // ---------------------------------------------------------------------------------------------
 template <int D>
-__global__ __launch_bounds__(128) void flash_bwd_dq_f32_kernel(const BwdArgs a) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void flash_bwd_dq_f32_kernel(const BwdArgs a) {
   using Tile = BwdTileF32<D>;
   constexpr int DT = D / 32, PS = Tile::PS;
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  float* const q_lds = (float*)smem;
-  float* const do_lds = q_lds + Tile::ROWS * PS;
-  float* const k_lds = do_lds + Tile::ROWS * PS;
-  float* const v_lds = k_lds + Tile::TILE * PS;
+  float* const ring = (float*)smem;
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
@@ -65,10 +106,9 @@ __global__ __launch_bounds__(128) void flash_bwd_dq_f32_kernel(const BwdArgs a) 
   const int hk = h / (a.Hq / a.Hkv);
   const int q0_wg = qb * Tile::ROWS, q0 = q0_wg + wave * 32;
 
-  stage_rows<D, 128>(q_lds, (const float*)a.q + b * a.qs.b + (int64_t)q0_wg * a.qs.s + h * a.qs.h, a.qs.s,
-                     Tile::ROWS, tid);
-  stage_rows<D, 128>(do_lds, (const float*)a.dout + b * a.dos.b + (int64_t)q0_wg * a.dos.s + h * a.dos.h, a.dos.s,
-                     Tile::ROWS, tid);
+  float q_mine[D / 2], do_mine[D / 2];
+  own_rows<D>(q_mine, ring, (const float*)a.q + b * a.qs.b + (int64_t)q0_wg * a.qs.s + h * a.qs.h, a.qs.s, tid);
+  own_rows<D>(do_mine, ring, (const float*)a.dout + b * a.dos.b + (int64_t)q0_wg * a.dos.s + h * a.dos.h, a.dos.s, tid);
   const float* kp = (const float*)a.k + b * a.ks.b + hk * a.ks.h;
   const float* vp = (const float*)a.v + b * a.vs.b + hk * a.vs.h;
   const int64_t stat = ((int64_t)b * a.Hq + h) * a.T + q0 + l32;
@@ -95,55 +135,74 @@ __global__ __launch_bounds__(128) void flash_bwd_dq_f32_kernel(const BwdArgs a) 
   for (int i = 0; i < DT; i++)
 #pragma unroll
     for (int r = 0; r < 16; r++) dq[i][r] = 0.f;
-  const float* q_row = q_lds + (wave * 32 + l32) * PS;
-  const float* do_row = do_lds + (wave * 32 + l32) * PS;
 
+  // Tile t lives in ring buffer t % 2: K rows, then V rows.
+  float4 kx[Tile::LD4], vx[Tile::LD4];
+  __syncthreads();  // the owned rows have been read out of the ring
+  if (t_begin < t_end) {
+    tile_request<D>(kx, kp + (int64_t)t_begin * Tile::TILE * a.ks.s, a.ks.s, tid);
+    tile_request<D>(vx, vp + (int64_t)t_begin * Tile::TILE * a.vs.s, a.vs.s, tid);
+    float* buf = ring + (t_begin & 1) * Tile::BUF_WORDS;
+    tile_deposit<D>(buf, kx, tid);
+    tile_deposit<D>(buf + Tile::TILE_WORDS, vx, tid);
+  }
+  __syncthreads();
   for (int t = t_begin; t < t_end; t++) {
     const int k0 = t * Tile::TILE;
-    __syncthreads();  // previous tile consumed (and Q, dO staged on the first pass)
-    stage_rows<D, 128>(k_lds, kp + (int64_t)k0 * a.ks.s, a.ks.s, Tile::TILE, tid);
-    stage_rows<D, 128>(v_lds, vp + (int64_t)k0 * a.vs.s, a.vs.s, Tile::TILE, tid);
-    __syncthreads();
+    const bool more = t + 1 < t_end;
+    if (more) {  // the next tile's round trip runs under this tile's MFMAs
+      tile_request<D>(kx, kp + (int64_t)(k0 + Tile::TILE) * a.ks.s, a.ks.s, tid);
+      tile_request<D>(vx, vp + (int64_t)(k0 + Tile::TILE) * a.vs.s, a.vs.s, tid);
+    }
+    const float* k_lds = ring + (t & 1) * Tile::BUF_WORDS;
+    const float* v_lds = k_lds + Tile::TILE_WORDS;
     bool skip = false;
     if (a.mask_kind != AXL_MASK_NONE) {
       skip = k0 > qpos_max;
       if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) skip = skip || (qpos_min - (k0 + Tile::TILE - 1) > a.window);
     }
-    if (skip) continue;
-    floatx16 s, dp;
+    if (!skip) {
+      floatx16 s, dp;
 #pragma unroll
-    for (int r = 0; r < 16; r++) s[r] = dp[r] = 0.f;
-    const float* k_row = k_lds + l32 * PS;
-    const float* v_row = v_lds + l32 * PS;
-#pragma unroll 8
-    for (int d2 = 0; d2 < D / 2; d2++) {
-      s = __builtin_amdgcn_mfma_f32_32x32x2f32(k_row[2 * d2 + g], q_row[2 * d2 + g], s, 0, 0, 0);
-      dp = __builtin_amdgcn_mfma_f32_32x32x2f32(v_row[2 * d2 + g], do_row[2 * d2 + g], dp, 0, 0, 0);
-    }
+      for (int r = 0; r < 16; r++) s[r] = dp[r] = 0.f;
+      const float* k_row = k_lds + l32 * PS;
+      const float* v_row = v_lds + l32 * PS;
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-      const int kpos = k0 + 8 * (r / 4) + 4 * g + (r % 4);
-      bool keep = true;
-      if (a.mask_kind != AXL_MASK_NONE) {
-        const int diff = qpos - kpos;
-        keep = diff >= 0;
-        if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) keep = keep && diff <= a.window;
+      for (int d2 = 0; d2 < D / 2; d2++) {
+        s = __builtin_amdgcn_mfma_f32_32x32x2f32(k_row[2 * d2 + g], q_mine[d2], s, 0, 0, 0);
+        dp = __builtin_amdgcn_mfma_f32_32x32x2f32(v_row[2 * d2 + g], do_mine[d2], dp, 0, 0, 0);
       }
-      if (seg_k) keep = keep && (seg_k[kpos] == seg_q);
-      float logit = s[r] * a.scale;
-      if (bias_row) logit += bias_at(a.aux, bias_row, kpos);
-      const float p = keep ? expf(logit - lse_q) : 0.f;
-      float dpe = dp[r];
-      if (drop_row) dpe = drop_row[kpos] ? 0.f : dpe * a.aux.keep_scale;
-      s[r] = p * (dpe - delta_q);  // dS^T
-    }
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-      const float* k_col = k_lds + (8 * (r / 4) + 4 * g + (r % 4)) * PS + l32;
+      for (int r = 0; r < 16; r++) {
+        const int kpos = k0 + 8 * (r / 4) + 4 * g + (r % 4);
+        bool keep = true;
+        if (a.mask_kind != AXL_MASK_NONE) {
+          const int diff = qpos - kpos;
+          keep = diff >= 0;
+          if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) keep = keep && diff <= a.window;
+        }
+        if (seg_k) keep = keep && (seg_k[kpos] == seg_q);
+        float logit = s[r] * a.scale;
+        if (bias_row) logit += bias_at(a.aux, bias_row, kpos);
+        const float p = keep ? expf(logit - lse_q) : 0.f;
+        float dpe = dp[r];
+        if (drop_row) dpe = drop_row[kpos] ? 0.f : dpe * a.aux.keep_scale;
+        s[r] = p * (dpe - delta_q);  // dS^T
+      }
 #pragma unroll
-      for (int dt = 0; dt < DT; dt++)
-        dq[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(k_col[32 * dt], s[r], dq[dt], 0, 0, 0);
+      for (int r = 0; r < 16; r++) {
+        const float* k_col = k_lds + (8 * (r / 4) + 4 * g + (r % 4)) * PS + l32;
+#pragma unroll
+        for (int dt = 0; dt < DT; dt++)
+          dq[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(k_col[32 * dt], s[r], dq[dt], 0, 0, 0);
+      }
     }
+    if (more) {  // the other buffer was last read a tile ago, before the barrier that ended that tile
+      float* buf = ring + ((t + 1) & 1) * Tile::BUF_WORDS;
+      tile_deposit<D>(buf, kx, tid);
+      tile_deposit<D>(buf + Tile::TILE_WORDS, vx, tid);
+    }
+    __syncthreads();
   }
 
   float* dqp = (float*)a.dq + b * a.dqs.b + (int64_t)(q0 + l32) * a.dqs.s + h * a.dqs.h;
@@ -158,23 +217,19 @@ __global__ __launch_bounds__(128) void flash_bwd_dq_f32_kernel(const BwdArgs a) 
 }
 
 // ---------------------------------------------------------------------------------------------
-// dK/dV: a workgroup owns 64 keys of one kv head and loops over the query heads of its group and
+// dK/dV: a workgroup owns 128 keys of one kv head and loops over the query heads of its group and
 // over 32-query tiles.
 //   S[q][key] = Q K^T and dP[q][key] = dO V^T (A = Q / dO row l32 of the tile, B = K / V row l32), so
 //   lane (l32, g) holds key l32 and queries 8(r/4) + 4g + (r%4);
 //   dV^T[d][key] += dO^T[d][q] P[q][key],  dK^T[d][key] += Q^T[d][q] dS[q][key].
 // ---------------------------------------------------------------------------------------------
 template <int D>
-__global__ __launch_bounds__(128) void flash_bwd_dkdv_f32_kernel(const BwdArgs a) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void flash_bwd_dkdv_f32_kernel(const BwdArgs a) {
   using Tile = BwdTileF32<D>;
   constexpr int DT = D / 32, PS = Tile::PS;
   extern __shared__ __attribute__((aligned(16))) char smem[];
-  float* const k_lds = (float*)smem;
-  float* const v_lds = k_lds + Tile::ROWS * PS;
-  float* const q_lds = v_lds + Tile::ROWS * PS;
-  float* const do_lds = q_lds + Tile::TILE * PS;
-  float* const lse_lds = do_lds + Tile::TILE * PS;
-  float* const delta_lds = lse_lds + Tile::TILE;
+  float* const ring = (float*)smem;
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
@@ -185,10 +240,19 @@ __global__ __launch_bounds__(128) void flash_bwd_dkdv_f32_kernel(const BwdArgs a
   const int k0_wg = kb * Tile::ROWS, k0 = k0_wg + wave * 32;
   const int kpos = k0 + l32;
 
-  stage_rows<D, 128>(k_lds, (const float*)a.k + b * a.ks.b + (int64_t)k0_wg * a.ks.s + hk * a.ks.h, a.ks.s,
-                     Tile::ROWS, tid);
-  stage_rows<D, 128>(v_lds, (const float*)a.v + b * a.vs.b + (int64_t)k0_wg * a.vs.s + hk * a.vs.h, a.vs.s,
-                     Tile::ROWS, tid);
+  float k_mine[D / 2];
+  own_rows<D>(k_mine, ring, (const float*)a.k + b * a.ks.b + (int64_t)k0_wg * a.ks.s + hk * a.ks.h, a.ks.s, tid);
+  float* const v_own = ring + 2 * Tile::BUF_WORDS;   // the 128 owned V rows stay in LDS
+  {
+    const float* src = (const float*)a.v + b * a.vs.b + (int64_t)k0_wg * a.vs.s + hk * a.vs.h;
+    for (int i = tid; i < Tile::ROWS * (D / 4); i += Tile::NT) {
+      const int row = i / (D / 4), c4 = i % (D / 4);
+      const float4 x = *(const float4*)(src + (int64_t)row * a.vs.s + c4 * 4);
+      float* dst = v_own + row * PS + c4 * 4;
+      dst[0] = x.x; dst[1] = x.y; dst[2] = x.z; dst[3] = x.w;
+    }
+  }
+  const float* v_row = v_own + (wave * 32 + l32) * PS;
 
   // Query rows that can see a key of this block: qpos >= first key, qpos <= last key + window.
   int q_begin = 0, q_end = a.T;
@@ -199,6 +263,7 @@ __global__ __launch_bounds__(128) void flash_bwd_dkdv_f32_kernel(const BwdArgs a
   }
   const int t_begin = q_begin / Tile::TILE;
   const int t_end = (q_end + Tile::TILE - 1) / Tile::TILE;
+  const int nt = max(t_end - t_begin, 0);
   const int seg_k = a.seg ? a.seg[(int64_t)b * a.T + kpos] : 0;
   const int32_t* seg_q = a.seg ? a.seg + (int64_t)b * a.T : nullptr;
 
@@ -207,40 +272,56 @@ __global__ __launch_bounds__(128) void flash_bwd_dkdv_f32_kernel(const BwdArgs a
   for (int i = 0; i < DT; i++)
 #pragma unroll
     for (int r = 0; r < 16; r++) dk[i][r] = dv[i][r] = 0.f;
-  const float* k_row = k_lds + (wave * 32 + l32) * PS;
-  const float* v_row = v_lds + (wave * 32 + l32) * PS;
 
-  for (int hh = 0; hh < G; hh++) {
-    const int h = hk * G + hh;
-    const float* qp = (const float*)a.q + b * a.qs.b + h * a.qs.h;
-    const float* dop = (const float*)a.dout + b * a.dos.b + h * a.dos.h;
-    const int64_t stat = ((int64_t)b * a.Hq + h) * a.T;
-    const char* bias_base = a.aux.bias ? a.aux.bias + b * a.aux.bias_sb + h * a.aux.bias_sh : nullptr;
-    const uint8_t* drop_base = a.aux.drop ? a.aux.drop + b * a.aux.drop_sb + h * a.aux.drop_sh : nullptr;
-    for (int t = t_begin; t < t_end; t++) {
-      const int qt0 = t * Tile::TILE;
-      __syncthreads();  // previous tile consumed (and K, V staged on the first pass)
-      stage_rows<D, 128>(q_lds, qp + (int64_t)qt0 * a.qs.s, a.qs.s, Tile::TILE, tid);
-      stage_rows<D, 128>(do_lds, dop + (int64_t)qt0 * a.dos.s, a.dos.s, Tile::TILE, tid);
-      if (tid < Tile::TILE) {
-        lse_lds[tid] = a.lse[stat + qt0 + tid];
-        delta_lds[tid] = -a.ndelta[stat + qt0 + tid];
-      }
-      __syncthreads();
-      bool skip = false;
-      if (a.mask_kind != AXL_MASK_NONE) {
-        skip = qt0 + 31 + a.q_off < k0;  // every query of the tile lies before this wavefront's keys
-        if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) skip = skip || (qt0 + a.q_off - (k0 + 31) > a.window);
-      }
-      if (skip) continue;
+  // Step e of the loop is query tile t_begin + e % nt of query head hk G + e / nt; it lives in ring
+  // buffer e % 2: Q rows, dO rows, lse and delta of the 32 queries.
+  const int steps = nt * G;
+  float4 qx[Tile::LD4], dox[Tile::LD4];
+  float stat_x = 0.f;  // threads 0..31: lse, 32..63: delta of query tid % 32
+  auto request = [&](int e) __attribute__((always_inline)) {
+    const int h = hk * G + e / nt, qt0 = (t_begin + e % nt) * Tile::TILE;
+    tile_request<D>(qx, (const float*)a.q + b * a.qs.b + h * a.qs.h + (int64_t)qt0 * a.qs.s, a.qs.s, tid);
+    tile_request<D>(dox, (const float*)a.dout + b * a.dos.b + h * a.dos.h + (int64_t)qt0 * a.dos.s, a.dos.s, tid);
+    const int64_t row = ((int64_t)b * a.Hq + h) * a.T + qt0 + (tid & 31);
+    if (tid < 32) stat_x = a.lse[row];
+    else if (tid < 64) stat_x = -a.ndelta[row];
+  };
+  auto deposit = [&](int e) __attribute__((always_inline)) {
+    float* buf = ring + (e & 1) * Tile::BUF_WORDS;
+    tile_deposit<D>(buf, qx, tid);
+    tile_deposit<D>(buf + Tile::TILE_WORDS, dox, tid);
+    if (tid < 64) buf[2 * Tile::TILE_WORDS + tid] = stat_x;
+  };
+  __syncthreads();  // the owned rows have been read out of the ring
+  if (steps > 0) {
+    request(0);
+    deposit(0);
+  }
+  __syncthreads();
+  for (int e = 0; e < steps; e++) {
+    const int h = hk * G + e / nt, qt0 = (t_begin + e % nt) * Tile::TILE;
+    const bool more = e + 1 < steps;
+    if (more) request(e + 1);  // the next tile's round trip runs under this tile's MFMAs
+    const float* q_lds = ring + (e & 1) * Tile::BUF_WORDS;
+    const float* do_lds = q_lds + Tile::TILE_WORDS;
+    const float* lse_lds = q_lds + 2 * Tile::TILE_WORDS;
+    const float* delta_lds = lse_lds + Tile::TILE;
+    bool skip = false;
+    if (a.mask_kind != AXL_MASK_NONE) {
+      skip = qt0 + 31 + a.q_off < k0;  // every query of the tile lies before this wavefront's keys
+      if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) skip = skip || (qt0 + a.q_off - (k0 + 31) > a.window);
+    }
+    if (!skip) {
+      const char* bias_base = a.aux.bias ? a.aux.bias + b * a.aux.bias_sb + h * a.aux.bias_sh : nullptr;
+      const uint8_t* drop_base = a.aux.drop ? a.aux.drop + b * a.aux.drop_sb + h * a.aux.drop_sh : nullptr;
       floatx16 s, dp;
 #pragma unroll
       for (int r = 0; r < 16; r++) s[r] = dp[r] = 0.f;
       const float* q_row = q_lds + l32 * PS;
       const float* do_row = do_lds + l32 * PS;
-#pragma unroll 8
+#pragma unroll
       for (int d2 = 0; d2 < D / 2; d2++) {
-        s = __builtin_amdgcn_mfma_f32_32x32x2f32(q_row[2 * d2 + g], k_row[2 * d2 + g], s, 0, 0, 0);
+        s = __builtin_amdgcn_mfma_f32_32x32x2f32(q_row[2 * d2 + g], k_mine[d2], s, 0, 0, 0);
         dp = __builtin_amdgcn_mfma_f32_32x32x2f32(do_row[2 * d2 + g], v_row[2 * d2 + g], dp, 0, 0, 0);
       }
       floatx16 pd;  // probabilities after dropout, for dV
@@ -279,6 +360,8 @@ __global__ __launch_bounds__(128) void flash_bwd_dkdv_f32_kernel(const BwdArgs a
         }
       }
     }
+    if (more) deposit(e + 1);  // the other buffer was last read a step ago, before the barrier that ended it
+    __syncthreads();
   }
 
   float* dkp = (float*)a.dk + b * a.dks.b + (int64_t)kpos * a.dks.s + hk * a.dks.h;
@@ -301,9 +384,9 @@ static hipError_t launch_f32(const BwdArgs& a, int phases, hipStream_t stream) {
   hipError_t err = hipSuccess;
   if (phases & AXL_BWD_DKDV) {
     auto kernel = flash_bwd_dkdv_f32_kernel<D>;
-    err = allow_dynamic_lds((const void*)kernel, Tile::LDS_BYTES);
+    err = allow_dynamic_lds((const void*)kernel, Tile::LDS_BYTES_DKDV);
     if (err != hipSuccess) return err;
-    hipLaunchKernelGGL(kernel, dim3((a.S / Tile::ROWS) * a.B * a.Hkv), dim3(128), Tile::LDS_BYTES, stream, a);
+    hipLaunchKernelGGL(kernel, dim3((a.S / Tile::ROWS) * a.B * a.Hkv), dim3(Tile::NT), Tile::LDS_BYTES_DKDV, stream, a);
     err = hipGetLastError();
     if (err != hipSuccess) return err;
   }
@@ -311,7 +394,7 @@ static hipError_t launch_f32(const BwdArgs& a, int phases, hipStream_t stream) {
     auto kernel = flash_bwd_dq_f32_kernel<D>;
     err = allow_dynamic_lds((const void*)kernel, Tile::LDS_BYTES);
     if (err != hipSuccess) return err;
-    hipLaunchKernelGGL(kernel, dim3((a.T / Tile::ROWS) * a.B * a.Hq), dim3(128), Tile::LDS_BYTES, stream, a);
+    hipLaunchKernelGGL(kernel, dim3((a.T / Tile::ROWS) * a.B * a.Hq), dim3(Tile::NT), Tile::LDS_BYTES, stream, a);
     err = hipGetLastError();
   }
   return err;
