@@ -602,9 +602,12 @@ struct FwdTileF32 {
   static constexpr int VSTRIDE = D * 4;       // lanes read consecutive d of one row: no pad needed
   static constexpr int KBYTES = BK * KSTRIDE;
   static constexpr int VBYTES = BK * VSTRIDE;
+  static constexpr int BUF_BYTES = KBYTES + VBYTES;   // one K / V tile; tile t lives in buffer t % 2
   static constexpr int QSTRIDE = D * 4 + 4;
-  static constexpr int QBYTES = BQ * QSTRIDE;
-  static constexpr int LDS_BYTES = QBYTES + KBYTES + VBYTES;
+  static constexpr int QBYTES = BQ * QSTRIDE;         // the query block passes through the same memory once
+  static constexpr int LDS_BYTES = 2 * BUF_BYTES > QBYTES ? 2 * BUF_BYTES : QBYTES;
+  static constexpr int LD4 = BK * (D / 4) / 256;      // float4 loads per thread and tensor tile
+  static_assert(BK * (D / 4) % 256 == 0, "a tile divides evenly over the threads");
 };
 
 template <int D>
@@ -613,8 +616,6 @@ __global__ __launch_bounds__(256) void flash_fwd_f32_kernel(const FwdArgs a) {
   constexpr int DT = D / 32;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   float* const q_lds = (float*)smem;
-  float* const k_lds = (float*)(smem + Tile::QBYTES);
-  float* const v_lds = (float*)(smem + Tile::QBYTES + Tile::KBYTES);
   constexpr int QS = Tile::QSTRIDE / 4, KS = Tile::KSTRIDE / 4, VS = Tile::VSTRIDE / 4;
 
   const int tid = threadIdx.x;
@@ -631,13 +632,22 @@ __global__ __launch_bounds__(256) void flash_fwd_f32_kernel(const FwdArgs a) {
   const float* kp = (const float*)a.k + b * a.ks.b + hk * a.ks.h;
   const float* vp = (const float*)a.v + b * a.vs.b + hk * a.vs.h;
 
-  // Stage the 128 x D query block (fp32) in LDS once.
+  // The 128 x D query block (fp32) passes through LDS once; a lane keeps the half of its own row that
+  // its MFMAs read (elements 2 d2 + g) in registers.
   for (int i = tid; i < Tile::BQ * (D / 4); i += 256) {
     const int row = i / (D / 4), c4 = i % (D / 4);
     const float4 x = *(const float4*)(qg + (int64_t)row * a.qs.s + c4 * 4);
     float* dst = q_lds + row * QS + c4 * 4;
     dst[0] = x.x; dst[1] = x.y; dst[2] = x.z; dst[3] = x.w;
   }
+  __syncthreads();
+  float q_mine[D / 2];
+  {
+    const float* q_row = q_lds + (wave * 32 + l32) * QS;
+#pragma unroll
+    for (int d2 = 0; d2 < D / 2; d2++) q_mine[d2] = q_row[2 * d2 + g];
+  }
+  __syncthreads();  // the ring of K / V tiles takes the memory over
 
   int k_begin = 0, k_end = a.S;
   if (a.mask_kind != AXL_MASK_NONE) {
@@ -665,35 +675,55 @@ __global__ __launch_bounds__(256) void flash_fwd_f32_kernel(const FwdArgs a) {
     m_run = a.sink[h];
     l_run = g == 0 ? 1.f : 0.f;
   }
-  const float* q_row = q_lds + (wave * 32 + l32) * QS;
+  // The K / V tile of 32 keys from global memory into this thread's registers, and from there into a
+  // ring buffer: the next tile's round trip runs under the current tile's MFMAs, one barrier per tile.
+  float4 kx[Tile::LD4], vx[Tile::LD4];
+  auto request = [&](int k0) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < Tile::LD4; i++) {
+      const int e = tid + i * 256, row = e / (D / 4), c4 = e % (D / 4);
+      kx[i] = *(const float4*)(kp + (int64_t)(k0 + row) * a.ks.s + c4 * 4);
+      vx[i] = *(const float4*)(vp + (int64_t)(k0 + row) * a.vs.s + c4 * 4);
+    }
+  };
+  auto deposit = [&](int t) __attribute__((always_inline)) {
+    float* k_dst = (float*)(smem + (t & 1) * Tile::BUF_BYTES);
+    float* v_dst = (float*)(smem + (t & 1) * Tile::BUF_BYTES + Tile::KBYTES);
+#pragma unroll
+    for (int i = 0; i < Tile::LD4; i++) {
+      const int e = tid + i * 256, row = e / (D / 4), c4 = e % (D / 4);
+      float* kd = k_dst + row * KS + c4 * 4;
+      kd[0] = kx[i].x; kd[1] = kx[i].y; kd[2] = kx[i].z; kd[3] = kx[i].w;
+      *(float4*)(v_dst + row * VS + c4 * 4) = vx[i];
+    }
+  };
+  if (t_begin < t_end) {
+    request(t_begin * Tile::BK);
+    deposit(t_begin);
+  }
+  __syncthreads();
 
   for (int t = t_begin; t < t_end; t++) {
     const int k0 = t * Tile::BK;
-    __syncthreads();  // previous tile fully consumed (and Q staged on the first pass)
-    for (int i = tid; i < Tile::BK * (D / 4); i += 256) {
-      const int row = i / (D / 4), c4 = i % (D / 4);
-      const float4 x = *(const float4*)(kp + (int64_t)(k0 + row) * a.ks.s + c4 * 4);
-      const float4 y = *(const float4*)(vp + (int64_t)(k0 + row) * a.vs.s + c4 * 4);
-      float* kd = k_lds + row * KS + c4 * 4;
-      kd[0] = x.x; kd[1] = x.y; kd[2] = x.z; kd[3] = x.w;
-      *(float4*)(v_lds + row * VS + c4 * 4) = y;
-    }
-    __syncthreads();
+    const bool more = t + 1 < t_end;
+    if (more) request(k0 + Tile::BK);
+    const float* k_lds = (const float*)(smem + (t & 1) * Tile::BUF_BYTES);
+    const float* v_lds = (const float*)(smem + (t & 1) * Tile::BUF_BYTES + Tile::KBYTES);
     bool skip = false;
     if (a.mask_kind != AXL_MASK_NONE) {
       skip = k0 > qpos_max;
       if (a.mask_kind == AXL_MASK_SLIDING_WINDOW)
         skip = skip || (qpos_min - (k0 + Tile::BK - 1) > a.window);
     }
-    if (skip) continue;
+    if (!skip) {
     // S^T[key][q]: A = K (lane: key row l32, k index g), B = Q^T (lane: query l32, k index g).
     floatx16 s;
 #pragma unroll
     for (int r = 0; r < 16; r++) s[r] = 0.f;
     const float* k_row = k_lds + l32 * KS;
-#pragma unroll 8
+#pragma unroll
     for (int d2 = 0; d2 < D / 2; d2++) {
-      s = __builtin_amdgcn_mfma_f32_32x32x2f32(k_row[2 * d2 + g], q_row[2 * d2 + g], s, 0, 0, 0);
+      s = __builtin_amdgcn_mfma_f32_32x32x2f32(k_row[2 * d2 + g], q_mine[d2], s, 0, 0, 0);
     }
     // Register r of lane group g is key k0 + 8(r/4) + 4g + (r%4).
     if (bias_row) {  // logits = scale * qk + bias: pre-divide so the common scale below applies
@@ -751,6 +781,9 @@ __global__ __launch_bounds__(256) void flash_fwd_f32_kernel(const FwdArgs a) {
       for (int dt = 0; dt < DT; dt++)
         o[dt] = __builtin_amdgcn_mfma_f32_32x32x2f32(v_row[32 * dt], s[r], o[dt], 0, 0, 0);
     }
+    }  // tile not skipped
+    if (more) deposit(t + 1);  // that buffer was last read a tile ago, before the barrier that ended it
+    __syncthreads();
   }
 
   const float l_tot = xor32_sum(l_run);
