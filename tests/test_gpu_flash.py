@@ -896,6 +896,29 @@ def test_ds_workspace_backward_through_the_plugin_config():
         assert all(torch.equal(x, y) for x, y in zip(g, grads[0]))
 
 
+def test_plugin_takes_the_ds_workspace_in_slices_when_the_whole_does_not_fit():
+    """A limit just below the whole dS workspace, on a shape whose slices still fill the GPU: the default
+    configuration keeps the dS of 7 of the 8 kv heads at a time (then the last one), and the gradients are
+    bit-identical to the kernel called directly with the whole workspace; the same through
+    `ops.flash_bwd(ds_workspace=None, ds_workspace_limit=...)`."""
+    b, t, hq, hkv, d = 8, 2048, 8, 8, 64
+    q, k, v, do = (x.cuda() for x in _inputs(b, t, hq, hkv, d, torch.bfloat16))
+    full, plain = ops.flash_bwd_ds_workspace_bytes(q, k, mask_kind=ops.MASK_CAUSAL)
+    assert ops.select_ds_slice(q, k, mask_kind=ops.MASK_CAUSAL, limit=full - 1) == (True, hkv - 1)
+    kw = dict(softmax_scale=d ** -0.5, mask_kind=ops.MASK_CAUSAL)
+    out, lse = ops.flash_fwd(q, k, v, **kw)
+    direct = ops.flash_bwd(q, k, v, out, lse, do, ds_workspace=True, **kw)
+    auto = ops.flash_bwd(q, k, v, out, lse, do, ds_workspace=None, ds_workspace_limit=full - 1, **kw)
+    assert all(torch.equal(x, y) for x, y in zip(auto, direct))
+    pos = dict(target_positions=torch.arange(t)[None], source_positions=torch.arange(t)[None])
+    bias = ab.CompositeAttentionBias([ab.CausalAttentionBias(**pos)])
+    qd, kd, vd = (x.clone().requires_grad_(True) for x in (q, k, v))
+    fa = HipFlashAttention.default_config().set(softmax_scale=d ** -0.5, bwd_workspace_limit_bytes=full - 1).instantiate()
+    res = fa(dict(query=qd, key=kd, value=vd, bias=bias))
+    grads = torch.autograd.grad(res, (qd, kd, vd), do)
+    assert torch.equal(res, out) and all(torch.equal(x, y) for x, y in zip(grads, direct))
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_rows_without_a_visible_key(dtype):
     """Causal rows at negative positions see no key: out = 0, lse = -inf, and the backward leaves dq of
