@@ -3,10 +3,13 @@ axlearn/common/flash_attention/gpu_attention.py to put the HIP kernels behind
 `flash_attention_implementation`.
 
 This module needs jax and the FFI library `libaxl_attn_ffi.so` (built from csrc/ffi_shim.cc against
-jaxlib's `xla/ffi/api/ffi.h`).  Neither exists in this repository's environment, so nothing here is
-imported by the package or exercised by its tests: it is the source of the reference-side binding,
-kept next to the torch host mirror (`hip_attention.py`, `hip_decoding.py`) whose behaviour it repeats
-call for call.
+jaxlib's `xla/ffi/api/ffi.h`).  Neither exists in this repository's environment, so the package never
+imports it: it is the source of the reference-side binding, kept next to the torch host mirror
+(`hip_attention.py`, `hip_decoding.py`) whose behaviour it repeats call for call.  The tests run it under
+eager stand-ins for the few jax names it uses (tests/jax_stand_in.py: torch tensors for arrays, and an
+`ffi_call` that fills the C-ABI structures as the shim does and runs the kernels), which shows that its
+classes and its custom_vjp pair give the torch side's bits with the workspace sizes computed here; XLA,
+jax's own machinery and the compiled shim stay untested.
 
 It mirrors, name for name:
   * `flash_attention` with its `jax.custom_vjp` and residuals `(q, k, v, bias, segment_ids, prng_key,

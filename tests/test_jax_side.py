@@ -1,0 +1,194 @@
+"""flash_attention/jax_ffi.py, the JAX side of the XLA FFI binding, executed under the stand-ins of
+tests/jax_stand_in.py (jax is not installed here): see that module for what this does and does not show."""
+
+import ctypes
+
+import pytest
+import torch
+
+from axlearn_amd import _lib
+from axlearn_amd import attention_bias as ab
+from axlearn_amd import ops
+import jax_stand_in  # tests/jax_stand_in.py (pytest puts the test directory on sys.path)
+from oracle import ref_attention as ref
+
+RESIDUAL = "gpu_attention.flash_residuals"   # remat.py:13-58 matches this name
+
+
+def _size_query(b, t, s, hq, hkv, d, mask_kind, has_seg, flags):
+    p = _lib.AxlFlashBwdParams(batch=b, q_len=t, kv_len=s, num_q_heads=hq, num_kv_heads=hkv, head_dim=d, dtype=0,
+                               mask_kind=mask_kind, segment_ids=1 if has_seg else None, flags=flags)
+    return int(_lib.load().axl_flash_bwd_workspace_bytes(ctypes.byref(p)))
+
+
+def test_jax_side_imports_and_registers_every_target():
+    with jax_stand_in.installed() as (mod, state):
+        assert sorted(state.registered) == sorted((t, "ROCM") for t in jax_stand_in.HANDLERS)
+        for name in ("flash_attention", "HipFlashAttention", "HipDecoding", "HipPagedAttention", "hip_scatter_update_pages"):
+            assert hasattr(mod, name)
+    import sys
+
+    assert "jax" not in sys.modules and jax_stand_in.JAX_SIDE not in sys.modules and not hasattr(torch.Tensor, "astype")
+
+
+@pytest.mark.parametrize("shape,seg,want_flags", [
+    ((2, 256, 256, 8, 2, 128), False, 1),            # fits: the dS workspace whole
+    ((2, 256, 256, 8, 2, 128), True, 1),
+    ((1, 32768, 32768, 64, 8, 128), False, 1 | 2 << 8),  # 69 GB whole: two kv heads at a time under the 18 GB limit
+    ((1, 32768, 32768, 32, 1, 128), False, 0),        # 34 GB in one kv head, which cannot be sliced: the recomputing pair
+    ((2, 256, 384, 8, 2, 128), False, 1),             # q_len != kv_len: the flag is passed and ignored by the library
+])
+def test_custom_vjp_pair_sizes_the_workspace_as_the_library_asks(shape, seg, want_flags):
+    """The pair given to `defvjp`, with every tensor on the meta device and no kernel run: the forward
+    tags out and lse for the remat policy and keeps the residuals of gpu_attention.py:420-424; the
+    backward declares a workspace result of exactly axl_flash_bwd_workspace_bytes for the flags it
+    chose (whole, in slices of kv heads, or none), and returns no gradient for bias, ids and mask."""
+    b, t, s, hq, hkv, d = shape
+    with jax_stand_in.installed() as (mod, state):
+        state.execute, state.device = False, "meta"
+        mk = lambda *dims: torch.empty(dims, dtype=torch.bfloat16, device="meta")
+        q, k, v = mk(b, t, hq, d), mk(b, s, hkv, d), mk(b, s, hkv, d)
+        ids = torch.empty((b, t), dtype=torch.int64, device="meta") if seg else None
+        args = (q, k, v, None, ids, None, d ** -0.5, mod.MASK_CAUSAL, 0, 0.0, False)
+        out, pullback = mod.flash_attention.vjp(*args)
+        assert state.checkpoint_names == [RESIDUAL, RESIDUAL]
+        target, operands, attrs, results = state.calls[0]
+        assert target == "AxlFlashFwd" and results == [(b, t, hq, d), (b, hq, t)]
+        assert operands[3] == ((b, t) if seg else (0,)) and operands[4:] == [(0,)] * 4
+        assert attrs["mask_kind"] == 1 and abs(attrs["softmax_scale"] - d ** -0.5) < 1e-7
+        grads = pullback(torch.empty_like(out))
+        assert len(grads) == 6 and grads[3:] == (None, None, None)
+        assert [tuple(g.shape) for g in grads[:3]] == [tuple(x.shape) for x in (q, k, v)]
+        target, operands, attrs, results = state.calls[1]
+        assert target == "AxlFlashBwd" and attrs["flags"] == want_flags
+        want_ws = _size_query(b, t, s, hq, hkv, d, 1, seg, want_flags)
+        assert results[3:] == [(0,), (want_ws,)]
+        if want_flags >> 8:
+            assert want_ws <= mod.BWD_WORKSPACE_LIMIT_BYTES < _size_query(b, t, s, hq, hkv, d, 1, seg, 1)
+        # calling the function itself is the forward alone
+        n = len(state.calls)
+        assert mod.flash_attention(*args).shape == out.shape and len(state.calls) == n + 1
+
+
+def test_forced_choices_of_the_backward_workspace():
+    b, t, hq, hkv, d = 1, 512, 4, 2, 128
+    with jax_stand_in.installed() as (mod, state):
+        state.execute, state.device = False, "meta"
+        mk = lambda h: torch.empty((b, t, h, d), dtype=torch.float16, device="meta")
+        args = (mk(hq), mk(hkv), mk(hkv), None, None, None, 0.1, mod.MASK_SLIDING_WINDOW, 100, 0.0, False)
+        for forced, flags in ((False, 0), (True, 1)):
+            mod.BWD_DS_WORKSPACE = forced
+            out, pullback = mod.flash_attention.vjp(*args)
+            pullback(torch.empty_like(out))
+            assert state.calls[-1][2]["flags"] == flags and state.calls[-1][2]["sliding_window"] == 100
+            assert state.calls[-1][3][4] == (_size_query(b, t, t, hq, hkv, d, 2, False, flags),)
+
+
+def _inputs(b, t, hq, hkv, d, dtype, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    mk = lambda h: torch.randn(b, t, h, d, generator=g).to(dtype).cuda()
+    return mk(hq), mk(hkv), mk(hkv), mk(hq)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("window,seg", [(None, False), (None, True), (100, True)])
+def test_jax_side_flash_attention_runs_the_kernels_like_the_torch_side(window, seg):
+    """`HipFlashAttention.__call__` and the custom_vjp pair of the JAX side on the GPU, through the C ABI
+    with the buffers the stand-in FFI allocates from the declared result types: bit-identical to
+    `ops.flash_fwd` / `ops.flash_bwd` with the torch side's default policy."""
+    b, t, hq, hkv, d = 2, 384, 8, 2, 128
+    q, k, v, do = _inputs(b, t, hq, hkv, d, torch.bfloat16)
+    ids = (torch.arange(t)[None] // torch.tensor([[100], [190]])).int().cuda() + 1 if seg else None
+    pos = dict(target_positions=torch.arange(t)[None].cuda(), source_positions=torch.arange(t)[None].cuda())
+    mask = ab.CausalAttentionBias(**pos) if window is None else ab.SlidingWindowAttentionBias(
+        ab.sliding_window_causal_mask(window), sliding_window_size=window, **pos)
+    bias = ab.CompositeAttentionBias([mask] + ([ab.SegmentIdAttentionBias(ids)] if seg else []))
+    scale = d ** -0.5
+    kw = dict(softmax_scale=scale, mask_kind=ops.MASK_CAUSAL if window is None else ops.MASK_SLIDING_WINDOW,
+              sliding_window=window or 0, segment_ids=ids)
+    want_out, want_lse = ops.flash_fwd(q, k, v, **kw)
+    want = ops.flash_bwd(q, k, v, want_out, want_lse, do, ds_workspace=None, **kw)[:3]
+    with jax_stand_in.installed() as (mod, state):
+        fa = mod.HipFlashAttention.default_config().set(softmax_scale=scale).instantiate()
+        batch = dict(query=q, key=k, value=v, bias=bias)
+        assert fa.is_supported(batch, kv_cache_type=None)
+        assert torch.equal(fa(batch), want_out)
+        assert state.calls[-1][0] == "AxlFlashFwd" and state.calls[-1][2]["mask_kind"] == kw["mask_kind"]
+        out, pullback = mod.flash_attention.vjp(q, k, v, None, ids, None, scale, kw["mask_kind"], kw["sliding_window"], 0.0, False)
+        assert torch.equal(out, want_out) and state.checkpoint_names == [RESIDUAL, RESIDUAL]
+        dq, dk, dv = pullback(do)[:3]
+        assert state.calls[-1][2]["flags"] == 1   # the dS workspace fits
+        for name, got, exp in (("dq", dq, want[0]), ("dk", dk, want[1]), ("dv", dv, want[2])):
+            assert torch.equal(got, exp), name
+
+
+@pytest.mark.gpu
+def test_jax_side_flash_attention_with_bias_and_dropout():
+    """An arbitrary mask fn becomes a dense bias once, an explicit bias is added to it, and the dropout
+    mask is drawn by the caller: the same operands given to the torch side give the same bits."""
+    b, t, hq, hkv, d, rate = 1, 256, 4, 4, 64, 0.25
+    q, k, v, do = _inputs(b, t, hq, hkv, d, torch.float16, seed=3)
+    pos = dict(target_positions=torch.arange(t)[None].cuda(), source_positions=torch.arange(t)[None].cuda())
+    strided = lambda qp, kp: (qp >= kp) & ((qp - kp) % 3 != 1)
+    dense = torch.randn(1, hq, t, t, generator=torch.Generator().manual_seed(5)).cuda()
+    bias = ab.CompositeAttentionBias([ab.MaskFnAttentionBias(strided, **pos), ab.TensorAttentionBias(dense)])
+    with jax_stand_in.installed() as (mod, state):
+        fa = mod.HipFlashAttention.default_config().set(softmax_scale=0.125, dropout_rate=rate).instantiate()
+        got = fa(dict(query=q, key=k, value=v, bias=bias, prng_key=11))
+        import jax  # the stand-in
+
+        drop = jax.random.bernoulli(11, rate, (b, hq, t, t))
+        target, operands, attrs, _ = state.calls[-1]
+        assert operands[5] == (1, hq, t, t) and operands[6] == (b, hq, t, t) and attrs["mask_kind"] == 0
+        assert abs(attrs["dropout_rate"] - rate) < 1e-7
+        full = bias.value().float()
+        want, lse = ops.flash_fwd(q, k, v, softmax_scale=0.125, mask_kind=ops.MASK_NONE, bias=full,
+                                  dropout_mask=drop, dropout_rate=rate)
+        assert torch.equal(got, want)
+        out, pullback = mod.flash_attention.vjp(q, k, v, full, None, drop, 0.125, 0, 0, rate, False)
+        grads = pullback(do)
+        exp = ops.flash_bwd(q, k, v, want, lse, do, softmax_scale=0.125, mask_kind=ops.MASK_NONE, bias=full,
+                            dropout_mask=drop, dropout_rate=rate)[:3]
+        for g, e in zip(grads[:3], exp):
+            assert torch.equal(g, e)
+
+
+@pytest.mark.gpu
+def test_jax_side_decode_classes_and_page_insert():
+    """`HipDecoding`, `HipPagedAttention` and `hip_scatter_update_pages` of the JAX side against the torch
+    side's `ops.decode` / `ops.paged_decode` / `ops.paged_kv_insert` on the same operands: identical bits
+    (the deterministic flag is off on both sides, and one call's split is a function of the shapes)."""
+    hq, hkv, d, page, pps, b = 8, 2, 128, 16, 8, 3
+    qq, kp, vp, tables, lengths = ref.paged_inputs(5, batch=b, num_heads=hq, num_kv_heads=hkv, head_dim=d,
+                                                    page_size=page, pages_per_seq=pps, min_len=10, max_len=page * pps)
+    qq, kp, vp, tables, lengths = (x.cuda() for x in (qq, kp, vp, tables, lengths))
+    kv_len = page * pps
+    causal = ab.CompositeAttentionBias([ab.CausalAttentionBias(
+        target_positions=(lengths.long() - 1)[:, None], source_positions=torch.arange(kv_len)[None].cuda())])
+    with jax_stand_in.installed() as (mod, state):
+        paged = mod.HipPagedAttention.default_config().set(softmax_scale=0.3).instantiate()
+        got = paged(dict(query=qq, key=kp, value=vp, bias=causal, page_tables=tables))
+        want = ops.paged_decode(qq.reshape(b, hq, d), kp, vp, tables, lengths, softmax_scale=0.3)
+        assert got.shape == (b, 1, hq, d) and torch.equal(got.reshape(b, hq, d), want)
+        # contiguous cache: the same keys gathered
+        kk, vv = (ref.reconstruct_kv(tables.cpu(), x.cpu()).contiguous().cuda() for x in (kp, vp))
+        dec = mod.HipDecoding.default_config().set(softmax_scale=0.3).instantiate()
+        got_c = dec(dict(query=qq, key=kk, value=vv, bias=causal))
+        want_c = ops.decode(qq.reshape(b, hq, d), kk, vv, lengths, softmax_scale=0.3)
+        assert torch.equal(got_c.reshape(b, hq, d), want_c)
+        # a mask fn that is neither causal nor a window: evaluated on the host as a row of 0 / NEG_INF
+        even = lambda qp, kp_: (kp_ <= qp) & (kp_ % 2 == 0)
+        other = ab.CompositeAttentionBias([ab.MaskFnAttentionBias(
+            even, target_positions=(lengths.long() - 1)[:, None], source_positions=torch.arange(kv_len)[None].cuda())])
+        got_m = dec(dict(query=qq, key=kk, value=vv, bias=other))
+        assert state.calls[-1][1][4] == (b, 1, kv_len)
+        row = torch.where(even((lengths.long() - 1)[:, None], torch.arange(kv_len)[None].cuda()), 0.0, ab.NEG_INF)
+        want_m = ops.decode(qq.reshape(b, hq, d), kk, vv, lengths, softmax_scale=0.3, bias=row[:, None, :].float())
+        assert torch.equal(got_m.reshape(b, hq, d), want_m)
+        # page insert, in place
+        kproj, vproj = torch.randn(2, hkv, b, 1, d, generator=torch.Generator().manual_seed(7)).to(kp.dtype).cuda()
+        positions = (lengths - 1).clamp(min=0)
+        k2, v2 = kp.clone(), vp.clone()
+        ops.paged_kv_insert(k2, v2, kproj[:, :, 0].transpose(0, 1), vproj[:, :, 0].transpose(0, 1), tables, positions)
+        k1, v1 = mod.hip_scatter_update_pages(kp, vp, kproj, vproj, tables, positions)
+        assert k1.data_ptr() == kp.data_ptr() and torch.equal(k1, k2) and torch.equal(v1, v2)
