@@ -13,9 +13,11 @@
 // axlearn_amd/flash_attention/jax_ffi.py.
 //
 // Build (not part of the default `make`: the header ships with jaxlib, which this repository's
-// environment does not have, so this file has not been compiled here):
+// environment does not have):
 //   hipcc -O2 -std=c++17 -fPIC -shared -I$(python -c 'import jax; print(jax.ffi.include_dir())')
 //         -I../../include ffi_shim.cc -L.. -laxl_attn_hip -o ../libaxl_attn_ffi.so
+// Here the file is compiled, and its handlers are run by the tests, against a stand-in for that header
+// which keeps the names and accessors this file uses (tests/xla_ffi_stand_in/).
 //
 // Conventions.  Every buffer is a device buffer owned by XLA; the library allocates nothing, so the
 // workspaces are extra RESULTS of the custom call (XLA allocates them, the Python wrapper drops

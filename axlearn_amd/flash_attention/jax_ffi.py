@@ -7,9 +7,10 @@ jaxlib's `xla/ffi/api/ffi.h`).  Neither exists in this repository's environment,
 imports it: it is the source of the reference-side binding, kept next to the torch host mirror
 (`hip_attention.py`, `hip_decoding.py`) whose behaviour it repeats call for call.  The tests run it under
 eager stand-ins for the few jax names it uses (tests/jax_stand_in.py: torch tensors for arrays, and an
-`ffi_call` that fills the C-ABI structures as the shim does and runs the kernels), which shows that its
-classes and its custom_vjp pair give the torch side's bits with the workspace sizes computed here; XLA,
-jax's own machinery and the compiled shim stay untested.
+`ffi_call` that hands operands, results and attributes to the handlers of csrc/ffi_shim.cc, built against
+a stand-in for jaxlib's header), which shows that its classes and its custom_vjp pair give the torch
+side's bits with the workspace sizes computed here; XLA, jax's own machinery and the shim against the
+real header stay untested.
 
 It mirrors, name for name:
   * `flash_attention` with its `jax.custom_vjp` and residuals `(q, k, v, bias, segment_ids, prng_key,

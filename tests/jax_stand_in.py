@@ -11,16 +11,18 @@ environment.  `installed()` puts the handful of names it uses into `sys.modules`
   * `jax.custom_vjp`, `jax.jit`, `jax.ShapeDtypeStruct` and `checkpoint_name` are the obvious eager
     forms (`custom_vjp` keeps the pair given to `defvjp`, `vjp()` below runs it; `checkpoint_name`
     returns its argument and records the name it was given);
-  * `jax.ffi.ffi_call(target, result_types)(*operands, **attributes)` allocates the results and runs the
-    C-ABI entry point that `csrc/ffi_shim.cc` binds to `target`, filling the parameter structure from
-    operand shapes and attributes the way the shim does (dense row-major strides, a zero-element buffer
-    for an absent operand, workspaces as extra results of exactly the declared size), through the ctypes
-    mirror of include/axl_attn.h.  Every call is also appended to `State.calls`.
+  * `jax.ffi.ffi_call(target, result_types)(*operands, **attributes)` allocates the results (a workspace
+    is a result of exactly the declared size; an aliased result is the donated operand), builds the call
+    frame and runs the handler of that target in `csrc/ffi_shim.cc` itself, compiled against a stand-in
+    for jaxlib's `xla/ffi/api/ffi.h` (tests/xla_ffi_stand_in/): operands and results as dense buffers with
+    dtype and dimensions, scalars as named attributes of exact type.  Every call is also appended to
+    `State.calls`.
 
-What this cannot show: XLA, jax's tracing and differentiation machinery, and the compiled shim.  What it
-does show: that the module imports with the names it uses, that its classes and its custom_vjp pair run
-to completion on the real kernels with the workspace sizes it computes, and that the results are those
-of the torch-side mirror.
+What this cannot show: XLA, jax's tracing and differentiation machinery, and the shim against the real
+header.  What it does show: that the module imports with the names it uses, that the shim compiles and
+its handlers fill the C-ABI structures correctly from what the JAX side passes, that the classes and the
+custom_vjp pair run to completion on the real kernels with the workspace sizes computed on the JAX side,
+and that the results are those of the torch-side mirror.
 """
 
 from __future__ import annotations
@@ -28,6 +30,7 @@ from __future__ import annotations
 import contextlib
 import ctypes
 import importlib
+import os
 import sys
 import types
 
@@ -82,149 +85,93 @@ def _jit(fun=None, **_):
     return fun if fun is not None else (lambda f: f)
 
 
-def _elements(t):
-    return 0 if t is None else t.numel()
+TARGETS = ("AxlFlashFwd", "AxlFlashBwd", "AxlDecode", "AxlPagedDecode", "AxlPagedKvInsert")
+SHIM_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "xla_ffi_stand_in")
+SHIM_PATH = os.path.join(SHIM_DIR, "libaxl_attn_ffi_standin.so")
+# xla::ffi::DataType
+_DATA_TYPE = {torch.bool: 1, torch.int32: 4, torch.int64: 5, torch.uint8: 6, torch.float16: 10, torch.float32: 11,
+              torch.bfloat16: 16}
+_ERROR_CODE = {3: "INVALID_ARGUMENT", 12: "UNIMPLEMENTED", 13: "INTERNAL"}
 
 
-def _or_null(t):
-    return None if _elements(t) == 0 else t.data_ptr()
+class _Buffer(ctypes.Structure):
+    _fields_ = [("data", ctypes.c_void_p), ("dtype", ctypes.c_int32), ("rank", ctypes.c_int32),
+                ("dims", ctypes.POINTER(ctypes.c_int64))]
 
 
-def _dense4(shape):
-    return _lib.AxlStrides(shape[1] * shape[2] * shape[3], shape[2] * shape[3], shape[3])
+class _Attr(ctypes.Structure):
+    _fields_ = [("name", ctypes.c_char_p), ("kind", ctypes.c_int32), ("i32", ctypes.c_int32), ("f32", ctypes.c_float)]
 
 
-def _fill_aux(bias, drop, rate):
-    aux = _lib.AxlAttnAux()
-    if _elements(bias):
-        d = bias.shape
-        assert len(d) == 4
-        aux.bias, aux.bias_dtype = bias.data_ptr(), _lib.dtype_code(bias.dtype)
-        aux.bias_row_stride = d[3]
-        aux.bias_head_stride = 0 if d[1] == 1 else d[2] * d[3]
-        aux.bias_batch_stride = 0 if d[0] == 1 else d[1] * d[2] * d[3]
-    if _elements(drop):
-        d = drop.shape
-        assert len(d) == 4 and drop.dtype == torch.uint8
-        aux.dropout_mask, aux.dropout_rate = drop.data_ptr(), rate
-        aux.drop_row_stride, aux.drop_head_stride, aux.drop_batch_stride = d[3], d[2] * d[3], d[1] * d[2] * d[3]
-    return aux
+class _CallFrame(ctypes.Structure):
+    _fields_ = [("stream", ctypes.c_void_p), ("n_args", ctypes.c_int32), ("args", ctypes.POINTER(_Buffer)),
+                ("n_rets", ctypes.c_int32), ("rets", ctypes.POINTER(_Buffer)), ("n_attrs", ctypes.c_int32),
+                ("attrs", ctypes.POINTER(_Attr)), ("error_code", ctypes.c_int32), ("error", ctypes.c_char * 1024)]
 
 
-def _fill_decode_bias(bias):
-    out = _lib.AxlDecodeBias()
-    if _elements(bias):
-        d = bias.shape
-        assert len(d) == 3
-        out.bias, out.dtype = bias.data_ptr(), _lib.dtype_code(bias.dtype)
-        out.head_stride = 0 if d[1] == 1 else d[2]
-        out.batch_stride = 0 if d[0] == 1 else d[1] * d[2]
-    return out
+class FfiError(RuntimeError):
+    """A handler of the shim returned an xla::ffi::Error."""
+
+    def __init__(self, code: int, message: str):
+        super().__init__(f"{_ERROR_CODE.get(code, code)}: {message}")
+        self.code = code
 
 
-def _flash_fwd(ops, res, at):
-    q, k, v, segment_ids, logit_sink, bias, dropout_mask, q_pos_offsets = ops
-    out, lse = res
-    p = _lib.AxlFlashFwdParams(
-        q=q.data_ptr(), k=k.data_ptr(), v=v.data_ptr(), out=out.data_ptr(), lse=lse.data_ptr(),
-        segment_ids=_or_null(segment_ids), q_strides=_dense4(q.shape), k_strides=_dense4(k.shape),
-        v_strides=_dense4(v.shape), out_strides=_dense4(out.shape), batch=q.shape[0], q_len=q.shape[1],
-        num_q_heads=q.shape[2], head_dim=q.shape[3], kv_len=k.shape[1], num_kv_heads=k.shape[2],
-        dtype=_lib.dtype_code(q.dtype), mask_kind=at["mask_kind"], sliding_window=at["sliding_window"],
-        q_pos_offset=at["q_pos_offset"], softmax_scale=at["softmax_scale"], logit_sink=_or_null(logit_sink),
-        q_pos_offsets=_or_null(q_pos_offsets), aux=_fill_aux(bias, dropout_mask, at["dropout_rate"]))
-    return "axl_flash_fwd", p
+_shim = None
 
 
-def _flash_bwd(ops, res, at):
-    q, k, v, out, d_out, lse, segment_ids, logit_sink, bias, dropout_mask = ops
-    dq, dk, dv, d_sink, workspace = res
-    p = _lib.AxlFlashBwdParams(
-        q=q.data_ptr(), k=k.data_ptr(), v=v.data_ptr(), out=out.data_ptr(), d_out=d_out.data_ptr(), lse=lse.data_ptr(),
-        dq=dq.data_ptr(), dk=dk.data_ptr(), dv=dv.data_ptr(), segment_ids=_or_null(segment_ids),
-        q_strides=_dense4(q.shape), k_strides=_dense4(k.shape), v_strides=_dense4(v.shape),
-        out_strides=_dense4(out.shape), d_out_strides=_dense4(d_out.shape), dq_strides=_dense4(dq.shape),
-        dk_strides=_dense4(dk.shape), dv_strides=_dense4(dv.shape), batch=q.shape[0], q_len=q.shape[1],
-        num_q_heads=q.shape[2], head_dim=q.shape[3], kv_len=k.shape[1], num_kv_heads=k.shape[2],
-        dtype=_lib.dtype_code(q.dtype), mask_kind=at["mask_kind"], sliding_window=at["sliding_window"],
-        q_pos_offset=at["q_pos_offset"], softmax_scale=at["softmax_scale"], workspace=_or_null(workspace),
-        workspace_bytes=workspace.numel(), logit_sink=_or_null(logit_sink), d_logit_sink=_or_null(d_sink),
-        aux=_fill_aux(bias, dropout_mask, at["dropout_rate"]), flags=at["flags"])
-    return "axl_flash_bwd", p
+def load_shim() -> ctypes.CDLL:
+    """csrc/ffi_shim.cc built against the stand-in header (tests/xla_ffi_stand_in/Makefile; `build()` of
+    __graft_entry__.py makes it)."""
+    global _shim
+    if _shim is None:
+        if not os.path.exists(SHIM_PATH):
+            raise RuntimeError(f"{SHIM_PATH} is missing: make -C {SHIM_DIR}")
+        _lib.load()
+        _shim = ctypes.CDLL(SHIM_PATH)
+    return _shim
 
 
-def _decode(ops, res, at):
-    q, k, v, lengths, bias = ops
-    out, workspace = res
-    assert q.dim() == 3 and k.dim() == 4
-    p = _lib.AxlDecodeParams(
-        q=q.data_ptr(), k=k.data_ptr(), v=v.data_ptr(), lengths=lengths.data_ptr(), out=out.data_ptr(),
-        k_strides=_dense4(k.shape), v_strides=_dense4(v.shape), batch=q.shape[0], num_q_heads=q.shape[1],
-        head_dim=q.shape[2], kv_len=k.shape[1], num_kv_heads=k.shape[2], dtype=_lib.dtype_code(q.dtype),
-        sliding_window=at["sliding_window"], softmax_scale=at["softmax_scale"], workspace=_or_null(workspace),
-        workspace_bytes=workspace.numel(), flags=at["flags"] & _lib.DECODE_DETERMINISTIC, bias=_fill_decode_bias(bias))
-    return "axl_decode", p
+def _buffers(tensors, keep):
+    arr = (_Buffer * len(tensors))()
+    for slot, t in zip(arr, tensors):
+        dims = (ctypes.c_int64 * max(t.dim(), 1))(*t.shape)
+        keep.append(dims)
+        slot.data, slot.dtype, slot.rank, slot.dims = t.data_ptr() if t.numel() else None, _DATA_TYPE[t.dtype], t.dim(), dims
+    return arr
 
 
-def _paged_decode(ops, res, at):
-    q, k_pages, v_pages, page_tables, lengths, bias = ops
-    out, workspace = res
-    assert q.dim() == 3 and k_pages.dim() == 4 and page_tables.dim() == 2
-    p = _lib.AxlPagedDecodeParams(
-        q=q.data_ptr(), k_pages=k_pages.data_ptr(), v_pages=v_pages.data_ptr(), page_tables=page_tables.data_ptr(),
-        lengths=lengths.data_ptr(), out=out.data_ptr(), batch=q.shape[0], num_q_heads=q.shape[1], head_dim=q.shape[2],
-        num_kv_heads=k_pages.shape[0], num_pages=k_pages.shape[1], page_size=k_pages.shape[2],
-        pages_per_seq=page_tables.shape[1], dtype=_lib.dtype_code(q.dtype), sliding_window=at["sliding_window"],
-        softmax_scale=at["softmax_scale"], workspace=_or_null(workspace), workspace_bytes=workspace.numel(),
-        flags=at["flags"] & _lib.DECODE_DETERMINISTIC, bias=_fill_decode_bias(bias))
-    return "axl_paged_decode", p
-
-
-def _page_insert(ops, res, at):
-    del at
-    k_pages, v_pages, k_proj, v_proj, page_indices, key_positions = ops
-    k_out, v_out = res
-    assert k_out.data_ptr() == k_pages.data_ptr() and v_out.data_ptr() == v_pages.data_ptr()  # aliased
-    pd, jd, idd = k_pages.shape, k_proj.shape, page_indices.shape
-    assert len(pd) == 4 and len(jd) == 4 and len(idd) == 2
-    p = _lib.AxlPageInsertParams(
-        k_pages=k_out.data_ptr(), v_pages=v_out.data_ptr(), k_proj=k_proj.data_ptr(), v_proj=v_proj.data_ptr(),
-        page_indices=page_indices.data_ptr(), key_positions=key_positions.data_ptr(),
-        k_proj_batch_stride=jd[3], v_proj_batch_stride=jd[3], k_proj_head_stride=jd[1] * jd[2] * jd[3],
-        v_proj_head_stride=jd[1] * jd[2] * jd[3], batch=idd[0], pages_per_seq=idd[1], num_kv_heads=pd[0],
-        num_pages=pd[1], page_size=pd[2], head_dim=pd[3], dtype=_lib.dtype_code(k_pages.dtype),
-        broadcast_positions=int(key_positions.numel() == 1 and idd[0] > 1))
-    return "axl_paged_kv_insert", p
-
-
-# target -> (handler, operands, results, attributes with the type the shim binds them as)
-HANDLERS = {
-    "AxlFlashFwd": (_flash_fwd, 8, 2, dict(softmax_scale=np.float32, mask_kind=np.int32, sliding_window=np.int32,
-                                           q_pos_offset=np.int32, dropout_rate=np.float32)),
-    "AxlFlashBwd": (_flash_bwd, 10, 5, dict(softmax_scale=np.float32, mask_kind=np.int32, sliding_window=np.int32,
-                                            q_pos_offset=np.int32, dropout_rate=np.float32, flags=np.int32)),
-    "AxlDecode": (_decode, 5, 2, dict(softmax_scale=np.float32, sliding_window=np.int32, flags=np.int32)),
-    "AxlPagedDecode": (_paged_decode, 6, 2, dict(softmax_scale=np.float32, sliding_window=np.int32, flags=np.int32)),
-    "AxlPagedKvInsert": (_page_insert, 6, 2, {}),
-}
+def _run_handler(target, operands, results, attributes):
+    """One custom call: the frame XLA would hand to the handler, then the handler itself."""
+    keep = []
+    attrs = (_Attr * max(len(attributes), 1))()
+    for slot, (name, value) in zip(attrs, attributes.items()):
+        slot.name = name.encode()
+        if type(value) is np.int32:       # XLA FFI decodes scalars by exact type: no conversions
+            slot.kind, slot.i32 = 0, int(value)
+        elif type(value) is np.float32:
+            slot.kind, slot.f32 = 1, float(value)
+        else:
+            raise TypeError(f"{target}: attribute {name} must be np.int32 or np.float32, got {type(value)}")
+    stream = _lib.current_stream_ptr() if torch.cuda.is_available() else None
+    frame = _CallFrame(stream=stream, n_args=len(operands), args=_buffers(operands, keep),
+                       n_rets=len(results), rets=_buffers(results, keep), n_attrs=len(attributes), attrs=attrs)
+    handler = getattr(load_shim(), target)
+    handler.restype, handler.argtypes = ctypes.c_int, [ctypes.POINTER(_CallFrame)]
+    if handler(ctypes.byref(frame)) != 0:
+        raise FfiError(frame.error_code, frame.error.decode())
 
 
 def _ffi_call(state: State):
     def ffi_call(target, result_types, input_output_aliases=None):
-        handler, n_operands, n_results, attr_types = HANDLERS[target]
         assert any(t == target for t, _ in state.registered), f"{target} was never registered"
 
         def call(*operands, **attributes):
-            assert len(operands) == n_operands and len(result_types) == n_results, target
-            assert list(attributes) == list(attr_types), (target, list(attributes))
-            for name, value in attributes.items():  # XLA FFI decodes attributes by exact type
-                assert type(value) is attr_types[name], (target, name, type(value))
             device = operands[0].device
-            aliases = input_output_aliases or {}
-            alias_of = {r: o for o, r in aliases.items()}
+            alias_of = {r: o for o, r in (input_output_aliases or {}).items()}
             results = []
             for i, rt in enumerate(result_types):
-                if i in alias_of:
+                if i in alias_of:   # a donated operand: XLA hands its buffer back as the result
                     src = operands[alias_of[i]]
                     assert tuple(src.shape) == rt.shape and src.dtype == rt.dtype
                     results.append(src)
@@ -233,10 +180,9 @@ def _ffi_call(state: State):
             state.calls.append((target, [tuple(o.shape) for o in operands],
                                 {k: v.item() for k, v in attributes.items()}, [tuple(r.shape) for r in results]))
             if state.execute:
-                for o in operands:
+                for o in operands:   # XLA buffers are dense and live on the device
                     assert o.numel() == 0 or (o.device.type == "cuda" and o.is_contiguous()), (target, o.shape, o.device)
-                entry, params = handler(operands, results, {k: v.item() for k, v in attributes.items()})
-                _lib.check(getattr(_lib.load(), entry)(ctypes.byref(params), _lib.current_stream_ptr()))
+                _run_handler(target, operands, results, attributes)
             return tuple(results)
 
         return call
@@ -313,7 +259,7 @@ def installed():
 
     def cdll(path, *args, **kwargs):
         if str(path).endswith("libaxl_attn_ffi.so"):   # the compiled shim: its symbols are only registered
-            return types.SimpleNamespace(**{target: target for target in HANDLERS})
+            return types.SimpleNamespace(**{target: target for target in TARGETS})
         return real_cdll(path, *args, **kwargs)
 
     sys.modules.update(fakes)

@@ -626,9 +626,8 @@ def test_forward_kernel_keeps_the_distance_behind_its_assembly_mfma_chains():
 
 
 def test_ffi_shim_and_jax_side_stay_in_step_with_the_abi():
-    """csrc/ffi_shim.cc cannot be compiled here (no jaxlib headers) and flash_attention/jax_ffi.py only runs
-    under stand-ins (test_jax_side.py), so an ABI change could leave the pair behind unnoticed.  Checked
-    from their text:
+    """csrc/ffi_shim.cc and flash_attention/jax_ffi.py only build and run under stand-ins here
+    (test_jax_side.py: no jaxlib headers, no jax), so the pair is also checked from its text:
     every field the shim fills exists in the header's structure of that name (through the ctypes mirror,
     itself checked against the header), every handler binds as many operands, results and attributes -
     by name - as the JAX side passes to `jax.ffi.ffi_call`, and every registered target has a handler."""

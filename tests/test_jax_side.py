@@ -3,6 +3,7 @@ tests/jax_stand_in.py (jax is not installed here): see that module for what this
 
 import ctypes
 
+import numpy as np
 import pytest
 import torch
 
@@ -23,12 +24,37 @@ def _size_query(b, t, s, hq, hkv, d, mask_kind, has_seg, flags):
 
 def test_jax_side_imports_and_registers_every_target():
     with jax_stand_in.installed() as (mod, state):
-        assert sorted(state.registered) == sorted((t, "ROCM") for t in jax_stand_in.HANDLERS)
+        assert sorted(state.registered) == sorted((t, "ROCM") for t in jax_stand_in.TARGETS)
         for name in ("flash_attention", "HipFlashAttention", "HipDecoding", "HipPagedAttention", "hip_scatter_update_pages"):
             assert hasattr(mod, name)
     import sys
 
     assert "jax" not in sys.modules and jax_stand_in.JAX_SIDE not in sys.modules and not hasattr(torch.Tensor, "astype")
+
+
+def test_shim_builds_against_the_stand_in_header_and_checks_its_frame():
+    """csrc/ffi_shim.cc compiled against tests/xla_ffi_stand_in (not jaxlib's header, which is absent
+    here): the library loads without a GPU, exports a handler per target, and a handler given a frame
+    that does not match its binding - operand count, attribute type, attribute name - says so before
+    any kernel entry point is reached."""
+    shim = jax_stand_in.load_shim()
+    for target in jax_stand_in.TARGETS:
+        assert hasattr(shim, target)
+    x = torch.zeros((2, 4, 8), dtype=torch.bfloat16)
+    ok_attrs = dict(softmax_scale=np.float32(1.0), sliding_window=np.int32(-1), flags=np.int32(0))
+    with pytest.raises(jax_stand_in.FfiError, match="wrong number of operands") as err:
+        jax_stand_in._run_handler("AxlDecode", [x] * 4, [x, x], ok_attrs)
+    assert err.value.code == 3
+    with pytest.raises(jax_stand_in.FfiError, match="attribute sliding_window has the wrong type"):
+        jax_stand_in._run_handler("AxlDecode", [x] * 5, [x, x], dict(ok_attrs, sliding_window=np.float32(-1)))
+    renamed = dict(softmax_scale=np.float32(1.0), window=np.int32(-1), flags=np.int32(0))
+    with pytest.raises(jax_stand_in.FfiError, match="attribute sliding_window is missing"):
+        jax_stand_in._run_handler("AxlDecode", [x] * 5, [x, x], renamed)
+    with pytest.raises(TypeError, match="must be np.int32 or np.float32"):
+        jax_stand_in._run_handler("AxlDecode", [x] * 5, [x, x], dict(ok_attrs, flags=0))
+    # ranks are checked by the handler itself, again before the library is called
+    with pytest.raises(jax_stand_in.FfiError, match=r"q must be \[B,Hq,D\]"):
+        jax_stand_in._run_handler("AxlDecode", [x] * 5, [x, x], ok_attrs)
 
 
 @pytest.mark.parametrize("shape,seg,want_flags", [
@@ -192,3 +218,27 @@ def test_jax_side_decode_classes_and_page_insert():
         ops.paged_kv_insert(k2, v2, kproj[:, :, 0].transpose(0, 1), vproj[:, :, 0].transpose(0, 1), tables, positions)
         k1, v1 = mod.hip_scatter_update_pages(kp, vp, kproj, vproj, tables, positions)
         assert k1.data_ptr() == kp.data_ptr() and torch.equal(k1, k2) and torch.equal(v1, v2)
+
+
+@pytest.mark.gpu
+def test_shim_reports_the_library_errors_as_ffi_errors():
+    """A request the library declines comes back as UNIMPLEMENTED with the library's message, a malformed
+    one as INVALID_ARGUMENT (`Fail` in the shim): what XLA would raise as an XlaRuntimeError."""
+    b, hq, hkv, d = 2, 4, 2, 128
+    q = torch.zeros((b, hq, d), dtype=torch.bfloat16, device="cuda")
+    pools = torch.zeros((hkv, 8, 8, d), dtype=torch.bfloat16, device="cuda")    # 8-token pages
+    tables = torch.zeros((b, 4), dtype=torch.int32, device="cuda")
+    lengths = torch.full((b,), 5, dtype=torch.int32, device="cuda")
+    none = torch.zeros((0,), device="cuda")
+    out, ws = torch.empty_like(q), torch.empty((1 << 20,), dtype=torch.uint8, device="cuda")
+    attrs = dict(softmax_scale=np.float32(1.0), sliding_window=np.int32(-1), flags=np.int32(0))
+    with pytest.raises(jax_stand_in.FfiError, match="page") as err:
+        jax_stand_in._run_handler("AxlPagedDecode", [q, pools, pools, tables, lengths, none], [out, ws], attrs)
+    assert err.value.code == 12
+    pools16 = torch.zeros((hkv, 8, 16, d), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(jax_stand_in.FfiError, match="workspace") as err:
+        jax_stand_in._run_handler("AxlPagedDecode", [q, pools16, pools16, tables, lengths, none], [out, ws[:16]], attrs)
+    assert err.value.code == 3
+    jax_stand_in._run_handler("AxlPagedDecode", [q, pools16, pools16, tables, lengths, none], [out, ws], attrs)
+    torch.cuda.synchronize()
+    assert torch.equal(out, torch.zeros_like(out))   # all-zero V rows
