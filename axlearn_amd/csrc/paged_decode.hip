@@ -67,6 +67,7 @@ struct DecArgs {
   int* ticket;                 // [0] blocks handed out: zero when the split kernel starts (zeroed by
                                // decode_plan_kernel, or left at zero by the previous call's combine kernel)
   int deterministic;           // fixed work decomposition: results reproducible bit for bit
+  int static_only;             // no more blocks than workgroups: block i goes to workgroup i, the counter is not used
 };
 
 // Tokens per tile: the unit the kernels stream and compute on.  A pool page of 16 << page_shift
@@ -248,7 +249,7 @@ __global__ __launch_bounds__(256) void decode_split_kernel(const DecArgs a) {
   const int rec = run_e;
   if (tid == 0 && first_segment) {
     next_n = min(max_run, max(1, (n_blocks - handed) / (4 * n_wg)));
-    next_e = atomicAdd(&a.ticket[0], next_n);
+    next_e = a.static_only ? n_blocks : atomicAdd(&a.ticket[0], next_n);
   }
   first_segment = false;
 
@@ -763,9 +764,21 @@ __global__ __launch_bounds__(256) void decode_split_f32_kernel(const DecArgs a) 
 constexpr int kStages128 = 2;
 constexpr int kStages64 = 4;
 
-static int pick_chunk_pages(int pps) {
+// Workgroups the split kernel keeps resident on the GPU it is tuned for (two on each of 256 CUs).
+constexpr int kSplitSlots = 512;
+
+// Pages per block of work.  `rows` = (sequence, kv head group) pairs of the call.
+static int pick_chunk_pages(int pps, int64_t rows) {
   // 32 pages = 512 tokens = 256 KB of K+V per workgroup at head_dim 128.
   int cp = 32;
+  // A small call (one sequence, a short context) has fewer such blocks than the GPU has workgroup slots
+  // and is bound by the latency of a block's few rounds of loads: shorter blocks, about one per slot,
+  // down to 8 pages (one round of the four wavefronts' rings).
+  if (rows > 0 && rows * ((pps + cp - 1) / cp) < kSplitSlots) {
+    const int64_t per_row = kSplitSlots / rows;
+    cp = (int)(((pps + per_row - 1) / per_row + 3) / 4 * 4);
+    cp = cp < 8 ? 8 : (cp > 32 ? 32 : cp);
+  }
   if (pps < cp) cp = ((pps + 3) / 4) * 4;
   if (pps > cp * kMaxChunks) cp = ((pps + kMaxChunks - 1) / kMaxChunks + 3) / 4 * 4;
   return cp < 4 ? 4 : cp;
@@ -793,7 +806,7 @@ static int page_shift_of(int page_size) {
 
 static size_t ws_bytes_for(int batch, int hq, int hkv, int d, int tiles, bool bias) {
   const int G = hq / hkv;
-  const int cp = pick_chunk_pages(tiles);
+  const int cp = pick_chunk_pages(tiles, (int64_t)batch * hkv * groups_of(G));
   const int nch = (tiles + cp - 1) / cp;
   return ws_bytes(batch, hkv * groups_of(G), nch, gp_of(G, bias), width_of(d));
 }
@@ -848,7 +861,7 @@ static int launch_common(DecArgs a, int flags, hipStream_t stream, const char* w
   const int gp = gp_of(a.G, bias);
   a.ngrp = groups_of(a.G);
   a.Hv = a.Hkv * a.ngrp;
-  a.chunk_pages = pick_chunk_pages(a.pps);
+  a.chunk_pages = pick_chunk_pages(a.pps, (int64_t)a.B * a.Hv);
   if (a.chunk_pages > 256)
     return set_error(AXL_ERR_UNSUPPORTED, "%s: context longer than %d tokens", who, 256 * kMaxChunks * kPage);
   a.nch = (a.pps + a.chunk_pages - 1) / a.chunk_pages;
@@ -866,7 +879,10 @@ static int launch_common(DecArgs a, int flags, hipStream_t stream, const char* w
   // Two workgroups fit a CU (LDS); the split kernel is persistent and strides over its work items.
   const dim3 grid(2 * cu_count());
   hipError_t err = hipSuccess;
-  if (!(flags & AXL_DECODE_WORKSPACE_REUSED))
+  // With at most one block per workgroup (a bound the shapes give: the lengths live on the device) the
+  // blocks are dealt by workgroup index and the counter is neither read nor zeroed.
+  a.static_only = (int64_t)(a.B < kMaxBatch ? a.B : kMaxBatch) * a.Hv * a.nch <= (int64_t)grid.x;
+  if (!(flags & AXL_DECODE_WORKSPACE_REUSED) && !a.static_only)
     hipLaunchKernelGGL(decode_plan_kernel, dim3(1), dim3(64), 0, stream, a.ticket);
 #define AXL_DEC(E, DD, GG, NS, BB)                                                              \
   do {                                                                                          \
@@ -916,7 +932,7 @@ static int launch_f32(DecArgs a, hipStream_t stream, const char* who) {
   const int gp = gp_of(a.G, a.bias != nullptr);
   a.ngrp = groups_of(a.G);
   a.Hv = a.Hkv * a.ngrp;
-  a.chunk_pages = pick_chunk_pages(a.pps);
+  a.chunk_pages = pick_chunk_pages(a.pps, (int64_t)a.B * a.Hv);
   if (a.chunk_pages > 256)
     return set_error(AXL_ERR_UNSUPPORTED, "%s: context longer than %d tokens", who, 256 * kMaxChunks * kPage);
   if (a.B > 65535) return set_error(AXL_ERR_UNSUPPORTED, "%s: more than 65535 sequences in fp32", who);

@@ -8,13 +8,13 @@ per combination, milliseconds per call.  The kernels are reached the way the ref
 reaches them: through the kernel classes' `is_supported` + `__call__` (`HipFlashAttention`,
 `HipDecoding`), with the mask given as an attention bias.
 
-Differences in method: the time is the median of `--iters` calls between device events after
-`--warmup` calls, instead of one call behind two large GEMMs (:163-206).  The reference times a
-jitted function, i.e. device work without per-call Python; here the forward-only and decode calls are
-captured into a graph once and the replays are timed, for the same reason (`--eager` times plain
-calls, which for the smallest shapes measures this module's Python).  `use_bwd=True` times the
-forward and the backward of `mean(out)` together, eagerly, which is what `jax.grad` of the forward
-computes.
+Method, as the reference's `measure` (:163-206): every timed call is enqueued behind two large GEMMs, so
+that the device events bracket device work and neither the launch latency of an idle GPU (25 us here,
+more than the smallest decode calls take) nor this module's Python, which runs while the GEMMs do; the
+time is the median of `--iters` such calls after `--warmup` calls (the reference reports one).
+`--graph` captures the forward-only and decode calls once and times the replays instead (a replay has a
+floor of 13 us here, whatever it holds).  `use_bwd=True` times the forward and the backward of `mean(out)`
+together, which is what `jax.grad` of the forward computes.
 
 Run: python -m axlearn_amd.flash_attention.hip_attention_benchmark [--quick] [--iters N]
 """
@@ -35,9 +35,10 @@ from axlearn_amd.kv_cache import KVCache
 
 
 def _bias(q_len: int, kv_len: int, sw_sz: int, query_offset: int, device) -> ab.BaseAttentionBias:
+    # int32 positions, as jnp.arange gives the reference's benchmark
     pos = dict(
-        target_positions=(torch.arange(q_len, device=device) + query_offset)[None],
-        source_positions=torch.arange(kv_len, device=device)[None],
+        target_positions=(torch.arange(q_len, device=device, dtype=torch.int32) + query_offset)[None],
+        source_positions=torch.arange(kv_len, device=device, dtype=torch.int32)[None],
     )
     if sw_sz != -1:
         return ab.CompositeAttentionBias([
@@ -48,7 +49,9 @@ def _bias(q_len: int, kv_len: int, sw_sz: int, query_offset: int, device) -> ab.
 
 def measure(fn, warmup: int, iters: int, graph: bool = False) -> float:
     """Median milliseconds of `fn()` over `iters` calls, timed with device events; with `graph` the
-    call is captured once and its replays are timed."""
+    call is captured once and its replays are timed.  Each timed call is enqueued while two large GEMMs
+    still run ahead of it, so its launch is hidden and the events see device time only
+    (gpu_attention_benchmark.py:163-206)."""
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
@@ -63,9 +66,12 @@ def measure(fn, warmup: int, iters: int, graph: bool = False) -> float:
         fn = captured.replay
         fn()
         torch.cuda.synchronize()
+    x = torch.ones((8192, 8192), dtype=torch.float16, device="cuda")   # a GEMM of about a millisecond
     times = []
     for _ in range(iters):
         start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for _ in range(2):
+            _ = x @ x
         start.record()
         fn()
         end.record()
@@ -87,7 +93,7 @@ def bench_flash_attention(
     dtype=torch.float16,
     warmup: int = 3,
     iters: int = 10,
-    graph: bool = True,
+    graph: bool = False,
 ) -> float:
     if use_bwd and is_decode:
         raise ValueError("use_bwd and is_decode cannot both be true.")
@@ -152,9 +158,9 @@ def main() -> None:
     ap.add_argument("--quick", action="store_true", help="a subset of every sweep")
     ap.add_argument("--iters", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--eager", action="store_true", help="time plain calls instead of graph replays")
+    ap.add_argument("--graph", action="store_true", help="time graph replays instead of plain calls")
     args = ap.parse_args()
-    opts = dict(warmup=args.warmup, iters=args.iters, graph=not args.eager)
+    opts = dict(warmup=args.warmup, iters=args.iters, graph=args.graph)
     benchmark_decode(opts, args.quick)
     benchmark_prefill(opts, use_bwd=False, quick=args.quick)
     benchmark_prefill(opts, use_bwd=True, quick=args.quick)
