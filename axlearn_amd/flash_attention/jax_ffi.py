@@ -13,11 +13,12 @@ side's bits with the workspace sizes computed here; XLA, jax's own machinery and
 real header stay untested.
 
 It mirrors, name for name:
-  * `flash_attention` with its `jax.custom_vjp` and residuals `(q, k, v, bias, segment_ids, prng_key,
-    out, lse)` (gpu_attention.py:247-287, :420-424, :789): `out` and `lse` carry
+  * `flash_attention` with its `jax.custom_vjp` and residuals `(q, k, v, bias, segment_ids, dropout mask,
+    logit_sink, out, lse)` (gpu_attention.py:247-287, :420-424, :789): `out` and `lse` carry
     `checkpoint_name(..., f"gpu_attention.{FLASH_ATTN_RESIDUAL_NAME}")`, the name the remat policy
     `save_and_offload_only_these_names_regex` matches (axlearn/common/flash_attention/remat.py:9-58);
-  * `PallasGPUFlashAttention` (gpu_attention.py:929-992) as `HipFlashAttention`, `GPUDecoding`
+  * `PallasGPUFlashAttention` (gpu_attention.py:929-992) as `HipFlashAttention` (any head_dim up to 128,
+    `logit_sink`, and incremental prefill over a contiguous cache, as the torch-side class), `GPUDecoding`
     (gpu_decoding.py:286-352) as `HipDecoding`, `GPUPagedAttention` (gpu_paged_attention.py:299-379)
     as `HipPagedAttention`, to be listed first in `BACKENDS["gpu"]` / `PAGED_ATTN_BACKENDS["gpu"]`
     (flash_attention/utils.py:31-58);
@@ -110,14 +111,14 @@ def _bwd_workspace_bytes(b, t, s, hq, hkv, d, dtype_code, mask_kind, has_seg, fl
 _DTYPE_CODE = {jnp.dtype(jnp.bfloat16): 0, jnp.dtype(jnp.float32): 1, jnp.dtype(jnp.float16): 2}
 
 
-@functools.partial(jax.custom_vjp, nondiff_argnums=(6, 7, 8, 9, 10))
-def flash_attention(query, key, value, bias, segment_ids, dropout_mask, softmax_scale, mask_kind,
-                    sliding_window, dropout_rate, logit_sink_present):
+@functools.partial(jax.custom_vjp, nondiff_argnums=(7, 8, 9, 10))
+def flash_attention(query, key, value, bias, segment_ids, dropout_mask, logit_sink, softmax_scale, mask_kind,
+                    sliding_window, dropout_rate):
     """Same contract as gpu_attention.py:250-287 with the block-size / warp arguments gone (the kernels
-    pick their own tiles) and the dropout mask instead of the prng key (drawn by the caller with
-    `jax.random.bernoulli(prng_key, dropout_rate, [B,H,T,S])`, as :374-385 does before its kernel)."""
-    del logit_sink_present
-    out, _ = _fwd_call(query, key, value, bias, segment_ids, dropout_mask, None, softmax_scale, mask_kind,
+    pick their own tiles), the dropout mask instead of the prng key (drawn by the caller with
+    `jax.random.bernoulli(prng_key, dropout_rate, [B,H,T,S])`, as :374-385 does before its kernel), and
+    `logit_sink` [Hq] (attention.py:608-626; None for none), which gets a gradient like q, k and v."""
+    out, _ = _fwd_call(query, key, value, bias, segment_ids, dropout_mask, logit_sink, softmax_scale, mask_kind,
                        sliding_window, dropout_rate)
     return out
 
@@ -138,21 +139,19 @@ def _fwd_call(query, key, value, bias, segment_ids, dropout_mask, logit_sink, so
         sliding_window=np.int32(sliding_window), q_pos_offset=np.int32(0), dropout_rate=np.float32(dropout_rate))
 
 
-def _flash_fwd(query, key, value, bias, segment_ids, dropout_mask, softmax_scale, mask_kind, sliding_window,
-               dropout_rate, logit_sink_present):
-    del logit_sink_present
-    out, lse = _fwd_call(query, key, value, bias, segment_ids, dropout_mask, None, softmax_scale, mask_kind,
+def _flash_fwd(query, key, value, bias, segment_ids, dropout_mask, logit_sink, softmax_scale, mask_kind,
+               sliding_window, dropout_rate):
+    out, lse = _fwd_call(query, key, value, bias, segment_ids, dropout_mask, logit_sink, softmax_scale, mask_kind,
                          sliding_window, dropout_rate)
     # The names the remat policy looks for (remat.py:13-58): saving or offloading exactly these two
     # tensors lets the backward skip the forward kernel.
     out = checkpoint_name(out, f"gpu_attention.{FLASH_ATTN_RESIDUAL_NAME}")
     lse = checkpoint_name(lse, f"gpu_attention.{FLASH_ATTN_RESIDUAL_NAME}")
-    return out, (query, key, value, bias, segment_ids, dropout_mask, out, lse)
+    return out, (query, key, value, bias, segment_ids, dropout_mask, logit_sink, out, lse)
 
 
-def _flash_bwd(softmax_scale, mask_kind, sliding_window, dropout_rate, logit_sink_present, res, d_out):
-    del logit_sink_present
-    query, key, value, bias, segment_ids, dropout_mask, out, lse = res
+def _flash_bwd(softmax_scale, mask_kind, sliding_window, dropout_rate, res, d_out):
+    query, key, value, bias, segment_ids, dropout_mask, logit_sink, out, lse = res
     b, t, hq, d = query.shape
     s, hkv = key.shape[1], key.shape[2]
     size_args = (b, t, s, hq, hkv, d, _DTYPE_CODE[jnp.dtype(query.dtype)], mask_kind, segment_ids is not None)
@@ -168,26 +167,69 @@ def _flash_bwd(softmax_scale, mask_kind, sliding_window, dropout_rate, logit_sin
             heads -= 1
         flags = flags | (heads << 8) if heads >= 1 and heads * per_head >= 256 else 0
         ws_bytes = _bwd_workspace_bytes(*size_args, flags)
-    dq, dk, dv, _, _ = jax.ffi.ffi_call(
+    dq, dk, dv, d_sink, _ = jax.ffi.ffi_call(
         "AxlFlashBwd",
         (jax.ShapeDtypeStruct(query.shape, query.dtype), jax.ShapeDtypeStruct(key.shape, key.dtype),
-         jax.ShapeDtypeStruct(value.shape, value.dtype), jax.ShapeDtypeStruct((0,), jnp.float32),
+         jax.ShapeDtypeStruct(value.shape, value.dtype),
+         jax.ShapeDtypeStruct((0,) if logit_sink is None else (hq,), jnp.float32),
          jax.ShapeDtypeStruct((ws_bytes,), jnp.uint8)),
     )(query, key, value, out, d_out, lse,
-      _empty(jnp.int32) if segment_ids is None else segment_ids.astype(jnp.int32), _empty(jnp.float32),
+      _empty(jnp.int32) if segment_ids is None else segment_ids.astype(jnp.int32),
+      _empty(jnp.float32) if logit_sink is None else logit_sink.astype(jnp.float32),
       _empty(jnp.float32) if bias is None else bias,
       _empty(jnp.uint8) if dropout_mask is None else dropout_mask.astype(jnp.uint8),
       softmax_scale=np.float32(softmax_scale), mask_kind=np.int32(mask_kind), sliding_window=np.int32(sliding_window),
       q_pos_offset=np.int32(0), dropout_rate=np.float32(dropout_rate), flags=np.int32(flags))
     # No gradient for bias, segment ids or the dropout mask, as `_mha_backward` returns (:786).
-    return dq, dk, dv, None, None, None
+    return dq, dk, dv, None, None, None, (None if logit_sink is None else d_sink.astype(logit_sink.dtype))
 
 
 flash_attention.defvjp(_flash_fwd, _flash_bwd)
 
 
+def _width(head_dim: int):
+    """Compiled width the kernels run a head dim at: 64 or 128 (None above that, gpu_attention.py:954)."""
+    return 64 if head_dim <= 64 else (128 if head_dim <= 128 else None)
+
+
+def _runs_at_native_head_dim(query: Tensor, key: Tensor, aux: bool) -> bool:
+    """Head dims 64 and 128 always; other multiples of 8 in bf16 / f16 without bias or dropout mask when
+    the (dense) rows are at least one compiled width apart.  Everything else is zero-padded to the width:
+    zero columns of q / k add nothing to the logits, zero columns of v give output columns that are
+    sliced off again (the Pallas kernel pads inside its blocks instead, gpu_attention.py:172-176)."""
+    d = query.shape[-1]
+    if d in (64, 128):
+        return True
+    if d % 8 != 0 or aux or query.dtype == jnp.float32:
+        return False
+    return query.shape[2] * d >= _width(d) and key.shape[2] * d >= _width(d)
+
+
+def _pad_last(x: Tensor, width: int) -> Tensor:
+    return x if x.shape[-1] == width else jnp.pad(x, ((0, 0),) * (x.ndim - 1) + ((0, width - x.shape[-1]),))
+
+
 class HipFlashAttention(BaseFlashAttention):
-    """Stands where `PallasGPUFlashAttention` does (gpu_attention.py:929-992)."""
+    """Stands where `PallasGPUFlashAttention` does (gpu_attention.py:929-992).  With `kv_cache_type=KVCache`
+    and more than one query row it serves incremental prefill (utils_test.py:361-478): a chunk of queries
+    per sequence at its own offset into the contiguous cache, forward only."""
+
+    _kv_cache_type = None
+
+    def _incremental_supported(self, input_batch) -> bool:
+        query, key = input_batch["query"], input_batch["key"]
+        if key.shape[1] % 128 != 0:
+            return self._log_unsupported(f"{key.shape[1]=} is not divisible by 128")
+        if self.config.dropout_rate != 0.0:
+            raise ValueError("Dropout rate cannot be set for decoding!")
+        mask, segment_ids, explicit = split(input_batch["bias"], MaskFnAttentionBias, SegmentIdAttentionBias)
+        if segment_ids.has_value() or explicit.has_value():
+            return self._log_unsupported("incremental prefill takes a causal or sliding-window mask only.")
+        if not isinstance(mask, (CausalAttentionBias, SlidingWindowAttentionBias)) or mask.target_positions is None:
+            return self._log_unsupported("incremental prefill needs a causal / sliding-window mask with target_positions.")
+        if mask.target_positions.shape[1] != query.shape[1]:
+            return self._log_unsupported("target_positions do not match the query length.")
+        return True
 
     def is_supported(self, input_batch: Nested[Tensor | BaseAttentionBias], kv_cache_type=None) -> bool:
         if not super().is_supported(input_batch=input_batch, kv_cache_type=kv_cache_type):
@@ -195,14 +237,41 @@ class HipFlashAttention(BaseFlashAttention):
         query, key = input_batch["query"], input_batch["key"]
         if query.dtype not in (jnp.bfloat16, jnp.float16, jnp.float32) or key.dtype != query.dtype:
             return self._log_unsupported(f"{query.dtype=} / {key.dtype=}")
-        if not self._check_block_size(input_batch=input_batch, block_size=128):
+        if kv_cache_type is not None:
+            if kv_cache_type.__name__ != "KVCache":
+                return self._log_unsupported(f"{kv_cache_type=}")
+            if not self._incremental_supported(input_batch):
+                return False
+        elif not self._check_block_size(input_batch=input_batch, block_size=128):
             return False
-        if query.shape[-1] not in (64, 128):
-            return self._log_unsupported(f"head_dim {query.shape[-1]} (supported: 64, 128)")
+        self._kv_cache_type = kv_cache_type
+        if _width(query.shape[-1]) is None:
+            return self._log_unsupported(f"head_dim {query.shape[-1]} > 128")
+        if self.config.dropout_rate > 0.0 and input_batch.get("prng_key", None) is None:
+            return self._log_unsupported("dropout needs input_batch['prng_key'].")
         return True
+
+    def _incremental_prefill(self, input_batch) -> Tensor:
+        """Queries at per-sequence offsets into the cache; rows padded up to the 128-row block.  The
+        positions of a chunk are taken to be consecutive (they are, in `extend_step`)."""
+        cfg = self.config
+        query, key, value = input_batch["query"], input_batch["key"], input_batch["value"]
+        mask, _, _ = split(input_batch["bias"], MaskFnAttentionBias, SegmentIdAttentionBias)
+        window = int(mask.sliding_window_size) if isinstance(mask, SlidingWindowAttentionBias) else 0
+        b, t, _, d = query.shape
+        offsets = jnp.broadcast_to(mask.target_positions[:, 0], (b,)).astype(jnp.int32)
+        width = d if _runs_at_native_head_dim(query, key, aux=False) else _width(d)
+        rows = -(-t // 128) * 128
+        q = jnp.pad(query, ((0, 0), (0, rows - t), (0, 0), (0, width - d)))
+        out, _ = _fwd_call(q, _pad_last(key, width), _pad_last(value, width), None, None, None,
+                           input_batch.get("logit_sink", None), cfg.softmax_scale,
+                           MASK_SLIDING_WINDOW if window else MASK_CAUSAL, window, 0.0, q_pos_offsets=offsets)
+        return out[:, :t, :, :d]
 
     @functools.partial(jax.jit, static_argnames=["self"])
     def __call__(self, input_batch: Nested[Tensor | BaseAttentionBias]) -> Tensor:
+        if self._kv_cache_type is not None:
+            return self._incremental_prefill(input_batch)
         cfg = self.config
         query, key, value = input_batch["query"], input_batch["key"], input_batch["value"]
         mask_kind, window, segment_ids, dense = _mask_of(input_batch["bias"])
@@ -210,9 +279,13 @@ class HipFlashAttention(BaseFlashAttention):
         if cfg.dropout_rate > 0.0:
             b, t, hq, _ = query.shape
             dropout_mask = jax.random.bernoulli(input_batch["prng_key"], cfg.dropout_rate, (b, hq, t, key.shape[1]))
+        d = query.shape[-1]
+        if not _runs_at_native_head_dim(query, key, aux=dense is not None or dropout_mask is not None):
+            query, key, value = (_pad_last(x, _width(d)) for x in (query, key, value))
         # K / V keep their Hkv heads: no repeat_kv_heads (gpu_attention.py:975-976 repeats them).
-        return flash_attention(query, key, value, dense, segment_ids, dropout_mask, cfg.softmax_scale, mask_kind,
-                               window, cfg.dropout_rate, False)
+        out = flash_attention(query, key, value, dense, segment_ids, dropout_mask, input_batch.get("logit_sink", None),
+                              cfg.softmax_scale, mask_kind, window, cfg.dropout_rate)
+        return out[..., :d]
 
 
 def _lengths(bias: BaseAttentionBias, batch: int) -> Tensor:

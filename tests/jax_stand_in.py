@@ -205,6 +205,12 @@ def _numpy_like(state: State):
         return torch.where(cond, a, b)
 
     jnp.where = where
+
+    def pad(x, pad_width):   # ((before, after), ...) per dimension, zeros
+        flat = [n for pair in reversed(pad_width) for n in pair]
+        return torch.nn.functional.pad(x, flat) if any(flat) else x
+
+    jnp.pad = pad
     return jnp
 
 

@@ -75,7 +75,7 @@ def test_custom_vjp_pair_sizes_the_workspace_as_the_library_asks(shape, seg, wan
         mk = lambda *dims: torch.empty(dims, dtype=torch.bfloat16, device="meta")
         q, k, v = mk(b, t, hq, d), mk(b, s, hkv, d), mk(b, s, hkv, d)
         ids = torch.empty((b, t), dtype=torch.int64, device="meta") if seg else None
-        args = (q, k, v, None, ids, None, d ** -0.5, mod.MASK_CAUSAL, 0, 0.0, False)
+        args = (q, k, v, None, ids, None, None, d ** -0.5, mod.MASK_CAUSAL, 0, 0.0)
         out, pullback = mod.flash_attention.vjp(*args)
         assert state.checkpoint_names == [RESIDUAL, RESIDUAL]
         target, operands, attrs, results = state.calls[0]
@@ -83,7 +83,7 @@ def test_custom_vjp_pair_sizes_the_workspace_as_the_library_asks(shape, seg, wan
         assert operands[3] == ((b, t) if seg else (0,)) and operands[4:] == [(0,)] * 4
         assert attrs["mask_kind"] == 1 and abs(attrs["softmax_scale"] - d ** -0.5) < 1e-7
         grads = pullback(torch.empty_like(out))
-        assert len(grads) == 6 and grads[3:] == (None, None, None)
+        assert len(grads) == 7 and grads[3:] == (None, None, None, None)
         assert [tuple(g.shape) for g in grads[:3]] == [tuple(x.shape) for x in (q, k, v)]
         target, operands, attrs, results = state.calls[1]
         assert target == "AxlFlashBwd" and attrs["flags"] == want_flags
@@ -101,7 +101,7 @@ def test_forced_choices_of_the_backward_workspace():
     with jax_stand_in.installed() as (mod, state):
         state.execute, state.device = False, "meta"
         mk = lambda h: torch.empty((b, t, h, d), dtype=torch.float16, device="meta")
-        args = (mk(hq), mk(hkv), mk(hkv), None, None, None, 0.1, mod.MASK_SLIDING_WINDOW, 100, 0.0, False)
+        args = (mk(hq), mk(hkv), mk(hkv), None, None, None, None, 0.1, mod.MASK_SLIDING_WINDOW, 100, 0.0)
         for forced, flags in ((False, 0), (True, 1)):
             mod.BWD_DS_WORKSPACE = forced
             out, pullback = mod.flash_attention.vjp(*args)
@@ -140,7 +140,7 @@ def test_jax_side_flash_attention_runs_the_kernels_like_the_torch_side(window, s
         assert fa.is_supported(batch, kv_cache_type=None)
         assert torch.equal(fa(batch), want_out)
         assert state.calls[-1][0] == "AxlFlashFwd" and state.calls[-1][2]["mask_kind"] == kw["mask_kind"]
-        out, pullback = mod.flash_attention.vjp(q, k, v, None, ids, None, scale, kw["mask_kind"], kw["sliding_window"], 0.0, False)
+        out, pullback = mod.flash_attention.vjp(q, k, v, None, ids, None, None, scale, kw["mask_kind"], kw["sliding_window"], 0.0)
         assert torch.equal(out, want_out) and state.checkpoint_names == [RESIDUAL, RESIDUAL]
         dq, dk, dv = pullback(do)[:3]
         assert state.calls[-1][2]["flags"] == 1   # the dS workspace fits
@@ -171,12 +171,98 @@ def test_jax_side_flash_attention_with_bias_and_dropout():
         want, lse = ops.flash_fwd(q, k, v, softmax_scale=0.125, mask_kind=ops.MASK_NONE, bias=full,
                                   dropout_mask=drop, dropout_rate=rate)
         assert torch.equal(got, want)
-        out, pullback = mod.flash_attention.vjp(q, k, v, full, None, drop, 0.125, 0, 0, rate, False)
+        out, pullback = mod.flash_attention.vjp(q, k, v, full, None, drop, None, 0.125, 0, 0, rate)
         grads = pullback(do)
         exp = ops.flash_bwd(q, k, v, want, lse, do, softmax_scale=0.125, mask_kind=ops.MASK_NONE, bias=full,
                             dropout_mask=drop, dropout_rate=rate)[:3]
         for g, e in zip(grads[:3], exp):
             assert torch.equal(g, e)
+
+
+@pytest.mark.gpu
+def test_jax_side_logit_sink_gets_a_gradient():
+    """`logit_sink` is a differentiable argument of the custom_vjp: the forward passes it to the kernel,
+    the backward declares the [Hq] result and returns it; same bits as the torch side."""
+    b, t, hq, hkv, d = 2, 256, 8, 4, 128
+    q, k, v, do = _inputs(b, t, hq, hkv, d, torch.bfloat16, seed=4)
+    sink = torch.linspace(-1.0, 2.0, hq).cuda()
+    kw = dict(softmax_scale=d ** -0.5, mask_kind=ops.MASK_CAUSAL, logit_sink=sink)
+    want_out, want_lse = ops.flash_fwd(q, k, v, **kw)
+    want = ops.flash_bwd(q, k, v, want_out, want_lse, do, ds_workspace=None, **kw)
+    assert len(want) == 4
+    pos = dict(target_positions=torch.arange(t)[None].cuda(), source_positions=torch.arange(t)[None].cuda())
+    bias = ab.CompositeAttentionBias([ab.CausalAttentionBias(**pos)])
+    with jax_stand_in.installed() as (mod, state):
+        fa = mod.HipFlashAttention.default_config().set(softmax_scale=d ** -0.5).instantiate()
+        batch = dict(query=q, key=k, value=v, bias=bias, logit_sink=sink)
+        assert fa.is_supported(batch, kv_cache_type=None) and torch.equal(fa(batch), want_out)
+        out, pullback = mod.flash_attention.vjp(q, k, v, None, None, None, sink, d ** -0.5, 1, 0, 0.0)
+        grads = pullback(do)
+        assert state.calls[-1][1][7] == (hq,) and state.calls[-1][3][3] == (hq,)
+        for got, exp in zip(grads[:3] + (grads[6],), want):
+            assert torch.equal(got, exp)
+        assert grads[3:6] == (None, None, None)
+
+
+@pytest.mark.gpu
+def test_jax_side_head_dims_between_the_compiled_widths():
+    """head_dim 72 goes to the kernels as it is (16-bit, no bias: `_runs_at_native_head_dim`), with a dense
+    bias it is zero-padded to 128 and the output sliced; head_dim 40 with one head (rows closer than a
+    compiled width) is padded too.  Each case gives the torch-side class's bits."""
+    from axlearn_amd.flash_attention.hip_attention import HipFlashAttention as TorchSide
+
+    for (hq, hkv, d, with_bias) in ((4, 2, 72, False), (4, 2, 72, True), (1, 1, 40, False)):
+        b, t = 2, 256
+        q, k, v, _ = _inputs(b, t, hq, hkv, d, torch.bfloat16, seed=6)
+        pos = dict(target_positions=torch.arange(t)[None].cuda(), source_positions=torch.arange(t)[None].cuda())
+        parts = [ab.CausalAttentionBias(**pos)]
+        if with_bias:
+            parts.append(ab.TensorAttentionBias(torch.randn(1, 1, t, t, generator=torch.Generator().manual_seed(8)).cuda()))
+        batch = dict(query=q, key=k, value=v, bias=ab.CompositeAttentionBias(parts))
+        torch_side = TorchSide.default_config().set(softmax_scale=0.2).instantiate()
+        assert torch_side.is_supported(batch, kv_cache_type=None)
+        with torch.no_grad():
+            want = torch_side(batch)
+        with jax_stand_in.installed() as (mod, state):
+            fa = mod.HipFlashAttention.default_config().set(softmax_scale=0.2).instantiate()
+            assert fa.is_supported(batch, kv_cache_type=None)
+            got = fa(batch)
+            native = d == 72 and not with_bias
+            assert state.calls[-1][1][0] == (b, t, hq, d if native else (128 if d > 64 else 64))
+        assert got.shape == want.shape and torch.equal(got, want)
+
+
+@pytest.mark.gpu
+def test_jax_side_incremental_prefill():
+    """`kv_cache_type=KVCache` with a chunk of queries per sequence, each at its own offset into the cache
+    (utils_test.py:361-478): rows padded to the 128-row block, offsets passed as the q_pos_offsets
+    operand; the torch-side class's bits, for a causal mask and for a window."""
+    from axlearn_amd.flash_attention.hip_attention import HipFlashAttention as TorchSide
+    from axlearn_amd.kv_cache import KVCache
+
+    b, t, s, hq, hkv, d = 3, 40, 512, 8, 2, 128
+    g = torch.Generator().manual_seed(9)
+    q = torch.randn(b, t, hq, d, generator=g).to(torch.bfloat16).cuda()
+    k = torch.randn(b, s, hkv, d, generator=g).to(torch.bfloat16).cuda()
+    v = torch.randn(b, s, hkv, d, generator=g).to(torch.bfloat16).cuda()
+    starts = torch.tensor([0, 130, 472])
+    pos = dict(target_positions=(starts[:, None] + torch.arange(t)[None]).cuda(), source_positions=torch.arange(s)[None].cuda())
+    for window in (None, 64):
+        mask = ab.CausalAttentionBias(**pos) if window is None else ab.SlidingWindowAttentionBias(
+            ab.sliding_window_causal_mask(window), sliding_window_size=window, **pos)
+        batch = dict(query=q, key=k, value=v, bias=ab.CompositeAttentionBias([mask]))
+        torch_side = TorchSide.default_config().set(softmax_scale=d ** -0.5).instantiate()
+        assert torch_side.is_supported(batch, kv_cache_type=KVCache)
+        with torch.no_grad():
+            want = torch_side(batch)
+        with jax_stand_in.installed() as (mod, state):
+            fa = mod.HipFlashAttention.default_config().set(softmax_scale=d ** -0.5).instantiate()
+            assert fa.is_supported(batch, kv_cache_type=KVCache)
+            got = fa(batch)
+            target, operands, attrs, _ = state.calls[-1]
+            assert target == "AxlFlashFwd" and operands[0] == (b, 128, hq, d) and operands[7] == (b,)
+            assert attrs["mask_kind"] == (1 if window is None else 2) and attrs["sliding_window"] == (window or 0)
+        assert got.shape == (b, t, hq, d) and torch.equal(got, want)
 
 
 @pytest.mark.gpu
