@@ -312,8 +312,33 @@ def _decode_mask_and_bias(bias: BaseAttentionBias, lengths: Tensor, kv_len: int)
     return -1, row if dense is None else dense.astype(jnp.float32) + row
 
 
+def _decode_supported(self, input_batch) -> bool:
+    """What the decode kernels take, beyond the base classes' checks (the torch-side classes' gate)."""
+    query = input_batch["query"]
+    if input_batch.get("logit_sink", None) is not None:
+        return self._log_unsupported("logit_sink is not supported.")   # as gpu_decoding.py:299
+    ok = (jnp.bfloat16, jnp.float16, jnp.float32)
+    if query.dtype not in ok or input_batch["key"].dtype not in ok or input_batch["value"].dtype not in ok:
+        return self._log_unsupported(f"{query.dtype=} / {input_batch['key'].dtype=}")
+    if query.shape[-1] > 128 or query.shape[-1] % 8 != 0:
+        return self._log_unsupported(f"head_dim {query.shape[-1]} (supported: multiples of 8 up to 128)")
+    if not self.config.softmax_scale > 0.0:
+        return self._log_unsupported(f"{self.config.softmax_scale=} must be positive")
+    mask, _ = split(input_batch["bias"], MaskFnAttentionBias)
+    if mask is None or getattr(mask, "target_positions", None) is None:
+        return self._log_unsupported("decode needs a mask bias with target_positions.")
+    return True
+
+
 class HipDecoding(BaseSingleStepDecoding):
     """Stands where `GPUDecoding` does (gpu_decoding.py:286-352)."""
+
+    def is_supported(self, input_batch: Nested[Tensor | BaseAttentionBias], kv_cache_type=None) -> bool:
+        if not super().is_supported(input_batch=input_batch, kv_cache_type=kv_cache_type):
+            return False
+        if kv_cache_type is None or kv_cache_type.__name__ != "KVCache":
+            return self._log_unsupported(f"{kv_cache_type=}")
+        return _decode_supported(self, input_batch)
 
     @functools.partial(jax.jit, static_argnames=["self"])
     def __call__(self, input_batch: Nested[Tensor | BaseAttentionBias]) -> Tensor:
@@ -332,6 +357,19 @@ class HipDecoding(BaseSingleStepDecoding):
 
 class HipPagedAttention(BasePagedAttention):
     """Stands where `GPUPagedAttention` does (gpu_paged_attention.py:299-379)."""
+
+    def is_supported(self, input_batch: Nested[Tensor | BaseAttentionBias], kv_cache_type=None) -> bool:
+        if not super().is_supported(input_batch=input_batch, kv_cache_type=kv_cache_type):
+            return False
+        if not self._check_block_size(input_batch, block_size=self.config.gpu_block_size):
+            return False
+        page_size = input_batch["key"].shape[2]
+        # the reference's gate (gpu_paged_attention.py:313-321): fewer than 16 pages per compute block
+        if self.config.gpu_block_size / page_size >= 16:
+            return self._log_unsupported(f"pages per compute block must stay below 16, got {page_size=}")
+        if page_size < 16 or page_size & (page_size - 1):
+            return self._log_unsupported(f"page size {page_size} (supported: 16 times a power of two)")
+        return _decode_supported(self, input_batch)
 
     @functools.partial(jax.jit, static_argnames=["self"])
     def __call__(self, input_batch: Nested[Tensor | BaseAttentionBias]) -> Tensor:

@@ -278,14 +278,22 @@ def test_jax_side_decode_classes_and_page_insert():
     causal = ab.CompositeAttentionBias([ab.CausalAttentionBias(
         target_positions=(lengths.long() - 1)[:, None], source_positions=torch.arange(kv_len)[None].cuda())])
     with jax_stand_in.installed() as (mod, state):
+        from axlearn_amd.kv_cache import KVCache, PagedKVCache
+
         paged = mod.HipPagedAttention.default_config().set(softmax_scale=0.3).instantiate()
-        got = paged(dict(query=qq, key=kp, value=vp, bias=causal, page_tables=tables))
+        pbatch = dict(query=qq, key=kp, value=vp, bias=causal, page_tables=tables)
+        assert paged.is_supported(pbatch, kv_cache_type=PagedKVCache) and not paged.is_supported(pbatch, kv_cache_type=KVCache)
+        assert not paged.is_supported(dict(pbatch, key=kp[:, :, :8], value=vp[:, :, :8]), kv_cache_type=PagedKVCache)  # 8-token pages
+        got = paged(pbatch)
         want = ops.paged_decode(qq.reshape(b, hq, d), kp, vp, tables, lengths, softmax_scale=0.3)
         assert got.shape == (b, 1, hq, d) and torch.equal(got.reshape(b, hq, d), want)
         # contiguous cache: the same keys gathered
         kk, vv = (ref.reconstruct_kv(tables.cpu(), x.cpu()).contiguous().cuda() for x in (kp, vp))
         dec = mod.HipDecoding.default_config().set(softmax_scale=0.3).instantiate()
-        got_c = dec(dict(query=qq, key=kk, value=vv, bias=causal))
+        cbatch = dict(query=qq, key=kk, value=vv, bias=causal)
+        assert dec.is_supported(cbatch, kv_cache_type=KVCache) and not dec.is_supported(cbatch, kv_cache_type=None)
+        assert not dec.is_supported(dict(cbatch, logit_sink=torch.zeros(hq).cuda()), kv_cache_type=KVCache)
+        got_c = dec(cbatch)
         want_c = ops.decode(qq.reshape(b, hq, d), kk, vv, lengths, softmax_scale=0.3)
         assert torch.equal(got_c.reshape(b, hq, d), want_c)
         # a mask fn that is neither causal nor a window: evaluated on the host as a row of 0 / NEG_INF
