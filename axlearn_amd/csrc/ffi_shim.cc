@@ -269,6 +269,11 @@ ffi::Error PagedKvInsert(hipStream_t stream, ffi::AnyBuffer k_pages, ffi::AnyBuf
 
 }  // namespace
 
+// The ABI version of include/axl_attn.h this file was compiled against: the Python side compares it with
+// axl_abi_version() of the core library before it registers the handlers (the structures are filled here
+// and read there).
+extern "C" int axl_ffi_shim_abi_version() { return AXL_ATTN_ABI_VERSION; }
+
 XLA_FFI_DEFINE_HANDLER_SYMBOL(AxlFlashFwd, FlashFwd,
                               ffi::Ffi::Bind()
                                   .Ctx<ffi::PlatformStream<hipStream_t>>()

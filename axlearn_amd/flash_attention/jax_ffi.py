@@ -60,6 +60,9 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _FFI_LIB = ctypes.CDLL(os.path.join(_HERE, "..", "libaxl_attn_ffi.so"))
 _CORE_LIB = ctypes.CDLL(os.path.join(_HERE, "..", "libaxl_attn_hip.so"))
 
+if _FFI_LIB.axl_ffi_shim_abi_version() != _CORE_LIB.axl_abi_version():
+    raise ImportError(f"libaxl_attn_ffi.so was built against ABI {_FFI_LIB.axl_ffi_shim_abi_version()} of "
+                      f"include/axl_attn.h, libaxl_attn_hip.so implements {_CORE_LIB.axl_abi_version()}: rebuild the shim")
 for _name in ("AxlFlashFwd", "AxlFlashBwd", "AxlDecode", "AxlPagedDecode", "AxlPagedKvInsert"):
     jax.ffi.register_ffi_target(_name, jax.ffi.pycapsule(getattr(_FFI_LIB, _name)), platform="ROCM")
 

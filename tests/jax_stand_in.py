@@ -128,7 +128,11 @@ def load_shim() -> ctypes.CDLL:
         if not os.path.exists(SHIM_PATH):
             raise RuntimeError(f"{SHIM_PATH} is missing: make -C {SHIM_DIR}")
         _lib.load()
-        _shim = ctypes.CDLL(SHIM_PATH)
+        shim = ctypes.CDLL(SHIM_PATH)
+        if shim.axl_ffi_shim_abi_version() != _lib.ABI_VERSION:
+            raise RuntimeError(f"{SHIM_PATH} was built against ABI {shim.axl_ffi_shim_abi_version()}, "
+                               f"the library has {_lib.ABI_VERSION}: make -C {SHIM_DIR}")
+        _shim = shim
     return _shim
 
 
@@ -264,8 +268,9 @@ def installed():
     real_cdll = ctypes.CDLL
 
     def cdll(path, *args, **kwargs):
-        if str(path).endswith("libaxl_attn_ffi.so"):   # the compiled shim: its symbols are only registered
-            return types.SimpleNamespace(**{target: target for target in TARGETS})
+        if str(path).endswith("libaxl_attn_ffi.so"):   # the compiled shim: its handler symbols are only registered
+            return types.SimpleNamespace(axl_ffi_shim_abi_version=load_shim().axl_ffi_shim_abi_version,
+                                         **{target: target for target in TARGETS})
         return real_cdll(path, *args, **kwargs)
 
     sys.modules.update(fakes)
