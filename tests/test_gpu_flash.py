@@ -423,6 +423,38 @@ def test_closed_forms_and_determinism():
         assert torch.equal(a, c)
 
 
+@pytest.mark.parametrize("dtype,d", [(torch.bfloat16, 128), (torch.float16, 64), (torch.bfloat16, 72)])
+@pytest.mark.parametrize("mask,seg", [("causal", False), ("causal", True), ("window", False), ("window", True), ("none", False)])
+def test_results_do_not_depend_on_what_ran_before(dtype, d, mask, seg):
+    """The same call three times, with other kernels and freshly dirtied workspaces in between: identical
+    bits, for the recomputing backward, the dS-workspace backward whole and in slices of kv heads, and the
+    forward.  A register read too early behind an assembly MFMA chain shows up exactly here: as values
+    that change from run to run."""
+    b, t, hq, hkv = 2, 1024, 8, 2
+    q, k, v, do = (x.cuda() for x in _inputs(b, t, hq, hkv, d, dtype))
+    segs = ref.packed_segment_ids(11, b, t, max_docs=4).cuda() if seg else None
+    kw = dict(softmax_scale=d ** -0.5, segment_ids=segs,
+              mask_kind={"causal": ops.MASK_CAUSAL, "window": ops.MASK_SLIDING_WINDOW, "none": ops.MASK_NONE}[mask],
+              sliding_window=300 if mask == "window" else 0)
+    runs = []
+    for i in range(3):
+        dirt = torch.full((48 << 20,), float(i) - 1.5, device="cuda")   # what the next allocations will find
+        del dirt
+        out, lse = ops.flash_fwd(q, k, v, **kw)
+        grads = [out, lse]
+        for ds, heads in ((False, 0), (True, 0), (True, 1)):
+            grads += list(ops.flash_bwd(q, k, v, out, lse, do, ds_workspace=ds, ds_slice_kv_heads=heads, **kw)[:3])
+        torch.cuda.synchronize()
+        runs.append([x.clone() for x in grads])
+        _ = torch.randn(1 << 20, device="cuda").sort()   # something else on the GPU in between
+    for other in runs[1:]:
+        for i, (a, c) in enumerate(zip(runs[0], other)):
+            assert torch.equal(a, c), f"result {i} differs between runs"
+    # and the three backward forms agree with each other on dk / dv bit for bit where they share the kernel
+    dq_r, dk_r, dv_r, dq_w, dk_w, dv_w, dq_s, dk_s, dv_s = runs[0][2:]
+    assert torch.equal(dk_w, dk_s) and torch.equal(dv_w, dv_s) and torch.equal(dq_w, dq_s)
+
+
 def test_strided_inputs():
     """q/k/v sliced out of one fused [B,T,H+2Hkv,D] projection (non-contiguous heads stride)."""
     b, t, hq, hkv, d = 1, 256, 4, 2, 128
