@@ -21,6 +21,8 @@
 //     head are placed on the same XCD so its L2 serves the re-reads.
 #include <type_traits>
 
+#include <cstdlib>
+
 #include "common.h"
 
 namespace axl {
@@ -800,6 +802,304 @@ __global__ __launch_bounds__(256) void flash_fwd_f32_kernel(const FwdArgs a) {
   if (a.lse && g == 0) a.lse[((int64_t)b * a.Hq + h) * a.T + q0 + l32] = m_run + logf(l_tot);
 }
 
+// ---------------------------------------------------------------------------------------------
+// fp32 forward on the 16-bit matrix instruction.  This GPU multiplies bf16 sixteen times as fast as
+// fp32 (v_mfma_f32_32x32x16_bf16 against v_mfma_f32_32x32x2_f32), so an fp32 operand travels as three
+// bf16 values, x = hi + mid + lo (8 + 8 + 8 bits of significand, each the rounded remainder of the one
+// before: the split is exact), and a product of two operands as the six partial products that matter,
+//   a b ~ a_lo b_hi + a_hi b_lo + a_mid b_mid + a_mid b_hi + a_hi b_mid + a_hi b_hi,
+// accumulated in fp32 by the instruction; the three products left out are below 2^-24 of the result.
+// Measured against float64 the error is that of an fp32 dot product (or smaller: fewer roundings).
+// Six 32-cycle instructions per 16 elements of the inner dimension instead of eight 64-cycle ones.
+//
+// Mapping as in the kernel above (a wavefront owns 32 query rows, a 32-key tile per step, S^T and O^T
+// accumulators with the query as the lane's column), operand layouts as in the 16-bit kernel: K rows
+// are read in the order swap_bits_2_3, so that registers 0..7 / 8..15 of a lane's S^T column are the
+// keys 8g .. 8g+7 of the tile's first / second half and, split and packed, are the B operand of
+// O^T += V^T P^T as they stand; V^T comes out of transposing LDS reads.  K and V tiles go from global
+// memory through registers, where they are split, into three 16-bit planes each in LDS.
+// ---------------------------------------------------------------------------------------------
+template <int D>
+struct FwdTileF32x {
+  static constexpr int BQ = 128;
+  static constexpr int BK = 32;
+  static constexpr int KSTRIDE = D * 2 + 16;  // bytes per key row of a plane: 16 rows read by 16 lanes hit all banks
+  static constexpr int VSTRIDE = D * 2 + 64;  // the same for the 4 rows x 2 halves of a transposing read
+  static constexpr int KPLANE = BK * KSTRIDE, VPLANE = BK * VSTRIDE;
+  static constexpr int BUF_BYTES = 3 * (KPLANE + VPLANE);   // one K / V tile; tile t lives in buffer t % 2
+  static constexpr int QSTRIDE = D * 4 + 4;
+  static constexpr int QBYTES = BQ * QSTRIDE;               // the query block passes through the same memory once
+  static constexpr int LDS_BYTES = 2 * BUF_BYTES > QBYTES ? 2 * BUF_BYTES : QBYTES;
+  static constexpr int LD4 = BK * (D / 4) / 256;            // float4 loads per thread and tensor tile
+  static_assert(BK * (D / 4) % 256 == 0, "a tile divides evenly over the threads");
+};
+
+// Two fp32 values as three pairs of bf16: hi = rn(x), mid = rn(x - hi), lo = rn(x - hi - mid).
+struct Split3x2 {
+  bf16x2 part[3];
+};
+__device__ __forceinline__ Split3x2 split3(float x0, float x1) {
+  Split3x2 r;
+  r.part[0] = pack_bf16(x0, x1);
+  const unsigned hb = __builtin_bit_cast(unsigned, r.part[0]);
+  const float r0 = x0 - __uint_as_float(hb << 16), r1 = x1 - __uint_as_float(hb & 0xffff0000u);
+  r.part[1] = pack_bf16(r0, r1);
+  const unsigned mb = __builtin_bit_cast(unsigned, r.part[1]);
+  r.part[2] = pack_bf16(r0 - __uint_as_float(mb << 16), r1 - __uint_as_float(mb & 0xffff0000u));
+  return r;
+}
+// Eight fp32 values as the three MFMA operands hi, mid, lo.
+struct Split3x8 {
+  union {
+    bf16x8 v;
+    bf16x2 p[4];
+  } part[3];
+};
+__device__ __forceinline__ void split3x8(const float (&x)[8], Split3x8& out) {
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const Split3x2 s = split3(x[2 * i], x[2 * i + 1]);
+#pragma unroll
+    for (int p = 0; p < 3; p++) out.part[p].p[i] = s.part[p];
+  }
+}
+// c += a b from the split operands: the six partial products, the small ones first.
+__device__ __forceinline__ floatx16 mfma_split(const bf16x8 (&a)[3], const bf16x8 (&b)[3], floatx16 c) {
+  c = ElemBf16::mfma_32x32x16(a[2], b[0], c);
+  c = ElemBf16::mfma_32x32x16(a[0], b[2], c);
+  c = ElemBf16::mfma_32x32x16(a[1], b[1], c);
+  c = ElemBf16::mfma_32x32x16(a[1], b[0], c);
+  c = ElemBf16::mfma_32x32x16(a[0], b[1], c);
+  c = ElemBf16::mfma_32x32x16(a[0], b[0], c);
+  return c;
+}
+
+template <int D>
+__global__ __launch_bounds__(256) void flash_fwd_f32x_kernel(const FwdArgs a) {
+  using Tile = FwdTileF32x<D>;
+  constexpr int DT = D / 32, KSTEPS = D / 16;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  float* const q_lds = (float*)smem;
+  constexpr int QS = Tile::QSTRIDE / 4;
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+  int qb, b, h;
+  decode_block(blockIdx.x, a.T / Tile::BQ, a.B, a.Hq, a.Hkv, 1 << 20, qb, b, h);
+  const int hk = h / (a.Hq / a.Hkv);
+  const int q_off = a.q_off + (a.q_offs ? a.q_offs[b] : 0);  // position of this sequence's query row 0
+  const int q0_wg = qb * Tile::BQ;
+  const int q0 = q0_wg + wave * 32;
+
+  const float* qg = (const float*)a.q + b * a.qs.b + (int64_t)q0_wg * a.qs.s + h * a.qs.h;
+  const float* kp = (const float*)a.k + b * a.ks.b + hk * a.ks.h;
+  const float* vp = (const float*)a.v + b * a.vs.b + hk * a.vs.h;
+
+  // The 128 x D query block passes through LDS once; a lane keeps, split, the half of its own row that its
+  // MFMAs read (elements 16 s + 8 g .. + 7 of every 16).
+  for (int i = tid; i < Tile::BQ * (D / 4); i += 256) {
+    const int row = i / (D / 4), c4 = i % (D / 4);
+    const float4 x = *(const float4*)(qg + (int64_t)row * a.qs.s + c4 * 4);
+    float* dst = q_lds + row * QS + c4 * 4;
+    dst[0] = x.x; dst[1] = x.y; dst[2] = x.z; dst[3] = x.w;
+  }
+  __syncthreads();
+  bf16x8 q_mine[KSTEPS][3];
+  {
+    const float* q_row = q_lds + (wave * 32 + l32) * QS;
+#pragma unroll
+    for (int s = 0; s < KSTEPS; s++) {
+      float x[8];
+#pragma unroll
+      for (int j = 0; j < 8; j++) x[j] = q_row[16 * s + 8 * g + j];
+      Split3x8 sp;
+      split3x8(x, sp);
+#pragma unroll
+      for (int p = 0; p < 3; p++) q_mine[s][p] = sp.part[p].v;
+    }
+  }
+  __syncthreads();  // the ring of K / V tiles takes the memory over
+
+  int k_begin = 0, k_end = a.S;
+  if (a.mask_kind != AXL_MASK_NONE) {
+    k_end = min(a.S, q0_wg + Tile::BQ + q_off);
+    if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) k_begin = max(0, q0_wg + q_off - a.window);
+  }
+  const int t_begin = k_begin / Tile::BK;
+  const int t_end = (k_end + Tile::BK - 1) / Tile::BK;
+  const int qpos = q0 + l32 + q_off;
+  const int qpos_min = q0 + q_off, qpos_max = q0 + 31 + q_off;
+  const int seg_q = a.seg ? a.seg[(int64_t)b * a.T + q0 + l32] : 0;
+  const int32_t* seg_k = a.seg ? a.seg + (int64_t)b * a.T : nullptr;
+  const char* bias_row = nullptr;
+  const uint8_t* drop_row = nullptr;
+  if (a.aux.bias) bias_row = a.aux.bias + b * a.aux.bias_sb + h * a.aux.bias_sh + (int64_t)(q0 + l32) * a.aux.bias_sr;
+  if (a.aux.drop) drop_row = a.aux.drop + b * a.aux.drop_sb + h * a.aux.drop_sh + (int64_t)(q0 + l32) * a.aux.drop_sr;
+
+  floatx16 o[DT];
+#pragma unroll
+  for (int i = 0; i < DT; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) o[i][r] = 0.f;
+  float m_run = kNegInf, l_run = 0.f;
+  if (a.sink) {  // the sink logit counts as an already-processed key without a value row
+    m_run = a.sink[h];
+    l_run = g == 0 ? 1.f : 0.f;
+  }
+  // The K / V tile of 32 keys from global memory into this thread's registers, and from there, split, into
+  // a ring buffer: the next tile's round trip runs under the current tile's MFMAs, one barrier per tile.
+  float4 kx[Tile::LD4], vx[Tile::LD4];
+  auto request = [&](int k0) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < Tile::LD4; i++) {
+      const int e = tid + i * 256, row = e / (D / 4), c4 = e % (D / 4);
+      kx[i] = *(const float4*)(kp + (int64_t)(k0 + row) * a.ks.s + c4 * 4);
+      vx[i] = *(const float4*)(vp + (int64_t)(k0 + row) * a.vs.s + c4 * 4);
+    }
+  };
+  auto deposit = [&](int t) __attribute__((always_inline)) {
+    char* k_dst = smem + (t & 1) * Tile::BUF_BYTES;
+    char* v_dst = k_dst + 3 * Tile::KPLANE;
+#pragma unroll
+    for (int i = 0; i < Tile::LD4; i++) {
+      const int e = tid + i * 256, row = e / (D / 4), c4 = e % (D / 4);
+      const Split3x2 k01 = split3(kx[i].x, kx[i].y), k23 = split3(kx[i].z, kx[i].w);
+      const Split3x2 v01 = split3(vx[i].x, vx[i].y), v23 = split3(vx[i].z, vx[i].w);
+#pragma unroll
+      for (int p = 0; p < 3; p++) {
+        union { bf16x2 h[2]; uint2 u; } kw, vw;
+        kw.h[0] = k01.part[p]; kw.h[1] = k23.part[p];
+        vw.h[0] = v01.part[p]; vw.h[1] = v23.part[p];
+        *(uint2*)(k_dst + p * Tile::KPLANE + row * Tile::KSTRIDE + c4 * 8) = kw.u;
+        *(uint2*)(v_dst + p * Tile::VPLANE + row * Tile::VSTRIDE + c4 * 8) = vw.u;
+      }
+    }
+  };
+  if (t_begin < t_end) {
+    request(t_begin * Tile::BK);
+    deposit(t_begin);
+  }
+  __syncthreads();
+
+  // Per-lane read offsets.  K: the row of key swap_bits_2_3(l32), 16 bytes at d = 16 s + 8 g.  V: transposing
+  // reads at row 8 g + j16 / 4 (+4 for the second half, +16 for the tile's second 16 keys), columns
+  // 32 dt + 16 half + 4 (j16 % 4) .. + 3.
+  const int k_off = swap_bits_2_3(l32) * Tile::KSTRIDE + 16 * g;
+  const int j16 = lane & 15, half = (lane >> 4) & 1;
+  const int v_off = (8 * g + (j16 >> 2)) * Tile::VSTRIDE + (16 * half + 4 * (j16 & 3)) * 2;
+
+  for (int t = t_begin; t < t_end; t++) {
+    const int k0 = t * Tile::BK;
+    const bool more = t + 1 < t_end;
+    if (more) request(k0 + Tile::BK);
+    const char* k_lds = smem + (t & 1) * Tile::BUF_BYTES;
+    const char* v_lds = k_lds + 3 * Tile::KPLANE;
+    bool skip = false;
+    if (a.mask_kind != AXL_MASK_NONE) {
+      skip = k0 > qpos_max;
+      if (a.mask_kind == AXL_MASK_SLIDING_WINDOW)
+        skip = skip || (qpos_min - (k0 + Tile::BK - 1) > a.window);
+    }
+    if (!skip) {
+    // S^T[key][q]: A = K rows, B = Q^T.
+    floatx16 s;
+#pragma unroll
+    for (int r = 0; r < 16; r++) s[r] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks++) {
+      bf16x8 kf[3];
+#pragma unroll
+      for (int p = 0; p < 3; p++) kf[p] = *(const bf16x8*)(k_lds + p * Tile::KPLANE + k_off + 32 * ks);
+      s = mfma_split(kf, q_mine[ks], s);
+    }
+    // Register r of lane group g is key k0 + 16 (r / 8) + 8 g + r % 8.
+    if (bias_row) {  // logits = scale * qk + bias: pre-divide so the common scale below applies
+#pragma unroll
+      for (int r4 = 0; r4 < 4; r4++) {
+        float bv[4];
+        load_bias<4>(bias_row, k0 + 16 * (r4 / 2) + 8 * g + 4 * (r4 % 2), a.aux.bias_f32, bv);
+#pragma unroll
+        for (int j = 0; j < 4; j++) s[4 * r4 + j] += bv[j] * a.aux.inv_scale;
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      const int kpos = k0 + 16 * (r / 8) + 8 * g + (r % 8);
+      bool keep = true;
+      if (a.mask_kind != AXL_MASK_NONE) {
+        const int diff = qpos - kpos;
+        keep = diff >= 0;
+        if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) keep = keep && diff <= a.window;
+      }
+      if (seg_k) keep = keep && (seg_k[kpos] == seg_q);
+      s[r] = keep ? s[r] * a.scale : kMasked;
+    }
+    float mx = m_run;
+#pragma unroll
+    for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[r]);
+    mx = xor32_max(mx);
+    const float corr = expf(m_run - mx);
+    m_run = mx;
+    float lsum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+      s[r] = expf(s[r] - mx);
+      lsum += s[r];
+    }
+    l_run = l_run * corr + lsum;
+    if (drop_row) {  // dropped probabilities leave P V but stay in the row sum
+#pragma unroll
+      for (int r4 = 0; r4 < 4; r4++) {
+        const unsigned w = *(const unsigned*)(drop_row + k0 + 16 * (r4 / 2) + 8 * g + 4 * (r4 % 2));
+#pragma unroll
+        for (int j = 0; j < 4; j++) s[4 * r4 + j] = ((w >> (8 * j)) & 0xffu) ? 0.f : s[4 * r4 + j];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < DT; i++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) o[i][r] *= corr;
+    // O^T[d][q] += V^T[d][key] P^T[key][q], 16 keys per step.
+#pragma unroll
+    for (int kk = 0; kk < 2; kk++) {
+      float pr[8];
+#pragma unroll
+      for (int j = 0; j < 8; j++) pr[j] = s[8 * kk + j];
+      Split3x8 ps;
+      split3x8(pr, ps);
+      const bf16x8 pf[3] = {ps.part[0].v, ps.part[1].v, ps.part[2].v};
+#pragma unroll
+      for (int dt = 0; dt < DT; dt++) {
+        union { bf16x8 v; shortx4 hlf[2]; } vf[3];
+#pragma unroll
+        for (int p = 0; p < 3; p++) {
+          const char* va = v_lds + p * Tile::VPLANE + v_off + 16 * kk * Tile::VSTRIDE + 64 * dt;
+          vf[p].hlf[0] = lds_read_tr16(va);
+          vf[p].hlf[1] = lds_read_tr16(va + 4 * Tile::VSTRIDE);
+        }
+        const bf16x8 vfa[3] = {vf[0].v, vf[1].v, vf[2].v};
+        o[dt] = mfma_split(vfa, pf, o[dt]);
+      }
+    }
+    }  // tile not skipped
+    if (more) deposit(t + 1);  // that buffer was last read a tile ago, before the barrier that ended it
+    __syncthreads();
+  }
+
+  const float l_tot = xor32_sum(l_run);
+  const float inv_l = (l_tot > 0.f ? 1.0f / l_tot : 0.f) * a.aux.keep_scale;  // no visible key: zeros
+  float* op = (float*)a.out + b * a.os.b + (int64_t)(q0 + l32) * a.os.s + h * a.os.h;
+#pragma unroll
+  for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+    for (int rq = 0; rq < 4; rq++) {
+      float4 w = {o[dt][4 * rq + 0] * inv_l, o[dt][4 * rq + 1] * inv_l, o[dt][4 * rq + 2] * inv_l,
+                  o[dt][4 * rq + 3] * inv_l};
+      *(float4*)(op + 32 * dt + 8 * rq + 4 * g) = w;
+    }
+  if (a.lse && g == 0) a.lse[((int64_t)b * a.Hq + h) * a.T + q0 + l32] = m_run + logf(l_tot);
+}
+
 static Strides3 to_s3(const AxlStrides& s) { return Strides3{s.batch, s.seq, s.head}; }
 
 int launch_flash_fwd(const AxlFlashFwdParams& p, hipStream_t stream) {
@@ -841,8 +1141,15 @@ int launch_flash_fwd(const AxlFlashFwdParams& p, hipStream_t stream) {
   } else if (p.dtype == AXL_F16) {
     AXL_LAUNCH_FWD16(ElemF16);
   } else {
-    if (p.head_dim == 128) AXL_LAUNCH_FWD(flash_fwd_f32_kernel<128>, FwdTileF32<128>);
-    else AXL_LAUNCH_FWD(flash_fwd_f32_kernel<64>, FwdTileF32<64>);
+    // AXL_F32_MFMA=1 in the environment: the kernel on the fp32 matrix instruction (for comparison).
+    static const bool true_f32 = [] { const char* e = getenv("AXL_F32_MFMA"); return e && e[0] == '1'; }();
+    if (true_f32) {
+      if (p.head_dim == 128) AXL_LAUNCH_FWD(flash_fwd_f32_kernel<128>, FwdTileF32<128>);
+      else AXL_LAUNCH_FWD(flash_fwd_f32_kernel<64>, FwdTileF32<64>);
+    } else {
+      if (p.head_dim == 128) AXL_LAUNCH_FWD(flash_fwd_f32x_kernel<128>, FwdTileF32x<128>);
+      else AXL_LAUNCH_FWD(flash_fwd_f32x_kernel<64>, FwdTileF32x<64>);
+    }
   }
 #undef AXL_LAUNCH_FWD16
 #undef AXL_LAUNCH_FWD

@@ -341,7 +341,8 @@ def bench_c1(steps, warmup, cpu_baseline):
     res = dict(
         workload="C1: causal MHA forward, fp32, B2 H4 T512 D64", value=tfl, unit="TFLOP/s", ms_per_step=ms,
         algorithmic_gflop=flops / 1e9,
-        roofline=dict(kernel="flash_fwd_f32_kernel", bound="mfma", achieved=tfl, peak=MFMA_F32_PEAK_TFLOPS,
+        arithmetic="fp32 operands as three bf16 parts each, six bf16 MFMA partial products per product, fp32 accumulation",
+        roofline=dict(kernel="flash_fwd_f32x_kernel", bound="mfma", achieved=tfl, peak=MFMA_F32_PEAK_TFLOPS,
                       unit="TFLOP/s", frac=tfl / MFMA_F32_PEAK_TFLOPS, traffic=None,
                       traffic_source="not measured: 32 workgroups, 0.27 GFLOP, bound by launch latency"),
     )
