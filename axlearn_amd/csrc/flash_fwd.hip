@@ -819,9 +819,10 @@ __global__ __launch_bounds__(256) void flash_fwd_f32_kernel(const FwdArgs a) {
 // O^T += V^T P^T as they stand; V^T comes out of transposing LDS reads.  K and V tiles go from global
 // memory through registers, where they are split, into three 16-bit planes each in LDS.
 // ---------------------------------------------------------------------------------------------
-template <int D>
+template <int D, int NW>
 struct FwdTileF32x {
-  static constexpr int BQ = 128;
+  static constexpr int NT = 64 * NW;          // threads: NW wavefronts of 32 query rows
+  static constexpr int BQ = 32 * NW;
   static constexpr int BK = 32;
   static constexpr int KSTRIDE = D * 2 + 16;  // bytes per key row of a plane: 16 rows read by 16 lanes hit all banks
   static constexpr int VSTRIDE = D * 2 + 64;  // the same for the 4 rows x 2 halves of a transposing read
@@ -830,8 +831,8 @@ struct FwdTileF32x {
   static constexpr int QSTRIDE = D * 4 + 4;
   static constexpr int QBYTES = BQ * QSTRIDE;               // the query block passes through the same memory once
   static constexpr int LDS_BYTES = 2 * BUF_BYTES > QBYTES ? 2 * BUF_BYTES : QBYTES;
-  static constexpr int LD4 = BK * (D / 4) / 256;            // float4 loads per thread and tensor tile
-  static_assert(BK * (D / 4) % 256 == 0, "a tile divides evenly over the threads");
+  static constexpr int LD4 = BK * (D / 4) / NT;             // float4 loads per thread and tensor tile
+  static_assert(BK * (D / 4) % NT == 0, "a tile divides evenly over the threads");
 };
 
 // Two fp32 values as three pairs of bf16: hi = rn(x), mid = rn(x - hi), lo = rn(x - hi - mid).
@@ -874,9 +875,9 @@ __device__ __forceinline__ floatx16 mfma_split(const bf16x8 (&a)[3], const bf16x
   return c;
 }
 
-template <int D>
-__global__ __launch_bounds__(256) void flash_fwd_f32x_kernel(const FwdArgs a) {
-  using Tile = FwdTileF32x<D>;
+template <int D, int NW>
+__global__ __launch_bounds__(64 * NW) void flash_fwd_f32x_kernel(const FwdArgs a) {
+  using Tile = FwdTileF32x<D, NW>;
   constexpr int DT = D / 32, KSTEPS = D / 16;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   float* const q_lds = (float*)smem;
@@ -897,13 +898,16 @@ __global__ __launch_bounds__(256) void flash_fwd_f32x_kernel(const FwdArgs a) {
 
   // The 128 x D query block passes through LDS once; a lane keeps, split, the half of its own row that its
   // MFMAs read (elements 16 s + 8 g .. + 7 of every 16).
-  for (int i = tid; i < Tile::BQ * (D / 4); i += 256) {
+  for (int i = tid; i < Tile::BQ * (D / 4); i += Tile::NT) {
     const int row = i / (D / 4), c4 = i % (D / 4);
     const float4 x = *(const float4*)(qg + (int64_t)row * a.qs.s + c4 * 4);
     float* dst = q_lds + row * QS + c4 * 4;
     dst[0] = x.x; dst[1] = x.y; dst[2] = x.z; dst[3] = x.w;
   }
   __syncthreads();
+  // Logits are kept in units of log2: Q is multiplied by scale * log2(e) ahead of its split, the
+  // exponentials are exp2 (v_exp_f32, 1 ulp), and lse is converted back at the end.
+  const float c = a.scale * kLog2e;
   bf16x8 q_mine[KSTEPS][3];
   {
     const float* q_row = q_lds + (wave * 32 + l32) * QS;
@@ -911,7 +915,7 @@ __global__ __launch_bounds__(256) void flash_fwd_f32x_kernel(const FwdArgs a) {
     for (int s = 0; s < KSTEPS; s++) {
       float x[8];
 #pragma unroll
-      for (int j = 0; j < 8; j++) x[j] = q_row[16 * s + 8 * g + j];
+      for (int j = 0; j < 8; j++) x[j] = q_row[16 * s + 8 * g + j] * c;
       Split3x8 sp;
       split3x8(x, sp);
 #pragma unroll
@@ -943,7 +947,7 @@ __global__ __launch_bounds__(256) void flash_fwd_f32x_kernel(const FwdArgs a) {
     for (int r = 0; r < 16; r++) o[i][r] = 0.f;
   float m_run = kNegInf, l_run = 0.f;
   if (a.sink) {  // the sink logit counts as an already-processed key without a value row
-    m_run = a.sink[h];
+    m_run = a.sink[h] * kLog2e;
     l_run = g == 0 ? 1.f : 0.f;
   }
   // The K / V tile of 32 keys from global memory into this thread's registers, and from there, split, into
@@ -952,7 +956,7 @@ __global__ __launch_bounds__(256) void flash_fwd_f32x_kernel(const FwdArgs a) {
   auto request = [&](int k0) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < Tile::LD4; i++) {
-      const int e = tid + i * 256, row = e / (D / 4), c4 = e % (D / 4);
+      const int e = tid + i * Tile::NT, row = e / (D / 4), c4 = e % (D / 4);
       kx[i] = *(const float4*)(kp + (int64_t)(k0 + row) * a.ks.s + c4 * 4);
       vx[i] = *(const float4*)(vp + (int64_t)(k0 + row) * a.vs.s + c4 * 4);
     }
@@ -962,7 +966,7 @@ __global__ __launch_bounds__(256) void flash_fwd_f32x_kernel(const FwdArgs a) {
     char* v_dst = k_dst + 3 * Tile::KPLANE;
 #pragma unroll
     for (int i = 0; i < Tile::LD4; i++) {
-      const int e = tid + i * 256, row = e / (D / 4), c4 = e % (D / 4);
+      const int e = tid + i * Tile::NT, row = e / (D / 4), c4 = e % (D / 4);
       const Split3x2 k01 = split3(kx[i].x, kx[i].y), k23 = split3(kx[i].z, kx[i].w);
       const Split3x2 v01 = split3(vx[i].x, vx[i].y), v23 = split3(vx[i].z, vx[i].w);
 #pragma unroll
@@ -1013,40 +1017,59 @@ __global__ __launch_bounds__(256) void flash_fwd_f32x_kernel(const FwdArgs a) {
       s = mfma_split(kf, q_mine[ks], s);
     }
     // Register r of lane group g is key k0 + 16 (r / 8) + 8 g + r % 8.
-    if (bias_row) {  // logits = scale * qk + bias: pre-divide so the common scale below applies
+    if (bias_row) {  // logits = scale * qk + bias, in units of log2
 #pragma unroll
       for (int r4 = 0; r4 < 4; r4++) {
         float bv[4];
         load_bias<4>(bias_row, k0 + 16 * (r4 / 2) + 8 * g + 4 * (r4 % 2), a.aux.bias_f32, bv);
 #pragma unroll
-        for (int j = 0; j < 4; j++) s[4 * r4 + j] += bv[j] * a.aux.inv_scale;
+        for (int j = 0; j < 4; j++) s[4 * r4 + j] += bv[j] * kLog2e;
       }
     }
+    // A tile in the interior of the wavefront's range (every key at or before its first query and inside
+    // the window of its last one, no segment ids) has nothing to mask.
+    bool interior = seg_k == nullptr;
+    if (a.mask_kind != AXL_MASK_NONE) {
+      interior = interior && k0 + Tile::BK - 1 <= qpos_min;
+      if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) interior = interior && qpos_max - k0 <= a.window;
+    }
+    if (!interior) {
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-      const int kpos = k0 + 16 * (r / 8) + 8 * g + (r % 8);
-      bool keep = true;
-      if (a.mask_kind != AXL_MASK_NONE) {
-        const int diff = qpos - kpos;
-        keep = diff >= 0;
-        if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) keep = keep && diff <= a.window;
+      for (int r = 0; r < 16; r++) {
+        const int kpos = k0 + 16 * (r / 8) + 8 * g + (r % 8);
+        bool keep = true;
+        if (a.mask_kind != AXL_MASK_NONE) {
+          const int diff = qpos - kpos;
+          keep = diff >= 0;
+          if (a.mask_kind == AXL_MASK_SLIDING_WINDOW) keep = keep && diff <= a.window;
+        }
+        if (seg_k) keep = keep && (seg_k[kpos] == seg_q);
+        s[r] = keep ? s[r] : kMasked;
       }
-      if (seg_k) keep = keep && (seg_k[kpos] == seg_q);
-      s[r] = keep ? s[r] * a.scale : kMasked;
     }
     float mx = m_run;
 #pragma unroll
     for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[r]);
     mx = xor32_max(mx);
-    const float corr = expf(m_run - mx);
+    // The running maximum moves in the first few tiles of a row and rarely after: the rescaling is left
+    // out (its factor would be exactly 1) unless it moved for some row of the wavefront.
+    const bool moved = __builtin_amdgcn_ballot_w64(mx != m_run) != 0;
+    if (moved) {
+      const float corr = fast_exp2(m_run - mx);
+      l_run *= corr;
+#pragma unroll
+      for (int i = 0; i < DT; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[i][r] *= corr;
+    }
     m_run = mx;
     float lsum = 0.f;
 #pragma unroll
     for (int r = 0; r < 16; r++) {
-      s[r] = expf(s[r] - mx);
+      s[r] = fast_exp2(s[r] - mx);
       lsum += s[r];
     }
-    l_run = l_run * corr + lsum;
+    l_run += lsum;
     if (drop_row) {  // dropped probabilities leave P V but stay in the row sum
 #pragma unroll
       for (int r4 = 0; r4 < 4; r4++) {
@@ -1055,10 +1078,6 @@ __global__ __launch_bounds__(256) void flash_fwd_f32x_kernel(const FwdArgs a) {
         for (int j = 0; j < 4; j++) s[4 * r4 + j] = ((w >> (8 * j)) & 0xffu) ? 0.f : s[4 * r4 + j];
       }
     }
-#pragma unroll
-    for (int i = 0; i < DT; i++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) o[i][r] *= corr;
     // O^T[d][q] += V^T[d][key] P^T[key][q], 16 keys per step.
 #pragma unroll
     for (int kk = 0; kk < 2; kk++) {
@@ -1097,7 +1116,7 @@ __global__ __launch_bounds__(256) void flash_fwd_f32x_kernel(const FwdArgs a) {
                   o[dt][4 * rq + 3] * inv_l};
       *(float4*)(op + 32 * dt + 8 * rq + 4 * g) = w;
     }
-  if (a.lse && g == 0) a.lse[((int64_t)b * a.Hq + h) * a.T + q0 + l32] = m_run + logf(l_tot);
+  if (a.lse && g == 0) a.lse[((int64_t)b * a.Hq + h) * a.T + q0 + l32] = m_run * kLn2 + logf(l_tot);
 }
 
 static Strides3 to_s3(const AxlStrides& s) { return Strides3{s.batch, s.seq, s.head}; }
@@ -1147,8 +1166,19 @@ int launch_flash_fwd(const AxlFlashFwdParams& p, hipStream_t stream) {
       if (p.head_dim == 128) AXL_LAUNCH_FWD(flash_fwd_f32_kernel<128>, FwdTileF32<128>);
       else AXL_LAUNCH_FWD(flash_fwd_f32_kernel<64>, FwdTileF32<64>);
     } else {
-      if (p.head_dim == 128) AXL_LAUNCH_FWD(flash_fwd_f32x_kernel<128>, FwdTileF32x<128>);
-      else AXL_LAUNCH_FWD(flash_fwd_f32x_kernel<64>, FwdTileF32x<64>);
+      // eight wavefronts (two per SIMD, 256 query rows share a tile's split) where the length allows
+      static const bool four = [] { const char* e = getenv("AXL_F32X_WAVES"); return e && e[0] == '4'; }();
+      using T128x8 = FwdTileF32x<128, 8>;
+      using T64x8 = FwdTileF32x<64, 8>;
+      using T128x4 = FwdTileF32x<128, 4>;
+      using T64x4 = FwdTileF32x<64, 4>;
+      if (p.q_len % 256 == 0 && !four) {
+        if (p.head_dim == 128) AXL_LAUNCH_FWD((flash_fwd_f32x_kernel<128, 8>), T128x8);
+        else AXL_LAUNCH_FWD((flash_fwd_f32x_kernel<64, 8>), T64x8);
+      } else {
+        if (p.head_dim == 128) AXL_LAUNCH_FWD((flash_fwd_f32x_kernel<128, 4>), T128x4);
+        else AXL_LAUNCH_FWD((flash_fwd_f32x_kernel<64, 4>), T64x4);
+      }
     }
   }
 #undef AXL_LAUNCH_FWD16

@@ -342,9 +342,10 @@ def bench_c1(steps, warmup, cpu_baseline):
         workload="C1: causal MHA forward, fp32, B2 H4 T512 D64", value=tfl, unit="TFLOP/s", ms_per_step=ms,
         algorithmic_gflop=flops / 1e9,
         arithmetic="fp32 operands as three bf16 parts each, six bf16 MFMA partial products per product, fp32 accumulation",
-        roofline=dict(kernel="flash_fwd_f32x_kernel", bound="mfma", achieved=tfl, peak=MFMA_F32_PEAK_TFLOPS,
-                      unit="TFLOP/s", frac=tfl / MFMA_F32_PEAK_TFLOPS, traffic=None,
-                      traffic_source="not measured: 32 workgroups, 0.27 GFLOP, bound by launch latency"),
+        executed_tflops=6.0 * tfl, fp32_mfma_peak_tflops=MFMA_F32_PEAK_TFLOPS,
+        roofline=dict(kernel="flash_fwd_f32x_kernel", bound="mfma", achieved=tfl, peak=MFMA_BF16_PEAK_TFLOPS,
+                      unit="TFLOP/s", frac=tfl / MFMA_BF16_PEAK_TFLOPS, traffic=None,
+                      traffic_source="not measured: 16 workgroups, 0.27 GFLOP, bound by launch latency"),
     )
     if cpu_baseline:
         from oracle import ref_attention as ref
