@@ -835,46 +835,6 @@ struct FwdTileF32x {
   static_assert(BK * (D / 4) % NT == 0, "a tile divides evenly over the threads");
 };
 
-// Two fp32 values as three pairs of bf16: hi = rn(x), mid = rn(x - hi), lo = rn(x - hi - mid).
-struct Split3x2 {
-  bf16x2 part[3];
-};
-__device__ __forceinline__ Split3x2 split3(float x0, float x1) {
-  Split3x2 r;
-  r.part[0] = pack_bf16(x0, x1);
-  const unsigned hb = __builtin_bit_cast(unsigned, r.part[0]);
-  const float r0 = x0 - __uint_as_float(hb << 16), r1 = x1 - __uint_as_float(hb & 0xffff0000u);
-  r.part[1] = pack_bf16(r0, r1);
-  const unsigned mb = __builtin_bit_cast(unsigned, r.part[1]);
-  r.part[2] = pack_bf16(r0 - __uint_as_float(mb << 16), r1 - __uint_as_float(mb & 0xffff0000u));
-  return r;
-}
-// Eight fp32 values as the three MFMA operands hi, mid, lo.
-struct Split3x8 {
-  union {
-    bf16x8 v;
-    bf16x2 p[4];
-  } part[3];
-};
-__device__ __forceinline__ void split3x8(const float (&x)[8], Split3x8& out) {
-#pragma unroll
-  for (int i = 0; i < 4; i++) {
-    const Split3x2 s = split3(x[2 * i], x[2 * i + 1]);
-#pragma unroll
-    for (int p = 0; p < 3; p++) out.part[p].p[i] = s.part[p];
-  }
-}
-// c += a b from the split operands: the six partial products, the small ones first.
-__device__ __forceinline__ floatx16 mfma_split(const bf16x8 (&a)[3], const bf16x8 (&b)[3], floatx16 c) {
-  c = ElemBf16::mfma_32x32x16(a[2], b[0], c);
-  c = ElemBf16::mfma_32x32x16(a[0], b[2], c);
-  c = ElemBf16::mfma_32x32x16(a[1], b[1], c);
-  c = ElemBf16::mfma_32x32x16(a[1], b[0], c);
-  c = ElemBf16::mfma_32x32x16(a[0], b[1], c);
-  c = ElemBf16::mfma_32x32x16(a[0], b[0], c);
-  return c;
-}
-
 template <int D, int NW>
 __global__ __launch_bounds__(64 * NW) void flash_fwd_f32x_kernel(const FwdArgs a) {
   using Tile = FwdTileF32x<D, NW>;
