@@ -399,14 +399,16 @@ struct BwdTileF32x {
   static constexpr int NT = 256;
   static constexpr int ROWS = 128;
   static constexpr int TILE = 32;
-  static constexpr int STRIDE = D * 2 + 16;            // bytes per row of a plane: the 16 rows of a row read hit all banks
+  static constexpr int STRIDE = D * 2;                 // bytes per row of a tile plane: unpadded, 16-byte chunks swizzled
+                                                       // (tile_swizzle: free of bank conflicts for both kinds of read)
+  static constexpr int OWN_STRIDE = D * 2 + 16;        // rows of the owned planes, read one row per lane: padded
   static constexpr int PLANE = TILE * STRIDE;
   static constexpr int TENSOR = 3 * PLANE;
   static constexpr int BUF_BYTES = 2 * TENSOR + 2 * TILE * 4;   // two tensors' tiles, two rows of statistics
   static constexpr int PS = D + 1;                     // words per row of the fp32 pass of the owned rows
   static constexpr int OWN_BYTES = ROWS * PS * 4;
   static constexpr int LDS_BYTES = 2 * BUF_BYTES > OWN_BYTES ? 2 * BUF_BYTES : OWN_BYTES;
-  static constexpr int OWN_PLANE = ROWS * STRIDE;       // one plane of an owned tensor kept in LDS (dK/dV kernel: K)
+  static constexpr int OWN_PLANE = ROWS * OWN_STRIDE;   // one plane of an owned tensor kept in LDS (dK/dV kernel: K)
   static constexpr int LDS_BYTES_DKDV = 3 * OWN_PLANE + BUF_BYTES > OWN_BYTES ? 3 * OWN_PLANE + BUF_BYTES : OWN_BYTES;
   static constexpr int LD4 = TILE * (D / 4) / NT;
   static_assert(TILE * (D / 4) % NT == 0, "a tile divides evenly over the threads");
@@ -453,7 +455,7 @@ __device__ __forceinline__ void tile_deposit_split(char* planes, const float4 (&
     for (int p = 0; p < 3; p++) {
       union { bf16x2 h[2]; uint2 u; } w;
       w.h[0] = lo2.part[p]; w.h[1] = hi2.part[p];
-      *(uint2*)(planes + p * Tile::PLANE + row * Tile::STRIDE + c4 * 8) = w.u;
+      *(uint2*)(planes + p * Tile::PLANE + row * Tile::STRIDE + (((c4 >> 1) ^ tile_swizzle<D>(row)) << 4) + (c4 & 1) * 8) = w.u;
     }
   }
 }
@@ -466,23 +468,43 @@ __device__ __forceinline__ void tile_request_x(float4 (&x)[BwdTileF32x<D>::LD4],
     x[i] = *(const float4*)(src + (int64_t)row * stride + c4 * 4);
   }
 }
-// Row-read operand (A) of k-step `ks` from a tile's planes; `row_off` = swap_bits_2_3(l32) * STRIDE + 16 g.
+// Per-lane read offsets into a tile plane.
 template <int D>
-__device__ __forceinline__ void read_rows(bf16x8 (&f)[3], const char* planes, int row_off, int ks) {
+struct TileReadOffsets {
+  int row_base, row_xor;          // row read: row swap_bits_2_3(l32), chunk (2 ks + g) ^ swizzle
+  int tr_base[2], tr_xor[2];      // transposing read: rows 8 g + j16 / 4 and + 4, byte column (16 half + 4 (j16 % 4)) * 2 + 64 dt
+  int tr_col;
+  __device__ __forceinline__ void init(int lane) {
+    using Tile = BwdTileF32x<D>;
+    const int l32 = lane & 31, g = lane >> 5, j16 = lane & 15, half = (lane >> 4) & 1;
+    const int row = swap_bits_2_3(l32);
+    row_base = row * Tile::STRIDE;
+    row_xor = (16 * g) ^ (tile_swizzle<D>(row) << 4);
+    const int t_row = 8 * g + (j16 >> 2), col = (16 * half + 4 * (j16 & 3)) * 2;
+    tr_col = col & ~15;
+    tr_base[0] = t_row * Tile::STRIDE + (col & 15);
+    tr_base[1] = tr_base[0] + 4 * Tile::STRIDE;
+    tr_xor[0] = tile_swizzle<D>(t_row) << 4;
+    tr_xor[1] = tile_swizzle<D>(t_row + 4) << 4;
+  }
+};
+// Row-read operand (A) of k-step `ks` from a tile's planes.
+template <int D>
+__device__ __forceinline__ void read_rows(bf16x8 (&f)[3], const char* planes, const TileReadOffsets<D>& o, int ks) {
 #pragma unroll
-  for (int p = 0; p < 3; p++) f[p] = *(const bf16x8*)(planes + p * BwdTileF32x<D>::PLANE + row_off + 32 * ks);
+  for (int p = 0; p < 3; p++) f[p] = *(const bf16x8*)(planes + p * BwdTileF32x<D>::PLANE + o.row_base + ((32 * ks) ^ o.row_xor));
 }
-// Transposed operand (A) for the tile's rows 16 kk + 8 g .. + 7 and columns 32 dt + l32; `tr_off` =
-// (8 g + j16 / 4) * STRIDE + (16 half + 4 (j16 % 4)) * 2.
+// Transposed operand (A) for the tile's rows 16 kk + 8 g .. + 7 and columns 32 dt + l32.
 template <int D>
-__device__ __forceinline__ void read_transposed(bf16x8 (&f)[3], const char* planes, int tr_off, int kk, int dt) {
+__device__ __forceinline__ void read_transposed(bf16x8 (&f)[3], const char* planes, const TileReadOffsets<D>& o, int kk,
+                                                int dt) {
   using Tile = BwdTileF32x<D>;
 #pragma unroll
   for (int p = 0; p < 3; p++) {
     union { bf16x8 v; shortx4 hlf[2]; } u;
-    const char* at = planes + p * Tile::PLANE + tr_off + 16 * kk * Tile::STRIDE + 64 * dt;
-    u.hlf[0] = lds_read_tr16(at);
-    u.hlf[1] = lds_read_tr16(at + 4 * Tile::STRIDE);
+    const char* at = planes + p * Tile::PLANE + 16 * kk * Tile::STRIDE;   // rows + 16: the same swizzle
+    u.hlf[0] = lds_read_tr16(at + o.tr_base[0] + ((o.tr_col + 64 * dt) ^ o.tr_xor[0]));
+    u.hlf[1] = lds_read_tr16(at + o.tr_base[1] + ((o.tr_col + 64 * dt) ^ o.tr_xor[1]));
     f[p] = u.v;
   }
 }
@@ -544,9 +566,8 @@ void flash_bwd_dq_f32x_kernel(const BwdArgs a) {
 #pragma unroll
     for (int r = 0; r < 16; r++) dq[i][r] = 0.f;
 
-  const int row_off = swap_bits_2_3(l32) * Tile::STRIDE + 16 * g;
-  const int j16 = lane & 15, half = (lane >> 4) & 1;
-  const int tr_off = (8 * g + (j16 >> 2)) * Tile::STRIDE + (16 * half + 4 * (j16 & 3)) * 2;
+  TileReadOffsets<D> off;
+  off.init(lane);
 
   // Tile t lives in ring buffer t % 2: the planes of K, then of V.
   float4 kx[Tile::LD4], vx[Tile::LD4];
@@ -580,8 +601,8 @@ void flash_bwd_dq_f32x_kernel(const BwdArgs a) {
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ks++) {
         bf16x8 kf[3], vf[3];
-        read_rows<D>(kf, k_lds, row_off, ks);
-        read_rows<D>(vf, v_lds, row_off, ks);
+        read_rows<D>(kf, k_lds, off, ks);
+        read_rows<D>(vf, v_lds, off, ks);
         s = mfma_split(kf, q_mine[ks], s);
         dp = mfma_split(vf, do_mine[ks], dp);
       }
@@ -623,7 +644,7 @@ void flash_bwd_dq_f32x_kernel(const BwdArgs a) {
 #pragma unroll
         for (int dt = 0; dt < DT; dt++) {
           bf16x8 kt[3];
-          read_transposed<D>(kt, k_lds, tr_off, kk, dt);
+          read_transposed<D>(kt, k_lds, off, kk, dt);
           dq[dt] = mfma_split(kt, dsf, dq[dt]);
         }
       }
@@ -681,11 +702,11 @@ void flash_bwd_dkdv_f32x_kernel(const BwdArgs a) {
       for (int p = 0; p < 3; p++) {
         union { bf16x2 h[2]; uint2 u; } w;
         w.h[0] = lo2.part[p]; w.h[1] = hi2.part[p];
-        *(uint2*)(smem + p * Tile::OWN_PLANE + row * Tile::STRIDE + c4 * 8) = w.u;
+        *(uint2*)(smem + p * Tile::OWN_PLANE + row * Tile::OWN_STRIDE + c4 * 8) = w.u;
       }
     }
   }
-  const char* const k_own = smem + (wave * 32 + l32) * Tile::STRIDE + 16 * g;   // this lane's key, d = 8 g ..
+  const char* const k_own = smem + (wave * 32 + l32) * Tile::OWN_STRIDE + 16 * g;   // this lane's key, d = 8 g ..
   char* const tile_buf = smem + 3 * Tile::OWN_PLANE;
 
   // Query rows that can see a key of this block: qpos >= first key, qpos <= last key + window.
@@ -707,9 +728,8 @@ void flash_bwd_dkdv_f32x_kernel(const BwdArgs a) {
 #pragma unroll
     for (int r = 0; r < 16; r++) dk[i][r] = dv[i][r] = 0.f;
 
-  const int row_off = swap_bits_2_3(l32) * Tile::STRIDE + 16 * g;
-  const int j16 = lane & 15, half = (lane >> 4) & 1;
-  const int tr_off = (8 * g + (j16 >> 2)) * Tile::STRIDE + (16 * half + 4 * (j16 & 3)) * 2;
+  TileReadOffsets<D> off;
+  off.init(lane);
 
   // Step e of the loop is query tile t_begin + e % nt of query head hk G + e / nt: the planes of Q, then
   // of dO, then lse (in log2 units) and delta of the 32 queries.
@@ -758,8 +778,8 @@ void flash_bwd_dkdv_f32x_kernel(const BwdArgs a) {
 #pragma unroll
       for (int ks = 0; ks < KSTEPS; ks++) {
         bf16x8 qf[3], dof[3];
-        read_rows<D>(qf, q_lds, row_off, ks);
-        read_rows<D>(dof, do_lds, row_off, ks);
+        read_rows<D>(qf, q_lds, off, ks);
+        read_rows<D>(dof, do_lds, off, ks);
         bf16x8 kf[3];
 #pragma unroll
         for (int p = 0; p < 3; p++) kf[p] = *(const bf16x8*)(k_own + p * Tile::OWN_PLANE + 32 * ks);
@@ -816,8 +836,8 @@ void flash_bwd_dkdv_f32x_kernel(const BwdArgs a) {
 #pragma unroll
         for (int dt = 0; dt < DT; dt++) {
           bf16x8 dot[3], qt[3];
-          read_transposed<D>(dot, do_lds, tr_off, kk, dt);
-          read_transposed<D>(qt, q_lds, tr_off, kk, dt);
+          read_transposed<D>(dot, do_lds, off, kk, dt);
+          read_transposed<D>(qt, q_lds, off, kk, dt);
           dv[dt] = mfma_split(dot, pf, dv[dt]);
           dk[dt] = mfma_split(qt, dsf, dk[dt]);
         }
