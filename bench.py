@@ -1,6 +1,6 @@
 """Benchmark of the MI355X attention kernel path (one GPU).
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|c1|c2|c3|c4|c5] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload all|c1|c2|c3|c4|c5|f32] [--no-cpu-baseline]
 
 The headline workload (BASELINE.json configs[1], "C2") is causal GQA flash attention forward +
 backward, bf16, batch 4, 32 query heads / 8 kv heads, seq 4096, head_dim 128: a step is one forward
@@ -15,7 +15,8 @@ device's memory (C2: 2.15 GB, C3: 8.7 GB) and recomputes dS in the dQ kernel whe
 `backend_overrides` (`--recompute` / `--ds-workspace` force it for the headline).
 The paged-decode half of the metric (configs[3], "C4") is measured in the same run and reported in
 the `paged_decode` object of the same JSON line.  With the default `--workload all` the line also
-carries `c1` (configs[0]: the fp32 case the reference itself runs on CPU), `c3` (sliding window +
+carries `c1` (configs[0]: the fp32 case the reference itself runs on CPU), `f32_row` (the fp32 row of the
+reference's own kernel benchmark, forward and backward), `c3` (sliding window +
 packed segments) and `c5` (one GPU's share of a 32768-token sequence), each with its own `roofline`
 and `cpu_baseline`.
 
@@ -326,6 +327,31 @@ def cpu_baseline_flash(cfg, budget_s=8.0):
     )
 
 
+def bench_f32_row(steps, warmup):
+    """The fp32 row of the reference's own kernel benchmark (gpu_attention_benchmark.py:55-59, :93-97):
+    causal MHA, batch 2, 32 heads, 4096 tokens, head_dim 128, forward and backward through the C ABI.  A
+    side line: fp32 products are formed from bf16 parts on the bf16 matrix instruction."""
+    from axlearn_amd import ops
+
+    dev = torch.device("cuda:0")
+    B, T, H, D = 2, 4096, 32, 128
+    q, k, v, do = (normal_tensor(s, (B, T, H, D), torch.float32, dev) for s in (0, 1, 2, 3))
+    kw = dict(softmax_scale=D ** -0.5, mask_kind=ops.MASK_CAUSAL)
+    out, lse = ops.flash_fwd(q, k, v, **kw)
+    bufs = ops.flash_bwd_buffers(q, k, v, mask_kind=ops.MASK_CAUSAL)
+    n = max(3, steps // 4)
+    ms_fwd = _time_region(lambda: ops.flash_fwd(q, k, v, **kw), n, min(warmup, 2))
+    ms_bwd = _time_region(lambda: ops.flash_bwd(q, k, v, out, lse, do, buffers=bufs, **kw), n, min(warmup, 2))
+    fl_fwd = 4.0 * B * H * T * T * D / 2.0
+    return dict(
+        workload="reference benchmark row: causal MHA fwd / bwd, fp32, B2 H32 T4096 D128",
+        arithmetic="fp32 operands as three bf16 parts each, six bf16 MFMA partial products per product, fp32 accumulation",
+        fwd_ms=ms_fwd, bwd_ms=ms_bwd, fwd_tflops=fl_fwd / (ms_fwd * 1e-3) / 1e12,
+        bwd_tflops=2.5 * fl_fwd / (ms_bwd * 1e-3) / 1e12, fp32_mfma_peak_tflops=MFMA_F32_PEAK_TFLOPS,
+        kernels=["flash_fwd_f32x_kernel", "flash_bwd_dkdv_f32x_kernel", "flash_bwd_dq_f32x_kernel"],
+    )
+
+
 def bench_c1(steps, warmup, cpu_baseline):
     """C1 (configs[0]): causal MHA forward, fp32, B2 H4 T512 D64, scale 1/8.  The CPU oracle is the
     subject (timed in full); the fp32 forward kernel is timed, and checked against it, beside it."""
@@ -475,7 +501,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="all", choices=["all", "c1", "c2", "c3", "c4", "c5"],
+    ap.add_argument("--workload", default="all", choices=["all", "c1", "c2", "c3", "c4", "c5", "f32"],
                     help="all: headline C2 + C4, with C1, C3 and C5 as extra keys of the same line")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-decode", action="store_true", help="skip the paged-decode half of the metric")
@@ -511,6 +537,10 @@ def main():
         if "cpu_baseline" in dec:
             line["cpu_baseline"] = dec["cpu_baseline"]
         line["paged_decode"] = dec
+    elif args.workload == "f32":
+        res = bench_f32_row(args.steps, args.warmup)
+        line.update(value=res["fwd_tflops"], unit="TFLOP/s", ms_per_step=res["fwd_ms"], dtype="f32",
+                    config=dict(workload=res["workload"]), f32_row=res)
     elif args.workload == "c1":
         res = bench_c1(args.steps, args.warmup, cpu_base)
         line.update(value=res["value"], unit="TFLOP/s", ms_per_step=res["ms_per_step"], dtype="f32",
@@ -547,6 +577,7 @@ def main():
             other("c2", res, args.steps, args.warmup)
             line["machine"] = calibrate_mfma()
             line["c1"] = bench_c1(args.steps, args.warmup, cpu_base)
+            line["f32_row"] = bench_f32_row(args.steps, args.warmup)
             line["c3"] = bench_flash(dict(_flash_workload("c3"), ds_workspace=forced), max(5, args.steps // 2), 2, cpu_base)
             other("c3", line["c3"], max(5, args.steps // 2), 2)
             line["c5"] = bench_flash(dict(_flash_workload("c5"), ds_workspace=forced), max(3, args.steps // 4), 1, cpu_base)
