@@ -31,6 +31,20 @@ int launch_decode(const AxlDecodeParams& p, hipStream_t stream);
 size_t decode_workspace_bytes(const AxlDecodeParams& p);
 int launch_page_insert(const AxlPageInsertParams& p, hipStream_t stream);
 
+// Compute units of the current device (256 on an MI355X; that figure too if the query fails), looked up once.
+int cu_count() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+      n = v;
+    else
+      n = 256;
+  }
+  return n;
+}
+
 hipError_t allow_dynamic_lds(const void* kernel, int bytes) {
   int dev = 0;
   hipError_t err = hipGetDevice(&dev);

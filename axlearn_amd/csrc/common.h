@@ -584,4 +584,7 @@ int set_error(int code, const char* fmt, ...);
 // first time the kernel is launched on the current device; later launches only look the pair up.
 hipError_t allow_dynamic_lds(const void* kernel, int bytes);
 
+// Compute units of the current device, looked up once (defined in api.hip).
+int cu_count();
+
 }  // namespace axl

@@ -1126,13 +1126,14 @@ int launch_flash_fwd(const AxlFlashFwdParams& p, hipStream_t stream) {
       if (p.head_dim == 128) AXL_LAUNCH_FWD(flash_fwd_f32_kernel<128>, FwdTileF32<128>);
       else AXL_LAUNCH_FWD(flash_fwd_f32_kernel<64>, FwdTileF32<64>);
     } else {
-      // eight wavefronts (two per SIMD, 256 query rows share a tile's split) where the length allows
+      // eight wavefronts (two per SIMD, 256 query rows share a tile's split) where the length allows and such
+      // workgroups are still at least as many as the CUs (a small call is bound by its longest workgroup)
       static const bool four = [] { const char* e = getenv("AXL_F32X_WAVES"); return e && e[0] == '4'; }();
       using T128x8 = FwdTileF32x<128, 8>;
       using T64x8 = FwdTileF32x<64, 8>;
       using T128x4 = FwdTileF32x<128, 4>;
       using T64x4 = FwdTileF32x<64, 4>;
-      if (p.q_len % 256 == 0 && !four) {
+      if (p.q_len % 256 == 0 && !four && (int64_t)(p.q_len / 256) * p.batch * p.num_q_heads >= cu_count()) {
         if (p.head_dim == 128) AXL_LAUNCH_FWD((flash_fwd_f32x_kernel<128, 8>), T128x8);
         else AXL_LAUNCH_FWD((flash_fwd_f32x_kernel<64, 8>), T64x8);
       } else {

@@ -832,19 +832,6 @@ static void set_bias(DecArgs& a, const AxlDecodeBias& x, float scale) {
   a.inv_scale = 1.0f / scale;
 }
 
-static int cu_count() {
-  static int n = 0;
-  if (n == 0) {
-    int dev = 0, v = 0;
-    if (hipGetDevice(&dev) == hipSuccess &&
-        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
-      n = v;
-    else
-      n = 256;
-  }
-  return n;
-}
-
 // AXL_DECODE_DETERMINISTIC in the environment, read once: the default for calls that do not set the flag.
 static bool deterministic_by_default() {
   static const bool v = [] {

@@ -371,7 +371,7 @@ def bench_c1(steps, warmup, cpu_baseline):
         executed_tflops=6.0 * tfl, fp32_mfma_peak_tflops=MFMA_F32_PEAK_TFLOPS,
         roofline=dict(kernel="flash_fwd_f32x_kernel", bound="mfma", achieved=tfl, peak=MFMA_BF16_PEAK_TFLOPS,
                       unit="TFLOP/s", frac=tfl / MFMA_BF16_PEAK_TFLOPS, traffic=None,
-                      traffic_source="not measured: 16 workgroups, 0.27 GFLOP, bound by launch latency"),
+                      traffic_source="not measured: 32 workgroups, 0.27 GFLOP, bound by launch latency"),
     )
     if cpu_baseline:
         from oracle import ref_attention as ref
