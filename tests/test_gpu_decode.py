@@ -75,6 +75,43 @@ def test_paged_and_contiguous_decode_against_ref(b, s, h, d, padding, kv_head_fa
     assert ref.max_abs(got.cpu(), det.cpu().float()) <= 2e-3
 
 
+@pytest.mark.parametrize("b,s,h,hkv", [
+    (1, 1024, 8, 8),     # 8 rows of 64 pages: 8-page blocks, dealt by workgroup index
+    (4, 2048, 8, 8),     # 32 rows: exactly as many 8-page blocks as workgroup slots
+    (5, 2048, 8, 8),     # 40 rows: 12-page blocks, 11 per row
+    (3, 1040, 32, 2),    # a last block shorter than the others
+    (32, 1024, 8, 8),    # 256 rows of two 32-page blocks: not shortened, still one block per workgroup
+    (33, 1024, 8, 8),    # one row more: drawn from the counter again
+])
+def test_small_calls_take_short_blocks(b, s, h, hkv):
+    """Calls with fewer 32-page blocks than the split kernel has workgroup slots (512 on an MI355X) take
+    shorter blocks and, where the shapes bound the blocks by the workgroups, are dealt by workgroup index
+    without the work counter: ragged lengths, with and without a window, against the oracle, on a
+    workspace full of NaN bit patterns (a counter that was read, or a record that was not written,
+    shows), and bit-identical between the paged and the contiguous form under the fixed decomposition."""
+    d = 128
+    pps = (s + 15) // 16
+    q, kp, vp, tables, lengths = ref.paged_inputs(21, batch=b, num_heads=h, num_kv_heads=hkv, head_dim=d, page_size=16,
+                                                   pages_per_seq=pps, min_len=1, max_len=s)
+    lengths[0] = s   # the longest context takes every block of its row
+    scale = d ** -0.5
+    args = (q[:, 0].cuda(), kp.cuda(), vp.cuda(), tables.cuda(), lengths.cuda())
+    need = ops.paged_decode_workspace_bytes(b, h, hkv, d, pps)
+    for window in (-1, 200):
+        want = ref.reference_decode(q, kp, vp, lengths, softmax_scale=scale, page_tables=tables,
+                                    sliding_window=None if window < 0 else window)[:, 0]
+        ws = torch.full((need,), 0xFF, dtype=torch.uint8, device="cuda")
+        got = ops.paged_decode(*args, softmax_scale=scale, sliding_window=window, workspace=ws)
+        assert torch.isfinite(got.float()).all() and _ok(got.cpu(), want), (window, ref.rel_l2(got.cpu(), want))
+        kk, vv = ref.reconstruct_kv(tables, kp), ref.reconstruct_kv(tables, vp)
+        with _deterministic():
+            ws.fill_(0xFF)
+            det_p = ops.paged_decode(*args, softmax_scale=scale, sliding_window=window, workspace=ws)
+            det_c = ops.decode(args[0], kk[:, :s].contiguous().cuda(), vv[:, :s].contiguous().cuda(), args[4],
+                               softmax_scale=scale, sliding_window=window)
+        assert _ok(det_p.cpu(), want) and torch.equal(det_p, det_c)
+
+
 def test_ragged_lengths_and_brute_force():
     b, hq, hkv, d, pps = 5, 8, 2, 128, 24
     q, kp, vp, tables, lengths = ref.paged_inputs(7, batch=b, num_heads=hq, num_kv_heads=hkv, head_dim=d,
