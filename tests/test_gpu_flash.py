@@ -130,10 +130,18 @@ def test_backward_matches_oracle(b, t, hq, hkv, d, mask, window, seg):
     wq, wk, wv = ref.reference_mha_grads(q, k, v, do, spec, softmax_scale=scale)
     qc, kc, vc, doc = q.cuda(), k.cuda(), v.cuda(), do.cuda()
     out, lse = ops.flash_fwd(qc, kc, vc, softmax_scale=scale, **kw)
+    _assert_close("out", out, ref.reference_mha(q, k, v, spec, softmax_scale=scale), dtype)
     dq, dk, dv = ops.flash_bwd(qc, kc, vc, out, lse, doc, softmax_scale=scale, **kw)
-    _assert_close("dq", dq, wq, dtype)
-    _assert_close("dk", dk, wk, dtype)
-    _assert_close("dv", dv, wv, dtype)
+    if hq * t >= 16384:
+        # dk / dv of the two large cases sum a thousand rows of several heads into elements of magnitude
+        # 3 to 10, whose fp32 spacing alone is up to 1e-6: the bar scales with the largest element there.
+        for name, got, want in (("dq", dq, wq), ("dk", dk, wk), ("dv", dv, wv)):
+            err, top = ref.max_abs(got.cpu(), want), float(want.abs().max())
+            assert err <= FP32_MAX_ABS * max(1.0, top), f"{name}: max-abs {err:.3e}, largest element {top:.2f}"
+    else:
+        _assert_close("dq", dq, wq, dtype)
+        _assert_close("dk", dk, wk, dtype)
+        _assert_close("dv", dv, wv, dtype)
 
 
 @pytest.mark.parametrize("b,t,hq,hkv,d,mask,window,seg", [
@@ -156,9 +164,16 @@ def test_float16_backward_matches_oracle(b, t, hq, hkv, d, mask, window, seg):
     out, lse = ops.flash_fwd(qc, kc, vc, softmax_scale=scale, **kw)
     _assert_close("out", out, ref.reference_mha(q, k, v, spec, softmax_scale=scale), dtype)
     dq, dk, dv = ops.flash_bwd(qc, kc, vc, out, lse, doc, softmax_scale=scale, **kw)
-    _assert_close("dq", dq, wq, dtype)
-    _assert_close("dk", dk, wk, dtype)
-    _assert_close("dv", dv, wv, dtype)
+    if hq * t >= 16384:
+        # dk / dv of the two large cases sum a thousand rows of several heads into elements of magnitude
+        # 3 to 10, whose fp32 spacing alone is up to 1e-6: the bar scales with the largest element there.
+        for name, got, want in (("dq", dq, wq), ("dk", dk, wk), ("dv", dv, wv)):
+            err, top = ref.max_abs(got.cpu(), want), float(want.abs().max())
+            assert err <= FP32_MAX_ABS * max(1.0, top), f"{name}: max-abs {err:.3e}, largest element {top:.2f}"
+    else:
+        _assert_close("dq", dq, wq, dtype)
+        _assert_close("dk", dk, wk, dtype)
+        _assert_close("dv", dv, wv, dtype)
     bufs = (torch.zeros_like(dq), torch.zeros_like(dk), torch.zeros_like(dv),
             ops.flash_bwd_buffers(qc, kc, vc, mask_kind=kw["mask_kind"], segment_ids=kw.get("segment_ids"))[3])
     for phase in (1, 2, 4):  # delta, dK/dV, dQ
@@ -176,6 +191,9 @@ def test_float16_backward_matches_oracle(b, t, hq, hkv, d, mask, window, seg):
     (1, 128, 384, 2, 1, 128, "none", None, False),
     (1, 640, 640, 2, 1, 64, "sliding", 33, False),
     (1, 256, 512, 4, 2, 64, "causal", None, False),
+    # enough 256-row blocks for every CU: the forward runs its workgroups of eight wavefronts
+    (2, 1024, 1024, 32, 8, 128, "causal", None, False),
+    (4, 512, 512, 32, 32, 64, "sliding", 100, True),
 ])
 def test_float32_backward_matches_oracle(b, t, s, hq, hkv, d, mask, window, seg):
     """float32 forward + backward (gpu_attention_test.py:197 runs float16 and float32; the reference
@@ -189,10 +207,18 @@ def test_float32_backward_matches_oracle(b, t, s, hq, hkv, d, mask, window, seg)
     wq, wk, wv = ref.reference_mha_grads(q, k, v, do, spec, softmax_scale=scale)
     qc, kc, vc, doc = q.cuda(), k.cuda(), v.cuda(), do.cuda()
     out, lse = ops.flash_fwd(qc, kc, vc, softmax_scale=scale, **kw)
+    _assert_close("out", out, ref.reference_mha(q, k, v, spec, softmax_scale=scale), dtype)
     dq, dk, dv = ops.flash_bwd(qc, kc, vc, out, lse, doc, softmax_scale=scale, **kw)
-    _assert_close("dq", dq, wq, dtype)
-    _assert_close("dk", dk, wk, dtype)
-    _assert_close("dv", dv, wv, dtype)
+    if hq * t >= 16384:
+        # dk / dv of the two large cases sum a thousand rows of several heads into elements of magnitude
+        # 3 to 10, whose fp32 spacing alone is up to 1e-6: the bar scales with the largest element there.
+        for name, got, want in (("dq", dq, wq), ("dk", dk, wk), ("dv", dv, wv)):
+            err, top = ref.max_abs(got.cpu(), want), float(want.abs().max())
+            assert err <= FP32_MAX_ABS * max(1.0, top), f"{name}: max-abs {err:.3e}, largest element {top:.2f}"
+    else:
+        _assert_close("dq", dq, wq, dtype)
+        _assert_close("dk", dk, wk, dtype)
+        _assert_close("dv", dv, wv, dtype)
     bufs = (torch.zeros_like(dq), torch.zeros_like(dk), torch.zeros_like(dv),
             ops.flash_bwd_buffers(qc, kc, vc, mask_kind=kw["mask_kind"], segment_ids=kw.get("segment_ids"))[3])
     for phase in (1, 2, 4):  # delta, dK/dV, dQ
