@@ -226,6 +226,45 @@ def test_float32_backward_matches_oracle(b, t, s, hq, hkv, d, mask, window, seg)
     assert torch.equal(bufs[0], dq) and torch.equal(bufs[1], dk) and torch.equal(bufs[2], dv)
 
 
+def test_float32_kernels_on_the_fp32_matrix_instruction_agree():
+    """The library keeps its first fp32 kernels (v_mfma_f32_32x32x2_f32) behind AXL_F32_MFMA=1, read once per
+    process: a child process runs them on the inputs this process gives the default kernels (fp32 products
+    from split bf16 operands); forward, lse and gradients agree to the fp32 bar (scaled by the largest
+    element for the gradients, which sum hundreds of rows)."""
+    import os
+    import subprocess
+    import sys
+    import tempfile
+
+    b, t, hq, hkv, d = 1, 512, 8, 2, 128
+    q, k, v, do = (x.cuda() for x in _inputs(b, t, hq, hkv, d, torch.float32))
+    segs = ref.packed_segment_ids(4, b, t, max_docs=3).cuda()
+    kw = dict(softmax_scale=d ** -0.5, mask_kind=ops.MASK_SLIDING_WINDOW, sliding_window=300, segment_ids=segs)
+    out, lse = ops.flash_fwd(q, k, v, **kw)
+    mine = [out, lse] + list(ops.flash_bwd(q, k, v, out, lse, do, **kw)[:3])
+    child = (
+        "import sys, torch\n"
+        "from axlearn_amd import ops\n"
+        "x = torch.load(sys.argv[1], weights_only=True)\n"
+        "kw = dict(softmax_scale=x['scale'], mask_kind=ops.MASK_SLIDING_WINDOW, sliding_window=300, segment_ids=x['segs'].cuda())\n"
+        "q, k, v, do = (x[n].cuda() for n in ('q', 'k', 'v', 'do'))\n"
+        "out, lse = ops.flash_fwd(q, k, v, **kw)\n"
+        "res = [out, lse] + list(ops.flash_bwd(q, k, v, out, lse, do, **kw)[:3])\n"
+        "torch.save([r.cpu() for r in res], sys.argv[2])\n"
+    )
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    with tempfile.TemporaryDirectory() as tmp:
+        src, dst = os.path.join(tmp, "in.pt"), os.path.join(tmp, "out.pt")
+        torch.save(dict(q=q.cpu(), k=k.cpu(), v=v.cpu(), do=do.cpu(), segs=segs.cpu(), scale=d ** -0.5), src)
+        env = dict(os.environ, AXL_F32_MFMA="1", PYTHONPATH=root + os.pathsep + os.environ.get("PYTHONPATH", ""))
+        subprocess.run([sys.executable, "-c", child, src, dst], check=True, env=env, timeout=110, cwd=root)
+        theirs = torch.load(dst, weights_only=True)
+    for name, a, c in zip(("out", "lse", "dq", "dk", "dv"), mine, theirs):
+        err, top = ref.max_abs(a.cpu(), c.double()), float(c.abs().max())
+        assert err <= 2 * FP32_MAX_ABS * max(1.0, top), f"{name}: the two kernel families differ by {err:.3e} (largest element {top:.2f})"
+        assert not torch.equal(a.cpu(), c) or name == "lse", f"{name}: identical bits - the child did not run the other kernels"
+
+
 @pytest.mark.parametrize("mask,window", [("causal", None), ("sliding", 333)])
 @pytest.mark.parametrize("d", [64, 128])
 def test_backward_with_more_keys_than_queries(mask, window, d):
